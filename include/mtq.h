@@ -1,0 +1,204 @@
+/*
+ * mtq.h -- C-ABI of libmtq_hip.so: MI355X (gfx950) affine-quantized matmul.
+ *
+ * This is the boundary a HIP backend of the reference's runtime binds. The
+ * reference reaches its GPU through two Rust call sites, both of which move
+ * flat byte buffers bound by position:
+ *   - Context::dispatch_with_grid(kernel, buffers, fn_consts, grid, tpg)
+ *       crates/metaltile-runtime/src/context.rs:269-283   (tests)
+ *   - GpuRunner::{new, compile, buffer_bytes, buffer_zeros, read_bytes,
+ *       measure, flush_slc}
+ *       crates/metaltile-std/src/runner.rs:253,287,317,324,354,413,455 (bench)
+ * Each entry point below names the reference interface it replaces.
+ *
+ * Conventions
+ *   - Every function returns 0 on success or a negative MTQ_ERR_* code; the
+ *     message for the calling thread's last failure is mtq_last_error().
+ *     Nothing throws or aborts across this boundary (the reference builds with
+ *     panic = "abort", Cargo.toml:87).
+ *   - Device pointers are plain `void*` obtained from mtq_alloc (or any other
+ *     HIP allocation on the same device). The caller owns host memory; the
+ *     library copies in and out (reference: single_dispatch.rs:163-171, 100-117).
+ *   - Kernels are enqueued on the library's stream and do not block the host
+ *     unless stated; mtq_download and mtq_sync wait for them.
+ *   - Element dtype T of scales / biases / x / out is MTQ_F32, MTQ_F16 or
+ *     MTQ_BF16. Weights are unsigned codes packed LSB-first into little-endian
+ *     u32 words, row-major [N][K*bits/32]; w_hat = scale_g*q + bias_g with
+ *     g = k / group_size; sums are f32; results are rounded to T on store
+ *     (crates/metaltile-std/src/mlx/quantized.rs:5374-5404).
+ *   - There is no CPU fallback: without a usable GPU every call fails with
+ *     MTQ_ERR_NO_DEVICE.
+ *   - Single-threaded use per process, like the reference's runner
+ *     (crates/metaltile-std/src/runner.rs:209-229).
+ */
+#ifndef MTQ_H
+#define MTQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MTQ_API __attribute__((visibility("default")))
+
+/* element dtypes (reference: metaltile_core::dtype::DType F32 / F16 / BF16) */
+enum { MTQ_F32 = 0, MTQ_F16 = 1, MTQ_BF16 = 2 };
+
+/* error codes -- counterpart of MetalTileError, crates/metaltile-runtime/src/error.rs:8-55 */
+enum {
+    MTQ_OK = 0,
+    MTQ_ERR_NO_DEVICE = -1,      /* NoDevice */
+    MTQ_ERR_BAD_ARG = -2,        /* Buffer / invalid argument */
+    MTQ_ERR_SHAPE = -3,          /* Dispatch: shape violates a kernel precondition */
+    MTQ_ERR_BUFFER_SIZE = -4,    /* BufferSize{param, expected, actual} */
+    MTQ_ERR_UNKNOWN_KERNEL = -5, /* no kernel of that name: caller may fall back */
+    MTQ_ERR_HIP = -6,            /* Dispatch: runtime failure */
+    MTQ_ERR_UNSUPPORTED = -7     /* valid request without a kernel in this build */
+};
+
+/* A bound buffer: device pointer plus its length in bytes (the reference binds
+ * `Vec<u8>` and checks lengths, single_dispatch.rs:154-158). */
+typedef struct mtq_buf {
+    void *ptr;
+    size_t bytes;
+} mtq_buf;
+
+typedef struct mtq_device_info {
+    char name[128];
+    char arch[32];          /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+    int compute_units;
+    int clock_khz;          /* engine clock reported by the runtime */
+    int memory_clock_khz;
+    int memory_bus_bits;
+    size_t total_memory;    /* bytes */
+    int l2_bytes;
+    int lds_per_cu_bytes;
+} mtq_device_info;
+
+/* ---- lifetime / device -------------------------------------------------- */
+
+/* Replaces GpuRunner::new (crates/metaltile-std/src/runner.rs:253-285) and
+ * Context::new (crates/metaltile-runtime/src/context.rs:174): pick the device,
+ * create the stream and timing events. Idempotent for the same device. */
+MTQ_API int mtq_init(int device);
+MTQ_API int mtq_shutdown(void);
+/* Thread-local message of the last failing call ("" if none). */
+MTQ_API const char *mtq_last_error(void);
+/* Replaces GpuRunner::device_name (crates/metaltile-std/src/runner.rs:95). */
+MTQ_API int mtq_device_name(char *out, size_t cap);
+MTQ_API int mtq_get_device_info(mtq_device_info *out);
+/* Use a caller-owned hipStream_t (passed as void*) for all later launches;
+ * NULL restores the library's own stream. */
+MTQ_API int mtq_set_stream(void *hip_stream);
+
+/* ---- buffers ------------------------------------------------------------ */
+
+/* Replace GpuRunner::buffer_zeros / buffer_bytes / read_bytes
+ * (crates/metaltile-std/src/runner.rs:317-360) and Context::upload_resident
+ * (crates/metaltile-runtime/src/context.rs:330-337). mtq_alloc zero-fills. */
+MTQ_API int mtq_alloc(size_t bytes, void **dptr);
+MTQ_API int mtq_free(void *dptr);
+MTQ_API int mtq_upload(void *dptr, const void *host, size_t bytes);
+MTQ_API int mtq_download(void *host, const void *dptr, size_t bytes);
+MTQ_API int mtq_memset(void *dptr, int byte_value, size_t bytes);
+MTQ_API int mtq_sync(void);
+
+/* ---- typed entry points (device pointers) ------------------------------- */
+
+/* qmv: out[m,n] = sum_k w_hat[n,k] * x[m,k] for a small batch of rows (M >= 1).
+ * Replaces mt_qmv / mt_qmv_int8_fast / mt_qmm / mt_qmm_bm2 / mt_qmm_bm4 and the
+ * int8 trio (crates/metaltile-std/src/mlx/quantized.rs:8, 1475, 343, 650,
+ * 1072, 1602, 1719, 1870), dequant_gemv_int{2..8} and _int4_fast
+ * (crates/metaltile-std/src/ffai/dequant_gemv.rs:52-341) and mt_qmv_b* / mt_qmm_b*
+ * (quantized.rs:4273-4392). bits in 2..8; group_size divides K. */
+MTQ_API int mtq_qmv(int dtype, int bits, uint32_t group_size, const void *w, const void *scales,
+                    const void *biases, const void *x, void *out, uint32_t M, uint32_t N,
+                    uint32_t K);
+
+/* qmm: same product for any M; routes by M like mt_qmm_for
+ * (crates/metaltile-std/src/mlx/quantized.rs:5040-5065): large M runs the
+ * LDS-dequant + MFMA tile kernel (replaces mt_qmm_mma / _m16 / _int8 / _int2,
+ * quantized.rs:2106, 2408, 2731, 3330), small M the qmv family. */
+MTQ_API int mtq_qmm(int dtype, int bits, uint32_t group_size, const void *w, const void *scales,
+                    const void *biases, const void *x, void *out, uint32_t M, uint32_t N,
+                    uint32_t K);
+
+/* gather_qmv, CSR view: out[t,n] = sum_k x[t,k] * w_hat[E(t)][n,k], E(t) = first
+ * e with t < expert_offsets[e+1] (0 if none). Replaces
+ * mt_moe_gather_qmm_int4{,_m8,_m16,_m32} and _b* (crates/metaltile-std/src/ffai/moe.rs:358,
+ * 634, 900, 1363, 461-605). w is [E][N][K*bits/32], scales/biases [E][N][K/G],
+ * x [T][K], expert_offsets u32[E+1], out [T][N]. */
+MTQ_API int mtq_gather_qmv_csr(int dtype, int bits, uint32_t group_size, const void *x,
+                               const void *w, const void *scales, const void *biases,
+                               const uint32_t *expert_offsets, void *out, uint32_t T, uint32_t N,
+                               uint32_t K, uint32_t E);
+
+/* gather_qmv, per-row view: E(t) = indices[t]; rows need not be sorted; rows
+ * whose index is >= E are left untouched. Replaces mt_moe_gather_qmm_mma_int4 /
+ * _bm16 / _mma_int8 / _mma_b* (crates/metaltile-std/src/ffai/moe.rs:2256, 2857, 3231,
+ * 2552-2835). */
+MTQ_API int mtq_gather_qmv_indices(int dtype, int bits, uint32_t group_size, const void *x,
+                                   const void *w, const void *scales, const void *biases,
+                                   const uint32_t *indices, void *out, uint32_t T, uint32_t N,
+                                   uint32_t K, uint32_t E);
+
+/* gather_qmv, single view: one row against slab expert_index[0] (read on the
+ * device, no host round trip; ids >= E are clamped to E-1). Replaces
+ * dequant_gemv_int4_expert_indexed
+ * (crates/metaltile-std/src/ffai/dequant_gemv_expert_indexed.rs:58-105). */
+MTQ_API int mtq_gather_qmv_single(int dtype, int bits, uint32_t group_size, const void *w,
+                                  const void *scales, const void *biases, const void *input,
+                                  const uint32_t *expert_index, void *output, uint32_t N,
+                                  uint32_t K, uint32_t E);
+
+/* ---- name-keyed dispatch (the reference's binding convention) ----------- */
+
+/* Replaces Context::dispatch_with_grid (crates/metaltile-runtime/src/context.rs:269-283)
+ * and GpuRunner::compile + measure(.., 0, 1) (crates/metaltile-std/src/runner.rs:287, 413):
+ * `kernel_name` is the reference kernel's `name` ("mt_qmv", "mt_qmm_mma",
+ * "dequant_gemv_int4", "mt_moe_gather_qmm_int4", ...), `bufs` are its tensor
+ * parameters in signature order, `consts` its constexprs in signature order
+ * (crates/metaltile-std/src/run_kernel.rs:183-188, 210-234). grid/tpg describe
+ * the Metal launch and are accepted for compatibility; the HIP launch is
+ * derived from name, dtype, constexprs and buffer lengths. Buffers shorter
+ * than the op needs fail with MTQ_ERR_BUFFER_SIZE. Blocks until the kernel has
+ * finished; *elapsed_us (may be NULL) receives its GPU duration. An unknown
+ * name fails with MTQ_ERR_UNKNOWN_KERNEL so a caller can fall back. */
+MTQ_API int mtq_dispatch(const char *kernel_name, int dtype, const mtq_buf *bufs, int n_bufs,
+                         const uint32_t *consts, int n_consts, const uint32_t grid[3],
+                         const uint32_t tpg[3], double *elapsed_us);
+
+/* Replaces GpuRunner::measure (crates/metaltile-std/src/runner.rs:198-231, 413): `warmup`
+ * untimed launches, then `iters` launches whose individual GPU durations (us)
+ * are written to samples_us[iters]. */
+MTQ_API int mtq_measure(const char *kernel_name, int dtype, const mtq_buf *bufs, int n_bufs,
+                        const uint32_t *consts, int n_consts, const uint32_t grid[3],
+                        const uint32_t tpg[3], int warmup, int iters, double *samples_us);
+
+/* 1 if mtq_dispatch knows `kernel_name`, else 0. */
+MTQ_API int mtq_kernel_supported(const char *kernel_name);
+/* Number of names mtq_dispatch knows, and the i-th of them (NULL past the end). */
+MTQ_API int mtq_kernel_count(void);
+MTQ_API const char *mtq_kernel_name(int i);
+
+/* Replaces mt_qmm_for (crates/metaltile-std/src/mlx/quantized.rs:5040-5065): the name of
+ * the reference kernel its selector would pick for M rows. */
+MTQ_API const char *mtq_qmm_for(int dtype, uint32_t m);
+
+/* Replaces GpuRunner::flush_slc (crates/metaltile-std/src/runner.rs:455-475): read-modify-
+ * write a scratch region larger than the last-level cache so the next launch
+ * starts cold. */
+MTQ_API int mtq_flush_cache(void);
+
+/* Timing helper for callers that launch through the typed entry points: the
+ * next launch made by this thread attaches GPU timestamps; mtq_timed_last_us
+ * waits for it and returns its duration. */
+MTQ_API int mtq_timed_begin(void);
+MTQ_API int mtq_timed_last_us(double *elapsed_us);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MTQ_H */

@@ -1,0 +1,89 @@
+"""ctypes binding of libmtq_hip.so (the C-ABI declared in include/mtq.h).
+
+The library is looked up in-tree (metaltile_amd/libmtq_hip.so). If it is
+missing, or no GPU is usable, callers get an exception: there is no fallback
+implementation behind this module.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+from .errors import MtqError
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmtq_hip.so")
+
+
+class MtqBuf(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("bytes", C.c_size_t)]
+
+
+class MtqDeviceInfo(C.Structure):
+    _fields_ = [
+        ("name", C.c_char * 128), ("arch", C.c_char * 32), ("compute_units", C.c_int),
+        ("clock_khz", C.c_int), ("memory_clock_khz", C.c_int), ("memory_bus_bits", C.c_int),
+        ("total_memory", C.c_size_t), ("l2_bytes", C.c_int), ("lds_per_cu_bytes", C.c_int),
+    ]
+
+
+_u32 = C.c_uint32
+_vp = C.c_void_p
+_u32p = C.POINTER(C.c_uint32)
+_dblp = C.POINTER(C.c_double)
+_bufp = C.POINTER(MtqBuf)
+
+# name -> (restype, argtypes); every symbol include/mtq.h declares
+SIGNATURES = {
+    "mtq_init": (C.c_int, [C.c_int]),
+    "mtq_shutdown": (C.c_int, []),
+    "mtq_last_error": (C.c_char_p, []),
+    "mtq_device_name": (C.c_int, [C.c_char_p, C.c_size_t]),
+    "mtq_get_device_info": (C.c_int, [C.POINTER(MtqDeviceInfo)]),
+    "mtq_set_stream": (C.c_int, [_vp]),
+    "mtq_alloc": (C.c_int, [C.c_size_t, C.POINTER(_vp)]),
+    "mtq_free": (C.c_int, [_vp]),
+    "mtq_upload": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "mtq_download": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "mtq_memset": (C.c_int, [_vp, C.c_int, C.c_size_t]),
+    "mtq_sync": (C.c_int, []),
+    "mtq_qmv": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
+    "mtq_qmm": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
+    "mtq_gather_qmv_csr": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32]),
+    "mtq_gather_qmv_indices": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32]),
+    "mtq_gather_qmv_single": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
+    "mtq_dispatch": (C.c_int, [C.c_char_p, C.c_int, _bufp, C.c_int, _u32p, C.c_int, _u32p, _u32p, _dblp]),
+    "mtq_measure": (C.c_int, [C.c_char_p, C.c_int, _bufp, C.c_int, _u32p, C.c_int, _u32p, _u32p, C.c_int, C.c_int, _dblp]),
+    "mtq_kernel_supported": (C.c_int, [C.c_char_p]),
+    "mtq_kernel_count": (C.c_int, []),
+    "mtq_kernel_name": (C.c_char_p, [C.c_int]),
+    "mtq_qmm_for": (C.c_char_p, [C.c_int, _u32]),
+    "mtq_flush_cache": (C.c_int, []),
+    "mtq_timed_begin": (C.c_int, []),
+    "mtq_timed_last_us": (C.c_int, [_dblp]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the shared library and bind every declared symbol."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise MtqError(-1, f"{LIB_PATH} is not built; run `python -m metaltile_amd.build` "
+                           "(there is no fallback implementation)")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        msg = load().mtq_last_error()
+        raise MtqError(rc, msg.decode("utf-8", "replace") if msg else "")

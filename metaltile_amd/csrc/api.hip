@@ -1,0 +1,631 @@
+// C-ABI of libmtq_hip.so (declared in include/mtq.h): device lifetime, buffers,
+// typed entry points, the reference's name-keyed dispatch and its measurement
+// loop. There is deliberately no CPU path in this file: without a GPU every
+// entry point fails with MTQ_ERR_NO_DEVICE.
+#include <hip/hip_ext.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../include/mtq.h"
+#include "mtq_internal.h"
+
+namespace mtq {
+
+static thread_local std::string g_err;
+
+int fail(int code, const std::string& msg) {
+    g_err = msg;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    g_err = std::string(what) + ": " + hipGetErrorString(e);
+    // clear the sticky "last error" so an unrelated later call does not report it
+    (void)hipGetLastError();
+    return e == hipErrorNoDevice || e == hipErrorInvalidDevice ? ERR_NO_DEVICE : ERR_HIP;
+}
+
+hipError_t launch_kernel(const void* fn, dim3 grid, dim3 block, void** args, size_t shmem,
+                         const LaunchCtx& lc) {
+    if (lc.start || lc.stop)
+        return hipExtLaunchKernel(fn, grid, block, args, shmem, lc.stream, lc.start, lc.stop, 0);
+    return hipLaunchKernel(fn, grid, block, args, shmem, lc.stream);
+}
+
+struct State {
+    bool ready = false;
+    int device = -1;
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;  // stream in use (own_stream or the caller's)
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    void* flush_buf = nullptr;
+    size_t flush_bytes = 0;
+    hipDeviceProp_t prop;
+    bool timed_armed = false;    // next typed launch attaches the events
+    bool timed_pending = false;  // events attached, not yet read
+};
+static State g;
+
+static int need_ready() {
+    if (!g.ready) return fail(ERR_NO_DEVICE, "mtq_init has not succeeded (no usable GPU?)");
+    return ERR_OK;
+}
+
+static LaunchCtx make_ctx() {
+    LaunchCtx lc;
+    lc.stream = g.stream;
+    if (g.timed_armed) {
+        lc.start = g.ev_start;
+        lc.stop = g.ev_stop;
+        g.timed_armed = false;
+        g.timed_pending = true;
+    }
+    return lc;
+}
+
+__global__ __launch_bounds__(256) void flush_kernel(uint4* p, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        uint4 v = p[i];
+        v.x += 1u;
+        p[i] = v;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// typed ops (shared by the C entry points and the name-keyed dispatch)
+// ---------------------------------------------------------------------------
+
+static size_t esize(int dt) { return dt == DT_F32 ? 4 : 2; }
+
+static int check_common(int dtype, int bits, uint32_t G, uint32_t N, uint32_t K) {
+    if (dtype != DT_F32 && dtype != DT_F16 && dtype != DT_BF16) return fail(ERR_BAD_ARG, "dtype must be MTQ_F32, MTQ_F16 or MTQ_BF16");
+    if (bits < 2 || bits > 8) return fail(ERR_BAD_ARG, "bits must be in 2..8");
+    if (N == 0 || K == 0) return fail(ERR_SHAPE, "N and K must be non-zero");
+    if (G == 0 || K % G) return fail(ERR_SHAPE, "group_size must be non-zero and divide K");
+    if ((uint64_t)K * bits % 32) return fail(ERR_SHAPE, "K*bits must be a multiple of 32");
+    return ERR_OK;
+}
+
+static int run_gemv(const QmvParams& p, const LaunchCtx& lc) {
+    int rc = launch_qmv_fast(p, lc);
+    if (rc == ERR_UNSUPPORTED) rc = launch_qmv_generic(p, lc);
+    return rc;
+}
+
+static int op_qmv(int dtype, int bits, uint32_t G, const void* w, const void* s, const void* b,
+                  const void* x, void* out, uint32_t M, uint32_t N, uint32_t K, const LaunchCtx& lc) {
+    int rc = check_common(dtype, bits, G, N, K);
+    if (rc) return rc;
+    if (M == 0) return ERR_OK;
+    if (!w || !s || !b || !x || !out) return fail(ERR_BAD_ARG, "null buffer");
+    QmvParams p;
+    p.dtype = dtype; p.bits = bits; p.group_size = G;
+    p.w = w; p.scales = s; p.biases = b; p.x = x; p.out = out;
+    p.M = M; p.N = N; p.K = K;
+    return run_gemv(p, lc);
+}
+
+// Kernel routing by M, the counterpart of mt_qmm_for
+// (crates/metaltile-std/src/mlx/quantized.rs:5040-5065): the MFMA tile kernel from M = 16
+// up, the GEMV family below that.
+static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s, const void* b,
+                  const void* x, void* out, uint32_t M, uint32_t N, uint32_t K, bool force_mma,
+                  const LaunchCtx& lc) {
+    int rc = check_common(dtype, bits, G, N, K);
+    if (rc) return rc;
+    if (M == 0) return ERR_OK;
+    if (!w || !s || !b || !x || !out) return fail(ERR_BAD_ARG, "null buffer");
+    if (M >= 16 || force_mma) {
+        QmmParams q;
+        q.dtype = dtype; q.bits = bits; q.group_size = G;
+        q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
+        q.M = M; q.N = N; q.K = K;
+        rc = launch_qmm_mfma(q, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
+    return op_qmv(dtype, bits, G, w, s, b, x, out, M, N, K, lc);
+}
+
+static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, const void* w,
+                     const void* s, const void* b, const uint32_t* route, void* out, uint32_t T,
+                     uint32_t N, uint32_t K, uint32_t E, const LaunchCtx& lc) {
+    int rc = check_common(dtype, bits, G, N, K);
+    if (rc) return rc;
+    if (E == 0) return fail(ERR_SHAPE, "n_experts must be non-zero");
+    if (mode != GATHER_SINGLE && T == 0) return ERR_OK;
+    if (!w || !s || !b || !x || !out || !route) return fail(ERR_BAD_ARG, "null buffer");
+    QmvParams p;
+    p.dtype = dtype; p.bits = bits; p.group_size = G;
+    p.w = w; p.scales = s; p.biases = b; p.x = x; p.out = out;
+    p.M = 1; p.N = N; p.K = K;
+    p.gather = mode; p.route = route; p.T = mode == GATHER_SINGLE ? 1 : T; p.E = E;
+    return run_gemv(p, lc);
+}
+
+// ---------------------------------------------------------------------------
+// name-keyed dispatch table
+// ---------------------------------------------------------------------------
+
+enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX };
+
+struct KernelDesc {
+    const char* name;
+    Family fam;
+    int bits;
+    int n_bufs;
+    int n_consts;
+};
+
+// Names are the reference kernels' `name` fields; buffer / constexpr order is
+// their signature order (files cited in include/mtq.h).
+static const KernelDesc kTable[] = {
+    // w, scales, biases, x, out | k, gs_per_row
+    {"mt_qmv", F_QMV, 4, 5, 2},
+    {"mt_qmv_int8_fast", F_QMV, 8, 5, 2},
+    // w, scales, biases, x, out | k, n, gs_per_row
+    {"mt_qmm", F_QMM, 4, 5, 3},
+    {"mt_qmm_bm2", F_QMM, 4, 5, 3},
+    {"mt_qmm_bm4", F_QMM, 4, 5, 3},
+    {"mt_qmm_int8_fast", F_QMM, 8, 5, 3},
+    {"mt_qmm_bm2_int8_fast", F_QMM, 8, 5, 3},
+    {"mt_qmm_bm4_int8_fast", F_QMM, 8, 5, 3},
+    {"mt_qmm_mma", F_QMM_MMA, 4, 5, 3},
+    {"mt_qmm_mma_m16", F_QMM_MMA, 4, 5, 3},
+    {"mt_qmm_mma_int8", F_QMM_MMA, 8, 5, 3},
+    {"mt_qmm_mma_m16_int8", F_QMM_MMA, 8, 5, 3},
+    {"mt_qmm_mma_int2", F_QMM_MMA, 2, 5, 3},
+    {"mt_qmm_mma_b3", F_QMM_MMA, 3, 5, 3},
+    {"mt_qmm_mma_b5", F_QMM_MMA, 5, 5, 3},
+    {"mt_qmm_mma_b6", F_QMM_MMA, 6, 5, 3},
+    // w, scales, biases, x, out | k, n, group_size
+    {"mt_qmv_b3", F_QB, 3, 5, 3}, {"mt_qmv_b4", F_QB, 4, 5, 3}, {"mt_qmv_b5", F_QB, 5, 5, 3},
+    {"mt_qmv_b6", F_QB, 6, 5, 3}, {"mt_qmv_b8", F_QB, 8, 5, 3},
+    {"mt_qmm_b3", F_QB, 3, 5, 3}, {"mt_qmm_b4", F_QB, 4, 5, 3}, {"mt_qmm_b5", F_QB, 5, 5, 3},
+    {"mt_qmm_b6", F_QB, 6, 5, 3}, {"mt_qmm_b8", F_QB, 8, 5, 3},
+    // weight, scales, biases, input, output | in_dim, group_size
+    {"dequant_gemv_int2", F_DGEMV, 2, 5, 2}, {"dequant_gemv_int3", F_DGEMV, 3, 5, 2},
+    {"dequant_gemv_int4", F_DGEMV, 4, 5, 2}, {"dequant_gemv_int5", F_DGEMV, 5, 5, 2},
+    {"dequant_gemv_int6", F_DGEMV, 6, 5, 2}, {"dequant_gemv_int8", F_DGEMV, 8, 5, 2},
+    {"dequant_gemv_int4_fast", F_DGEMV, 4, 5, 2},
+    // weights_stacked, scales_stacked, biases_stacked, input, expert_index, output | in_dim, out_dim, group_size
+    {"dequant_gemv_int4_expert_indexed", F_EXPERT, 4, 6, 3},
+    // x, weight_packed, scales, biases, expert_offsets, out | k_in, m_out, n_experts, group_size
+    {"mt_moe_gather_qmm_int4", F_GCSR, 4, 6, 4}, {"mt_moe_gather_qmm_int4_m8", F_GCSR, 4, 6, 4},
+    {"mt_moe_gather_qmm_int4_m16", F_GCSR, 4, 6, 4}, {"mt_moe_gather_qmm_int4_m32", F_GCSR, 4, 6, 4},
+    {"mt_moe_gather_qmm_b3", F_GCSR, 3, 6, 4}, {"mt_moe_gather_qmm_b5", F_GCSR, 5, 6, 4},
+    {"mt_moe_gather_qmm_b6", F_GCSR, 6, 6, 4}, {"mt_moe_gather_qmm_b8", F_GCSR, 8, 6, 4},
+    // x, w, scales, biases, indices, out | m_total, n_out, k_in, group_size
+    {"mt_moe_gather_qmm_mma_int4", F_GIDX, 4, 6, 4}, {"mt_moe_gather_qmm_mma_int4_bm16", F_GIDX, 4, 6, 4},
+    {"mt_moe_gather_qmm_mma_int8", F_GIDX, 8, 6, 4}, {"mt_moe_gather_qmm_mma_b3", F_GIDX, 3, 6, 4},
+    {"mt_moe_gather_qmm_mma_b5", F_GIDX, 5, 6, 4}, {"mt_moe_gather_qmm_mma_b6", F_GIDX, 6, 6, 4},
+    {"mt_moe_gather_qmm_mma_b8", F_GIDX, 8, 6, 4},
+};
+static const int kTableLen = (int)(sizeof(kTable) / sizeof(kTable[0]));
+
+static const KernelDesc* find_kernel(const char* name) {
+    if (!name) return nullptr;
+    for (int i = 0; i < kTableLen; i++)
+        if (!strcmp(kTable[i].name, name)) return &kTable[i];
+    return nullptr;
+}
+
+static int need_bytes(const mtq_buf& b, const char* param, uint64_t expected) {
+    if (!b.ptr && expected) return fail(ERR_BAD_ARG, std::string("buffer '") + param + "' is null");
+    if (b.bytes < expected) {
+        char m[200];
+        snprintf(m, sizeof m, "buffer '%s' too small: expected %llu bytes, got %llu", param,
+                 (unsigned long long)expected, (unsigned long long)b.bytes);
+        return fail(ERR_BUFFER_SIZE, m);
+    }
+    return ERR_OK;
+}
+
+#define MTQ_NEED(buf, name, n)                      \
+    do {                                            \
+        int rc__ = need_bytes(buf, name, n);        \
+        if (rc__) return rc__;                      \
+    } while (0)
+
+// Validates the bound buffers against the shape implied by (name, dtype,
+// constexprs, buffer lengths) and enqueues the kernel.
+static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, int n_bufs,
+                         const uint32_t* consts, int n_consts, const LaunchCtx& lc) {
+    if (dtype != DT_F32 && dtype != DT_F16 && dtype != DT_BF16) return fail(ERR_BAD_ARG, "dtype must be MTQ_F32, MTQ_F16 or MTQ_BF16");
+    if (n_bufs != d.n_bufs || n_consts != d.n_consts || !bufs || !consts) {
+        char m[200];
+        snprintf(m, sizeof m, "%s expects %d buffers and %d constexprs, got %d and %d", d.name,
+                 d.n_bufs, d.n_consts, n_bufs, n_consts);
+        return fail(ERR_BAD_ARG, m);
+    }
+    const uint64_t sz = esize(dtype);
+    const uint64_t bits = (uint64_t)d.bits;
+    switch (d.fam) {
+        case F_QMV:
+        case F_QMM:
+        case F_QMM_MMA:
+        case F_QB: {
+            uint32_t K = consts[0], N, G, M;
+            if (K == 0) return fail(ERR_SHAPE, "k must be non-zero");
+            if (d.fam == F_QMV) {
+                // mt_qmv has no `n` constexpr: N is the length of `out`
+                // (crates/metaltile-std/src/mlx/quantized.rs:8-16).
+                uint32_t gspr = consts[1];
+                if (gspr == 0 || K % gspr) return fail(ERR_SHAPE, "gs_per_row must divide k");
+                G = K / gspr;
+                N = (uint32_t)(bufs[4].bytes / sz);
+                M = 1;
+            } else {
+                N = consts[1];
+                if (d.fam == F_QB) {
+                    G = consts[2];
+                } else {
+                    uint32_t gspr = consts[2];
+                    if (gspr == 0 || K % gspr) return fail(ERR_SHAPE, "gs_per_row must divide k");
+                    G = K / gspr;
+                }
+                M = (uint32_t)(bufs[3].bytes / (K * sz));
+            }
+            if (N == 0) return fail(ERR_SHAPE, "n must be non-zero");
+            if (G == 0 || K % G) return fail(ERR_SHAPE, "group_size must divide k");
+            if (M == 0) return fail(ERR_BUFFER_SIZE, "buffer 'x' holds less than one row");
+            MTQ_NEED(bufs[0], "w", (uint64_t)N * K * bits / 8);
+            MTQ_NEED(bufs[1], "scales", (uint64_t)N * (K / G) * sz);
+            MTQ_NEED(bufs[2], "biases", (uint64_t)N * (K / G) * sz);
+            MTQ_NEED(bufs[3], "x", (uint64_t)M * K * sz);
+            MTQ_NEED(bufs[4], "out", (uint64_t)M * N * sz);
+            if (d.fam == F_QMM_MMA)
+                return op_qmm(dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr,
+                              bufs[4].ptr, M, N, K, true, lc);
+            return op_qmv(dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr,
+                          bufs[4].ptr, M, N, K, lc);
+        }
+        case F_DGEMV: {
+            uint32_t K = consts[0], G = consts[1];
+            uint32_t N = (uint32_t)(bufs[4].bytes / sz);
+            if (K == 0 || N == 0) return fail(ERR_SHAPE, "in_dim and out_dim must be non-zero");
+            if (G == 0 || K % G) return fail(ERR_SHAPE, "group_size must divide in_dim");
+            MTQ_NEED(bufs[0], "weight", (uint64_t)N * K * bits / 8);
+            MTQ_NEED(bufs[1], "scales", (uint64_t)N * (K / G) * sz);
+            MTQ_NEED(bufs[2], "biases", (uint64_t)N * (K / G) * sz);
+            MTQ_NEED(bufs[3], "input", (uint64_t)K * sz);
+            return op_qmv(dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr,
+                          bufs[4].ptr, 1, N, K, lc);
+        }
+        case F_EXPERT: {
+            uint32_t K = consts[0], N = consts[1], G = consts[2];
+            if (K == 0 || N == 0) return fail(ERR_SHAPE, "in_dim and out_dim must be non-zero");
+            if (G == 0 || K % G) return fail(ERR_SHAPE, "group_size must divide in_dim");
+            uint64_t slab = (uint64_t)N * K * bits / 8;
+            uint32_t E = (uint32_t)(bufs[0].bytes / slab);
+            if (E == 0) return fail(ERR_BUFFER_SIZE, "buffer 'weights_stacked' holds less than one expert");
+            MTQ_NEED(bufs[1], "scales_stacked", (uint64_t)E * N * (K / G) * sz);
+            MTQ_NEED(bufs[2], "biases_stacked", (uint64_t)E * N * (K / G) * sz);
+            MTQ_NEED(bufs[3], "input", (uint64_t)K * sz);
+            MTQ_NEED(bufs[4], "expert_index", 4);
+            MTQ_NEED(bufs[5], "output", (uint64_t)N * sz);
+            return op_gather(GATHER_SINGLE, dtype, d.bits, G, bufs[3].ptr, bufs[0].ptr, bufs[1].ptr,
+                             bufs[2].ptr, (const uint32_t*)bufs[4].ptr, bufs[5].ptr, 1, N, K, E, lc);
+        }
+        case F_GCSR: {
+            uint32_t K = consts[0], N = consts[1], E = consts[2], G = consts[3];
+            if (K == 0 || N == 0 || E == 0) return fail(ERR_SHAPE, "k_in, m_out and n_experts must be non-zero");
+            if (G == 0 || K % G) return fail(ERR_SHAPE, "group_size must divide k_in");
+            uint32_t T = (uint32_t)(bufs[0].bytes / (K * sz));
+            MTQ_NEED(bufs[1], "weight_packed", (uint64_t)E * N * K * bits / 8);
+            MTQ_NEED(bufs[2], "scales", (uint64_t)E * N * (K / G) * sz);
+            MTQ_NEED(bufs[3], "biases", (uint64_t)E * N * (K / G) * sz);
+            MTQ_NEED(bufs[4], "expert_offsets", (uint64_t)(E + 1) * 4);
+            MTQ_NEED(bufs[5], "out", (uint64_t)T * N * sz);
+            return op_gather(GATHER_CSR, dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr,
+                             bufs[3].ptr, (const uint32_t*)bufs[4].ptr, bufs[5].ptr, T, N, K, E, lc);
+        }
+        case F_GIDX: {
+            uint32_t T = consts[0], N = consts[1], K = consts[2], G = consts[3];
+            if (K == 0 || N == 0) return fail(ERR_SHAPE, "k_in and n_out must be non-zero");
+            if (G == 0 || K % G) return fail(ERR_SHAPE, "group_size must divide k_in");
+            uint64_t slab = (uint64_t)N * K * bits / 8;
+            uint32_t E = (uint32_t)(bufs[1].bytes / slab);
+            if (E == 0) return fail(ERR_BUFFER_SIZE, "buffer 'w' holds less than one expert");
+            MTQ_NEED(bufs[0], "x", (uint64_t)T * K * sz);
+            MTQ_NEED(bufs[2], "scales", (uint64_t)E * N * (K / G) * sz);
+            MTQ_NEED(bufs[3], "biases", (uint64_t)E * N * (K / G) * sz);
+            MTQ_NEED(bufs[4], "indices", (uint64_t)T * 4);
+            MTQ_NEED(bufs[5], "out", (uint64_t)T * N * sz);
+            return op_gather(GATHER_INDICES, dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr,
+                             bufs[3].ptr, (const uint32_t*)bufs[4].ptr, bufs[5].ptr, T, N, K, E, lc);
+        }
+    }
+    return fail(ERR_UNKNOWN_KERNEL, "unhandled kernel family");
+}
+
+}  // namespace mtq
+
+using namespace mtq;
+
+// ---------------------------------------------------------------------------
+// extern "C"
+// ---------------------------------------------------------------------------
+
+extern "C" {
+
+const char* mtq_last_error(void) { return g_err.c_str(); }
+
+int mtq_init(int device) {
+    if (g.ready && g.device == device) return MTQ_OK;
+    if (g.ready) mtq_shutdown();
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return fail(ERR_NO_DEVICE, "no HIP device available; this library has no CPU fallback");
+    }
+    if (device < 0 || device >= n) return fail(ERR_NO_DEVICE, "device index out of range");
+    MTQ_HIP(hipSetDevice(device));
+    MTQ_HIP(hipGetDeviceProperties(&g.prop, device));
+    if (strncmp(g.prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(ERR_NO_DEVICE, std::string("kernels are built for gfx950 only, device is ") + g.prop.gcnArchName);
+    MTQ_HIP(hipStreamCreateWithFlags(&g.own_stream, hipStreamNonBlocking));
+    MTQ_HIP(hipEventCreate(&g.ev_start));
+    MTQ_HIP(hipEventCreate(&g.ev_stop));
+    g.stream = g.own_stream;
+    g.device = device;
+    g.ready = true;
+    g.timed_armed = g.timed_pending = false;
+    return MTQ_OK;
+}
+
+int mtq_shutdown(void) {
+    if (!g.ready) return MTQ_OK;
+    (void)hipStreamSynchronize(g.stream);
+    if (g.flush_buf) (void)hipFree(g.flush_buf);
+    if (g.ev_start) (void)hipEventDestroy(g.ev_start);
+    if (g.ev_stop) (void)hipEventDestroy(g.ev_stop);
+    if (g.own_stream) (void)hipStreamDestroy(g.own_stream);
+    g = State();
+    return MTQ_OK;
+}
+
+int mtq_device_name(char* out, size_t cap) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (!out || cap == 0) return fail(ERR_BAD_ARG, "null output");
+    snprintf(out, cap, "%s", g.prop.name);
+    return MTQ_OK;
+}
+
+int mtq_get_device_info(mtq_device_info* out) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (!out) return fail(ERR_BAD_ARG, "null output");
+    memset(out, 0, sizeof *out);
+    snprintf(out->name, sizeof out->name, "%s", g.prop.name);
+    snprintf(out->arch, sizeof out->arch, "%s", g.prop.gcnArchName);
+    out->compute_units = g.prop.multiProcessorCount;
+    out->clock_khz = g.prop.clockRate;
+    out->memory_clock_khz = g.prop.memoryClockRate;
+    out->memory_bus_bits = g.prop.memoryBusWidth;
+    out->total_memory = g.prop.totalGlobalMem;
+    out->l2_bytes = g.prop.l2CacheSize;
+    out->lds_per_cu_bytes = (int)g.prop.maxSharedMemoryPerMultiProcessor;
+    return MTQ_OK;
+}
+
+int mtq_set_stream(void* hip_stream) {
+    int rc = need_ready();
+    if (rc) return rc;
+    g.stream = hip_stream ? (hipStream_t)hip_stream : g.own_stream;
+    return MTQ_OK;
+}
+
+int mtq_alloc(size_t bytes, void** dptr) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (!dptr) return fail(ERR_BAD_ARG, "null output");
+    *dptr = nullptr;
+    // sub-4-byte buffers are padded to 4 bytes (reference: single_dispatch.rs:142-152)
+    size_t n = bytes < 4 ? 4 : bytes;
+    MTQ_HIP(hipMalloc(dptr, n));
+    MTQ_HIP(hipMemsetAsync(*dptr, 0, n, g.stream));
+    return MTQ_OK;
+}
+
+int mtq_free(void* dptr) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (!dptr) return MTQ_OK;
+    MTQ_HIP(hipStreamSynchronize(g.stream));
+    MTQ_HIP(hipFree(dptr));
+    return MTQ_OK;
+}
+
+int mtq_upload(void* dptr, const void* host, size_t bytes) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (bytes == 0) return MTQ_OK;
+    if (!dptr || !host) return fail(ERR_BAD_ARG, "null pointer");
+    MTQ_HIP(hipMemcpyAsync(dptr, host, bytes, hipMemcpyHostToDevice, g.stream));
+    MTQ_HIP(hipStreamSynchronize(g.stream));
+    return MTQ_OK;
+}
+
+int mtq_download(void* host, const void* dptr, size_t bytes) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (bytes == 0) return MTQ_OK;
+    if (!dptr || !host) return fail(ERR_BAD_ARG, "null pointer");
+    MTQ_HIP(hipMemcpyAsync(host, dptr, bytes, hipMemcpyDeviceToHost, g.stream));
+    MTQ_HIP(hipStreamSynchronize(g.stream));
+    return MTQ_OK;
+}
+
+int mtq_memset(void* dptr, int byte_value, size_t bytes) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (bytes == 0) return MTQ_OK;
+    if (!dptr) return fail(ERR_BAD_ARG, "null pointer");
+    MTQ_HIP(hipMemsetAsync(dptr, byte_value, bytes, g.stream));
+    return MTQ_OK;
+}
+
+int mtq_sync(void) {
+    int rc = need_ready();
+    if (rc) return rc;
+    MTQ_HIP(hipStreamSynchronize(g.stream));
+    return MTQ_OK;
+}
+
+int mtq_qmv(int dtype, int bits, uint32_t group_size, const void* w, const void* scales,
+            const void* biases, const void* x, void* out, uint32_t M, uint32_t N, uint32_t K) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return op_qmv(dtype, bits, group_size, w, scales, biases, x, out, M, N, K, make_ctx());
+}
+
+int mtq_qmm(int dtype, int bits, uint32_t group_size, const void* w, const void* scales,
+            const void* biases, const void* x, void* out, uint32_t M, uint32_t N, uint32_t K) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return op_qmm(dtype, bits, group_size, w, scales, biases, x, out, M, N, K, false, make_ctx());
+}
+
+int mtq_gather_qmv_csr(int dtype, int bits, uint32_t group_size, const void* x, const void* w,
+                       const void* scales, const void* biases, const uint32_t* expert_offsets,
+                       void* out, uint32_t T, uint32_t N, uint32_t K, uint32_t E) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return op_gather(GATHER_CSR, dtype, bits, group_size, x, w, scales, biases, expert_offsets, out,
+                     T, N, K, E, make_ctx());
+}
+
+int mtq_gather_qmv_indices(int dtype, int bits, uint32_t group_size, const void* x, const void* w,
+                           const void* scales, const void* biases, const uint32_t* indices,
+                           void* out, uint32_t T, uint32_t N, uint32_t K, uint32_t E) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return op_gather(GATHER_INDICES, dtype, bits, group_size, x, w, scales, biases, indices, out, T,
+                     N, K, E, make_ctx());
+}
+
+int mtq_gather_qmv_single(int dtype, int bits, uint32_t group_size, const void* w,
+                          const void* scales, const void* biases, const void* input,
+                          const uint32_t* expert_index, void* output, uint32_t N, uint32_t K,
+                          uint32_t E) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return op_gather(GATHER_SINGLE, dtype, bits, group_size, input, w, scales, biases, expert_index,
+                     output, 1, N, K, E, make_ctx());
+}
+
+int mtq_kernel_supported(const char* kernel_name) { return find_kernel(kernel_name) ? 1 : 0; }
+int mtq_kernel_count(void) { return kTableLen; }
+const char* mtq_kernel_name(int i) { return i >= 0 && i < kTableLen ? kTable[i].name : nullptr; }
+
+const char* mtq_qmm_for(int dtype, uint32_t m) {
+    (void)dtype;  // the reference's choice does not depend on dtype (only its LDS skew does)
+    if (m >= 32 && m % 32 == 0) return "mt_qmm_mma";
+    if (m == 16) return "mt_qmm_mma_m16";
+    if (m >= 4 && m % 4 == 0) return "mt_qmm_bm4";
+    if (m >= 2 && m % 2 == 0) return "mt_qmm_bm2";
+    return "mt_qmm";
+}
+
+int mtq_dispatch(const char* kernel_name, int dtype, const mtq_buf* bufs, int n_bufs,
+                 const uint32_t* consts, int n_consts, const uint32_t grid[3], const uint32_t tpg[3],
+                 double* elapsed_us) {
+    (void)grid;
+    (void)tpg;
+    int rc = need_ready();
+    if (rc) return rc;
+    const KernelDesc* d = find_kernel(kernel_name);
+    if (!d) return fail(ERR_UNKNOWN_KERNEL, std::string("unknown kernel '") + (kernel_name ? kernel_name : "(null)") + "'");
+    LaunchCtx lc;
+    lc.stream = g.stream;
+    lc.start = g.ev_start;
+    lc.stop = g.ev_stop;
+    rc = dispatch_desc(*d, dtype, bufs, n_bufs, consts, n_consts, lc);
+    if (rc) return rc;
+    MTQ_HIP(hipStreamSynchronize(g.stream));
+    if (elapsed_us) {
+        float ms = 0.f;
+        hipError_t e = hipEventElapsedTime(&ms, g.ev_start, g.ev_stop);
+        if (e != hipSuccess) { (void)hipGetLastError(); ms = 0.f; }  // op enqueued no kernel
+        *elapsed_us = (double)ms * 1000.0;
+    }
+    return MTQ_OK;
+}
+
+int mtq_measure(const char* kernel_name, int dtype, const mtq_buf* bufs, int n_bufs,
+                const uint32_t* consts, int n_consts, const uint32_t grid[3], const uint32_t tpg[3],
+                int warmup, int iters, double* samples_us) {
+    (void)grid;
+    (void)tpg;
+    int rc = need_ready();
+    if (rc) return rc;
+    const KernelDesc* d = find_kernel(kernel_name);
+    if (!d) return fail(ERR_UNKNOWN_KERNEL, std::string("unknown kernel '") + (kernel_name ? kernel_name : "(null)") + "'");
+    if (warmup < 0 || iters < 0 || (iters > 0 && !samples_us)) return fail(ERR_BAD_ARG, "bad warmup/iters/samples");
+    LaunchCtx plain;
+    plain.stream = g.stream;
+    for (int i = 0; i < warmup; i++) {
+        rc = dispatch_desc(*d, dtype, bufs, n_bufs, consts, n_consts, plain);
+        if (rc) return rc;
+    }
+    MTQ_HIP(hipStreamSynchronize(g.stream));
+    LaunchCtx timed = plain;
+    timed.start = g.ev_start;
+    timed.stop = g.ev_stop;
+    for (int i = 0; i < iters; i++) {
+        rc = dispatch_desc(*d, dtype, bufs, n_bufs, consts, n_consts, timed);
+        if (rc) return rc;
+        MTQ_HIP(hipEventSynchronize(g.ev_stop));
+        float ms = 0.f;
+        MTQ_HIP(hipEventElapsedTime(&ms, g.ev_start, g.ev_stop));
+        samples_us[i] = (double)ms * 1000.0;
+    }
+    return MTQ_OK;
+}
+
+int mtq_flush_cache(void) {
+    int rc = need_ready();
+    if (rc) return rc;
+    const size_t want = (size_t)768 << 20;  // > 256 MB last-level cache + 8 x 4 MB L2
+    if (!g.flush_buf) {
+        MTQ_HIP(hipMalloc(&g.flush_buf, want));
+        MTQ_HIP(hipMemsetAsync(g.flush_buf, 0, want, g.stream));
+        g.flush_bytes = want;
+    }
+    hipLaunchKernelGGL(flush_kernel, dim3(2048), dim3(256), 0, g.stream, (uint4*)g.flush_buf,
+                       g.flush_bytes / sizeof(uint4));
+    MTQ_HIP(hipGetLastError());
+    MTQ_HIP(hipStreamSynchronize(g.stream));
+    return MTQ_OK;
+}
+
+int mtq_timed_begin(void) {
+    int rc = need_ready();
+    if (rc) return rc;
+    g.timed_armed = true;
+    g.timed_pending = false;
+    return MTQ_OK;
+}
+
+int mtq_timed_last_us(double* elapsed_us) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (!elapsed_us) return fail(ERR_BAD_ARG, "null output");
+    if (!g.timed_pending) return fail(ERR_BAD_ARG, "no timed launch pending (call mtq_timed_begin, then one op)");
+    MTQ_HIP(hipEventSynchronize(g.ev_stop));
+    float ms = 0.f;
+    MTQ_HIP(hipEventElapsedTime(&ms, g.ev_start, g.ev_stop));
+    *elapsed_us = (double)ms * 1000.0;
+    g.timed_pending = false;
+    return MTQ_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,244 @@
+// Device-side building blocks shared by the affine-quantized kernels (gfx950).
+//
+// Packed-weight format (reference: crates/metaltile-std/src/mlx/quantized.rs:5393-5396):
+// codes q in [0, 2^bits) packed LSB-first into little-endian u32 words,
+// row-major [N, K*bits/32]; dequantised weight = scale_g * q + bias_g with
+// g = k / group_size; every load is widened to f32 and all sums are f32.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mtq_types.h"
+
+namespace mtq {
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
+
+template <int DT> struct Elem;
+template <> struct Elem<DT_F32> { typedef float type; };
+template <> struct Elem<DT_F16> { typedef uint16_t type; };
+template <> struct Elem<DT_BF16> { typedef uint16_t type; };
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    uint16_t u = (uint16_t)h;
+    _Float16 f;
+    __builtin_memcpy(&f, &u, 2);
+    return (float)f;
+}
+
+template <int DT> __device__ __forceinline__ float load_elem(const void* p, size_t i) {
+    if constexpr (DT == DT_F32) return ((const float*)p)[i];
+    else if constexpr (DT == DT_F16) return f16_bits_to_f32(((const uint16_t*)p)[i]);
+    else return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+
+// f32 -> element store, round to nearest even (the reference's `.cast::<T>()`
+// on store, crates/metaltile-std/src/mlx/quantized.rs:303-306).
+template <int DT> __device__ __forceinline__ void store_elem(void* p, size_t i, float v) {
+    if constexpr (DT == DT_F32) {
+        ((float*)p)[i] = v;
+    } else if constexpr (DT == DT_F16) {
+        _Float16 h = (_Float16)v;
+        uint16_t u;
+        __builtin_memcpy(&u, &h, 2);
+        ((uint16_t*)p)[i] = u;
+    } else {
+        __bf16 h = (__bf16)v;
+        uint16_t u;
+        __builtin_memcpy(&u, &h, 2);
+        ((uint16_t*)p)[i] = u;
+    }
+}
+
+template <int DT> __device__ __forceinline__ uint16_t f32_to_elem_bits(float v) {
+    uint16_t u;
+    if constexpr (DT == DT_F16) {
+        _Float16 h = (_Float16)v;
+        __builtin_memcpy(&u, &h, 2);
+    } else {
+        __bf16 h = (__bf16)v;
+        __builtin_memcpy(&u, &h, 2);
+    }
+    return u;
+}
+
+// ---- cross-lane sums -------------------------------------------------------
+
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over aligned segments of `seg` lanes (seg a power of two, 1..64); every
+// lane of a segment ends up holding the segment's sum. Lanes exchange with
+// their xor-partners, so the summation order is fixed by the lane layout.
+__device__ __forceinline__ float seg_allreduce(float v, int seg) {
+    if (seg >= 2) v += dpp_f32<0xB1>(v);    // quad_perm [1,0,3,2]
+    if (seg >= 4) v += dpp_f32<0x4E>(v);    // quad_perm [2,3,0,1]
+    if (seg >= 8) v += dpp_f32<0x141>(v);   // row_half_mirror
+    if (seg >= 16) v += dpp_f32<0x140>(v);  // row_mirror
+    if (seg >= 32) v += __shfl_xor(v, 16, 64);
+    if (seg >= 64) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+// ---- x-slice holders and the per-chunk dot ---------------------------------
+//
+// A "chunk" is 16 bytes of packed weights (one dwordx4 load): CPC = 128/bits
+// codes. A thread owns one chunk position of the row and keeps the matching
+// CPC activations in registers for every row it visits.
+//
+// Two arithmetic paths:
+//  * dot2 path (f16/bf16 activations, 2- and 4-bit codes): a masked pair of
+//    codes OR-ed into the mantissa of 2^7 (bf16) or 2^10 (f16) is the pair
+//    (MAGIC+q_a, MAGIC+q_b) in element format; v_dot2_f32_{bf16,f16} multiplies
+//    it with the matching activation pair and accumulates in f32. The MAGIC
+//    offset is folded into the bias: s*(dot - MAGIC*sum_x) + b*sum_x =
+//    s*dot + (b - MAGIC*s)*sum_x.
+//  * cvt path (f32 activations, or 8-bit codes): byte -> f32 convert and an f32
+//    FMA per code.
+
+template <int DT, int BITS> struct PathSel {
+    static constexpr bool kDot2 = (DT != DT_F32) && (BITS == 2 || BITS == 4);
+    static constexpr float kMagic = kDot2 ? (DT == DT_BF16 ? 128.0f : 1024.0f) : 0.0f;
+};
+
+template <int DT> __device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float acc) {
+    if constexpr (DT == DT_BF16) {
+        bf16x2_t av, bv;
+        __builtin_memcpy(&av, &a, 4);
+        __builtin_memcpy(&bv, &b, 4);
+        return __builtin_amdgcn_fdot2_f32_bf16(av, bv, acc, false);
+    } else {
+        half2_t av, bv;
+        __builtin_memcpy(&av, &a, 4);
+        __builtin_memcpy(&bv, &b, 4);
+        return __builtin_amdgcn_fdot2(av, bv, acc, false);
+    }
+}
+
+template <int DT, int BITS, bool DOT2 = PathSel<DT, BITS>::kDot2> struct XSlice;
+
+// dot2 path: activations kept as 16-bit pairs arranged to match the code pairs
+// a single mask extracts from one weight dword.
+template <int DT, int BITS> struct XSlice<DT, BITS, true> {
+    static constexpr int CPC = 128 / BITS;   // codes per 16-byte chunk
+    static constexpr int CPD = 32 / BITS;    // codes per dword
+    uint32_t xp[CPC / 2];
+    float xsum[2];  // sum of the activations of dwords {0,1} and {2,3}
+
+    // The chunk's CPC activations start at element `i0` of `x` (16-byte aligned).
+    __device__ __forceinline__ void load(const void* x, size_t i0) {
+        const uint4* xv = (const uint4*)((const uint16_t*)x + i0);
+        float s01 = 0.f, s23 = 0.f;
+        if constexpr (BITS == 4) {
+#pragma unroll
+            for (int d = 0; d < 4; d++) {  // dword d of the chunk <-> 8 activations
+                uint4 v = xv[d];
+                xp[4 * d + 0] = (v.x & 0xFFFFu) | (v.z << 16);          // (x0,x4)
+                xp[4 * d + 1] = (v.x >> 16) | (v.z & 0xFFFF0000u);      // (x1,x5)
+                xp[4 * d + 2] = (v.y & 0xFFFFu) | (v.w << 16);          // (x2,x6)
+                xp[4 * d + 3] = (v.y >> 16) | (v.w & 0xFFFF0000u);      // (x3,x7)
+                float s = sum8(v);
+                if (d < 2) s01 += s; else s23 += s;
+            }
+        } else {  // BITS == 2: dword d <-> 16 activations, pairs (x_i, x_{i+8})
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                uint4 a = xv[2 * d], b = xv[2 * d + 1];
+                xp[8 * d + 0] = (a.x & 0xFFFFu) | (b.x << 16);
+                xp[8 * d + 1] = (a.x >> 16) | (b.x & 0xFFFF0000u);
+                xp[8 * d + 2] = (a.y & 0xFFFFu) | (b.y << 16);
+                xp[8 * d + 3] = (a.y >> 16) | (b.y & 0xFFFF0000u);
+                xp[8 * d + 4] = (a.z & 0xFFFFu) | (b.z << 16);
+                xp[8 * d + 5] = (a.z >> 16) | (b.z & 0xFFFF0000u);
+                xp[8 * d + 6] = (a.w & 0xFFFFu) | (b.w << 16);
+                xp[8 * d + 7] = (a.w >> 16) | (b.w & 0xFFFF0000u);
+                float s = sum8(a) + sum8(b);
+                if (d < 2) s01 += s; else s23 += s;
+            }
+        }
+        xsum[0] = s01;
+        xsum[1] = s23;
+    }
+    __device__ __forceinline__ void zero() {
+#pragma unroll
+        for (int i = 0; i < CPC / 2; i++) xp[i] = 0;
+        xsum[0] = xsum[1] = 0.f;
+    }
+    static __device__ __forceinline__ float cvt(uint32_t h) {
+        return DT == DT_BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
+    }
+    static __device__ __forceinline__ float sum8(uint4 v) {
+        float s = cvt(v.x & 0xFFFFu) + cvt(v.x >> 16);
+        s += cvt(v.y & 0xFFFFu) + cvt(v.y >> 16);
+        s += cvt(v.z & 0xFFFFu) + cvt(v.z >> 16);
+        s += cvt(v.w & 0xFFFFu) + cvt(v.w >> 16);
+        return s;
+    }
+    // sum over the codes of dword d of (MAGIC + q) * x
+    __device__ __forceinline__ float dot_dword(uint32_t w, int d, float acc) const {
+        constexpr uint32_t kOr = DT == DT_BF16 ? 0x43004300u : 0x64006400u;
+        if constexpr (BITS == 4) {
+            acc = dot2_acc<DT>((w & 0x000F000Fu) | kOr, xp[4 * d + 0], acc);
+            acc = dot2_acc<DT>(((w >> 4) & 0x000F000Fu) | kOr, xp[4 * d + 1], acc);
+            acc = dot2_acc<DT>(((w >> 8) & 0x000F000Fu) | kOr, xp[4 * d + 2], acc);
+            acc = dot2_acc<DT>(((w >> 12) & 0x000F000Fu) | kOr, xp[4 * d + 3], acc);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                acc = dot2_acc<DT>(((w >> (2 * i)) & 0x00030003u) | kOr, xp[8 * d + i], acc);
+        }
+        return acc;
+    }
+};
+
+// cvt path: activations kept as f32.
+template <int DT, int BITS> struct XSlice<DT, BITS, false> {
+    static constexpr int CPC = 128 / BITS;
+    static constexpr int CPD = 32 / BITS;
+    float xf[CPC];
+    float xsum[2];
+
+    __device__ __forceinline__ void load(const void* x, size_t i0) {
+        float s01 = 0.f, s23 = 0.f;
+#pragma unroll
+        for (int i = 0; i < CPC; i++) {
+            xf[i] = load_elem<DT>(x, i0 + i);
+            if (i < CPC / 2) s01 += xf[i]; else s23 += xf[i];
+        }
+        xsum[0] = s01;
+        xsum[1] = s23;
+    }
+    __device__ __forceinline__ void zero() {
+#pragma unroll
+        for (int i = 0; i < CPC; i++) xf[i] = 0.f;
+        xsum[0] = xsum[1] = 0.f;
+    }
+    __device__ __forceinline__ float dot_dword(uint32_t w, int d, float acc) const {
+        const float* x = xf + d * CPD;
+        if constexpr (BITS == 8) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc = fmaf((float)((w >> (8 * j)) & 0xFFu), x[j], acc);
+        } else if constexpr (BITS == 4) {
+            uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                acc = fmaf((float)((lo >> (8 * j)) & 0xFFu), x[2 * j], acc);
+                acc = fmaf((float)((hi >> (8 * j)) & 0xFFu), x[2 * j + 1], acc);
+            }
+        } else {  // BITS == 2: byte j of (w >> 2s) & 0x03030303 is code 4j+s
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                uint32_t m = (w >> (2 * s)) & 0x03030303u;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    acc = fmaf((float)((m >> (8 * j)) & 0xFFu), x[4 * j + s], acc);
+            }
+        }
+        return acc;
+    }
+};
+
+}  // namespace mtq

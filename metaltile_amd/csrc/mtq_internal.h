@@ -1,0 +1,91 @@
+// Host-side declarations shared between the kernel launchers and the C-ABI layer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "mtq_types.h"
+
+namespace mtq {
+
+// Error codes returned across the C-ABI (0 = success).
+enum : int {
+    ERR_OK = 0,
+    ERR_NO_DEVICE = -1,      // no usable GPU / library not initialised
+    ERR_BAD_ARG = -2,        // null pointer, zero size, unsupported dtype/bits
+    ERR_SHAPE = -3,          // shape violates the kernel's preconditions
+    ERR_BUFFER_SIZE = -4,    // a bound buffer is shorter than the op requires
+    ERR_UNKNOWN_KERNEL = -5, // name-keyed dispatch: name not in the table
+    ERR_HIP = -6,            // a HIP runtime call failed
+    ERR_UNSUPPORTED = -7,    // valid request this build has no kernel for
+};
+
+// Sets the calling thread's last-error string and returns `code`.
+int fail(int code, const std::string& msg);
+int hip_fail(hipError_t e, const char* what);
+
+#define MTQ_HIP(call)                                      \
+    do {                                                   \
+        hipError_t e__ = (call);                           \
+        if (e__ != hipSuccess) return ::mtq::hip_fail(e__, #call); \
+    } while (0)
+
+// Optional per-launch timing hooks: when both events are set they are attached
+// to the kernel dispatch itself, so their difference is the kernel's own GPU
+// duration (no launch gap, no host time).
+struct LaunchCtx {
+    hipStream_t stream = nullptr;
+    hipEvent_t start = nullptr;
+    hipEvent_t stop = nullptr;
+};
+
+hipError_t launch_kernel(const void* fn, dim3 grid, dim3 block, void** args, size_t shmem,
+                         const LaunchCtx& lc);
+
+// How the x/out rows of a GEMV-family launch are selected.
+enum GatherMode : int {
+    GATHER_NONE = 0,     // x[M,K] against one weight matrix
+    GATHER_CSR = 1,      // rows sorted by expert, expert_offsets[E+1]
+    GATHER_INDICES = 2,  // indices[T] gives the expert of each row
+    GATHER_SINGLE = 3,   // one row against slab expert_index[0]
+};
+
+struct QmvParams {
+    int dtype = 0;            // DT_F32 / DT_F16 / DT_BF16
+    int bits = 4;             // 2..8
+    uint32_t group_size = 64;
+    const void* w = nullptr;       // u32 [E?][N][K*bits/32]
+    const void* scales = nullptr;  // T   [E?][N][K/G]
+    const void* biases = nullptr;
+    const void* x = nullptr;       // T [M or T][K]
+    void* out = nullptr;           // T [M or T][N]
+    uint32_t M = 1, N = 0, K = 0;
+    int gather = GATHER_NONE;
+    const uint32_t* route = nullptr;  // expert_offsets / indices / expert_index
+    uint32_t T = 0;                   // rows (gather modes)
+    uint32_t E = 1;                   // experts
+};
+
+// Fast LDS/dot2 GEMV family (qmv.hip). Returns ERR_UNSUPPORTED when the shape
+// does not fit its geometry so the caller can fall back to the generic kernel.
+int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc);
+// One-wave-per-output kernel for any bit width 2..8 and any group size (generic.hip).
+int launch_qmv_generic(const QmvParams& p, const LaunchCtx& lc);
+
+struct QmmParams {
+    int dtype = 0;
+    int bits = 4;
+    uint32_t group_size = 64;
+    const void* w = nullptr;
+    const void* scales = nullptr;
+    const void* biases = nullptr;
+    const void* x = nullptr;  // T [M][K]
+    void* out = nullptr;      // T [M][N]
+    uint32_t M = 0, N = 0, K = 0;
+};
+// Tiled MFMA GEMM with weights dequantised into LDS (qmm.hip).
+int launch_qmm_mfma(const QmmParams& p, const LaunchCtx& lc);
+
+}  // namespace mtq

@@ -1,0 +1,59 @@
+"""Typed operator entry points on resident device buffers.
+
+Thin wrappers over mtq_qmv / mtq_qmm / mtq_gather_qmv_* of the C-ABI; argument
+meaning follows the reference kernels they replace (see include/mtq.h). All
+launches are asynchronous on the library stream; `GpuBuffer.read_*` waits.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+from . import _lib
+from .dtypes import DType
+from .runtime import GpuBuffer, _ensure_init
+
+
+def _p(b):
+    return b.ptr if isinstance(b, GpuBuffer) else int(b)
+
+
+def qmv(dtype: DType, bits: int, group_size: int, w, scales, biases, x, out, M: int, N: int, K: int):
+    lib = _ensure_init()
+    _lib.check(lib.mtq_qmv(int(dtype), bits, group_size, _p(w), _p(scales), _p(biases), _p(x), _p(out), M, N, K))
+
+
+def qmm(dtype: DType, bits: int, group_size: int, w, scales, biases, x, out, M: int, N: int, K: int):
+    lib = _ensure_init()
+    _lib.check(lib.mtq_qmm(int(dtype), bits, group_size, _p(w), _p(scales), _p(biases), _p(x), _p(out), M, N, K))
+
+
+def gather_qmv_csr(dtype, bits, group_size, x, w, scales, biases, expert_offsets, out, T, N, K, E):
+    lib = _ensure_init()
+    _lib.check(lib.mtq_gather_qmv_csr(int(dtype), bits, group_size, _p(x), _p(w), _p(scales), _p(biases),
+                                      _p(expert_offsets), _p(out), T, N, K, E))
+
+
+def gather_qmv_indices(dtype, bits, group_size, x, w, scales, biases, indices, out, T, N, K, E):
+    lib = _ensure_init()
+    _lib.check(lib.mtq_gather_qmv_indices(int(dtype), bits, group_size, _p(x), _p(w), _p(scales), _p(biases),
+                                          _p(indices), _p(out), T, N, K, E))
+
+
+def gather_qmv_single(dtype, bits, group_size, w, scales, biases, inp, expert_index, out, N, K, E):
+    lib = _ensure_init()
+    _lib.check(lib.mtq_gather_qmv_single(int(dtype), bits, group_size, _p(w), _p(scales), _p(biases),
+                                         _p(inp), _p(expert_index), _p(out), N, K, E))
+
+
+def timed(fn, *args, **kw) -> float:
+    """Run one op with GPU timestamps attached to its kernel; returns microseconds."""
+    lib = _ensure_init()
+    _lib.check(lib.mtq_timed_begin())
+    fn(*args, **kw)
+    us = C.c_double(0.0)
+    _lib.check(lib.mtq_timed_last_us(C.byref(us)))
+    return us.value
+
+
+def sync():
+    _lib.check(_ensure_init().mtq_sync())

@@ -1,0 +1,61 @@
+"""Binding order of the reference kernels this backend serves.
+
+For each kernel name: tensor parameters in signature order, constexprs in
+signature order, and which parameters are outputs (declared `mut` or named
+out / output, crates/metaltile-macros/src/legacy/sig_parser.rs:43-48,85).
+Sources: crates/metaltile-std/src/mlx/quantized.rs:8-16, 343-352, 4273-4285;
+ffai/dequant_gemv.rs:52-62; ffai/dequant_gemv_expert_indexed.rs:58-68;
+ffai/moe.rs:358-370, 2256-2268.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Tuple
+
+
+@dataclass(frozen=True)
+class KernelSignature:
+    name: str
+    bits: int
+    params: Tuple[str, ...]
+    constexprs: Tuple[str, ...]
+    outputs: Tuple[str, ...]
+
+
+_QM = ("w", "scales", "biases", "x", "out")
+_DG = ("weight", "scales", "biases", "input", "output")
+_EX = ("weights_stacked", "scales_stacked", "biases_stacked", "input", "expert_index", "output")
+_GC = ("x", "weight_packed", "scales", "biases", "expert_offsets", "out")
+_GI = ("x", "w", "scales", "biases", "indices", "out")
+
+KERNEL_SIGNATURES: Dict[str, KernelSignature] = {}
+
+
+def _add(name, bits, params, consts, outs):
+    KERNEL_SIGNATURES[name] = KernelSignature(name, bits, params, consts, outs)
+
+
+for _n, _b in (("mt_qmv", 4), ("mt_qmv_int8_fast", 8)):
+    _add(_n, _b, _QM, ("k", "gs_per_row"), ("out",))
+for _n, _b in (("mt_qmm", 4), ("mt_qmm_bm2", 4), ("mt_qmm_bm4", 4), ("mt_qmm_int8_fast", 8),
+               ("mt_qmm_bm2_int8_fast", 8), ("mt_qmm_bm4_int8_fast", 8), ("mt_qmm_mma", 4),
+               ("mt_qmm_mma_m16", 4), ("mt_qmm_mma_int8", 8), ("mt_qmm_mma_m16_int8", 8),
+               ("mt_qmm_mma_int2", 2), ("mt_qmm_mma_b3", 3), ("mt_qmm_mma_b5", 5), ("mt_qmm_mma_b6", 6)):
+    _add(_n, _b, _QM, ("k", "n", "gs_per_row"), ("out",))
+for _b in (3, 4, 5, 6, 8):
+    _add(f"mt_qmv_b{_b}", _b, _QM, ("k", "n", "group_size"), ("out",))
+    _add(f"mt_qmm_b{_b}", _b, _QM, ("k", "n", "group_size"), ("out",))
+for _b in (2, 3, 4, 5, 6, 8):
+    _add(f"dequant_gemv_int{_b}", _b, _DG, ("in_dim", "group_size"), ("output",))
+_add("dequant_gemv_int4_fast", 4, _DG, ("in_dim", "group_size"), ("output",))
+_add("dequant_gemv_int4_expert_indexed", 4, _EX, ("in_dim", "out_dim", "group_size"), ("output",))
+for _n, _b in (("mt_moe_gather_qmm_int4", 4), ("mt_moe_gather_qmm_int4_m8", 4),
+               ("mt_moe_gather_qmm_int4_m16", 4), ("mt_moe_gather_qmm_int4_m32", 4),
+               ("mt_moe_gather_qmm_b3", 3), ("mt_moe_gather_qmm_b5", 5), ("mt_moe_gather_qmm_b6", 6),
+               ("mt_moe_gather_qmm_b8", 8)):
+    _add(_n, _b, _GC, ("k_in", "m_out", "n_experts", "group_size"), ("out",))
+for _n, _b in (("mt_moe_gather_qmm_mma_int4", 4), ("mt_moe_gather_qmm_mma_int4_bm16", 4),
+               ("mt_moe_gather_qmm_mma_int8", 8), ("mt_moe_gather_qmm_mma_b3", 3),
+               ("mt_moe_gather_qmm_mma_b5", 5), ("mt_moe_gather_qmm_mma_b6", 6),
+               ("mt_moe_gather_qmm_mma_b8", 8)):
+    _add(_n, _b, _GI, ("m_total", "n_out", "k_in", "group_size"), ("out",))

@@ -1,0 +1,131 @@
+"""CPU-only checks of the host layer: selector, stats, packers, and that the
+C-ABI library loads and exports every symbol include/mtq.h declares."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import metaltile_amd as m
+from metaltile_amd import DType, _lib
+from metaltile_amd.signatures import KERNEL_SIGNATURES
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _have_gpu() -> bool:
+    return _lib.load().mtq_init(0) == 0
+
+
+# ---- selector: crates/metaltile-std/src/mlx/quantized.rs:5128-5199 ----------
+
+@pytest.mark.parametrize("impl", ["python", "c"])
+def test_selector_routes_like_reference(impl):
+    lib = _lib.load()
+    pick = (lambda dt, mm: m.mt_qmm_for(dt, mm)) if impl == "python" else \
+        (lambda dt, mm: lib.mtq_qmm_for(int(dt), mm).decode())
+    for mm in (32, 64, 96, 128):
+        assert pick(DType.F32, mm) == "mt_qmm_mma"
+    assert pick(DType.F32, 16) == "mt_qmm_mma_m16"
+    for mm in (4, 8, 12, 20, 24, 28, 36, 60):
+        assert pick(DType.F32, mm) == "mt_qmm_bm4"
+    for mm in (2, 6, 10, 14, 18, 22, 26, 30):
+        assert pick(DType.F32, mm) == "mt_qmm_bm2"
+    for mm in (1, 3, 5, 7, 9, 15, 31):
+        assert pick(DType.F32, mm) == "mt_qmm"
+    for dt in (DType.F32, DType.F16):
+        assert pick(dt, 8) == "mt_qmm_bm4"
+
+
+# ---- stats: crates/metaltile-std/src/stats.rs:57-84 --------------------------
+
+def test_bench_stats_reference_cases():
+    st = m.BenchStats.from_samples([1.0, 2.0, 3.0, 4.0, 10.0])
+    assert (st.min_us, st.median_us, st.p95_us, st.p99_us) == (1.0, 3.0, 10.0, 10.0)
+    assert st.stddev_us > 0.0
+    slow = m.BenchStats.from_samples([250.0] * 5 + [120.0] * 5)
+    fast = m.BenchStats.from_samples([250.0] * 4 + [120.0] * 6)
+    assert slow.median_us - fast.median_us >= 100.0
+    assert slow.min_us == 120.0 and fast.min_us == 120.0
+    with pytest.raises(ValueError):
+        m.BenchStats.from_samples([])
+
+
+def test_throughput_uses_min_sample():
+    st = m.BenchStats.from_samples([10.0, 5.0, 20.0])
+    assert m.to_gbps(st, 5e3) == pytest.approx(1.0)        # 5000 B / 5 us = 1 GB/s
+    assert m.to_gflops(st, 1e4) == pytest.approx(2.0)
+
+
+# ---- packers: crates/metaltile-std/src/utils.rs:72-127 -----------------------
+
+def test_pack_f32_reference_unit_values():
+    assert m.unpack_f32(m.pack_f32([0.0, 1.5, -2.25, 1024.0], DType.F32), DType.F32).tolist() == [0.0, 1.5, -2.25, 1024.0]
+    assert m.unpack_f32(m.pack_f32([0.0, 0.5, -0.5, 2.0], DType.F16), DType.F16).tolist() == [0.0, 0.5, -0.5, 2.0]
+    assert m.unpack_f32(m.pack_f32([1.0, 2.0, -0.5, 0.0], DType.BF16), DType.BF16).tolist() == [1.0, 2.0, -0.5, 0.0]
+    r = m.unpack_f32(m.pack_f32([0.1], DType.F16), DType.F16)[0]
+    assert abs(r - 0.1) < 1e-3 and r != np.float32(0.1)
+    for dt in (DType.F32, DType.F16, DType.BF16):
+        assert m.pack_f32([], dt) == b"" and m.unpack_f32(b"", dt).size == 0
+    assert m.unpack_f32(bytes([0, 0, 128, 63, 7]), DType.F32).tolist() == [1.0]
+    assert m.pack_f32([1.0], DType.U32) == (1).to_bytes(4, "little")
+    assert [len(m.pack_f32([1.0], dt)) for dt in (DType.F32, DType.F16, DType.BF16)] == [4, 2, 2]
+
+
+def test_pack_codes_matches_oracle_layout(oracle):
+    from metaltile_amd.synth import pack_codes
+    rng = np.random.default_rng(3)
+    for bits in (2, 3, 4, 5, 6, 8):
+        codes = rng.integers(0, 1 << bits, size=(7, 96), dtype=np.uint8)
+        assert np.array_equal(pack_codes(codes, bits), oracle.pack_codes(codes, bits))
+
+
+# ---- C-ABI surface -----------------------------------------------------------
+
+def _header_symbols():
+    text = open(os.path.join(ROOT, "include", "mtq.h")).read()
+    return re.findall(r"MTQ_API\s+[\w\s\*]+?\b(mtq_\w+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    names = _header_symbols()
+    assert len(names) >= 25
+    lib = C.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/mtq.h but not exported"
+    assert sorted(names) == sorted(_lib.SIGNATURES)
+
+
+def test_kernel_table_matches_python_signatures():
+    lib = _lib.load()
+    c_names = [lib.mtq_kernel_name(i).decode() for i in range(lib.mtq_kernel_count())]
+    assert sorted(c_names) == sorted(KERNEL_SIGNATURES)
+    assert lib.mtq_kernel_name(lib.mtq_kernel_count()) is None
+    assert lib.mtq_kernel_supported(b"mt_qmv") == 1 and lib.mtq_kernel_supported(b"mt_gemm") == 0
+    # names the reference registers for this path (tests + benches)
+    for n in ("mt_qmv", "mt_qmm", "mt_qmm_mma", "dequant_gemv_int2", "dequant_gemv_int4_expert_indexed",
+              "mt_moe_gather_qmm_int4_m8", "mt_moe_gather_qmm_mma_int4"):
+        assert n in c_names
+
+
+def test_no_gpu_means_error_not_fallback():
+    if _have_gpu():
+        pytest.skip("a GPU is present; the no-device path cannot be observed")
+    lib = _lib.load()
+    assert lib.mtq_init(0) == -1
+    assert b"no CPU fallback" in lib.mtq_last_error() or b"HIP device" in lib.mtq_last_error()
+    assert lib.mtq_qmv(0, 4, 64, None, None, None, None, None, 1, 8, 512) == -1
+    assert lib.mtq_sync() == -1
+    with pytest.raises(m.MtqError) as ei:
+        m.Context(0)
+    assert ei.value.code == -1
+
+
+def test_product_never_touches_the_oracle():
+    pkg = os.path.join(ROOT, "metaltile_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp", ".hpp")):
+                text = open(os.path.join(dirpath, f), errors="replace").read()
+                assert "oracle" not in text.lower(), f"{f} mentions the oracle"

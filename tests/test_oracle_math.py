@@ -1,0 +1,208 @@
+"""Pins the oracle's arithmetic: extraction, qmm/gemv, gather, quantise, stats.
+
+Nothing here retypes the oracle's formula: checks are a library f64 matmul on
+an independently unpacked matrix, closed forms, brute force on tiny inputs and
+identities the reference's own tests rely on.
+"""
+import numpy as np
+import pytest
+
+F32, F16, BF16 = 0, 1, 2
+
+
+def _rand_case(rng, n, k, bits, g, m):
+    codes = rng.integers(0, 1 << bits, size=(n, k), dtype=np.uint8)
+    s = (0.02 * np.abs(rng.standard_normal(n * (k // g))) + 1e-3).astype(np.float32)
+    b = (-(1 << (bits - 1)) * s + rng.standard_normal(s.size).astype(np.float32) * 1e-3).astype(np.float32)
+    x = rng.standard_normal(m * k).astype(np.float32)
+    return codes, s, b, x
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
+def test_extraction_brute_force_and_round_trip(oracle, bits):
+    rng = np.random.default_rng(bits)
+    n, k = 5, 64
+    codes = rng.integers(0, 1 << bits, size=(n, k), dtype=np.uint8)
+    w = oracle.pack_codes(codes, bits)
+    assert w.size == n * k * bits // 32
+    # pure-Python reader of the format definition: bit string, LSB first
+    for r in range(n):
+        words = w[r * (k * bits // 32):(r + 1) * (k * bits // 32)]
+        big = sum(int(v) << (32 * i) for i, v in enumerate(words))
+        for j in range(k):
+            assert (big >> (j * bits)) & ((1 << bits) - 1) == codes[r, j]
+    assert np.array_equal(oracle.unpack_codes(w, n, k, bits), codes)
+    assert np.array_equal(oracle.np_unpack_codes(w, n, k, bits), codes)
+
+
+def test_synth_packed_w_closed_form(oracle):
+    # quantized.rs:5355-5369: slot s of pack p holds (p*2654435761 + s) & mask
+    for bits in (2, 4, 8):
+        n, k = 3, 64
+        w = oracle.synth_packed_w(n, k, bits)
+        pf = 32 // bits
+        codes = oracle.np_unpack_codes(w, n, k, bits).reshape(-1)
+        for idx in (0, 1, pf - 1, pf, 5 * pf + 3, codes.size - 1):
+            p, s = divmod(idx, pf)
+            assert codes[idx] == ((p * 2654435761 + s) & 0xFFFFFFFF) & ((1 << bits) - 1)
+
+
+def test_synth_bitstream_matches_packed_layout_for_pow2(oracle):
+    # the bit-stream layout and the pack-aligned layout coincide for 2/4/8 bits
+    for bits in (2, 4, 8):
+        w = oracle.synth_bitstream_w(4, 64, bits)
+        codes = oracle.np_unpack_codes(w, 4, 64, bits)
+        for row, d in ((0, 0), (1, 7), (3, 63)):
+            want = (((row * 64 + d) * 2654435761 + d) & 0xFFFFFFFF) & ((1 << bits) - 1)
+            assert codes[row, d] == want
+
+
+@pytest.mark.parametrize("bits,g", [(2, 32), (2, 64), (3, 32), (4, 32), (4, 64), (4, 128), (5, 32), (6, 32), (8, 64), (8, 128)])
+def test_qmm_against_numpy_f64_matmul(oracle, bits, g):
+    rng = np.random.default_rng(100 + bits * 7 + g)
+    m, n, k = 3, 24, 256
+    codes, s, b, x = _rand_case(rng, n, k, bits, g, m)
+    w = oracle.pack_codes(codes, bits)
+    ref = oracle.np_qmm_f64(w, s, b, x, m, n, k, bits, g).reshape(-1)
+    got64 = oracle.qmm_f64(w, s, b, x, m, n, k, bits, g)
+    got32 = oracle.qmm(w, s, b, x, m, n, k, bits, g)
+    # the f64 oracle sums the same f32 weights as the library matmul: ~1e-13 apart
+    assert np.max(np.abs(got64 - ref)) < 1e-9
+    # sequential f32 accumulation over 256 terms of |.|~1: a few 1e-5
+    assert np.max(np.abs(got32 - ref)) < 2e-4
+    # a transposed operand, a dropped bias or a wrong group would be O(1) off
+    assert np.max(np.abs(ref)) > 0.5
+
+
+def test_qmm_closed_forms(oracle):
+    n, k, g, m = 6, 128, 32, 2
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(m * k).astype(np.float32)
+    s = (rng.random(n * k // g) + 0.5).astype(np.float32)
+    b = rng.standard_normal(n * k // g).astype(np.float32)
+    xg = x.reshape(m, k // g, g).astype(np.float64).sum(axis=2)            # [m, groups]
+    # all codes zero -> y = sum_g b_g * sum_{k in g} x_k
+    w0 = oracle.pack_codes(np.zeros((n, k), np.uint8), 4)
+    want = xg @ b.reshape(n, k // g).astype(np.float64).T
+    assert np.max(np.abs(oracle.qmm_f64(w0, s, b, x, m, n, k, 4, g).reshape(m, n) - want)) < 1e-9
+    # scale 1, bias 0, constant code c -> y = c * sum(x)
+    for bits, c in ((2, 3), (4, 9), (8, 200)):
+        wc = oracle.pack_codes(np.full((n, k), c, np.uint8), bits)
+        ones, zeros = np.ones(n * k // g, np.float32), np.zeros(n * k // g, np.float32)
+        y = oracle.qmm_f64(wc, ones, zeros, x, m, n, k, bits, g).reshape(m, n)
+        assert np.max(np.abs(y - c * x.reshape(m, k).astype(np.float64).sum(axis=1, keepdims=True))) < 1e-9
+
+
+def test_qmm_linearity_and_m1_equals_qmv(oracle):
+    rng = np.random.default_rng(9)
+    n, k, g, bits = 16, 256, 64, 4
+    codes, s, b, x = _rand_case(rng, n, k, bits, g, 2)
+    w = oracle.pack_codes(codes, bits)
+    x1, x2 = x[:k], x[k:]
+    y1 = oracle.qmm_f64(w, s, b, x1, 1, n, k, bits, g)
+    y2 = oracle.qmm_f64(w, s, b, x2, 1, n, k, bits, g)
+    y12 = oracle.qmm_f64(w, s, b, (2.0 * x1 - 0.5 * x2).astype(np.float32), 1, n, k, bits, g)
+    assert np.max(np.abs(y12 - (2.0 * y1 - 0.5 * y2))) < 1e-5
+    # rows of an M=2 qmm are the two qmv results, bit for bit (tests/qmm_gpu_correctness.rs:341)
+    both = oracle.qmm(w, s, b, x, 2, n, k, bits, g).reshape(2, n)
+    assert np.array_equal(both[0], oracle.qmm(w, s, b, x1, 1, n, k, bits, g))
+    assert np.array_equal(both[1], oracle.qmm(w, s, b, x2, 1, n, k, bits, g))
+
+
+def test_split_form_equals_direct_form(oracle):
+    # cpu_qmm_reference (tests/qmm_gpu_correctness.rs:73-108) vs qmm_oracle: same sum, f32 rounding apart
+    from tests.ref_setups import legacy_qmm_inputs
+    from metaltile_amd import DType
+    m, n, k = 8, 16, 512
+    w, s, b, x, g = legacy_qmm_inputs(m, n, k, DType.F32)
+    direct = oracle.qmm(w, s, b, x, m, n, k, 4, g)
+    split = oracle.qmm_split(w, s, b, x, m, n, k, 4, g)
+    ref = oracle.np_qmm_f64(w, s, b, x, m, n, k, 4, g).reshape(-1)
+    assert np.max(np.abs(direct - ref) / np.maximum(np.abs(ref), 1.0)) < 1e-5
+    assert np.max(np.abs(split - ref) / np.maximum(np.abs(ref), 1.0)) < 1e-5
+    assert ref.min() > 100.0  # the legacy inputs give large positive sums
+
+
+def test_mma_variant_rounds_weights(oracle):
+    rng = np.random.default_rng(21)
+    m, n, k, g, bits = 4, 8, 128, 64, 4
+    codes, s, b, x = _rand_case(rng, n, k, bits, g, m)
+    w = oracle.pack_codes(codes, bits)
+    for dt in (F16, BF16):
+        wd = oracle.round_through(oracle.np_dequant(w, s, b, n, k, bits, g).reshape(-1), dt).reshape(n, k)
+        want = x.reshape(m, k).astype(np.float64) @ wd.astype(np.float64).T
+        got = oracle.qmm_mma(w, s, b, x, m, n, k, bits, g, dt).reshape(m, n)
+        assert np.max(np.abs(got - want)) < 1e-9
+    exact = oracle.qmm_f64(w, s, b, x, m, n, k, bits, g)
+    assert np.max(np.abs(oracle.qmm_mma(w, s, b, x, m, n, k, bits, g, F32) - exact)) < 1e-12
+
+
+def test_csr_expert_resolution(oracle):
+    # moe.rs:376-385: first e with t < off[e+1], default 0
+    off = [0, 2, 5, 6]
+    assert [oracle.csr_expert(off, 3, t) for t in range(8)] == [0, 0, 1, 1, 1, 2, 0, 0]
+    assert [oracle.csr_expert([0, 0, 3, 3], 3, t) for t in range(4)] == [1, 1, 1, 0]
+
+
+def test_gather_identities(oracle):
+    rng = np.random.default_rng(33)
+    E, N, K, g, bits, T = 4, 12, 128, 32, 4, 9
+    codes = rng.integers(0, 16, size=(E * N, K), dtype=np.uint8)
+    w = oracle.pack_codes(codes, bits)
+    s = (0.02 * np.abs(rng.standard_normal(E * N * K // g)) + 1e-3).astype(np.float32)
+    b = (-8 * s).astype(np.float32)
+    x = rng.standard_normal(T * K).astype(np.float32)
+    off = np.array([0, 3, 3, 7, 9], dtype=np.uint32)
+    idx = np.array([0, 0, 0, 2, 2, 2, 2, 3, 3], dtype=np.uint32)
+    y_csr = oracle.gather_qmm(x, w, s, b, T, K, N, E, bits, g, expert_offsets=off).reshape(T, N)
+    y_idx = oracle.gather_qmm(x, w, s, b, T, K, N, E, bits, g, indices=idx).reshape(T, N)
+    assert np.array_equal(y_csr, y_idx)                      # CSR == indices after expansion
+    wpe, spe = N * K * bits // 32, N * K // g
+    for t in range(T):                                       # each row == plain qmv on its slab
+        e = int(idx[t])
+        want = oracle.qmm(w[e * wpe:(e + 1) * wpe], s[e * spe:(e + 1) * spe], b[e * spe:(e + 1) * spe],
+                          x[t * K:(t + 1) * K], 1, N, K, bits, g)
+        assert np.array_equal(y_idx[t], want)
+    perm = rng.permutation(T)                                # permuting rows permutes outputs
+    y_perm = oracle.gather_qmm(x.reshape(T, K)[perm].ravel(), w, s, b, T, K, N, E, bits, g,
+                               indices=idx[perm]).reshape(T, N)
+    assert np.array_equal(y_perm, y_idx[perm])
+    # expert-indexed(e) == row of the gather with that expert (dequant_gemv_expert_indexed.rs:47-53)
+    e = 2
+    y_e = oracle.expert_indexed(w, s, b, x[:K], e, N, K, g)
+    assert np.array_equal(y_e, oracle.gather_qmm(x[:K], w, s, b, 1, K, N, E, bits, g,
+                                                 indices=np.array([e], np.uint32)))
+    # f64 variant agrees with numpy on the slab
+    y64 = oracle.gather_qmm(x, w, s, b, T, K, N, E, bits, g, indices=idx, f64=True).reshape(T, N)
+    ref = oracle.np_qmm_f64(w[2 * wpe:3 * wpe], s[2 * spe:3 * spe], b[2 * spe:3 * spe], x[3 * K:4 * K], 1, N, K, bits, g)
+    assert np.max(np.abs(y64[3] - ref.reshape(-1))) < 1e-9
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
+def test_affine_quantize_round_trip(oracle, bits):
+    # quantized.rs:5283-5284 ramp; round trip within one step (affine_int2_gpu_correctness.rs:134-144)
+    g = 64 if bits in (2, 4, 8) else 32
+    n_groups = 8
+    i = np.arange(n_groups * g)
+    v = (((i % 37).astype(np.float32) - 18.0) * np.float32(0.05)).astype(np.float32)
+    codes, s, b = oracle.affine_quantize(v, g, bits, F32)
+    grp = v.reshape(n_groups, g)
+    assert np.allclose(b, grp.min(axis=1)) and np.allclose(s, (grp.max(axis=1) - grp.min(axis=1)) / ((1 << bits) - 1))
+    assert codes.max() <= (1 << bits) - 1
+    w = oracle.pack_codes(codes.reshape(1, -1), bits)
+    back = oracle.affine_dequantize(w, s, b, v.size, g, bits)
+    assert np.max(np.abs(back - v) / np.repeat(s, g)) <= 0.5 + 1e-4
+    # constant group -> scale 1, bias = the constant, all codes 0
+    c, s1, b1 = oracle.affine_quantize(np.full(g, 0.25, np.float32), g, bits, F32)
+    assert s1[0] == 1.0 and b1[0] == 0.25 and not c.any()
+
+
+def test_bench_stats_reference_values(oracle):
+    # stats.rs:57-84
+    st = oracle.bench_stats([1.0, 2.0, 3.0, 4.0, 10.0])
+    assert (st["min_us"], st["median_us"], st["p95_us"], st["p99_us"]) == (1.0, 3.0, 10.0, 10.0)
+    assert st["stddev_us"] > 0
+    slow = oracle.bench_stats([250.0] * 5 + [120.0] * 5)
+    fast = oracle.bench_stats([250.0] * 4 + [120.0] * 6)
+    assert slow["median_us"] - fast["median_us"] >= 100.0 and slow["min_us"] == fast["min_us"] == 120.0
+    assert abs(st["mean_us"] - 4.0) < 1e-12 and abs(st["stddev_us"] - np.std([1, 2, 3, 4, 10])) < 1e-12
