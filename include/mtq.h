@@ -177,6 +177,35 @@ MTQ_API int mtq_measure(const char *kernel_name, int dtype, const mtq_buf *bufs,
                         const uint32_t *consts, int n_consts, const uint32_t grid[3],
                         const uint32_t tpg[3], int warmup, int iters, double *samples_us);
 
+/* One entry of a dispatch chain: the arguments of mtq_dispatch minus grid/tpg. */
+typedef struct mtq_dispatch_spec {
+    const char *kernel_name;
+    int dtype;
+    const mtq_buf *bufs;
+    int n_bufs;
+    const uint32_t *consts;
+    int n_consts;
+} mtq_dispatch_spec;
+
+/* Replaces Context::dispatch_chain over resident buffers
+ * (crates/metaltile-runtime/src/context.rs:363-401; used with upload_resident by the
+ * reference's perf tests, crates/metaltile-std/tests/qmm_gpu_correctness.rs:587-621):
+ * enqueue the `n` dispatches in order, `repeat` times over, with no host wait
+ * in between, then wait for the last. per_kernel_us (NULL or n*repeat entries)
+ * receives each dispatch's own GPU duration; wall_us (may be NULL) the host
+ * clock from the first enqueue to completion of the last; stream_us (may be
+ * NULL) the time between two events recorded on the stream before the first
+ * and after the last dispatch. Attaching per-kernel events costs host time per
+ * launch, so ask for per_kernel_us and for the bracketing times in separate calls. */
+MTQ_API int mtq_dispatch_chain(const mtq_dispatch_spec *specs, int n, int repeat,
+                               double *per_kernel_us, double *wall_us, double *stream_us);
+
+/* Plain device-to-device copy kernel of `bytes` (a multiple of 16), enqueued
+ * `repeat` times; avg_us (may be NULL) receives the mean GPU duration. No
+ * counterpart in the reference: it is the known-size kernel hardware-counter
+ * readings are calibrated against. */
+MTQ_API int mtq_copy_kernel(void *dst, const void *src, size_t bytes, int repeat, double *avg_us);
+
 /* 1 if mtq_dispatch knows `kernel_name`, else 0. */
 MTQ_API int mtq_kernel_supported(const char *kernel_name);
 /* Number of names mtq_dispatch knows, and the i-th of them (NULL past the end). */
@@ -191,6 +220,14 @@ MTQ_API const char *mtq_qmm_for(int dtype, uint32_t m);
  * write a scratch region larger than the last-level cache so the next launch
  * starts cold. */
 MTQ_API int mtq_flush_cache(void);
+
+/* Tuning knobs (no counterpart in the reference). Known names:
+ *   "qmv.kernel"           0 = choose per shape (default), 1 = one-shot kernel, 2 = streaming kernel
+ *   "qmv.rows_per_thread"  one-shot kernel: 0 = choose per shape, or 4 / 7 / 8
+ *   "qmv.stream_depth"     streaming kernel: 0 = choose per shape, or 4 / 8 loads in flight per thread
+ *   "qmv.stream_batches"   streaming kernel: 0 = choose per shape, or 1..16 batches per thread
+ * Unknown names or values fail with MTQ_ERR_BAD_ARG. */
+MTQ_API int mtq_set_option(const char *name, int value);
 
 /* Timing helper for callers that launch through the typed entry points: the
  * next launch made by this thread attaches GPU timestamps; mtq_timed_last_us

@@ -19,6 +19,11 @@ class MtqBuf(C.Structure):
     _fields_ = [("ptr", C.c_void_p), ("bytes", C.c_size_t)]
 
 
+class MtqDispatchSpec(C.Structure):
+    _fields_ = [("kernel_name", C.c_char_p), ("dtype", C.c_int), ("bufs", C.POINTER(MtqBuf)),
+                ("n_bufs", C.c_int), ("consts", C.POINTER(C.c_uint32)), ("n_consts", C.c_int)]
+
+
 class MtqDeviceInfo(C.Structure):
     _fields_ = [
         ("name", C.c_char * 128), ("arch", C.c_char * 32), ("compute_units", C.c_int),
@@ -54,11 +59,14 @@ SIGNATURES = {
     "mtq_gather_qmv_single": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "mtq_dispatch": (C.c_int, [C.c_char_p, C.c_int, _bufp, C.c_int, _u32p, C.c_int, _u32p, _u32p, _dblp]),
     "mtq_measure": (C.c_int, [C.c_char_p, C.c_int, _bufp, C.c_int, _u32p, C.c_int, _u32p, _u32p, C.c_int, C.c_int, _dblp]),
+    "mtq_dispatch_chain": (C.c_int, [C.POINTER(MtqDispatchSpec), C.c_int, C.c_int, _dblp, _dblp, _dblp]),
+    "mtq_copy_kernel": (C.c_int, [_vp, _vp, C.c_size_t, C.c_int, _dblp]),
     "mtq_kernel_supported": (C.c_int, [C.c_char_p]),
     "mtq_kernel_count": (C.c_int, []),
     "mtq_kernel_name": (C.c_char_p, [C.c_int]),
     "mtq_qmm_for": (C.c_char_p, [C.c_int, _u32]),
     "mtq_flush_cache": (C.c_int, []),
+    "mtq_set_option": (C.c_int, [C.c_char_p, C.c_int]),
     "mtq_timed_begin": (C.c_int, []),
     "mtq_timed_last_us": (C.c_int, [_dblp]),
 }

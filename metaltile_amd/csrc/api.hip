@@ -5,6 +5,8 @@
 #include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
+#include <time.h>
+
 #include <cstdio>
 #include <cstring>
 #include <string>
@@ -34,6 +36,11 @@ hipError_t launch_kernel(const void* fn, dim3 grid, dim3 block, void** args, siz
     if (lc.start || lc.stop)
         return hipExtLaunchKernel(fn, grid, block, args, shmem, lc.stream, lc.start, lc.stop, 0);
     return hipLaunchKernel(fn, grid, block, args, shmem, lc.stream);
+}
+
+Options& options() {
+    static Options o;
+    return o;
 }
 
 struct State {
@@ -75,6 +82,12 @@ __global__ __launch_bounds__(256) void flush_kernel(uint4* p, size_t n) {
         v.x += 1u;
         p[i] = v;
     }
+}
+
+__global__ __launch_bounds__(256) void copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] = src[i];
 }
 
 // ---------------------------------------------------------------------------
@@ -591,6 +604,99 @@ int mtq_measure(const char* kernel_name, int dtype, const mtq_buf* bufs, int n_b
     return MTQ_OK;
 }
 
+int mtq_dispatch_chain(const mtq_dispatch_spec* specs, int n, int repeat, double* per_kernel_us,
+                       double* wall_us, double* stream_us) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (n < 0 || repeat < 0 || (n > 0 && !specs)) return fail(ERR_BAD_ARG, "bad chain arguments");
+    const size_t total = (size_t)n * (size_t)repeat;
+    if (total == 0) {
+        if (wall_us) *wall_us = 0.0;
+        if (stream_us) *stream_us = 0.0;
+        return MTQ_OK;
+    }
+    if (per_kernel_us && total > 65536) return fail(ERR_BAD_ARG, "per-kernel timing is limited to 65536 dispatches per chain");
+    std::vector<const KernelDesc*> descs((size_t)n);
+    for (int i = 0; i < n; i++) {
+        descs[i] = find_kernel(specs[i].kernel_name);
+        if (!descs[i]) return fail(ERR_UNKNOWN_KERNEL, std::string("unknown kernel '") + (specs[i].kernel_name ? specs[i].kernel_name : "(null)") + "'");
+    }
+    std::vector<hipEvent_t> ev;
+    auto drop_events = [&]() { for (hipEvent_t e : ev) (void)hipEventDestroy(e); };
+    if (per_kernel_us) {
+        ev.resize(total * 2, nullptr);
+        for (size_t i = 0; i < ev.size(); i++) {
+            hipError_t e = hipEventCreate(&ev[i]);
+            if (e != hipSuccess) { ev.resize(i); drop_events(); return hip_fail(e, "hipEventCreate"); }
+        }
+    }
+    hipError_t he = hipStreamSynchronize(g.stream);
+    if (he != hipSuccess) { drop_events(); return hip_fail(he, "hipStreamSynchronize"); }
+    struct timespec t0, t1;
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    if (stream_us) {
+        he = hipEventRecord(g.ev_start, g.stream);
+        if (he != hipSuccess) { drop_events(); return hip_fail(he, "hipEventRecord"); }
+    }
+    size_t idx = 0;
+    for (int r = 0; r < repeat; r++)
+        for (int i = 0; i < n; i++, idx++) {
+            LaunchCtx lc;
+            lc.stream = g.stream;
+            if (per_kernel_us) { lc.start = ev[2 * idx]; lc.stop = ev[2 * idx + 1]; }
+            rc = dispatch_desc(*descs[i], specs[i].dtype, specs[i].bufs, specs[i].n_bufs, specs[i].consts,
+                               specs[i].n_consts, lc);
+            if (rc) { (void)hipStreamSynchronize(g.stream); drop_events(); return rc; }
+        }
+    if (stream_us) {
+        he = hipEventRecord(g.ev_stop, g.stream);
+        if (he != hipSuccess) { (void)hipStreamSynchronize(g.stream); drop_events(); return hip_fail(he, "hipEventRecord"); }
+    }
+    he = hipStreamSynchronize(g.stream);
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    if (he != hipSuccess) { drop_events(); return hip_fail(he, "hipStreamSynchronize"); }
+    if (stream_us) {
+        float ms = 0.f;
+        he = hipEventElapsedTime(&ms, g.ev_start, g.ev_stop);
+        if (he != hipSuccess) { drop_events(); return hip_fail(he, "hipEventElapsedTime"); }
+        *stream_us = (double)ms * 1000.0;
+    }
+    if (wall_us) *wall_us = (double)(t1.tv_sec - t0.tv_sec) * 1e6 + (double)(t1.tv_nsec - t0.tv_nsec) * 1e-3;
+    if (per_kernel_us)
+        for (size_t i = 0; i < total; i++) {
+            float ms = 0.f;
+            if (hipEventElapsedTime(&ms, ev[2 * i], ev[2 * i + 1]) != hipSuccess) { (void)hipGetLastError(); ms = 0.f; }
+            per_kernel_us[i] = (double)ms * 1000.0;
+        }
+    drop_events();
+    return MTQ_OK;
+}
+
+int mtq_copy_kernel(void* dst, const void* src, size_t bytes, int repeat, double* avg_us) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (!dst || !src || bytes == 0 || bytes % 16 || repeat < 1) return fail(ERR_BAD_ARG, "copy: need non-null pointers, bytes % 16 == 0, repeat >= 1");
+    size_t n = bytes / 16;
+    double sum = 0.0;
+    for (int r = 0; r < repeat; r++) {
+        LaunchCtx lc;
+        lc.stream = g.stream;
+        lc.start = g.ev_start;
+        lc.stop = g.ev_stop;
+        uint4* d = (uint4*)dst;
+        const uint4* s = (const uint4*)src;
+        void* args[] = {&d, &s, &n};
+        hipError_t e = launch_kernel((const void*)copy_kernel, dim3(4096), dim3(256), args, 0, lc);
+        if (e != hipSuccess) return hip_fail(e, "copy kernel launch");
+        MTQ_HIP(hipEventSynchronize(g.ev_stop));
+        float ms = 0.f;
+        MTQ_HIP(hipEventElapsedTime(&ms, g.ev_start, g.ev_stop));
+        sum += (double)ms * 1000.0;
+    }
+    if (avg_us) *avg_us = sum / repeat;
+    return MTQ_OK;
+}
+
 int mtq_flush_cache(void) {
     int rc = need_ready();
     if (rc) return rc;
@@ -605,6 +711,31 @@ int mtq_flush_cache(void) {
     MTQ_HIP(hipGetLastError());
     MTQ_HIP(hipStreamSynchronize(g.stream));
     return MTQ_OK;
+}
+
+int mtq_set_option(const char* name, int value) {
+    if (!name) return fail(ERR_BAD_ARG, "null option name");
+    if (!strcmp(name, "qmv.rows_per_thread")) {
+        if (value != 0 && value != 4 && value != 7 && value != 8) return fail(ERR_BAD_ARG, "qmv.rows_per_thread must be 0, 4, 7 or 8");
+        options().qmv_rows_per_thread = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmv.kernel")) {
+        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmv.kernel must be 0 (auto), 1 (one-shot) or 2 (streaming)");
+        options().qmv_kernel = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmv.stream_depth")) {
+        if (value != 0 && value != 4 && value != 8) return fail(ERR_BAD_ARG, "qmv.stream_depth must be 0, 4 or 8");
+        options().qmv_stream_depth = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmv.stream_batches")) {
+        if (value < 0 || value > 16) return fail(ERR_BAD_ARG, "qmv.stream_batches must be in 0..16");
+        options().qmv_stream_batches = value;
+        return MTQ_OK;
+    }
+    return fail(ERR_BAD_ARG, std::string("unknown option '") + name + "'");
 }
 
 int mtq_timed_begin(void) {

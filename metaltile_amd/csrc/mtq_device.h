@@ -128,14 +128,21 @@ template <int DT, int BITS> struct XSlice<DT, BITS, true> {
     uint32_t xp[CPC / 2];
     float xsum[2];  // sum of the activations of dwords {0,1} and {2,3}
 
+    static constexpr int NRAW = CPC / 8;  // 16-byte vectors of activations per chunk
     // The chunk's CPC activations start at element `i0` of `x` (16-byte aligned).
-    __device__ __forceinline__ void load(const void* x, size_t i0) {
+    // load_raw only issues the loads; prepare() does the register shuffling, so a
+    // caller can put other loads between the two.
+    __device__ __forceinline__ void load_raw(const void* x, size_t i0, uint4 (&raw)[NRAW]) const {
         const uint4* xv = (const uint4*)((const uint16_t*)x + i0);
+#pragma unroll
+        for (int i = 0; i < NRAW; i++) raw[i] = xv[i];
+    }
+    __device__ __forceinline__ void prepare(const uint4 (&raw)[NRAW]) {
         float s01 = 0.f, s23 = 0.f;
         if constexpr (BITS == 4) {
 #pragma unroll
             for (int d = 0; d < 4; d++) {  // dword d of the chunk <-> 8 activations
-                uint4 v = xv[d];
+                uint4 v = raw[d];
                 xp[4 * d + 0] = (v.x & 0xFFFFu) | (v.z << 16);          // (x0,x4)
                 xp[4 * d + 1] = (v.x >> 16) | (v.z & 0xFFFF0000u);      // (x1,x5)
                 xp[4 * d + 2] = (v.y & 0xFFFFu) | (v.w << 16);          // (x2,x6)
@@ -146,7 +153,7 @@ template <int DT, int BITS> struct XSlice<DT, BITS, true> {
         } else {  // BITS == 2: dword d <-> 16 activations, pairs (x_i, x_{i+8})
 #pragma unroll
             for (int d = 0; d < 4; d++) {
-                uint4 a = xv[2 * d], b = xv[2 * d + 1];
+                uint4 a = raw[2 * d], b = raw[2 * d + 1];
                 xp[8 * d + 0] = (a.x & 0xFFFFu) | (b.x << 16);
                 xp[8 * d + 1] = (a.x >> 16) | (b.x & 0xFFFF0000u);
                 xp[8 * d + 2] = (a.y & 0xFFFFu) | (b.y << 16);
@@ -161,6 +168,11 @@ template <int DT, int BITS> struct XSlice<DT, BITS, true> {
         }
         xsum[0] = s01;
         xsum[1] = s23;
+    }
+    __device__ __forceinline__ void load(const void* x, size_t i0) {
+        uint4 raw[NRAW];
+        load_raw(x, i0, raw);
+        prepare(raw);
     }
     __device__ __forceinline__ void zero() {
 #pragma unroll
@@ -201,15 +213,43 @@ template <int DT, int BITS> struct XSlice<DT, BITS, false> {
     float xf[CPC];
     float xsum[2];
 
-    __device__ __forceinline__ void load(const void* x, size_t i0) {
+    // raw activations: 16-byte vectors of element storage
+    static constexpr int NRAW = DT == DT_F32 ? CPC / 4 : CPC / 8;
+    __device__ __forceinline__ void load_raw(const void* x, size_t i0, uint4 (&raw)[NRAW]) const {
+        const uint4* xv = DT == DT_F32 ? (const uint4*)((const float*)x + i0)
+                                       : (const uint4*)((const uint16_t*)x + i0);
+#pragma unroll
+        for (int i = 0; i < NRAW; i++) raw[i] = xv[i];
+    }
+    __device__ __forceinline__ void prepare(const uint4 (&raw)[NRAW]) {
+#pragma unroll
+        for (int i = 0; i < NRAW; i++) {
+            const uint32_t u[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if constexpr (DT == DT_F32) {
+                    xf[4 * i + j] = __uint_as_float(u[j]);
+                } else if constexpr (DT == DT_F16) {
+                    xf[8 * i + 2 * j] = f16_bits_to_f32(u[j] & 0xFFFFu);
+                    xf[8 * i + 2 * j + 1] = f16_bits_to_f32(u[j] >> 16);
+                } else {
+                    xf[8 * i + 2 * j] = bf16_bits_to_f32(u[j] & 0xFFFFu);
+                    xf[8 * i + 2 * j + 1] = bf16_bits_to_f32(u[j] >> 16);
+                }
+            }
+        }
         float s01 = 0.f, s23 = 0.f;
 #pragma unroll
         for (int i = 0; i < CPC; i++) {
-            xf[i] = load_elem<DT>(x, i0 + i);
             if (i < CPC / 2) s01 += xf[i]; else s23 += xf[i];
         }
         xsum[0] = s01;
         xsum[1] = s23;
+    }
+    __device__ __forceinline__ void load(const void* x, size_t i0) {
+        uint4 raw[NRAW];
+        load_raw(x, i0, raw);
+        prepare(raw);
     }
     __device__ __forceinline__ void zero() {
 #pragma unroll

@@ -68,6 +68,15 @@ struct QmvParams {
     uint32_t E = 1;                   // experts
 };
 
+// Tuning overrides set through mtq_set_option (0 = automatic).
+struct Options {
+    int qmv_rows_per_thread = 0;  // one-shot kernel: weight rows per thread
+    int qmv_kernel = 0;           // 0 auto, 1 one-shot only, 2 prefer streaming
+    int qmv_stream_depth = 0;     // streaming kernel: ring depth (4 / 8)
+    int qmv_stream_batches = 0;   // streaming kernel: batches per thread
+};
+Options& options();
+
 // Fast LDS/dot2 GEMV family (qmv.hip). Returns ERR_UNSUPPORTED when the shape
 // does not fit its geometry so the caller can fall back to the generic kernel.
 int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc);

@@ -1,0 +1,7 @@
+// Instantiates the qmv kernel family for element dtype bf16 (see qmv_impl.h).
+#include "qmv_impl.h"
+
+namespace mtq {
+template int qmv_launch_dtype<DT_BF16>(QmvKArgs&, int, int, const QmvGeom&, const LaunchCtx&);
+template int qmv_stream_launch_dtype<DT_BF16>(QmvSArgs&, int, int, const QmvSGeom&, const LaunchCtx&);
+}

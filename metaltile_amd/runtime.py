@@ -203,6 +203,40 @@ class GpuRunner:
                                          int(warmup), int(iters), samples))
         return [samples[i] for i in range(iters)]
 
+    def dispatch_chain(self, specs, repeat: int = 1, per_kernel: bool = True, stream_events: bool = False):
+        """Enqueue `specs` = [(kernel, dtype, bufs, consts), ...] back to back,
+        `repeat` times, with no host wait in between (the reference's
+        `Context::dispatch_chain` over resident buffers,
+        crates/metaltile-runtime/src/context.rs:363-401). Returns
+        (per-dispatch GPU durations in us or None, wall-clock us, time between
+        two events bracketing the chain on the stream in us or None)."""
+        n = len(specs)
+        arr = (_lib.MtqDispatchSpec * max(n, 1))()
+        keep = []
+        for i, (kernel, dtype, bufs, consts) in enumerate(specs):
+            sig = KERNEL_SIGNATURES[kernel]
+            barr, carr = _bind(sig, bufs, consts)
+            name = kernel.encode()
+            keep.append((barr, carr, name))
+            arr[i].kernel_name = name
+            arr[i].dtype = int(dtype)
+            arr[i].bufs = barr
+            arr[i].n_bufs = len(sig.params)
+            arr[i].consts = carr
+            arr[i].n_consts = len(sig.constexprs)
+        total = n * repeat
+        per = (C.c_double * max(total, 1))() if per_kernel else None
+        wall = C.c_double(0.0)
+        sus = C.c_double(0.0)
+        _lib.check(self._lib.mtq_dispatch_chain(arr, n, int(repeat), per, C.byref(wall),
+                                                C.byref(sus) if stream_events else None))
+        return ([per[i] for i in range(total)] if per_kernel else None), wall.value, (sus.value if stream_events else None)
+
+    def copy_kernel(self, dst: GpuBuffer, src: GpuBuffer, nbytes: int, repeat: int = 1) -> float:
+        us = C.c_double(0.0)
+        _lib.check(self._lib.mtq_copy_kernel(dst.ptr, src.ptr, int(nbytes), int(repeat), C.byref(us)))
+        return us.value
+
     def flush_slc(self) -> None:
         _lib.check(self._lib.mtq_flush_cache())
 
