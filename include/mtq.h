@@ -226,6 +226,7 @@ MTQ_API int mtq_flush_cache(void);
  *   "qmv.rows_per_thread"  one-shot kernel: 0 = choose per shape, or 4 / 7 / 8
  *   "qmv.stream_depth"     streaming kernel: 0 = choose per shape, or 4 / 8 loads in flight per thread
  *   "qmv.stream_batches"   streaming kernel: 0 = choose per shape, or 1..16 batches per thread
+ *   "qmm.splits"           MFMA qmm: 0 = choose per shape, or the number of K slices per output tile
  * Unknown names or values fail with MTQ_ERR_BAD_ARG. */
 MTQ_API int mtq_set_option(const char *name, int value);
 

@@ -725,6 +725,11 @@ int mtq_set_option(const char* name, int value) {
         options().qmv_kernel = value;
         return MTQ_OK;
     }
+    if (!strcmp(name, "qmm.splits")) {
+        if (value < 0 || value > 64) return fail(ERR_BAD_ARG, "qmm.splits must be in 0..64");
+        options().qmm_splits = value;
+        return MTQ_OK;
+    }
     if (!strcmp(name, "qmv.stream_depth")) {
         if (value != 0 && value != 4 && value != 8) return fail(ERR_BAD_ARG, "qmv.stream_depth must be 0, 4 or 8");
         options().qmv_stream_depth = value;

@@ -74,6 +74,7 @@ struct Options {
     int qmv_kernel = 0;           // 0 auto, 1 one-shot only, 2 prefer streaming
     int qmv_stream_depth = 0;     // streaming kernel: ring depth (4 / 8)
     int qmv_stream_batches = 0;   // streaming kernel: batches per thread
+    int qmm_splits = 0;           // MFMA qmm: K splits per tile (0 = choose per shape)
 };
 Options& options();
 

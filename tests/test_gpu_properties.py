@@ -73,14 +73,16 @@ def test_batched_rows_equal_single_rows(M):
 
 def test_qmm_rows_match_qmv_within_tolerance():
     """M=2048 prefill (too large for the CPU oracle in this suite): every 64th row
-    against the M=1 GEMV path, which is itself checked against the oracle."""
+    against the M=1 GEMV path, which is itself checked against the oracle. The
+    MFMA path rounds dequantised weights to bf16 as the reference's mma kernels do,
+    so the bound is the reference's bf16 one (tests/qmm_gpu_correctness.rs:2085-2106)."""
     M, N, K, G = 2048, 4096, 4096, 64
     print("[case] qmm M=2048 vs qmv rows", flush=True)
     c = make_case(15, DType.BF16, 4, G, M, N, K)
     got = _run(DType.BF16, 4, G, c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, entry=ops.qmm).reshape(M, N)
     for mrow in range(0, M, 64):
         one = _run(DType.BF16, 4, G, c.w, c.scales_f, c.biases_f, c.x_f[mrow * K:(mrow + 1) * K], 1, N, K)
-        assert rel_err(got[mrow], one) <= 2e-2
+        assert rel_err(got[mrow], one) <= 5e-2
 
 
 def test_gather_single_expert_equals_plain_qmm():
