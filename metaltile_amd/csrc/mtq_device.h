@@ -118,6 +118,13 @@ template <int DT> __device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t
     }
 }
 
+// MAGIC pair (2^7 twice in bf16, 2^10 twice in f16) as an opaque VGPR value.
+template <int DT> __device__ __forceinline__ uint32_t magic_or_vgpr() {
+    uint32_t k = DT == DT_BF16 ? 0x43004300u : 0x64006400u;
+    asm volatile("" : "+v"(k));
+    return k;
+}
+
 template <int DT, int BITS, bool DOT2 = PathSel<DT, BITS>::kDot2> struct XSlice;
 
 // dot2 path: activations kept as 16-bit pairs arranged to match the code pairs
@@ -127,6 +134,7 @@ template <int DT, int BITS> struct XSlice<DT, BITS, true> {
     static constexpr int CPD = 32 / BITS;    // codes per dword
     uint32_t xp[CPC / 2];
     float xsum[2];  // sum of the activations of dwords {0,1} and {2,3}
+    uint32_t kor;   // MAGIC pair, held in a VGPR (set by prepare / zero)
 
     static constexpr int NRAW = CPC / 8;  // 16-byte vectors of activations per chunk
     // The chunk's CPC activations start at element `i0` of `x` (16-byte aligned).
@@ -138,6 +146,7 @@ template <int DT, int BITS> struct XSlice<DT, BITS, true> {
         for (int i = 0; i < NRAW; i++) raw[i] = xv[i];
     }
     __device__ __forceinline__ void prepare(const uint4 (&raw)[NRAW]) {
+        kor = magic_or_vgpr<DT>();
         float s01 = 0.f, s23 = 0.f;
         if constexpr (BITS == 4) {
 #pragma unroll
@@ -175,6 +184,7 @@ template <int DT, int BITS> struct XSlice<DT, BITS, true> {
         prepare(raw);
     }
     __device__ __forceinline__ void zero() {
+        kor = magic_or_vgpr<DT>();
 #pragma unroll
         for (int i = 0; i < CPC / 2; i++) xp[i] = 0;
         xsum[0] = xsum[1] = 0.f;
@@ -191,7 +201,10 @@ template <int DT, int BITS> struct XSlice<DT, BITS, true> {
     }
     // sum over the codes of dword d of (MAGIC + q) * x
     __device__ __forceinline__ float dot_dword(uint32_t w, int d, float acc) const {
-        constexpr uint32_t kOr = DT == DT_BF16 ? 0x43004300u : 0x64006400u;
+        // The OR constant lives in a VGPR the optimiser cannot see through: with
+        // the mask as the one scalar/literal operand, (w & mask) | k then fits a
+        // single v_and_or_b32 (two literal constants would not).
+        const uint32_t kOr = kor;
         if constexpr (BITS == 4) {
             acc = dot2_acc<DT>((w & 0x000F000Fu) | kOr, xp[4 * d + 0], acc);
             acc = dot2_acc<DT>(((w >> 4) & 0x000F000Fu) | kOr, xp[4 * d + 1], acc);
