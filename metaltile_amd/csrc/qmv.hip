@@ -61,7 +61,7 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
             const double waves_per_cu = (double)grid / cus * (tpb / 64);
             double score = waste + idle;
             if (waves_per_cu < 8.0) score += (8.0 - waves_per_cu) * 0.04;
-            if (waves_per_cu > 16.0) score += (waves_per_cu - 16.0) * 0.02;
+            if (waves_per_cu > 32.0) score += (waves_per_cu - 32.0) * 0.02;
             // Measured on the 14336x4096 / 4096x14336 shapes: small workgroups do
             // best one batch deep (more, shorter-lived workgroups), wide ones two.
             if (nb == 1) score += tpb > 256 ? 0.15 : -0.05;
