@@ -157,7 +157,7 @@ def main():
             "pct_hbm_peak_whole_job": round(100.0 * gbs / HBM_PEAK_GBS, 2),
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_from_profiles("qmv_bf16_b4_llama_mlp"),
-                         "kernel": "qmv_kernel<bf16,4bit,MB=1>", "bytes_per_launch": launch_bytes,
+                         "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, 1 row>", "bytes_per_launch": launch_bytes,
                          "avg_launch_us_timed_region": round(kern_avg, 3),
                          "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(st.min_us, 3),
                                                "median_us": round(st.median_us, 3), "p95_us": round(st.p95_us, 3),
