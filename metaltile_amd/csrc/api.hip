@@ -725,6 +725,18 @@ int mtq_set_option(const char* name, int value) {
         options().qmv_kernel = value;
         return MTQ_OK;
     }
+    if (!strcmp(name, "qmv.mfma")) {
+        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmv.mfma must be 0 (auto), 1 (off) or 2 (prefer)");
+        options().qmv_mfma = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmv.mfma_kp") || !strcmp(name, "qmv.mfma_rbw") || !strcmp(name, "qmv.mfma_nrb")) {
+        if (value < 0 || value > 16) return fail(ERR_BAD_ARG, "qmv.mfma_* must be in 0..16");
+        if (name[9] == 'k') options().qmv_mfma_kp = value;
+        else if (name[9] == 'r') options().qmv_mfma_rbw = value;
+        else options().qmv_mfma_nrb = value;
+        return MTQ_OK;
+    }
     if (!strcmp(name, "qmm.splits")) {
         if (value < 0 || value > 64) return fail(ERR_BAD_ARG, "qmm.splits must be in 0..64");
         options().qmm_splits = value;

@@ -75,12 +75,18 @@ struct Options {
     int qmv_stream_depth = 0;     // streaming kernel: ring depth (4 / 8)
     int qmv_stream_batches = 0;   // streaming kernel: batches per thread
     int qmm_splits = 0;           // MFMA qmm: K splits per tile (0 = choose per shape)
+    int qmv_mfma = 0;             // matrix-core qmv: 0 auto, 1 never, 2 whenever the shape fits
+    int qmv_mfma_kp = 0;          // matrix-core qmv: K parts per row block
+    int qmv_mfma_rbw = 0;         // matrix-core qmv: row blocks walked in parallel per workgroup
+    int qmv_mfma_nrb = 0;         // matrix-core qmv: row blocks per wave
 };
 Options& options();
 
 // Fast LDS/dot2 GEMV family (qmv.hip). Returns ERR_UNSUPPORTED when the shape
 // does not fit its geometry so the caller can fall back to the generic kernel.
 int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc);
+// Matrix-core streaming GEMV family for f16/bf16 (qmv_mfma.hip); same contract.
+int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc);
 // One-wave-per-output kernel for any bit width 2..8 and any group size (generic.hip).
 int launch_qmv_generic(const QmvParams& p, const LaunchCtx& lc);
 

@@ -106,6 +106,10 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
 }
 
 int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {
+    if (options().qmv_mfma != 1) {
+        int rc = launch_qmv_mfma(p, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
     if (p.bits != 2 && p.bits != 4 && p.bits != 8)
         return fail(ERR_UNSUPPORTED, "fast qmv: bits must be 2, 4 or 8");
     const uint32_t cpc = 128u / (uint32_t)p.bits;

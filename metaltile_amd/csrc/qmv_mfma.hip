@@ -1,0 +1,143 @@
+// Host side of the matrix-core qmv / gather_qmv kernel (qmv_mfma_impl.h): checks
+// that a request fits its geometry, picks the launch shape and calls the
+// per-dtype instantiation. Requests that do not fit return ERR_UNSUPPORTED so
+// the caller can use the dot2 family or the generic kernel.
+#include "qmv_mfma_impl.h"
+
+namespace mtq {
+
+extern template int qmv_mfma_launch_dtype<DT_F16>(QmvMArgs&, int, int, const QmvMGeom&, const LaunchCtx&);
+extern template int qmv_mfma_launch_dtype<DT_BF16>(QmvMArgs&, int, int, const QmvMGeom&, const LaunchCtx&);
+
+namespace {
+bool is_pow2(uint32_t v) { return v && !(v & (v - 1)); }
+uint32_t ilog2(uint32_t v) { uint32_t l = 0; while ((1u << l) < v) l++; return l; }
+constexpr size_t kLdsBudget = 150 * 1024;  // of the 160 KB per CU
+
+size_t lds_bytes(uint32_t R, uint32_t K, uint32_t nch, uint32_t rows_wg, uint32_t gpr, uint32_t KP, uint32_t list_cap) {
+    return (size_t)R * K * 2 + (size_t)R * nch * 4 + ((size_t)rows_wg * gpr + 1) * 8 +
+           (size_t)KP * rows_wg * R * 4 + (size_t)list_cap * 4 + 64;
+}
+}  // namespace
+
+int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
+    if (p.dtype != DT_F16 && p.dtype != DT_BF16) return fail(ERR_UNSUPPORTED, "mfma qmv: f16/bf16 only");
+    if (!(p.bits == 2 || p.bits == 4 || (p.bits == 8 && p.dtype == DT_F16)))
+        return fail(ERR_UNSUPPORTED, "mfma qmv: bits");
+    if (p.N == 0 || p.K == 0) return fail(ERR_UNSUPPORTED, "mfma qmv: empty");
+    const uint64_t rb64 = (uint64_t)p.K * p.bits / 8;
+    if (((uint64_t)p.K * p.bits) % 2048 || rb64 > (1u << 24)) return fail(ERR_UNSUPPORTED, "mfma qmv: row is not whole 256-byte segments");
+    const uint32_t RB = (uint32_t)rb64, nseg = RB / 256, nch = RB / 16, cpc = 128u / (uint32_t)p.bits;
+    const uint32_t G = p.group_size;
+    if (!is_pow2(G) || G < cpc || p.K % G) return fail(ERR_UNSUPPORTED, "mfma qmv: group size");
+    const uint32_t gpr = p.K / G;
+    if (gpr % 4) return fail(ERR_UNSUPPORTED, "mfma qmv: groups per row not a multiple of 4");
+    if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
+        return fail(ERR_UNSUPPORTED, "mfma qmv: operands must be 16-byte aligned");
+    const bool gather = p.gather == GATHER_CSR || p.gather == GATHER_INDICES;
+    const uint32_t rows = gather ? p.T : (p.gather == GATHER_SINGLE ? 1u : p.M);
+    if (rows == 0) return ERR_OK;
+    const Options& opt = options();
+
+    // K parts: keep 4..8 segments per wave and row block where the row allows
+    uint32_t KP = 1;
+    if (opt.qmv_mfma_kp) {
+        KP = (uint32_t)opt.qmv_mfma_kp;
+        if (nseg % KP) return fail(ERR_BAD_ARG, "qmv.mfma_kp must divide the row's segment count");
+    } else {
+        uint32_t best = 1;
+        double best_score = 1e30;
+        for (uint32_t kp = 1; kp <= nseg && kp <= 16; kp++) {
+            if (nseg % kp) continue;
+            const uint32_t spp = nseg / kp, padded = (spp + 3) / 4 * 4;
+            double score = (double)(padded - spp) / spp;          // wasted ring slots
+            if (spp > 8) score += 0.05 * (spp - 8);               // long walks: few waves per row block
+            if (spp < 4) score += 0.5;
+            score += 0.01 * kp;
+            if (score < best_score) { best_score = score; best = kp; }
+        }
+        KP = best;
+    }
+    const uint32_t spp = nseg / KP;
+
+    // activation rows per pass
+    int mp = 4, s = 1;
+    uint32_t rows_per_launch = rows;
+    if (p.gather == GATHER_NONE) {
+        if (rows == 1) mp = 1; else if (rows == 2) mp = 2;
+        if (rows > 4) s = rows > 8 ? 4 : 2;
+        rows_per_launch = rows > 16 ? 16 : rows;
+    } else if (p.gather == GATHER_SINGLE) {
+        mp = 1;
+    } else {
+        const uint32_t avg = (rows + p.E - 1) / (p.E ? p.E : 1);
+        s = avg > 4 ? 4 : (avg > 2 ? 2 : 1);
+        if (p.bits == 2 && s > 2) s = 2;  // the 16-row 2-bit variant does not fit the register file
+    }
+    const uint32_t maxt = s >= 2 ? 512u : 1024u;
+    if (64u * KP > maxt) return fail(ERR_UNSUPPORTED, "mfma qmv: too many K parts");
+    uint32_t RBW = opt.qmv_mfma_rbw ? (uint32_t)opt.qmv_mfma_rbw : (256u / (64u * KP) ? 256u / (64u * KP) : 1u);
+    while (64u * KP * RBW > maxt && RBW > 1) RBW--;
+    uint32_t nrb = opt.qmv_mfma_nrb ? (uint32_t)opt.qmv_mfma_nrb : 1u;
+    const uint32_t list_cap = p.gather == GATHER_INDICES ? p.T : 0;
+    // shrink until the workgroup's LDS fits
+    while (lds_bytes((uint32_t)(mp * s), p.K, nch, 4 * RBW * nrb, gpr, KP, list_cap) > kLdsBudget) {
+        if (nrb > 1) nrb--;
+        else if (s > 1) s /= 2;
+        else if (RBW > 1) RBW--;
+        else return fail(ERR_UNSUPPORTED, "mfma qmv: activations do not fit in LDS");
+    }
+    const uint32_t R = (uint32_t)(mp * s);
+    if (p.gather == GATHER_NONE && rows_per_launch > R) rows_per_launch = R;
+
+    if (p.gather == GATHER_NONE && rows > rows_per_launch) {
+        // more activation rows than one pass holds: one launch per R rows
+        for (uint32_t m0 = 0; m0 < rows; m0 += rows_per_launch) {
+            QmvParams q2 = p;
+            q2.M = rows - m0 < rows_per_launch ? rows - m0 : rows_per_launch;
+            q2.x = (const char*)p.x + (size_t)m0 * p.K * 2;
+            q2.out = (char*)p.out + (size_t)m0 * p.N * 2;
+            LaunchCtx l2 = lc;
+            if (m0) l2.start = nullptr;
+            if (m0 + rows_per_launch < rows) l2.stop = nullptr;
+            int rc = launch_qmv_mfma(q2, l2);
+            if (rc) return rc;
+        }
+        return ERR_OK;
+    }
+
+    QmvMArgs a;
+    a.w = (const unsigned char*)p.w;
+    a.scales = p.scales;
+    a.biases = p.biases;
+    a.x = p.x;
+    a.out = p.out;
+    a.route = p.route;
+    a.M = rows;
+    a.N = p.N;
+    a.K = p.K;
+    a.T = p.T;
+    a.E = p.E;
+    a.RB = RB;
+    a.nch = nch;
+    a.spp = spp;
+    a.KP = KP;
+    a.RBW = RBW;
+    a.nrb = nrb;
+    a.gpr = gpr;
+    a.log2g = ilog2(G);
+    a.list_cap = list_cap;
+    QmvMGeom g;
+    g.mp = mp;
+    g.s = s;
+    g.tpb = 64u * KP * RBW;
+    const uint32_t rows_wg = 4 * RBW * nrb;
+    g.shmem = lds_bytes(R, p.K, nch, rows_wg, gpr, KP, list_cap);
+    g.grid = dim3((p.N + rows_wg - 1) / rows_wg, gather ? p.E : 1, 1);
+    switch (p.dtype) {
+        case DT_F16: return qmv_mfma_launch_dtype<DT_F16>(a, p.bits, p.gather, g, lc);
+        default: return qmv_mfma_launch_dtype<DT_BF16>(a, p.bits, p.gather, g, lc);
+    }
+}
+
+}  // namespace mtq

@@ -1,0 +1,406 @@
+// Streaming qmv / small-batch qmm / gather_qmv kernel for f16 and bf16
+// activations on gfx950 that does its dot products on the matrix cores.
+// Included by qmv_mfma_f16.hip and qmv_mfma_bf16.hip (one element dtype each).
+//
+// Replaces the same reference kernels as the dot2 family in qmv_impl.h
+// (mt_qmv, mt_qmm, mt_qmm_bm{2,4}: crates/metaltile-std/src/mlx/quantized.rs:8-308,
+// 343-621, 650, 1072; mt_moe_gather_qmm_int4{,_m8,_m16,_m32} and the per-row
+// ABI: crates/metaltile-std/src/ffai/moe.rs:358-433, 634, 900, 1363, 2256-2550;
+// dequant_gemv_int4_expert_indexed:
+// crates/metaltile-std/src/ffai/dequant_gemv_expert_indexed.rs:58-105) for shapes
+// whose rows are a whole number of 256-byte segments.
+//
+// Geometry. v_mfma_f32_4x4x4_16b_{f16,bf16} is sixteen independent 4x4x4
+// products: in block b (lanes 4b..4b+3), lane 4b+j supplies column j of B, lane
+// 4b+i supplies row i of A, and lane 4b+j receives D[0..3][j]. Here B's column j
+// is four codes of weight row r0+j, A's row i is the matching four activations
+// of activation row i, so lane (j, b) accumulates, for ITS OWN 16 bytes of
+// weights, the partial dot products with up to four activation rows at once.
+// One wave-wide 128-bit load therefore covers 4 weight rows x 256 contiguous
+// bytes (lane = 4*q + r: row r, 16-byte chunk q of the segment), which streams
+// from HBM at the rate of a plain linear read.
+//
+// Codes never leave integer form: a masked pair of codes OR-ed into the mantissa
+// of 2^7 (bf16) or 2^10 (f16) IS the pair (MAGIC+q_a, MAGIC+q_b) in element
+// format and goes straight into the B operand. A chunk lies inside one
+// quantisation group, so after the chunk's MFMAs
+//     out += s * (D - MAGIC*sum_x) + b * sum_x = s*D + (b - MAGIC*s) * sum_x
+// with sum_x the sum of the chunk's activations (precomputed once per
+// workgroup). Activations live in LDS, permuted once into MFMA operand order,
+// together with the per-chunk sums and the (s, b - MAGIC*s) pairs of the
+// workgroup's rows.
+//
+// A wave walks along K for a block of four weight rows (optionally a 1/KP part
+// of K), keeping D weight loads in flight in a register ring, then reduces its
+// lanes' totals once per row block. Gather modes add blockIdx.y = expert and run
+// the expert's activation rows R = MP*S at a time.
+#pragma once
+#include "mtq_device.h"
+#include "mtq_internal.h"
+
+namespace mtq {
+
+typedef uint32_t m_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t m_u32x2 __attribute__((ext_vector_type(2)));
+typedef short m_s16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 m_f16x4 __attribute__((ext_vector_type(4)));
+typedef float m_f32x4 __attribute__((ext_vector_type(4)));
+
+struct QmvMArgs {
+    const unsigned char* w;
+    const void* scales;
+    const void* biases;
+    const void* x;
+    void* out;
+    const uint32_t* route;
+    uint32_t M, N, K, T, E;
+    uint32_t RB;        // bytes per packed weight row
+    uint32_t nch;       // 16-byte chunks per row
+    uint32_t spp;       // 256-byte segments per K part
+    uint32_t KP;        // K parts (waves sharing a row block)
+    uint32_t RBW;       // row blocks walked in parallel by one workgroup
+    uint32_t nrb;       // row blocks per wave, one after the other
+    uint32_t gpr, log2g;
+    uint32_t list_cap;  // capacity of the row list (indices mode)
+};
+
+struct QmvMGeom {
+    int mp, s;          // activation rows per MFMA set (1, 2, 4) and sets
+    uint32_t tpb;
+    size_t shmem;
+    dim3 grid;
+};
+
+template <int DT> __device__ __forceinline__ m_f32x4 mfma4(m_u32x2 a, m_u32x2 b, m_f32x4 c) {
+    if constexpr (DT == DT_BF16) {
+        return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(m_s16x4, a), __builtin_bit_cast(m_s16x4, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(m_f16x4, a), __builtin_bit_cast(m_f16x4, b), c, 0, 0, 0);
+    }
+}
+
+// Position, inside a u32 word's PF codes, of the activation that pairs with the
+// o-th element of the word's MFMA operand sequence: MFMA t of a word multiplies
+// pair words (2t, 2t+1) = codes (2t, 2t+PF/2, 2t+1, 2t+1+PF/2).
+template <int PF> __host__ __device__ constexpr int mfma_src_index(int o) {
+    const int t = o / 4, e = o % 4;
+    return 2 * t + (e >> 1) + (e & 1) * (PF / 2);
+}
+
+template <int DT, int BITS, int MP, int S, int D, int MODE, int MAXT>
+__global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
+    constexpr int PF = 32 / BITS;   // codes per u32 word
+    constexpr int CPC = 4 * PF;     // codes per 16-byte chunk
+    constexpr int NP = PF / 2;      // 16-byte activation pieces per chunk
+    constexpr int R = MP * S;       // activation rows per pass
+    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
+    constexpr uint32_t MAGIC2 = DT == DT_BF16 ? 0x43004300u : 0x64006400u;
+    constexpr uint32_t MASK = ((1u << BITS) - 1u) * 0x00010001u;
+    constexpr uint32_t NOROW = 0xFFFFFFFFu;
+    static_assert(DT != DT_BF16 || BITS <= 7, "an 8-bit code does not fit the bf16 mantissa");
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    const uint32_t rows_wg = 4u * a.RBW * a.nrb;
+    m_u32x4* XL = (m_u32x4*)smem;                                    // [S][NP][nch][MP] pieces
+    float* XS = (float*)(XL + (size_t)S * NP * a.nch * MP);          // [S][nch][MP] chunk sums
+    float2* SB = (float2*)(XS + (size_t)S * a.nch * MP);             // [rows_wg][gpr] + one zero pair
+    float* RED = (float*)(SB + (size_t)rows_wg * a.gpr + 1);         // [KP][rows_wg][R]
+    uint32_t* rowlist = (uint32_t*)(RED + (size_t)a.KP * rows_wg * R);
+    __shared__ uint32_t s_meta[4];
+
+    const uint32_t tid = threadIdx.x, TPB = blockDim.x;
+    const uint32_t lane = tid & 63u, wave = tid >> 6;
+    const uint32_t r = lane & 3u, q = lane >> 2;
+    const uint32_t kp = wave % a.KP, rbw = wave / a.KP;
+    const uint32_t row0 = blockIdx.x * rows_wg;
+
+    // ---- routing: which activation rows does this workgroup serve? ----------
+    uint32_t expert = 0, cnt = a.M, lo = 0, n1 = a.M, lo2 = 0;
+    if constexpr (MODE == GATHER_CSR) {
+        expert = blockIdx.y;
+        // E(t) = first e with t < off[e+1], else 0 (crates/metaltile-std/src/ffai/moe.rs:376-385)
+        uint32_t mx = 0, l = 0;
+        for (uint32_t j = 1; j <= a.E; j++) {
+            uint32_t o = a.route[j];
+            if (j <= expert) l = max(l, o);
+            mx = max(mx, o);
+        }
+        uint32_t hi = min(a.route[expert + 1], a.T);
+        lo = l;
+        n1 = hi > lo ? hi - lo : 0;
+        lo2 = min(mx, a.T);
+        uint32_t n2 = expert == 0 ? a.T - lo2 : 0;
+        cnt = n1 + n2;
+        if (cnt == 0) return;
+    } else if constexpr (MODE == GATHER_INDICES) {
+        expert = blockIdx.y;
+        if (tid < 64) {
+            uint32_t n = 0;
+            for (uint32_t t0 = 0; t0 < a.T; t0 += 64) {
+                uint32_t t = t0 + lane;
+                bool hit = t < a.T && a.route[t] == expert;
+                unsigned long long m = __ballot(hit);
+                if (hit) rowlist[n + __popcll(m & ((1ull << lane) - 1ull))] = t;
+                n += (uint32_t)__popcll(m);
+            }
+            if (lane == 0) s_meta[0] = n;
+        }
+        __syncthreads();
+        cnt = s_meta[0];
+        if (cnt == 0) return;
+    } else if constexpr (MODE == GATHER_SINGLE) {
+        expert = min(a.route[0], a.E - 1);  // an out-of-range id must not fault the GPU
+        cnt = 1;
+    }
+    auto batch_row = [&](uint32_t j) -> uint32_t {
+        if (j >= cnt) return NOROW;
+        if constexpr (MODE == GATHER_CSR) return j < n1 ? lo + j : lo2 + (j - n1);
+        else if constexpr (MODE == GATHER_INDICES) return rowlist[j];
+        else return j;
+    };
+
+    const size_t slab_rows = (size_t)expert * a.N;
+    const unsigned char* wbase = a.w + slab_rows * a.RB + (size_t)(kp * a.spp) * 256u + q * 16u;
+    const uint32_t sppD = (a.spp + D - 1) / D * D;  // steps per row block, padded to whole rings
+
+    // Address of the 16 bytes this lane loads at step (rb, sg). Steps past the
+    // end of a row block or of the wave's work re-read a valid address; what they
+    // load is multiplied by a zero scale.
+    auto w_ptr = [&](uint32_t rb, uint32_t sg) -> const m_u32x4* {
+        rb = min(rb, a.nrb - 1);
+        sg = min(sg, a.spp - 1);
+        const uint32_t row = min(row0 + (rb * a.RBW + rbw) * 4u + r, a.N - 1);
+        return (const m_u32x4*)(wbase + (size_t)row * a.RB + (size_t)sg * 256u);
+    };
+
+    const uint32_t n_pass = (MODE == GATHER_CSR || MODE == GATHER_INDICES) ? (cnt + R - 1) / R : 1u;
+    for (uint32_t pass = 0; pass < n_pass; pass++) {
+        // ---- weights first: D loads per lane in flight during the staging ----
+        m_u32x4 ring[D];
+#pragma unroll
+        for (int d = 0; d < D; d++) ring[d] = __builtin_nontemporal_load(w_ptr(0, d));
+
+        // ---- (s, b - MAGIC*s) pairs of the workgroup's rows -------------------
+        if (pass == 0) {
+            const uint32_t nvec = rows_wg * a.gpr / 4;
+            for (uint32_t v = tid; v < nvec; v += TPB) {
+                const uint32_t e = v * 4, rl = e / a.gpr, g = e - rl * a.gpr;
+                const size_t src = (slab_rows + min(row0 + rl, a.N - 1)) * a.gpr + g;
+                const uint2 sv = *(const uint2*)((const uint16_t*)a.scales + src);
+                const uint2 bv = *(const uint2*)((const uint16_t*)a.biases + src);
+                float s4[4], b4[4];
+                if constexpr (DT == DT_BF16) {
+                    s4[0] = bf16_bits_to_f32(sv.x & 0xFFFFu); s4[1] = bf16_bits_to_f32(sv.x >> 16);
+                    s4[2] = bf16_bits_to_f32(sv.y & 0xFFFFu); s4[3] = bf16_bits_to_f32(sv.y >> 16);
+                    b4[0] = bf16_bits_to_f32(bv.x & 0xFFFFu); b4[1] = bf16_bits_to_f32(bv.x >> 16);
+                    b4[2] = bf16_bits_to_f32(bv.y & 0xFFFFu); b4[3] = bf16_bits_to_f32(bv.y >> 16);
+                } else {
+                    s4[0] = f16_bits_to_f32(sv.x & 0xFFFFu); s4[1] = f16_bits_to_f32(sv.x >> 16);
+                    s4[2] = f16_bits_to_f32(sv.y & 0xFFFFu); s4[3] = f16_bits_to_f32(sv.y >> 16);
+                    b4[0] = f16_bits_to_f32(bv.x & 0xFFFFu); b4[1] = f16_bits_to_f32(bv.x >> 16);
+                    b4[2] = f16_bits_to_f32(bv.y & 0xFFFFu); b4[3] = f16_bits_to_f32(bv.y >> 16);
+                }
+                float4* dst = (float4*)(SB + e);
+                dst[0] = make_float4(s4[0], b4[0] - MAGIC * s4[0], s4[1], b4[1] - MAGIC * s4[1]);
+                dst[1] = make_float4(s4[2], b4[2] - MAGIC * s4[2], s4[3], b4[3] - MAGIC * s4[3]);
+            }
+            if (tid == 0) SB[rows_wg * a.gpr] = make_float2(0.f, 0.f);
+        }
+
+        // ---- activations of this pass: permute into operand order, chunk sums --
+        const uint32_t base_row = pass * R;
+        for (uint32_t task = tid; task < (uint32_t)R * a.nch; task += TPB) {
+            const uint32_t i = task / a.nch, c = task - i * a.nch;
+            const uint32_t t = batch_row(base_row + i);
+            uint32_t raw[NP * 4];
+            if (t != NOROW) {
+                const m_u32x4* src = (const m_u32x4*)((const uint16_t*)a.x + (size_t)t * a.K + (size_t)c * CPC);
+#pragma unroll
+                for (int p = 0; p < NP; p++) {
+                    const m_u32x4 v = src[p];
+                    raw[4 * p] = v.x; raw[4 * p + 1] = v.y; raw[4 * p + 2] = v.z; raw[4 * p + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NP * 4; j++) raw[j] = 0u;
+            }
+            float sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < NP * 4; j++) {
+                if constexpr (DT == DT_BF16) sum += bf16_bits_to_f32(raw[j] & 0xFFFFu) + bf16_bits_to_f32(raw[j] >> 16);
+                else sum += f16_bits_to_f32(raw[j] & 0xFFFFu) + f16_bits_to_f32(raw[j] >> 16);
+            }
+            const uint32_t s = i / MP, i4 = i % MP;
+            XS[((size_t)s * a.nch + c) * MP + i4] = sum;
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                uint32_t o[4];
+#pragma unroll
+                for (int dw = 0; dw < 4; dw++) {
+                    uint32_t h[2];
+#pragma unroll
+                    for (int e2 = 0; e2 < 2; e2++) {
+                        const int oe = p * 8 + dw * 2 + e2;          // element of the chunk's operand sequence
+                        const int wi = oe / PF;                      // word it belongs to
+                        const int se = wi * PF + mfma_src_index<PF>(oe % PF);  // source element
+                        h[e2] = (se & 1) ? (raw[se >> 1] >> 16) : (raw[se >> 1] & 0xFFFFu);
+                    }
+                    o[dw] = h[0] | (h[1] << 16);
+                }
+                m_u32x4 piece = {o[0], o[1], o[2], o[3]};
+                XL[(((size_t)s * NP + p) * a.nch + c) * MP + i4] = piece;
+            }
+        }
+        __syncthreads();
+
+        // ---- stream ------------------------------------------------------------
+        const uint32_t arow = r & (uint32_t)(MP - 1);
+        for (uint32_t rb = 0; rb < a.nrb; rb++) {
+            float tot[S][MP];
+#pragma unroll
+            for (int s = 0; s < S; s++)
+#pragma unroll
+                for (int i = 0; i < MP; i++) tot[s][i] = 0.f;
+            const uint32_t row_local = (rb * a.RBW + rbw) * 4u + r;
+            const uint32_t sb_row = row_local * a.gpr;
+            for (uint32_t sg0 = 0; sg0 < sppD; sg0 += D) {
+                const bool wrap = sg0 + D >= sppD;
+                const uint32_t nrb_i = wrap ? rb + 1 : rb;
+                const uint32_t nsg0 = wrap ? 0u : sg0 + D;
+#pragma unroll
+                for (int d = 0; d < D; d++) {
+                    const uint32_t sg = sg0 + d;
+                    const bool valid = sg < a.spp;
+                    const uint32_t c = (kp * a.spp + min(sg, a.spp - 1)) * 16u + q;
+                    // operands from LDS
+                    m_u32x4 av[S][NP];
+                    float xs[S][MP];
+#pragma unroll
+                    for (int s = 0; s < S; s++) {
+#pragma unroll
+                        for (int p = 0; p < NP; p++)
+                            av[s][p] = XL[(((size_t)s * NP + p) * a.nch + c) * MP + arow];
+#pragma unroll
+                        for (int i = 0; i < MP; i++) xs[s][i] = XS[((size_t)s * a.nch + c) * MP + i];
+                    }
+                    const uint32_t g = (c * (uint32_t)CPC) >> a.log2g;
+                    const float2 sb = SB[valid ? sb_row + g : rows_wg * a.gpr];
+                    const m_u32x4 wv = ring[d];
+                    ring[d] = __builtin_nontemporal_load(w_ptr(nrb_i, nsg0 + d));
+                    // codes -> B operands, MFMAs
+                    m_f32x4 acc[S];
+#pragma unroll
+                    for (int wi = 0; wi < 4; wi++) {
+                        const uint32_t word = wv[wi];
+                        uint32_t pw[PF / 2];
+#pragma unroll
+                        for (int j = 0; j < PF / 2; j++) pw[j] = ((word >> (BITS * j)) & MASK) | MAGIC2;
+#pragma unroll
+                        for (int t = 0; t < PF / 4; t++) {
+                            const int m = wi * (PF / 4) + t;       // MFMA index within the chunk
+                            const m_u32x2 b = {pw[2 * t], pw[2 * t + 1]};
+#pragma unroll
+                            for (int s = 0; s < S; s++) {
+                                const m_u32x4 piece = av[s][m / 2];
+                                const m_u32x2 aop = (m & 1) ? m_u32x2{piece.z, piece.w} : m_u32x2{piece.x, piece.y};
+                                const m_f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                                acc[s] = mfma4<DT>(aop, b, m == 0 ? zero : acc[s]);
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int s = 0; s < S; s++)
+#pragma unroll
+                        for (int i = 0; i < MP; i++) {
+                            tot[s][i] = fmaf(sb.x, acc[s][i], tot[s][i]);
+                            tot[s][i] = fmaf(sb.y, xs[s][i], tot[s][i]);
+                        }
+                }
+            }
+            // lanes of one weight row (same r, all q) add up: q spans lane bits 2..5
+#pragma unroll
+            for (int s = 0; s < S; s++)
+#pragma unroll
+                for (int i = 0; i < MP; i++) {
+                    float v = tot[s][i];
+                    v += dpp_f32<0x124>(v);  // row_ror:4
+                    v += dpp_f32<0x128>(v);  // row_ror:8
+                    v += __shfl_xor(v, 16, 64);
+                    v += __shfl_xor(v, 32, 64);
+                    if (q == 0) RED[((size_t)kp * rows_wg + row_local) * R + s * MP + i] = v;
+                }
+        }
+        __syncthreads();
+
+        // ---- add the K parts and store ----------------------------------------
+        const uint32_t live = min((uint32_t)R, cnt - base_row);
+        for (uint32_t idx = tid; idx < rows_wg * live; idx += TPB) {
+            const uint32_t i = idx / rows_wg, rl = idx - i * rows_wg;
+            const uint32_t row = row0 + rl;
+            if (row >= a.N) continue;
+            float v = 0.f;
+            for (uint32_t k2 = 0; k2 < a.KP; k2++) v += RED[((size_t)k2 * rows_wg + rl) * R + i];
+            const uint32_t t = batch_row(base_row + i);
+            store_elem<DT>(a.out, (size_t)t * a.N + row, v);
+        }
+        if (pass + 1 < n_pass) __syncthreads();
+    }
+}
+
+template <int DT, int BITS, int MP, int S, int MODE>
+int qmv_mfma_launch_one(QmvMArgs& a, const QmvMGeom& g, const LaunchCtx& lc) {
+    constexpr int MAXT = S >= 2 ? 512 : 1024;
+    if (g.tpb > (uint32_t)MAXT) return fail(ERR_UNSUPPORTED, "mfma qmv: workgroup too large for this row count");
+    const void* fn = (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT>;
+    if (g.shmem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.shmem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
+    }
+    void* args[] = {&a};
+    hipError_t e = launch_kernel(fn, g.grid, dim3(g.tpb), args, g.shmem, lc);
+    if (e != hipSuccess) return hip_fail(e, "mfma qmv kernel launch");
+    return ERR_OK;
+}
+
+template <int DT, int BITS, int MODE>
+int qmv_mfma_launch_rows(QmvMArgs& a, const QmvMGeom& g, const LaunchCtx& lc) {
+    if constexpr (MODE == GATHER_SINGLE) {
+        return qmv_mfma_launch_one<DT, BITS, 1, 1, MODE>(a, g, lc);
+    } else if constexpr (MODE == GATHER_NONE) {
+        if (g.s == 1) {
+            switch (g.mp) {
+                case 1: return qmv_mfma_launch_one<DT, BITS, 1, 1, MODE>(a, g, lc);
+                case 2: return qmv_mfma_launch_one<DT, BITS, 2, 1, MODE>(a, g, lc);
+                default: return qmv_mfma_launch_one<DT, BITS, 4, 1, MODE>(a, g, lc);
+            }
+        }
+        if (g.s == 2) return qmv_mfma_launch_one<DT, BITS, 4, 2, MODE>(a, g, lc);
+        return qmv_mfma_launch_one<DT, BITS, 4, 4, MODE>(a, g, lc);
+    } else {
+        if (g.s == 1) return qmv_mfma_launch_one<DT, BITS, 4, 1, MODE>(a, g, lc);
+        if (g.s == 2) return qmv_mfma_launch_one<DT, BITS, 4, 2, MODE>(a, g, lc);
+        return qmv_mfma_launch_one<DT, BITS, 4, 4, MODE>(a, g, lc);
+    }
+}
+
+template <int DT, int BITS>
+int qmv_mfma_launch_mode(QmvMArgs& a, int mode, const QmvMGeom& g, const LaunchCtx& lc) {
+    switch (mode) {
+        case GATHER_NONE: return qmv_mfma_launch_rows<DT, BITS, GATHER_NONE>(a, g, lc);
+        case GATHER_CSR: return qmv_mfma_launch_rows<DT, BITS, GATHER_CSR>(a, g, lc);
+        case GATHER_INDICES: return qmv_mfma_launch_rows<DT, BITS, GATHER_INDICES>(a, g, lc);
+        default: return qmv_mfma_launch_rows<DT, BITS, GATHER_SINGLE>(a, g, lc);
+    }
+}
+
+template <int DT> int qmv_mfma_launch_dtype(QmvMArgs& a, int bits, int mode, const QmvMGeom& g, const LaunchCtx& lc) {
+    switch (bits) {
+        case 2: return qmv_mfma_launch_mode<DT, 2>(a, mode, g, lc);
+        case 4: return qmv_mfma_launch_mode<DT, 4>(a, mode, g, lc);
+        default:
+            if constexpr (DT == DT_F16) return qmv_mfma_launch_mode<DT, 8>(a, mode, g, lc);
+            else return fail(ERR_UNSUPPORTED, "mfma qmv: 8-bit codes need f16 activations");
+    }
+}
+
+}  // namespace mtq
