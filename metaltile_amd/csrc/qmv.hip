@@ -106,9 +106,16 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
 }
 
 int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {
-    if (options().qmv_mfma != 1) {
-        int rc = launch_qmv_mfma(p, lc);
-        if (rc != ERR_UNSUPPORTED) return rc;
+    {
+        // The matrix-core kernel wins as soon as more than one activation row shares
+        // the weight stream (and for every gather); a single row is as fast on the
+        // dot2 kernels below.
+        const bool many = p.gather == GATHER_CSR || p.gather == GATHER_INDICES || (p.gather == GATHER_NONE && p.M >= 2);
+        const int mode = options().qmv_mfma;
+        if (mode == 2 || (mode == 0 && many)) {
+            int rc = launch_qmv_mfma(p, lc);
+            if (rc != ERR_UNSUPPORTED) return rc;
+        }
     }
     if (p.bits != 2 && p.bits != 4 && p.bits != 8)
         return fail(ERR_UNSUPPORTED, "fast qmv: bits must be 2, 4 or 8");

@@ -74,11 +74,25 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
         s = avg > 4 ? 4 : (avg > 2 ? 2 : 1);
         if (p.bits == 2 && s > 2) s = 2;  // the 16-row 2-bit variant does not fit the register file
     }
-    const uint32_t maxt = s >= 2 ? 512u : 1024u;
+    const uint32_t maxt = (s >= 4 || (s >= 2 && p.bits == 2)) ? 512u : 1024u;
     if (64u * KP > maxt) return fail(ERR_UNSUPPORTED, "mfma qmv: too many K parts");
-    uint32_t RBW = opt.qmv_mfma_rbw ? (uint32_t)opt.qmv_mfma_rbw : (256u / (64u * KP) ? 256u / (64u * KP) : 1u);
-    while (64u * KP * RBW > maxt && RBW > 1) RBW--;
-    uint32_t nrb = opt.qmv_mfma_nrb ? (uint32_t)opt.qmv_mfma_nrb : 1u;
+    // Rows per workgroup: about one to two workgroups per compute unit (measured
+    // best on 14336x4096, 4096x14336 and 8192x8192), as many of the row blocks
+    // side by side as the workgroup size allows, the rest one after the other.
+    uint32_t rows_target = 8;
+    while (rows_target < 32 && (uint64_t)rows_target * 2 * 256 <= p.N) rows_target *= 2;
+    // A gather workgroup stages up to R activation rows of K elements before it
+    // streams: give it four times the rows so that staging stays small beside
+    // the weights it serves.
+    if (gather) rows_target = 128;
+    uint32_t RBW = rows_target / 4 < 16 ? rows_target / 4 : 16;
+    while (64u * KP * RBW > maxt && RBW > 1) RBW /= 2;
+    uint32_t nrb = rows_target / 4 / RBW;
+    if (opt.qmv_mfma_rbw) {
+        RBW = (uint32_t)opt.qmv_mfma_rbw;
+        if (64u * KP * RBW > maxt) return fail(ERR_BAD_ARG, "qmv.mfma_rbw: workgroup too large");
+    }
+    if (opt.qmv_mfma_nrb) nrb = (uint32_t)opt.qmv_mfma_nrb;
     const uint32_t list_cap = p.gather == GATHER_INDICES ? p.T : 0;
     // shrink until the workgroup's LDS fits
     while (lds_bytes((uint32_t)(mp * s), p.K, nch, 4 * RBW * nrb, gpr, KP, list_cap) > kLdsBudget) {

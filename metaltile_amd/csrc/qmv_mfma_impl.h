@@ -38,7 +38,17 @@
 #include "mtq_device.h"
 #include "mtq_internal.h"
 
+#include <type_traits>
+
 namespace mtq {
+
+// Keeps memory operations from being moved across this point by the optimiser
+// and by the machine scheduler; emits no instruction.
+#define MTQ_MFMA_KEEP_ORDER()               \
+    do {                                    \
+        asm volatile("" ::: "memory");      \
+        __builtin_amdgcn_sched_barrier(0);  \
+    } while (0)
 
 typedef uint32_t m_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t m_u32x2 __attribute__((ext_vector_type(2)));
@@ -175,52 +185,34 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
 
     const uint32_t n_pass = (MODE == GATHER_CSR || MODE == GATHER_INDICES) ? (cnt + R - 1) / R : 1u;
     for (uint32_t pass = 0; pass < n_pass; pass++) {
-        // ---- weights first: D loads per lane in flight during the staging ----
-        m_u32x4 ring[D];
-#pragma unroll
-        for (int d = 0; d < D; d++) ring[d] = __builtin_nontemporal_load(w_ptr(0, d));
-
-        // ---- (s, b - MAGIC*s) pairs of the workgroup's rows -------------------
-        if (pass == 0) {
-            const uint32_t nvec = rows_wg * a.gpr / 4;
-            for (uint32_t v = tid; v < nvec; v += TPB) {
-                const uint32_t e = v * 4, rl = e / a.gpr, g = e - rl * a.gpr;
-                const size_t src = (slab_rows + min(row0 + rl, a.N - 1)) * a.gpr + g;
-                const uint2 sv = *(const uint2*)((const uint16_t*)a.scales + src);
-                const uint2 bv = *(const uint2*)((const uint16_t*)a.biases + src);
-                float s4[4], b4[4];
-                if constexpr (DT == DT_BF16) {
-                    s4[0] = bf16_bits_to_f32(sv.x & 0xFFFFu); s4[1] = bf16_bits_to_f32(sv.x >> 16);
-                    s4[2] = bf16_bits_to_f32(sv.y & 0xFFFFu); s4[3] = bf16_bits_to_f32(sv.y >> 16);
-                    b4[0] = bf16_bits_to_f32(bv.x & 0xFFFFu); b4[1] = bf16_bits_to_f32(bv.x >> 16);
-                    b4[2] = bf16_bits_to_f32(bv.y & 0xFFFFu); b4[3] = bf16_bits_to_f32(bv.y >> 16);
-                } else {
-                    s4[0] = f16_bits_to_f32(sv.x & 0xFFFFu); s4[1] = f16_bits_to_f32(sv.x >> 16);
-                    s4[2] = f16_bits_to_f32(sv.y & 0xFFFFu); s4[3] = f16_bits_to_f32(sv.y >> 16);
-                    b4[0] = f16_bits_to_f32(bv.x & 0xFFFFu); b4[1] = f16_bits_to_f32(bv.x >> 16);
-                    b4[2] = f16_bits_to_f32(bv.y & 0xFFFFu); b4[3] = f16_bits_to_f32(bv.y >> 16);
-                }
-                float4* dst = (float4*)(SB + e);
-                dst[0] = make_float4(s4[0], b4[0] - MAGIC * s4[0], s4[1], b4[1] - MAGIC * s4[1]);
-                dst[1] = make_float4(s4[2], b4[2] - MAGIC * s4[2], s4[3], b4[3] - MAGIC * s4[3]);
-            }
-            if (tid == 0) SB[rows_wg * a.gpr] = make_float2(0.f, 0.f);
-        }
-
-        // ---- activations of this pass: permute into operand order, chunk sums --
+        // Loads return in issue order, so the small ones go first: this thread's
+        // first activation chunk and its first four (scale, bias) elements, then D
+        // weight loads per lane, which stay in flight while the small data are
+        // staged into LDS. All of it is straight-line code on clamped addresses so
+        // that the waits count exactly.
         const uint32_t base_row = pass * R;
-        for (uint32_t task = tid; task < (uint32_t)R * a.nch; task += TPB) {
+        const uint32_t live = min((uint32_t)R, cnt - base_row);
+        // Rows past the pass's last live row are never staged: what the matrix
+        // cores compute from their LDS slots lands in output rows nobody stores.
+        const uint32_t ntask = live * a.nch;
+        const uint32_t nvec = rows_wg * a.gpr / 4;
+        uint32_t raw[NP * 4];
+        bool row_live;
+        auto x_load = [&](uint32_t task) {
             const uint32_t i = task / a.nch, c = task - i * a.nch;
-            const uint32_t t = batch_row(base_row + i);
-            uint32_t raw[NP * 4];
-            if (t != NOROW) {
-                const m_u32x4* src = (const m_u32x4*)((const uint16_t*)a.x + (size_t)t * a.K + (size_t)c * CPC);
+            uint32_t t = batch_row(base_row + i);
+            row_live = t != NOROW;
+            if (!row_live) t = batch_row(base_row);  // the pass's first row always exists
+            const m_u32x4* src = (const m_u32x4*)((const uint16_t*)a.x + (size_t)t * a.K + (size_t)c * CPC);
 #pragma unroll
-                for (int p = 0; p < NP; p++) {
-                    const m_u32x4 v = src[p];
-                    raw[4 * p] = v.x; raw[4 * p + 1] = v.y; raw[4 * p + 2] = v.z; raw[4 * p + 3] = v.w;
-                }
-            } else {
+            for (int p = 0; p < NP; p++) {
+                const m_u32x4 v = src[p];
+                raw[4 * p] = v.x; raw[4 * p + 1] = v.y; raw[4 * p + 2] = v.z; raw[4 * p + 3] = v.w;
+            }
+        };
+        auto x_store = [&](uint32_t task) {
+            const uint32_t i = task / a.nch, c = task - i * a.nch;
+            if (!row_live) {
 #pragma unroll
                 for (int j = 0; j < NP * 4; j++) raw[j] = 0u;
             }
@@ -250,20 +242,72 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                 m_u32x4 piece = {o[0], o[1], o[2], o[3]};
                 XL[(((size_t)s * NP + p) * a.nch + c) * MP + i4] = piece;
             }
+        };
+        uint2 sv, bv;
+        auto sb_load = [&](uint32_t v) {
+            const uint32_t e = v * 4, rl = e / a.gpr, g = e - rl * a.gpr;
+            const size_t src = (slab_rows + min(row0 + rl, a.N - 1)) * a.gpr + g;
+            sv = *(const uint2*)((const uint16_t*)a.scales + src);
+            bv = *(const uint2*)((const uint16_t*)a.biases + src);
+        };
+        auto sb_store = [&](uint32_t v) {
+            float s4[4], b4[4];
+            if constexpr (DT == DT_BF16) {
+                s4[0] = bf16_bits_to_f32(sv.x & 0xFFFFu); s4[1] = bf16_bits_to_f32(sv.x >> 16);
+                s4[2] = bf16_bits_to_f32(sv.y & 0xFFFFu); s4[3] = bf16_bits_to_f32(sv.y >> 16);
+                b4[0] = bf16_bits_to_f32(bv.x & 0xFFFFu); b4[1] = bf16_bits_to_f32(bv.x >> 16);
+                b4[2] = bf16_bits_to_f32(bv.y & 0xFFFFu); b4[3] = bf16_bits_to_f32(bv.y >> 16);
+            } else {
+                s4[0] = f16_bits_to_f32(sv.x & 0xFFFFu); s4[1] = f16_bits_to_f32(sv.x >> 16);
+                s4[2] = f16_bits_to_f32(sv.y & 0xFFFFu); s4[3] = f16_bits_to_f32(sv.y >> 16);
+                b4[0] = f16_bits_to_f32(bv.x & 0xFFFFu); b4[1] = f16_bits_to_f32(bv.x >> 16);
+                b4[2] = f16_bits_to_f32(bv.y & 0xFFFFu); b4[3] = f16_bits_to_f32(bv.y >> 16);
+            }
+            float4* dst = (float4*)(SB + (size_t)v * 4);
+            dst[0] = make_float4(s4[0], b4[0] - MAGIC * s4[0], s4[1], b4[1] - MAGIC * s4[1]);
+            dst[1] = make_float4(s4[2], b4[2] - MAGIC * s4[2], s4[3], b4[3] - MAGIC * s4[3]);
+        };
+
+        x_load(min(tid, ntask - 1));
+        if (pass == 0) sb_load(min(tid, nvec - 1));
+        MTQ_MFMA_KEEP_ORDER();
+        m_u32x4 ring[D];
+#pragma unroll
+        for (int d = 0; d < D; d++) ring[d] = __builtin_nontemporal_load(w_ptr(0, d));
+        MTQ_MFMA_KEEP_ORDER();
+        if (tid < ntask) x_store(tid);
+        if (pass == 0) {
+            if (tid < nvec) sb_store(tid);
+            if (tid == 0) SB[rows_wg * a.gpr] = make_float2(0.f, 0.f);
+            for (uint32_t v = tid + TPB; v < nvec; v += TPB) {
+                sb_load(v);
+                sb_store(v);
+            }
+        }
+        for (uint32_t task = tid + TPB; task < ntask; task += TPB) {
+            x_load(task);
+            x_store(task);
         }
         __syncthreads();
 
         // ---- stream ------------------------------------------------------------
         const uint32_t arow = r & (uint32_t)(MP - 1);
-        for (uint32_t rb = 0; rb < a.nrb; rb++) {
-            float tot[S][MP];
+        const uint32_t kor = magic_or_vgpr<DT>();
+        // One ring turn = D steps. Every turn but the wave's last issues the loads
+        // of the turn after it; the last one is a separate copy of the body without
+        // loads, so no load is ever issued twice and the loop stays branch-free
+        // around its loads.
+        float tot[S][MP];
 #pragma unroll
-            for (int s = 0; s < S; s++)
+        for (int s = 0; s < S; s++)
 #pragma unroll
-                for (int i = 0; i < MP; i++) tot[s][i] = 0.f;
+            for (int i = 0; i < MP; i++) tot[s][i] = 0.f;
+        uint32_t rb = 0, sg0 = 0;
+        auto turn = [&](auto issue_tag) {
+            constexpr bool ISSUE = decltype(issue_tag)::value;
             const uint32_t row_local = (rb * a.RBW + rbw) * 4u + r;
             const uint32_t sb_row = row_local * a.gpr;
-            for (uint32_t sg0 = 0; sg0 < sppD; sg0 += D) {
+            {
                 const bool wrap = sg0 + D >= sppD;
                 const uint32_t nrb_i = wrap ? rb + 1 : rb;
                 const uint32_t nsg0 = wrap ? 0u : sg0 + D;
@@ -286,7 +330,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                     const uint32_t g = (c * (uint32_t)CPC) >> a.log2g;
                     const float2 sb = SB[valid ? sb_row + g : rows_wg * a.gpr];
                     const m_u32x4 wv = ring[d];
-                    ring[d] = __builtin_nontemporal_load(w_ptr(nrb_i, nsg0 + d));
+                    if constexpr (ISSUE) ring[d] = __builtin_nontemporal_load(w_ptr(nrb_i, nsg0 + d));
                     // codes -> B operands, MFMAs
                     m_f32x4 acc[S];
 #pragma unroll
@@ -294,7 +338,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                         const uint32_t word = wv[wi];
                         uint32_t pw[PF / 2];
 #pragma unroll
-                        for (int j = 0; j < PF / 2; j++) pw[j] = ((word >> (BITS * j)) & MASK) | MAGIC2;
+                        for (int j = 0; j < PF / 2; j++) pw[j] = ((word >> (BITS * j)) & MASK) | kor;
 #pragma unroll
                         for (int t = 0; t < PF / 4; t++) {
                             const int m = wi * (PF / 4) + t;       // MFMA index within the chunk
@@ -316,24 +360,33 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                             tot[s][i] = fmaf(sb.y, xs[s][i], tot[s][i]);
                         }
                 }
-            }
-            // lanes of one weight row (same r, all q) add up: q spans lane bits 2..5
+                if (wrap) {
+                    // lanes of one weight row (same r, all q) add up: q spans lane bits 2..5
 #pragma unroll
-            for (int s = 0; s < S; s++)
+                    for (int s = 0; s < S; s++)
 #pragma unroll
-                for (int i = 0; i < MP; i++) {
-                    float v = tot[s][i];
-                    v += dpp_f32<0x124>(v);  // row_ror:4
-                    v += dpp_f32<0x128>(v);  // row_ror:8
-                    v += __shfl_xor(v, 16, 64);
-                    v += __shfl_xor(v, 32, 64);
-                    if (q == 0) RED[((size_t)kp * rows_wg + row_local) * R + s * MP + i] = v;
+                        for (int i = 0; i < MP; i++) {
+                            float v = tot[s][i];
+                            v += dpp_f32<0x124>(v);  // row_ror:4
+                            v += dpp_f32<0x128>(v);  // row_ror:8
+                            v += __shfl_xor(v, 16, 64);
+                            v += __shfl_xor(v, 32, 64);
+                            if (q == 0) RED[((size_t)kp * rows_wg + row_local) * R + s * MP + i] = v;
+                            tot[s][i] = 0.f;
+                        }
+                    rb++;
+                    sg0 = 0;
+                } else {
+                    sg0 += D;
                 }
-        }
+            }
+        };
+        const uint32_t n_turns = a.nrb * (sppD / D);
+        for (uint32_t it = 0; it + 1 < n_turns; it++) turn(std::true_type{});
+        turn(std::false_type{});
         __syncthreads();
 
         // ---- add the K parts and store ----------------------------------------
-        const uint32_t live = min((uint32_t)R, cnt - base_row);
         for (uint32_t idx = tid; idx < rows_wg * live; idx += TPB) {
             const uint32_t i = idx / rows_wg, rl = idx - i * rows_wg;
             const uint32_t row = row0 + rl;
@@ -349,7 +402,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
 
 template <int DT, int BITS, int MP, int S, int MODE>
 int qmv_mfma_launch_one(QmvMArgs& a, const QmvMGeom& g, const LaunchCtx& lc) {
-    constexpr int MAXT = S >= 2 ? 512 : 1024;
+    constexpr int MAXT = (S >= 4 || (S >= 2 && BITS == 2)) ? 512 : 1024;
     if (g.tpb > (uint32_t)MAXT) return fail(ERR_UNSUPPORTED, "mfma qmv: workgroup too large for this row count");
     const void* fn = (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT>;
     if (g.shmem > 48 * 1024) {
