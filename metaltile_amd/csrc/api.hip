@@ -134,11 +134,15 @@ static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s,
     if (rc) return rc;
     if (M == 0) return ERR_OK;
     if (!w || !s || !b || !x || !out) return fail(ERR_BAD_ARG, "null buffer");
-    if (M >= 16 || force_mma) {
+    if (M >= 32 || force_mma) {
         QmmParams q;
         q.dtype = dtype; q.bits = bits; q.group_size = G;
         q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
         q.M = M; q.N = N; q.K = K;
+        if (options().qmm_kernel != 1) {
+            rc = launch_qmm_direct(q, lc);
+            if (rc != ERR_UNSUPPORTED) return rc;
+        }
         rc = launch_qmm_mfma(q, lc);
         if (rc != ERR_UNSUPPORTED) return rc;
     }
@@ -735,6 +739,16 @@ int mtq_set_option(const char* name, int value) {
         if (name[9] == 'k') options().qmv_mfma_kp = value;
         else if (name[9] == 'r') options().qmv_mfma_rbw = value;
         else options().qmv_mfma_nrb = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmm.kernel")) {
+        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmm.kernel must be 0 (auto), 1 (LDS tiling) or 2 (direct)");
+        options().qmm_kernel = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmm.tile_rows")) {
+        if (value != 0 && value != 64 && value != 128) return fail(ERR_BAD_ARG, "qmm.tile_rows must be 0, 64 or 128");
+        options().qmm_tile_rows = value;
         return MTQ_OK;
     }
     if (!strcmp(name, "qmm.splits")) {

@@ -75,6 +75,8 @@ struct Options {
     int qmv_stream_depth = 0;     // streaming kernel: ring depth (4 / 8)
     int qmv_stream_batches = 0;   // streaming kernel: batches per thread
     int qmm_splits = 0;           // MFMA qmm: K splits per tile (0 = choose per shape)
+    int qmm_kernel = 0;           // MFMA qmm: 0 auto, 1 both operands through LDS, 2 weights direct to registers
+    int qmm_tile_rows = 0;        // direct qmm: activation rows per tile (0 = choose; 64, 128)
     int qmv_mfma = 0;             // matrix-core qmv: 0 auto, 1 never, 2 whenever the shape fits
     int qmv_mfma_kp = 0;          // matrix-core qmv: K parts per row block
     int qmv_mfma_rbw = 0;         // matrix-core qmv: row blocks walked in parallel per workgroup
@@ -103,5 +105,7 @@ struct QmmParams {
 };
 // Tiled MFMA GEMM with weights dequantised into LDS (qmm.hip).
 int launch_qmm_mfma(const QmmParams& p, const LaunchCtx& lc);
+// 64x128 tiles, weights converted in MFMA operand registers, activations through LDS (qmm_direct.hip).
+int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc);
 
 }  // namespace mtq

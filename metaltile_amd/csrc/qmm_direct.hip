@@ -1,0 +1,253 @@
+// qmm for gfx950, second tiling: weights go from global memory straight into
+// MFMA operand registers; only the activation tile passes through LDS.
+//
+// Replaces the same reference kernels as qmm.hip (mt_qmm_mma / _m16 / _int8 /
+// _m16_int8 / _int2, crates/metaltile-std/src/mlx/quantized.rs:2106-2405, 2408,
+// 2731, 2990, 3330) with the same semantics: s*q + b is rounded to the element
+// dtype before the multiply (quantized.rs:2267-2274), products accumulate in
+// f32, the result is rounded on store.
+//
+// Why a second tiling. LDS on this part reads ~230 B/clk per compute unit but
+// writes only ~70 B/clk, so a tile that writes both operands to LDS is bound by
+// those writes; and at M = 512 a 128x128 tiling yields 128 workgroups for 256
+// compute units. Here a workgroup of 512 threads (8 waves) owns a 64 (M) x 128
+// (N) tile: 256 workgroups at M = 512. The eight waves are 2 K-groups x 4
+// N-waves: per iteration of 128 k, K-group g takes k in [64g, 64g+64) and wave
+// wn the weight rows [32wn, 32wn+32). A lane of the 32x32x16 MFMA layout (row
+// l%32, k-half l/32) loads exactly its own 32 codes of that 64-k slice (one
+// 4*bits-byte load), its row's scale and bias for that slice, converts eight
+// codes per MFMA step and never shares them: no weight byte is written to LDS
+// and no code is converted twice. The 64 x 128 activation tile is written to LDS
+// once per iteration (32 bytes per thread) and read by every wave of the
+// matching K-group. Two waves per SIMD (one of each K-group) let one wave's
+// conversions run under the other's MFMAs. The K-groups' accumulators meet in
+// LDS once, at the end.
+//
+// Loads run two iterations ahead (two register sets); the activation tile is
+// double-buffered in LDS; one barrier per iteration. Workgroup ids are remapped
+// so that an XCD (ids congruent mod 8) works on all M-tiles of a contiguous run
+// of N-tiles: its L2 holds its slice of W once and X once.
+#include "mtq_internal.h"
+#include "qmm_common.h"
+
+namespace mtq {
+
+// Keeps memory operations from being moved across this point by the optimiser
+// and the machine scheduler (loads must be issued a full iteration before the
+// values are needed); emits no instruction.
+#define QD_KEEP_ORDER()                     \
+    do {                                    \
+        asm volatile("" ::: "memory");      \
+        __builtin_amdgcn_sched_barrier(0);  \
+    } while (0)
+
+struct QmmDArgs {
+    const unsigned char* w;
+    const unsigned char* scales;
+    const unsigned char* biases;
+    const unsigned char* x;
+    void* out;
+    uint32_t M, N, K;
+    uint32_t log2g, gpr;
+    uint32_t m_tiles, n_tiles, iters;
+    uint32_t m_tile_rows;  // 64 or 128
+};
+
+constexpr int DBN = 128, DBK = 128;
+constexpr int DLD = DBK * 2 + 16;        // LDS row stride in bytes
+
+// MB = 32-row activation blocks per wave (tile height DBM = 32*MB): every
+// converted weight fragment feeds MB MFMAs, so the conversion cost per MFMA
+// falls with MB; MB = 4 is the compute-bound shape, MB = 2 gives twice the
+// workgroups for small M.
+template <int DT, int BITS, int PD, int MB>
+__global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
+    constexpr int DBM = 32 * MB;
+    constexpr int DBUF = DBM * DLD;          // one activation tile
+    constexpr int XV = DBM * DBK * 2 / 512 / 16;  // 16-byte vectors of the tile per thread
+    extern __shared__ __align__(16) unsigned char lds[];  // 2 * DBUF bytes
+    static_assert(2 * DBUF >= DBM * DBN * 4, "the K-group reduction reuses the tile buffers");
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t kg = wave >> 2, wn = wave & 3u;
+    const uint32_t fr = lane & 31u, fh = lane >> 5;
+
+    const uint32_t total = a.m_tiles * a.n_tiles;
+    uint32_t vid = blockIdx.x;
+    if (total % 8 == 0) vid = (blockIdx.x & 7u) * (total / 8) + (blockIdx.x >> 3);
+    const uint32_t nt = vid / a.m_tiles, mt = vid % a.m_tiles;
+    const uint32_t m0 = mt * DBM, n0 = nt * DBN;
+
+    // activations: thread t moves 32 bytes of row t/8 (bytes [32*(t%8), +32) of the iteration's 256)
+    const uint32_t xr = tid >> 3, xc = tid & 7u;
+    uint32_t xoff[XV / 2];
+#pragma unroll
+    for (int i = 0; i < XV / 2; i++) xoff[i] = min(m0 + xr + 64 * i, a.M - 1) * (a.K * 2) + xc * 32;
+    // weights: row n0 + 32*wn + fr, codes [64*kg + 32*fh, +32) of the iteration
+    const uint32_t wrow = n0 + wn * 32 + fr;  // < N: N is a multiple of 128
+    const uint32_t woff = wrow * (a.K * BITS / 8) + (kg * 64 + fh * 32) * BITS / 8;
+    const uint32_t soff = wrow * a.gpr * 2;
+    const uint32_t kofs = kg * 64 + fh * 32;  // k offset of this lane's codes inside an iteration
+
+    // PD register sets: the loads of iteration it + PD are issued at the top of
+    // iteration it, so PD iterations of work cover the memory latency.
+    q_u32x4 px[PD][XV];
+    uint32_t pw[PD][BITS];
+    uint32_t ps[PD], pb[PD];
+
+#define QD_LOAD(IT, SET)                                                                 \
+    do {                                                                                 \
+        const uint32_t it_ = min((uint32_t)(IT), a.iters - 1);                           \
+        const unsigned char* xs_ = a.x + (size_t)it_ * (DBK * 2);                        \
+        _Pragma("unroll") for (int i = 0; i < XV / 2; i++) {                             \
+            px[SET][2 * i] = *(const q_u32x4*)(xs_ + xoff[i]);                           \
+            px[SET][2 * i + 1] = *(const q_u32x4*)(xs_ + xoff[i] + 16);                  \
+        }                                                                                \
+        const unsigned char* ws_ = a.w + (size_t)it_ * (DBK * BITS / 8) + woff;          \
+        if constexpr (BITS == 2) {                                                       \
+            const uint2 t_ = *(const uint2*)(ws_);                                       \
+            pw[SET][0] = t_.x;                                                           \
+            pw[SET][1] = t_.y;                                                           \
+        } else {                                                                         \
+            _Pragma("unroll") for (int i = 0; i < BITS / 4; i++) {                       \
+                const q_u32x4 t_ = *(const q_u32x4*)(ws_ + 16 * i);                      \
+                pw[SET][4 * i] = t_.x;                                                   \
+                pw[SET][4 * i + 1] = t_.y;                                               \
+                pw[SET][4 * i + 2] = t_.z;                                               \
+                pw[SET][4 * i + 3] = t_.w;                                               \
+            }                                                                            \
+        }                                                                                \
+        const uint32_t g_ = (it_ * DBK + kofs) >> a.log2g;                               \
+        ps[SET] = *(const uint16_t*)(a.scales + soff + (size_t)g_ * 2);                  \
+        pb[SET] = *(const uint16_t*)(a.biases + soff + (size_t)g_ * 2);                  \
+    } while (0)
+
+#define QD_STORE_X(BUF, SET)                                                             \
+    do {                                                                                 \
+        unsigned char* d_ = lds + (BUF) * DBUF + xr * DLD + xc * 32;                     \
+        _Pragma("unroll") for (int i = 0; i < XV / 2; i++) {                             \
+            *(q_u32x4*)(d_ + 64 * i * DLD) = px[SET][2 * i];                             \
+            *(q_u32x4*)(d_ + 64 * i * DLD + 16) = px[SET][2 * i + 1];                    \
+        }                                                                                \
+    } while (0)
+
+    f32x16 acc[MB];
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[i][v] = 0.f;
+
+#pragma unroll
+    for (int j = 0; j < PD; j++) QD_LOAD(j, j);
+    QD_STORE_X(0, 0);
+    __syncthreads();
+
+    // fragment of activation row (32*bi + fr), k = kofs + 8*j .. +8 of the iteration
+    const unsigned char* Abase = lds + fr * DLD + kofs * 2;
+    for (uint32_t it0 = 0; it0 < a.iters; it0 += PD) {
+#pragma unroll
+        for (int par = 0; par < PD; par++) {
+            const uint32_t it = it0 + par;
+            // set `par` holds iteration `it`: copy out what the MFMAs need, refill with it+PD
+            uint32_t cw[BITS];
+#pragma unroll
+            for (int i = 0; i < BITS; i++) cw[i] = pw[par][i];
+            const float s = elem_bits_to_f32<DT>(ps[par]), b = elem_bits_to_f32<DT>(pb[par]);
+            QD_LOAD(it + PD, par);
+            QD_KEEP_ORDER();
+            const unsigned char* A0 = Abase + (par & 1) * DBUF;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                uint4 af[MB];
+#pragma unroll
+                for (int bi = 0; bi < MB; bi++) af[bi] = *(const uint4*)(A0 + bi * 32 * DLD + j * 16);
+                const uint4 bq = dequant8<DT, BITS>(cw, j, s, b);
+#pragma unroll
+                for (int bi = 0; bi < MB; bi++) acc[bi] = mfma32<DT>(af[bi], bq, acc[bi]);
+            }
+            // activations of it+1 (next set, loaded PD-1 iterations ago) go to the other buffer
+            QD_KEEP_ORDER();
+            QD_STORE_X((par + 1) & 1, (par + 1) % PD);
+            __syncthreads();
+        }
+    }
+#undef QD_LOAD
+#undef QD_STORE_X
+
+    // ---- K-group 1 hands its accumulators to K-group 0 through LDS -----------
+    float* red = (float*)lds;  // [wn][bi][v][lane]
+    if (kg == 1) {
+#pragma unroll
+        for (int bi = 0; bi < MB; bi++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) red[((wn * MB + bi) * 16 + v) * 64 + lane] = acc[bi][v];
+    }
+    __syncthreads();
+    if (kg == 1) return;
+    // accumulator layout: column j = lane%32, row i = 8*(v/4) + 4*(lane/32) + v%4
+    const uint32_t col = n0 + wn * 32 + fr;
+#pragma unroll
+    for (int bi = 0; bi < MB; bi++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const uint32_t row = m0 + bi * 32 + 8 * (v / 4) + 4 * fh + (v % 4);
+            const float r = acc[bi][v] + red[((wn * MB + bi) * 16 + v) * 64 + lane];
+            if (row < a.M) store_elem<DT>(a.out, (size_t)row * a.N + col, r);
+        }
+}
+
+template <int DT> static int launch_dt(QmmDArgs& a, int bits, const LaunchCtx& lc) {
+    const void* fn;
+    const bool tall = a.m_tile_rows == 128;
+    switch (bits) {
+        case 2: fn = tall ? (const void*)qmm_direct_kernel<DT, 2, 2, 4> : (const void*)qmm_direct_kernel<DT, 2, 2, 2>; break;
+        case 4: fn = tall ? (const void*)qmm_direct_kernel<DT, 4, 2, 4> : (const void*)qmm_direct_kernel<DT, 4, 2, 2>; break;
+        default: fn = tall ? (const void*)qmm_direct_kernel<DT, 8, 2, 4> : (const void*)qmm_direct_kernel<DT, 8, 2, 2>; break;
+    }
+    const size_t shmem = 2 * (size_t)a.m_tile_rows * DLD;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
+    void* args[] = {&a};
+    e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles), dim3(512), args, shmem, lc);
+    if (e != hipSuccess) return hip_fail(e, "qmm direct kernel launch");
+    return ERR_OK;
+}
+
+int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
+    if (p.dtype != DT_F16 && p.dtype != DT_BF16)
+        return fail(ERR_UNSUPPORTED, "direct qmm: f16 / bf16 activations only");
+    if (p.bits != 2 && p.bits != 4 && p.bits != 8) return fail(ERR_UNSUPPORTED, "direct qmm: bits must be 2, 4 or 8");
+    const uint32_t G = p.group_size;
+    if (p.M == 0 || p.N % DBN || p.K % (2 * DBK) || G < 32 || (G & (G - 1)) || p.K % G)
+        return fail(ERR_UNSUPPORTED, "direct qmm: N % 128, K % 256 or group size");
+    if ((uint64_t)p.M * p.K * 2 >= (1ull << 32) || (uint64_t)p.N * p.K * p.bits / 8 >= (1ull << 32))
+        return fail(ERR_UNSUPPORTED, "direct qmm: operand larger than 4 GiB");
+    if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16) return fail(ERR_UNSUPPORTED, "direct qmm: w and x must be 16-byte aligned");
+    QmmDArgs a;
+    a.w = (const unsigned char*)p.w;
+    a.scales = (const unsigned char*)p.scales;
+    a.biases = (const unsigned char*)p.biases;
+    a.x = (const unsigned char*)p.x;
+    a.out = p.out;
+    a.M = p.M;
+    a.N = p.N;
+    a.K = p.K;
+    uint32_t l = 0;
+    while ((1u << l) < G) l++;
+    a.log2g = l;
+    a.gpr = p.K / G;
+    // 128-row tiles convert each weight once per 4 MFMAs instead of once per 2, but
+    // halve the workgroup count: used once they still fill the chip (measured at
+    // N = K = 4096: M = 512 runs 40 us on 64-row tiles, 50 us on 128-row tiles;
+    // M = 2048 runs 157 us and 105 us).
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    const uint64_t tall_tiles = (uint64_t)((p.M + 127) / 128) * (p.N / DBN);
+    a.m_tile_rows = options().qmm_tile_rows ? (uint32_t)options().qmm_tile_rows : (tall_tiles >= (uint64_t)cus ? 128u : 64u);
+    a.m_tiles = (p.M + a.m_tile_rows - 1) / a.m_tile_rows;
+    a.n_tiles = p.N / DBN;
+    a.iters = p.K / DBK;  // even
+    return p.dtype == DT_BF16 ? launch_dt<DT_BF16>(a, p.bits, lc) : launch_dt<DT_F16>(a, p.bits, lc);
+}
+
+}  // namespace mtq
