@@ -37,7 +37,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=8, help="distinct MLP weight sets streamed per step")
-    ap.add_argument("--workload", default="qmv", choices=["qmv", "qmm", "gather", "copy"],
+    ap.add_argument("--workload", default="qmv", choices=["qmv", "qmm", "gather", "quantize", "dequantize", "copy"],
                     help="qmv is the headline; qmm / gather report the other configurations; "
                          "copy runs only the known-size copy kernel (counter calibration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -228,6 +228,41 @@ def main():
                          "frac": round(nbytes / kern_avg / 1e3 / HBM_PEAK_GBS, 4),
                          "traffic": traffic_from_profiles("gather_bf16_b4_e8"), "avg_launch_us_timed_region": round(kern_avg, 3),
                          "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(float(per.min()), 3)}},
+        })
+        print(json.dumps(out))
+        return
+
+    if a.workload in ("quantize", "dequantize"):
+        # the packed format's writer / reader on one Llama MLP matrix, 8 rotating copies
+        N, K, G, bits = 14336, 4096, 64, 4
+        n = N * K
+        rng = np.random.default_rng(9000)
+        wf = m.pack_f32((rng.standard_normal(n).astype(np.float32) * np.float32(0.05)), dt)
+        sets = 1 if a.hot else 6
+        specs, keep = [], []
+        for i in range(sets):
+            if a.workload == "quantize":
+                bufs = {"w": GpuBuffer.from_bytes(wf), "out": GpuBuffer(n * bits // 8),
+                        "scales": GpuBuffer(n // G * 2), "biases": GpuBuffer(n // G * 2)}
+            else:
+                c = make_case(9100, dt, bits, G, 1, N, K)
+                bufs = {"w": GpuBuffer.from_bytes(c.w.tobytes()), "scales": GpuBuffer.from_bytes(c.scales_bytes),
+                        "biases": GpuBuffer.from_bytes(c.biases_bytes), "out": GpuBuffer(n * 2)}
+            keep.append(bufs)
+            specs.append((f"mt_affine_{a.workload}_int{bits}", dt, bufs, {"group_size": G}))
+        nbytes = n * 2 + n * bits // 8 + 2 * (n // G) * 2
+        runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
+        _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+        kern_avg = chain_us / (a.steps * len(specs))
+        out.update({
+            "metric": f"affine {a.workload} GB/s (4-bit g64 bf16, 14336x4096 elements)",
+            "value": round(nbytes * len(specs) * a.steps / wall_us / 1e3, 1), "unit": "GB/s",
+            "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
+            "config": {"workload": f"affine {a.workload} 4-bit g64 bf16, 14336x4096 elements", "launches_per_step": len(specs),
+                       "bytes_per_launch": nbytes, "device": info["name"] or info["arch"]},
+            "roofline": {"bound": "hbm", "achieved": round(nbytes / kern_avg / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(nbytes / kern_avg / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
+                         "avg_launch_us_timed_region": round(kern_avg, 3)},
         })
         print(json.dumps(out))
         return

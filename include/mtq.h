@@ -153,6 +153,27 @@ MTQ_API int mtq_gather_qmv_single(int dtype, int bits, uint32_t group_size, cons
                                   const uint32_t *expert_index, void *output, uint32_t N,
                                   uint32_t K, uint32_t E);
 
+/* ---- the packed format's writer and reader ------------------------------ */
+
+/* Affine quantise: per group of `group_size` consecutive elements of w (T[n_elem]),
+ * scale = (max - min) / (2^bits - 1) (1 when below 1e-7), bias = min,
+ * code = trunc(clamp((v - bias) * (1 / scale) + 0.5, 0, 2^bits - 1)); codes go to
+ * `out` as an LSB-first bit stream of u32 words (n_elem * bits / 32 of them),
+ * scale and bias to scales / biases (T[n_elem / group_size]). Replaces
+ * mt_affine_quantize_int{2,3,4,5,6,8}
+ * (crates/metaltile-std/src/mlx/quantized.rs:3629-3671, 3707, 3793, 3871, 3935, 4005).
+ * bits in 2..8; group_size a multiple of 8 (4-, 8-bit), 16 (2-bit) or 32 (other
+ * widths) with a power-of-two quotient; n_elem a multiple of group_size. */
+MTQ_API int mtq_affine_quantize(int dtype, int bits, uint32_t group_size, const void *w, void *out,
+                                void *scales, void *biases, size_t n_elem);
+
+/* Affine dequantise: out[i] = scales[i / group_size] * code_i + biases[i / group_size]
+ * rounded to T. Replaces mt_affine_dequantize_int{2,3,4,5,6,8}
+ * (crates/metaltile-std/src/mlx/quantized.rs:3575-3611, 3681, 3762, 4081, 4127, 4179).
+ * Same constraints as mtq_affine_quantize. */
+MTQ_API int mtq_affine_dequantize(int dtype, int bits, uint32_t group_size, const void *w,
+                                  const void *scales, const void *biases, void *out, size_t n_elem);
+
 /* ---- name-keyed dispatch (the reference's binding convention) ----------- */
 
 /* Replaces Context::dispatch_with_grid (crates/metaltile-runtime/src/context.rs:269-283)

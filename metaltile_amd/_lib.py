@@ -57,6 +57,8 @@ SIGNATURES = {
     "mtq_gather_qmv_csr": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32]),
     "mtq_gather_qmv_indices": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32]),
     "mtq_gather_qmv_single": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
+    "mtq_affine_quantize": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, C.c_size_t]),
+    "mtq_affine_dequantize": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, C.c_size_t]),
     "mtq_dispatch": (C.c_int, [C.c_char_p, C.c_int, _bufp, C.c_int, _u32p, C.c_int, _u32p, _u32p, _dblp]),
     "mtq_measure": (C.c_int, [C.c_char_p, C.c_int, _bufp, C.c_int, _u32p, C.c_int, _u32p, _u32p, C.c_int, C.c_int, _dblp]),
     "mtq_dispatch_chain": (C.c_int, [C.POINTER(MtqDispatchSpec), C.c_int, C.c_int, _dblp, _dblp, _dblp]),

@@ -1,0 +1,240 @@
+// Affine quantise / dequantise for gfx950: the writer and the reader of the
+// packed weight format the matmul kernels consume.
+//
+// Replaces mt_affine_quantize_int{2,3,4,5,6,8} and mt_affine_dequantize_int{2,3,4,5,6,8}
+// (crates/metaltile-std/src/mlx/quantized.rs:3575-3866, 3871-4230).
+//
+// Quantise, per group of `group_size` consecutive elements
+// (quantized.rs:3642-3671): mn/mx = min/max of the group as f32,
+// scale = (mx - mn) / (2^bits - 1), replaced by 1 when below 1e-7; bias = mn;
+// code = trunc(clamp((v - bias) * (1 / scale) + 0.5, 0, 2^bits - 1)) formed with
+// the f32 scale and bias; scale and bias are then stored rounded to the element
+// dtype. Codes are integers and must not depend on instruction selection, so
+// the subtract, multiply and add are issued as separately rounded operations
+// (never contracted into an FMA) and the divisions are IEEE-correct.
+// Dequantise: out = scale * code + bias, multiply and add rounded separately,
+// then rounded to the element dtype (quantized.rs:3599-3604).
+//
+// Both are bandwidth kernels. A lane owns EPL consecutive elements: 8 for 4- and
+// 8-bit codes, 16 for 2-bit, 32 for the widths whose codes straddle words (32
+// codes of any width are a whole number of words). Its packed words and its
+// elements are contiguous, so neighbouring lanes read and write neighbouring
+// bytes; the G/EPL lanes of a group find the group's min and max with xor
+// shuffles.
+#include "mtq_device.h"
+#include "mtq_internal.h"
+
+// Every a*b+c in this file is two rounded operations, as in the reference's CPU
+// loops (crates/metaltile-std/src/mlx/quantized.rs:5296-5303): a fused multiply-add can move a quantised value across a code
+// boundary and changes the last bit of a dequantised one.
+#pragma STDC FP_CONTRACT OFF
+
+namespace mtq {
+
+typedef uint32_t a_u32x4 __attribute__((ext_vector_type(4)));
+
+struct AffineArgs {
+    const void* in;     // quantise: T[n_elem]; dequantise: u32 words
+    void* out;          // quantise: u32 words;  dequantise: T[n_elem]
+    void* scales;       // T[n_elem / G]
+    void* biases;
+    uint64_t n_elem;
+    uint32_t group_size;
+    uint32_t lanes_per_group;  // G / EPL, a power of two
+    uint32_t log2g;            // G is EPL * lanes_per_group: a power of two as well
+};
+
+template <int BITS> struct AffineGeom {
+    static constexpr int EPL = (BITS == 4 || BITS == 8) ? 8 : (BITS == 2 ? 16 : 32);
+    static constexpr int NW = EPL * BITS / 32;  // packed words per lane
+};
+
+// EPL consecutive elements -> f32
+template <int DT, int EPL> __device__ __forceinline__ void load_elems(const void* p, uint64_t i0, float (&v)[EPL]) {
+    if constexpr (DT == DT_F32) {
+        const float4* s = (const float4*)((const float*)p + i0);
+#pragma unroll
+        for (int j = 0; j < EPL / 4; j++) {
+            const float4 t = s[j];
+            v[4 * j] = t.x; v[4 * j + 1] = t.y; v[4 * j + 2] = t.z; v[4 * j + 3] = t.w;
+        }
+    } else {
+        const a_u32x4* s = (const a_u32x4*)((const uint16_t*)p + i0);
+#pragma unroll
+        for (int j = 0; j < EPL / 8; j++) {
+            const a_u32x4 t = s[j];
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                if constexpr (DT == DT_BF16) {
+                    v[8 * j + 2 * d] = bf16_bits_to_f32(t[d] & 0xFFFFu);
+                    v[8 * j + 2 * d + 1] = bf16_bits_to_f32(t[d] >> 16);
+                } else {
+                    v[8 * j + 2 * d] = f16_bits_to_f32(t[d] & 0xFFFFu);
+                    v[8 * j + 2 * d + 1] = f16_bits_to_f32(t[d] >> 16);
+                }
+            }
+        }
+    }
+}
+
+template <int DT, int EPL> __device__ __forceinline__ void store_elems(void* p, uint64_t i0, const float (&v)[EPL]) {
+    if constexpr (DT == DT_F32) {
+        float4* d = (float4*)((float*)p + i0);
+#pragma unroll
+        for (int j = 0; j < EPL / 4; j++) d[j] = make_float4(v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]);
+    } else {
+        a_u32x4* d = (a_u32x4*)((uint16_t*)p + i0);
+#pragma unroll
+        for (int j = 0; j < EPL / 8; j++) {
+            a_u32x4 t;
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                t[k] = (uint32_t)f32_to_elem_bits<DT>(v[8 * j + 2 * k]) | ((uint32_t)f32_to_elem_bits<DT>(v[8 * j + 2 * k + 1]) << 16);
+            d[j] = t;
+        }
+    }
+}
+
+template <int DT, int BITS>
+__global__ __launch_bounds__(256) void affine_quantize_kernel(AffineArgs a) {
+#pragma clang fp contract(off)
+    constexpr int EPL = AffineGeom<BITS>::EPL, NW = AffineGeom<BITS>::NW;
+    const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t i0 = t * EPL;
+    if (i0 >= a.n_elem) return;  // whole groups leave together: n_elem is a multiple of G
+    float v[EPL];
+    load_elems<DT, EPL>(a.in, i0, v);
+    float mn = v[0], mx = v[0];
+#pragma unroll
+    for (int i = 1; i < EPL; i++) {
+        mn = v[i] < mn ? v[i] : mn;
+        mx = v[i] > mx ? v[i] : mx;
+    }
+    // the group's lanes are consecutive and aligned to their (power-of-two) count
+    for (uint32_t d = 1; d < a.lanes_per_group; d <<= 1) {
+        const float omn = __shfl_xor(mn, (int)d, 64), omx = __shfl_xor(mx, (int)d, 64);
+        mn = omn < mn ? omn : mn;
+        mx = omx > mx ? omx : mx;
+    }
+    constexpr float QMAX = (float)((1u << BITS) - 1u);
+    float scale = (mx - mn) / QMAX;
+    if (scale < 1.0e-7f) scale = 1.0f;
+    const float inv = 1.0f / scale, bias = mn;
+    uint32_t words[NW];
+#pragma unroll
+    for (int j = 0; j < NW; j++) words[j] = 0u;
+#pragma unroll
+    for (int i = 0; i < EPL; i++) {
+        const float d = v[i] - bias;
+        const float p = d * inv;
+        float q = p + 0.5f;
+        q = q < 0.0f ? 0.0f : q;
+        q = q > QMAX ? QMAX : q;
+        const uint32_t c = (uint32_t)q;
+        const int pos = i * BITS, wi = pos / 32, sh = pos % 32;
+        words[wi] |= c << sh;
+        if (sh + BITS > 32) words[wi + 1] |= c >> (32 - sh);
+    }
+    uint32_t* dst = (uint32_t*)a.out + t * NW;
+    if constexpr (NW == 1) {
+        dst[0] = words[0];
+    } else if constexpr (NW == 2) {
+        *(uint2*)dst = make_uint2(words[0], words[1]);
+    } else {
+#pragma unroll
+        for (int j = 0; j < NW; j++) dst[j] = words[j];
+    }
+    if ((t & (a.lanes_per_group - 1)) == 0) {
+        const uint64_t g = i0 >> a.log2g;
+        store_elem<DT>(a.scales, g, scale);
+        store_elem<DT>(a.biases, g, bias);
+    }
+}
+
+template <int DT, int BITS>
+__global__ __launch_bounds__(256) void affine_dequantize_kernel(AffineArgs a) {
+#pragma clang fp contract(off)
+    constexpr int EPL = AffineGeom<BITS>::EPL, NW = AffineGeom<BITS>::NW;
+    const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t i0 = t * EPL;
+    if (i0 >= a.n_elem) return;
+    const uint32_t* src = (const uint32_t*)a.in + t * NW;
+    uint32_t words[NW];
+    if constexpr (NW == 2) {
+        const uint2 w2 = *(const uint2*)src;
+        words[0] = w2.x;
+        words[1] = w2.y;
+    } else {
+#pragma unroll
+        for (int j = 0; j < NW; j++) words[j] = src[j];
+    }
+    const uint64_t g = i0 >> a.log2g;
+    const float scale = load_elem<DT>(a.scales, g), bias = load_elem<DT>(a.biases, g);
+    float v[EPL];
+#pragma unroll
+    for (int i = 0; i < EPL; i++) {
+        const int pos = i * BITS, wi = pos / 32, sh = pos % 32;
+        uint32_t c = words[wi] >> sh;
+        if (sh + BITS > 32) c |= words[wi + 1] << (32 - sh);
+        c &= (1u << BITS) - 1u;
+        const float p = scale * (float)c;
+        v[i] = p + bias;
+    }
+    store_elems<DT, EPL>(a.out, i0, v);
+}
+
+template <int DT, int BITS> static int launch_one(bool quantize, AffineArgs& a, const LaunchCtx& lc) {
+    constexpr int EPL = AffineGeom<BITS>::EPL;
+    if (a.group_size % EPL) return fail(ERR_UNSUPPORTED, "affine: group_size must be a multiple of the lane's run (8, 16 or 32 elements)");
+    a.lanes_per_group = a.group_size / EPL;
+    if (a.lanes_per_group & (a.lanes_per_group - 1) || a.lanes_per_group > 64)
+        return fail(ERR_UNSUPPORTED, "affine: group_size / run must be a power of two up to 64");
+    a.log2g = 0;
+    while ((1u << a.log2g) < a.group_size) a.log2g++;
+    const uint64_t threads = a.n_elem / EPL;
+    const uint64_t blocks = (threads + 255) / 256;
+    if (blocks == 0) return ERR_OK;
+    if (blocks > 0x7FFFFFFFull) return fail(ERR_SHAPE, "affine: too many elements for one launch");
+    const void* fn = quantize ? (const void*)affine_quantize_kernel<DT, BITS> : (const void*)affine_dequantize_kernel<DT, BITS>;
+    void* args[] = {&a};
+    hipError_t e = launch_kernel(fn, dim3((uint32_t)blocks), dim3(256), args, 0, lc);
+    if (e != hipSuccess) return hip_fail(e, "affine kernel launch");
+    return ERR_OK;
+}
+
+template <int DT> static int launch_bits(bool quantize, int bits, AffineArgs& a, const LaunchCtx& lc) {
+    switch (bits) {
+        case 2: return launch_one<DT, 2>(quantize, a, lc);
+        case 3: return launch_one<DT, 3>(quantize, a, lc);
+        case 4: return launch_one<DT, 4>(quantize, a, lc);
+        case 5: return launch_one<DT, 5>(quantize, a, lc);
+        case 6: return launch_one<DT, 6>(quantize, a, lc);
+        case 7: return launch_one<DT, 7>(quantize, a, lc);
+        default: return launch_one<DT, 8>(quantize, a, lc);
+    }
+}
+
+int launch_affine(bool quantize, int dtype, int bits, uint32_t group_size, const void* in, void* out,
+                  void* scales, void* biases, uint64_t n_elem, const LaunchCtx& lc) {
+    if (bits < 2 || bits > 8) return fail(ERR_BAD_ARG, "bits must be in 2..8");
+    if (group_size == 0 || n_elem % group_size) return fail(ERR_SHAPE, "n_elem must be a whole number of groups");
+    if (n_elem == 0) return ERR_OK;
+    if (!in || !out || !scales || !biases) return fail(ERR_BAD_ARG, "null buffer");
+    if ((uintptr_t)in % 16 || (uintptr_t)out % 16) return fail(ERR_UNSUPPORTED, "affine: buffers must be 16-byte aligned");
+    AffineArgs a;
+    a.in = in;
+    a.out = out;
+    a.scales = scales;
+    a.biases = biases;
+    a.n_elem = n_elem;
+    a.group_size = group_size;
+    a.lanes_per_group = 1;
+    switch (dtype) {
+        case DT_F32: return launch_bits<DT_F32>(quantize, bits, a, lc);
+        case DT_F16: return launch_bits<DT_F16>(quantize, bits, a, lc);
+        case DT_BF16: return launch_bits<DT_BF16>(quantize, bits, a, lc);
+        default: return fail(ERR_BAD_ARG, "unknown dtype");
+    }
+}
+
+}  // namespace mtq

@@ -169,7 +169,7 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
 // name-keyed dispatch table
 // ---------------------------------------------------------------------------
 
-enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX };
+enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ };
 
 struct KernelDesc {
     const char* name;
@@ -222,6 +222,14 @@ static const KernelDesc kTable[] = {
     {"mt_moe_gather_qmm_mma_int8", F_GIDX, 8, 6, 4}, {"mt_moe_gather_qmm_mma_b3", F_GIDX, 3, 6, 4},
     {"mt_moe_gather_qmm_mma_b5", F_GIDX, 5, 6, 4}, {"mt_moe_gather_qmm_mma_b6", F_GIDX, 6, 6, 4},
     {"mt_moe_gather_qmm_mma_b8", F_GIDX, 8, 6, 4},
+    // w, out, scales, biases | group_size
+    {"mt_affine_quantize_int2", F_AQ, 2, 4, 1}, {"mt_affine_quantize_int3", F_AQ, 3, 4, 1},
+    {"mt_affine_quantize_int4", F_AQ, 4, 4, 1}, {"mt_affine_quantize_int5", F_AQ, 5, 4, 1},
+    {"mt_affine_quantize_int6", F_AQ, 6, 4, 1}, {"mt_affine_quantize_int8", F_AQ, 8, 4, 1},
+    // w, scales, biases, out | group_size
+    {"mt_affine_dequantize_int2", F_ADQ, 2, 4, 1}, {"mt_affine_dequantize_int3", F_ADQ, 3, 4, 1},
+    {"mt_affine_dequantize_int4", F_ADQ, 4, 4, 1}, {"mt_affine_dequantize_int5", F_ADQ, 5, 4, 1},
+    {"mt_affine_dequantize_int6", F_ADQ, 6, 4, 1}, {"mt_affine_dequantize_int8", F_ADQ, 8, 4, 1},
 };
 static const int kTableLen = (int)(sizeof(kTable) / sizeof(kTable[0]));
 
@@ -356,6 +364,30 @@ static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, in
             MTQ_NEED(bufs[5], "out", (uint64_t)T * N * sz);
             return op_gather(GATHER_INDICES, dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr,
                              bufs[3].ptr, (const uint32_t*)bufs[4].ptr, bufs[5].ptr, T, N, K, E, lc);
+        }
+        case F_AQ: {
+            // element count = length of the input tensor (one workgroup per group in
+            // the reference, crates/metaltile-std/src/mlx/quantized.rs:3636-3638)
+            const uint32_t G = consts[0];
+            if (G == 0) return fail(ERR_SHAPE, "group_size must be non-zero");
+            const uint64_t n = bufs[0].bytes / sz;
+            if (n % G) return fail(ERR_SHAPE, "'w' must hold a whole number of groups");
+            MTQ_NEED(bufs[1], "out", n * bits / 8);
+            MTQ_NEED(bufs[2], "scales", n / G * sz);
+            MTQ_NEED(bufs[3], "biases", n / G * sz);
+            return launch_affine(true, dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, n, lc);
+        }
+        case F_ADQ: {
+            // element count = length of the output tensor (one thread per packed word
+            // in the reference, crates/metaltile-std/src/mlx/quantized.rs:3582-3585)
+            const uint32_t G = consts[0];
+            if (G == 0) return fail(ERR_SHAPE, "group_size must be non-zero");
+            const uint64_t n = bufs[3].bytes / sz;
+            if (n % G) return fail(ERR_SHAPE, "'out' must hold a whole number of groups");
+            MTQ_NEED(bufs[0], "w", n * bits / 8);
+            MTQ_NEED(bufs[1], "scales", n / G * sz);
+            MTQ_NEED(bufs[2], "biases", n / G * sz);
+            return launch_affine(false, dtype, d.bits, G, bufs[0].ptr, bufs[3].ptr, bufs[1].ptr, bufs[2].ptr, n, lc);
         }
     }
     return fail(ERR_UNKNOWN_KERNEL, "unhandled kernel family");
@@ -537,6 +569,23 @@ int mtq_gather_qmv_single(int dtype, int bits, uint32_t group_size, const void* 
     if (rc) return rc;
     return op_gather(GATHER_SINGLE, dtype, bits, group_size, input, w, scales, biases, expert_index,
                      output, 1, N, K, E, make_ctx());
+}
+
+int mtq_affine_quantize(int dtype, int bits, uint32_t group_size, const void* w, void* out,
+                        void* scales, void* biases, size_t n_elem) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (dtype != DT_F32 && dtype != DT_F16 && dtype != DT_BF16) return fail(ERR_BAD_ARG, "dtype must be MTQ_F32, MTQ_F16 or MTQ_BF16");
+    return launch_affine(true, dtype, bits, group_size, w, out, scales, biases, n_elem, make_ctx());
+}
+
+int mtq_affine_dequantize(int dtype, int bits, uint32_t group_size, const void* w, const void* scales,
+                          const void* biases, void* out, size_t n_elem) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (dtype != DT_F32 && dtype != DT_F16 && dtype != DT_BF16) return fail(ERR_BAD_ARG, "dtype must be MTQ_F32, MTQ_F16 or MTQ_BF16");
+    return launch_affine(false, dtype, bits, group_size, w, out, const_cast<void*>(scales),
+                         const_cast<void*>(biases), n_elem, make_ctx());
 }
 
 int mtq_kernel_supported(const char* kernel_name) { return find_kernel(kernel_name) ? 1 : 0; }

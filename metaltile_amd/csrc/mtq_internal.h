@@ -108,4 +108,9 @@ int launch_qmm_mfma(const QmmParams& p, const LaunchCtx& lc);
 // 64x128 tiles, weights converted in MFMA operand registers, activations through LDS (qmm_direct.hip).
 int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc);
 
+// Affine quantise (quantize = true: T[n_elem] -> packed words + scales + biases) and
+// dequantise (packed words + scales + biases -> T[n_elem]) (affine.hip).
+int launch_affine(bool quantize, int dtype, int bits, uint32_t group_size, const void* in, void* out,
+                  void* scales, void* biases, uint64_t n_elem, const LaunchCtx& lc);
+
 }  // namespace mtq

@@ -45,6 +45,18 @@ def gather_qmv_single(dtype, bits, group_size, w, scales, biases, inp, expert_in
                                          _p(inp), _p(expert_index), _p(out), N, K, E))
 
 
+def affine_quantize(dtype, bits, group_size, w, out, scales, biases, n_elem):
+    """w: T[n_elem] -> out: packed u32 words, scales / biases: T[n_elem / group_size]."""
+    lib = _ensure_init()
+    _lib.check(lib.mtq_affine_quantize(int(dtype), bits, group_size, _p(w), _p(out), _p(scales), _p(biases), n_elem))
+
+
+def affine_dequantize(dtype, bits, group_size, w, scales, biases, out, n_elem):
+    """w: packed u32 words + scales / biases -> out: T[n_elem]."""
+    lib = _ensure_init()
+    _lib.check(lib.mtq_affine_dequantize(int(dtype), bits, group_size, _p(w), _p(scales), _p(biases), _p(out), n_elem))
+
+
 def timed(fn, *args, **kw) -> float:
     """Run one op with GPU timestamps attached to its kernel; returns microseconds."""
     lib = _ensure_init()

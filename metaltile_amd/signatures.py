@@ -5,7 +5,8 @@ signature order, and which parameters are outputs (declared `mut` or named
 out / output, crates/metaltile-macros/src/legacy/sig_parser.rs:43-48,85).
 Sources: crates/metaltile-std/src/mlx/quantized.rs:8-16, 343-352, 4273-4285;
 ffai/dequant_gemv.rs:52-62; ffai/dequant_gemv_expert_indexed.rs:58-68;
-ffai/moe.rs:358-370, 2256-2268.
+ffai/moe.rs:358-370, 2256-2268; mlx/quantized.rs:3575-3581, 3629-3635 (affine
+quantise / dequantise).
 """
 from __future__ import annotations
 
@@ -59,3 +60,7 @@ for _n, _b in (("mt_moe_gather_qmm_mma_int4", 4), ("mt_moe_gather_qmm_mma_int4_b
                ("mt_moe_gather_qmm_mma_b5", 5), ("mt_moe_gather_qmm_mma_b6", 6),
                ("mt_moe_gather_qmm_mma_b8", 8)):
     _add(_n, _b, _GI, ("m_total", "n_out", "k_in", "group_size"), ("out",))
+for _b in (2, 3, 4, 5, 6, 8):
+    _add(f"mt_affine_quantize_int{_b}", _b, ("w", "out", "scales", "biases"), ("group_size",),
+         ("out", "scales", "biases"))
+    _add(f"mt_affine_dequantize_int{_b}", _b, ("w", "scales", "biases", "out"), ("group_size",), ("out",))
