@@ -71,7 +71,26 @@ def build(force: bool = False, verbose: bool = True) -> str:
             raise RuntimeError(f"link failed:\n{r.stderr}")
     if verbose:
         print(f"built {LIB}")
+    build_driver(force, verbose)
     return LIB
+
+
+DRIVER = os.path.join(HERE, "tile_bench")
+
+
+def build_driver(force: bool = False, verbose: bool = True) -> str:
+    """Host-only bench driver over the C-ABI (csrc/tile_bench.cpp), linked against the library beside it."""
+    src = os.path.join(CSRC, "tile_bench.cpp")
+    inc = os.path.join(HERE, "..", "include")
+    if force or _stale(DRIVER, [src, os.path.join(inc, "mtq.h"), LIB]):
+        cmd = ["g++", "-O2", "-std=c++17", "-Wall", "-I", inc, src, "-o", DRIVER, "-L", HERE, "-lmtq_hip",
+               "-Wl,-rpath,$ORIGIN"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"driver build failed:\n{r.stderr}")
+        if verbose:
+            print(f"built {DRIVER}")
+    return DRIVER
 
 
 if __name__ == "__main__":

@@ -444,7 +444,8 @@ int mtq_device_name(char* out, size_t cap) {
     int rc = need_ready();
     if (rc) return rc;
     if (!out || cap == 0) return fail(ERR_BAD_ARG, "null output");
-    snprintf(out, cap, "%s", g.prop.name);
+    // some driver stacks report an empty marketing name: fall back to the ISA name
+    snprintf(out, cap, "%s", g.prop.name[0] ? g.prop.name : g.prop.gcnArchName);
     return MTQ_OK;
 }
 

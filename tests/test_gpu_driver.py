@@ -1,0 +1,22 @@
+"""The C++ bench driver (the mirror of `tile bench -f ...`) against the real library on the GPU."""
+import json
+import subprocess
+
+import pytest
+
+from metaltile_amd.build import DRIVER
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("flt,rows", [("mlx/quantized/qmv", 7), ("ffai/moe/gather_qmm_int4", 4), ("expert_indexed", 1)])
+def test_driver_runs_reference_benches(flt, rows):
+    print(f"[case] tile_bench -f {flt}", flush=True)
+    r = subprocess.run([DRIVER, "-f", flt, "--dtype", "bf16", "--warmup", "3", "--iters", "5"],
+                       capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stderr
+    out = [json.loads(l) for l in r.stdout.strip().splitlines()]
+    assert len(out) == rows
+    for row in out:
+        assert set(("op", "subop", "shape", "metric", "ref", "mt")) <= set(row)
+        assert row["metric"] == "GB/s" and row["mt"] > 1.0 and row["min_us"] > 0.0

@@ -129,3 +129,36 @@ def test_product_never_touches_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp", ".hpp")):
                 text = open(os.path.join(dirpath, f), errors="replace").read()
                 assert "oracle" not in text.lower(), f"{f} mentions the oracle"
+
+
+def test_bench_driver_lists_the_reference_registrations():
+    """The C++ driver names every bench it mirrors; each maps to a kernel the library and the Python mirror know."""
+    import subprocess
+    from metaltile_amd.build import DRIVER
+    from metaltile_amd.signatures import KERNEL_SIGNATURES
+    if not os.path.exists(DRIVER):
+        from metaltile_amd.build import build
+        build(verbose=False)
+    out = subprocess.run([DRIVER, "--list"], capture_output=True, text=True, check=True).stdout
+    rows = [l.split("\t") for l in out.strip().splitlines()]
+    assert len(rows) >= 49
+    names = [r[0] for r in rows]
+    assert len(set(names)) == len(names)
+    for must in ("mlx/quantized/qmv", "mlx/quantized/qmm_mma", "ffai/dequant_gemv/int4_fast",
+                 "ffai/dequant_gemv_expert_indexed/int4", "ffai/moe/gather_qmm_int4", "ffai/moe/gather_qmm_mma_int4"):
+        assert must in names
+    for _, kernel in rows:
+        assert kernel in KERNEL_SIGNATURES, kernel
+
+
+def test_bench_driver_fails_loudly_without_a_gpu():
+    import subprocess
+    import metaltile_amd as m
+    from metaltile_amd.build import DRIVER
+    try:
+        m.GpuRunner(0)
+    except m.MtqError:
+        r = subprocess.run([DRIVER, "-f", "mlx/quantized/qmv"], capture_output=True, text=True)
+        assert r.returncode != 0 and "no HIP device" in r.stderr
+    else:
+        pytest.skip("a GPU is present")
