@@ -78,9 +78,21 @@ def cpu_baseline_qmv(seconds: float):
         el = time.perf_counter() - t0
         if el >= seconds:
             break
+    # the same loop on one thread, as the reference's single-threaded setup() runs it
+    reps1, t1 = 0, time.perf_counter()
+    while True:
+        c = cases[reps1 % len(cases)]
+        o.qmm(c.w, c.scales_f, c.biases_f, c.x_f, 1, c.N, c.K, 4, 64, threads=1)
+        reps1 += 1
+        el1 = time.perf_counter() - t1
+        if el1 >= seconds / 3:
+            break
+    one = qmv_bytes(14336, 4096, 4, 64, 1, 2) * reps1 / el1 / 1e9
     return {"value": round(nbytes * reps / el / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": f"{reps} passes over one layer (gate, up 14336x4096; down 4096x14336), "
-                      f"f32-sequential oracle, {el:.1f} s, row-parallel over {cores} threads"}
+                      f"f32-sequential oracle, {el:.1f} s, row-parallel over {cores} threads; "
+                      f"one thread: {one:.3f} GB/s over {reps1} matrices in {el1:.1f} s",
+            "value_one_thread": round(one, 3)}
 
 
 def main():
