@@ -784,6 +784,16 @@ int mtq_set_option(const char* name, int value) {
         options().qmv_mfma = value;
         return MTQ_OK;
     }
+    if (!strcmp(name, "qmv.mfma_sets")) {
+        if (value != 0 && value != 1 && value != 2 && value != 4) return fail(ERR_BAD_ARG, "qmv.mfma_sets must be 0, 1, 2 or 4");
+        options().qmv_mfma_sets = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmv.mfma_delay")) {
+        if (value < 0 || value > 64) return fail(ERR_BAD_ARG, "qmv.mfma_delay must be in 0..64");
+        options().qmv_mfma_delay = value;
+        return MTQ_OK;
+    }
     if (!strcmp(name, "qmv.mfma_kp") || !strcmp(name, "qmv.mfma_rbw") || !strcmp(name, "qmv.mfma_nrb")) {
         if (value < 0 || value > 16) return fail(ERR_BAD_ARG, "qmv.mfma_* must be in 0..16");
         if (name[9] == 'k') options().qmv_mfma_kp = value;

@@ -81,6 +81,8 @@ struct Options {
     int qmv_mfma_kp = 0;          // matrix-core qmv: K parts per row block
     int qmv_mfma_rbw = 0;         // matrix-core qmv: row blocks walked in parallel per workgroup
     int qmv_mfma_nrb = 0;         // matrix-core qmv: row blocks per wave
+    int qmv_mfma_sets = 0;        // matrix-core gather: 4-row MFMA sets per pass (0 = choose; 1, 2, 4)
+    int qmv_mfma_delay = 0;       // matrix-core qmv: pause (x512 clocks) before the first weight loads
 };
 Options& options();
 

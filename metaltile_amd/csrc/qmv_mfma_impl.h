@@ -72,6 +72,7 @@ struct QmvMArgs {
     uint32_t nrb;       // row blocks per wave, one after the other
     uint32_t gpr, log2g;
     uint32_t list_cap;  // capacity of the row list (indices mode)
+    uint32_t delay;     // units of 512 clocks between the small loads and the first weight loads
 };
 
 struct QmvMGeom {
@@ -270,6 +271,8 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
 
         x_load(min(tid, ntask - 1));
         if (pass == 0) sb_load(min(tid, nvec - 1));
+        MTQ_MFMA_KEEP_ORDER();
+        for (uint32_t i = 0; i < a.delay; i++) __builtin_amdgcn_s_sleep(8);
         MTQ_MFMA_KEEP_ORDER();
         m_u32x4 ring[D];
 #pragma unroll
