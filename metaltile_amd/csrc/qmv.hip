@@ -110,7 +110,9 @@ int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {
         // The matrix-core kernel wins as soon as more than one activation row shares
         // the weight stream (and for every gather); a single row is as fast on the
         // dot2 kernels below.
-        const bool many = p.gather == GATHER_CSR || p.gather == GATHER_INDICES || (p.gather == GATHER_NONE && p.M >= 2);
+        // Widths 3, 5 and 6 have no dot2 kernel: the matrix-core kernel is their fast path.
+        const bool many = p.gather == GATHER_CSR || p.gather == GATHER_INDICES || (p.gather == GATHER_NONE && p.M >= 2) ||
+                          p.bits == 3 || p.bits == 5 || p.bits == 6;
         const int mode = options().qmv_mfma;
         if (mode == 2 || (mode == 0 && many)) {
             int rc = launch_qmv_mfma(p, lc);

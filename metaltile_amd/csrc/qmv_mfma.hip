@@ -8,6 +8,8 @@ namespace mtq {
 
 extern template int qmv_mfma_launch_dtype<DT_F16>(QmvMArgs&, int, int, const QmvMGeom&, const LaunchCtx&);
 extern template int qmv_mfma_launch_dtype<DT_BF16>(QmvMArgs&, int, int, const QmvMGeom&, const LaunchCtx&);
+extern template int qmv_mfma_launch_dtype_odd<DT_F16>(QmvMArgs&, int, int, const QmvMGeom&, const LaunchCtx&);
+extern template int qmv_mfma_launch_dtype_odd<DT_BF16>(QmvMArgs&, int, int, const QmvMGeom&, const LaunchCtx&);
 
 namespace {
 bool is_pow2(uint32_t v) { return v && !(v & (v - 1)); }
@@ -22,17 +24,21 @@ size_t lds_bytes(uint32_t R, uint32_t K, uint32_t nch, uint32_t rows_wg, uint32_
 
 int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     if (p.dtype != DT_F16 && p.dtype != DT_BF16) return fail(ERR_UNSUPPORTED, "mfma qmv: f16/bf16 only");
-    if (!(p.bits == 2 || p.bits == 4 || (p.bits == 8 && p.dtype == DT_F16)))
+    const bool odd = p.bits == 3 || p.bits == 5 || p.bits == 6;
+    if (!(p.bits == 2 || p.bits == 4 || (p.bits == 8 && p.dtype == DT_F16) || odd))
         return fail(ERR_UNSUPPORTED, "mfma qmv: bits");
     if (p.N == 0 || p.K == 0) return fail(ERR_UNSUPPORTED, "mfma qmv: empty");
+    // a lane's chunk: 16 bytes (128/bits codes), or 32 codes = bits dwords where codes straddle words
+    const uint32_t cpc = odd ? 32u : 128u / (uint32_t)p.bits, cb = odd ? 4u * (uint32_t)p.bits : 16u;
     const uint64_t rb64 = (uint64_t)p.K * p.bits / 8;
-    if (((uint64_t)p.K * p.bits) % 2048 || rb64 > (1u << 24)) return fail(ERR_UNSUPPORTED, "mfma qmv: row is not whole 256-byte segments");
-    const uint32_t RB = (uint32_t)rb64, nseg = RB / 256, nch = RB / 16, cpc = 128u / (uint32_t)p.bits;
+    if (p.K % (16u * cpc) || rb64 > (1u << 24)) return fail(ERR_UNSUPPORTED, "mfma qmv: row is not whole wave-wide segments");
+    const uint32_t RB = (uint32_t)rb64, nseg = p.K / (16u * cpc), nch = p.K / cpc;
+    (void)cb;
     const uint32_t G = p.group_size;
     if (!is_pow2(G) || G < cpc || p.K % G) return fail(ERR_UNSUPPORTED, "mfma qmv: group size");
     const uint32_t gpr = p.K / G;
     if (gpr % 4) return fail(ERR_UNSUPPORTED, "mfma qmv: groups per row not a multiple of 4");
-    if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
+    if ((uintptr_t)p.w % (odd ? 4 : 16) || (uintptr_t)p.x % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
         return fail(ERR_UNSUPPORTED, "mfma qmv: operands must be 16-byte aligned");
     const bool gather = p.gather == GATHER_CSR || p.gather == GATHER_INDICES;
     const uint32_t rows = gather ? p.T : (p.gather == GATHER_SINGLE ? 1u : p.M);
@@ -79,7 +85,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
         if (p.bits == 2 && s > 2) s = 2;  // the 16-row 2-bit variant does not fit the register file
         if (opt.qmv_mfma_sets) s = opt.qmv_mfma_sets;
     }
-    const uint32_t maxt = (s >= 4 || (s >= 2 && p.bits == 2)) ? 512u : 1024u;
+    const uint32_t maxt = (s >= 4 || (s >= 2 && p.bits != 4 && p.bits != 8)) ? 512u : 1024u;
     if (64u * KP > maxt) return fail(ERR_UNSUPPORTED, "mfma qmv: too many K parts");
     // Rows per workgroup: about one to two workgroups per compute unit (measured
     // best on 14336x4096, 4096x14336 and 8192x8192), as many of the row blocks
@@ -155,6 +161,9 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     const uint32_t rows_wg = 4 * RBW * nrb;
     g.shmem = lds_bytes(R, p.K, nch, rows_wg, gpr, KP, list_cap);
     g.grid = dim3((p.N + rows_wg - 1) / rows_wg, gather ? p.E : 1, 1);
+    if (odd)
+        return p.dtype == DT_F16 ? qmv_mfma_launch_dtype_odd<DT_F16>(a, p.bits, p.gather, g, lc)
+                                 : qmv_mfma_launch_dtype_odd<DT_BF16>(a, p.bits, p.gather, g, lc);
     switch (p.dtype) {
         case DT_F16: return qmv_mfma_launch_dtype<DT_F16>(a, p.bits, p.gather, g, lc);
         default: return qmv_mfma_launch_dtype<DT_BF16>(a, p.bits, p.gather, g, lc);

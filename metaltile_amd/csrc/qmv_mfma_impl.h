@@ -90,25 +90,85 @@ template <int DT> __device__ __forceinline__ m_f32x4 mfma4(m_u32x2 a, m_u32x2 b,
     }
 }
 
-// Position, inside a u32 word's PF codes, of the activation that pairs with the
-// o-th element of the word's MFMA operand sequence: MFMA t of a word multiplies
-// pair words (2t, 2t+1) = codes (2t, 2t+PF/2, 2t+1, 2t+1+PF/2).
-template <int PF> __host__ __device__ constexpr int mfma_src_index(int o) {
-    const int t = o / 4, e = o % 4;
-    return 2 * t + (e >> 1) + (e & 1) * (PF / 2);
-}
+// How one lane's run of packed codes maps to MFMA B operands, per code width.
+//   NWD   dwords a lane loads per step (its chunk)
+//   CPC   codes in that chunk (a multiple of 8); the chunk must lie in one group
+//   src() position, in the chunk's activations, of the element that multiplies
+//         the o-th element of the chunk's operand sequence
+// Widths that divide 32 (2, 4, 8): the chunk is 16 bytes and a masked dword gives
+// pairs (code j, code j + PF/2) of one word, so MFMA t of a word multiplies codes
+// (2t, 2t+PF/2, 2t+1, 2t+1+PF/2). Other widths (3, 5, 6, 7): the chunk is 32 codes
+// = BITS whole dwords of the bit stream, codes are extracted one by one (bit-field
+// extract, or a funnel shift where a code straddles two words) and paired in
+// natural order.
+template <int BITS> struct MfmaCodec {
+    static constexpr bool kPow2 = (32 % BITS) == 0;
+    static constexpr int PF = kPow2 ? 32 / BITS : 0;     // codes per dword (power-of-two widths)
+    static constexpr int NWD = kPow2 ? 4 : BITS;
+    static constexpr int CPC = kPow2 ? 4 * PF : 32;
+    static constexpr int CB = NWD * 4;                    // chunk bytes
+    __host__ __device__ static constexpr int src(int o) {
+        if (!kPow2) return o;
+        const int wi = o / PF, oo = o % PF, t = oo / 4, e = oo % 4;
+        return wi * PF + 2 * t + (e >> 1) + (e & 1) * (PF / 2);
+    }
+    // dwords of the chunk -> CPC/2 pair words (MAGIC+q_a | (MAGIC+q_b) << 16); MFMA m takes pairs 2m, 2m+1
+    static __device__ __forceinline__ void pairs(const uint32_t (&w)[NWD], uint32_t kor, uint32_t (&pw)[CPC / 2]) {
+        if constexpr (kPow2) {
+            constexpr uint32_t MASK = ((1u << BITS) - 1u) * 0x00010001u;
+#pragma unroll
+            for (int wi = 0; wi < 4; wi++)
+#pragma unroll
+                for (int j = 0; j < PF / 2; j++) pw[wi * (PF / 2) + j] = ((w[wi] >> (BITS * j)) & MASK) | kor;
+        } else {
+            constexpr uint32_t M1 = (1u << BITS) - 1u;
+#pragma unroll
+            for (int j = 0; j < CPC / 2; j++) {
+                uint32_t c[2];
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const int pos = (2 * j + e) * BITS, wi = pos / 32, sh = pos % 32;
+                    if (sh + BITS <= 32) c[e] = (w[wi] >> sh) & M1;
+                    else c[e] = __builtin_amdgcn_alignbit(w[wi + 1 < NWD ? wi + 1 : wi], w[wi], sh) & M1;
+                }
+                pw[j] = (c[0] | (c[1] << 16)) | kor;
+            }
+        }
+    }
+    static __device__ __forceinline__ void load(const unsigned char* p, uint32_t (&w)[NWD]) {
+        typedef uint32_t v4 __attribute__((ext_vector_type(4), aligned(4)));
+        typedef uint32_t v3 __attribute__((ext_vector_type(3), aligned(4)));
+        typedef uint32_t v2 __attribute__((ext_vector_type(2), aligned(4)));
+        if constexpr (NWD == 3) {
+            const v3 t = __builtin_nontemporal_load((const v3*)p);
+            w[0] = t.x; w[1] = t.y; w[2] = t.z;
+        } else {
+            const v4 t = __builtin_nontemporal_load((const v4*)p);
+            w[0] = t.x; w[1] = t.y; w[2] = t.z; w[3] = t.w;
+            if constexpr (NWD == 5) {
+                w[4] = __builtin_nontemporal_load((const uint32_t*)(p + 16));
+            } else if constexpr (NWD == 6) {
+                const v2 u = __builtin_nontemporal_load((const v2*)(p + 16));
+                w[4] = u.x; w[5] = u.y;
+            } else if constexpr (NWD == 7) {
+                const v3 u = __builtin_nontemporal_load((const v3*)(p + 16));
+                w[4] = u.x; w[5] = u.y; w[6] = u.z;
+            }
+        }
+    }
+};
 
 template <int DT, int BITS, int MP, int S, int D, int MODE, int MAXT>
 __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
-    constexpr int PF = 32 / BITS;   // codes per u32 word
-    constexpr int CPC = 4 * PF;     // codes per 16-byte chunk
-    constexpr int NP = PF / 2;      // 16-byte activation pieces per chunk
+    typedef MfmaCodec<BITS> Codec;
+    constexpr int CPC = Codec::CPC;  // codes per lane chunk
+    constexpr int NWD = Codec::NWD;  // dwords per lane chunk
+    constexpr int NP = CPC / 8;      // 16-byte activation pieces per chunk
     constexpr int R = MP * S;       // activation rows per pass
     constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
-    constexpr uint32_t MAGIC2 = DT == DT_BF16 ? 0x43004300u : 0x64006400u;
-    constexpr uint32_t MASK = ((1u << BITS) - 1u) * 0x00010001u;
     constexpr uint32_t NOROW = 0xFFFFFFFFu;
     static_assert(DT != DT_BF16 || BITS <= 7, "an 8-bit code does not fit the bf16 mantissa");
+    static_assert(CPC % 8 == 0 && CPC / 2 >= 2, "chunk must be whole activation pieces");
 
     extern __shared__ __align__(16) unsigned char smem[];
     const uint32_t rows_wg = 4u * a.RBW * a.nrb;
@@ -171,17 +231,18 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     };
 
     const size_t slab_rows = (size_t)expert * a.N;
-    const unsigned char* wbase = a.w + slab_rows * a.RB + (size_t)(kp * a.spp) * 256u + q * 16u;
+    constexpr uint32_t SEGB = 16u * Codec::CB;  // bytes of one weight row covered by a wave-wide load
+    const unsigned char* wbase = a.w + slab_rows * a.RB + (size_t)(kp * a.spp) * SEGB + q * (uint32_t)Codec::CB;
     const uint32_t sppD = (a.spp + D - 1) / D * D;  // steps per row block, padded to whole rings
 
     // Address of the 16 bytes this lane loads at step (rb, sg). Steps past the
     // end of a row block or of the wave's work re-read a valid address; what they
     // load is multiplied by a zero scale.
-    auto w_ptr = [&](uint32_t rb, uint32_t sg) -> const m_u32x4* {
+    auto w_ptr = [&](uint32_t rb, uint32_t sg) -> const unsigned char* {
         rb = min(rb, a.nrb - 1);
         sg = min(sg, a.spp - 1);
         const uint32_t row = min(row0 + (rb * a.RBW + rbw) * 4u + r, a.N - 1);
-        return (const m_u32x4*)(wbase + (size_t)row * a.RB + (size_t)sg * 256u);
+        return wbase + (size_t)row * a.RB + (size_t)sg * SEGB;
     };
 
     const uint32_t n_pass = (MODE == GATHER_CSR || MODE == GATHER_INDICES) ? (cnt + R - 1) / R : 1u;
@@ -234,8 +295,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
 #pragma unroll
                     for (int e2 = 0; e2 < 2; e2++) {
                         const int oe = p * 8 + dw * 2 + e2;          // element of the chunk's operand sequence
-                        const int wi = oe / PF;                      // word it belongs to
-                        const int se = wi * PF + mfma_src_index<PF>(oe % PF);  // source element
+                        const int se = Codec::src(oe);               // source element
                         h[e2] = (se & 1) ? (raw[se >> 1] >> 16) : (raw[se >> 1] & 0xFFFFu);
                     }
                     o[dw] = h[0] | (h[1] << 16);
@@ -274,9 +334,9 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         MTQ_MFMA_KEEP_ORDER();
         for (uint32_t i = 0; i < a.delay; i++) __builtin_amdgcn_s_sleep(8);
         MTQ_MFMA_KEEP_ORDER();
-        m_u32x4 ring[D];
+        uint32_t ring[D][NWD];
 #pragma unroll
-        for (int d = 0; d < D; d++) ring[d] = __builtin_nontemporal_load(w_ptr(0, d));
+        for (int d = 0; d < D; d++) Codec::load(w_ptr(0, d), ring[d]);
         MTQ_MFMA_KEEP_ORDER();
         if (tid < ntask) x_store(tid);
         if (pass == 0) {
@@ -332,27 +392,20 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                     }
                     const uint32_t g = (c * (uint32_t)CPC) >> a.log2g;
                     const float2 sb = SB[valid ? sb_row + g : rows_wg * a.gpr];
-                    const m_u32x4 wv = ring[d];
-                    if constexpr (ISSUE) ring[d] = __builtin_nontemporal_load(w_ptr(nrb_i, nsg0 + d));
+                    uint32_t pw[CPC / 2];
+                    Codec::pairs(ring[d], kor, pw);
+                    if constexpr (ISSUE) Codec::load(w_ptr(nrb_i, nsg0 + d), ring[d]);
                     // codes -> B operands, MFMAs
                     m_f32x4 acc[S];
 #pragma unroll
-                    for (int wi = 0; wi < 4; wi++) {
-                        const uint32_t word = wv[wi];
-                        uint32_t pw[PF / 2];
+                    for (int m = 0; m < CPC / 4; m++) {  // MFMA m of the chunk: codes 4m .. 4m+3 of its operand sequence
+                        const m_u32x2 b = {pw[2 * m], pw[2 * m + 1]};
 #pragma unroll
-                        for (int j = 0; j < PF / 2; j++) pw[j] = ((word >> (BITS * j)) & MASK) | kor;
-#pragma unroll
-                        for (int t = 0; t < PF / 4; t++) {
-                            const int m = wi * (PF / 4) + t;       // MFMA index within the chunk
-                            const m_u32x2 b = {pw[2 * t], pw[2 * t + 1]};
-#pragma unroll
-                            for (int s = 0; s < S; s++) {
-                                const m_u32x4 piece = av[s][m / 2];
-                                const m_u32x2 aop = (m & 1) ? m_u32x2{piece.z, piece.w} : m_u32x2{piece.x, piece.y};
-                                const m_f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-                                acc[s] = mfma4<DT>(aop, b, m == 0 ? zero : acc[s]);
-                            }
+                        for (int s = 0; s < S; s++) {
+                            const m_u32x4 piece = av[s][m / 2];
+                            const m_u32x2 aop = (m & 1) ? m_u32x2{piece.z, piece.w} : m_u32x2{piece.x, piece.y};
+                            const m_f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                            acc[s] = mfma4<DT>(aop, b, m == 0 ? zero : acc[s]);
                         }
                     }
 #pragma unroll
@@ -405,7 +458,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
 
 template <int DT, int BITS, int MP, int S, int MODE>
 int qmv_mfma_launch_one(QmvMArgs& a, const QmvMGeom& g, const LaunchCtx& lc) {
-    constexpr int MAXT = (S >= 4 || (S >= 2 && BITS == 2)) ? 512 : 1024;
+    constexpr int MAXT = (S >= 4 || (S >= 2 && BITS != 4 && BITS != 8)) ? 512 : 1024;
     if (g.tpb > (uint32_t)MAXT) return fail(ERR_UNSUPPORTED, "mfma qmv: workgroup too large for this row count");
     const void* fn = (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT>;
     if (g.shmem > 48 * 1024) {
@@ -456,6 +509,16 @@ template <int DT> int qmv_mfma_launch_dtype(QmvMArgs& a, int bits, int mode, con
         default:
             if constexpr (DT == DT_F16) return qmv_mfma_launch_mode<DT, 8>(a, mode, g, lc);
             else return fail(ERR_UNSUPPORTED, "mfma qmv: 8-bit codes need f16 activations");
+    }
+}
+
+// Widths whose codes straddle words (3, 5, 6): instantiated in their own translation units.
+template <int DT> int qmv_mfma_launch_dtype_odd(QmvMArgs& a, int bits, int mode, const QmvMGeom& g, const LaunchCtx& lc) {
+    switch (bits) {
+        case 3: return qmv_mfma_launch_mode<DT, 3>(a, mode, g, lc);
+        case 5: return qmv_mfma_launch_mode<DT, 5>(a, mode, g, lc);
+        case 6: return qmv_mfma_launch_mode<DT, 6>(a, mode, g, lc);
+        default: return fail(ERR_UNSUPPORTED, "mfma qmv: code width");
     }
 }
 
