@@ -25,7 +25,7 @@ size_t lds_bytes(uint32_t R, uint32_t K, uint32_t nch, uint32_t rows_wg, uint32_
 int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     if (p.dtype != DT_F16 && p.dtype != DT_BF16) return fail(ERR_UNSUPPORTED, "mfma qmv: f16/bf16 only");
     const bool odd = p.bits == 3 || p.bits == 5 || p.bits == 6;
-    if (!(p.bits == 2 || p.bits == 4 || (p.bits == 8 && p.dtype == DT_F16) || odd))
+    if (!(p.bits == 2 || p.bits == 4 || p.bits == 8 || odd))
         return fail(ERR_UNSUPPORTED, "mfma qmv: bits");
     if (p.N == 0 || p.K == 0) return fail(ERR_UNSUPPORTED, "mfma qmv: empty");
     // a lane's chunk: 16 bytes (128/bits codes), or 32 codes = bits dwords where codes straddle words

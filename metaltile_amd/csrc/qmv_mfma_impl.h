@@ -101,8 +101,14 @@ template <int DT> __device__ __forceinline__ m_f32x4 mfma4(m_u32x2 a, m_u32x2 b,
 // = BITS whole dwords of the bit stream, codes are extracted one by one (bit-field
 // extract, or a funnel shift where a code straddles two words) and paired in
 // natural order.
-template <int BITS> struct MfmaCodec {
+// 8-bit codes do not fit the 7 mantissa bits of bf16: there the chunk is fed as
+// two 4-bit planes (PLANES = 2), high nibbles first; the accumulator is scaled by
+// 16 between the planes, so sum = 16*sum(hi*x) + sum(lo*x) and the offset to
+// remove is MAGIC*(16+1) per activation.
+template <int DT, int BITS> struct MfmaCodec {
     static constexpr bool kPow2 = (32 % BITS) == 0;
+    static constexpr int PLANES = (DT == DT_BF16 && BITS == 8) ? 2 : 1;
+    static constexpr float kMagic = (DT == DT_BF16 ? 128.0f : 1024.0f) * (PLANES == 2 ? 17.0f : 1.0f);
     static constexpr int PF = kPow2 ? 32 / BITS : 0;     // codes per dword (power-of-two widths)
     static constexpr int NWD = kPow2 ? 4 : BITS;
     static constexpr int CPC = kPow2 ? 4 * PF : 32;
@@ -113,8 +119,17 @@ template <int BITS> struct MfmaCodec {
         return wi * PF + 2 * t + (e >> 1) + (e & 1) * (PF / 2);
     }
     // dwords of the chunk -> CPC/2 pair words (MAGIC+q_a | (MAGIC+q_b) << 16); MFMA m takes pairs 2m, 2m+1
-    static __device__ __forceinline__ void pairs(const uint32_t (&w)[NWD], uint32_t kor, uint32_t (&pw)[CPC / 2]) {
-        if constexpr (kPow2) {
+    static __device__ __forceinline__ void pairs(const uint32_t (&w)[NWD], uint32_t kor, uint32_t (&pw)[PLANES * (CPC / 2)]) {
+        if constexpr (PLANES == 2) {
+            // plane 0 = high nibbles, plane 1 = low nibbles of the byte pairs (b_j, b_{j+2})
+#pragma unroll
+            for (int wi = 0; wi < 4; wi++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    pw[wi * 2 + j] = ((w[wi] >> (8 * j + 4)) & 0x000F000Fu) | kor;
+                    pw[CPC / 2 + wi * 2 + j] = ((w[wi] >> (8 * j)) & 0x000F000Fu) | kor;
+                }
+        } else if constexpr (kPow2) {
             constexpr uint32_t MASK = ((1u << BITS) - 1u) * 0x00010001u;
 #pragma unroll
             for (int wi = 0; wi < 4; wi++)
@@ -160,14 +175,13 @@ template <int BITS> struct MfmaCodec {
 
 template <int DT, int BITS, int MP, int S, int D, int MODE, int MAXT>
 __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
-    typedef MfmaCodec<BITS> Codec;
+    typedef MfmaCodec<DT, BITS> Codec;
     constexpr int CPC = Codec::CPC;  // codes per lane chunk
     constexpr int NWD = Codec::NWD;  // dwords per lane chunk
     constexpr int NP = CPC / 8;      // 16-byte activation pieces per chunk
     constexpr int R = MP * S;       // activation rows per pass
-    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
+    constexpr float MAGIC = Codec::kMagic;
     constexpr uint32_t NOROW = 0xFFFFFFFFu;
-    static_assert(DT != DT_BF16 || BITS <= 7, "an 8-bit code does not fit the bf16 mantissa");
     static_assert(CPC % 8 == 0 && CPC / 2 >= 2, "chunk must be whole activation pieces");
 
     extern __shared__ __align__(16) unsigned char smem[];
@@ -392,20 +406,29 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                     }
                     const uint32_t g = (c * (uint32_t)CPC) >> a.log2g;
                     const float2 sb = SB[valid ? sb_row + g : rows_wg * a.gpr];
-                    uint32_t pw[CPC / 2];
+                    uint32_t pw[Codec::PLANES * (CPC / 2)];
                     Codec::pairs(ring[d], kor, pw);
                     if constexpr (ISSUE) Codec::load(w_ptr(nrb_i, nsg0 + d), ring[d]);
                     // codes -> B operands, MFMAs
                     m_f32x4 acc[S];
 #pragma unroll
-                    for (int m = 0; m < CPC / 4; m++) {  // MFMA m of the chunk: codes 4m .. 4m+3 of its operand sequence
-                        const m_u32x2 b = {pw[2 * m], pw[2 * m + 1]};
+                    for (int pl = 0; pl < Codec::PLANES; pl++) {
 #pragma unroll
-                        for (int s = 0; s < S; s++) {
-                            const m_u32x4 piece = av[s][m / 2];
-                            const m_u32x2 aop = (m & 1) ? m_u32x2{piece.z, piece.w} : m_u32x2{piece.x, piece.y};
-                            const m_f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-                            acc[s] = mfma4<DT>(aop, b, m == 0 ? zero : acc[s]);
+                        for (int m = 0; m < CPC / 4; m++) {  // MFMA m of the chunk: codes 4m .. 4m+3 of its operand sequence
+                            const m_u32x2 b = {pw[pl * (CPC / 2) + 2 * m], pw[pl * (CPC / 2) + 2 * m + 1]};
+#pragma unroll
+                            for (int s = 0; s < S; s++) {
+                                const m_u32x4 piece = av[s][m / 2];
+                                const m_u32x2 aop = (m & 1) ? m_u32x2{piece.z, piece.w} : m_u32x2{piece.x, piece.y};
+                                const m_f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                                acc[s] = mfma4<DT>(aop, b, (m == 0 && pl == 0) ? zero : acc[s]);
+                            }
+                        }
+                        if (pl + 1 < Codec::PLANES) {
+#pragma unroll
+                            for (int s = 0; s < S; s++)
+#pragma unroll
+                                for (int i = 0; i < MP; i++) acc[s][i] *= 16.0f;  // only the live rows are read later
                         }
                     }
 #pragma unroll
@@ -506,9 +529,7 @@ template <int DT> int qmv_mfma_launch_dtype(QmvMArgs& a, int bits, int mode, con
     switch (bits) {
         case 2: return qmv_mfma_launch_mode<DT, 2>(a, mode, g, lc);
         case 4: return qmv_mfma_launch_mode<DT, 4>(a, mode, g, lc);
-        default:
-            if constexpr (DT == DT_F16) return qmv_mfma_launch_mode<DT, 8>(a, mode, g, lc);
-            else return fail(ERR_UNSUPPORTED, "mfma qmv: 8-bit codes need f16 activations");
+        default: return qmv_mfma_launch_mode<DT, 8>(a, mode, g, lc);
     }
 }
 
