@@ -806,6 +806,11 @@ int mtq_set_option(const char* name, int value) {
         options().qmm_kernel = value;
         return MTQ_OK;
     }
+    if (!strcmp(name, "qmm.prefetch")) {
+        if (value != 0 && value != 2 && value != 4) return fail(ERR_BAD_ARG, "qmm.prefetch must be 0, 2 or 4");
+        options().qmm_prefetch = value;
+        return MTQ_OK;
+    }
     if (!strcmp(name, "qmm.tile_rows")) {
         if (value != 0 && value != 64 && value != 128) return fail(ERR_BAD_ARG, "qmm.tile_rows must be 0, 64 or 128");
         options().qmm_tile_rows = value;

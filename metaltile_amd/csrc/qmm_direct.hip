@@ -60,7 +60,11 @@ constexpr int DLD = DBK * 2 + 16;        // LDS row stride in bytes
 // converted weight fragment feeds MB MFMAs, so the conversion cost per MFMA
 // falls with MB; MB = 4 is the compute-bound shape, MB = 2 gives twice the
 // workgroups for small M.
-template <int DT, int BITS, int PD, int MB>
+// SBL: the scales and biases of the tile's 128 weight rows are staged once in LDS
+// (coalesced, one line per row) instead of being fetched per lane and iteration:
+// a wave-wide 2-byte load from 32 different rows costs the L1 as many tag lookups
+// as the weight load itself.
+template <int DT, int BITS, int PD, int MB, bool SBL>
 __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
     constexpr int DBM = 32 * MB;
     constexpr int DBUF = DBM * DLD;          // one activation tile
@@ -94,6 +98,11 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
     q_u32x4 px[PD][XV];
     uint32_t pw[PD][BITS];
     uint32_t ps[PD], pb[PD];
+    // LDS after the two activation tiles: [128 rows][gpr + 2] scales, then the same for biases
+    const uint32_t sbld = a.gpr + 2;  // row stride in elements; (gpr + 2) / 2 dwords is odd for gpr % 4 == 0: rows spread over the banks
+    uint16_t* sbS = (uint16_t*)(lds + 2 * DBUF);
+    uint16_t* sbB = sbS + DBN * sbld;
+    const uint32_t sbrow = (wn * 32 + fr) * sbld;
 
 #define QD_LOAD(IT, SET)                                                                 \
     do {                                                                                 \
@@ -117,9 +126,11 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
                 pw[SET][4 * i + 3] = t_.w;                                               \
             }                                                                            \
         }                                                                                \
-        const uint32_t g_ = (it_ * DBK + kofs) >> a.log2g;                               \
-        ps[SET] = *(const uint16_t*)(a.scales + soff + (size_t)g_ * 2);                  \
-        pb[SET] = *(const uint16_t*)(a.biases + soff + (size_t)g_ * 2);                  \
+        if constexpr (!SBL) {                                                            \
+            const uint32_t g_ = (it_ * DBK + kofs) >> a.log2g;                           \
+            ps[SET] = *(const uint16_t*)(a.scales + soff + (size_t)g_ * 2);              \
+            pb[SET] = *(const uint16_t*)(a.biases + soff + (size_t)g_ * 2);              \
+        }                                                                                \
     } while (0)
 
 #define QD_STORE_X(BUF, SET)                                                             \
@@ -131,6 +142,17 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
         }                                                                                \
     } while (0)
 
+    auto scale_bias = [&](uint32_t it_, int set, float& s_, float& b_) {
+        if constexpr (SBL) {
+            const uint32_t g_ = (min(it_, a.iters - 1) * DBK + kofs) >> a.log2g;
+            s_ = elem_bits_to_f32<DT>(sbS[sbrow + g_]);
+            b_ = elem_bits_to_f32<DT>(sbB[sbrow + g_]);
+        } else {
+            s_ = elem_bits_to_f32<DT>(ps[set]);
+            b_ = elem_bits_to_f32<DT>(pb[set]);
+        }
+    };
+
     f32x16 acc[MB];
 #pragma unroll
     for (int i = 0; i < MB; i++)
@@ -140,6 +162,27 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
 #pragma unroll
     for (int j = 0; j < PD; j++) QD_LOAD(j, j);
     QD_STORE_X(0, 0);
+    if constexpr (SBL) {
+        // 128 rows x gpr elements each of scales and biases: thread t copies elements [c0, c0 + per) of row t/4
+        const uint32_t row = tid >> 2, per = a.gpr / 4, c0 = (tid & 3u) * per;  // gpr % 4 == 0
+        const uint16_t* gs = (const uint16_t*)a.scales + (size_t)(n0 + row) * a.gpr + c0;
+        const uint16_t* gb = (const uint16_t*)a.biases + (size_t)(n0 + row) * a.gpr + c0;
+        for (uint32_t i = 0; i < per; i += 2) {  // per is even when gpr % 8 == 0
+            *(uint32_t*)(sbS + row * sbld + c0 + i) = *(const uint32_t*)(gs + i);
+            *(uint32_t*)(sbB + row * sbld + c0 + i) = *(const uint32_t*)(gb + i);
+        }
+        __syncthreads();
+    }
+    // Software pipeline: the weights of iteration it+1 are converted while the
+    // MFMAs of iteration it run, one conversion group behind every MFMA, so the
+    // matrix cores and the vector ALU are busy at the same time inside one wave.
+    uint4 bq[2][4];  // converted fragments: [it & 1][MFMA step]
+    {
+        float s0, b0;
+        scale_bias(0, 0, s0, b0);
+#pragma unroll
+        for (int j = 0; j < 4; j++) bq[0][j] = dequant8<DT, BITS>(pw[0], j, s0, b0);
+    }
     __syncthreads();
 
     // fragment of activation row (32*bi + fr), k = kofs + 8*j .. +8 of the iteration
@@ -148,26 +191,39 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
 #pragma unroll
         for (int par = 0; par < PD; par++) {
             const uint32_t it = it0 + par;
-            // set `par` holds iteration `it`: copy out what the MFMAs need, refill with it+PD
+            const int nx = (par + 1) % PD;  // set holding iteration it+1 (loaded PD-1 iterations ago)
+            // set `par` held iteration `it`, whose weights were converted during iteration it-1
+            // and whose activations are in LDS: refill it with iteration it+PD
             uint32_t cw[BITS];
 #pragma unroll
-            for (int i = 0; i < BITS; i++) cw[i] = pw[par][i];
-            const float s = elem_bits_to_f32<DT>(ps[par]), b = elem_bits_to_f32<DT>(pb[par]);
+            for (int i = 0; i < BITS; i++) cw[i] = pw[nx][i];
+            float s, b;
+            scale_bias(it + 1, nx, s, b);
             QD_LOAD(it + PD, par);
             QD_KEEP_ORDER();
             const unsigned char* A0 = Abase + (par & 1) * DBUF;
+            uint4 af[4][MB];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int bi = 0; bi < MB; bi++) af[j][bi] = *(const uint4*)(A0 + bi * 32 * DLD + j * 16);
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                uint4 af[MB];
 #pragma unroll
-                for (int bi = 0; bi < MB; bi++) af[bi] = *(const uint4*)(A0 + bi * 32 * DLD + j * 16);
-                const uint4 bq = dequant8<DT, BITS>(cw, j, s, b);
-#pragma unroll
-                for (int bi = 0; bi < MB; bi++) acc[bi] = mfma32<DT>(af[bi], bq, acc[bi]);
+                for (int bi = 0; bi < MB; bi++) acc[bi] = mfma32<DT>(af[j][bi], bq[par & 1][j], acc[bi]);
+                bq[(par + 1) & 1][j] = dequant8<DT, BITS>(cw, j, s, b);
             }
-            // activations of it+1 (next set, loaded PD-1 iterations ago) go to the other buffer
+            // ask the scheduler for: the LDS reads first, then one MFMA followed by its
+            // share of the conversion's vector instructions, 4*MB times
+            __builtin_amdgcn_sched_group_barrier(0x100, 4 * MB, 0);
+#pragma unroll
+            for (int g = 0; g < 4 * MB; g++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, (96 + 4 * MB - 1) / (4 * MB), 0);
+            }
+            // activations of it+1 go to the other buffer
             QD_KEEP_ORDER();
-            QD_STORE_X((par + 1) & 1, (par + 1) % PD);
+            QD_STORE_X((par + 1) & 1, nx);
             __syncthreads();
         }
     }
@@ -199,12 +255,24 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
 template <int DT> static int launch_dt(QmmDArgs& a, int bits, const LaunchCtx& lc) {
     const void* fn;
     const bool tall = a.m_tile_rows == 128;
+    // register sets of loads in flight: 4 where the iteration count allows (the
+    // weights of iteration it+1 are consumed during iteration it, so 2 sets would
+    // leave a single iteration between a load and its use)
+    int pd = options().qmm_prefetch ? options().qmm_prefetch : 2;
+    if (a.iters % 4) pd = 2;
+    // scales and biases of the tile's rows in LDS when they fit beside the activation tiles
+    const size_t sb_lds = (size_t)2 * DBN * (a.gpr + 2) * 2;
+    const bool sbl = a.gpr % 8 == 0 && sb_lds <= 64 * 1024;
+#define QD_PICK2(B, P, MBv) (sbl ? (const void*)qmm_direct_kernel<DT, B, P, MBv, true> : (const void*)qmm_direct_kernel<DT, B, P, MBv, false>)
+#define QD_PICK(B) fn = tall ? (pd == 4 ? QD_PICK2(B, 4, 4) : QD_PICK2(B, 2, 4)) : (pd == 4 ? QD_PICK2(B, 4, 2) : QD_PICK2(B, 2, 2))
     switch (bits) {
-        case 2: fn = tall ? (const void*)qmm_direct_kernel<DT, 2, 2, 4> : (const void*)qmm_direct_kernel<DT, 2, 2, 2>; break;
-        case 4: fn = tall ? (const void*)qmm_direct_kernel<DT, 4, 2, 4> : (const void*)qmm_direct_kernel<DT, 4, 2, 2>; break;
-        default: fn = tall ? (const void*)qmm_direct_kernel<DT, 8, 2, 4> : (const void*)qmm_direct_kernel<DT, 8, 2, 2>; break;
+        case 2: QD_PICK(2); break;
+        case 4: QD_PICK(4); break;
+        default: QD_PICK(8); break;
     }
-    const size_t shmem = 2 * (size_t)a.m_tile_rows * DLD;
+#undef QD_PICK2
+#undef QD_PICK
+    const size_t shmem = 2 * (size_t)a.m_tile_rows * DLD + (sbl ? sb_lds : 0);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     void* args[] = {&a};
