@@ -70,7 +70,7 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
     constexpr int DBUF = DBM * DLD;          // one activation tile
     constexpr int XV = DBM * DBK * 2 / 512 / 16;  // 16-byte vectors of the tile per thread
     extern __shared__ __align__(16) unsigned char lds[];  // 2 * DBUF bytes
-    static_assert(2 * DBUF >= DBM * DBN * 4, "the K-group reduction reuses the tile buffers");
+    // the epilogue needs DBM*DBN*(4+2) bytes: partial sums, then the element tile (checked on the host)
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t kg = wave >> 2, wn = wave & 3u;
@@ -163,13 +163,17 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
     for (int j = 0; j < PD; j++) QD_LOAD(j, j);
     QD_STORE_X(0, 0);
     if constexpr (SBL) {
-        // 128 rows x gpr elements each of scales and biases: thread t copies elements [c0, c0 + per) of row t/4
-        const uint32_t row = tid >> 2, per = a.gpr / 4, c0 = (tid & 3u) * per;  // gpr % 4 == 0
-        const uint16_t* gs = (const uint16_t*)a.scales + (size_t)(n0 + row) * a.gpr + c0;
-        const uint16_t* gb = (const uint16_t*)a.biases + (size_t)(n0 + row) * a.gpr + c0;
-        for (uint32_t i = 0; i < per; i += 2) {  // per is even when gpr % 8 == 0
-            *(uint32_t*)(sbS + row * sbld + c0 + i) = *(const uint32_t*)(gs + i);
-            *(uint32_t*)(sbB + row * sbld + c0 + i) = *(const uint32_t*)(gb + i);
+        // 128 rows x gpr elements each of scales and biases, 16 bytes per load: vector v of
+        // the tile covers elements [8*(v % vpr), +8) of row v / vpr
+        const uint32_t vpr = a.gpr / 8, nvec = DBN * vpr;
+        for (uint32_t v = tid; v < nvec; v += 512) {
+            const uint32_t row = v / vpr, c0 = (v - row * vpr) * 8;
+            const q_u32x4 sv = *(const q_u32x4*)((const uint16_t*)a.scales + (size_t)(n0 + row) * a.gpr + c0);
+            const q_u32x4 bv = *(const q_u32x4*)((const uint16_t*)a.biases + (size_t)(n0 + row) * a.gpr + c0);
+            uint32_t* ds = (uint32_t*)(sbS + row * sbld + c0);
+            uint32_t* db = (uint32_t*)(sbB + row * sbld + c0);
+            ds[0] = sv.x; ds[1] = sv.y; ds[2] = sv.z; ds[3] = sv.w;
+            db[0] = bv.x; db[1] = bv.y; db[2] = bv.z; db[3] = bv.w;
         }
         __syncthreads();
     }
@@ -239,17 +243,30 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
             for (int v = 0; v < 16; v++) red[((wn * MB + bi) * 16 + v) * 64 + lane] = acc[bi][v];
     }
     __syncthreads();
-    if (kg == 1) return;
-    // accumulator layout: column j = lane%32, row i = 8*(v/4) + 4*(lane/32) + v%4
-    const uint32_t col = n0 + wn * 32 + fr;
+    // accumulator layout: column j = lane%32, row i = 8*(v/4) + 4*(lane/32) + v%4.
+    // K-group 0 adds, rounds to the element dtype and writes the tile to LDS as
+    // [row][128 columns], behind the partial sums.
+    uint16_t* otile = (uint16_t*)(lds + DBM * DBN * 4);  // DBM x DBN elements, behind the partial sums
+    if (kg == 0) {
 #pragma unroll
-    for (int bi = 0; bi < MB; bi++)
+        for (int bi = 0; bi < MB; bi++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const uint32_t row = m0 + bi * 32 + 8 * (v / 4) + 4 * fh + (v % 4);
-            const float r = acc[bi][v] + red[((wn * MB + bi) * 16 + v) * 64 + lane];
-            if (row < a.M) store_elem<DT>(a.out, (size_t)row * a.N + col, r);
-        }
+            for (int v = 0; v < 16; v++) {
+                const uint32_t lrow = bi * 32 + 8 * (v / 4) + 4 * fh + (v % 4);
+                const float r = acc[bi][v] + red[((wn * MB + bi) * 16 + v) * 64 + lane];
+                otile[lrow * DBN + wn * 32 + fr] = f32_to_elem_bits<DT>(r);
+            }
+    }
+    __syncthreads();
+    // all 512 threads store the tile, 16 bytes each, whole 256-byte rows
+    constexpr int VPT = DBM * DBN * 2 / 16 / 512;  // 16-byte vectors per thread
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const uint32_t v = tid + i * 512, lrow = v >> 4, c16 = v & 15u;
+        const uint32_t row = m0 + lrow;
+        if (row < a.M)
+            *(q_u32x4*)((uint16_t*)a.out + (size_t)row * a.N + n0 + c16 * 8) = *(const q_u32x4*)(otile + lrow * DBN + c16 * 8);
+    }
 }
 
 template <int DT> static int launch_dt(QmmDArgs& a, int bits, const LaunchCtx& lc) {
@@ -272,7 +289,9 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, const LaunchCtx& l
     }
 #undef QD_PICK2
 #undef QD_PICK
-    const size_t shmem = 2 * (size_t)a.m_tile_rows * DLD + (sbl ? sb_lds : 0);
+    size_t shmem = 2 * (size_t)a.m_tile_rows * DLD + (sbl ? sb_lds : 0);
+    const size_t epilogue = (size_t)a.m_tile_rows * DBN * 6;  // f32 partial sums + the element tile
+    if (shmem < epilogue) shmem = epilogue;
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     void* args[] = {&a};
@@ -290,7 +309,8 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
         return fail(ERR_UNSUPPORTED, "direct qmm: N % 128, K % 256 or group size");
     if ((uint64_t)p.M * p.K * 2 >= (1ull << 32) || (uint64_t)p.N * p.K * p.bits / 8 >= (1ull << 32))
         return fail(ERR_UNSUPPORTED, "direct qmm: operand larger than 4 GiB");
-    if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16) return fail(ERR_UNSUPPORTED, "direct qmm: w and x must be 16-byte aligned");
+    if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.out % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
+        return fail(ERR_UNSUPPORTED, "direct qmm: operands must be 16-byte aligned");
     QmmDArgs a;
     a.w = (const unsigned char*)p.w;
     a.scales = (const unsigned char*)p.scales;
