@@ -806,9 +806,9 @@ int mtq_set_option(const char* name, int value) {
         options().qmm_kernel = value;
         return MTQ_OK;
     }
-    if (!strcmp(name, "qmm.prefetch")) {
-        if (value != 0 && value != 2 && value != 4) return fail(ERR_BAD_ARG, "qmm.prefetch must be 0, 2 or 4");
-        options().qmm_prefetch = value;
+    if (!strcmp(name, "qmm.kgroups")) {
+        if (value != 0 && value != 2 && value != 4) return fail(ERR_BAD_ARG, "qmm.kgroups must be 0, 2 or 4");
+        options().qmm_kgroups = value;
         return MTQ_OK;
     }
     if (!strcmp(name, "qmm.tile_rows")) {

@@ -53,8 +53,6 @@ struct QmmDArgs {
     uint32_t m_tile_rows;  // 64 or 128
 };
 
-constexpr int DBN = 128, DBK = 128;
-constexpr int DLD = DBK * 2 + 16;        // LDS row stride in bytes
 
 // MB = 32-row activation blocks per wave (tile height DBM = 32*MB): every
 // converted weight fragment feeds MB MFMAs, so the conversion cost per MFMA
@@ -64,8 +62,16 @@ constexpr int DLD = DBK * 2 + 16;        // LDS row stride in bytes
 // (coalesced, one line per row) instead of being fetched per lane and iteration:
 // a wave-wide 2-byte load from 32 different rows costs the L1 as many tag lookups
 // as the weight load itself.
-template <int DT, int BITS, int PD, int MB, bool SBL>
+// KG: K-groups per workgroup (2 or 4). The 8 waves are KG K-groups x 8/KG N-waves;
+// the tile is 32*MB rows x 32*(8/KG) columns and an iteration covers 64*KG k. KG = 4
+// halves the tile width, which doubles the number of 128-row tiles for small M.
+template <int DT, int BITS, int PD, int MB, bool SBL, int KG>
 __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
+    constexpr int NWV = 8 / KG;              // N-waves
+    constexpr int DBN = 32 * NWV, DBK = 64 * KG;
+    constexpr int DLD = DBK * 2 + 16;        // LDS row stride in bytes
+    constexpr int TPR = DBK * 2 / 32;        // threads per activation row (32 bytes each)
+    constexpr int RS = 512 / TPR;            // rows covered by one pass of the workgroup
     constexpr int DBM = 32 * MB;
     constexpr int DBUF = DBM * DLD;          // one activation tile
     constexpr int XV = DBM * DBK * 2 / 512 / 16;  // 16-byte vectors of the tile per thread
@@ -73,7 +79,7 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
     // the epilogue needs DBM*DBN*(4+2) bytes: partial sums, then the element tile (checked on the host)
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t kg = wave >> 2, wn = wave & 3u;
+    const uint32_t kg = wave / NWV, wn = wave % NWV;
     const uint32_t fr = lane & 31u, fh = lane >> 5;
 
     const uint32_t total = a.m_tiles * a.n_tiles;
@@ -82,13 +88,13 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
     const uint32_t nt = vid / a.m_tiles, mt = vid % a.m_tiles;
     const uint32_t m0 = mt * DBM, n0 = nt * DBN;
 
-    // activations: thread t moves 32 bytes of row t/8 (bytes [32*(t%8), +32) of the iteration's 256)
-    const uint32_t xr = tid >> 3, xc = tid & 7u;
+    // activations: thread t moves 32 bytes of row t/TPR (bytes [32*(t%TPR), +32) of the iteration's row)
+    const uint32_t xr = tid / TPR, xc = tid % TPR;
     uint32_t xoff[XV / 2];
 #pragma unroll
-    for (int i = 0; i < XV / 2; i++) xoff[i] = min(m0 + xr + 64 * i, a.M - 1) * (a.K * 2) + xc * 32;
+    for (int i = 0; i < XV / 2; i++) xoff[i] = min(m0 + xr + RS * i, a.M - 1) * (a.K * 2) + xc * 32;
     // weights: row n0 + 32*wn + fr, codes [64*kg + 32*fh, +32) of the iteration
-    const uint32_t wrow = n0 + wn * 32 + fr;  // < N: N is a multiple of 128
+    const uint32_t wrow = n0 + wn * 32 + fr;  // < N: N is a multiple of the tile width
     const uint32_t woff = wrow * (a.K * BITS / 8) + (kg * 64 + fh * 32) * BITS / 8;
     const uint32_t soff = wrow * a.gpr * 2;
     const uint32_t kofs = kg * 64 + fh * 32;  // k offset of this lane's codes inside an iteration
@@ -98,7 +104,7 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
     q_u32x4 px[PD][XV];
     uint32_t pw[PD][BITS];
     uint32_t ps[PD], pb[PD];
-    // LDS after the two activation tiles: [128 rows][gpr + 2] scales, then the same for biases
+    // LDS after the two activation tiles: [DBN rows][gpr + 2] scales, then the same for biases
     const uint32_t sbld = a.gpr + 2;  // row stride in elements; (gpr + 2) / 2 dwords is odd for gpr % 4 == 0: rows spread over the banks
     uint16_t* sbS = (uint16_t*)(lds + 2 * DBUF);
     uint16_t* sbB = sbS + DBN * sbld;
@@ -137,8 +143,8 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
     do {                                                                                 \
         unsigned char* d_ = lds + (BUF) * DBUF + xr * DLD + xc * 32;                     \
         _Pragma("unroll") for (int i = 0; i < XV / 2; i++) {                             \
-            *(q_u32x4*)(d_ + 64 * i * DLD) = px[SET][2 * i];                             \
-            *(q_u32x4*)(d_ + 64 * i * DLD + 16) = px[SET][2 * i + 1];                    \
+            *(q_u32x4*)(d_ + RS * i * DLD) = px[SET][2 * i];                             \
+            *(q_u32x4*)(d_ + RS * i * DLD + 16) = px[SET][2 * i + 1];                    \
         }                                                                                \
     } while (0)
 
@@ -163,7 +169,7 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
     for (int j = 0; j < PD; j++) QD_LOAD(j, j);
     QD_STORE_X(0, 0);
     if constexpr (SBL) {
-        // 128 rows x gpr elements each of scales and biases, 16 bytes per load: vector v of
+        // DBN rows x gpr elements each of scales and biases, 16 bytes per load: vector v of
         // the tile covers elements [8*(v % vpr), +8) of row v / vpr
         const uint32_t vpr = a.gpr / 8, nvec = DBN * vpr;
         for (uint32_t v = tid; v < nvec; v += 512) {
@@ -206,20 +212,41 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
             QD_LOAD(it + PD, par);
             QD_KEEP_ORDER();
             const unsigned char* A0 = Abase + (par & 1) * DBUF;
-            uint4 af[4][MB];
+            // Activation fragments: all four MFMA steps' worth up front (fastest), or two
+            // steps ahead of their use where the register file would not hold them all.
+            constexpr bool kAllUpFront = !(MB == 4 && KG == 4);
+            if constexpr (kAllUpFront) {
+                uint4 af[4][MB];
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+                for (int j = 0; j < 4; j++)
 #pragma unroll
-                for (int bi = 0; bi < MB; bi++) af[j][bi] = *(const uint4*)(A0 + bi * 32 * DLD + j * 16);
+                    for (int bi = 0; bi < MB; bi++) af[j][bi] = *(const uint4*)(A0 + bi * 32 * DLD + j * 16);
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+                for (int j = 0; j < 4; j++) {
 #pragma unroll
-                for (int bi = 0; bi < MB; bi++) acc[bi] = mfma32<DT>(af[j][bi], bq[par & 1][j], acc[bi]);
-                bq[(par + 1) & 1][j] = dequant8<DT, BITS>(cw, j, s, b);
+                    for (int bi = 0; bi < MB; bi++) acc[bi] = mfma32<DT>(af[j][bi], bq[par & 1][j], acc[bi]);
+                    bq[(par + 1) & 1][j] = dequant8<DT, BITS>(cw, j, s, b);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x100, 4 * MB, 0);
+            } else {
+                uint4 af[2][MB];
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int bi = 0; bi < MB; bi++) af[j][bi] = *(const uint4*)(A0 + bi * 32 * DLD + j * 16);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+#pragma unroll
+                    for (int bi = 0; bi < MB; bi++) acc[bi] = mfma32<DT>(af[j & 1][bi], bq[par & 1][j], acc[bi]);
+                    if (j + 2 < 4) {
+#pragma unroll
+                        for (int bi = 0; bi < MB; bi++) af[j & 1][bi] = *(const uint4*)(A0 + bi * 32 * DLD + (j + 2) * 16);
+                    }
+                    bq[(par + 1) & 1][j] = dequant8<DT, BITS>(cw, j, s, b);
+                }
             }
-            // ask the scheduler for: the LDS reads first, then one MFMA followed by its
-            // share of the conversion's vector instructions, 4*MB times
-            __builtin_amdgcn_sched_group_barrier(0x100, 4 * MB, 0);
+            // ask the scheduler for one MFMA followed by its share of the conversion's
+            // vector instructions, 4*MB times
 #pragma unroll
             for (int g = 0; g < 4 * MB; g++) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -234,64 +261,71 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
 #undef QD_LOAD
 #undef QD_STORE_X
 
-    // ---- K-group 1 hands its accumulators to K-group 0 through LDS -----------
-    float* red = (float*)lds;  // [wn][bi][v][lane]
-    if (kg == 1) {
+    // ---- the other K-groups hand their accumulators to K-group 0 through LDS ---
+    float* red = (float*)lds;  // [kg - 1][wn][bi][v][lane]
+    constexpr int GRP = NWV * MB * 16 * 64;  // floats per K-group
+    if (kg != 0) {
 #pragma unroll
         for (int bi = 0; bi < MB; bi++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) red[((wn * MB + bi) * 16 + v) * 64 + lane] = acc[bi][v];
+            for (int v = 0; v < 16; v++) red[(kg - 1) * GRP + ((wn * MB + bi) * 16 + v) * 64 + lane] = acc[bi][v];
     }
     __syncthreads();
     // accumulator layout: column j = lane%32, row i = 8*(v/4) + 4*(lane/32) + v%4.
     // K-group 0 adds, rounds to the element dtype and writes the tile to LDS as
-    // [row][128 columns], behind the partial sums.
-    uint16_t* otile = (uint16_t*)(lds + DBM * DBN * 4);  // DBM x DBN elements, behind the partial sums
+    // [row][DBN columns], behind the partial sums.
+    uint16_t* otile = (uint16_t*)(lds + (KG - 1) * GRP * 4);
     if (kg == 0) {
 #pragma unroll
         for (int bi = 0; bi < MB; bi++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const uint32_t lrow = bi * 32 + 8 * (v / 4) + 4 * fh + (v % 4);
-                const float r = acc[bi][v] + red[((wn * MB + bi) * 16 + v) * 64 + lane];
+                float r = acc[bi][v];
+#pragma unroll
+                for (int g = 0; g < KG - 1; g++) r += red[g * GRP + ((wn * MB + bi) * 16 + v) * 64 + lane];
                 otile[lrow * DBN + wn * 32 + fr] = f32_to_elem_bits<DT>(r);
             }
     }
     __syncthreads();
-    // all 512 threads store the tile, 16 bytes each, whole 256-byte rows
-    constexpr int VPT = DBM * DBN * 2 / 16 / 512;  // 16-byte vectors per thread
+    // all 512 threads store the tile, 16 bytes each, whole rows
+    constexpr int VPR = DBN / 8;                    // 16-byte vectors per tile row
+    constexpr int VPT = DBM * VPR / 512;            // vectors per thread
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
-        const uint32_t v = tid + i * 512, lrow = v >> 4, c16 = v & 15u;
+        const uint32_t v = tid + i * 512, lrow = v / VPR, c16 = v % VPR;
         const uint32_t row = m0 + lrow;
         if (row < a.M)
             *(q_u32x4*)((uint16_t*)a.out + (size_t)row * a.N + n0 + c16 * 8) = *(const q_u32x4*)(otile + lrow * DBN + c16 * 8);
     }
 }
 
-template <int DT> static int launch_dt(QmmDArgs& a, int bits, const LaunchCtx& lc) {
+// LDS of one workgroup: two activation tiles, the tile's scales and biases, and at the
+// end the K-groups' partial sums followed by the element tile.
+static size_t lds_need(uint32_t rows, uint32_t kg, uint32_t gpr, bool sbl) {
+    const uint32_t dbn = 32 * (8 / kg), dbk = 64 * kg;
+    size_t main_loop = 2 * (size_t)rows * (dbk * 2 + 16) + (sbl ? (size_t)2 * dbn * (gpr + 2) * 2 : 0);
+    size_t epilogue = (size_t)(kg - 1) * rows * dbn * 4 + (size_t)rows * dbn * 2;
+    return main_loop > epilogue ? main_loop : epilogue;
+}
+
+template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, const LaunchCtx& lc) {
     const void* fn;
     const bool tall = a.m_tile_rows == 128;
-    // register sets of loads in flight: 4 where the iteration count allows (the
-    // weights of iteration it+1 are consumed during iteration it, so 2 sets would
-    // leave a single iteration between a load and its use)
-    int pd = options().qmm_prefetch ? options().qmm_prefetch : 2;
-    if (a.iters % 4) pd = 2;
+    const uint32_t dbn = 32 * (8 / kgroups);
     // scales and biases of the tile's rows in LDS when they fit beside the activation tiles
-    const size_t sb_lds = (size_t)2 * DBN * (a.gpr + 2) * 2;
-    const bool sbl = a.gpr % 8 == 0 && sb_lds <= 64 * 1024;
-#define QD_PICK2(B, P, MBv) (sbl ? (const void*)qmm_direct_kernel<DT, B, P, MBv, true> : (const void*)qmm_direct_kernel<DT, B, P, MBv, false>)
-#define QD_PICK(B) fn = tall ? (pd == 4 ? QD_PICK2(B, 4, 4) : QD_PICK2(B, 2, 4)) : (pd == 4 ? QD_PICK2(B, 4, 2) : QD_PICK2(B, 2, 2))
+    const bool sbl = a.gpr % 8 == 0 && (size_t)2 * dbn * (a.gpr + 2) * 2 <= 48 * 1024;
+    const size_t shmem = lds_need(a.m_tile_rows, kgroups, a.gpr, sbl);
+    if (shmem > 160 * 1024) return fail(ERR_UNSUPPORTED, "direct qmm: tile does not fit in LDS");
+#define QD_PICK3(B, MBv, KGv) (sbl ? (const void*)qmm_direct_kernel<DT, B, 2, MBv, true, KGv> : (const void*)qmm_direct_kernel<DT, B, 2, MBv, false, KGv>)
+#define QD_PICK(B) fn = kgroups == 4 ? (tall ? QD_PICK3(B, 4, 4) : QD_PICK3(B, 2, 4)) : (tall ? QD_PICK3(B, 4, 2) : QD_PICK3(B, 2, 2))
     switch (bits) {
         case 2: QD_PICK(2); break;
         case 4: QD_PICK(4); break;
         default: QD_PICK(8); break;
     }
-#undef QD_PICK2
 #undef QD_PICK
-    size_t shmem = 2 * (size_t)a.m_tile_rows * DLD + (sbl ? sb_lds : 0);
-    const size_t epilogue = (size_t)a.m_tile_rows * DBN * 6;  // f32 partial sums + the element tile
-    if (shmem < epilogue) shmem = epilogue;
+#undef QD_PICK3
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     void* args[] = {&a};
@@ -305,8 +339,8 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
         return fail(ERR_UNSUPPORTED, "direct qmm: f16 / bf16 activations only");
     if (p.bits != 2 && p.bits != 4 && p.bits != 8) return fail(ERR_UNSUPPORTED, "direct qmm: bits must be 2, 4 or 8");
     const uint32_t G = p.group_size;
-    if (p.M == 0 || p.N % DBN || p.K % (2 * DBK) || G < 32 || (G & (G - 1)) || p.K % G)
-        return fail(ERR_UNSUPPORTED, "direct qmm: N % 128, K % 256 or group size");
+    if (p.M == 0 || p.N % 128 || p.K % 512 || G < 32 || (G & (G - 1)) || p.K % G)
+        return fail(ERR_UNSUPPORTED, "direct qmm: N % 128, K % 512 or group size");
     if ((uint64_t)p.M * p.K * 2 >= (1ull << 32) || (uint64_t)p.N * p.K * p.bits / 8 >= (1ull << 32))
         return fail(ERR_UNSUPPORTED, "direct qmm: operand larger than 4 GiB");
     if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.out % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
@@ -324,18 +358,24 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
     while ((1u << l) < G) l++;
     a.log2g = l;
     a.gpr = p.K / G;
-    // 128-row tiles convert each weight once per 4 MFMAs instead of once per 2, but
-    // halve the workgroup count: used once they still fill the chip (measured at
-    // N = K = 4096: M = 512 runs 40 us on 64-row tiles, 50 us on 128-row tiles;
-    // M = 2048 runs 157 us and 105 us).
+    // Tile choice, measured at N = K = 4096: 128 x 128 tiles (each converted weight
+    // feeds 4 MFMAs) win once they fill the chip (M >= 1024: 42-47 us against 50);
+    // below that 64 x 128 (M = 512: 29 us against 37-42); and when even those leave
+    // half the chip idle, 64 x 64 tiles on 4 K-groups (M = 128: 18.6 us against 26).
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    const uint64_t tall_tiles = (uint64_t)((p.M + 127) / 128) * (p.N / DBN);
-    a.m_tile_rows = options().qmm_tile_rows ? (uint32_t)options().qmm_tile_rows : (tall_tiles >= (uint64_t)cus ? 128u : 64u);
-    a.m_tiles = (p.M + a.m_tile_rows - 1) / a.m_tile_rows;
-    a.n_tiles = p.N / DBN;
-    a.iters = p.K / DBK;  // even
-    return p.dtype == DT_BF16 ? launch_dt<DT_BF16>(a, p.bits, lc) : launch_dt<DT_F16>(a, p.bits, lc);
+    const uint64_t tall_wide = (uint64_t)((p.M + 127) / 128) * (p.N / 128);
+    const uint64_t short_wide = (uint64_t)((p.M + 63) / 64) * (p.N / 128);
+    uint32_t rows = 64, kgroups = 2;
+    if (tall_wide >= (uint64_t)cus) { rows = 128; kgroups = 2; }
+    else if (short_wide * 2 <= (uint64_t)cus) { rows = 64; kgroups = 4; }  // few tiles: halve their width
+    if (options().qmm_tile_rows) rows = (uint32_t)options().qmm_tile_rows;
+    if (options().qmm_kgroups) kgroups = (uint32_t)options().qmm_kgroups;
+    a.m_tile_rows = rows;
+    a.m_tiles = (p.M + rows - 1) / rows;
+    a.n_tiles = p.N / (32 * (8 / kgroups));
+    a.iters = p.K / (64 * kgroups);  // even: K % 512 == 0
+    return p.dtype == DT_BF16 ? launch_dt<DT_BF16>(a, p.bits, kgroups, lc) : launch_dt<DT_F16>(a, p.bits, kgroups, lc);
 }
 
 }  // namespace mtq
