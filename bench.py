@@ -37,7 +37,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=8, help="distinct MLP weight sets streamed per step")
-    ap.add_argument("--workload", default="qmv", choices=["qmv", "qmm", "gather", "quantize", "dequantize", "copy"],
+    ap.add_argument("--workload", default="qmv", choices=["qmv", "qkv", "qmm", "gather", "quantize", "dequantize", "copy"],
                     help="qmv is the headline; qmm / gather report the other configurations; "
                          "copy runs only the known-size copy kernel (counter calibration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -177,6 +177,43 @@ def main():
         })
         if not a.no_cpu:
             out["cpu_baseline"] = cpu_baseline_qmv(a.cpu_seconds)
+        print(json.dumps(out))
+        return
+
+    if a.workload == "qkv":
+        # The fused Q/K/V projection of one decode step (Llama-3-8B: 4096 + 1024 + 1024 rows of 4096),
+        # one launch per layer, rotating over `layers` weight sets.
+        K, Ns = 4096, (4096, 1024, 1024)
+        specs, keep, launch_bytes = [], [], 0
+        for layer in range(a.layers):
+            bufs = {"out": GpuBuffer(sum(Ns) * 2)}
+            for j, (tag, n) in enumerate(zip("qkv", Ns)):
+                c = make_case(7000 + layer * 3 + j, dt, 4, 64, 1, n, K)
+                bufs[f"w_{tag}"], bufs[f"scales_{tag}"], bufs[f"biases_{tag}"] = (
+                    GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes), GpuBuffer.from_bytes(c.biases_bytes))
+                if j == 0:
+                    bufs["x"] = GpuBuffer.from_bytes(c.x_bytes)
+            keep.append(bufs)
+            specs.append(("ffai_batched_qkv_qgemv_fast", dt, bufs,
+                          {"out_q": Ns[0], "out_k": Ns[1], "out_v": Ns[2], "in_dim": K, "group_size": 64}))
+        launch_bytes = sum(qmv_bytes(n, K, 4, 64, 1, 2) for n in Ns) - 2 * K * 2   # x is read once
+        runner.flush_slc()
+        runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
+        _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+        kern_avg = chain_us / (a.steps * len(specs))
+        gbs = launch_bytes * len(specs) * a.steps / wall_us / 1e3
+        achieved = launch_bytes / kern_avg / 1e3
+        out.update({
+            "metric": "fused QKV qmv GB/s (4-bit g64 bf16, 4096+1024+1024 rows of 4096)", "value": round(gbs, 1), "unit": "GB/s",
+            "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
+            "config": {"workload": "ffai_batched_qkv_qgemv_fast 4-bit g64 bf16, Llama-3-8B attention projections, batch 1",
+                       "launches_per_step": len(specs), "bytes_per_launch": launch_bytes,
+                       "device": info["name"] or info["arch"]},
+            "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                         "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, 1 row>, 3 matrices per launch",
+                         "avg_launch_us_timed_region": round(kern_avg, 3)},
+        })
         print(json.dumps(out))
         return
 

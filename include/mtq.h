@@ -153,6 +153,18 @@ MTQ_API int mtq_gather_qmv_single(int dtype, int bits, uint32_t group_size, cons
                                   const uint32_t *expert_index, void *output, uint32_t N,
                                   uint32_t K, uint32_t E);
 
+/* Batched qmv: n_mats (1..4) weight matrices of the same K, code width and group size
+ * against ONE activation row, in one launch: outs[j][n] = sum_k w_hat_j[n,k] * x[k].
+ * Replaces ffai_batched_qkv_qgemv / _fast (three matrices, one concatenated output:
+ * pass outs[j] = out + offset; crates/metaltile-std/src/ffai/batched_qkv_qgemv.rs:42-59,
+ * 157-174) and ffai_batched_4_qgemv_fast (four matrices, four outputs;
+ * crates/metaltile-std/src/ffai/batched_4_qgemv.rs:60-84), and fuses e.g. the gate and
+ * up projections of an MLP. w / scales / biases / outs / N are host arrays of n_mats
+ * device pointers / row counts. */
+MTQ_API int mtq_qmv_batched(int dtype, int bits, uint32_t group_size, int n_mats, const void *const *w,
+                            const void *const *scales, const void *const *biases, const void *x,
+                            void *const *outs, const uint32_t *N, uint32_t K);
+
 /* ---- the packed format's writer and reader ------------------------------ */
 
 /* Affine quantise: per group of `group_size` consecutive elements of w (T[n_elem]),

@@ -149,6 +149,35 @@ static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s,
     return op_qmv(dtype, bits, G, w, s, b, x, out, M, N, K, lc);
 }
 
+// Fused projections: one launch when the shape fits the streaming kernel, else one qmv per matrix.
+static int op_qmv_batched(int dtype, int bits, uint32_t G, int n, const void* const* w, const void* const* s,
+                          const void* const* b, const void* x, void* const* outs, const uint32_t* N, uint32_t K,
+                          const LaunchCtx& lc) {
+    if (n < 1 || n > 4 || !w || !s || !b || !outs || !N || !x) return fail(ERR_BAD_ARG, "batched qmv: 1..4 matrices, non-null arrays");
+    for (int j = 0; j < n; j++) {
+        int rc = check_common(dtype, bits, G, N[j], K);
+        if (rc) return rc;
+        if (!w[j] || !s[j] || !b[j] || !outs[j]) return fail(ERR_BAD_ARG, "null buffer");
+    }
+    if (n >= 2) {
+        QmvParams p;
+        p.dtype = dtype; p.bits = bits; p.group_size = G; p.x = x; p.K = K;
+        QmvBatch qb;
+        qb.n = n;
+        for (int j = 0; j < n; j++) { qb.w[j] = w[j]; qb.scales[j] = s[j]; qb.biases[j] = b[j]; qb.out[j] = outs[j]; qb.N[j] = N[j]; }
+        int rc = launch_qmv_batched(p, qb, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
+    for (int j = 0; j < n; j++) {
+        LaunchCtx l2 = lc;
+        if (j) l2.start = nullptr;
+        if (j + 1 < n) l2.stop = nullptr;
+        int rc = op_qmv(dtype, bits, G, w[j], s[j], b[j], x, outs[j], 1, N[j], K, l2);
+        if (rc) return rc;
+    }
+    return ERR_OK;
+}
+
 static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, const void* w,
                      const void* s, const void* b, const uint32_t* route, void* out, uint32_t T,
                      uint32_t N, uint32_t K, uint32_t E, const LaunchCtx& lc) {
@@ -169,7 +198,7 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
 // name-keyed dispatch table
 // ---------------------------------------------------------------------------
 
-enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ };
+enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4 };
 
 struct KernelDesc {
     const char* name;
@@ -222,6 +251,10 @@ static const KernelDesc kTable[] = {
     {"mt_moe_gather_qmm_mma_int8", F_GIDX, 8, 6, 4}, {"mt_moe_gather_qmm_mma_b3", F_GIDX, 3, 6, 4},
     {"mt_moe_gather_qmm_mma_b5", F_GIDX, 5, 6, 4}, {"mt_moe_gather_qmm_mma_b6", F_GIDX, 6, 6, 4},
     {"mt_moe_gather_qmm_mma_b8", F_GIDX, 8, 6, 4},
+    // x, (w, scales, biases) x 3, out | out_q, out_k, out_v, in_dim, group_size
+    {"ffai_batched_qkv_qgemv", F_BQKV, 4, 11, 5}, {"ffai_batched_qkv_qgemv_fast", F_BQKV, 4, 11, 5},
+    // x, (w, scales, biases) x 4, a_out .. d_out | out_a .. out_d, in_dim, group_size
+    {"ffai_batched_4_qgemv_fast", F_B4, 4, 17, 6},
     // w, out, scales, biases | group_size
     {"mt_affine_quantize_int2", F_AQ, 2, 4, 1}, {"mt_affine_quantize_int3", F_AQ, 3, 4, 1},
     {"mt_affine_quantize_int4", F_AQ, 4, 4, 1}, {"mt_affine_quantize_int5", F_AQ, 5, 4, 1},
@@ -364,6 +397,37 @@ static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, in
             MTQ_NEED(bufs[5], "out", (uint64_t)T * N * sz);
             return op_gather(GATHER_INDICES, dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr,
                              bufs[3].ptr, (const uint32_t*)bufs[4].ptr, bufs[5].ptr, T, N, K, E, lc);
+        }
+        case F_BQKV:
+        case F_B4: {
+            const int n = d.fam == F_BQKV ? 3 : 4;
+            const uint32_t K = consts[n], G = consts[n + 1];
+            if (K == 0 || G == 0 || K % G) return fail(ERR_SHAPE, "group_size must divide in_dim");
+            MTQ_NEED(bufs[0], "x", (uint64_t)K * sz);
+            const void *w[4], *s[4], *b[4];
+            void* outs[4];
+            uint32_t N[4];
+            uint64_t off = 0, total = 0;
+            for (int j = 0; j < n; j++) total += consts[j];
+            if (d.fam == F_BQKV) MTQ_NEED(bufs[10], "out", total * sz);
+            for (int j = 0; j < n; j++) {
+                N[j] = consts[j];
+                if (N[j] == 0) return fail(ERR_SHAPE, "every out_* must be non-zero");
+                MTQ_NEED(bufs[1 + 3 * j], "w_*", (uint64_t)N[j] * K * bits / 8);
+                MTQ_NEED(bufs[2 + 3 * j], "scales_*", (uint64_t)N[j] * (K / G) * sz);
+                MTQ_NEED(bufs[3 + 3 * j], "biases_*", (uint64_t)N[j] * (K / G) * sz);
+                w[j] = bufs[1 + 3 * j].ptr;
+                s[j] = bufs[2 + 3 * j].ptr;
+                b[j] = bufs[3 + 3 * j].ptr;
+                if (d.fam == F_BQKV) {
+                    outs[j] = (char*)bufs[10].ptr + off * sz;  // Q, K, V concatenated in that order
+                    off += N[j];
+                } else {
+                    MTQ_NEED(bufs[13 + j], "*_out", (uint64_t)N[j] * sz);
+                    outs[j] = bufs[13 + j].ptr;
+                }
+            }
+            return op_qmv_batched(dtype, d.bits, G, n, w, s, b, bufs[0].ptr, outs, N, K, lc);
         }
         case F_AQ: {
             // element count = length of the input tensor (one workgroup per group in
@@ -570,6 +634,14 @@ int mtq_gather_qmv_single(int dtype, int bits, uint32_t group_size, const void* 
     if (rc) return rc;
     return op_gather(GATHER_SINGLE, dtype, bits, group_size, input, w, scales, biases, expert_index,
                      output, 1, N, K, E, make_ctx());
+}
+
+int mtq_qmv_batched(int dtype, int bits, uint32_t group_size, int n_mats, const void* const* w,
+                    const void* const* scales, const void* const* biases, const void* x, void* const* outs,
+                    const uint32_t* N, uint32_t K) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return op_qmv_batched(dtype, bits, group_size, n_mats, w, scales, biases, x, outs, N, K, make_ctx());
 }
 
 int mtq_affine_quantize(int dtype, int bits, uint32_t group_size, const void* w, void* out,

@@ -68,6 +68,17 @@ struct QmvParams {
     uint32_t E = 1;                   // experts
 };
 
+// Several weight matrices with the same K, code width and group size against one
+// activation row (the fused projections of a decode step).
+struct QmvBatch {
+    int n = 0;                       // 2..4 matrices
+    const void* w[4] = {};
+    const void* scales[4] = {};
+    const void* biases[4] = {};
+    void* out[4] = {};
+    uint32_t N[4] = {};
+};
+
 // Tuning overrides set through mtq_set_option (0 = automatic).
 struct Options {
     int qmv_rows_per_thread = 0;  // one-shot kernel: weight rows per thread
@@ -90,6 +101,10 @@ Options& options();
 // Fast LDS/dot2 GEMV family (qmv.hip). Returns ERR_UNSUPPORTED when the shape
 // does not fit its geometry so the caller can fall back to the generic kernel.
 int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc);
+// One launch for all matrices of `b` (p carries dtype, bits, group size, x, K; its
+// w / scales / biases / out / N are ignored). ERR_UNSUPPORTED when the shape does not
+// fit the streaming kernel: the caller then runs the matrices one by one.
+int launch_qmv_batched(const QmvParams& p, const QmvBatch& b, const LaunchCtx& lc);
 // Matrix-core streaming GEMV family for f16/bf16 (qmv_mfma.hip); same contract.
 int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc);
 // One-wave-per-output kernel for any bit width 2..8 and any group size (generic.hip).

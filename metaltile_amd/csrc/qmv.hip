@@ -35,7 +35,7 @@ static int num_cus() {
 // and at least two batches are pipelined. Returns ERR_UNSUPPORTED when the
 // shape is better served by the one-shot kernel.
 static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint32_t tpb, uint32_t rows,
-                             const LaunchCtx& lc) {
+                             const LaunchCtx& lc, const QmvBatch* batch = nullptr) {
     const uint32_t G = p.group_size, gpr = p.K / G;
     if (C % 64 || gpr % 4 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
         return fail(ERR_UNSUPPORTED, "stream qmv: geometry");
@@ -50,12 +50,21 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
             if (opt.qmv_stream_batches && (uint32_t)opt.qmv_stream_batches != nb) continue;
             const uint32_t rpw = d * nb * rps;
             if (rpw > p.N + d * rps) break;
-            const uint32_t grid = (p.N + rpw - 1) / rpw;
+            uint32_t grid = (p.N + rpw - 1) / rpw;
+            if (batch) {  // workgroups that do work, over all matrices
+                grid = 0;
+                for (int j = 0; j < batch->n; j++) grid += (batch->N[j] + rpw - 1) / rpw;
+            }
             const uint64_t vecs = (uint64_t)rpw * gpr / 4;
             if ((vecs + tpb - 1) / tpb > 4) break;
             const size_t lds = (size_t)rpw * gpr * 8 + (size_t)rpw * rows * (C / 64) * 4;
             if (lds > 64 * 1024) break;
-            const double waste = (double)((uint64_t)grid * rpw - p.N) / p.N;
+            uint64_t n_all = p.N;
+            if (batch) {
+                n_all = 0;
+                for (int j = 0; j < batch->n; j++) n_all += batch->N[j];
+            }
+            const double waste = (double)((uint64_t)grid * rpw - n_all) / n_all;
             const uint32_t rounds = (grid + cus - 1) / cus;
             const double idle = (double)(rounds * cus - grid) / (rounds * cus);
             const double waves_per_cu = (double)grid / cus * (tpb / 64);
@@ -88,6 +97,18 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
     a.rows_per_wg = best_d * best_nb * rps;
     a.nb = best_nb;
     a.E = p.E;
+    a.nmat = 0;
+    if (batch) {
+        a.nmat = (uint32_t)batch->n;
+        for (int j = 0; j < 4; j++) {
+            const int k = j < batch->n ? j : 0;  // unused slots repeat matrix 0
+            a.mw[j] = batch->w[k];
+            a.ms[j] = batch->scales[k];
+            a.mbias[j] = batch->biases[k];
+            a.mo[j] = batch->out[k];
+            a.mn[j] = batch->N[k];
+        }
+    }
     QmvSGeom g;
     g.mb = (int)rows;
     g.d = (int)best_d;
@@ -96,13 +117,41 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
     g.sbi = per_thread <= 1 ? 1 : per_thread <= 2 ? 2 : 4;
     g.tpb = tpb;
     g.shmem = (size_t)a.rows_per_wg * gpr * 8 + (size_t)a.rows_per_wg * rows * a.wpr * 4;
-    g.grid = dim3((p.N + a.rows_per_wg - 1) / a.rows_per_wg, 1, 1);
+    g.grid = dim3((p.N + a.rows_per_wg - 1) / a.rows_per_wg, batch ? (uint32_t)batch->n : 1u, 1);
     switch (p.dtype) {
         case DT_F32: return qmv_stream_launch_dtype<DT_F32>(a, p.bits, p.gather, g, lc);
         case DT_F16: return qmv_stream_launch_dtype<DT_F16>(a, p.bits, p.gather, g, lc);
         case DT_BF16: return qmv_stream_launch_dtype<DT_BF16>(a, p.bits, p.gather, g, lc);
         default: return fail(ERR_BAD_ARG, "unknown dtype");
     }
+}
+
+int launch_qmv_batched(const QmvParams& p0, const QmvBatch& b, const LaunchCtx& lc) {
+    if (b.n < 2 || b.n > 4) return fail(ERR_BAD_ARG, "batched qmv takes 2 to 4 matrices");
+    if (p0.bits != 2 && p0.bits != 4 && p0.bits != 8) return fail(ERR_UNSUPPORTED, "batched qmv: bits must be 2, 4 or 8");
+    QmvParams p = p0;
+    p.gather = GATHER_NONE;
+    p.M = 1;
+    p.N = 0;
+    for (int j = 0; j < b.n; j++) {
+        if (!b.w[j] || !b.scales[j] || !b.biases[j] || !b.out[j] || b.N[j] == 0) return fail(ERR_BAD_ARG, "batched qmv: null buffer or empty matrix");
+        if ((uintptr_t)b.w[j] % 16 || (uintptr_t)b.scales[j] % 16 || (uintptr_t)b.biases[j] % 16)
+            return fail(ERR_UNSUPPORTED, "batched qmv: operands must be 16-byte aligned");
+        if (b.N[j] > p.N) p.N = b.N[j];  // the geometry (and the grid) follow the tallest matrix
+    }
+    p.w = b.w[0];
+    p.scales = b.scales[0];
+    p.biases = b.biases[0];
+    p.out = b.out[0];
+    const uint32_t cpc = 128u / (uint32_t)p.bits;
+    if (p.K == 0 || p.K % cpc) return fail(ERR_UNSUPPORTED, "batched qmv: K*bits % 128 != 0");
+    const uint32_t G = p.group_size;
+    if (!is_pow2(G) || G * 2 < cpc || p.K % G) return fail(ERR_UNSUPPORTED, "batched qmv: group size");
+    const uint32_t C = p.K / cpc;
+    if (C > 1024 || C % 64 || (uintptr_t)p.x % 16) return fail(ERR_UNSUPPORTED, "batched qmv: row geometry");
+    uint32_t rps = 1;
+    while (C * rps < 256 && C * rps * 2 <= 1024) rps *= 2;
+    return launch_qmv_stream(p, C, rps, C * rps, 1, lc, &b);
 }
 
 int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {

@@ -347,6 +347,14 @@ struct QmvSArgs {
     uint32_t rows_per_wg;    // multiple of D*rps
     uint32_t nb;             // batches of D rows per thread
     uint32_t E;
+    // Batched launch (several weight matrices against the same activations, blockIdx.y
+    // = matrix): per-matrix operands; nmat = 0 for a plain launch.
+    uint32_t nmat;
+    uint32_t mn[4];
+    const void* mw[4];
+    const void* ms[4];
+    const void* mbias[4];
+    void* mo[4];
 };
 
 typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
@@ -393,21 +401,37 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
     const uint32_t rsub = tid / a.C;
     const uint32_t lane = tid & 63u;
     const uint32_t rb = blockIdx.x * a.rows_per_wg;
-    const uint32_t rows_here = min(a.rows_per_wg, a.N - rb);     // >= 1 by construction of the grid
+    // operands of this workgroup's matrix (selected with scalar compares: an indexed
+    // read of the argument arrays would go through scratch memory)
+    const u32x4* Wm = a.w;
+    const void* Sm = a.scales;
+    const void* Bm = a.biases;
+    void* Om = a.out;
+    uint32_t Nm = a.N;
+    if (a.nmat) {
+        const uint32_t j = blockIdx.y;
+        Wm = (const u32x4*)(j == 0 ? a.mw[0] : j == 1 ? a.mw[1] : j == 2 ? a.mw[2] : a.mw[3]);
+        Sm = j == 0 ? a.ms[0] : j == 1 ? a.ms[1] : j == 2 ? a.ms[2] : a.ms[3];
+        Bm = j == 0 ? a.mbias[0] : j == 1 ? a.mbias[1] : j == 2 ? a.mbias[2] : a.mbias[3];
+        Om = j == 0 ? a.mo[0] : j == 1 ? a.mo[1] : j == 2 ? a.mo[2] : a.mo[3];
+        Nm = j == 0 ? a.mn[0] : j == 1 ? a.mn[1] : j == 2 ? a.mn[2] : a.mn[3];
+        if (rb >= Nm) return;  // the grid is sized for the tallest matrix
+    }
+    const uint32_t rows_here = min(a.rows_per_wg, Nm - rb);      // >= 1 by construction of the grid
     const uint32_t k0 = c * CPC;
 
     uint32_t expert = 0;
     if constexpr (MODE == GATHER_SINGLE) expert = min(a.route[0], a.E - 1);
-    const size_t slab_rows = (size_t)expert * a.N;
-    const u32x4* wbase = a.w + (slab_rows + rb) * a.C + c;
+    const size_t slab_rows = (size_t)expert * Nm;
+    const u32x4* wbase = Wm + (slab_rows + rb) * a.C + c;
 
     // ---- loads, smallest first ----------------------------------------------
     const size_t sb0 = (slab_rows + rb) * a.gpr;
     const uint32_t n_sb = rows_here * a.gpr;
     sbvec_t sraw[SBI], braw[SBI];
     {
-        const sbvec_t* sp = (const sbvec_t*)((const elem_t*)a.scales + sb0);
-        const sbvec_t* bp = (const sbvec_t*)((const elem_t*)a.biases + sb0);
+        const sbvec_t* sp = (const sbvec_t*)((const elem_t*)Sm + sb0);
+        const sbvec_t* bp = (const sbvec_t*)((const elem_t*)Bm + sb0);
         const uint32_t last = n_sb / 4 - 1;
 #pragma unroll
         for (int j = 0; j < SBI; j++) {
@@ -505,7 +529,7 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
         if (mb >= a.M) continue;
         float sum = 0.f;
         for (uint32_t wi = 0; wi < a.wpr; wi++) sum += part[o * a.wpr + wi];
-        store_elem<DT>(a.out, (size_t)mb * a.N + rb + rl, sum);
+        store_elem<DT>(Om, (size_t)mb * Nm + rb + rl, sum);
     }
 }
 

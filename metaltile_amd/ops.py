@@ -45,6 +45,15 @@ def gather_qmv_single(dtype, bits, group_size, w, scales, biases, inp, expert_in
                                          _p(inp), _p(expert_index), _p(out), N, K, E))
 
 
+def qmv_batched(dtype, bits, group_size, ws, scales, biases, x, outs, Ns, K):
+    """2..4 weight matrices (lists of buffers) against one activation row, one launch."""
+    lib = _ensure_init()
+    n = len(ws)
+    arr = lambda bufs: (C.c_void_p * n)(*[_p(b) for b in bufs])
+    _lib.check(lib.mtq_qmv_batched(int(dtype), bits, group_size, n, arr(ws), arr(scales), arr(biases), _p(x), arr(outs),
+                                   (C.c_uint32 * n)(*Ns), K))
+
+
 def affine_quantize(dtype, bits, group_size, w, out, scales, biases, n_elem):
     """w: T[n_elem] -> out: packed u32 words, scales / biases: T[n_elem / group_size]."""
     lib = _ensure_init()

@@ -64,3 +64,10 @@ for _b in (2, 3, 4, 5, 6, 8):
     _add(f"mt_affine_quantize_int{_b}", _b, ("w", "out", "scales", "biases"), ("group_size",),
          ("out", "scales", "biases"))
     _add(f"mt_affine_dequantize_int{_b}", _b, ("w", "scales", "biases", "out"), ("group_size",), ("out",))
+_QKV = ("x", "w_q", "scales_q", "biases_q", "w_k", "scales_k", "biases_k", "w_v", "scales_v", "biases_v", "out")
+for _n in ("ffai_batched_qkv_qgemv", "ffai_batched_qkv_qgemv_fast"):
+    _add(_n, 4, _QKV, ("out_q", "out_k", "out_v", "in_dim", "group_size"), ("out",))
+_add("ffai_batched_4_qgemv_fast", 4,
+     ("x", "w_a", "scales_a", "biases_a", "w_b", "scales_b", "biases_b", "w_c", "scales_c", "biases_c",
+      "w_d", "scales_d", "biases_d", "a_out", "b_out", "c_out", "d_out"),
+     ("out_a", "out_b", "out_c", "out_d", "in_dim", "group_size"), ("a_out", "b_out", "c_out", "d_out"))
