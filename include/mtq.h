@@ -165,6 +165,17 @@ MTQ_API int mtq_qmv_batched(int dtype, int bits, uint32_t group_size, int n_mats
                             const void *const *scales, const void *const *biases, const void *x,
                             void *const *outs, const uint32_t *N, uint32_t K);
 
+/* RMSNorm fused into qmv: out[n] = sum_k w_hat[n,k] * (x[k] * norm_weight[k] * inv_rms),
+ * inv_rms = 1 / sqrt(mean(x^2) + eps_buf[0]); eps_buf is a DEVICE pointer to one f32, as in the
+ * reference. Replaces ffai_rms_norm_qgemv / _fast (4-bit) and ffai_rms_norm_qgemv_int8_fast
+ * (crates/metaltile-std/src/ffai/rms_norm_qgemv.rs:53-125, 128-456, 459-...). The normalised
+ * activation is an f32 value as in the reference; the f16 / bf16 kernels carry it as a rounded
+ * value plus a rounded remainder (16 significant bits). Rows the fused kernel does not take are
+ * normalised into a library-owned buffer first (allocated on first use, grown on demand). */
+MTQ_API int mtq_rms_norm_qmv(int dtype, int bits, uint32_t group_size, const void *x, const void *norm_weight,
+                             const void *w, const void *scales, const void *biases, void *out, const float *eps_buf,
+                             uint32_t N, uint32_t K);
+
 /* ---- the packed format's writer and reader ------------------------------ */
 
 /* Affine quantise: per group of `group_size` consecutive elements of w (T[n_elem]),

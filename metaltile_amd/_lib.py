@@ -59,6 +59,7 @@ SIGNATURES = {
     "mtq_gather_qmv_single": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "mtq_qmv_batched": (C.c_int, [C.c_int, C.c_int, _u32, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
                                   C.POINTER(C.c_void_p), _vp, C.POINTER(C.c_void_p), _u32p, _u32]),
+    "mtq_rms_norm_qmv": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32]),
     "mtq_affine_quantize": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, C.c_size_t]),
     "mtq_affine_dequantize": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, C.c_size_t]),
     "mtq_dispatch": (C.c_int, [C.c_char_p, C.c_int, _bufp, C.c_int, _u32p, C.c_int, _u32p, _u32p, _dblp]),

@@ -50,6 +50,8 @@ struct State {
     hipStream_t stream = nullptr;  // stream in use (own_stream or the caller's)
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     void* flush_buf = nullptr;
+    void* norm_buf = nullptr;     // normalised activation row (two-step norm + qmv)
+    size_t norm_bytes = 0;
     size_t flush_bytes = 0;
     hipDeviceProp_t prop;
     bool timed_armed = false;    // next typed launch attaches the events
@@ -149,6 +151,48 @@ static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s,
     return op_qmv(dtype, bits, G, w, s, b, x, out, M, N, K, lc);
 }
 
+// RMSNorm fused into qmv: inside the streaming kernel when the row fits it, else the
+// row is normalised into a library-owned buffer and an ordinary qmv follows.
+static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const void* norm_w, const void* w,
+                           const void* s, const void* b, void* out, const float* eps, uint32_t N, uint32_t K,
+                           const LaunchCtx& lc) {
+    int rc = check_common(dtype, bits, G, N, K);
+    if (rc) return rc;
+    if (!x || !norm_w || !w || !s || !b || !out || !eps) return fail(ERR_BAD_ARG, "null buffer");
+    QmvParams p;
+    p.dtype = dtype; p.bits = bits; p.group_size = G; p.w = w; p.scales = s; p.biases = b; p.x = x; p.out = out;
+    p.N = N; p.K = K;
+    rc = launch_qmv_norm(p, norm_w, eps, lc);
+    if (rc != ERR_UNSUPPORTED) return rc;
+    // scratch: the normalised row(s), then for 16-bit types the two partial outputs
+    const size_t sz = esize(dtype);
+    const uint32_t rows = dtype == DT_F32 ? 1u : 2u;
+    const size_t x_bytes = ((size_t)rows * K * sz + 255) & ~(size_t)255;
+    const size_t need = x_bytes + (rows == 2 ? (size_t)2 * N * sz : 0);
+    if (g.norm_bytes < need) {
+        if (g.norm_buf) {
+            MTQ_HIP(hipStreamSynchronize(g.stream));  // earlier launches may still read the old buffer
+            MTQ_HIP(hipFree(g.norm_buf));
+            g.norm_buf = nullptr;
+            g.norm_bytes = 0;
+        }
+        const size_t cap = need < 65536 ? 65536 : need;
+        MTQ_HIP(hipMalloc(&g.norm_buf, cap));
+        g.norm_bytes = cap;
+    }
+    LaunchCtx first = lc, mid = lc, last = lc;
+    first.stop = nullptr;
+    mid.start = mid.stop = nullptr;
+    last.start = nullptr;
+    rc = launch_rms_norm(dtype, x, norm_w, eps, g.norm_buf, K, first);
+    if (rc) return rc;
+    if (rows == 1) return op_qmv(dtype, bits, G, w, s, b, g.norm_buf, out, 1, N, K, last);
+    char* part = (char*)g.norm_buf + x_bytes;
+    rc = op_qmv(dtype, bits, G, w, s, b, g.norm_buf, part, 2, N, K, mid);
+    if (rc) return rc;
+    return launch_add_rows(dtype, part, part + (size_t)N * sz, out, N, last);
+}
+
 // Fused projections: one launch when the shape fits the streaming kernel, else one qmv per matrix.
 static int op_qmv_batched(int dtype, int bits, uint32_t G, int n, const void* const* w, const void* const* s,
                           const void* const* b, const void* x, void* const* outs, const uint32_t* N, uint32_t K,
@@ -198,7 +242,7 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
 // name-keyed dispatch table
 // ---------------------------------------------------------------------------
 
-enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4 };
+enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_NORMQ };
 
 struct KernelDesc {
     const char* name;
@@ -255,6 +299,9 @@ static const KernelDesc kTable[] = {
     {"ffai_batched_qkv_qgemv", F_BQKV, 4, 11, 5}, {"ffai_batched_qkv_qgemv_fast", F_BQKV, 4, 11, 5},
     // x, (w, scales, biases) x 4, a_out .. d_out | out_a .. out_d, in_dim, group_size
     {"ffai_batched_4_qgemv_fast", F_B4, 4, 17, 6},
+    // x, norm_weight, weight, scales, biases, output, eps_buf | in_dim, group_size
+    {"ffai_rms_norm_qgemv", F_NORMQ, 4, 7, 2}, {"ffai_rms_norm_qgemv_fast", F_NORMQ, 4, 7, 2},
+    {"ffai_rms_norm_qgemv_int8_fast", F_NORMQ, 8, 7, 2},
     // w, out, scales, biases | group_size
     {"mt_affine_quantize_int2", F_AQ, 2, 4, 1}, {"mt_affine_quantize_int3", F_AQ, 3, 4, 1},
     {"mt_affine_quantize_int4", F_AQ, 4, 4, 1}, {"mt_affine_quantize_int5", F_AQ, 5, 4, 1},
@@ -398,6 +445,20 @@ static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, in
             return op_gather(GATHER_INDICES, dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr,
                              bufs[3].ptr, (const uint32_t*)bufs[4].ptr, bufs[5].ptr, T, N, K, E, lc);
         }
+        case F_NORMQ: {
+            const uint32_t K = consts[0], G = consts[1];
+            const uint32_t N = (uint32_t)(bufs[5].bytes / sz);
+            if (K == 0 || N == 0) return fail(ERR_SHAPE, "in_dim and out_dim must be non-zero");
+            if (G == 0 || K % G) return fail(ERR_SHAPE, "group_size must divide in_dim");
+            MTQ_NEED(bufs[0], "x", (uint64_t)K * sz);
+            MTQ_NEED(bufs[1], "norm_weight", (uint64_t)K * sz);
+            MTQ_NEED(bufs[2], "weight", (uint64_t)N * K * bits / 8);
+            MTQ_NEED(bufs[3], "scales", (uint64_t)N * (K / G) * sz);
+            MTQ_NEED(bufs[4], "biases", (uint64_t)N * (K / G) * sz);
+            MTQ_NEED(bufs[6], "eps_buf", 4);
+            return op_rms_norm_qmv(dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, bufs[4].ptr,
+                                   bufs[5].ptr, (const float*)bufs[6].ptr, N, K, lc);
+        }
         case F_BQKV:
         case F_B4: {
             const int n = d.fam == F_BQKV ? 3 : 4;
@@ -497,6 +558,9 @@ int mtq_shutdown(void) {
     if (!g.ready) return MTQ_OK;
     (void)hipStreamSynchronize(g.stream);
     if (g.flush_buf) (void)hipFree(g.flush_buf);
+    if (g.norm_buf) (void)hipFree(g.norm_buf);
+    g.norm_buf = nullptr;
+    g.norm_bytes = 0;
     if (g.ev_start) (void)hipEventDestroy(g.ev_start);
     if (g.ev_stop) (void)hipEventDestroy(g.ev_stop);
     if (g.own_stream) (void)hipStreamDestroy(g.own_stream);
@@ -642,6 +706,13 @@ int mtq_qmv_batched(int dtype, int bits, uint32_t group_size, int n_mats, const 
     int rc = need_ready();
     if (rc) return rc;
     return op_qmv_batched(dtype, bits, group_size, n_mats, w, scales, biases, x, outs, N, K, make_ctx());
+}
+
+int mtq_rms_norm_qmv(int dtype, int bits, uint32_t group_size, const void* x, const void* norm_weight, const void* w,
+                     const void* scales, const void* biases, void* out, const float* eps_buf, uint32_t N, uint32_t K) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return op_rms_norm_qmv(dtype, bits, group_size, x, norm_weight, w, scales, biases, out, eps_buf, N, K, make_ctx());
 }
 
 int mtq_affine_quantize(int dtype, int bits, uint32_t group_size, const void* w, void* out,

@@ -104,6 +104,13 @@ int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc);
 // One launch for all matrices of `b` (p carries dtype, bits, group size, x, K; its
 // w / scales / biases / out / N are ignored). ERR_UNSUPPORTED when the shape does not
 // fit the streaming kernel: the caller then runs the matrices one by one.
+// RMSNorm of the activation row fused into the streaming qmv (eps: device f32).
+// ERR_UNSUPPORTED when the shape does not fit: the caller normalises into scratch first.
+int launch_qmv_norm(const QmvParams& p, const void* norm_w, const float* eps, const LaunchCtx& lc);
+// Standalone x'[k] = x[k] * norm_w[k] * rsqrt(mean(x^2) + eps): one f32 row, or for f16 / bf16
+// two rows of K elements (rounded value, rounded remainder).
+int launch_rms_norm(int dtype, const void* x, const void* norm_w, const float* eps, void* out, uint32_t K, const LaunchCtx& lc);
+int launch_add_rows(int dtype, const void* a, const void* b, void* out, uint32_t n, const LaunchCtx& lc);
 int launch_qmv_batched(const QmvParams& p, const QmvBatch& b, const LaunchCtx& lc);
 // Matrix-core streaming GEMV family for f16/bf16 (qmv_mfma.hip); same contract.
 int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc);

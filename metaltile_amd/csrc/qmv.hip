@@ -12,6 +12,9 @@ extern template int qmv_launch_dtype<DT_BF16>(QmvKArgs&, int, int, const QmvGeom
 extern template int qmv_stream_launch_dtype<DT_F32>(QmvSArgs&, int, int, const QmvSGeom&, const LaunchCtx&);
 extern template int qmv_stream_launch_dtype<DT_F16>(QmvSArgs&, int, int, const QmvSGeom&, const LaunchCtx&);
 extern template int qmv_stream_launch_dtype<DT_BF16>(QmvSArgs&, int, int, const QmvSGeom&, const LaunchCtx&);
+extern template int qmv_stream_norm_launch_dtype<DT_F32>(QmvSArgs&, int, const QmvSGeom&, const LaunchCtx&);
+extern template int qmv_stream_norm_launch_dtype<DT_F16>(QmvSArgs&, int, const QmvSGeom&, const LaunchCtx&);
+extern template int qmv_stream_norm_launch_dtype<DT_BF16>(QmvSArgs&, int, const QmvSGeom&, const LaunchCtx&);
 
 static bool is_pow2(uint32_t v) { return v && !(v & (v - 1)); }
 static uint32_t ilog2(uint32_t v) { uint32_t l = 0; while ((1u << l) < v) l++; return l; }
@@ -35,7 +38,8 @@ static int num_cus() {
 // and at least two batches are pipelined. Returns ERR_UNSUPPORTED when the
 // shape is better served by the one-shot kernel.
 static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint32_t tpb, uint32_t rows,
-                             const LaunchCtx& lc, const QmvBatch* batch = nullptr) {
+                             const LaunchCtx& lc, const QmvBatch* batch = nullptr,
+                             const void* norm_w = nullptr, const float* eps = nullptr) {
     const uint32_t G = p.group_size, gpr = p.K / G;
     if (C % 64 || gpr % 4 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
         return fail(ERR_UNSUPPORTED, "stream qmv: geometry");
@@ -74,6 +78,13 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
             // Measured on the 14336x4096 / 4096x14336 shapes: small workgroups do
             // best one batch deep (more, shorter-lived workgroups), wide ones two.
             if (nb == 1) score += tpb > 256 ? 0.15 : -0.05;
+            if (norm_w) {
+                // Every workgroup repeats the normalisation of the row, which costs about as
+                // much vector work as 8 weight rows per thread: take the longest workgroups
+                // that still leave 7 waves per CU (measured on 14336x4096, 4096x14336, 4096x4096).
+                if (d != 4) continue;
+                score = waste + (waves_per_cu >= 7.0 ? 1.0 / nb : 10.0 + (7.0 - waves_per_cu));
+            }
             if (score < best) { best = score; best_d = d; best_nb = nb; }
         }
     }
@@ -97,6 +108,8 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
     a.rows_per_wg = best_d * best_nb * rps;
     a.nb = best_nb;
     a.E = p.E;
+    a.norm_w = norm_w;
+    a.eps = eps;
     a.nmat = 0;
     if (batch) {
         a.nmat = (uint32_t)batch->n;
@@ -118,6 +131,15 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
     g.tpb = tpb;
     g.shmem = (size_t)a.rows_per_wg * gpr * 8 + (size_t)a.rows_per_wg * rows * a.wpr * 4;
     g.grid = dim3((p.N + a.rows_per_wg - 1) / a.rows_per_wg, batch ? (uint32_t)batch->n : 1u, 1);
+    if (norm_w) {
+        g.shmem += 16 * sizeof(float);  // one partial sum of squares per wave
+        switch (p.dtype) {
+            case DT_F32: return qmv_stream_norm_launch_dtype<DT_F32>(a, p.bits, g, lc);
+            case DT_F16: return qmv_stream_norm_launch_dtype<DT_F16>(a, p.bits, g, lc);
+            case DT_BF16: return qmv_stream_norm_launch_dtype<DT_BF16>(a, p.bits, g, lc);
+            default: return fail(ERR_BAD_ARG, "unknown dtype");
+        }
+    }
     switch (p.dtype) {
         case DT_F32: return qmv_stream_launch_dtype<DT_F32>(a, p.bits, p.gather, g, lc);
         case DT_F16: return qmv_stream_launch_dtype<DT_F16>(a, p.bits, p.gather, g, lc);
@@ -152,6 +174,24 @@ int launch_qmv_batched(const QmvParams& p0, const QmvBatch& b, const LaunchCtx& 
     uint32_t rps = 1;
     while (C * rps < 256 && C * rps * 2 <= 1024) rps *= 2;
     return launch_qmv_stream(p, C, rps, C * rps, 1, lc, &b);
+}
+
+int launch_qmv_norm(const QmvParams& p0, const void* norm_w, const float* eps, const LaunchCtx& lc) {
+    if (p0.bits != 4 && p0.bits != 8) return fail(ERR_UNSUPPORTED, "norm + qmv: bits must be 4 or 8");
+    QmvParams p = p0;
+    p.gather = GATHER_NONE;
+    p.M = 1;
+    const uint32_t cpc = 128u / (uint32_t)p.bits;
+    if (p.K == 0 || p.N == 0 || p.K % cpc) return fail(ERR_UNSUPPORTED, "norm + qmv: K*bits % 128 != 0");
+    const uint32_t G = p.group_size;
+    if (!is_pow2(G) || G * 2 < cpc || p.K % G) return fail(ERR_UNSUPPORTED, "norm + qmv: group size");
+    const uint32_t C = p.K / cpc;
+    if (C > 1024 || C % 64) return fail(ERR_UNSUPPORTED, "norm + qmv: row geometry");
+    if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)norm_w % 16)
+        return fail(ERR_UNSUPPORTED, "norm + qmv: w, x and norm_weight must be 16-byte aligned");
+    uint32_t rps = 1;
+    while (C * rps < 256 && C * rps * 2 <= 1024) rps *= 2;
+    return launch_qmv_stream(p, C, rps, C * rps, 1, lc, nullptr, norm_w, eps);
 }
 
 int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {

@@ -355,6 +355,9 @@ struct QmvSArgs {
     const void* ms[4];
     const void* mbias[4];
     void* mo[4];
+    // Fused RMSNorm (NORM kernels): per-element norm weights T[K] and a device f32 holding eps.
+    const void* norm_w;
+    const float* eps;
 };
 
 typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
@@ -382,8 +385,58 @@ __device__ __forceinline__ float wave_reduce4(float v0, float v1, float v2, floa
     return row16_allreduce(swap16_add(swap32_add(v0, v1), swap32_add(v2, v3)));
 }
 
-template <int DT, int BITS, int MB, int D, int MODE, int MAXT, int SBI>
+// One 16-byte vector of activations (4 f32 or 8 16-bit elements): sum of squares, and
+// in-place (x * w) * inv rounded to the element type.
+template <int DT> __device__ __forceinline__ float raw_sumsq(uint4 v) {
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        if constexpr (DT == DT_F32) {
+            const float f = __uint_as_float(u[j]);
+            s += f * f;
+        } else {
+            const float lo = DT == DT_BF16 ? bf16_bits_to_f32(u[j] & 0xFFFFu) : f16_bits_to_f32(u[j] & 0xFFFFu);
+            const float hi = DT == DT_BF16 ? bf16_bits_to_f32(u[j] >> 16) : f16_bits_to_f32(u[j] >> 16);
+            s += lo * lo;
+            s += hi * hi;
+        }
+    }
+    return s;
+}
+// (x * w) * inv of one vector, as the element-type value `hi` nearest to it and (16-bit
+// types) the rounded remainder `lo`: hi + lo carries 16 significant bits of the f32 product.
+template <int DT> __device__ __forceinline__ void raw_normed(uint4 xv, uint4 wv, float inv, uint4& hi, uint4& lo) {
+    const uint32_t x[4] = {xv.x, xv.y, xv.z, xv.w};
+    const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        if constexpr (DT == DT_F32) {
+            h[j] = __float_as_uint(__uint_as_float(x[j]) * __uint_as_float(w[j]) * inv);
+            l[j] = 0;
+        } else {
+            auto up = [](uint32_t b) { return DT == DT_BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b); };
+            const float v0 = up(x[j] & 0xFFFFu) * up(w[j] & 0xFFFFu) * inv;
+            const float v1 = up(x[j] >> 16) * up(w[j] >> 16) * inv;
+            const uint32_t h0 = f32_to_elem_bits<DT>(v0), h1 = f32_to_elem_bits<DT>(v1);
+            h[j] = h0 | (h1 << 16);
+            l[j] = (uint32_t)f32_to_elem_bits<DT>(v0 - up(h0)) | ((uint32_t)f32_to_elem_bits<DT>(v1 - up(h1)) << 16);
+        }
+    }
+    hi = make_uint4(h[0], h[1], h[2], h[3]);
+    lo = make_uint4(l[0], l[1], l[2], l[3]);
+}
+
+// NORM: the activation row is RMS-normalised on the fly, x'[k] = x[k] * norm_w[k] *
+// rsqrt(mean(x^2) + eps) (crates/metaltile-std/src/ffai/rms_norm_qgemv.rs:64-77,104-106),
+// every workgroup recomputing the row's sum of squares from the slice its threads hold.
+// The dot2 path takes 16-bit operands: for f16 / bf16 the f32 x' is carried as two rows,
+// its rounded value and the rounded remainder (MB = 2), whose dots are added.
+template <int DT, int BITS, int MB, int D, int MODE, int MAXT, int SBI, bool NORM = false>
 __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
+    static_assert(!NORM || (MB == (DT == DT_F32 ? 1 : 2) && MODE == GATHER_NONE), "the fused norm takes one plain activation row");
+    constexpr int MBR = NORM ? 1 : MB;  // activation rows as the caller sees them
     static_assert(D == 4 || D == 8, "ring depth");
     typedef XSlice<DT, BITS> XS;
     typedef typename Elem<DT>::type elem_t;
@@ -394,6 +447,7 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     float2* sb = (float2*)smem;                                   // [rows_per_wg][gpr]
     float* part = (float*)(sb + (size_t)a.rows_per_wg * a.gpr);   // [rows_per_wg][MB][wpr]
+    float* ssq_part = part + (size_t)a.rows_per_wg * MBR * a.wpr;  // [waves] (NORM only)
 
     const uint32_t tid = threadIdx.x;
     const uint32_t TPB = blockDim.x;
@@ -444,9 +498,17 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
     XS xs[MB];
     uint4 xraw[MB][XS::NRAW];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
+    for (int mb = 0; mb < MBR; mb++) {
         const uint32_t t = mb < (int)a.M ? mb : 0;
         xs[mb].load_raw(a.x, (size_t)t * a.K + k0, xraw[mb]);
+    }
+    uint4 nraw[NORM ? XS::NRAW : 1];
+    float eps = 0.f;
+    if constexpr (NORM) {
+        // issued ahead of the weight stream: loads return in order, so a late load of eps
+        // would wait for the whole first ring
+        eps = a.eps[0];
+        xs[0].load_raw(a.norm_w, k0, nraw);
     }
     MTQ_KEEP_LOAD_ORDER();
     u32x4 ring[D];
@@ -470,7 +532,29 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
             dst[1] = make_float4(sv[2], bv[2] - MAGIC * sv[2], sv[3], bv[3] - MAGIC * sv[3]);
         }
     }
+    if constexpr (NORM) {
+        // threads of the first row slot hold the whole activation row between them
+        float ssq = 0.f;
+        if (rsub == 0) {
+#pragma unroll
+            for (int i = 0; i < XS::NRAW; i++) ssq += raw_sumsq<DT>(xraw[0][i]);
+        }
+        ssq = seg_allreduce(ssq, 64);
+        if (lane == 0) ssq_part[tid >> 6] = ssq;
+    }
     __syncthreads();
+    if constexpr (NORM) {
+        float tot = 0.f;
+        for (uint32_t wv = 0; wv < (TPB >> 6); wv++) tot += ssq_part[wv];
+        const float inv = 1.0f / sqrtf(tot / (float)a.K + eps);
+#pragma unroll
+        for (int i = 0; i < XS::NRAW; i++) {
+            uint4 hi, lo;
+            raw_normed<DT>(xraw[0][i], nraw[i], inv, hi, lo);
+            xraw[0][i] = hi;
+            if constexpr (MB == 2) xraw[1][i] = lo;
+        }
+    }
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) xs[mb].prepare(xraw[mb]);
 
@@ -499,6 +583,7 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
                 v += p1.x * d23 + p1.y * xs[mb].xsum[1];
                 acc[d][mb] = v;
             }
+            if constexpr (NORM && MB == 2) acc[d][0] += acc[d][1];
             if constexpr (decltype(issue_next)::value) {
                 const uint32_t rn = min((j + D) * a.rps + rsub, rows_here - 1);
                 ring[d] = __builtin_nontemporal_load(wbase + (size_t)rn * a.C);
@@ -508,13 +593,13 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
 #pragma unroll
         for (int h = 0; h < D / 4; h++) {
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
+            for (int mb = 0; mb < MBR; mb++) {
                 const float tot = wave_reduce4(acc[4 * h + 0][mb], acc[4 * h + 1][mb], acc[4 * h + 2][mb],
                                                acc[4 * h + 3][mb]);
                 if ((lane & 15u) == 0) {
                     const uint32_t j = b * D + 4 * h + my_slot;
                     const uint32_t rl = j * a.rps + rsub;
-                    if (rl < rows_here) part[(rl * MB + mb) * a.wpr + wir] = tot;
+                    if (rl < rows_here) part[(rl * MBR + mb) * a.wpr + wir] = tot;
                 }
             }
         }
@@ -524,8 +609,8 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
     batch(a.nb - 1, std::false_type{});
 
     __syncthreads();
-    for (uint32_t o = tid; o < rows_here * MB; o += TPB) {
-        const uint32_t rl = o / MB, mb = o % MB;
+    for (uint32_t o = tid; o < rows_here * MBR; o += TPB) {
+        const uint32_t rl = o / MBR, mb = o % MBR;
         if (mb >= a.M) continue;
         float sum = 0.f;
         for (uint32_t wi = 0; wi < a.wpr; wi++) sum += part[o * a.wpr + wi];
@@ -611,6 +696,33 @@ static int qmv_stream_launch_sbi(QmvSArgs& a, const QmvSGeom& g, const LaunchCtx
     hipError_t e = launch_kernel(fn, g.grid, dim3(g.tpb), args, g.shmem, lc);
     if (e != hipSuccess) return hip_fail(e, "qmv stream kernel launch");
     return ERR_OK;
+}
+
+// Fused-RMSNorm instances: one activation row, 4- or 8-bit codes.
+template <int DT, int BITS, int D>
+static int qmv_stream_norm_launch_d(QmvSArgs& a, const QmvSGeom& g, const LaunchCtx& lc) {
+    constexpr int MBN = DT == DT_F32 ? 1 : 2;  // 16-bit types carry the normalised row as value + remainder
+    const void* fn;
+    switch (g.sbi) {
+        case 1: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 1, true>; break;
+        case 2: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 2, true>; break;
+        default: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 4, true>; break;
+    }
+    if (g.shmem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.shmem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
+    }
+    void* args[] = {&a};
+    hipError_t e = launch_kernel(fn, g.grid, dim3(g.tpb), args, g.shmem, lc);
+    if (e != hipSuccess) return hip_fail(e, "norm + qmv stream kernel launch");
+    return ERR_OK;
+}
+
+template <int DT> int qmv_stream_norm_launch_dtype(QmvSArgs& a, int bits, const QmvSGeom& g, const LaunchCtx& lc) {
+    if (g.mb != 1 || (g.d != 4 && g.d != 8)) return fail(ERR_UNSUPPORTED, "norm + qmv: no kernel instance for this geometry");
+    if (bits == 4) return g.d == 4 ? qmv_stream_norm_launch_d<DT, 4, 4>(a, g, lc) : qmv_stream_norm_launch_d<DT, 4, 8>(a, g, lc);
+    if (bits == 8) return g.d == 4 ? qmv_stream_norm_launch_d<DT, 8, 4>(a, g, lc) : qmv_stream_norm_launch_d<DT, 8, 8>(a, g, lc);
+    return fail(ERR_UNSUPPORTED, "norm + qmv: 4- or 8-bit codes");
 }
 
 template <int DT, int BITS, int MODE>

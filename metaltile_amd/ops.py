@@ -54,6 +54,13 @@ def qmv_batched(dtype, bits, group_size, ws, scales, biases, x, outs, Ns, K):
                                    (C.c_uint32 * n)(*Ns), K))
 
 
+def rms_norm_qmv(dtype, bits, group_size, x, norm_weight, w, scales, biases, out, eps_buf, N, K):
+    """out = qmv(w_hat, rms_norm(x) * norm_weight); eps_buf is a device buffer holding one f32."""
+    lib = _ensure_init()
+    _lib.check(lib.mtq_rms_norm_qmv(int(dtype), bits, group_size, _p(x), _p(norm_weight), _p(w), _p(scales), _p(biases),
+                                    _p(out), _p(eps_buf), N, K))
+
+
 def affine_quantize(dtype, bits, group_size, w, out, scales, biases, n_elem):
     """w: T[n_elem] -> out: packed u32 words, scales / biases: T[n_elem / group_size]."""
     lib = _ensure_init()

@@ -71,3 +71,5 @@ _add("ffai_batched_4_qgemv_fast", 4,
      ("x", "w_a", "scales_a", "biases_a", "w_b", "scales_b", "biases_b", "w_c", "scales_c", "biases_c",
       "w_d", "scales_d", "biases_d", "a_out", "b_out", "c_out", "d_out"),
      ("out_a", "out_b", "out_c", "out_d", "in_dim", "group_size"), ("a_out", "b_out", "c_out", "d_out"))
+for _n, _b in (("ffai_rms_norm_qgemv", 4), ("ffai_rms_norm_qgemv_fast", 4), ("ffai_rms_norm_qgemv_int8_fast", 8)):
+    _add(_n, _b, ("x", "norm_weight", "weight", "scales", "biases", "output", "eps_buf"), ("in_dim", "group_size"), ("output",))

@@ -24,6 +24,9 @@
  *   gather / expert   single expert == plain qmm, CSR == indices after
  *                     expansion, row permutation, expert e == slab e gemv.
  *   quantize          round trip within one step, constant group -> scale 1.
+ *   rms_norm_qgemv    numpy restatement (dequant matrix @ normalised row), unit norm
+ *                     weights with a constant row (inv_rms in closed form), scale
+ *                     invariance in x, eps -> large limit.
  *   stats             reference unit-test values (stats.rs:57-84).
  * No function here is "parity unpinned".
  */
@@ -404,6 +407,39 @@ MTQ_ORACLE_API void mtq_oracle_expert_indexed(const uint32_t *weight, const floa
         out[row] = dot_row_f32(weight + (expert * out_dim + row) * ppr,
                                scales + (expert * out_dim + row) * ng,
                                biases + (expert * out_dim + row) * ng, input, in_dim, 4, group_size);
+}
+
+/* Fused RMSNorm + quantized GEMV: normed[d] = x[d] * norm_weight[d] * inv_rms with
+ * inv_rms = 1 / sqrt(sum(x^2) / in_dim + eps), then the f32-sequential dequant dot.
+ * Reference: crates/metaltile-std/tests/rms_norm_qgemv_gpu_correctness.rs:59-91 (CPU form)
+ * and crates/metaltile-std/src/ffai/rms_norm_qgemv.rs:64-77,92-106 (kernel). `normed`
+ * (in_dim floats, may be NULL) receives the normalised activation. When out_f64 is not
+ * NULL the dot is also accumulated in f64 from the same f32 `normed` and f32 weights. */
+MTQ_ORACLE_API void mtq_oracle_rms_norm_qgemv(const uint32_t *weight, const float *scales, const float *biases,
+                                              const float *x, const float *norm_weight, size_t in_dim,
+                                              size_t group_size, size_t out_dim, uint32_t bits, float eps,
+                                              float *out, double *out_f64, float *normed) {
+    float ssq = 0.0f;
+    for (size_t d = 0; d < in_dim; d++) ssq += x[d] * x[d];
+    float inv_rms = 1.0f / sqrtf(ssq / (float)in_dim + eps);
+    size_t wpr = in_dim * bits / 32, ng = in_dim / group_size;
+    float *nx = (float *)malloc(in_dim * sizeof(float));
+    for (size_t d = 0; d < in_dim; d++) nx[d] = x[d] * norm_weight[d] * inv_rms;
+    if (normed) memcpy(normed, nx, in_dim * sizeof(float));
+    for (size_t row = 0; row < out_dim; row++) {
+        const uint32_t *rw = weight + row * wpr;
+        const float *rs = scales + row * ng, *rb = biases + row * ng;
+        float acc = 0.0f;
+        double acc64 = 0.0;
+        for (size_t d = 0; d < in_dim; d++) {
+            float w_real = (float)extract_code(rw, d, bits) * rs[d / group_size] + rb[d / group_size];
+            acc += w_real * nx[d];
+            acc64 += (double)w_real * (double)nx[d];
+        }
+        out[row] = acc;
+        if (out_f64) out_f64[row] = acc64;
+    }
+    free(nx);
 }
 
 /* ------------------------------------------------------------------ */

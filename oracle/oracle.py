@@ -174,6 +174,17 @@ def expert_indexed(weight, scales, biases, inp, expert, out_dim, in_dim, group_s
     return out
 
 
+def rms_norm_qgemv(w, scales, biases, x, norm_weight, in_dim, group_size, out_dim, bits, eps):
+    """Returns (out f32 sequential, out f64-accumulated, normalised activation f32)."""
+    w, scales, biases, x, norm_weight = _u32(w), _f32(scales), _f32(biases), _f32(x), _f32(norm_weight)
+    out = np.empty(out_dim, dtype=np.float32)
+    out64 = np.empty(out_dim, dtype=np.float64)
+    normed = np.empty(in_dim, dtype=np.float32)
+    lib().mtq_oracle_rms_norm_qgemv(_p(w), _p(scales), _p(biases), _p(x), _p(norm_weight), _sz(in_dim), _sz(group_size),
+                                    _sz(out_dim), C.c_uint32(bits), C.c_float(eps), _p(out), _p(out64), _p(normed))
+    return out, out64, normed
+
+
 def affine_quantize(v, group_size: int, bits: int, dt: int):
     v = _f32(v).ravel()
     ng = v.size // group_size

@@ -206,3 +206,43 @@ def test_bench_stats_reference_values(oracle):
     fast = oracle.bench_stats([250.0] * 4 + [120.0] * 6)
     assert slow["median_us"] - fast["median_us"] >= 100.0 and slow["min_us"] == fast["min_us"] == 120.0
     assert abs(st["mean_us"] - 4.0) < 1e-12 and abs(st["stddev_us"] - np.std([1, 2, 3, 4, 10])) < 1e-12
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_rms_norm_qgemv_against_numpy_and_closed_forms(oracle, bits):
+    """Fused RMSNorm + GEMV: (a) equals a library matmul of the independently unpacked weight
+    matrix with a numpy-normalised row; (b) a constant row c with unit norm weights has
+    inv_rms = 1/sqrt(c^2+eps) in closed form, so the output is qmv(w, ones) * c * inv_rms;
+    (c) scaling x by 4 leaves the output unchanged when eps = 0 (a dropped 1/in_dim or a
+    missing square root breaks this); (d) eps >> mean(x^2) gives out ~ qmv(x*nw)/sqrt(eps)."""
+    rng = np.random.default_rng(4242 + bits)
+    n, k, g = 12, 256, 64
+    codes, s, b, x = _rand_case(rng, n, k, bits, g, 1)
+    nw = (1.0 + 0.2 * rng.standard_normal(k)).astype(np.float32)
+    w = oracle.pack_codes(codes, bits)
+    eps = np.float32(1e-5)
+    out32, out64, normed = oracle.rms_norm_qgemv(w, s, b, x, nw, k, g, n, bits, eps)
+    # (a) numpy in f64 throughout
+    xd, nwd = x.astype(np.float64), nw.astype(np.float64)
+    inv = 1.0 / np.sqrt(np.mean(xd * xd) + float(eps))
+    wd = oracle.np_dequant(w, s, b, n, k, bits, g).astype(np.float64).reshape(n, k)
+    ref = wd @ (xd * nwd * inv)
+    assert np.max(np.abs(normed - xd * nwd * inv)) < 1e-5
+    assert np.max(np.abs(out64 - ref)) < 1e-4
+    assert np.max(np.abs(out32 - ref)) < 5e-4
+    assert np.max(np.abs(ref)) > 0.3
+    # (b) constant row, unit weights
+    c = np.float32(0.75)
+    xc, ones = np.full(k, c, dtype=np.float32), np.ones(k, dtype=np.float32)
+    o32, o64, _ = oracle.rms_norm_qgemv(w, s, b, xc, ones, k, g, n, bits, eps)
+    rowsum = oracle.qmm_f64(w, s, b, ones, 1, n, k, bits, g)
+    assert np.max(np.abs(o64 - rowsum * float(c) / np.sqrt(float(c) ** 2 + float(eps)))) < 1e-4
+    # (c) scale invariance at eps = 0
+    a32, a64, _ = oracle.rms_norm_qgemv(w, s, b, x, nw, k, g, n, bits, np.float32(0.0))
+    b32, b64, _ = oracle.rms_norm_qgemv(w, s, b, 4.0 * x, nw, k, g, n, bits, np.float32(0.0))
+    assert np.max(np.abs(a64 - b64)) < 1e-5
+    # (d) large eps
+    big = np.float32(1e6)
+    d32, d64, _ = oracle.rms_norm_qgemv(w, s, b, x, nw, k, g, n, bits, big)
+    plain = oracle.qmm_f64(w, s, b, x * nw, 1, n, k, bits, g)
+    assert np.max(np.abs(d64 * 1e3 - plain)) < 1e-4 * max(1.0, np.max(np.abs(plain)))
