@@ -176,6 +176,38 @@ MTQ_API int mtq_rms_norm_qmv(int dtype, int bits, uint32_t group_size, const voi
                              const void *w, const void *scales, const void *biases, void *out, const float *eps_buf,
                              uint32_t N, uint32_t K);
 
+/* ---- MoE routing around gather_qmv -------------------------------------------------- */
+
+/* Top-k experts per token row and their softmax weights. logits T[n_rows, n_experts] ->
+ * indices_out u32[n_rows, k], weights_out T[n_rows, k]. norm_topk_prob 1: softmax over the chosen
+ * k; 0: softmax over all experts, not renormalised. n_experts <= 1024, k <= 32. Ties go to the
+ * smaller index; NaN is never chosen. Replaces mt_moe_router_topk
+ * (crates/metaltile-std/src/ffai/moe.rs:65-199). */
+MTQ_API int mtq_moe_router_topk(int dtype, const void *router_logits, uint32_t *indices_out, void *weights_out,
+                                uint32_t n_rows, uint32_t n_experts, uint32_t k, uint32_t norm_topk_prob);
+
+/* Stable sort of the n_tokens * k (token, slot) entries of `indices` by expert, on the device:
+ * sort_token_idx u32[n*k] (source token of each sorted row: input of mtq_moe_permute),
+ * inv_perm u32[n_tokens, k] (sorted row of each entry: input of mtq_moe_unpermute) and
+ * expert_offsets u32[n_experts + 1] (CSR bounds: input of mtq_gather_qmv_csr). The reference has
+ * no kernel for this step: its callers sort on the host (crates/metaltile-std/src/ffai/moe.rs:
+ * 256-275 describes the two permutations). At most 32768 entries; expert ids >= n_experts are
+ * treated as n_experts - 1. */
+MTQ_API int mtq_moe_sort_by_expert(const uint32_t *indices, uint32_t n_tokens, uint32_t k, uint32_t n_experts,
+                                   uint32_t *sort_token_idx, uint32_t *inv_perm, uint32_t *expert_offsets);
+
+/* permuted[p, :] = tokens[sort_token_idx[p], :], p < n_permuted. A source index >= n_tokens gives
+ * a zero row. Replaces mt_moe_permute (crates/metaltile-std/src/ffai/moe.rs:282-302). */
+MTQ_API int mtq_moe_permute(int dtype, const void *tokens, const uint32_t *sort_token_idx, void *permuted,
+                            uint32_t n_tokens, uint32_t n_permuted, uint32_t hidden);
+
+/* out[t, h] = sum_j top_k_weights[t, j] * expert_outputs[inv_perm[t, j], h] (f32, j ascending).
+ * A position >= n_permuted contributes nothing. Replaces mt_moe_unpermute
+ * (crates/metaltile-std/src/ffai/moe.rs:225-251). */
+MTQ_API int mtq_moe_unpermute(int dtype, const void *expert_outputs, const uint32_t *inv_perm,
+                              const void *top_k_weights, void *out, uint32_t n_tokens, uint32_t n_permuted,
+                              uint32_t hidden, uint32_t k);
+
 /* ---- the packed format's writer and reader ------------------------------ */
 
 /* Affine quantise: per group of `group_size` consecutive elements of w (T[n_elem]),

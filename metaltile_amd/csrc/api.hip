@@ -242,7 +242,7 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
 // name-keyed dispatch table
 // ---------------------------------------------------------------------------
 
-enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_NORMQ };
+enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_NORMQ, F_ROUTER, F_PERMUTE, F_UNPERMUTE };
 
 struct KernelDesc {
     const char* name;
@@ -302,6 +302,12 @@ static const KernelDesc kTable[] = {
     // x, norm_weight, weight, scales, biases, output, eps_buf | in_dim, group_size
     {"ffai_rms_norm_qgemv", F_NORMQ, 4, 7, 2}, {"ffai_rms_norm_qgemv_fast", F_NORMQ, 4, 7, 2},
     {"ffai_rms_norm_qgemv_int8_fast", F_NORMQ, 8, 7, 2},
+    // router_logits, indices_out, weights_out | n_experts, k, norm_topk_prob
+    {"mt_moe_router_topk", F_ROUTER, 0, 3, 3},
+    // tokens, sort_token_idx, permuted | hidden
+    {"mt_moe_permute", F_PERMUTE, 0, 3, 1},
+    // expert_outputs, inv_perm, top_k_weights, out | hidden, k
+    {"mt_moe_unpermute", F_UNPERMUTE, 0, 4, 2},
     // w, out, scales, biases | group_size
     {"mt_affine_quantize_int2", F_AQ, 2, 4, 1}, {"mt_affine_quantize_int3", F_AQ, 3, 4, 1},
     {"mt_affine_quantize_int4", F_AQ, 4, 4, 1}, {"mt_affine_quantize_int5", F_AQ, 5, 4, 1},
@@ -444,6 +450,32 @@ static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, in
             MTQ_NEED(bufs[5], "out", (uint64_t)T * N * sz);
             return op_gather(GATHER_INDICES, dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr,
                              bufs[3].ptr, (const uint32_t*)bufs[4].ptr, bufs[5].ptr, T, N, K, E, lc);
+        }
+        case F_ROUTER: {
+            const uint32_t E = consts[0], k = consts[1];
+            if (E == 0 || k == 0) return fail(ERR_SHAPE, "n_experts and k must be non-zero");
+            const uint32_t rows = (uint32_t)(bufs[1].bytes / ((uint64_t)4 * k));
+            MTQ_NEED(bufs[0], "router_logits", (uint64_t)rows * E * sz);
+            MTQ_NEED(bufs[2], "weights_out", (uint64_t)rows * k * sz);
+            return launch_moe_router_topk(dtype, bufs[0].ptr, (uint32_t*)bufs[1].ptr, bufs[2].ptr, rows, E, k, consts[2], lc);
+        }
+        case F_PERMUTE: {
+            const uint32_t H = consts[0];
+            if (H == 0) return fail(ERR_SHAPE, "hidden must be non-zero");
+            const uint32_t n_perm = (uint32_t)(bufs[1].bytes / 4);
+            const uint32_t n_tok = (uint32_t)(bufs[0].bytes / ((uint64_t)H * sz));
+            MTQ_NEED(bufs[2], "permuted", (uint64_t)n_perm * H * sz);
+            return launch_moe_permute(dtype, bufs[0].ptr, (const uint32_t*)bufs[1].ptr, bufs[2].ptr, n_tok, n_perm, H, lc);
+        }
+        case F_UNPERMUTE: {
+            const uint32_t H = consts[0], k = consts[1];
+            if (H == 0 || k == 0) return fail(ERR_SHAPE, "hidden and k must be non-zero");
+            const uint32_t n_tok = (uint32_t)(bufs[3].bytes / ((uint64_t)H * sz));
+            const uint32_t n_perm = (uint32_t)(bufs[0].bytes / ((uint64_t)H * sz));
+            MTQ_NEED(bufs[1], "inv_perm", (uint64_t)n_tok * k * 4);
+            MTQ_NEED(bufs[2], "top_k_weights", (uint64_t)n_tok * k * sz);
+            return launch_moe_unpermute(dtype, bufs[0].ptr, (const uint32_t*)bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, n_tok,
+                                        n_perm, H, k, lc);
         }
         case F_NORMQ: {
             const uint32_t K = consts[0], G = consts[1];
@@ -713,6 +745,34 @@ int mtq_rms_norm_qmv(int dtype, int bits, uint32_t group_size, const void* x, co
     int rc = need_ready();
     if (rc) return rc;
     return op_rms_norm_qmv(dtype, bits, group_size, x, norm_weight, w, scales, biases, out, eps_buf, N, K, make_ctx());
+}
+
+int mtq_moe_router_topk(int dtype, const void* router_logits, uint32_t* indices_out, void* weights_out, uint32_t n_rows,
+                        uint32_t n_experts, uint32_t k, uint32_t norm_topk_prob) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return launch_moe_router_topk(dtype, router_logits, indices_out, weights_out, n_rows, n_experts, k, norm_topk_prob, make_ctx());
+}
+
+int mtq_moe_sort_by_expert(const uint32_t* indices, uint32_t n_tokens, uint32_t k, uint32_t n_experts,
+                           uint32_t* sort_token_idx, uint32_t* inv_perm, uint32_t* expert_offsets) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return launch_moe_sort(indices, n_tokens, k, n_experts, sort_token_idx, inv_perm, expert_offsets, make_ctx());
+}
+
+int mtq_moe_permute(int dtype, const void* tokens, const uint32_t* sort_token_idx, void* permuted, uint32_t n_tokens,
+                    uint32_t n_permuted, uint32_t hidden) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return launch_moe_permute(dtype, tokens, sort_token_idx, permuted, n_tokens, n_permuted, hidden, make_ctx());
+}
+
+int mtq_moe_unpermute(int dtype, const void* expert_outputs, const uint32_t* inv_perm, const void* top_k_weights, void* out,
+                      uint32_t n_tokens, uint32_t n_permuted, uint32_t hidden, uint32_t k) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return launch_moe_unpermute(dtype, expert_outputs, inv_perm, top_k_weights, out, n_tokens, n_permuted, hidden, k, make_ctx());
 }
 
 int mtq_affine_quantize(int dtype, int bits, uint32_t group_size, const void* w, void* out,

@@ -110,6 +110,15 @@ int launch_qmv_norm(const QmvParams& p, const void* norm_w, const float* eps, co
 // Standalone x'[k] = x[k] * norm_w[k] * rsqrt(mean(x^2) + eps): one f32 row, or for f16 / bf16
 // two rows of K elements (rounded value, rounded remainder).
 int launch_rms_norm(int dtype, const void* x, const void* norm_w, const float* eps, void* out, uint32_t K, const LaunchCtx& lc);
+// MoE routing (moe.hip)
+int launch_moe_router_topk(int dtype, const void* logits, uint32_t* indices, void* weights, uint32_t n_rows,
+                           uint32_t n_experts, uint32_t k, uint32_t norm_topk_prob, const LaunchCtx& lc);
+int launch_moe_sort(const uint32_t* indices, uint32_t n_tokens, uint32_t k, uint32_t n_experts, uint32_t* sort_token_idx,
+                    uint32_t* inv_perm, uint32_t* expert_offsets, const LaunchCtx& lc);
+int launch_moe_permute(int dtype, const void* tokens, const uint32_t* sort_token_idx, void* permuted, uint32_t n_tokens,
+                       uint32_t n_permuted, uint32_t hidden, const LaunchCtx& lc);
+int launch_moe_unpermute(int dtype, const void* expert_outputs, const uint32_t* inv_perm, const void* weights, void* out,
+                         uint32_t n_tokens, uint32_t n_permuted, uint32_t hidden, uint32_t k, const LaunchCtx& lc);
 int launch_add_rows(int dtype, const void* a, const void* b, void* out, uint32_t n, const LaunchCtx& lc);
 int launch_qmv_batched(const QmvParams& p, const QmvBatch& b, const LaunchCtx& lc);
 // Matrix-core streaming GEMV family for f16/bf16 (qmv_mfma.hip); same contract.

@@ -61,6 +61,29 @@ def rms_norm_qmv(dtype, bits, group_size, x, norm_weight, w, scales, biases, out
                                     _p(out), _p(eps_buf), N, K))
 
 
+def moe_router_topk(dtype, router_logits, indices_out, weights_out, n_rows, n_experts, k, norm_topk_prob=1):
+    lib = _ensure_init()
+    _lib.check(lib.mtq_moe_router_topk(int(dtype), _p(router_logits), _p(indices_out), _p(weights_out), n_rows, n_experts, k,
+                                       norm_topk_prob))
+
+
+def moe_sort_by_expert(indices, n_tokens, k, n_experts, sort_token_idx, inv_perm, expert_offsets):
+    lib = _ensure_init()
+    _lib.check(lib.mtq_moe_sort_by_expert(_p(indices), n_tokens, k, n_experts, _p(sort_token_idx), _p(inv_perm),
+                                          _p(expert_offsets)))
+
+
+def moe_permute(dtype, tokens, sort_token_idx, permuted, n_tokens, n_permuted, hidden):
+    lib = _ensure_init()
+    _lib.check(lib.mtq_moe_permute(int(dtype), _p(tokens), _p(sort_token_idx), _p(permuted), n_tokens, n_permuted, hidden))
+
+
+def moe_unpermute(dtype, expert_outputs, inv_perm, top_k_weights, out, n_tokens, n_permuted, hidden, k):
+    lib = _ensure_init()
+    _lib.check(lib.mtq_moe_unpermute(int(dtype), _p(expert_outputs), _p(inv_perm), _p(top_k_weights), _p(out), n_tokens,
+                                     n_permuted, hidden, k))
+
+
 def affine_quantize(dtype, bits, group_size, w, out, scales, biases, n_elem):
     """w: T[n_elem] -> out: packed u32 words, scales / biases: T[n_elem / group_size]."""
     lib = _ensure_init()

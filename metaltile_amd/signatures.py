@@ -73,3 +73,7 @@ _add("ffai_batched_4_qgemv_fast", 4,
      ("out_a", "out_b", "out_c", "out_d", "in_dim", "group_size"), ("a_out", "b_out", "c_out", "d_out"))
 for _n, _b in (("ffai_rms_norm_qgemv", 4), ("ffai_rms_norm_qgemv_fast", 4), ("ffai_rms_norm_qgemv_int8_fast", 8)):
     _add(_n, _b, ("x", "norm_weight", "weight", "scales", "biases", "output", "eps_buf"), ("in_dim", "group_size"), ("output",))
+_add("mt_moe_router_topk", 0, ("router_logits", "indices_out", "weights_out"), ("n_experts", "k", "norm_topk_prob"),
+     ("indices_out", "weights_out"))
+_add("mt_moe_permute", 0, ("tokens", "sort_token_idx", "permuted"), ("hidden",), ("permuted",))
+_add("mt_moe_unpermute", 0, ("expert_outputs", "inv_perm", "top_k_weights", "out"), ("hidden", "k"), ("out",))

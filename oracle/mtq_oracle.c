@@ -27,6 +27,9 @@
  *   rms_norm_qgemv    numpy restatement (dequant matrix @ normalised row), unit norm
  *                     weights with a constant row (inv_rms in closed form), scale
  *                     invariance in x, eps -> large limit.
+ *   moe routing       numpy stable argsort + library softmax, the reference tests' tie-break,
+ *                     k = 1 and NaN/Inf cases; unpermute against a numpy einsum; permute and
+ *                     the expert sort are numpy one-liners (take, stable argsort) in oracle.py.
  *   stats             reference unit-test values (stats.rs:57-84).
  * No function here is "parity unpinned".
  */
@@ -440,6 +443,62 @@ MTQ_ORACLE_API void mtq_oracle_rms_norm_qgemv(const uint32_t *weight, const floa
         if (out_f64) out_f64[row] = acc64;
     }
     free(nx);
+}
+
+/* ------------------------------------------------------------------ */
+/* MoE routing around the gathered matmul                              */
+/* ------------------------------------------------------------------ */
+
+/* Top-k experts per token row and their softmax weights.
+ * k passes of argmax with strict '>' from (-inf, index 0), already-chosen experts masked,
+ * so ties go to the smaller index and NaN never wins; weight = exp(v - max_all) / divisor
+ * with divisor = sum over the chosen k (norm_topk_prob = 1) or over all experts (0).
+ * Reference: crates/metaltile-std/src/ffai/moe.rs:65-199 (kernel) and
+ * crates/metaltile-std/tests/moe_gpu_correctness.rs:55-93 (its CPU form). */
+MTQ_ORACLE_API void mtq_oracle_moe_router_topk(const float *logits, size_t n_rows, size_t n_experts, size_t k,
+                                               int norm_topk_prob, uint32_t *indices, float *weights) {
+    for (size_t row = 0; row < n_rows; row++) {
+        const float *z = logits + row * n_experts;
+        float max_all = -INFINITY;
+        for (size_t j = 0; j < n_experts; j++)
+            if (z[j] > max_all) max_all = z[j];
+        float sum_all = 0.0f;
+        for (size_t j = 0; j < n_experts; j++) sum_all += expf(z[j] - max_all);
+        uint32_t *idx = indices + row * k;
+        float vals[32];
+        for (size_t it = 0; it < k; it++) {
+            float best = -INFINITY;
+            uint32_t bi = 0;
+            for (size_t j = 0; j < n_experts; j++) {
+                int taken = 0;
+                for (size_t p = 0; p < it; p++) taken |= idx[p] == (uint32_t)j;
+                if (taken) continue;
+                if (z[j] > best) { best = z[j]; bi = (uint32_t)j; }
+            }
+            idx[it] = bi;
+            vals[it] = best;
+        }
+        float e[32], sum_chosen = 0.0f;
+        for (size_t j = 0; j < k; j++) { e[j] = expf(vals[j] - max_all); sum_chosen += e[j]; }
+        float divisor = norm_topk_prob == 1 ? sum_chosen : sum_all;
+        for (size_t j = 0; j < k; j++) weights[row * k + j] = e[j] / divisor;
+    }
+}
+
+/* out[token, h] = sum_j w[token, j] * expert_outputs[inv_perm[token, j], h], f32, j ascending,
+ * product and sum rounded separately.
+ * Reference: crates/metaltile-std/src/ffai/moe.rs:225-251. */
+MTQ_ORACLE_API void mtq_oracle_moe_unpermute(const float *expert_outputs, const uint32_t *inv_perm, const float *w,
+                                             size_t n_tokens, size_t hidden, size_t k, float *out) {
+    for (size_t t = 0; t < n_tokens; t++)
+        for (size_t h = 0; h < hidden; h++) {
+            float acc = 0.0f;
+            for (size_t j = 0; j < k; j++) {
+                float prod = w[t * k + j] * expert_outputs[(size_t)inv_perm[t * k + j] * hidden + h];
+                acc = acc + prod;
+            }
+            out[t * hidden + h] = acc;
+        }
 }
 
 /* ------------------------------------------------------------------ */

@@ -185,6 +185,40 @@ def rms_norm_qgemv(w, scales, biases, x, norm_weight, in_dim, group_size, out_di
     return out, out64, normed
 
 
+def moe_router_topk(logits, n_rows: int, n_experts: int, k: int, norm_topk_prob: int = 1):
+    logits = _f32(logits)
+    idx = np.empty(n_rows * k, dtype=np.uint32)
+    w = np.empty(n_rows * k, dtype=np.float32)
+    lib().mtq_oracle_moe_router_topk(_p(logits), _sz(n_rows), _sz(n_experts), _sz(k), C.c_int(norm_topk_prob), _p(idx), _p(w))
+    return idx, w
+
+
+def moe_unpermute(expert_outputs, inv_perm, weights, n_tokens: int, hidden: int, k: int) -> np.ndarray:
+    eo, ip, w = _f32(expert_outputs), _u32(inv_perm), _f32(weights)
+    out = np.empty(n_tokens * hidden, dtype=np.float32)
+    lib().mtq_oracle_moe_unpermute(_p(eo), _p(ip), _p(w), _sz(n_tokens), _sz(hidden), _sz(k), _p(out))
+    return out
+
+
+def moe_permute(tokens, sort_token_idx, hidden: int) -> np.ndarray:
+    """permuted[p, :] = tokens[sort_token_idx[p], :] (crates/metaltile-std/src/ffai/moe.rs:282-302); any dtype."""
+    t = np.asarray(tokens).reshape(-1, hidden)
+    return t[np.asarray(sort_token_idx, dtype=np.int64)].reshape(-1)
+
+
+def moe_sort_by_expert(indices, n_tokens: int, k: int, n_experts: int):
+    """The caller-side sort the reference describes (crates/metaltile-std/src/ffai/moe.rs:256-275):
+    a stable argsort of the flattened (token * k + slot) expert ids. Returns sort_token_idx [n*k]
+    (source token of each sorted position), inv_perm [n, k] (sorted position of each (token, slot))
+    and expert_offsets [E + 1] (CSR bounds of each expert's rows)."""
+    flat = np.asarray(indices, dtype=np.int64).reshape(-1)
+    order = np.argsort(flat, kind="stable")
+    inv = np.empty_like(order)
+    inv[order] = np.arange(order.size)
+    offsets = np.concatenate([[0], np.cumsum(np.bincount(flat, minlength=n_experts))])
+    return (order // k).astype(np.uint32), inv.astype(np.uint32), offsets.astype(np.uint32)
+
+
 def affine_quantize(v, group_size: int, bits: int, dt: int):
     v = _f32(v).ravel()
     ng = v.size // group_size

@@ -246,3 +246,82 @@ def test_rms_norm_qgemv_against_numpy_and_closed_forms(oracle, bits):
     d32, d64, _ = oracle.rms_norm_qgemv(w, s, b, x, nw, k, g, n, bits, big)
     plain = oracle.qmm_f64(w, s, b, x * nw, 1, n, k, bits, g)
     assert np.max(np.abs(d64 * 1e3 - plain)) < 1e-4 * max(1.0, np.max(np.abs(plain)))
+
+
+def _np_topk(logits, k, mode):
+    """Independent restatement: stable descending argsort + library softmax."""
+    from scipy.special import softmax
+    z = np.asarray(logits, dtype=np.float64)
+    order = np.argsort(-z, axis=1, kind="stable")[:, :k]
+    zs = np.take_along_axis(z, order, axis=1)
+    w = softmax(zs, axis=1) if mode == 1 else np.take_along_axis(softmax(z, axis=1), order, axis=1)
+    return order.astype(np.uint32), w
+
+
+@pytest.mark.parametrize("mode", [1, 0])
+def test_moe_router_topk_against_numpy(oracle, mode):
+    # the reference test's logits (moe_gpu_correctness.rs:103-106) and a random draw
+    n_rows, n_exp, k = 8, 64, 4
+    i = np.arange(n_rows * n_exp, dtype=np.float32)
+    logits = np.fmod(i * np.float32(0.13), np.float32(7.0)) - np.float32(3.5) + i * np.float32(0.001)
+    for lg, (r, e, kk) in ((logits, (n_rows, n_exp, k)),
+                           (np.random.default_rng(3).standard_normal(16 * 128).astype(np.float32), (16, 128, 8))):
+        idx, w = oracle.moe_router_topk(lg, r, e, kk, mode)
+        ridx, rw = _np_topk(lg.reshape(r, e), kk, mode)
+        assert np.array_equal(idx.reshape(r, kk), ridx)
+        assert np.max(np.abs(w.reshape(r, kk) - rw)) < 1e-6
+        if mode == 1:
+            assert np.allclose(w.reshape(r, kk).sum(axis=1), 1.0, atol=1e-6)
+        else:
+            assert np.all(w.reshape(r, kk).sum(axis=1) < 1.0)
+
+
+def test_moe_router_topk_reference_edge_cases(oracle):
+    # tie -> smaller index first (moe_gpu_correctness.rs:316-335)
+    z = np.zeros(8, dtype=np.float32)
+    z[2] = z[5] = 3.0
+    idx, _ = oracle.moe_router_topk(z, 1, 8, 2)
+    assert idx.tolist() == [2, 5]
+    # k = 1 -> weight exactly 1 (:288-313)
+    idx, w = oracle.moe_router_topk(np.arange(32, dtype=np.float32), 1, 32, 1)
+    assert idx.tolist() == [31] and w.tolist() == [1.0]
+    # NaN never chosen, +Inf first, -Inf not chosen, no duplicates (:524-597)
+    n_exp, k = 16, 4
+    lg = np.tile(np.arange(n_exp, dtype=np.float32) * np.float32(0.1), 4)
+    lg[5] = np.nan
+    lg[n_exp + 7] = np.inf
+    lg[2 * n_exp + 3] = -np.inf
+    lg[3 * n_exp + 2] = np.nan
+    lg[3 * n_exp + 11] = np.inf
+    idx, _ = oracle.moe_router_topk(lg, 4, n_exp, k)
+    idx = idx.reshape(4, k)
+    assert all(len(set(r.tolist())) == k for r in idx)
+    assert idx[1, 0] == 7 and idx[3, 0] == 11
+    assert 3 not in idx[2] and 5 not in idx[0] and 2 not in idx[3]
+
+
+def test_moe_unpermute_permute_sort(oracle):
+    rng = np.random.default_rng(9)
+    T, k, E, H = 12, 3, 7, 40
+    logits = rng.standard_normal(T * E).astype(np.float32)
+    idx, w = oracle.moe_router_topk(logits, T, E, k)
+    sti, inv, offs = oracle.moe_sort_by_expert(idx, T, k, E)
+    flat = idx.astype(np.int64)
+    # sorted positions are grouped by expert in CSR order, stably
+    assert np.all(np.diff(flat[np.argsort(inv)]) >= 0)
+    assert offs[0] == 0 and offs[-1] == T * k
+    for e in range(E):
+        seg = np.argsort(inv)[offs[e]:offs[e + 1]]
+        assert np.all(flat[seg] == e) and np.all(np.diff(seg) > 0)
+    assert np.array_equal(sti, (np.argsort(inv) // k).astype(np.uint32))
+    tokens = rng.standard_normal(T * H).astype(np.float32)
+    perm = oracle.moe_permute(tokens, sti, H).reshape(T * k, H)
+    for t in range(T):
+        for j in range(k):
+            assert np.array_equal(perm[inv[t * k + j]], tokens.reshape(T, H)[t])
+    # unpermute of the permuted rows gives sum_j w_j * token = token (weights sum to 1)
+    out = oracle.moe_unpermute(perm.reshape(-1), inv, w, T, H, k).reshape(T, H)
+    ein = np.einsum("tj,tjh->th", w.reshape(T, k).astype(np.float64),
+                    perm[inv.reshape(T, k)].astype(np.float64))
+    assert np.max(np.abs(out - ein)) < 1e-6
+    assert np.max(np.abs(out - tokens.reshape(T, H))) < 1e-5
