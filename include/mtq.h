@@ -208,6 +208,17 @@ MTQ_API int mtq_moe_unpermute(int dtype, const void *expert_outputs, const uint3
                               const void *top_k_weights, void *out, uint32_t n_tokens, uint32_t n_permuted,
                               uint32_t hidden, uint32_t k);
 
+/* Fused MoE decode step for one token: out[i] = sum_k slot_weights[k] * sum_d w_hat[expert_indices[k]][i][d] *
+ * silu(gate_k[d]) * up_k[d], 4-bit weights stacked [n_experts, out_dim, in_dim/8]. gates / ups: host arrays of
+ * n_slots (1..8) device pointers to T[in_dim]; expert_indices u32[n_slots] and slot_weights T[n_slots] on the
+ * device (the outputs of the router). in_dim % 32 == 0, in_dim <= 4096, group_size a power of two >= 32.
+ * Replaces ffai_moe_down_swiglu_accum_int4_chain8 (8 slots;
+ * crates/metaltile-std/src/ffai/moe_down_swiglu_accum.rs:146-282). */
+MTQ_API int mtq_moe_down_swiglu_accum(int dtype, uint32_t group_size, uint32_t n_slots, const void *const *gates,
+                                      const void *const *ups, const uint32_t *expert_indices, const void *slot_weights,
+                                      const void *w, const void *scales, const void *biases, void *out, uint32_t in_dim,
+                                      uint32_t out_dim, uint32_t n_experts);
+
 /* ---- the packed format's writer and reader ------------------------------ */
 
 /* Affine quantise: per group of `group_size` consecutive elements of w (T[n_elem]),

@@ -64,6 +64,8 @@ SIGNATURES = {
     "mtq_moe_sort_by_expert": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp]),
     "mtq_moe_permute": (C.c_int, [C.c_int, _vp, _vp, _vp, _u32, _u32, _u32]),
     "mtq_moe_unpermute": (C.c_int, [C.c_int, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32]),
+    "mtq_moe_down_swiglu_accum": (C.c_int, [C.c_int, _u32, _u32, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), _vp, _vp, _vp,
+                                            _vp, _vp, _vp, _u32, _u32, _u32]),
     "mtq_affine_quantize": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, C.c_size_t]),
     "mtq_affine_dequantize": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, C.c_size_t]),
     "mtq_dispatch": (C.c_int, [C.c_char_p, C.c_int, _bufp, C.c_int, _u32p, C.c_int, _u32p, _u32p, _dblp]),

@@ -242,7 +242,7 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
 // name-keyed dispatch table
 // ---------------------------------------------------------------------------
 
-enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_NORMQ, F_ROUTER, F_PERMUTE, F_UNPERMUTE };
+enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_NORMQ, F_ROUTER, F_PERMUTE, F_UNPERMUTE, F_MOEDOWN };
 
 struct KernelDesc {
     const char* name;
@@ -308,6 +308,9 @@ static const KernelDesc kTable[] = {
     {"mt_moe_permute", F_PERMUTE, 0, 3, 1},
     // expert_outputs, inv_perm, top_k_weights, out | hidden, k
     {"mt_moe_unpermute", F_UNPERMUTE, 0, 4, 2},
+    // gate_0, up_0, ..., gate_7, up_7, expert_indices, slot_weights, weights_stacked, scales_stacked, biases_stacked,
+    // output | in_dim, out_dim, group_size
+    {"ffai_moe_down_swiglu_accum_int4_chain8", F_MOEDOWN, 4, 22, 3},
     // w, out, scales, biases | group_size
     {"mt_affine_quantize_int2", F_AQ, 2, 4, 1}, {"mt_affine_quantize_int3", F_AQ, 3, 4, 1},
     {"mt_affine_quantize_int4", F_AQ, 4, 4, 1}, {"mt_affine_quantize_int5", F_AQ, 5, 4, 1},
@@ -476,6 +479,28 @@ static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, in
             MTQ_NEED(bufs[2], "top_k_weights", (uint64_t)n_tok * k * sz);
             return launch_moe_unpermute(dtype, bufs[0].ptr, (const uint32_t*)bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, n_tok,
                                         n_perm, H, k, lc);
+        }
+        case F_MOEDOWN: {
+            const uint32_t K = consts[0], N = consts[1], G = consts[2];
+            if (K == 0 || N == 0) return fail(ERR_SHAPE, "in_dim and out_dim must be non-zero");
+            if (G == 0 || K % G) return fail(ERR_SHAPE, "group_size must divide in_dim");
+            const void *gates[8], *ups[8];
+            for (int k = 0; k < 8; k++) {
+                MTQ_NEED(bufs[2 * k], "gate_*", (uint64_t)K * sz);
+                MTQ_NEED(bufs[2 * k + 1], "up_*", (uint64_t)K * sz);
+                gates[k] = bufs[2 * k].ptr;
+                ups[k] = bufs[2 * k + 1].ptr;
+            }
+            MTQ_NEED(bufs[16], "expert_indices", 32);
+            MTQ_NEED(bufs[17], "slot_weights", 8 * sz);
+            const uint64_t slab = (uint64_t)N * K / 2;
+            const uint32_t E = (uint32_t)(bufs[18].bytes / slab);
+            if (E == 0) return fail(ERR_BUFFER_SIZE, "buffer 'weights_stacked' holds less than one expert");
+            MTQ_NEED(bufs[19], "scales_stacked", (uint64_t)E * N * (K / G) * sz);
+            MTQ_NEED(bufs[20], "biases_stacked", (uint64_t)E * N * (K / G) * sz);
+            MTQ_NEED(bufs[21], "output", (uint64_t)N * sz);
+            return launch_moe_down_swiglu(dtype, G, 8, gates, ups, (const uint32_t*)bufs[16].ptr, bufs[17].ptr, bufs[18].ptr,
+                                          bufs[19].ptr, bufs[20].ptr, bufs[21].ptr, K, N, E, lc);
         }
         case F_NORMQ: {
             const uint32_t K = consts[0], G = consts[1];
@@ -773,6 +798,15 @@ int mtq_moe_unpermute(int dtype, const void* expert_outputs, const uint32_t* inv
     int rc = need_ready();
     if (rc) return rc;
     return launch_moe_unpermute(dtype, expert_outputs, inv_perm, top_k_weights, out, n_tokens, n_permuted, hidden, k, make_ctx());
+}
+
+int mtq_moe_down_swiglu_accum(int dtype, uint32_t group_size, uint32_t n_slots, const void* const* gates, const void* const* ups,
+                              const uint32_t* expert_indices, const void* slot_weights, const void* w, const void* scales,
+                              const void* biases, void* out, uint32_t in_dim, uint32_t out_dim, uint32_t n_experts) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return launch_moe_down_swiglu(dtype, group_size, n_slots, gates, ups, expert_indices, slot_weights, w, scales, biases, out,
+                                  in_dim, out_dim, n_experts, make_ctx());
 }
 
 int mtq_affine_quantize(int dtype, int bits, uint32_t group_size, const void* w, void* out,

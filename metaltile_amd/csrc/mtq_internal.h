@@ -119,6 +119,9 @@ int launch_moe_permute(int dtype, const void* tokens, const uint32_t* sort_token
                        uint32_t n_permuted, uint32_t hidden, const LaunchCtx& lc);
 int launch_moe_unpermute(int dtype, const void* expert_outputs, const uint32_t* inv_perm, const void* weights, void* out,
                          uint32_t n_tokens, uint32_t n_permuted, uint32_t hidden, uint32_t k, const LaunchCtx& lc);
+int launch_moe_down_swiglu(int dtype, uint32_t group_size, uint32_t n_slots, const void* const* gates, const void* const* ups,
+                           const uint32_t* experts, const void* slot_w, const void* w, const void* scales, const void* biases,
+                           void* out, uint32_t in_dim, uint32_t out_dim, uint32_t n_experts, const LaunchCtx& lc);
 int launch_add_rows(int dtype, const void* a, const void* b, void* out, uint32_t n, const LaunchCtx& lc);
 int launch_qmv_batched(const QmvParams& p, const QmvBatch& b, const LaunchCtx& lc);
 // Matrix-core streaming GEMV family for f16/bf16 (qmv_mfma.hip); same contract.

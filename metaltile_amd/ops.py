@@ -84,6 +84,16 @@ def moe_unpermute(dtype, expert_outputs, inv_perm, top_k_weights, out, n_tokens,
                                      n_permuted, hidden, k))
 
 
+def moe_down_swiglu_accum(dtype, group_size, gates, ups, expert_indices, slot_weights, w, scales, biases, out, in_dim, out_dim,
+                          n_experts):
+    """gates / ups: lists of 1..8 device buffers T[in_dim] (one per routed slot)."""
+    lib = _ensure_init()
+    n = len(gates)
+    arr = lambda bufs: (C.c_void_p * n)(*[_p(b) for b in bufs])
+    _lib.check(lib.mtq_moe_down_swiglu_accum(int(dtype), group_size, n, arr(gates), arr(ups), _p(expert_indices),
+                                             _p(slot_weights), _p(w), _p(scales), _p(biases), _p(out), in_dim, out_dim, n_experts))
+
+
 def affine_quantize(dtype, bits, group_size, w, out, scales, biases, n_elem):
     """w: T[n_elem] -> out: packed u32 words, scales / biases: T[n_elem / group_size]."""
     lib = _ensure_init()

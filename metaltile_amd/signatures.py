@@ -77,3 +77,7 @@ _add("mt_moe_router_topk", 0, ("router_logits", "indices_out", "weights_out"), (
      ("indices_out", "weights_out"))
 _add("mt_moe_permute", 0, ("tokens", "sort_token_idx", "permuted"), ("hidden",), ("permuted",))
 _add("mt_moe_unpermute", 0, ("expert_outputs", "inv_perm", "top_k_weights", "out"), ("hidden", "k"), ("out",))
+_add("ffai_moe_down_swiglu_accum_int4_chain8", 4,
+     tuple(n for k in range(8) for n in (f"gate_{k}", f"up_{k}")) + ("expert_indices", "slot_weights", "weights_stacked",
+                                                                      "scales_stacked", "biases_stacked", "output"),
+     ("in_dim", "out_dim", "group_size"), ("output",))

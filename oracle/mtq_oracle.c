@@ -30,6 +30,8 @@
  *   moe routing       numpy stable argsort + library softmax, the reference tests' tie-break,
  *                     k = 1 and NaN/Inf cases; unpermute against a numpy einsum; permute and
  *                     the expert sort are numpy one-liners (take, stable argsort) in oracle.py.
+ *   moe_down_swiglu   numpy silu + the (pinned) expert-indexed GEMV + numpy slot sum; one slot with
+ *                     weight 1 == expert-indexed GEMV of the swiglu row; zero gates -> zero output.
  *   stats             reference unit-test values (stats.rs:57-84).
  * No function here is "parity unpinned".
  */
@@ -499,6 +501,43 @@ MTQ_ORACLE_API void mtq_oracle_moe_unpermute(const float *expert_outputs, const 
             }
             out[t * hidden + h] = acc;
         }
+}
+
+/* Fused MoE decode step: out[i] = sum_k slot_w[k] * sum_d dequant(W[expert[k]][i][d]) * silu(gate_k[d]) * up_k[d],
+ * silu(g) = g / (1 + exp(-g)), as the unfused chain in f32: swiglu, one 4-bit GEMV per slot
+ * (f32 sequential), then acc[i] += slot_w[k] * down[i]. gates / ups: n_slots rows of in_dim.
+ * out_f64 (may be NULL): same inner activations, dots and the slot sum accumulated in f64.
+ * Reference: crates/metaltile-std/tests/moe_down_swiglu_accum_gpu_correctness.rs:99-183 and
+ * crates/metaltile-std/src/ffai/moe_down_swiglu_accum.rs:240-275. */
+MTQ_ORACLE_API void mtq_oracle_moe_down_swiglu_accum(const float *gates, const float *ups, const uint32_t *experts,
+                                                     const float *slot_w, size_t n_slots, const uint32_t *weights,
+                                                     const float *scales, const float *biases, size_t in_dim,
+                                                     size_t out_dim, size_t group_size, float *out, double *out_f64) {
+    size_t ppr = in_dim / 8, ng = in_dim / group_size;
+    float *inner = (float *)malloc(in_dim * sizeof(float));
+    for (size_t i = 0; i < out_dim; i++) { out[i] = 0.0f; if (out_f64) out_f64[i] = 0.0; }
+    for (size_t k = 0; k < n_slots; k++) {
+        for (size_t d = 0; d < in_dim; d++) {
+            float g = gates[k * in_dim + d];
+            float silu = g / (1.0f + expf(-g));
+            inner[d] = silu * ups[k * in_dim + d];
+        }
+        size_t e = experts[k];
+        for (size_t row = 0; row < out_dim; row++) {
+            const uint32_t *rw = weights + (e * out_dim + row) * ppr;
+            const float *rs = scales + (e * out_dim + row) * ng, *rb = biases + (e * out_dim + row) * ng;
+            float acc = 0.0f;
+            double acc64 = 0.0;
+            for (size_t d = 0; d < in_dim; d++) {
+                float wv = (float)extract_code(rw, d, 4) * rs[d / group_size] + rb[d / group_size];
+                acc += wv * inner[d];
+                acc64 += (double)wv * (double)inner[d];
+            }
+            out[row] += slot_w[k] * acc;
+            if (out_f64) out_f64[row] += (double)slot_w[k] * acc64;
+        }
+    }
+    free(inner);
 }
 
 /* ------------------------------------------------------------------ */

@@ -219,6 +219,18 @@ def moe_sort_by_expert(indices, n_tokens: int, k: int, n_experts: int):
     return (order // k).astype(np.uint32), inv.astype(np.uint32), offsets.astype(np.uint32)
 
 
+def moe_down_swiglu_accum(gates, ups, experts, slot_w, weights, scales, biases, in_dim, out_dim, group_size):
+    """gates / ups: [n_slots, in_dim]. Returns (f32 chain, f64-accumulated)."""
+    gates, ups, slot_w = _f32(gates), _f32(ups), _f32(slot_w)
+    experts, weights, scales, biases = _u32(experts), _u32(weights), _f32(scales), _f32(biases)
+    n_slots = experts.size
+    out = np.empty(out_dim, dtype=np.float32)
+    out64 = np.empty(out_dim, dtype=np.float64)
+    lib().mtq_oracle_moe_down_swiglu_accum(_p(gates), _p(ups), _p(experts), _p(slot_w), _sz(n_slots), _p(weights), _p(scales),
+                                           _p(biases), _sz(in_dim), _sz(out_dim), _sz(group_size), _p(out), _p(out64))
+    return out, out64
+
+
 def affine_quantize(v, group_size: int, bits: int, dt: int):
     v = _f32(v).ravel()
     ng = v.size // group_size

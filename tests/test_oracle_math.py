@@ -325,3 +325,31 @@ def test_moe_unpermute_permute_sort(oracle):
                     perm[inv.reshape(T, k)].astype(np.float64))
     assert np.max(np.abs(out - ein)) < 1e-6
     assert np.max(np.abs(out - tokens.reshape(T, H))) < 1e-5
+
+
+def test_moe_down_swiglu_accum_against_composition(oracle):
+    """The fused MoE decode oracle against numpy silu + the expert-indexed GEMV oracle (pinned
+    above) + a numpy slot sum; one slot of weight 1 reduces to that GEMV; zero gates give zero."""
+    rng = np.random.default_rng(31)
+    E, n, k, g, slots = 6, 20, 256, 64, 8
+    codes = rng.integers(0, 16, size=(E * n, k), dtype=np.uint8)
+    s = (0.02 * np.abs(rng.standard_normal(E * n * (k // g))) + 1e-3).astype(np.float32)
+    b = (-8 * s + rng.standard_normal(s.size).astype(np.float32) * 1e-3).astype(np.float32)
+    w = oracle.pack_codes(codes, 4)
+    gates = rng.standard_normal((slots, k)).astype(np.float32) * 1.5
+    ups = rng.standard_normal((slots, k)).astype(np.float32)
+    experts = np.array([3, 1, 5, 0, 2, 4, 1, 3], dtype=np.uint32)
+    sw = np.array([0.31, 0.19, 0.12, 0.08, 0.06, 0.05, 0.04, 0.03], dtype=np.float32)
+    out32, out64 = oracle.moe_down_swiglu_accum(gates, ups, experts, sw, w, s, b, k, n, g)
+    g64 = gates.astype(np.float64)
+    inner = (g64 / (1.0 + np.exp(-g64))) * ups.astype(np.float64)
+    ref = np.zeros(n)
+    for j in range(slots):
+        ref += float(sw[j]) * oracle.expert_indexed(w, s, b, inner[j].astype(np.float32), int(experts[j]), n, k, g).astype(np.float64)
+    assert np.max(np.abs(out64 - ref)) < 1e-4 and np.max(np.abs(out32 - ref)) < 2e-4
+    assert np.max(np.abs(ref)) > 0.05
+    one32, _ = oracle.moe_down_swiglu_accum(gates[:1], ups[:1], experts[:1], np.ones(1, dtype=np.float32), w, s, b, k, n, g)
+    single = oracle.expert_indexed(w, s, b, inner[0].astype(np.float32), int(experts[0]), n, k, g)
+    assert np.max(np.abs(one32 - single)) < 1e-4
+    z32, z64 = oracle.moe_down_swiglu_accum(np.zeros_like(gates), ups, experts, sw, w, s, b, k, n, g)
+    assert not z32.any() and not z64.any()
