@@ -153,6 +153,14 @@ MTQ_API int mtq_gather_qmv_single(int dtype, int bits, uint32_t group_size, cons
                                   const uint32_t *expert_index, void *output, uint32_t N,
                                   uint32_t K, uint32_t E);
 
+/* qvm: out[m, c] = sum_d w_hat[d, c] * x[m, d] against the TRANSPOSED packed weight: w u32 [K, N*bits/32]
+ * (row d holds the N codes of K-position d), scales / biases T [K/G, N] (groups along K), x T [M, K],
+ * out T [M, N]. bits 2..8. Replaces mt_qvm_b{3,4,5,6,8} (crates/metaltile-std/src/mlx/quantized.rs:4397-4530)
+ * and mt_qvm_int4_fast (:4582-4700). K is cut into slices whose f32 partial rows go through a
+ * library-owned buffer (allocated on first use, grown on demand). */
+MTQ_API int mtq_qvm(int dtype, int bits, uint32_t group_size, const void *w, const void *scales, const void *biases,
+                    const void *x, void *out, uint32_t M, uint32_t N, uint32_t K);
+
 /* Batched qmv: n_mats (1..4) weight matrices of the same K, code width and group size
  * against ONE activation row, in one launch: outs[j][n] = sum_k w_hat_j[n,k] * x[k].
  * Replaces ffai_batched_qkv_qgemv / _fast (three matrices, one concatenated output:

@@ -50,7 +50,7 @@ struct State {
     hipStream_t stream = nullptr;  // stream in use (own_stream or the caller's)
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     void* flush_buf = nullptr;
-    void* norm_buf = nullptr;     // normalised activation row (two-step norm + qmv)
+    void* norm_buf = nullptr;     // library-owned scratch: normalised rows, qvm partial sums
     size_t norm_bytes = 0;
     size_t flush_bytes = 0;
     hipDeviceProp_t prop;
@@ -151,6 +151,38 @@ static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s,
     return op_qmv(dtype, bits, G, w, s, b, x, out, M, N, K, lc);
 }
 
+// Library-owned device scratch (normalised rows, qvm partial sums): grown on demand, never shrunk.
+static int ensure_scratch(size_t need) {
+    if (g.norm_bytes >= need) return ERR_OK;
+    if (g.norm_buf) {
+        MTQ_HIP(hipStreamSynchronize(g.stream));  // earlier launches may still use the old buffer
+        MTQ_HIP(hipFree(g.norm_buf));
+        g.norm_buf = nullptr;
+        g.norm_bytes = 0;
+    }
+    const size_t cap = need < 65536 ? 65536 : need;
+    MTQ_HIP(hipMalloc(&g.norm_buf, cap));
+    g.norm_bytes = cap;
+    return ERR_OK;
+}
+
+static int op_qvm(int dtype, int bits, uint32_t G, const void* w, const void* s, const void* b, const void* x, void* out,
+                  uint32_t M, uint32_t N, uint32_t K, const LaunchCtx& lc) {
+    if (dtype != DT_F32 && dtype != DT_F16 && dtype != DT_BF16) return fail(ERR_BAD_ARG, "dtype must be MTQ_F32, MTQ_F16 or MTQ_BF16");
+    if (bits < 2 || bits > 8) return fail(ERR_BAD_ARG, "bits must be in 2..8");
+    if (N == 0 || K == 0) return fail(ERR_SHAPE, "N and K must be non-zero");
+    if (G == 0 || K % G) return fail(ERR_SHAPE, "group_size must be non-zero and divide K");
+    if ((uint64_t)N * bits % 32) return fail(ERR_SHAPE, "N*bits must be a multiple of 32");
+    if (M == 0) return ERR_OK;
+    if (!w || !s || !b || !x || !out) return fail(ERR_BAD_ARG, "null buffer");
+    int rc = ensure_scratch(qvm_scratch_bytes(bits, G, M, N, K));
+    if (rc) return rc;
+    QmvParams p;
+    p.dtype = dtype; p.bits = bits; p.group_size = G; p.w = w; p.scales = s; p.biases = b; p.x = x; p.out = out;
+    p.M = M; p.N = N; p.K = K;
+    return launch_qvm(p, g.norm_buf, lc);
+}
+
 // RMSNorm fused into qmv: inside the streaming kernel when the row fits it, else the
 // row is normalised into a library-owned buffer and an ordinary qmv follows.
 static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const void* norm_w, const void* w,
@@ -169,17 +201,8 @@ static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const
     const uint32_t rows = dtype == DT_F32 ? 1u : 2u;
     const size_t x_bytes = ((size_t)rows * K * sz + 255) & ~(size_t)255;
     const size_t need = x_bytes + (rows == 2 ? (size_t)2 * N * sz : 0);
-    if (g.norm_bytes < need) {
-        if (g.norm_buf) {
-            MTQ_HIP(hipStreamSynchronize(g.stream));  // earlier launches may still read the old buffer
-            MTQ_HIP(hipFree(g.norm_buf));
-            g.norm_buf = nullptr;
-            g.norm_bytes = 0;
-        }
-        const size_t cap = need < 65536 ? 65536 : need;
-        MTQ_HIP(hipMalloc(&g.norm_buf, cap));
-        g.norm_bytes = cap;
-    }
+    rc = ensure_scratch(need);
+    if (rc) return rc;
     LaunchCtx first = lc, mid = lc, last = lc;
     first.stop = nullptr;
     mid.start = mid.stop = nullptr;
@@ -242,7 +265,7 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
 // name-keyed dispatch table
 // ---------------------------------------------------------------------------
 
-enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_NORMQ, F_ROUTER, F_PERMUTE, F_UNPERMUTE, F_MOEDOWN };
+enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_NORMQ, F_ROUTER, F_PERMUTE, F_UNPERMUTE, F_MOEDOWN, F_QVM, F_QVM_FAST };
 
 struct KernelDesc {
     const char* name;
@@ -311,6 +334,11 @@ static const KernelDesc kTable[] = {
     // gate_0, up_0, ..., gate_7, up_7, expert_indices, slot_weights, weights_stacked, scales_stacked, biases_stacked,
     // output | in_dim, out_dim, group_size
     {"ffai_moe_down_swiglu_accum_int4_chain8", F_MOEDOWN, 4, 22, 3},
+    // w, scales, biases, x, out | k, n, group_size (transposed weight [K, N])
+    {"mt_qvm_b3", F_QVM, 3, 5, 3}, {"mt_qvm_b4", F_QVM, 4, 5, 3}, {"mt_qvm_b5", F_QVM, 5, 5, 3},
+    {"mt_qvm_b6", F_QVM, 6, 5, 3}, {"mt_qvm_b8", F_QVM, 8, 5, 3},
+    // w, scales, biases, x, out | k, n, gs_per_col
+    {"mt_qvm_int4_fast", F_QVM_FAST, 4, 5, 3},
     // w, out, scales, biases | group_size
     {"mt_affine_quantize_int2", F_AQ, 2, 4, 1}, {"mt_affine_quantize_int3", F_AQ, 3, 4, 1},
     {"mt_affine_quantize_int4", F_AQ, 4, 4, 1}, {"mt_affine_quantize_int5", F_AQ, 5, 4, 1},
@@ -479,6 +507,24 @@ static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, in
             MTQ_NEED(bufs[2], "top_k_weights", (uint64_t)n_tok * k * sz);
             return launch_moe_unpermute(dtype, bufs[0].ptr, (const uint32_t*)bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, n_tok,
                                         n_perm, H, k, lc);
+        }
+        case F_QVM:
+        case F_QVM_FAST: {
+            const uint32_t K = consts[0], N = consts[1];
+            if (K == 0 || N == 0 || consts[2] == 0) return fail(ERR_SHAPE, "k, n and the group constexpr must be non-zero");
+            uint32_t G = consts[2];
+            if (d.fam == F_QVM_FAST) {
+                if (K % consts[2]) return fail(ERR_SHAPE, "gs_per_col must divide k");
+                G = K / consts[2];
+            }
+            if (K % G) return fail(ERR_SHAPE, "group_size must divide k");
+            const uint32_t M = (uint32_t)(bufs[4].bytes / ((uint64_t)N * sz));
+            if (M == 0) return fail(ERR_BUFFER_SIZE, "buffer 'out' holds less than one row");
+            MTQ_NEED(bufs[0], "w", (uint64_t)K * N * bits / 8);
+            MTQ_NEED(bufs[1], "scales", (uint64_t)(K / G) * N * sz);
+            MTQ_NEED(bufs[2], "biases", (uint64_t)(K / G) * N * sz);
+            MTQ_NEED(bufs[3], "x", (uint64_t)M * K * sz);
+            return op_qvm(dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, bufs[4].ptr, M, N, K, lc);
         }
         case F_MOEDOWN: {
             const uint32_t K = consts[0], N = consts[1], G = consts[2];
@@ -757,6 +803,13 @@ int mtq_gather_qmv_single(int dtype, int bits, uint32_t group_size, const void* 
                      output, 1, N, K, E, make_ctx());
 }
 
+int mtq_qvm(int dtype, int bits, uint32_t group_size, const void* w, const void* scales, const void* biases, const void* x,
+            void* out, uint32_t M, uint32_t N, uint32_t K) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return op_qvm(dtype, bits, group_size, w, scales, biases, x, out, M, N, K, make_ctx());
+}
+
 int mtq_qmv_batched(int dtype, int bits, uint32_t group_size, int n_mats, const void* const* w,
                     const void* const* scales, const void* const* biases, const void* x, void* const* outs,
                     const uint32_t* N, uint32_t K) {
@@ -1009,6 +1062,16 @@ int mtq_set_option(const char* name, int value) {
     if (!strcmp(name, "qmv.rows_per_thread")) {
         if (value != 0 && value != 4 && value != 7 && value != 8) return fail(ERR_BAD_ARG, "qmv.rows_per_thread must be 0, 4, 7 or 8");
         options().qmv_rows_per_thread = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qvm.wgs")) {
+        if (value < 0 || value > 65536) return fail(ERR_BAD_ARG, "qvm.wgs must be in 0..65536");
+        options().qvm_wgs = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "moe_down.rows")) {
+        if (value < 0 || value > 4096) return fail(ERR_BAD_ARG, "moe_down.rows must be in 0..4096");
+        options().moe_down_rows = value;
         return MTQ_OK;
     }
     if (!strcmp(name, "qmv.kernel")) {

@@ -246,25 +246,53 @@ struct UnpermuteArgs {
 
 // out[t, h] = sum_j w[t, j] * expert_outputs[inv_perm[t, j], h] in f32, j ascending, product and
 // sum rounded separately; a position past the permuted row count contributes nothing.
-template <int DT> __global__ __launch_bounds__(256) void moe_unpermute_kernel(UnpermuteArgs a) {
+// VEC elements per thread and step (16-byte loads when the row length and the pointers allow).
+template <int DT, int VEC> __global__ __launch_bounds__(256) void moe_unpermute_kernel(UnpermuteArgs a) {
 #pragma clang fp contract(off)
+    typedef typename Elem<DT>::type elem_t;
     __shared__ uint32_t pos[32];
     __shared__ float wt[32];
     const uint32_t t = blockIdx.x;
     if (threadIdx.x < a.k) {
-        pos[threadIdx.x] = a.inv_perm[(size_t)t * a.k + threadIdx.x];
+        const uint32_t p = a.inv_perm[(size_t)t * a.k + threadIdx.x];
+        pos[threadIdx.x] = p < a.n_permuted ? p : 0xFFFFFFFFu;  // out-of-range slots are skipped below
         wt[threadIdx.x] = load_elem<DT>(a.weights, (size_t)t * a.k + threadIdx.x);
     }
     __syncthreads();
-    for (uint32_t h = threadIdx.x; h < a.hidden; h += 256) {
-        float acc = 0.f;
+    for (uint32_t h = threadIdx.x * VEC; h < a.hidden; h += 256 * VEC) {
+        float acc[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; i++) acc[i] = 0.f;
         for (uint32_t j = 0; j < a.k; j++) {
-            if (pos[j] >= a.n_permuted) continue;
-            const float prod = wt[j] * load_elem<DT>(a.expert_outputs, (size_t)pos[j] * a.hidden + h);
-            acc = acc + prod;
+            if (pos[j] == 0xFFFFFFFFu) continue;  // uniform over the workgroup
+            elem_t v[VEC];
+            const elem_t* src = (const elem_t*)a.expert_outputs + (size_t)pos[j] * a.hidden + h;
+            if constexpr (VEC > 1) {
+                *(uint4*)v = *(const uint4*)src;
+            } else {
+                v[0] = src[0];
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                const float prod = wt[j] * load_elem<DT>(v, i);
+                acc[i] = acc[i] + prod;
+            }
         }
-        store_elem<DT>(a.out, (size_t)t * a.hidden + h, acc);
+        elem_t o[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; i++) store_elem<DT>(o, i, acc[i]);
+        elem_t* dst = (elem_t*)a.out + (size_t)t * a.hidden + h;
+        if constexpr (VEC > 1) {
+            *(uint4*)dst = *(const uint4*)o;
+        } else {
+            dst[0] = o[0];
+        }
     }
+}
+
+template <int DT> static const void* unpermute_fn(bool vec) {
+    constexpr int V = DT == DT_F32 ? 4 : 8;
+    return vec ? (const void*)moe_unpermute_kernel<DT, V> : (const void*)moe_unpermute_kernel<DT, 1>;
 }
 
 int launch_moe_unpermute(int dtype, const void* expert_outputs, const uint32_t* inv_perm, const void* weights, void* out,
@@ -274,11 +302,13 @@ int launch_moe_unpermute(int dtype, const void* expert_outputs, const uint32_t* 
     if (n_tokens == 0) return ERR_OK;
     if (!expert_outputs || !inv_perm || !weights || !out) return fail(ERR_BAD_ARG, "null buffer");
     UnpermuteArgs a{expert_outputs, inv_perm, weights, out, n_permuted, hidden, k};
+    const uint32_t vec = dtype == DT_F32 ? 4 : 8;
+    const bool wide = hidden % vec == 0 && (uintptr_t)expert_outputs % 16 == 0 && (uintptr_t)out % 16 == 0;
     const void* fn;
     switch (dtype) {
-        case DT_F32: fn = (const void*)moe_unpermute_kernel<DT_F32>; break;
-        case DT_F16: fn = (const void*)moe_unpermute_kernel<DT_F16>; break;
-        case DT_BF16: fn = (const void*)moe_unpermute_kernel<DT_BF16>; break;
+        case DT_F32: fn = unpermute_fn<DT_F32>(wide); break;
+        case DT_F16: fn = unpermute_fn<DT_F16>(wide); break;
+        case DT_BF16: fn = unpermute_fn<DT_BF16>(wide); break;
         default: return fail(ERR_BAD_ARG, "unknown dtype");
     }
     void* args[] = {&a};

@@ -21,7 +21,7 @@ struct MoeDownArgs {
     const void* scales;
     const void* biases;
     void* out;
-    uint32_t in_dim, out_dim, log2g, n_experts, n_slots, rows_per_wg;
+    uint32_t in_dim, out_dim, log2g, n_experts, n_slots, rows_per_wg, wide_acts;
 };
 
 template <int DT> __global__ __launch_bounds__(256) void moe_down_swiglu_kernel(MoeDownArgs a) {
@@ -29,17 +29,52 @@ template <int DT> __global__ __launch_bounds__(256) void moe_down_swiglu_kernel(
     __shared__ uint32_t expert_of[8];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     if (tid < a.n_slots) expert_of[tid] = min(a.experts[tid], a.n_experts - 1);
-    for (uint32_t k = 0; k < a.n_slots; k++) {
-        // scalar selects: an indexed read of the argument arrays would go through scratch memory
-        const void* gp = k == 0 ? a.gate[0] : k == 1 ? a.gate[1] : k == 2 ? a.gate[2] : k == 3 ? a.gate[3]
-                       : k == 4 ? a.gate[4] : k == 5 ? a.gate[5] : k == 6 ? a.gate[6] : a.gate[7];
-        const void* upp = k == 0 ? a.up[0] : k == 1 ? a.up[1] : k == 2 ? a.up[2] : k == 3 ? a.up[3]
-                        : k == 4 ? a.up[4] : k == 5 ? a.up[5] : k == 6 ? a.up[6] : a.up[7];
-        const float sw = load_elem<DT>(a.slot_w, k);
-        for (uint32_t d = tid; d < a.in_dim; d += 256) {
-            const float g = load_elem<DT>(gp, d), u = load_elem<DT>(upp, d);
+    // Every (slot, 16-byte piece) of the gate / up rows is one item; a thread issues the loads of
+    // up to four items before it touches any of them, so the staging costs one memory round trip.
+    // Pointers are picked with compare-selects: an indexed read of the argument arrays would go
+    // through scratch memory.
+    auto gate_of = [&](uint32_t k) {
+        return k == 0 ? a.gate[0] : k == 1 ? a.gate[1] : k == 2 ? a.gate[2] : k == 3 ? a.gate[3]
+             : k == 4 ? a.gate[4] : k == 5 ? a.gate[5] : k == 6 ? a.gate[6] : a.gate[7];
+    };
+    auto up_of = [&](uint32_t k) {
+        return k == 0 ? a.up[0] : k == 1 ? a.up[1] : k == 2 ? a.up[2] : k == 3 ? a.up[3]
+             : k == 4 ? a.up[4] : k == 5 ? a.up[5] : k == 6 ? a.up[6] : a.up[7];
+    };
+    typedef typename Elem<DT>::type elem_t;
+    if (a.wide_acts) {
+        constexpr int V = DT == DT_F32 ? 4 : 8;  // elements per 16-byte load (in_dim % 32 == 0)
+        const uint32_t per_slot = a.in_dim / V, total = a.n_slots * per_slot;
+        for (uint32_t base = 0; base < total; base += 1024) {
+            uint4 gv[4], uv[4];
+            float sw[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint32_t it = min(base + u * 256 + tid, total - 1);
+                const uint32_t k = it / per_slot, d = (it - k * per_slot) * V;
+                gv[u] = *(const uint4*)((const elem_t*)gate_of(k) + d);
+                uv[u] = *(const uint4*)((const elem_t*)up_of(k) + d);
+                sw[u] = load_elem<DT>(a.slot_w, k);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint32_t it = base + u * 256 + tid;
+                if (it >= total) break;
+                const uint32_t k = it / per_slot, d = (it - k * per_slot) * V;
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    const float g = load_elem<DT>(&gv[u], i), up = load_elem<DT>(&uv[u], i);
+                    const float silu = g / (1.0f + expf(0.0f - g));
+                    inner[k * a.in_dim + d + i] = sw[u] * (silu * up);
+                }
+            }
+        }
+    } else {
+        for (uint32_t it = tid; it < a.n_slots * a.in_dim; it += 256) {
+            const uint32_t k = it / a.in_dim, d = it - k * a.in_dim;
+            const float g = load_elem<DT>(gate_of(k), d), up = load_elem<DT>(up_of(k), d);
             const float silu = g / (1.0f + expf(0.0f - g));
-            inner[k * a.in_dim + d] = sw * (silu * u);
+            inner[it] = load_elem<DT>(a.slot_w, k) * (silu * up);
         }
     }
     __syncthreads();
@@ -91,12 +126,15 @@ int launch_moe_down_swiglu(int dtype, uint32_t group_size, uint32_t n_slots, con
     if (!gates || !ups || !experts || !slot_w || !w || !scales || !biases || !out) return fail(ERR_BAD_ARG, "null buffer");
     if ((uintptr_t)w % 16) return fail(ERR_UNSUPPORTED, "moe down: weights must be 16-byte aligned");
     MoeDownArgs a;
+    bool wide = true;  // 16-byte loads of the gate / up rows
     for (uint32_t k = 0; k < 8; k++) {
         const uint32_t j = k < n_slots ? k : 0;
         if (!gates[j] || !ups[j]) return fail(ERR_BAD_ARG, "null gate / up buffer");
         a.gate[k] = gates[j];
         a.up[k] = ups[j];
+        if ((uintptr_t)gates[j] % 16 || (uintptr_t)ups[j] % 16) wide = false;
     }
+    a.wide_acts = wide ? 1u : 0u;
     a.experts = experts;
     a.slot_w = slot_w;
     a.w = (const uint32_t*)w;

@@ -81,6 +81,8 @@ struct QmvBatch {
 
 // Tuning overrides set through mtq_set_option (0 = automatic).
 struct Options {
+    int qvm_wgs = 0;              // qvm: target workgroup count (0 = 1024)
+    int moe_down_rows = 0;        // fused MoE down projection: rows per workgroup (0 = automatic)
     int qmv_rows_per_thread = 0;  // one-shot kernel: weight rows per thread
     int qmv_kernel = 0;           // 0 auto, 1 one-shot only, 2 prefer streaming
     int qmv_stream_depth = 0;     // streaming kernel: ring depth (4 / 8)
@@ -122,6 +124,10 @@ int launch_moe_unpermute(int dtype, const void* expert_outputs, const uint32_t* 
 int launch_moe_down_swiglu(int dtype, uint32_t group_size, uint32_t n_slots, const void* const* gates, const void* const* ups,
                            const uint32_t* experts, const void* slot_w, const void* w, const void* scales, const void* biases,
                            void* out, uint32_t in_dim, uint32_t out_dim, uint32_t n_experts, const LaunchCtx& lc);
+// qvm (qvm.hip): p.w is [K, N] packed along N, p.scales / p.biases [K/G, N]; scratch holds
+// qvm_scratch_bytes() of f32 partial rows.
+size_t qvm_scratch_bytes(int bits, uint32_t group_size, uint32_t M, uint32_t N, uint32_t K);
+int launch_qvm(const QmvParams& p, void* scratch, const LaunchCtx& lc);
 int launch_add_rows(int dtype, const void* a, const void* b, void* out, uint32_t n, const LaunchCtx& lc);
 int launch_qmv_batched(const QmvParams& p, const QmvBatch& b, const LaunchCtx& lc);
 // Matrix-core streaming GEMV family for f16/bf16 (qmv_mfma.hip); same contract.

@@ -116,6 +116,13 @@ const Bench kBenches[] = {
     {"mlx/quantized/qmv_b5", "mt_qmv_b5", ABI_QB, 5, 1, 4096, 4096, 64, 1},
     {"mlx/quantized/qmv_b6", "mt_qmv_b6", ABI_QB, 6, 1, 4096, 4096, 64, 1},
     {"mlx/quantized/qmv_b8", "mt_qmv_b8", ABI_QB, 8, 1, 4096, 4096, 64, 1},
+    // transposed weight [K, N]: same buffer totals as qmv at a square shape
+    {"mlx/quantized/qvm_int4_fast", "mt_qvm_int4_fast", ABI_QMM, 4, 1, 4096, 4096, 64, 1},
+    {"mlx/quantized/qvm_b3", "mt_qvm_b3", ABI_QB, 3, 1, 4096, 4096, 64, 1},
+    {"mlx/quantized/qvm_b4", "mt_qvm_b4", ABI_QB, 4, 1, 4096, 4096, 64, 1},
+    {"mlx/quantized/qvm_b5", "mt_qvm_b5", ABI_QB, 5, 1, 4096, 4096, 64, 1},
+    {"mlx/quantized/qvm_b6", "mt_qvm_b6", ABI_QB, 6, 1, 4096, 4096, 64, 1},
+    {"mlx/quantized/qvm_b8", "mt_qvm_b8", ABI_QB, 8, 1, 4096, 4096, 64, 1},
     {"mlx/quantized/qmm_b3", "mt_qmm_b3", ABI_QB, 3, 4, 4096, 4096, 64, 1},
     {"mlx/quantized/qmm_b4", "mt_qmm_b4", ABI_QB, 4, 4, 4096, 4096, 64, 1},
     {"mlx/quantized/qmm_b5", "mt_qmm_b5", ABI_QB, 5, 4, 4096, 4096, 64, 1},

@@ -45,6 +45,12 @@ def gather_qmv_single(dtype, bits, group_size, w, scales, biases, inp, expert_in
                                          _p(inp), _p(expert_index), _p(out), N, K, E))
 
 
+def qvm(dtype, bits, group_size, w, scales, biases, x, out, M, N, K):
+    """out[M, N] = x[M, K] @ w_hat, w packed [K, N*bits/32], scales / biases [K/G, N]."""
+    lib = _ensure_init()
+    _lib.check(lib.mtq_qvm(int(dtype), bits, group_size, _p(w), _p(scales), _p(biases), _p(x), _p(out), M, N, K))
+
+
 def qmv_batched(dtype, bits, group_size, ws, scales, biases, x, outs, Ns, K):
     """2..4 weight matrices (lists of buffers) against one activation row, one launch."""
     lib = _ensure_init()

@@ -81,3 +81,6 @@ _add("ffai_moe_down_swiglu_accum_int4_chain8", 4,
      tuple(n for k in range(8) for n in (f"gate_{k}", f"up_{k}")) + ("expert_indices", "slot_weights", "weights_stacked",
                                                                       "scales_stacked", "biases_stacked", "output"),
      ("in_dim", "out_dim", "group_size"), ("output",))
+for _b in (3, 4, 5, 6, 8):
+    _add(f"mt_qvm_b{_b}", _b, ("w", "scales", "biases", "x", "out"), ("k", "n", "group_size"), ("out",))
+_add("mt_qvm_int4_fast", 4, ("w", "scales", "biases", "x", "out"), ("k", "n", "gs_per_col"), ("out",))

@@ -27,6 +27,8 @@
  *   rms_norm_qgemv    numpy restatement (dequant matrix @ normalised row), unit norm
  *                     weights with a constant row (inv_rms in closed form), scale
  *                     invariance in x, eps -> large limit.
+ *   qvm               numpy f64 `x @ dequant(W)` on the [K, N] layout, and qvm(W) == qmv of the
+ *                     transposed, repacked matrix.
  *   moe routing       numpy stable argsort + library softmax, the reference tests' tie-break,
  *                     k = 1 and NaN/Inf cases; unpermute against a numpy einsum; permute and
  *                     the expert sort are numpy one-liners (take, stable argsort) in oracle.py.
@@ -445,6 +447,29 @@ MTQ_ORACLE_API void mtq_oracle_rms_norm_qgemv(const uint32_t *weight, const floa
         if (out_f64) out_f64[row] = acc64;
     }
     free(nx);
+}
+
+/* Vector-matrix product against a transposed packed weight: out[m, c] = sum_d w_hat[d, c] * x[m, d],
+ * W [K, N] packed along N (row d holds N codes), scales / biases [K/G, N] (groups along K).
+ * f32 sequential in d; out_f64 (may be NULL) accumulates the same f32 weights in f64.
+ * Reference: crates/metaltile-std/src/mlx/quantized.rs:5613-5635 (qvm_oracle) and :4397-4522 (kernels). */
+MTQ_ORACLE_API void mtq_oracle_qvm(const uint32_t *w, const float *scales, const float *biases, const float *x,
+                                   size_t m, size_t n, size_t k, uint32_t bits, size_t group_size, float *out,
+                                   double *out_f64) {
+    size_t wpr = n * bits / 32;
+    for (size_t row = 0; row < m; row++)
+        for (size_t c = 0; c < n; c++) {
+            float acc = 0.0f;
+            double acc64 = 0.0;
+            for (size_t d = 0; d < k; d++) {
+                size_t g = d / group_size;
+                float wv = (float)extract_code(w + d * wpr, c, bits) * scales[g * n + c] + biases[g * n + c];
+                acc += wv * x[row * k + d];
+                acc64 += (double)wv * (double)x[row * k + d];
+            }
+            out[row * n + c] = acc;
+            if (out_f64) out_f64[row * n + c] = acc64;
+        }
 }
 
 /* ------------------------------------------------------------------ */

@@ -185,6 +185,16 @@ def rms_norm_qgemv(w, scales, biases, x, norm_weight, in_dim, group_size, out_di
     return out, out64, normed
 
 
+def qvm(w, scales, biases, x, m, n, k, bits, group_size):
+    """W [K, N] packed along N, scales / biases [K/G, N]. Returns (f32 sequential, f64-accumulated), each [m, n]."""
+    w, scales, biases, x = _u32(w), _f32(scales), _f32(biases), _f32(x)
+    out = np.empty(m * n, dtype=np.float32)
+    out64 = np.empty(m * n, dtype=np.float64)
+    lib().mtq_oracle_qvm(_p(w), _p(scales), _p(biases), _p(x), _sz(m), _sz(n), _sz(k), C.c_uint32(bits), _sz(group_size),
+                         _p(out), _p(out64))
+    return out, out64
+
+
 def moe_router_topk(logits, n_rows: int, n_experts: int, k: int, norm_topk_prob: int = 1):
     logits = _f32(logits)
     idx = np.empty(n_rows * k, dtype=np.uint32)

@@ -141,7 +141,7 @@ def test_bench_driver_lists_the_reference_registrations():
         build(verbose=False)
     out = subprocess.run([DRIVER, "--list"], capture_output=True, text=True, check=True).stdout
     rows = [l.split("\t") for l in out.strip().splitlines()]
-    assert len(rows) >= 49
+    assert len(rows) >= 55
     names = [r[0] for r in rows]
     assert len(set(names)) == len(names)
     for must in ("mlx/quantized/qmv", "mlx/quantized/qmm_mma", "ffai/dequant_gemv/int4_fast",

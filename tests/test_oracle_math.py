@@ -353,3 +353,27 @@ def test_moe_down_swiglu_accum_against_composition(oracle):
     assert np.max(np.abs(one32 - single)) < 1e-4
     z32, z64 = oracle.moe_down_swiglu_accum(np.zeros_like(gates), ups, experts, sw, w, s, b, k, n, g)
     assert not z32.any() and not z64.any()
+
+
+@pytest.mark.parametrize("bits", [3, 4, 5, 6, 8])
+def test_qvm_against_numpy_and_transposed_qmv(oracle, bits):
+    """qvm on the [K, N] layout: (a) numpy f64 x @ dequant(W) with an independently unpacked
+    code matrix; (b) equals qmv of the transposed matrix repacked along K (scales transposed
+    too) -- a swapped axis in the code or scale indexing breaks one of the two."""
+    rng = np.random.default_rng(800 + bits)
+    m, n, k, g = 2, 64, 128, 32
+    codes = rng.integers(0, 1 << bits, size=(k, n), dtype=np.uint8)      # [K, N]
+    s = (0.02 * np.abs(rng.standard_normal((k // g, n))) + 1e-3).astype(np.float32)
+    b = (rng.standard_normal((k // g, n)) * 0.05).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = oracle.pack_codes(codes, bits)                                    # rows = K, packed along N
+    assert np.array_equal(oracle.np_unpack_codes(w, k, n, bits), codes)
+    out32, out64 = oracle.qvm(w, s, b, x, m, n, k, bits, g)
+    wd = codes.astype(np.float32) * np.repeat(s, g, axis=0) + np.repeat(b, g, axis=0)   # f32 products, as the oracle forms them
+    ref = x.astype(np.float64) @ wd.astype(np.float64)
+    assert np.max(np.abs(out64.reshape(m, n) - ref)) < 1e-9
+    assert np.max(np.abs(out32.reshape(m, n) - ref)) < 2e-4
+    assert np.max(np.abs(ref)) > 0.3
+    wt = oracle.pack_codes(np.ascontiguousarray(codes.T), bits)          # [N, K]
+    via_qmv = oracle.qmm_f64(wt, np.ascontiguousarray(s.T), np.ascontiguousarray(b.T), x, m, n, k, bits, g)
+    assert np.max(np.abs(via_qmv.reshape(m, n) - ref)) < 1e-9
