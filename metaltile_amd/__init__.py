@@ -9,6 +9,7 @@ from .dtypes import DType, pack_f32, unpack_f32, dtype_label  # noqa: F401
 from .errors import MtqError  # noqa: F401
 from .stats import BenchStats, to_gbps, to_gflops  # noqa: F401
 from .selector import mt_qmm_for  # noqa: F401
+from . import dynamic_m  # noqa: F401
 from .runtime import Context, DispatchResult, GpuRunner, GpuBuffer  # noqa: F401
 from . import ops  # noqa: F401
 

@@ -24,6 +24,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <ctime>
 #include <string>
 #include <vector>
 
@@ -42,6 +43,8 @@ struct Rng {
     }
     float unit() { return (float)((next() >> 40) * (1.0 / 16777216.0)); }
 };
+
+std::vector<std::string>* g_snapshot_rows = nullptr;  // set when --snapshot is given
 
 size_t esize(int dt) { return dt == MTQ_F32 ? 4 : 2; }
 const char* dt_label(int dt) { return dt == MTQ_F32 ? "f32" : dt == MTQ_F16 ? "f16" : "bf16"; }
@@ -263,6 +266,13 @@ int run_one(const Bench& bn, int dt, int warmup, int iters) {
     const double mn = us.front(), med = us[us.size() / 2];
     const char* slash = strrchr(bn.name, '/');
     const std::string op(bn.name, slash ? (size_t)(slash - bn.name) : strlen(bn.name));
+    if (g_snapshot_rows) {
+        // a row of the reference's snapshot file (crates/metaltile-cli/src/cmd/bench.rs:361-372, keys in serde_json's sorted order)
+        char row[512];
+        snprintf(row, sizeof row, "    {\n      \"metric\": \"GB/s\",\n      \"mt\": %.3f,\n      \"op\": \"%s\",\n      \"ref\": null,\n"
+                 "      \"shape\": \"%s\",\n      \"subop\": \"%s\"\n    }", (double)bytes / mn / 1e3, op.c_str(), shape, slash ? slash + 1 : bn.name);
+        g_snapshot_rows->push_back(row);
+    }
     printf("{\"op\": \"%s\", \"subop\": \"%s\", \"shape\": \"%s\", \"metric\": \"GB/s\", \"ref\": null, \"mt\": %.1f, "
            "\"min_us\": %.2f, \"median_us\": %.2f, \"bytes_moved\": %llu, \"kernel\": \"%s\"}\n",
            op.c_str(), slash ? slash + 1 : bn.name, shape, (double)bytes / mn / 1e3, mn, med, (unsigned long long)bytes, bn.kernel);
@@ -273,7 +283,7 @@ int run_one(const Bench& bn, int dt, int warmup, int iters) {
 }  // namespace
 
 int main(int argc, char** argv) {
-    std::string filter;
+    std::string filter, snapshot, note;
     bool list = false;
     int warmup = 15, iters = 10, device = 0;
     std::vector<int> dtypes = {MTQ_F32, MTQ_F16, MTQ_BF16};
@@ -281,6 +291,8 @@ int main(int argc, char** argv) {
         const std::string a = argv[i];
         if ((a == "-f" || a == "--filter") && i + 1 < argc) filter = argv[++i];
         else if (a == "--list") list = true;
+        else if (a == "--snapshot" && i + 1 < argc) snapshot = argv[++i];
+        else if (a == "--note" && i + 1 < argc) note = argv[++i];
         else if (a == "--warmup" && i + 1 < argc) warmup = atoi(argv[++i]);
         else if (a == "--iters" && i + 1 < argc) iters = atoi(argv[++i]);
         else if (a == "--device" && i + 1 < argc) device = atoi(argv[++i]);
@@ -288,7 +300,8 @@ int main(int argc, char** argv) {
             const std::string d = argv[++i];
             dtypes = {d == "f32" ? MTQ_F32 : d == "f16" ? MTQ_F16 : MTQ_BF16};
         } else {
-            fprintf(stderr, "usage: tile_bench [-f substring] [--dtype f32|f16|bf16] [--warmup N] [--iters N] [--device N] [--list]\n");
+            fprintf(stderr, "usage: tile_bench [-f substring] [--dtype f32|f16|bf16] [--warmup N] [--iters N] [--device N] [--list]\n"
+                            "                  [--snapshot out.json [--note text]]\n");
             return 2;
         }
     }
@@ -305,6 +318,8 @@ int main(int argc, char** argv) {
     mtq_device_name(name, sizeof name);
     fprintf(stderr, "device: %s\n", name);
     int failed = 0, ran = 0;
+    std::vector<std::string> rows;
+    if (!snapshot.empty()) g_snapshot_rows = &rows;
     for (const Bench& b : kBenches) {
         if (!filter.empty() && !strstr(b.name, filter.c_str())) continue;
         if (!mtq_kernel_supported(b.kernel)) {
@@ -317,6 +332,35 @@ int main(int argc, char** argv) {
                 fprintf(stderr, "%s %s: failed\n", b.name, dt_label(dt));
                 failed++;
             }
+        }
+    }
+    if (!snapshot.empty()) {
+        // the layout of the reference's `tile snap` files (crates/metaltile-cli/src/cmd/snap.rs:24-35), which `tile diff` reads
+        FILE* f = fopen(snapshot.c_str(), "w");
+        if (!f) {
+            fprintf(stderr, "cannot write %s\n", snapshot.c_str());
+            failed++;
+        } else {
+            mtq_device_info info;
+            char arch[128] = "";
+            if (mtq_get_device_info(&info) == 0) snprintf(arch, sizeof arch, "%s", info.arch);
+            char stamp[32];
+            const time_t now = time(nullptr);
+            strftime(stamp, sizeof stamp, "%Y-%m-%dT%H:%M:%SZ", gmtime(&now));
+            fprintf(f, "{\n  \"device\": \"%s\",\n  \"gpu_family\": \"%s\",\n  \"timestamp\": \"%s\",\n", name[0] ? name : arch, arch, stamp);
+            if (!note.empty()) {
+                std::string esc;
+                for (char c : note) {
+                    if (c == '"' || c == '\\') esc += '\\';
+                    if ((unsigned char)c >= 0x20) esc += c;
+                }
+                fprintf(f, "  \"note\": \"%s\",\n", esc.c_str());
+            }
+            fprintf(f, "  \"results\": [\n");
+            for (size_t i = 0; i < rows.size(); i++) fprintf(f, "%s%s\n", rows[i].c_str(), i + 1 < rows.size() ? "," : "");
+            fprintf(f, "  ]\n}\n");
+            fclose(f);
+            fprintf(stderr, "snapshot: %zu rows -> %s\n", rows.size(), snapshot.c_str());
         }
     }
     mtq_shutdown();

@@ -162,3 +162,20 @@ def test_bench_driver_fails_loudly_without_a_gpu():
         assert r.returncode != 0 and "no HIP device" in r.stderr
     else:
         pytest.skip("a GPU is present")
+
+
+def test_dynamic_m_helpers_match_reference_values():
+    """crates/metaltile-std/src/mlx/quantized_mma_dynamic_m.rs:116-160 (its unit tests)."""
+    from metaltile_amd import dynamic_m as d
+    assert [d.pad_t_to_bm(t) for t in (0, 1, 31, 32, 33, 37, 64, 4096, 4097)] == [0, 32, 32, 32, 64, 64, 64, 4096, 4128]
+    assert d.dispatch_grid(1, 128) == [4, 1, 1]
+    assert d.dispatch_grid(37, 128) == [4, 2, 1]
+    assert d.dispatch_grid(4096, 2048) == [64, 128, 1]
+    assert all(d.kernel_name_for(dt) == "mt_qmm_mma" for dt in (DType.F32, DType.F16, DType.BF16))
+    with pytest.raises(ValueError):
+        d.dispatch_grid(32, 100)
+    x = b"\x01" * 16
+    p = d.pad_x_rows_bytes(x, 2, 4, 2)
+    assert len(p) == 32 * 4 * 2 and p[:16] == x and not any(p[16:])
+    with pytest.raises(ValueError):
+        d.pad_x_rows_bytes(x, 3, 4, 2)
