@@ -210,7 +210,8 @@ def main():
                        "launches_per_step": len(specs), "bytes_per_launch": launch_bytes,
                        "device": info["name"] or info["arch"]},
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                         "frac": round(achieved / HBM_PEAK_GBS, 4),
+                         "traffic": traffic_from_profiles("qkv_fused_bf16_b4_llama_attn"),
                          "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, 1 row>, 3 matrices per launch",
                          "avg_launch_us_timed_region": round(kern_avg, 3)},
         })
