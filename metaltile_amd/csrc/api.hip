@@ -1095,7 +1095,7 @@ int mtq_set_option(const char* name, int value) {
         return MTQ_OK;
     }
     if (!strcmp(name, "qmv.mfma_kp") || !strcmp(name, "qmv.mfma_rbw") || !strcmp(name, "qmv.mfma_nrb")) {
-        if (value < 0 || value > 16) return fail(ERR_BAD_ARG, "qmv.mfma_* must be in 0..16");
+        if (value < 0 || value > 256) return fail(ERR_BAD_ARG, "qmv.mfma_* must be in 0..256");
         if (name[9] == 'k') options().qmv_mfma_kp = value;
         else if (name[9] == 'r') options().qmv_mfma_rbw = value;
         else options().qmv_mfma_nrb = value;

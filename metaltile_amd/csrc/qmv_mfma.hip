@@ -16,9 +16,31 @@ bool is_pow2(uint32_t v) { return v && !(v & (v - 1)); }
 uint32_t ilog2(uint32_t v) { uint32_t l = 0; while ((1u << l) < v) l++; return l; }
 constexpr size_t kLdsBudget = 150 * 1024;  // of the 160 KB per CU
 
-size_t lds_bytes(uint32_t R, uint32_t K, uint32_t nch, uint32_t rows_wg, uint32_t gpr, uint32_t KP, uint32_t list_cap) {
-    return (size_t)R * K * 2 + (size_t)R * nch * 4 + ((size_t)rows_wg * gpr + 1) * 8 +
+int num_cus_mfma() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0, v = 0;
+        n = (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) ? v : 256;
+    }
+    return n;
+}
+
+// waves = KP * RBW; gpw = (scale, bias) pairs per row in a wave's window
+size_t lds_bytes(uint32_t R, uint32_t K, uint32_t nch, uint32_t rows_wg, uint32_t waves, uint32_t gpw, uint32_t KP, uint32_t list_cap) {
+    return (size_t)R * K * 2 + (size_t)R * nch * 4 + ((size_t)waves * 4 * gpw + 1) * 8 +
            (size_t)KP * rows_wg * R * 4 + (size_t)list_cap * 4 + 64;
+}
+
+// Pairs per row that a wave's window must hold: the groups its K part touches, from a
+// multiple of 4 (8-byte loads) up to a whole number of 4-vectors.
+uint32_t window_pairs(uint32_t kp_count, uint32_t spp, uint32_t cpc, uint32_t log2g) {
+    uint32_t need = 4;
+    for (uint32_t kp = 0; kp < kp_count; kp++) {
+        const uint32_t first = (kp * spp * 16u * cpc) >> log2g, last = (((kp + 1) * spp * 16u * cpc) - 1u) >> log2g;
+        const uint32_t lo = first & ~3u, n = (last + 1 - lo + 3) / 4 * 4;
+        if (n > need) need = n;
+    }
+    return need;
 }
 }  // namespace
 
@@ -55,6 +77,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
         double best_score = 1e30;
         for (uint32_t kp = 1; kp <= nseg && kp <= 16; kp++) {
             if (nseg % kp) continue;
+            if (window_pairs(kp, nseg / kp, cpc, ilog2(G)) > 64) continue;  // a lane refills one 4-vector of its wave's window
             const uint32_t spp = nseg / kp, padded = (spp + 3) / 4 * 4;
             double score = (double)(padded - spp) / spp;          // wasted ring slots
             if (spp > 8) score += 0.05 * (spp - 8);               // long walks: few waves per row block
@@ -65,6 +88,8 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
         KP = best;
     }
     const uint32_t spp = nseg / KP;
+    const uint32_t gpw = window_pairs(KP, spp, cpc, ilog2(G));
+    if (gpw > 64) return fail(ERR_UNSUPPORTED, "mfma qmv: K part spans more than 64 groups");
 
     // activation rows per pass
     int mp = 4, s = 1;
@@ -77,11 +102,11 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
         mp = 1;
     } else {
         const uint32_t avg = (rows + p.E - 1) / (p.E ? p.E : 1);
-        // 4 rows per pass keep two workgroups per CU (32 KB of staged activations at
-        // K = 4096); experts with more rows take another pass over weights that are
-        // still in L2. Measured on 8 experts x 14336x4096 with 2..6 rows each: 75 us
-        // against 80 us at 8 rows per pass.
-        s = avg > 8 ? 4 : (avg > 4 ? 2 : 1);
+        // 8 rows per pass from an average of 3 rows per expert: with uneven routing some expert
+        // then has more than 4, and a second pass would stream its weights again (measured on
+        // 8 experts x 14336x4096 with 2..6 rows each: 1.29 x the algorithmic traffic at 4 rows
+        // per pass, 1.01 x at 8).
+        s = avg > 8 ? 4 : (avg >= 3 ? 2 : 1);
         if (p.bits == 2 && s > 2) s = 2;  // the 16-row 2-bit variant does not fit the register file
         if (opt.qmv_mfma_sets) s = opt.qmv_mfma_sets;
     }
@@ -92,14 +117,35 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     // side by side as the workgroup size allows, the rest one after the other.
     uint32_t rows_target = 8;
     while (rows_target < 32 && (uint64_t)rows_target * 2 * 256 <= p.N) rows_target *= 2;
-    // A gather workgroup stages up to R activation rows of K elements before it
-    // streams: give it twice the rows so that staging stays small beside the
-    // weights it serves.
-    if (gather) rows_target = 64;
-    const uint32_t rbw_cap = gather ? 8u : 16u;  // 512-thread gather workgroups: two per CU
+    const uint32_t rbw_cap = 16u;
     uint32_t RBW = rows_target / 4 < rbw_cap ? rows_target / 4 : rbw_cap;
     while (64u * KP * RBW > maxt && RBW > 1) RBW /= 2;
     uint32_t nrb = rows_target / 4 / RBW;
+    if (gather) {
+        // A gather workgroup stages up to R activation rows of K elements before it streams, so it
+        // should live long: the largest workgroup the instance allows, and as many row blocks one
+        // after the other as leave one workgroup (two when 4 rows are staged) per CU over the
+        // experts that can be hit. Measured on 8 experts x 14336x4096, 32 rows: 61 us with 7 row
+        // blocks of 64 rows per workgroup, 74 us with 4, 98 us with 14.
+        // Short rows (few steps per row block) want the row blocks one after the other in a
+        // narrow workgroup rather than side by side in a wide one: at least 16 steps per wave
+        // (E = 128 x 256x2048 with one row per expert: 15 us with 2 blocks side by side x 4 in
+        // sequence, 30 us with 16 side by side).
+        const uint64_t e_eff = p.E < rows ? p.E : rows;
+        const uint64_t slots = (uint64_t)num_cus_mfma() * (s == 1 ? 2 : 1);
+        const uint64_t units = ((uint64_t)p.N + 3) / 4 * e_eff;              // 4-row blocks over the experts that can be hit
+        uint64_t per_wg = (units + slots - 1) / slots;                       // blocks per workgroup
+        const uint64_t max_per_wg = ((uint64_t)p.N + 3) / 4;
+        if (per_wg > max_per_wg) per_wg = max_per_wg;
+        const uint32_t min_nrb = spp >= 16 ? 1u : (16u + spp - 1) / spp;
+        uint32_t rbw_max = rbw_cap;
+        while (64u * KP * rbw_max > maxt && rbw_max > 1) rbw_max /= 2;
+        RBW = 1;
+        while (RBW * 2 <= rbw_max && (uint64_t)RBW * 2 * min_nrb <= per_wg) RBW *= 2;
+        nrb = (uint32_t)((per_wg + RBW - 1) / RBW);
+        if (nrb < 1) nrb = 1;
+        if (nrb > 64) nrb = 64;
+    }
     if (opt.qmv_mfma_rbw) {
         RBW = (uint32_t)opt.qmv_mfma_rbw;
         if (64u * KP * RBW > maxt) return fail(ERR_BAD_ARG, "qmv.mfma_rbw: workgroup too large");
@@ -107,7 +153,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     if (opt.qmv_mfma_nrb) nrb = (uint32_t)opt.qmv_mfma_nrb;
     const uint32_t list_cap = p.gather == GATHER_INDICES ? p.T : 0;
     // shrink until the workgroup's LDS fits
-    while (lds_bytes((uint32_t)(mp * s), p.K, nch, 4 * RBW * nrb, gpr, KP, list_cap) > kLdsBudget) {
+    while (lds_bytes((uint32_t)(mp * s), p.K, nch, 4 * RBW * nrb, KP * RBW, gpw, KP, list_cap) > kLdsBudget) {
         if (nrb > 1) nrb--;
         else if (s > 1) s /= 2;
         else if (RBW > 1) RBW--;
@@ -151,6 +197,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     a.RBW = RBW;
     a.nrb = nrb;
     a.gpr = gpr;
+    a.gpw = gpw;
     a.log2g = ilog2(G);
     a.list_cap = list_cap;
     a.delay = (uint32_t)opt.qmv_mfma_delay;
@@ -159,7 +206,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     g.s = s;
     g.tpb = 64u * KP * RBW;
     const uint32_t rows_wg = 4 * RBW * nrb;
-    g.shmem = lds_bytes(R, p.K, nch, rows_wg, gpr, KP, list_cap);
+    g.shmem = lds_bytes(R, p.K, nch, rows_wg, KP * RBW, gpw, KP, list_cap);
     g.grid = dim3((p.N + rows_wg - 1) / rows_wg, gather ? p.E : 1, 1);
     if (odd)
         return p.dtype == DT_F16 ? qmv_mfma_launch_dtype_odd<DT_F16>(a, p.bits, p.gather, g, lc)

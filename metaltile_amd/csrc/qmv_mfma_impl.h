@@ -71,6 +71,7 @@ struct QmvMArgs {
     uint32_t RBW;       // row blocks walked in parallel by one workgroup
     uint32_t nrb;       // row blocks per wave, one after the other
     uint32_t gpr, log2g;
+    uint32_t gpw;       // (scale, bias) pairs per row that a wave keeps in LDS: the groups of its K part, whole 4-vectors, <= 64
     uint32_t list_cap;  // capacity of the row list (indices mode)
     uint32_t delay;     // units of 512 clocks between the small loads and the first weight loads
 };
@@ -173,7 +174,11 @@ template <int DT, int BITS> struct MfmaCodec {
     }
 };
 
-template <int DT, int BITS, int MP, int S, int D, int MODE, int MAXT>
+__device__ __forceinline__ uint32_t waves_of(const QmvMArgs& a) { return a.KP * a.RBW; }  // waves per workgroup
+
+// REFILL: the workgroup walks more than one row block (nrb > 1) and refills the waves' (scale, bias)
+// windows as it goes; the single-block instance carries none of that state.
+template <int DT, int BITS, int MP, int S, int D, int MODE, int MAXT, bool REFILL>
 __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     typedef MfmaCodec<DT, BITS> Codec;
     constexpr int CPC = Codec::CPC;  // codes per lane chunk
@@ -188,8 +193,9 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     const uint32_t rows_wg = 4u * a.RBW * a.nrb;
     m_u32x4* XL = (m_u32x4*)smem;                                    // [S][NP][nch][MP] pieces
     float* XS = (float*)(XL + (size_t)S * NP * a.nch * MP);          // [S][nch][MP] chunk sums
-    float2* SB = (float2*)(XS + (size_t)S * a.nch * MP);             // [rows_wg][gpr] + one zero pair
-    float* RED = (float*)(SB + (size_t)rows_wg * a.gpr + 1);         // [KP][rows_wg][R]
+    float2* SB = (float2*)(XS + (size_t)S * a.nch * MP);             // [waves][4 rows][gpw] + one zero pair
+    const uint32_t sb_zero = (waves_of(a)) * 4u * a.gpw;               // index of the zero pair
+    float* RED = (float*)(SB + (size_t)sb_zero + 1);                 // [KP][rows_wg][R]
     uint32_t* rowlist = (uint32_t*)(RED + (size_t)a.KP * rows_wg * R);
     __shared__ uint32_t s_meta[4];
 
@@ -248,6 +254,41 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     constexpr uint32_t SEGB = 16u * Codec::CB;  // bytes of one weight row covered by a wave-wide load
     const unsigned char* wbase = a.w + slab_rows * a.RB + (size_t)(kp * a.spp) * SEGB + q * (uint32_t)Codec::CB;
     const uint32_t sppD = (a.spp + D - 1) / D * D;  // steps per row block, padded to whole rings
+    // (scale, bias) pairs: every wave keeps those of its own 4 rows and its own K part in its own
+    // LDS window and refills it when it moves to the next row block, so the number of row blocks
+    // a workgroup walks is not bounded by LDS and no workgroup barrier sits in the refill.
+    const uint32_t g_lo = ((kp * a.spp * 16u * (uint32_t)CPC) >> a.log2g) & ~3u;  // first group of the window
+    const uint32_t sbw_off = wave * 4u * a.gpw;                 // this wave's window: [4 rows][gpw] pairs
+    const uint32_t sb_row = sbw_off + r * a.gpw - g_lo;          // + g = this lane's row, group g
+    // Lane l refills 4 pairs of the window: row l & 3, groups g_lo + 4 * (l >> 2) .. + 3 (gpw <= 64, so
+    // one 8-byte load of scales and one of biases per lane and refill).
+    struct SbRegs { uint2 s, b; };
+    auto sbw_load = [&](uint32_t rb, SbRegs& o) {
+        rb = min(rb, a.nrb - 1);
+        const uint32_t row = min(row0 + (rb * a.RBW + rbw) * 4u + (lane & 3u), a.N - 1);
+        const size_t src = (slab_rows + row) * a.gpr + min(g_lo + (lane >> 2) * 4u, a.gpr - 4);
+        o.s = *(const uint2*)((const uint16_t*)a.scales + src);
+        o.b = *(const uint2*)((const uint16_t*)a.biases + src);
+    };
+    auto sbw_store = [&](const SbRegs& o) {
+        if (lane < a.gpw) {  // gpw / 4 vectors for each of the 4 rows
+            float s4[4], b4[4];
+            if constexpr (DT == DT_BF16) {
+                s4[0] = bf16_bits_to_f32(o.s.x & 0xFFFFu); s4[1] = bf16_bits_to_f32(o.s.x >> 16);
+                s4[2] = bf16_bits_to_f32(o.s.y & 0xFFFFu); s4[3] = bf16_bits_to_f32(o.s.y >> 16);
+                b4[0] = bf16_bits_to_f32(o.b.x & 0xFFFFu); b4[1] = bf16_bits_to_f32(o.b.x >> 16);
+                b4[2] = bf16_bits_to_f32(o.b.y & 0xFFFFu); b4[3] = bf16_bits_to_f32(o.b.y >> 16);
+            } else {
+                s4[0] = f16_bits_to_f32(o.s.x & 0xFFFFu); s4[1] = f16_bits_to_f32(o.s.x >> 16);
+                s4[2] = f16_bits_to_f32(o.s.y & 0xFFFFu); s4[3] = f16_bits_to_f32(o.s.y >> 16);
+                b4[0] = f16_bits_to_f32(o.b.x & 0xFFFFu); b4[1] = f16_bits_to_f32(o.b.x >> 16);
+                b4[2] = f16_bits_to_f32(o.b.y & 0xFFFFu); b4[3] = f16_bits_to_f32(o.b.y >> 16);
+            }
+            float4* dst = (float4*)(SB + sbw_off + (lane & 3u) * a.gpw + (lane >> 2) * 4u);
+            dst[0] = make_float4(s4[0], b4[0] - MAGIC * s4[0], s4[1], b4[1] - MAGIC * s4[1]);
+            dst[1] = make_float4(s4[2], b4[2] - MAGIC * s4[2], s4[3], b4[3] - MAGIC * s4[3]);
+        }
+    };
 
     // Address of the 16 bytes this lane loads at step (rb, sg). Steps past the
     // end of a row block or of the wave's work re-read a valid address; what they
@@ -271,7 +312,6 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         // Rows past the pass's last live row are never staged: what the matrix
         // cores compute from their LDS slots lands in output rows nobody stores.
         const uint32_t ntask = live * a.nch;
-        const uint32_t nvec = rows_wg * a.gpr / 4;
         uint32_t raw[NP * 4];
         bool row_live;
         auto x_load = [&](uint32_t task) {
@@ -318,33 +358,10 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                 XL[(((size_t)s * NP + p) * a.nch + c) * MP + i4] = piece;
             }
         };
-        uint2 sv, bv;
-        auto sb_load = [&](uint32_t v) {
-            const uint32_t e = v * 4, rl = e / a.gpr, g = e - rl * a.gpr;
-            const size_t src = (slab_rows + min(row0 + rl, a.N - 1)) * a.gpr + g;
-            sv = *(const uint2*)((const uint16_t*)a.scales + src);
-            bv = *(const uint2*)((const uint16_t*)a.biases + src);
-        };
-        auto sb_store = [&](uint32_t v) {
-            float s4[4], b4[4];
-            if constexpr (DT == DT_BF16) {
-                s4[0] = bf16_bits_to_f32(sv.x & 0xFFFFu); s4[1] = bf16_bits_to_f32(sv.x >> 16);
-                s4[2] = bf16_bits_to_f32(sv.y & 0xFFFFu); s4[3] = bf16_bits_to_f32(sv.y >> 16);
-                b4[0] = bf16_bits_to_f32(bv.x & 0xFFFFu); b4[1] = bf16_bits_to_f32(bv.x >> 16);
-                b4[2] = bf16_bits_to_f32(bv.y & 0xFFFFu); b4[3] = bf16_bits_to_f32(bv.y >> 16);
-            } else {
-                s4[0] = f16_bits_to_f32(sv.x & 0xFFFFu); s4[1] = f16_bits_to_f32(sv.x >> 16);
-                s4[2] = f16_bits_to_f32(sv.y & 0xFFFFu); s4[3] = f16_bits_to_f32(sv.y >> 16);
-                b4[0] = f16_bits_to_f32(bv.x & 0xFFFFu); b4[1] = f16_bits_to_f32(bv.x >> 16);
-                b4[2] = f16_bits_to_f32(bv.y & 0xFFFFu); b4[3] = f16_bits_to_f32(bv.y >> 16);
-            }
-            float4* dst = (float4*)(SB + (size_t)v * 4);
-            dst[0] = make_float4(s4[0], b4[0] - MAGIC * s4[0], s4[1], b4[1] - MAGIC * s4[1]);
-            dst[1] = make_float4(s4[2], b4[2] - MAGIC * s4[2], s4[3], b4[3] - MAGIC * s4[3]);
-        };
-
         x_load(min(tid, ntask - 1));
-        if (pass == 0) sb_load(min(tid, nvec - 1));
+        SbRegs sb_now, sb_next;
+        sbw_load(0, sb_now);
+        if constexpr (REFILL) sbw_load(1, sb_next);
         MTQ_MFMA_KEEP_ORDER();
         for (uint32_t i = 0; i < a.delay; i++) __builtin_amdgcn_s_sleep(8);
         MTQ_MFMA_KEEP_ORDER();
@@ -353,14 +370,8 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         for (int d = 0; d < D; d++) Codec::load(w_ptr(0, d), ring[d]);
         MTQ_MFMA_KEEP_ORDER();
         if (tid < ntask) x_store(tid);
-        if (pass == 0) {
-            if (tid < nvec) sb_store(tid);
-            if (tid == 0) SB[rows_wg * a.gpr] = make_float2(0.f, 0.f);
-            for (uint32_t v = tid + TPB; v < nvec; v += TPB) {
-                sb_load(v);
-                sb_store(v);
-            }
-        }
+        sbw_store(sb_now);
+        if (tid == 0) SB[sb_zero] = make_float2(0.f, 0.f);
         for (uint32_t task = tid + TPB; task < ntask; task += TPB) {
             x_load(task);
             x_store(task);
@@ -383,7 +394,6 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         auto turn = [&](auto issue_tag) {
             constexpr bool ISSUE = decltype(issue_tag)::value;
             const uint32_t row_local = (rb * a.RBW + rbw) * 4u + r;
-            const uint32_t sb_row = row_local * a.gpr;
             {
                 const bool wrap = sg0 + D >= sppD;
                 const uint32_t nrb_i = wrap ? rb + 1 : rb;
@@ -405,7 +415,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                         for (int i = 0; i < MP; i++) xs[s][i] = XS[((size_t)s * a.nch + c) * MP + i];
                     }
                     const uint32_t g = (c * (uint32_t)CPC) >> a.log2g;
-                    const float2 sb = SB[valid ? sb_row + g : rows_wg * a.gpr];
+                    const float2 sb = SB[valid ? sb_row + g : sb_zero];
                     uint32_t pw[Codec::PLANES * (CPC / 2)];
                     Codec::pairs(ring[d], kor, pw);
                     if constexpr (ISSUE) Codec::load(w_ptr(nrb_i, nsg0 + d), ring[d]);
@@ -455,6 +465,12 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                         }
                     rb++;
                     sg0 = 0;
+                    // the window now holds a finished row block: refill it with the next one's pairs,
+                    // loaded one row block ago, and fetch the pairs of the block after that
+                    if constexpr (REFILL) {
+                        sbw_store(sb_next);
+                        if constexpr (ISSUE) sbw_load(rb + 1, sb_next);
+                    }
                 } else {
                     sg0 += D;
                 }
@@ -483,7 +499,8 @@ template <int DT, int BITS, int MP, int S, int MODE>
 int qmv_mfma_launch_one(QmvMArgs& a, const QmvMGeom& g, const LaunchCtx& lc) {
     constexpr int MAXT = (S >= 4 || (S >= 2 && BITS != 4 && BITS != 8)) ? 512 : 1024;
     if (g.tpb > (uint32_t)MAXT) return fail(ERR_UNSUPPORTED, "mfma qmv: workgroup too large for this row count");
-    const void* fn = (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT>;
+    const void* fn = a.nrb > 1 ? (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT, true>
+                               : (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT, false>;
     if (g.shmem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
