@@ -54,6 +54,8 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     const uint32_t cpc = odd ? 32u : 128u / (uint32_t)p.bits, cb = odd ? 4u * (uint32_t)p.bits : 16u;
     const uint64_t rb64 = (uint64_t)p.K * p.bits / 8;
     if (p.K % (16u * cpc) || rb64 > (1u << 24)) return fail(ERR_UNSUPPORTED, "mfma qmv: row is not whole wave-wide segments");
+    if (rb64 * p.N >= (1ull << 32) || (uint64_t)p.N * (p.K / p.group_size) >= (1ull << 31))
+        return fail(ERR_UNSUPPORTED, "mfma qmv: a weight matrix of 4 GiB or more");
     const uint32_t RB = (uint32_t)rb64, nseg = p.K / (16u * cpc), nch = p.K / cpc;
     (void)cb;
     const uint32_t G = p.group_size;

@@ -252,7 +252,12 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
 
     const size_t slab_rows = (size_t)expert * a.N;
     constexpr uint32_t SEGB = 16u * Codec::CB;  // bytes of one weight row covered by a wave-wide load
-    const unsigned char* wbase = a.w + slab_rows * a.RB + (size_t)(kp * a.spp) * SEGB + q * (uint32_t)Codec::CB;
+    // Uniform 64-bit bases (scalar registers) + 32-bit per-lane offsets inside the expert's slab
+    // (the host checks N * RB < 4 GiB): per-lane 64-bit pointers would cost a register pair each.
+    const unsigned char* wslab = a.w + slab_rows * a.RB;
+    const uint16_t* sslab = (const uint16_t*)a.scales + slab_rows * a.gpr;
+    const uint16_t* bslab = (const uint16_t*)a.biases + slab_rows * a.gpr;
+    const uint32_t woff = (kp * a.spp) * SEGB + q * (uint32_t)Codec::CB;
     const uint32_t sppD = (a.spp + D - 1) / D * D;  // steps per row block, padded to whole rings
     // (scale, bias) pairs: every wave keeps those of its own 4 rows and its own K part in its own
     // LDS window and refills it when it moves to the next row block, so the number of row blocks
@@ -263,12 +268,12 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     // Lane l refills 4 pairs of the window: row l & 3, groups g_lo + 4 * (l >> 2) .. + 3 (gpw <= 64, so
     // one 8-byte load of scales and one of biases per lane and refill).
     struct SbRegs { uint2 s, b; };
-    auto sbw_load = [&](uint32_t rb, SbRegs& o) {
+    auto sbw_load = [&](uint32_t rb, SbRegs& o, uint32_t nudge = 0u) {  // nudge: an opaque zero, see the pass loop
         rb = min(rb, a.nrb - 1);
         const uint32_t row = min(row0 + (rb * a.RBW + rbw) * 4u + (lane & 3u), a.N - 1);
-        const size_t src = (slab_rows + row) * a.gpr + min(g_lo + (lane >> 2) * 4u, a.gpr - 4);
-        o.s = *(const uint2*)((const uint16_t*)a.scales + src);
-        o.b = *(const uint2*)((const uint16_t*)a.biases + src);
+        const uint32_t src = row * a.gpr + min(g_lo + (lane >> 2) * 4u, a.gpr - 4) + nudge;
+        o.s = *(const uint2*)(sslab + src);
+        o.b = *(const uint2*)(bslab + src);
     };
     auto sbw_store = [&](const SbRegs& o) {
         if (lane < a.gpw) {  // gpw / 4 vectors for each of the 4 rows
@@ -293,11 +298,11 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     // Address of the 16 bytes this lane loads at step (rb, sg). Steps past the
     // end of a row block or of the wave's work re-read a valid address; what they
     // load is multiplied by a zero scale.
-    auto w_ptr = [&](uint32_t rb, uint32_t sg) -> const unsigned char* {
+    auto w_ptr = [&](uint32_t rb, uint32_t sg, uint32_t nudge = 0u) -> const unsigned char* {
         rb = min(rb, a.nrb - 1);
         sg = min(sg, a.spp - 1);
         const uint32_t row = min(row0 + (rb * a.RBW + rbw) * 4u + r, a.N - 1);
-        return wbase + (size_t)row * a.RB + (size_t)sg * SEGB;
+        return wslab + (uint32_t)(row * a.RB + sg * SEGB + woff + nudge);
     };
 
     const uint32_t n_pass = (MODE == GATHER_CSR || MODE == GATHER_INDICES) ? (cnt + R - 1) / R : 1u;
@@ -358,21 +363,26 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                 XL[(((size_t)s * NP + p) * a.nch + c) * MP + i4] = piece;
             }
         };
-        x_load(min(tid, ntask - 1));
+        // In the gather modes this body is a loop over passes. Index math of the staging and of the
+        // final store is cheap but would be hoisted out of that loop and then held in registers
+        // all through the streaming; an opaque copy of the thread id keeps it inside.
+        uint32_t ptid = tid, pzero = 0u;
+        if constexpr (MODE == GATHER_CSR || MODE == GATHER_INDICES) asm volatile("" : "+v"(ptid), "+v"(pzero));
+        x_load(min(ptid, ntask - 1));
         SbRegs sb_now, sb_next;
-        sbw_load(0, sb_now);
-        if constexpr (REFILL) sbw_load(1, sb_next);
+        sbw_load(0, sb_now, pzero);
+        if constexpr (REFILL) sbw_load(1, sb_next, pzero);
         MTQ_MFMA_KEEP_ORDER();
         for (uint32_t i = 0; i < a.delay; i++) __builtin_amdgcn_s_sleep(8);
         MTQ_MFMA_KEEP_ORDER();
         uint32_t ring[D][NWD];
 #pragma unroll
-        for (int d = 0; d < D; d++) Codec::load(w_ptr(0, d), ring[d]);
+        for (int d = 0; d < D; d++) Codec::load(w_ptr(0, d, pzero), ring[d]);
         MTQ_MFMA_KEEP_ORDER();
-        if (tid < ntask) x_store(tid);
+        if (ptid < ntask) x_store(ptid);
         sbw_store(sb_now);
         if (tid == 0) SB[sb_zero] = make_float2(0.f, 0.f);
-        for (uint32_t task = tid + TPB; task < ntask; task += TPB) {
+        for (uint32_t task = ptid + TPB; task < ntask; task += TPB) {
             x_load(task);
             x_store(task);
         }
@@ -482,7 +492,9 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         __syncthreads();
 
         // ---- add the K parts and store ----------------------------------------
-        for (uint32_t idx = tid; idx < rows_wg * live; idx += TPB) {
+        uint32_t stid = tid;
+        if constexpr (MODE == GATHER_CSR || MODE == GATHER_INDICES) asm volatile("" : "+v"(stid));
+        for (uint32_t idx = stid; idx < rows_wg * live; idx += TPB) {
             const uint32_t i = idx / rows_wg, rl = idx - i * rows_wg;
             const uint32_t row = row0 + rl;
             if (row >= a.N) continue;
