@@ -50,8 +50,8 @@ struct State {
     hipStream_t stream = nullptr;  // stream in use (own_stream or the caller's)
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     void* flush_buf = nullptr;
-    void* norm_buf = nullptr;     // library-owned scratch: normalised rows, qvm partial sums
-    size_t norm_bytes = 0;
+    void* scratch_buf = nullptr;     // library-owned scratch: normalised rows, qvm partial sums
+    size_t scratch_bytes = 0;
     size_t flush_bytes = 0;
     hipDeviceProp_t prop;
     bool timed_armed = false;    // next typed launch attaches the events
@@ -153,16 +153,16 @@ static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s,
 
 // Library-owned device scratch (normalised rows, qvm partial sums): grown on demand, never shrunk.
 static int ensure_scratch(size_t need) {
-    if (g.norm_bytes >= need) return ERR_OK;
-    if (g.norm_buf) {
+    if (g.scratch_bytes >= need) return ERR_OK;
+    if (g.scratch_buf) {
         MTQ_HIP(hipStreamSynchronize(g.stream));  // earlier launches may still use the old buffer
-        MTQ_HIP(hipFree(g.norm_buf));
-        g.norm_buf = nullptr;
-        g.norm_bytes = 0;
+        MTQ_HIP(hipFree(g.scratch_buf));
+        g.scratch_buf = nullptr;
+        g.scratch_bytes = 0;
     }
     const size_t cap = need < 65536 ? 65536 : need;
-    MTQ_HIP(hipMalloc(&g.norm_buf, cap));
-    g.norm_bytes = cap;
+    MTQ_HIP(hipMalloc(&g.scratch_buf, cap));
+    g.scratch_bytes = cap;
     return ERR_OK;
 }
 
@@ -180,7 +180,7 @@ static int op_qvm(int dtype, int bits, uint32_t G, const void* w, const void* s,
     QmvParams p;
     p.dtype = dtype; p.bits = bits; p.group_size = G; p.w = w; p.scales = s; p.biases = b; p.x = x; p.out = out;
     p.M = M; p.N = N; p.K = K;
-    return launch_qvm(p, g.norm_buf, lc);
+    return launch_qvm(p, g.scratch_buf, lc);
 }
 
 // RMSNorm fused into qmv: inside the streaming kernel when the row fits it, else the
@@ -207,11 +207,11 @@ static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const
     first.stop = nullptr;
     mid.start = mid.stop = nullptr;
     last.start = nullptr;
-    rc = launch_rms_norm(dtype, x, norm_w, eps, g.norm_buf, K, first);
+    rc = launch_rms_norm(dtype, x, norm_w, eps, g.scratch_buf, K, first);
     if (rc) return rc;
-    if (rows == 1) return op_qmv(dtype, bits, G, w, s, b, g.norm_buf, out, 1, N, K, last);
-    char* part = (char*)g.norm_buf + x_bytes;
-    rc = op_qmv(dtype, bits, G, w, s, b, g.norm_buf, part, 2, N, K, mid);
+    if (rows == 1) return op_qmv(dtype, bits, G, w, s, b, g.scratch_buf, out, 1, N, K, last);
+    char* part = (char*)g.scratch_buf + x_bytes;
+    rc = op_qmv(dtype, bits, G, w, s, b, g.scratch_buf, part, 2, N, K, mid);
     if (rc) return rc;
     return launch_add_rows(dtype, part, part + (size_t)N * sz, out, N, last);
 }
@@ -661,9 +661,9 @@ int mtq_shutdown(void) {
     if (!g.ready) return MTQ_OK;
     (void)hipStreamSynchronize(g.stream);
     if (g.flush_buf) (void)hipFree(g.flush_buf);
-    if (g.norm_buf) (void)hipFree(g.norm_buf);
-    g.norm_buf = nullptr;
-    g.norm_bytes = 0;
+    if (g.scratch_buf) (void)hipFree(g.scratch_buf);
+    g.scratch_buf = nullptr;
+    g.scratch_bytes = 0;
     if (g.ev_start) (void)hipEventDestroy(g.ev_start);
     if (g.ev_stop) (void)hipEventDestroy(g.ev_stop);
     if (g.own_stream) (void)hipStreamDestroy(g.own_stream);
