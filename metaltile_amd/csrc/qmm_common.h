@@ -57,15 +57,18 @@ __device__ __forceinline__ uint4 dequant8(const uint32_t* wr, int i, float s, fl
     float v[8];
     if constexpr (BITS == 4) {
         const uint32_t w = wr[i];
-        uint32_t e = w & 0x0F0F0F0Fu, o = (w >> 4) & 0x0F0F0F0Fu;
-        // Opaque to the optimiser: it would otherwise fold the masks into one bit-field extract per
-        // code and then convert byte 0; kept as they are, the byte-select converts (v_cvt_f32_ubyte0..3)
-        // take the codes straight out of `e` and `o`: 3 + 8 instead of ~15 instructions per dword.
+        // Even codes sit in the low nibbles of the four bytes, odd codes in the high nibbles. The high
+        // nibbles are converted where they are (as 16 * q) and multiplied by s / 16, which is exact, so
+        // no shift is needed. The masked copies are opaque to the optimiser: it would otherwise fold the
+        // masks into one bit-field extract per code and then convert byte 0; kept as they are, the
+        // byte-select converts (v_cvt_f32_ubyte0..3) take the codes straight out of `e` and `o`.
+        uint32_t e = w & 0x0F0F0F0Fu, o = w & 0xF0F0F0F0u;
         asm volatile("" : "+v"(e), "+v"(o));
+        const float s16 = s * 0.0625f;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             v[2 * j] = fmaf((float)((e >> (8 * j)) & 0xFFu), s, b);
-            v[2 * j + 1] = fmaf((float)((o >> (8 * j)) & 0xFFu), s, b);
+            v[2 * j + 1] = fmaf((float)((o >> (8 * j)) & 0xFFu), s16, b);
         }
     } else if constexpr (BITS == 8) {
 #pragma unroll
