@@ -199,8 +199,9 @@ MTQ_API int mtq_moe_router_topk(int dtype, const void *router_logits, uint32_t *
  * inv_perm u32[n_tokens, k] (sorted row of each entry: input of mtq_moe_unpermute) and
  * expert_offsets u32[n_experts + 1] (CSR bounds: input of mtq_gather_qmv_csr). The reference has
  * no kernel for this step: its callers sort on the host (crates/metaltile-std/src/ffai/moe.rs:
- * 256-275 describes the two permutations). At most 32768 entries; expert ids >= n_experts are
- * treated as n_experts - 1. */
+ * 256-275 describes the two permutations). Up to 2048 experts: any number of entries (counting
+ * sort); more experts: at most 32768 entries (sorting network). Expert ids >= n_experts are treated
+ * as n_experts - 1. */
 MTQ_API int mtq_moe_sort_by_expert(const uint32_t *indices, uint32_t n_tokens, uint32_t k, uint32_t n_experts,
                                    uint32_t *sort_token_idx, uint32_t *inv_perm, uint32_t *expert_offsets);
 

@@ -1064,6 +1064,11 @@ int mtq_set_option(const char* name, int value) {
         options().qmv_rows_per_thread = value;
         return MTQ_OK;
     }
+    if (!strcmp(name, "moe.sort")) {
+        if (value < 0 || value > 1) return fail(ERR_BAD_ARG, "moe.sort must be 0 (automatic) or 1 (bitonic network)");
+        options().moe_sort = value;
+        return MTQ_OK;
+    }
     if (!strcmp(name, "qvm.wgs")) {
         if (value < 0 || value > 65536) return fail(ERR_BAD_ARG, "qvm.wgs must be in 0..65536");
         options().qvm_wgs = value;

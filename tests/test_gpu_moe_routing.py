@@ -92,7 +92,8 @@ def test_router_rejects_bad_shapes():
     b.free()
 
 
-@pytest.mark.parametrize("T,k,E", [(1, 8, 128), (16, 2, 8), (37, 6, 60), (512, 8, 128), (4096, 8, 128), (3, 1, 1), (100, 4, 1024)])
+@pytest.mark.parametrize("T,k,E", [(1, 8, 128), (16, 2, 8), (37, 6, 60), (512, 8, 128), (4096, 8, 128), (3, 1, 1), (100, 4, 1024),
+                                   (10000, 8, 128), (700, 3, 2048), (1000, 8, 4096), (129, 8, 1), (20000, 2, 7)])
 def test_sort_by_expert(oracle, T, k, E):
     print(f"[case] moe_sort T={T} k={k} E={E}", flush=True)
     rng = np.random.default_rng(T + k + E)
@@ -108,10 +109,30 @@ def test_sort_by_expert(oracle, T, k, E):
         b.free()
 
 
+def test_sort_network_equals_counting_sort(oracle):
+    """Both device sorts give the oracle's permutation (the counting sort serves up to 2048 experts,
+    the network up to 32768 entries)."""
+    from metaltile_amd.runtime import _ensure_init
+    lib = _ensure_init()
+    T, k, E = 2000, 8, 128
+    idx = np.random.default_rng(4).integers(0, E, T * k).astype("<u4")
+    rsti, rinv, roffs = oracle.moe_sort_by_expert(idx, T, k, E)
+    di = GpuBuffer.from_bytes(idx.tobytes())
+    for mode in (1, 0):
+        assert lib.mtq_set_option(b"moe.sort", mode) == 0
+        sti, inv, offs = GpuBuffer(T * k * 4), GpuBuffer(T * k * 4), GpuBuffer((E + 1) * 4)
+        ops.moe_sort_by_expert(di, T, k, E, sti, inv, offs)
+        assert np.array_equal(_u32(sti, T * k), rsti) and np.array_equal(_u32(inv, T * k), rinv)
+        assert np.array_equal(_u32(offs, E + 1), roffs)
+        for b in (sti, inv, offs):
+            b.free()
+    di.free()
+
+
 def test_sort_limits():
     b = GpuBuffer(1 << 20)
     with pytest.raises(MtqError):
-        ops.moe_sort_by_expert(b, 4097, 8, 128, b, b, b)   # 32776 entries
+        ops.moe_sort_by_expert(b, 4097, 8, 4096, b, b, b)   # 32776 entries and more experts than the counting sort takes
     ops.moe_sort_by_expert(b, 0, 8, 4, b, b, b)             # no entries: offsets all zero
     assert _u32(b, 5).tolist() == [0, 0, 0, 0, 0]
     b.free()
