@@ -1112,7 +1112,7 @@ int mtq_set_option(const char* name, int value) {
         return MTQ_OK;
     }
     if (!strcmp(name, "qmm.kgroups")) {
-        if (value != 0 && value != 2 && value != 4) return fail(ERR_BAD_ARG, "qmm.kgroups must be 0, 2 or 4");
+        if (value != 0 && value != 1 && value != 2 && value != 4) return fail(ERR_BAD_ARG, "qmm.kgroups must be 0, 1, 2 or 4");
         options().qmm_kgroups = value;
         return MTQ_OK;
     }

@@ -62,19 +62,24 @@ struct QmmDArgs {
 // (coalesced, one line per row) instead of being fetched per lane and iteration:
 // a wave-wide 2-byte load from 32 different rows costs the L1 as many tag lookups
 // as the weight load itself.
-// KG: K-groups per workgroup (2 or 4). The 8 waves are KG K-groups x 8/KG N-waves;
+// KG: K-groups per workgroup (1, 2 or 4). For 2 and 4 the 8 waves are KG K-groups x 8/KG N-waves;
 // the tile is 32*MB rows x 32*(8/KG) columns and an iteration covers 64*KG k. KG = 4
 // halves the tile width, which doubles the number of 128-row tiles for small M.
+// KG = 1 is the half-size workgroup: 4 waves, all N-waves of one K-group, 32*MB x 128 tile,
+// 64 k per iteration and no partial sums to combine. Two such workgroups share a compute unit
+// and are not in step with each other, so one's LDS traffic runs under the other's MFMAs.
 template <int DT, int BITS, int PD, int MB, bool SBL, int KG>
-__global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
-    constexpr int NWV = 8 / KG;              // N-waves
+__global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArgs a) {
+    constexpr int NW = KG == 1 ? 4 : 8;      // waves
+    constexpr int NT = 64 * NW;              // threads
+    constexpr int NWV = NW / KG;             // N-waves
     constexpr int DBN = 32 * NWV, DBK = 64 * KG;
     constexpr int DLD = DBK * 2 + 16;        // LDS row stride in bytes
     constexpr int TPR = DBK * 2 / 32;        // threads per activation row (32 bytes each)
-    constexpr int RS = 512 / TPR;            // rows covered by one pass of the workgroup
+    constexpr int RS = NT / TPR;            // rows covered by one pass of the workgroup
     constexpr int DBM = 32 * MB;
     constexpr int DBUF = DBM * DLD;          // one activation tile
-    constexpr int XV = DBM * DBK * 2 / 512 / 16;  // 16-byte vectors of the tile per thread
+    constexpr int XV = DBM * DBK * 2 / NT / 16;  // 16-byte vectors of the tile per thread
     extern __shared__ __align__(16) unsigned char lds[];  // 2 * DBUF bytes
     // the epilogue needs DBM*DBN*(4+2) bytes: partial sums, then the element tile (checked on the host)
 
@@ -172,7 +177,7 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
         // DBN rows x gpr elements each of scales and biases, 16 bytes per load: vector v of
         // the tile covers elements [8*(v % vpr), +8) of row v / vpr
         const uint32_t vpr = a.gpr / 8, nvec = DBN * vpr;
-        for (uint32_t v = tid; v < nvec; v += 512) {
+        for (uint32_t v = tid; v < nvec; v += NT) {
             const uint32_t row = v / vpr, c0 = (v - row * vpr) * 8;
             const q_u32x4 sv = *(const q_u32x4*)((const uint16_t*)a.scales + (size_t)(n0 + row) * a.gpr + c0);
             const q_u32x4 bv = *(const q_u32x4*)((const uint16_t*)a.biases + (size_t)(n0 + row) * a.gpr + c0);
@@ -288,12 +293,12 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
             }
     }
     __syncthreads();
-    // all 512 threads store the tile, 16 bytes each, whole rows
+    // all threads store the tile, 16 bytes each, whole rows
     constexpr int VPR = DBN / 8;                    // 16-byte vectors per tile row
-    constexpr int VPT = DBM * VPR / 512;            // vectors per thread
+    constexpr int VPT = DBM * VPR / NT;            // vectors per thread
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
-        const uint32_t v = tid + i * 512, lrow = v / VPR, c16 = v % VPR;
+        const uint32_t v = tid + i * NT, lrow = v / VPR, c16 = v % VPR;
         const uint32_t row = m0 + lrow;
         if (row < a.M)
             *(q_u32x4*)((uint16_t*)a.out + (size_t)row * a.N + n0 + c16 * 8) = *(const q_u32x4*)(otile + lrow * DBN + c16 * 8);
@@ -303,7 +308,7 @@ __global__ __launch_bounds__(512) void qmm_direct_kernel(QmmDArgs a) {
 // LDS of one workgroup: two activation tiles, the tile's scales and biases, and at the
 // end the K-groups' partial sums followed by the element tile.
 static size_t lds_need(uint32_t rows, uint32_t kg, uint32_t gpr, bool sbl) {
-    const uint32_t dbn = 32 * (8 / kg), dbk = 64 * kg;
+    const uint32_t dbn = kg == 1 ? 128 : 32 * (8 / kg), dbk = 64 * kg;
     size_t main_loop = 2 * (size_t)rows * (dbk * 2 + 16) + (sbl ? (size_t)2 * dbn * (gpr + 2) * 2 : 0);
     size_t epilogue = (size_t)(kg - 1) * rows * dbn * 4 + (size_t)rows * dbn * 2;
     return main_loop > epilogue ? main_loop : epilogue;
@@ -312,13 +317,16 @@ static size_t lds_need(uint32_t rows, uint32_t kg, uint32_t gpr, bool sbl) {
 template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, const LaunchCtx& lc) {
     const void* fn;
     const bool tall = a.m_tile_rows == 128;
-    const uint32_t dbn = 32 * (8 / kgroups);
+    const uint32_t dbn = kgroups == 1 ? 128 : 32 * (8 / kgroups);
     // scales and biases of the tile's rows in LDS when they fit beside the activation tiles
     const bool sbl = a.gpr % 8 == 0 && (size_t)2 * dbn * (a.gpr + 2) * 2 <= 48 * 1024;
     const size_t shmem = lds_need(a.m_tile_rows, kgroups, a.gpr, sbl);
     if (shmem > 160 * 1024) return fail(ERR_UNSUPPORTED, "direct qmm: tile does not fit in LDS");
 #define QD_PICK3(B, MBv, KGv) (sbl ? (const void*)qmm_direct_kernel<DT, B, 2, MBv, true, KGv> : (const void*)qmm_direct_kernel<DT, B, 2, MBv, false, KGv>)
-#define QD_PICK(B) fn = kgroups == 4 ? (tall ? QD_PICK3(B, 4, 4) : QD_PICK3(B, 2, 4)) : (tall ? QD_PICK3(B, 4, 2) : QD_PICK3(B, 2, 2))
+#define QD_PICK(B)                                                                      \
+    fn = kgroups == 4   ? (tall ? QD_PICK3(B, 4, 4) : QD_PICK3(B, 2, 4))                \
+         : kgroups == 1 ? (tall ? QD_PICK3(B, 4, 1) : QD_PICK3(B, 2, 1))                \
+                        : (tall ? QD_PICK3(B, 4, 2) : QD_PICK3(B, 2, 2))
     switch (bits) {
         case 2: QD_PICK(2); break;
         case 4: QD_PICK(4); break;
@@ -329,7 +337,7 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     void* args[] = {&a};
-    e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles), dim3(512), args, shmem, lc);
+    e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles), dim3(kgroups == 1 ? 256 : 512), args, shmem, lc);
     if (e != hipSuccess) return hip_fail(e, "qmm direct kernel launch");
     return ERR_OK;
 }
@@ -367,13 +375,14 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
     const uint64_t tall_wide = (uint64_t)((p.M + 127) / 128) * (p.N / 128);
     const uint64_t short_wide = (uint64_t)((p.M + 63) / 64) * (p.N / 128);
     uint32_t rows = 64, kgroups = 2;
-    if (tall_wide >= (uint64_t)cus) { rows = 128; kgroups = 2; }
+    if (tall_wide >= 2 * (uint64_t)cus) { rows = 128; kgroups = 1; }  // two 4-wave workgroups per CU (M = 2048: 72-75 us against 80-84; M = 4096: 160-170 against 180-190)
+    else if (tall_wide >= (uint64_t)cus) { rows = 128; kgroups = 2; }
     else if (short_wide * 2 <= (uint64_t)cus) { rows = 64; kgroups = 4; }  // few tiles: halve their width
     if (options().qmm_tile_rows) rows = (uint32_t)options().qmm_tile_rows;
     if (options().qmm_kgroups) kgroups = (uint32_t)options().qmm_kgroups;
     a.m_tile_rows = rows;
     a.m_tiles = (p.M + rows - 1) / rows;
-    a.n_tiles = p.N / (32 * (8 / kgroups));
+    a.n_tiles = p.N / (kgroups == 1 ? 128 : 32 * (8 / kgroups));
     a.iters = p.K / (64 * kgroups);  // even: K % 512 == 0
     return p.dtype == DT_BF16 ? launch_dt<DT_BF16>(a, p.bits, kgroups, lc) : launch_dt<DT_F16>(a, p.bits, kgroups, lc);
 }

@@ -1,0 +1,53 @@
+"""Every tiling of the direct matrix-core qmm kernel (K-groups 1, 2, 4 x tile heights 64,
+128), forced through the library's options on one ragged shape, against the oracle's
+restatement of the reference's mma semantics (weights rounded to the element dtype
+before the multiply, crates/metaltile-std/src/mlx/quantized.rs:2267-2274).
+Tolerance: 2e-2 on max|a-e| / max(|e|, 1), the bound of the bf16 prefill configuration;
+bit-equal results between tilings are not required (partial sums meet in a different order)."""
+import numpy as np
+import pytest
+
+from metaltile_amd import DType, GpuBuffer, _lib, ops, unpack_f32
+from metaltile_amd.synth import make_case
+from tests.parity import rel_err
+
+pytestmark = pytest.mark.gpu
+
+ODT = {DType.F16: 1, DType.BF16: 2}
+
+
+@pytest.fixture
+def options():
+    lib = _lib.load()
+
+    def set_(name, value):
+        assert lib.mtq_set_option(name.encode(), value) == 0, name
+
+    yield set_
+    for name in ("qmm.kernel", "qmm.kgroups", "qmm.tile_rows"):
+        lib.mtq_set_option(name.encode(), 0)
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16])
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_direct_qmm_every_tiling(oracle, options, bits, dt):
+    M, N, K, G = 200, 256, 1024, 64          # last 128-row and 64-row tiles are ragged
+    c = make_case(5100 + bits, dt, bits, G, M, N, K)
+    exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    options("qmm.kernel", 2)
+    for kg in (1, 2, 4):
+        for rows in (64, 128):
+            print(f"[case] direct qmm {dt.name} b{bits} kgroups={kg} tile_rows={rows}", flush=True)
+            options("qmm.kgroups", kg)
+            options("qmm.tile_rows", rows)
+            out = GpuBuffer(M * N * dt.size_bytes)
+            ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+            got = unpack_f32(out.read_bytes(), dt)
+            out.free()
+            err = rel_err(got, exp)
+            assert err <= 2e-2, f"kgroups={kg} rows={rows}: rel err {err:.3e}"
+    for buf in (w, s, b, x):
+        buf.free()
