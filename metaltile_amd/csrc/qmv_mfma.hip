@@ -112,54 +112,68 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
         if (p.bits == 2 && s > 2) s = 2;  // the 16-row 2-bit variant does not fit the register file
         if (opt.qmv_mfma_sets) s = opt.qmv_mfma_sets;
     }
-    const uint32_t maxt = (s >= 4 || (s >= 2 && p.bits != 4 && p.bits != 8)) ? 512u : 1024u;
-    if (64u * KP > maxt) return fail(ERR_UNSUPPORTED, "mfma qmv: too many K parts");
-    // Rows per workgroup: about one to two workgroups per compute unit (measured
-    // best on 14336x4096, 4096x14336 and 8192x8192), as many of the row blocks
-    // side by side as the workgroup size allows, the rest one after the other.
-    uint32_t rows_target = 8;
-    while (rows_target < 32 && (uint64_t)rows_target * 2 * 256 <= p.N) rows_target *= 2;
+    // Rows per workgroup. Every workgroup stages all activation rows of a pass (R x K elements)
+    // before it streams, so the weight rows are dealt to one workgroup per compute unit, as many of
+    // its row blocks side by side as the workgroup size allows, the rest one after the other.
+    // Measured with 8 activation rows, 4-bit bf16: 128256x4096 63 us at 251 workgroups against
+    // 129 us at 4008; 57344x4096 33 against 57; 14336x4096 12.8 against 16.8.
+    // A gather workgroup additionally should live long: as many row blocks one after the other as
+    // leave one workgroup (two when 4 rows are staged) per CU over the experts that can be hit.
+    // Measured on 8 experts x 14336x4096, 32 rows: 61 us with 7 row blocks of 64 rows per
+    // workgroup, 74 us with 4, 98 us with 14. Short rows (few steps per row block) want the row
+    // blocks one after the other in a narrow workgroup rather than side by side in a wide one: at
+    // least 16 steps per wave (E = 128 x 256x2048 with one row per expert: 15 us with 2 blocks side
+    // by side x 4 in sequence, 30 us with 16 side by side).
+    // When the staged rows leave too little LDS: a narrower workgroup with the row blocks moved one
+    // after the other (the number of workgroups stays) down to 8 waves, which a CU needs to keep
+    // enough loads in flight (28672x8192, 8 rows: 100 us with 4-wave workgroups in one pass, 54 us
+    // in two passes of 16-wave ones); then up to half the rows per workgroup; then half the
+    // activation rows per pass, planned afresh, although every further pass streams the weights again.
     const uint32_t rbw_cap = 16u;
-    uint32_t RBW = rows_target / 4 < rbw_cap ? rows_target / 4 : rbw_cap;
-    while (64u * KP * RBW > maxt && RBW > 1) RBW /= 2;
-    uint32_t nrb = rows_target / 4 / RBW;
-    if (gather) {
-        // A gather workgroup stages up to R activation rows of K elements before it streams, so it
-        // should live long: the largest workgroup the instance allows, and as many row blocks one
-        // after the other as leave one workgroup (two when 4 rows are staged) per CU over the
-        // experts that can be hit. Measured on 8 experts x 14336x4096, 32 rows: 61 us with 7 row
-        // blocks of 64 rows per workgroup, 74 us with 4, 98 us with 14.
-        // Short rows (few steps per row block) want the row blocks one after the other in a
-        // narrow workgroup rather than side by side in a wide one: at least 16 steps per wave
-        // (E = 128 x 256x2048 with one row per expert: 15 us with 2 blocks side by side x 4 in
-        // sequence, 30 us with 16 side by side).
-        const uint64_t e_eff = p.E < rows ? p.E : rows;
-        const uint64_t slots = (uint64_t)num_cus_mfma() * (s == 1 ? 2 : 1);
-        const uint64_t units = ((uint64_t)p.N + 3) / 4 * e_eff;              // 4-row blocks over the experts that can be hit
-        uint64_t per_wg = (units + slots - 1) / slots;                       // blocks per workgroup
-        const uint64_t max_per_wg = ((uint64_t)p.N + 3) / 4;
-        if (per_wg > max_per_wg) per_wg = max_per_wg;
-        const uint32_t min_nrb = spp >= 16 ? 1u : (16u + spp - 1) / spp;
+    const uint32_t list_cap = p.gather == GATHER_INDICES ? p.T : 0;
+    uint32_t RBW = 1, nrb = 1;
+    for (;; s /= 2) {
+        const uint32_t maxt = (s >= 4 || (s >= 2 && p.bits != 4 && p.bits != 8)) ? 512u : 1024u;
+        if (64u * KP > maxt) {
+            if (s > 1) continue;
+            return fail(ERR_UNSUPPORTED, "mfma qmv: too many K parts");
+        }
         uint32_t rbw_max = rbw_cap;
         while (64u * KP * rbw_max > maxt && rbw_max > 1) rbw_max /= 2;
-        RBW = 1;
-        while (RBW * 2 <= rbw_max && (uint64_t)RBW * 2 * min_nrb <= per_wg) RBW *= 2;
-        nrb = (uint32_t)((per_wg + RBW - 1) / RBW);
-        if (nrb < 1) nrb = 1;
-        if (nrb > 64) nrb = 64;
-    }
-    if (opt.qmv_mfma_rbw) {
-        RBW = (uint32_t)opt.qmv_mfma_rbw;
-        if (64u * KP * RBW > maxt) return fail(ERR_BAD_ARG, "qmv.mfma_rbw: workgroup too large");
-    }
-    if (opt.qmv_mfma_nrb) nrb = (uint32_t)opt.qmv_mfma_nrb;
-    const uint32_t list_cap = p.gather == GATHER_INDICES ? p.T : 0;
-    // shrink until the workgroup's LDS fits
-    while (lds_bytes((uint32_t)(mp * s), p.K, nch, 4 * RBW * nrb, KP * RBW, gpw, KP, list_cap) > kLdsBudget) {
-        if (nrb > 1) nrb--;
-        else if (s > 1) s /= 2;
-        else if (RBW > 1) RBW--;
-        else return fail(ERR_UNSUPPORTED, "mfma qmv: activations do not fit in LDS");
+        const uint64_t blocks = ((uint64_t)p.N + 3) / 4;  // 4-row blocks of one matrix
+        if (gather) {
+            const uint64_t e_eff = p.E < rows ? p.E : rows;
+            const uint64_t slots = (uint64_t)num_cus_mfma() * (s == 1 ? 2 : 1);
+            uint64_t per_wg = (blocks * e_eff + slots - 1) / slots;
+            if (per_wg > blocks) per_wg = blocks;
+            const uint32_t min_nrb = spp >= 16 ? 1u : (16u + spp - 1) / spp;
+            RBW = 1;
+            while (RBW * 2 <= rbw_max && (uint64_t)RBW * 2 * min_nrb <= per_wg) RBW *= 2;
+            const uint64_t n = (per_wg + RBW - 1) / RBW;
+            nrb = n > 64 ? 64u : (n < 1 ? 1u : (uint32_t)n);
+        } else {
+            const uint64_t slots = (uint64_t)num_cus_mfma();
+            const uint64_t per_wg = (blocks + slots - 1) / slots;
+            RBW = 1;
+            while (RBW < rbw_max && RBW < per_wg) RBW *= 2;
+            const uint64_t n = (per_wg + RBW - 1) / RBW;
+            nrb = n > 64 ? 64u : (uint32_t)n;
+        }
+        if (opt.qmv_mfma_rbw) {
+            RBW = (uint32_t)opt.qmv_mfma_rbw;
+            if (64u * KP * RBW > maxt) return fail(ERR_BAD_ARG, "qmv.mfma_rbw: workgroup too large");
+        }
+        if (opt.qmv_mfma_nrb) nrb = (uint32_t)opt.qmv_mfma_nrb;
+        auto need = [&]() { return lds_bytes((uint32_t)(mp * s), p.K, nch, 4 * RBW * nrb, KP * RBW, gpw, KP, list_cap); };
+        const uint32_t nrb_planned = nrb;
+        const bool last = s == 1;  // nothing left to halve: shrink as far as it takes
+        while (need() > kLdsBudget) {
+            if (RBW > 1 && !opt.qmv_mfma_rbw && (last || KP * RBW / 2 >= 8)) { RBW /= 2; nrb = nrb * 2 > 64 ? 64 : nrb * 2; }
+            else if (nrb > 1 && (last || nrb * 2 > nrb_planned)) nrb--;
+            else break;
+        }
+        if (need() <= kLdsBudget) break;
+        if (last) return fail(ERR_UNSUPPORTED, "mfma qmv: activations do not fit in LDS");
     }
     const uint32_t R = (uint32_t)(mp * s);
     if (p.gather == GATHER_NONE && rows_per_launch > R) rows_per_launch = R;
