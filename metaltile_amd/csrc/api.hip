@@ -127,8 +127,12 @@ static int op_qmv(int dtype, int bits, uint32_t G, const void* w, const void* s,
 }
 
 // Kernel routing by M, the counterpart of mt_qmm_for
-// (crates/metaltile-std/src/mlx/quantized.rs:5040-5065): the MFMA tile kernel from M = 16
-// up, the GEMV family below that.
+// (crates/metaltile-std/src/mlx/quantized.rs:5040-5065, which sends M = 16 and the multiples
+// of 32 to its MMA kernels). Here the GEMV family takes 8 activation rows per pass over the
+// weights, so it serves up to 8 rows; the MFMA tile kernel takes over from 17 rows (a third
+// pass always loses: N = K = 4096, 20 rows, 17.5 us against 16.0) and, where the matrix has
+// enough column tiles to fill the chip with one row of tiles (N >= 8192), from 9 rows
+// (14336x4096, 12 rows: 22.7 us against 18.0; 4096x14336 stays: 38.6 against 59).
 static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s, const void* b,
                   const void* x, void* out, uint32_t M, uint32_t N, uint32_t K, bool force_mma,
                   const LaunchCtx& lc) {
@@ -136,7 +140,7 @@ static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s,
     if (rc) return rc;
     if (M == 0) return ERR_OK;
     if (!w || !s || !b || !x || !out) return fail(ERR_BAD_ARG, "null buffer");
-    if (M >= 32 || force_mma) {
+    if (M >= 17 || (M >= 9 && N >= 8192) || force_mma) {
         QmmParams q;
         q.dtype = dtype; q.bits = bits; q.group_size = G;
         q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;

@@ -51,3 +51,25 @@ def test_direct_qmm_every_tiling(oracle, options, bits, dt):
             assert err <= 2e-2, f"kgroups={kg} rows={rows}: rel err {err:.3e}"
     for buf in (w, s, b, x):
         buf.free()
+
+
+@pytest.mark.parametrize("N", [256, 8192])
+@pytest.mark.parametrize("M", [9, 16, 17, 31])
+def test_qmm_routing_between_8_and_32_rows(oracle, M, N):
+    """9..31 activation rows go to the GEMV family (exact dequantisation) or to the tile kernel
+    (weights rounded to bf16 first) depending on M and N; either way the result stays within the
+    reference's bf16 bound against exact dequantisation, 5e-2 on max|a-e| / max(|e|, 1)
+    (crates/metaltile-std/tests/qmm_gpu_correctness.rs:2085-2106)."""
+    K, G, bits, dt = 1024, 64, 4, DType.BF16
+    print(f"[case] qmm routing M={M} N={N}", flush=True)
+    c = make_case(5200 + M + N, dt, bits, G, M, N, K)
+    exp = oracle.qmm_f64(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    out = GpuBuffer(M * N * dt.size_bytes)
+    ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+    got = unpack_f32(out.read_bytes(), dt)
+    for buf in (w, s, b, x, out):
+        buf.free()
+    assert rel_err(got, exp) <= 5e-2
