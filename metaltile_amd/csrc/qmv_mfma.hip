@@ -59,7 +59,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     const uint32_t RB = (uint32_t)rb64, nseg = p.K / (16u * cpc), nch = p.K / cpc;
     (void)cb;
     const uint32_t G = p.group_size;
-    if (!is_pow2(G) || G < cpc || p.K % G) return fail(ERR_UNSUPPORTED, "mfma qmv: group size");
+    if (!is_pow2(G) || G < cpc || G > 16u * cpc || p.K % G) return fail(ERR_UNSUPPORTED, "mfma qmv: group size");
     const uint32_t gpr = p.K / G;
     if (gpr % 4) return fail(ERR_UNSUPPORTED, "mfma qmv: groups per row not a multiple of 4");
     if ((uintptr_t)p.w % (odd ? 4 : 16) || (uintptr_t)p.x % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)

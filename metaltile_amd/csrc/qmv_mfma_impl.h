@@ -191,7 +191,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
 
     extern __shared__ __align__(16) unsigned char smem[];
     const uint32_t rows_wg = 4u * a.RBW * a.nrb;
-    m_u32x4* XL = (m_u32x4*)smem;                                    // [S][NP][nch][MP] pieces
+    m_u32x4* XL = (m_u32x4*)smem;                                    // [S][nch / 16][NP][16][MP] pieces: one wave-wide step reads NP contiguous KB
     float* XS = (float*)(XL + (size_t)S * NP * a.nch * MP);          // [S][nch][MP] chunk sums
     float2* SB = (float2*)(XS + (size_t)S * a.nch * MP);             // [waves][4 rows][gpw] + one zero pair
     const uint32_t sb_zero = (waves_of(a)) * 4u * a.gpw;               // index of the zero pair
@@ -360,7 +360,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                     o[dw] = h[0] | (h[1] << 16);
                 }
                 m_u32x4 piece = {o[0], o[1], o[2], o[3]};
-                XL[(((size_t)s * NP + p) * a.nch + c) * MP + i4] = piece;
+                XL[(size_t)s * NP * a.nch * MP + ((((size_t)(c >> 4) * NP + p) * 16u + (c & 15u)) * MP + i4)] = piece;
             }
         };
         // In the gather modes this body is a loop over passes. Index math of the staging and of the
@@ -401,6 +401,16 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
 #pragma unroll
             for (int i = 0; i < MP; i++) tot[s][i] = 0.f;
         uint32_t rb = 0, sg0 = 0;
+        // LDS addresses as a per-lane constant plus a wave-uniform offset per step: the step index is
+        // uniform, so its share is scalar arithmetic and each read costs one vector add. (A wave-wide
+        // step covers 16 * CPC codes, a whole number of groups: the host checks G <= 16 * CPC.)
+        const uint32_t c_lane = kp * a.spp * 16u + q;
+        const unsigned char* xl_lane = (const unsigned char*)(XL + ((size_t)(kp * a.spp) * NP * 16u + q) * MP + arow);
+        const unsigned char* xs_lane = (const unsigned char*)(XS + (size_t)c_lane * MP);
+        const uint32_t sb_idx = sb_row + ((c_lane * (uint32_t)CPC) >> a.log2g);  // 32-bit sum: sb_row alone may have wrapped
+        const unsigned char* sb_lane = (const unsigned char*)(SB + sb_idx);
+        const unsigned char* sb_zero_p = (const unsigned char*)(SB + sb_zero);
+        const uint32_t xl_set = (uint32_t)NP * a.nch * MP * 16u, xs_set = a.nch * MP * 4u;  // bytes from one row set to the next
         auto turn = [&](auto issue_tag) {
             constexpr bool ISSUE = decltype(issue_tag)::value;
             const uint32_t row_local = (rb * a.RBW + rbw) * 4u + r;
@@ -412,7 +422,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                 for (int d = 0; d < D; d++) {
                     const uint32_t sg = sg0 + d;
                     const bool valid = sg < a.spp;
-                    const uint32_t c = (kp * a.spp + min(sg, a.spp - 1)) * 16u + q;
+                    const uint32_t sgc = min(sg, a.spp - 1);  // uniform
                     // operands from LDS
                     m_u32x4 av[S][NP];
                     float xs[S][MP];
@@ -420,12 +430,13 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                     for (int s = 0; s < S; s++) {
 #pragma unroll
                         for (int p = 0; p < NP; p++)
-                            av[s][p] = XL[(((size_t)s * NP + p) * a.nch + c) * MP + arow];
+                            av[s][p] = *(const m_u32x4*)(xl_lane + (sgc * ((uint32_t)NP * 16u * MP * 16u) + (uint32_t)s * xl_set) + p * (16 * MP * 16));
+                        const float* xsp = (const float*)(xs_lane + (sgc * (16u * MP * 4u) + (uint32_t)s * xs_set));
 #pragma unroll
-                        for (int i = 0; i < MP; i++) xs[s][i] = XS[((size_t)s * a.nch + c) * MP + i];
+                        for (int i = 0; i < MP; i++) xs[s][i] = xsp[i];
                     }
-                    const uint32_t g = (c * (uint32_t)CPC) >> a.log2g;
-                    const float2 sb = SB[valid ? sb_row + g : sb_zero];
+                    const uint32_t g_off = ((sgc * 16u * (uint32_t)CPC) >> a.log2g) * 8u;
+                    const float2 sb = *(const float2*)(valid ? sb_lane + g_off : sb_zero_p);
                     uint32_t pw[Codec::PLANES * (CPC / 2)];
                     Codec::pairs(ring[d], kor, pw);
                     if constexpr (ISSUE) Codec::load(w_ptr(nrb_i, nsg0 + d), ring[d]);
