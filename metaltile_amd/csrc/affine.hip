@@ -95,92 +95,120 @@ template <int DT, int EPL> __device__ __forceinline__ void store_elems(void* p, 
     }
 }
 
+// Chunks per thread (a chunk = one lane's EPL elements): several independent 16-byte loads in
+// flight per thread, issued before any of them is used. Chunk u of a thread is 256 lanes after
+// chunk u - 1, so every load and store instruction still covers contiguous bytes.
+template <int BITS> struct AffineUnroll {
+    static constexpr int U = AffineGeom<BITS>::EPL == 8 ? 4 : (AffineGeom<BITS>::EPL == 16 ? 2 : 1);
+};
+
 template <int DT, int BITS>
 __global__ __launch_bounds__(256) void affine_quantize_kernel(AffineArgs a) {
 #pragma clang fp contract(off)
-    constexpr int EPL = AffineGeom<BITS>::EPL, NW = AffineGeom<BITS>::NW;
-    const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const uint64_t i0 = t * EPL;
-    if (i0 >= a.n_elem) return;  // whole groups leave together: n_elem is a multiple of G
-    float v[EPL];
-    load_elems<DT, EPL>(a.in, i0, v);
-    float mn = v[0], mx = v[0];
+    constexpr int EPL = AffineGeom<BITS>::EPL, NW = AffineGeom<BITS>::NW, U = AffineUnroll<BITS>::U;
+    const uint64_t n_lanes = a.n_elem / EPL;  // whole groups: n_elem is a multiple of G, G of EPL
+    uint64_t t[U];
+    bool live[U];
+    float v[U][EPL];
 #pragma unroll
-    for (int i = 1; i < EPL; i++) {
-        mn = v[i] < mn ? v[i] : mn;
-        mx = v[i] > mx ? v[i] : mx;
+    for (int u = 0; u < U; u++) {
+        t[u] = ((uint64_t)blockIdx.x * U + u) * 256u + threadIdx.x;
+        live[u] = t[u] < n_lanes;  // the lanes of a group are live or not together (256 is a multiple of their count)
+        load_elems<DT, EPL>(a.in, (live[u] ? t[u] : n_lanes - 1) * EPL, v[u]);
     }
-    // the group's lanes are consecutive and aligned to their (power-of-two) count
-    for (uint32_t d = 1; d < a.lanes_per_group; d <<= 1) {
-        const float omn = __shfl_xor(mn, (int)d, 64), omx = __shfl_xor(mx, (int)d, 64);
-        mn = omn < mn ? omn : mn;
-        mx = omx > mx ? omx : mx;
-    }
-    constexpr float QMAX = (float)((1u << BITS) - 1u);
-    float scale = (mx - mn) / QMAX;
-    if (scale < 1.0e-7f) scale = 1.0f;
-    const float inv = 1.0f / scale, bias = mn;
-    uint32_t words[NW];
 #pragma unroll
-    for (int j = 0; j < NW; j++) words[j] = 0u;
+    for (int u = 0; u < U; u++) {
+        float mn = v[u][0], mx = v[u][0];
 #pragma unroll
-    for (int i = 0; i < EPL; i++) {
-        const float d = v[i] - bias;
-        const float p = d * inv;
-        float q = p + 0.5f;
-        q = q < 0.0f ? 0.0f : q;
-        q = q > QMAX ? QMAX : q;
-        const uint32_t c = (uint32_t)q;
-        const int pos = i * BITS, wi = pos / 32, sh = pos % 32;
-        words[wi] |= c << sh;
-        if (sh + BITS > 32) words[wi + 1] |= c >> (32 - sh);
-    }
-    uint32_t* dst = (uint32_t*)a.out + t * NW;
-    if constexpr (NW == 1) {
-        dst[0] = words[0];
-    } else if constexpr (NW == 2) {
-        *(uint2*)dst = make_uint2(words[0], words[1]);
-    } else {
+        for (int i = 1; i < EPL; i++) {
+            mn = v[u][i] < mn ? v[u][i] : mn;
+            mx = v[u][i] > mx ? v[u][i] : mx;
+        }
+        // the group's lanes are consecutive and aligned to their (power-of-two) count
+        for (uint32_t d = 1; d < a.lanes_per_group; d <<= 1) {
+            const float omn = __shfl_xor(mn, (int)d, 64), omx = __shfl_xor(mx, (int)d, 64);
+            mn = omn < mn ? omn : mn;
+            mx = omx > mx ? omx : mx;
+        }
+        constexpr float QMAX = (float)((1u << BITS) - 1u);
+        float scale = (mx - mn) / QMAX;
+        if (scale < 1.0e-7f) scale = 1.0f;
+        const float inv = 1.0f / scale, bias = mn;
+        uint32_t words[NW];
 #pragma unroll
-        for (int j = 0; j < NW; j++) dst[j] = words[j];
-    }
-    if ((t & (a.lanes_per_group - 1)) == 0) {
-        const uint64_t g = i0 >> a.log2g;
-        store_elem<DT>(a.scales, g, scale);
-        store_elem<DT>(a.biases, g, bias);
+        for (int j = 0; j < NW; j++) words[j] = 0u;
+#pragma unroll
+        for (int i = 0; i < EPL; i++) {
+            const float d = v[u][i] - bias;
+            const float p = d * inv;
+            float q = p + 0.5f;
+            q = q < 0.0f ? 0.0f : q;
+            q = q > QMAX ? QMAX : q;
+            const uint32_t c = (uint32_t)q;
+            const int pos = i * BITS, wi = pos / 32, sh = pos % 32;
+            words[wi] |= c << sh;
+            if (sh + BITS > 32) words[wi + 1] |= c >> (32 - sh);
+        }
+        if (!live[u]) continue;
+        uint32_t* dst = (uint32_t*)a.out + t[u] * NW;
+        if constexpr (NW == 1) {
+            dst[0] = words[0];
+        } else if constexpr (NW == 2) {
+            *(uint2*)dst = make_uint2(words[0], words[1]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NW; j++) dst[j] = words[j];
+        }
+        if ((t[u] & (a.lanes_per_group - 1)) == 0) {
+            const uint64_t g = (t[u] * EPL) >> a.log2g;
+            store_elem<DT>(a.scales, g, scale);
+            store_elem<DT>(a.biases, g, bias);
+        }
     }
 }
 
 template <int DT, int BITS>
 __global__ __launch_bounds__(256) void affine_dequantize_kernel(AffineArgs a) {
 #pragma clang fp contract(off)
-    constexpr int EPL = AffineGeom<BITS>::EPL, NW = AffineGeom<BITS>::NW;
-    const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const uint64_t i0 = t * EPL;
-    if (i0 >= a.n_elem) return;
-    const uint32_t* src = (const uint32_t*)a.in + t * NW;
-    uint32_t words[NW];
-    if constexpr (NW == 2) {
-        const uint2 w2 = *(const uint2*)src;
-        words[0] = w2.x;
-        words[1] = w2.y;
-    } else {
+    constexpr int EPL = AffineGeom<BITS>::EPL, NW = AffineGeom<BITS>::NW, U = AffineUnroll<BITS>::U;
+    const uint64_t n_lanes = a.n_elem / EPL;
+    uint64_t t[U];
+    bool live[U];
+    uint32_t words[U][NW];
+    float scale[U], bias[U];
 #pragma unroll
-        for (int j = 0; j < NW; j++) words[j] = src[j];
-    }
-    const uint64_t g = i0 >> a.log2g;
-    const float scale = load_elem<DT>(a.scales, g), bias = load_elem<DT>(a.biases, g);
-    float v[EPL];
+    for (int u = 0; u < U; u++) {
+        t[u] = ((uint64_t)blockIdx.x * U + u) * 256u + threadIdx.x;
+        live[u] = t[u] < n_lanes;
+        const uint64_t tc = live[u] ? t[u] : n_lanes - 1;
+        const uint32_t* src = (const uint32_t*)a.in + tc * NW;
+        if constexpr (NW == 2) {
+            const uint2 w2 = *(const uint2*)src;
+            words[u][0] = w2.x;
+            words[u][1] = w2.y;
+        } else {
 #pragma unroll
-    for (int i = 0; i < EPL; i++) {
-        const int pos = i * BITS, wi = pos / 32, sh = pos % 32;
-        uint32_t c = words[wi] >> sh;
-        if (sh + BITS > 32) c |= words[wi + 1] << (32 - sh);
-        c &= (1u << BITS) - 1u;
-        const float p = scale * (float)c;
-        v[i] = p + bias;
+            for (int j = 0; j < NW; j++) words[u][j] = src[j];
+        }
+        const uint64_t g = (tc * EPL) >> a.log2g;
+        scale[u] = load_elem<DT>(a.scales, g);
+        bias[u] = load_elem<DT>(a.biases, g);
     }
-    store_elems<DT, EPL>(a.out, i0, v);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        if (!live[u]) continue;
+        float v[EPL];
+#pragma unroll
+        for (int i = 0; i < EPL; i++) {
+            const int pos = i * BITS, wi = pos / 32, sh = pos % 32;
+            uint32_t c = words[u][wi] >> sh;
+            if (sh + BITS > 32) c |= words[u][wi + 1] << (32 - sh);
+            c &= (1u << BITS) - 1u;
+            const float p = scale[u] * (float)c;
+            v[i] = p + bias[u];
+        }
+        store_elems<DT, EPL>(a.out, t[u] * EPL, v);
+    }
 }
 
 template <int DT, int BITS> static int launch_one(bool quantize, AffineArgs& a, const LaunchCtx& lc) {
@@ -191,8 +219,9 @@ template <int DT, int BITS> static int launch_one(bool quantize, AffineArgs& a, 
         return fail(ERR_UNSUPPORTED, "affine: group_size / run must be a power of two up to 64");
     a.log2g = 0;
     while ((1u << a.log2g) < a.group_size) a.log2g++;
-    const uint64_t threads = a.n_elem / EPL;
-    const uint64_t blocks = (threads + 255) / 256;
+    const uint64_t lanes = a.n_elem / EPL;
+    const uint64_t per_block = 256ull * AffineUnroll<BITS>::U;
+    const uint64_t blocks = (lanes + per_block - 1) / per_block;
     if (blocks == 0) return ERR_OK;
     if (blocks > 0x7FFFFFFFull) return fail(ERR_SHAPE, "affine: too many elements for one launch");
     const void* fn = quantize ? (const void*)affine_quantize_kernel<DT, BITS> : (const void*)affine_dequantize_kernel<DT, BITS>;
