@@ -1121,7 +1121,7 @@ int mtq_set_option(const char* name, int value) {
         return MTQ_OK;
     }
     if (!strcmp(name, "qmm.tile_rows")) {
-        if (value != 0 && value != 64 && value != 128) return fail(ERR_BAD_ARG, "qmm.tile_rows must be 0, 64 or 128");
+        if (value != 0 && value != 32 && value != 64 && value != 128) return fail(ERR_BAD_ARG, "qmm.tile_rows must be 0, 32, 64 or 128");
         options().qmm_tile_rows = value;
         return MTQ_OK;
     }

@@ -50,7 +50,7 @@ struct QmmDArgs {
     uint32_t M, N, K;
     uint32_t log2g, gpr;
     uint32_t m_tiles, n_tiles, iters;
-    uint32_t m_tile_rows;  // 64 or 128
+    uint32_t m_tile_rows;  // 32 (4 K-groups only), 64 or 128
 };
 
 
@@ -295,12 +295,12 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
     __syncthreads();
     // all threads store the tile, 16 bytes each, whole rows
     constexpr int VPR = DBN / 8;                    // 16-byte vectors per tile row
-    constexpr int VPT = DBM * VPR / NT;            // vectors per thread
+    constexpr int VPT = (DBM * VPR + NT - 1) / NT;  // vectors per thread
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
         const uint32_t v = tid + i * NT, lrow = v / VPR, c16 = v % VPR;
         const uint32_t row = m0 + lrow;
-        if (row < a.M)
+        if (row < a.M && (DBM * VPR % NT == 0 || lrow < (uint32_t)DBM))
             *(q_u32x4*)((uint16_t*)a.out + (size_t)row * a.N + n0 + c16 * 8) = *(const q_u32x4*)(otile + lrow * DBN + c16 * 8);
     }
 }
@@ -324,7 +324,7 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
     if (shmem > 160 * 1024) return fail(ERR_UNSUPPORTED, "direct qmm: tile does not fit in LDS");
 #define QD_PICK3(B, MBv, KGv) (sbl ? (const void*)qmm_direct_kernel<DT, B, 2, MBv, true, KGv> : (const void*)qmm_direct_kernel<DT, B, 2, MBv, false, KGv>)
 #define QD_PICK(B)                                                                      \
-    fn = kgroups == 4   ? (tall ? QD_PICK3(B, 4, 4) : QD_PICK3(B, 2, 4))                \
+    fn = kgroups == 4   ? (tall ? QD_PICK3(B, 4, 4) : a.m_tile_rows == 32 ? QD_PICK3(B, 1, 4) : QD_PICK3(B, 2, 4)) \
          : kgroups == 1 ? (tall ? QD_PICK3(B, 4, 1) : QD_PICK3(B, 2, 1))                \
                         : (tall ? QD_PICK3(B, 4, 2) : QD_PICK3(B, 2, 2))
     switch (bits) {
@@ -377,9 +377,13 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
     uint32_t rows = 64, kgroups = 2;
     if (tall_wide >= 2 * (uint64_t)cus) { rows = 128; kgroups = 1; }  // two 4-wave workgroups per CU (M = 2048: 72-75 us against 80-84; M = 4096: 160-170 against 180-190)
     else if (tall_wide >= (uint64_t)cus) { rows = 128; kgroups = 2; }
-    else if (short_wide * 2 <= (uint64_t)cus) { rows = 64; kgroups = 4; }  // few tiles: halve their width
+    else if (short_wide * 2 <= (uint64_t)cus) {  // few tiles: halve their width, and their height for up to 32 rows
+        rows = p.M <= 32 ? 32 : 64;
+        kgroups = 4;
+    }
     if (options().qmm_tile_rows) rows = (uint32_t)options().qmm_tile_rows;
     if (options().qmm_kgroups) kgroups = (uint32_t)options().qmm_kgroups;
+    if (rows == 32 && kgroups != 4) return fail(ERR_BAD_ARG, "qmm.tile_rows 32 needs 4 K-groups");
     a.m_tile_rows = rows;
     a.m_tiles = (p.M + rows - 1) / rows;
     a.n_tiles = p.N / (kgroups == 1 ? 128 : 32 * (8 / kgroups));

@@ -1,5 +1,5 @@
 """Every tiling of the direct matrix-core qmm kernel (K-groups 1, 2, 4 x tile heights 64,
-128), forced through the library's options on one ragged shape, against the oracle's
+128, and 32 with 4 K-groups), forced through the library's options on one ragged shape, against the oracle's
 restatement of the reference's mma semantics (weights rounded to the element dtype
 before the multiply, crates/metaltile-std/src/mlx/quantized.rs:2267-2274).
 Tolerance: 2e-2 on max|a-e| / max(|e|, 1), the bound of the bf16 prefill configuration;
@@ -39,7 +39,7 @@ def test_direct_qmm_every_tiling(oracle, options, bits, dt):
                   GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
     options("qmm.kernel", 2)
     for kg in (1, 2, 4):
-        for rows in (64, 128):
+        for rows in ((32, 64, 128) if kg == 4 else (64, 128)):
             print(f"[case] direct qmm {dt.name} b{bits} kgroups={kg} tile_rows={rows}", flush=True)
             options("qmm.kgroups", kg)
             options("qmm.tile_rows", rows)
