@@ -1120,6 +1120,11 @@ int mtq_set_option(const char* name, int value) {
         options().qmm_kgroups = value;
         return MTQ_OK;
     }
+    if (!strcmp(name, "qmm.by_m")) {
+        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmm.by_m must be 0 (choose), 1 or 2 (off)");
+        options().qmm_by_m = value;
+        return MTQ_OK;
+    }
     if (!strcmp(name, "qmm.tile_rows")) {
         if (value != 0 && value != 32 && value != 64 && value != 128) return fail(ERR_BAD_ARG, "qmm.tile_rows must be 0, 32, 64 or 128");
         options().qmm_tile_rows = value;

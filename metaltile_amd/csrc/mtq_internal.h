@@ -91,6 +91,7 @@ struct Options {
     int qmm_splits = 0;           // MFMA qmm: K splits per tile (0 = choose per shape)
     int qmm_kernel = 0;           // MFMA qmm: 0 auto, 1 both operands through LDS, 2 weights direct to registers
     int qmm_kgroups = 0;          // direct qmm: K-groups per workgroup (0 = choose; 1, 2, 4)
+    int qmm_by_m = 0;             // direct qmm: 1 = an XCD keeps its M-tiles' activations and streams all weights
     int qmm_tile_rows = 0;        // direct qmm: activation rows per tile (0 = choose; 32, 64, 128)
     int qmv_mfma = 0;             // matrix-core qmv: 0 auto, 1 never, 2 whenever the shape fits
     int qmv_mfma_kp = 0;          // matrix-core qmv: K parts per row block

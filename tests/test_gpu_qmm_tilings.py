@@ -24,7 +24,7 @@ def options():
         assert lib.mtq_set_option(name.encode(), value) == 0, name
 
     yield set_
-    for name in ("qmm.kernel", "qmm.kgroups", "qmm.tile_rows"):
+    for name in ("qmm.kernel", "qmm.kgroups", "qmm.tile_rows", "qmm.by_m"):
         lib.mtq_set_option(name.encode(), 0)
 
 
@@ -43,12 +43,14 @@ def test_direct_qmm_every_tiling(oracle, options, bits, dt):
             print(f"[case] direct qmm {dt.name} b{bits} kgroups={kg} tile_rows={rows}", flush=True)
             options("qmm.kgroups", kg)
             options("qmm.tile_rows", rows)
-            out = GpuBuffer(M * N * dt.size_bytes)
-            ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
-            got = unpack_f32(out.read_bytes(), dt)
-            out.free()
-            err = rel_err(got, exp)
-            assert err <= 2e-2, f"kgroups={kg} rows={rows}: rel err {err:.3e}"
+            for by_m in (1, 2):  # both orders of walking the tiles
+                options("qmm.by_m", by_m)
+                out = GpuBuffer(M * N * dt.size_bytes)
+                ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+                got = unpack_f32(out.read_bytes(), dt)
+                out.free()
+                err = rel_err(got, exp)
+                assert err <= 2e-2, f"kgroups={kg} rows={rows} by_m={by_m}: rel err {err:.3e}"
     for buf in (w, s, b, x):
         buf.free()
 
