@@ -322,7 +322,23 @@ MTQ_API int mtq_flush_cache(void);
  *   "qmv.rows_per_thread"  one-shot kernel: 0 = choose per shape, or 4 / 7 / 8
  *   "qmv.stream_depth"     streaming kernel: 0 = choose per shape, or 4 / 8 loads in flight per thread
  *   "qmv.stream_batches"   streaming kernel: 0 = choose per shape, or 1..16 batches per thread
- *   "qmm.splits"           MFMA qmm: 0 = choose per shape, or the number of K slices per output tile
+ *   "qmv.mfma"             matrix-core GEMV kernel: 0 = choose per shape, 1 = never, 2 = wherever it applies
+ *   "qmv.mfma_delay"       matrix-core GEMV kernel: pause (x 512 clocks) before the first weight loads, 0..64;
+ *                          a measurement aid
+ *   "qmv.mfma_kp" / "qmv.mfma_rbw" / "qmv.mfma_nrb" / "qmv.mfma_sets"
+ *                          matrix-core GEMV geometry: K parts per row, row blocks side by side and one
+ *                          after the other per workgroup, 4-row activation sets per pass; 0 = choose
+ *   "qmm.kernel"           0 = choose per shape, 1 = tile kernel with both operands through LDS, 2 = tile
+ *                          kernel with the weights converted in registers
+ *   "qmm.kgroups"          register-operand tile kernel: K-groups per workgroup, 0 = choose, or 1 / 2 / 4
+ *   "qmm.tile_rows"        activation rows per tile, 0 = choose, or 32 (4 K-groups only) / 64 / 128
+ *   "qmm.by_m"             order in which workgroups walk the tiles: 0 = choose, 1 = the N-tiles of one M-tile
+ *                          first, 2 = the M-tiles of one N-tile first
+ *   "qmm.splits"           LDS tile kernel: 0 = choose per shape, or the number of K slices per output tile
+ *   "qvm.wgs"              qvm: workgroups to aim for when K is sliced, 0 = choose
+ *   "moe.sort"             expert sort: 0 = choose by size, 1 = always the bitonic network
+ *   "moe_down.rows"        fused MoE down projection: output rows per workgroup, 0 = choose
+ * Results do not depend on any of them beyond the order of floating-point sums.
  * Unknown names or values fail with MTQ_ERR_BAD_ARG. */
 MTQ_API int mtq_set_option(const char *name, int value);
 
