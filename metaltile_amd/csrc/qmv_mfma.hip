@@ -26,8 +26,8 @@ int num_cus_mfma() {
 }
 
 // waves = KP * RBW; gpw = (scale, bias) pairs per row in a wave's window
-size_t lds_bytes(uint32_t R, uint32_t K, uint32_t nch, uint32_t rows_wg, uint32_t waves, uint32_t gpw, uint32_t KP, uint32_t list_cap) {
-    return (size_t)R * K * 2 + (size_t)R * nch * 4 + ((size_t)waves * 4 * gpw + 1) * 8 +
+size_t lds_bytes(uint32_t R, uint32_t K, uint32_t nch, uint32_t gpr, uint32_t rows_wg, uint32_t waves, uint32_t gpw, uint32_t KP, uint32_t list_cap) {
+    return (size_t)R * K * 2 + (size_t)R * gpr * 4 + ((size_t)waves * 4 * gpw + 1) * 8 +
            (size_t)KP * rows_wg * R * 4 + (size_t)list_cap * 4 + 64;
 }
 
@@ -164,7 +164,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
             if (64u * KP * RBW > maxt) return fail(ERR_BAD_ARG, "qmv.mfma_rbw: workgroup too large");
         }
         if (opt.qmv_mfma_nrb) nrb = (uint32_t)opt.qmv_mfma_nrb;
-        auto need = [&]() { return lds_bytes((uint32_t)(mp * s), p.K, nch, 4 * RBW * nrb, KP * RBW, gpw, KP, list_cap); };
+        auto need = [&]() { return lds_bytes((uint32_t)(mp * s), p.K, nch, gpr, 4 * RBW * nrb, KP * RBW, gpw, KP, list_cap); };
         const uint32_t nrb_planned = nrb;
         const bool last = s == 1;  // nothing left to halve: shrink as far as it takes
         while (need() > kLdsBudget) {
@@ -222,7 +222,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     g.s = s;
     g.tpb = 64u * KP * RBW;
     const uint32_t rows_wg = 4 * RBW * nrb;
-    g.shmem = lds_bytes(R, p.K, nch, rows_wg, KP * RBW, gpw, KP, list_cap);
+    g.shmem = lds_bytes(R, p.K, nch, gpr, rows_wg, KP * RBW, gpw, KP, list_cap);
     g.grid = dim3((p.N + rows_wg - 1) / rows_wg, gather ? p.E : 1, 1);
     if (odd)
         return p.dtype == DT_F16 ? qmv_mfma_launch_dtype_odd<DT_F16>(a, p.bits, p.gather, g, lc)

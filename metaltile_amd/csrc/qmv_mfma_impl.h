@@ -192,8 +192,8 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     const uint32_t rows_wg = 4u * a.RBW * a.nrb;
     m_u32x4* XL = (m_u32x4*)smem;                                    // [S][nch / 16][NP][16][MP] pieces: one wave-wide step reads NP contiguous KB
-    float* XS = (float*)(XL + (size_t)S * NP * a.nch * MP);          // [S][nch][MP] chunk sums
-    float2* SB = (float2*)(XS + (size_t)S * a.nch * MP);             // [waves][4 rows][gpw] + one zero pair
+    float* XG = (float*)(XL + (size_t)S * NP * a.nch * MP);          // [S][gpr][MP] sums of the activations over each group
+    float2* SB = (float2*)(XG + (size_t)S * a.gpr * MP);             // [waves][4 rows][gpw] + one zero pair
     const uint32_t sb_zero = (waves_of(a)) * 4u * a.gpw;               // index of the zero pair
     float* RED = (float*)(SB + (size_t)sb_zero + 1);                 // [KP][rows_wg][R]
     uint32_t* rowlist = (uint32_t*)(RED + (size_t)a.KP * rows_wg * R);
@@ -331,6 +331,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                 raw[4 * p] = v.x; raw[4 * p + 1] = v.y; raw[4 * p + 2] = v.z; raw[4 * p + 3] = v.w;
             }
         };
+        const uint32_t cpg = (1u << a.log2g) / (uint32_t)CPC;  // chunks per group: a power of two, at most 16
         auto x_store = [&](uint32_t task) {
             const uint32_t i = task / a.nch, c = task - i * a.nch;
             if (!row_live) {
@@ -344,7 +345,12 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                 else sum += f16_bits_to_f32(raw[j] & 0xFFFFu) + f16_bits_to_f32(raw[j] >> 16);
             }
             const uint32_t s = i / MP, i4 = i % MP;
-            XS[((size_t)s * a.nch + c) * MP + i4] = sum;
+            // A group is cpg consecutive chunks of one row, staged by cpg consecutive lanes (tasks are
+            // dealt in order, a row is a multiple of 16 >= cpg chunks, and the lanes of such a block are
+            // all staging or all idle): butterfly over them, one lane writes. The bias term of a row
+            // block is then b' . (group sums), added once per row block instead of once per chunk.
+            for (uint32_t o = 1; o < cpg; o <<= 1) sum += __shfl_xor(sum, (int)o, 64);
+            if ((c & (cpg - 1u)) == 0u) XG[((size_t)s * a.gpr + c / cpg) * MP + i4] = sum;
 #pragma unroll
             for (int p = 0; p < NP; p++) {
                 uint32_t o[4];
@@ -406,11 +412,12 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         // step covers 16 * CPC codes, a whole number of groups: the host checks G <= 16 * CPC.)
         const uint32_t c_lane = kp * a.spp * 16u + q;
         const unsigned char* xl_lane = (const unsigned char*)(XL + ((size_t)(kp * a.spp) * NP * 16u + q) * MP + arow);
-        const unsigned char* xs_lane = (const unsigned char*)(XS + (size_t)c_lane * MP);
         const uint32_t sb_idx = sb_row + ((c_lane * (uint32_t)CPC) >> a.log2g);  // 32-bit sum: sb_row alone may have wrapped
         const unsigned char* sb_lane = (const unsigned char*)(SB + sb_idx);
         const unsigned char* sb_zero_p = (const unsigned char*)(SB + sb_zero);
-        const uint32_t xl_set = (uint32_t)NP * a.nch * MP * 16u, xs_set = a.nch * MP * 4u;  // bytes from one row set to the next
+        const uint32_t xl_set = (uint32_t)NP * a.nch * MP * 16u;  // bytes from one row set to the next
+        const uint32_t part_g0 = (kp * a.spp * 16u * (uint32_t)CPC) >> a.log2g;  // this wave's K part: whole groups
+        const uint32_t part_ng = (a.spp * 16u * (uint32_t)CPC) >> a.log2g;
         auto turn = [&](auto issue_tag) {
             constexpr bool ISSUE = decltype(issue_tag)::value;
             const uint32_t row_local = (rb * a.RBW + rbw) * 4u + r;
@@ -425,15 +432,11 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                     const uint32_t sgc = min(sg, a.spp - 1);  // uniform
                     // operands from LDS
                     m_u32x4 av[S][NP];
-                    float xs[S][MP];
 #pragma unroll
                     for (int s = 0; s < S; s++) {
 #pragma unroll
                         for (int p = 0; p < NP; p++)
                             av[s][p] = *(const m_u32x4*)(xl_lane + (sgc * ((uint32_t)NP * 16u * MP * 16u) + (uint32_t)s * xl_set) + p * (16 * MP * 16));
-                        const float* xsp = (const float*)(xs_lane + (sgc * (16u * MP * 4u) + (uint32_t)s * xs_set));
-#pragma unroll
-                        for (int i = 0; i < MP; i++) xs[s][i] = xsp[i];
                     }
                     const uint32_t g_off = ((sgc * 16u * (uint32_t)CPC) >> a.log2g) * 8u;
                     const float2 sb = *(const float2*)(valid ? sb_lane + g_off : sb_zero_p);
@@ -467,10 +470,20 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
 #pragma unroll
                         for (int i = 0; i < MP; i++) {
                             tot[s][i] = fmaf(sb.x, acc[s][i], tot[s][i]);
-                            tot[s][i] = fmaf(sb.y, xs[s][i], tot[s][i]);
                         }
                 }
                 if (wrap) {
+                    // bias term of this row block: the 16 lanes of a weight row share its K part's groups
+                    for (uint32_t gi = q; gi < part_ng; gi += 16u) {
+                        const uint32_t g = part_g0 + gi;
+                        const float bq = SB[sb_row + g].y;
+#pragma unroll
+                        for (int s = 0; s < S; s++) {
+                            const float* xg = XG + ((size_t)s * a.gpr + g) * MP;
+#pragma unroll
+                            for (int i = 0; i < MP; i++) tot[s][i] = fmaf(bq, xg[i], tot[s][i]);
+                        }
+                    }
                     // lanes of one weight row (same r, all q) add up: q spans lane bits 2..5
 #pragma unroll
                     for (int s = 0; s < S; s++)
