@@ -69,3 +69,23 @@ def test_gather_all_widths(oracle, bits, dt):
     assert rel_err(got.reshape(-1), exp.reshape(T, N)[perm].reshape(-1)) <= TOL[dt]
     for buf in (w, s, b, x, xb, r, out):
         buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.F16, DType.BF16], ids=lambda d: d.name)
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("G", [256, 512, 1024, 2048])
+@pytest.mark.parametrize("M", [1, 4, 8])
+def test_large_groups(oracle, M, G, bits, dt):
+    """Groups of 256..2048 codes: wider than one wave-wide step of the matrix-core GEMV for the
+    larger ones, which then hands the request to the other kernels of the family."""
+    N, K = 136, 4096
+    c = make_case(900 + bits + G + M, dt, bits, G, M, N, K, bias_rule="midpoint")
+    print(f"[case] large group {dt.name} b{bits} g{G} M{M}", flush=True)
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    out = GpuBuffer(M * N * dt.size_bytes)
+    ops.qmv(dt, bits, G, w, s, b, x, out, M, N, K)
+    got = unpack_f32(out.read_bytes(), dt)
+    assert rel_err(got, _expected(oracle, c)) <= TOL[dt]
+    for buf in (w, s, b, x, out):
+        buf.free()
