@@ -99,7 +99,7 @@ def main():
     a = parse_args()
     if a.gpus != 1:
         print(f"bench.py: this build runs on ONE GPU; --gpus {a.gpus} is not supported "
-              "(the path shards by rows / experts with no collective; see DESIGN.md).", file=sys.stderr)
+              "(the path would shard by weight rows or by experts, with no collective; nothing here uses a second GPU).", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
