@@ -194,20 +194,34 @@ int launch_qmv_norm(const QmvParams& p0, const void* norm_w, const float* eps, c
     return launch_qmv_stream(p, C, rps, C * rps, 1, lc, nullptr, norm_w, eps);
 }
 
+static int launch_qmv_dot2(const QmvParams& p, const LaunchCtx& lc);
+
 int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {
-    {
-        // The matrix-core kernel wins as soon as more than one activation row shares
-        // the weight stream (and for every gather); a single row is as fast on the
-        // dot2 kernels below.
-        // Widths 3, 5 and 6 have no dot2 kernel: the matrix-core kernel is their fast path.
-        const bool many = p.gather == GATHER_CSR || p.gather == GATHER_INDICES || (p.gather == GATHER_NONE && p.M >= 2) ||
-                          p.bits == 3 || p.bits == 5 || p.bits == 6;
-        const int mode = options().qmv_mfma;
-        if (mode == 2 || (mode == 0 && many)) {
-            int rc = launch_qmv_mfma(p, lc);
-            if (rc != ERR_UNSUPPORTED) return rc;
-        }
+    // The matrix-core kernel wins as soon as more than one activation row shares
+    // the weight stream (and for every gather); a single row is as fast on the
+    // dot2 kernels.
+    // Widths 3, 5 and 6 have no dot2 kernel: the matrix-core kernel is their fast path.
+    const bool many = p.gather == GATHER_CSR || p.gather == GATHER_INDICES || (p.gather == GATHER_NONE && p.M >= 2) ||
+                      p.bits == 3 || p.bits == 5 || p.bits == 6;
+    const int mode = options().qmv_mfma;
+    bool tried_mfma = false;
+    if (mode == 2 || (mode == 0 && many)) {
+        int rc = launch_qmv_mfma(p, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+        tried_mfma = true;
     }
+    int rc = launch_qmv_dot2(p, lc);
+    // Rows the dot2 kernels cannot tile (a chunk count that is neither whole waves nor a power of
+    // two, e.g. K = 3584 or 18944 with 4-bit codes) still fit the matrix-core kernel when they are
+    // whole 512-code segments: 18944x3584, one row, 98 us on the generic kernel against 12 us.
+    if (rc == ERR_UNSUPPORTED && !tried_mfma && mode != 1) {
+        const int rc2 = launch_qmv_mfma(p, lc);
+        if (rc2 != ERR_UNSUPPORTED) return rc2;
+    }
+    return rc;
+}
+
+static int launch_qmv_dot2(const QmvParams& p, const LaunchCtx& lc) {
     if (p.bits != 2 && p.bits != 4 && p.bits != 8)
         return fail(ERR_UNSUPPORTED, "fast qmv: bits must be 2, 4 or 8");
     const uint32_t cpc = 128u / (uint32_t)p.bits;

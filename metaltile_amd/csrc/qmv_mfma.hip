@@ -26,17 +26,19 @@ int num_cus_mfma() {
 }
 
 // waves = KP * RBW; gpw = (scale, bias) pairs per row in a wave's window
-size_t lds_bytes(uint32_t R, uint32_t K, uint32_t nch, uint32_t gpr, uint32_t rows_wg, uint32_t waves, uint32_t gpw, uint32_t KP, uint32_t list_cap) {
+size_t lds_bytes(uint32_t R, uint32_t K /* padded to whole steps */, uint32_t nch, uint32_t gpr, uint32_t rows_wg, uint32_t waves, uint32_t gpw, uint32_t KP, uint32_t list_cap) {
     return (size_t)R * K * 2 + (size_t)R * gpr * 4 + ((size_t)waves * 4 * gpw + 1) * 8 +
            (size_t)KP * rows_wg * R * 4 + (size_t)list_cap * 4 + 64;
 }
 
 // Pairs per row that a wave's window must hold: the groups its K part touches, from a
-// multiple of 4 (8-byte loads) up to a whole number of 4-vectors.
-uint32_t window_pairs(uint32_t kp_count, uint32_t spp, uint32_t cpc, uint32_t log2g) {
+// multiple of 4 (8-byte loads) up to a whole number of 4-vectors. Parts are spp wave-wide
+// steps of 16 * cpc codes; the last part ends with the row (K codes).
+uint32_t window_pairs(uint32_t kp_count, uint32_t spp, uint32_t cpc, uint32_t log2g, uint32_t K) {
     uint32_t need = 4;
     for (uint32_t kp = 0; kp < kp_count; kp++) {
-        const uint32_t first = (kp * spp * 16u * cpc) >> log2g, last = (((kp + 1) * spp * 16u * cpc) - 1u) >> log2g;
+        const uint64_t end = (uint64_t)(kp + 1) * spp * 16u * cpc;
+        const uint32_t first = (kp * spp * 16u * cpc) >> log2g, last = (uint32_t)(((end < K ? end : K) - 1u) >> log2g);
         const uint32_t lo = first & ~3u, n = (last + 1 - lo + 3) / 4 * 4;
         if (n > need) need = n;
     }
@@ -53,10 +55,12 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     // a lane's chunk: 16 bytes (128/bits codes), or 32 codes = bits dwords where codes straddle words
     const uint32_t cpc = odd ? 32u : 128u / (uint32_t)p.bits, cb = odd ? 4u * (uint32_t)p.bits : 16u;
     const uint64_t rb64 = (uint64_t)p.K * p.bits / 8;
-    if (p.K % (16u * cpc) || rb64 > (1u << 24)) return fail(ERR_UNSUPPORTED, "mfma qmv: row is not whole wave-wide segments");
+    if (p.K % cpc || rb64 > (1u << 24)) return fail(ERR_UNSUPPORTED, "mfma qmv: row is not whole lane chunks");
     if (rb64 * p.N >= (1ull << 32) || (uint64_t)p.N * (p.K / p.group_size) >= (1ull << 31))
         return fail(ERR_UNSUPPORTED, "mfma qmv: a weight matrix of 4 GiB or more");
-    const uint32_t RB = (uint32_t)rb64, nseg = p.K / (16u * cpc), nch = p.K / cpc;
+    // A wave-wide step covers 16 lane chunks of each of 4 rows; a row that is not a whole number of
+    // steps ends with a partial one (its idle lanes are fed zeros).
+    const uint32_t RB = (uint32_t)rb64, nch = p.K / cpc, nseg = (nch + 15u) / 16u, nchp = nseg * 16u;
     (void)cb;
     const uint32_t G = p.group_size;
     if (!is_pow2(G) || G < cpc || G > 16u * cpc || p.K % G) return fail(ERR_UNSUPPORTED, "mfma qmv: group size");
@@ -73,15 +77,16 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     uint32_t KP = 1;
     if (opt.qmv_mfma_kp) {
         KP = (uint32_t)opt.qmv_mfma_kp;
-        if (nseg % KP) return fail(ERR_BAD_ARG, "qmv.mfma_kp must divide the row's segment count");
+        if ((uint64_t)(KP - 1) * ((nseg + KP - 1) / KP) >= nseg) return fail(ERR_BAD_ARG, "qmv.mfma_kp leaves a K part empty");
     } else {
         uint32_t best = 1;
         double best_score = 1e30;
         for (uint32_t kp = 1; kp <= nseg && kp <= 16; kp++) {
-            if (nseg % kp) continue;
-            if (window_pairs(kp, nseg / kp, cpc, ilog2(G)) > 64) continue;  // a lane refills one 4-vector of its wave's window
-            const uint32_t spp = nseg / kp, padded = (spp + 3) / 4 * 4;
-            double score = (double)(padded - spp) / spp;          // wasted ring slots
+            // parts of spp steps each; the last may be shorter but not empty
+            const uint32_t spp = (nseg + kp - 1) / kp, padded = (spp + 3) / 4 * 4;
+            if ((uint64_t)(kp - 1) * spp >= nseg) continue;
+            if (window_pairs(kp, spp, cpc, ilog2(G), p.K) > 64) continue;  // a lane refills one 4-vector of its wave's window
+            double score = (double)((uint64_t)kp * padded - nseg) / nseg;  // wasted ring slots over all parts
             if (spp > 8) score += 0.05 * (spp - 8);               // long walks: few waves per row block
             if (spp < 4) score += 0.5;
             score += 0.01 * kp;
@@ -89,8 +94,8 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
         }
         KP = best;
     }
-    const uint32_t spp = nseg / KP;
-    const uint32_t gpw = window_pairs(KP, spp, cpc, ilog2(G));
+    const uint32_t spp = (nseg + KP - 1) / KP;
+    const uint32_t gpw = window_pairs(KP, spp, cpc, ilog2(G), p.K);
     if (gpw > 64) return fail(ERR_UNSUPPORTED, "mfma qmv: K part spans more than 64 groups");
 
     // activation rows per pass
@@ -164,7 +169,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
             if (64u * KP * RBW > maxt) return fail(ERR_BAD_ARG, "qmv.mfma_rbw: workgroup too large");
         }
         if (opt.qmv_mfma_nrb) nrb = (uint32_t)opt.qmv_mfma_nrb;
-        auto need = [&]() { return lds_bytes((uint32_t)(mp * s), p.K, nch, gpr, 4 * RBW * nrb, KP * RBW, gpw, KP, list_cap); };
+        auto need = [&]() { return lds_bytes((uint32_t)(mp * s), nchp * cpc, nch, gpr, 4 * RBW * nrb, KP * RBW, gpw, KP, list_cap); };
         const uint32_t nrb_planned = nrb;
         const bool last = s == 1;  // nothing left to halve: shrink as far as it takes
         while (need() > kLdsBudget) {
@@ -173,7 +178,16 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
             else break;
         }
         if (need() <= kLdsBudget) break;
-        if (last) return fail(ERR_UNSUPPORTED, "mfma qmv: activations do not fit in LDS");
+        if (last) {
+            // Not even one set of 4 rows: a plain batch can still go 2 rows, then 1 row, per pass
+            // (3584x18944 with 4 rows: two passes of 12 us against 343 us on the generic kernel).
+            if (p.gather == GATHER_NONE && mp > 1) {
+                mp /= 2;
+                s = 2;  // halved to 1 by the loop
+                continue;
+            }
+            return fail(ERR_UNSUPPORTED, "mfma qmv: activations do not fit in LDS");
+        }
     }
     const uint32_t R = (uint32_t)(mp * s);
     if (p.gather == GATHER_NONE && rows_per_launch > R) rows_per_launch = R;
@@ -208,6 +222,8 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     a.E = p.E;
     a.RB = RB;
     a.nch = nch;
+    a.nchp = nchp;
+    a.nseg = nseg;
     a.spp = spp;
     a.KP = KP;
     a.RBW = RBW;
@@ -222,7 +238,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     g.s = s;
     g.tpb = 64u * KP * RBW;
     const uint32_t rows_wg = 4 * RBW * nrb;
-    g.shmem = lds_bytes(R, p.K, nch, gpr, rows_wg, KP * RBW, gpw, KP, list_cap);
+    g.shmem = lds_bytes(R, nchp * cpc, nch, gpr, rows_wg, KP * RBW, gpw, KP, list_cap);
     g.grid = dim3((p.N + rows_wg - 1) / rows_wg, gather ? p.E : 1, 1);
     if (odd)
         return p.dtype == DT_F16 ? qmv_mfma_launch_dtype_odd<DT_F16>(a, p.bits, p.gather, g, lc)

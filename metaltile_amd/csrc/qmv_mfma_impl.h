@@ -65,8 +65,10 @@ struct QmvMArgs {
     const uint32_t* route;
     uint32_t M, N, K, T, E;
     uint32_t RB;        // bytes per packed weight row
-    uint32_t nch;       // 16-byte chunks per row
-    uint32_t spp;       // 256-byte segments per K part
+    uint32_t nch;       // lane chunks per row (K / CPC)
+    uint32_t nchp;      // nch rounded up to whole wave-wide steps of 16 chunks
+    uint32_t nseg;      // wave-wide steps per row (nchp / 16); the last one may be partial
+    uint32_t spp;       // steps per K part (the last part may be shorter)
     uint32_t KP;        // K parts (waves sharing a row block)
     uint32_t RBW;       // row blocks walked in parallel by one workgroup
     uint32_t nrb;       // row blocks per wave, one after the other
@@ -192,7 +194,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     const uint32_t rows_wg = 4u * a.RBW * a.nrb;
     m_u32x4* XL = (m_u32x4*)smem;                                    // [S][nch / 16][NP][16][MP] pieces: one wave-wide step reads NP contiguous KB
-    float* XG = (float*)(XL + (size_t)S * NP * a.nch * MP);          // [S][gpr][MP] sums of the activations over each group
+    float* XG = (float*)(XL + (size_t)S * NP * a.nchp * MP);          // [S][gpr][MP] sums of the activations over each group
     float2* SB = (float2*)(XG + (size_t)S * a.gpr * MP);             // [waves][4 rows][gpw] + one zero pair
     const uint32_t sb_zero = (waves_of(a)) * 4u * a.gpw;               // index of the zero pair
     float* RED = (float*)(SB + (size_t)sb_zero + 1);                 // [KP][rows_wg][R]
@@ -259,6 +261,11 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     const uint16_t* bslab = (const uint16_t*)a.biases + slab_rows * a.gpr;
     const uint32_t woff = (kp * a.spp) * SEGB + q * (uint32_t)Codec::CB;
     const uint32_t sppD = (a.spp + D - 1) / D * D;  // steps per row block, padded to whole rings
+    // This wave's K part may be shorter than the others (the last one), and in the row's last step
+    // only the first nch - 16 * (nseg - 1) lanes of a row have a chunk.
+    const uint32_t spp_eff = min(a.spp, a.nseg - kp * a.spp);
+    const bool short_lane = kp * a.spp + spp_eff == a.nseg && q >= a.nch - 16u * (a.nseg - 1u);
+    const uint32_t lane_steps = spp_eff - (short_lane ? 1u : 0u);  // steps in which this lane's chunk exists
     // (scale, bias) pairs: every wave keeps those of its own 4 rows and its own K part in its own
     // LDS window and refills it when it moves to the next row block, so the number of row blocks
     // a workgroup walks is not bounded by LDS and no workgroup barrier sits in the refill.
@@ -300,9 +307,9 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     // load is multiplied by a zero scale.
     auto w_ptr = [&](uint32_t rb, uint32_t sg, uint32_t nudge = 0u) -> const unsigned char* {
         rb = min(rb, a.nrb - 1);
-        sg = min(sg, a.spp - 1);
+        sg = min(sg, spp_eff - 1);
         const uint32_t row = min(row0 + (rb * a.RBW + rbw) * 4u + r, a.N - 1);
-        return wslab + (uint32_t)(row * a.RB + sg * SEGB + woff + nudge);
+        return wslab + (uint32_t)(row * a.RB + min(sg * SEGB + woff, a.RB - (uint32_t)Codec::CB) + nudge);
     };
 
     const uint32_t n_pass = (MODE == GATHER_CSR || MODE == GATHER_INDICES) ? (cnt + R - 1) / R : 1u;
@@ -316,15 +323,15 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         const uint32_t live = min((uint32_t)R, cnt - base_row);
         // Rows past the pass's last live row are never staged: what the matrix
         // cores compute from their LDS slots lands in output rows nobody stores.
-        const uint32_t ntask = live * a.nch;
+        const uint32_t ntask = live * a.nchp;  // chunks past the row's end are staged as zeros
         uint32_t raw[NP * 4];
         bool row_live;
         auto x_load = [&](uint32_t task) {
-            const uint32_t i = task / a.nch, c = task - i * a.nch;
+            const uint32_t i = task / a.nchp, c = task - i * a.nchp;
             uint32_t t = batch_row(base_row + i);
-            row_live = t != NOROW;
-            if (!row_live) t = batch_row(base_row);  // the pass's first row always exists
-            const m_u32x4* src = (const m_u32x4*)((const uint16_t*)a.x + (size_t)t * a.K + (size_t)c * CPC);
+            row_live = t != NOROW && c < a.nch;
+            if (t == NOROW) t = batch_row(base_row);  // the pass's first row always exists
+            const m_u32x4* src = (const m_u32x4*)((const uint16_t*)a.x + (size_t)t * a.K + (size_t)min(c, a.nch - 1) * CPC);
 #pragma unroll
             for (int p = 0; p < NP; p++) {
                 const m_u32x4 v = src[p];
@@ -333,7 +340,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         };
         const uint32_t cpg = (1u << a.log2g) / (uint32_t)CPC;  // chunks per group: a power of two, at most 16
         auto x_store = [&](uint32_t task) {
-            const uint32_t i = task / a.nch, c = task - i * a.nch;
+            const uint32_t i = task / a.nchp, c = task - i * a.nchp;
             if (!row_live) {
 #pragma unroll
                 for (int j = 0; j < NP * 4; j++) raw[j] = 0u;
@@ -350,7 +357,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
             // all staging or all idle): butterfly over them, one lane writes. The bias term of a row
             // block is then b' . (group sums), added once per row block instead of once per chunk.
             for (uint32_t o = 1; o < cpg; o <<= 1) sum += __shfl_xor(sum, (int)o, 64);
-            if ((c & (cpg - 1u)) == 0u) XG[((size_t)s * a.gpr + c / cpg) * MP + i4] = sum;
+            if ((c & (cpg - 1u)) == 0u && c < a.nch) XG[((size_t)s * a.gpr + c / cpg) * MP + i4] = sum;
 #pragma unroll
             for (int p = 0; p < NP; p++) {
                 uint32_t o[4];
@@ -366,7 +373,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                     o[dw] = h[0] | (h[1] << 16);
                 }
                 m_u32x4 piece = {o[0], o[1], o[2], o[3]};
-                XL[(size_t)s * NP * a.nch * MP + ((((size_t)(c >> 4) * NP + p) * 16u + (c & 15u)) * MP + i4)] = piece;
+                XL[(size_t)s * NP * a.nchp * MP + ((((size_t)(c >> 4) * NP + p) * 16u + (c & 15u)) * MP + i4)] = piece;
             }
         };
         // In the gather modes this body is a loop over passes. Index math of the staging and of the
@@ -415,9 +422,9 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         const uint32_t sb_idx = sb_row + ((c_lane * (uint32_t)CPC) >> a.log2g);  // 32-bit sum: sb_row alone may have wrapped
         const unsigned char* sb_lane = (const unsigned char*)(SB + sb_idx);
         const unsigned char* sb_zero_p = (const unsigned char*)(SB + sb_zero);
-        const uint32_t xl_set = (uint32_t)NP * a.nch * MP * 16u;  // bytes from one row set to the next
+        const uint32_t xl_set = (uint32_t)NP * a.nchp * MP * 16u;  // bytes from one row set to the next
         const uint32_t part_g0 = (kp * a.spp * 16u * (uint32_t)CPC) >> a.log2g;  // this wave's K part: whole groups
-        const uint32_t part_ng = (a.spp * 16u * (uint32_t)CPC) >> a.log2g;
+        const uint32_t part_ng = min(a.gpr, ((kp * a.spp + spp_eff) * 16u * (uint32_t)CPC) >> a.log2g) - part_g0;
         auto turn = [&](auto issue_tag) {
             constexpr bool ISSUE = decltype(issue_tag)::value;
             const uint32_t row_local = (rb * a.RBW + rbw) * 4u + r;
@@ -428,8 +435,8 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
 #pragma unroll
                 for (int d = 0; d < D; d++) {
                     const uint32_t sg = sg0 + d;
-                    const bool valid = sg < a.spp;
-                    const uint32_t sgc = min(sg, a.spp - 1);  // uniform
+                    const bool valid = sg < lane_steps;
+                    const uint32_t sgc = min(sg, spp_eff - 1);  // uniform
                     // operands from LDS
                     m_u32x4 av[S][NP];
 #pragma unroll

@@ -89,3 +89,48 @@ def test_large_groups(oracle, M, G, bits, dt):
     assert rel_err(got, _expected(oracle, c)) <= TOL[dt]
     for buf in (w, s, b, x, out):
         buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.F16, DType.BF16], ids=lambda d: d.name)
+@pytest.mark.parametrize("bits", [2, 3, 4, 6, 8])
+@pytest.mark.parametrize("K", [768, 1280, 3584, 11008, 18944])
+@pytest.mark.parametrize("M", [1, 3, 8])
+def test_rows_that_are_not_whole_steps(oracle, M, K, bits, dt):
+    """Row lengths of real models that are not a whole number of the kernels' wave-wide steps
+    (768, 1280, 11008: the last step is partial) or whose step count has no small divisor
+    (3584 = 7 steps, 18944 = 37: K parts of unequal length)."""
+    N, G = 52, 64
+    c = make_case(1100 + bits + K % 97 + M, dt, bits, G, M, N, K, bias_rule="midpoint")
+    print(f"[case] row length {K} {dt.name} b{bits} M{M}", flush=True)
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    out = GpuBuffer(M * N * dt.size_bytes)
+    ops.qmv(dt, bits, G, w, s, b, x, out, M, N, K)
+    got = unpack_f32(out.read_bytes(), dt)
+    assert rel_err(got, _expected(oracle, c)) <= TOL[dt]
+    for buf in (w, s, b, x, out):
+        buf.free()
+
+
+@pytest.mark.parametrize("K", [768, 11008])
+def test_gather_rows_that_are_not_whole_steps(oracle, K):
+    E, N, G, bits, dt = 4, 44, 64, 4, DType.BF16
+    counts = [5, 0, 2, 9]
+    T = sum(counts)
+    c = make_case(1200 + K % 89, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype("<u4")
+    indices = np.repeat(np.arange(E), counts).astype("<u4")
+    exp = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=indices, f64=True, threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    for view, route, fn in (("csr", offsets, ops.gather_qmv_csr), ("indices", indices, ops.gather_qmv_indices)):
+        print(f"[case] gather {view} row length {K}", flush=True)
+        out = GpuBuffer(T * N * dt.size_bytes)
+        r = GpuBuffer.from_bytes(route.tobytes())
+        fn(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+        got = unpack_f32(out.read_bytes(), dt)
+        assert rel_err(got, exp) <= TOL[dt], view
+        out.free(); r.free()
+    for buf in (w, s, b, x):
+        buf.free()
