@@ -163,6 +163,9 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
             s_ = elem_bits_to_f32<DT>(ps[set]);
             b_ = elem_bits_to_f32<DT>(pb[set]);
         }
+        // The loop runs whole pairs of iterations; with an odd count the one past the end works on
+        // re-read operands and must add nothing: zero scale and bias make its weights zero.
+        if (it_ >= a.iters) s_ = b_ = 0.f;
     };
 
     f32x16 acc[MB];
@@ -348,8 +351,8 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
         return fail(ERR_UNSUPPORTED, "direct qmm: f16 / bf16 activations only");
     if (p.bits != 2 && p.bits != 4 && p.bits != 8) return fail(ERR_UNSUPPORTED, "direct qmm: bits must be 2, 4 or 8");
     const uint32_t G = p.group_size;
-    if (p.M == 0 || p.N % 128 || p.K % 512 || G < 32 || (G & (G - 1)) || p.K % G)
-        return fail(ERR_UNSUPPORTED, "direct qmm: N % 128, K % 512 or group size");
+    if (p.M == 0 || p.N % 128 || p.K % 64 || G < 32 || (G & (G - 1)) || p.K % G)
+        return fail(ERR_UNSUPPORTED, "direct qmm: N % 128, K % 64 or group size");
     if ((uint64_t)p.M * p.K * 2 >= (1ull << 32) || (uint64_t)p.N * p.K * p.bits / 8 >= (1ull << 32))
         return fail(ERR_UNSUPPORTED, "direct qmm: operand larger than 4 GiB");
     if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.out % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
@@ -384,7 +387,17 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
     }
     if (options().qmm_tile_rows) rows = (uint32_t)options().qmm_tile_rows;
     if (options().qmm_kgroups) kgroups = (uint32_t)options().qmm_kgroups;
-    if (rows == 32 && kgroups != 4) return fail(ERR_BAD_ARG, "qmm.tile_rows 32 needs 4 K-groups");
+    // An iteration covers 64 k per K-group: K must be a multiple of 64 * K-groups (an odd number of
+    // iterations is fine). Rows that are not (K = 11008 = 43 * 256 is, 11072 = 173 * 64 is not for 2 or
+    // 4 K-groups) take fewer K-groups.
+    while (kgroups > 1 && p.K % (64u * kgroups)) {
+        if (options().qmm_kgroups) return fail(ERR_BAD_ARG, "qmm.kgroups: K must be a multiple of 64 * K-groups");
+        kgroups /= 2;
+    }
+    if (rows == 32 && kgroups != 4) {
+        if (options().qmm_tile_rows) return fail(ERR_BAD_ARG, "qmm.tile_rows 32 needs 4 K-groups");
+        rows = 64;
+    }
     a.m_tile_rows = rows;
     // Workgroup ids congruent mod 8 share an XCD and its L2. Whichever operand is smaller is
     // streamed by every XCD and the larger one is split between them (activations larger than the
@@ -393,7 +406,7 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
     a.by_m = options().qmm_by_m == 1 || (options().qmm_by_m == 0 && x_bytes > w_bytes);
     a.m_tiles = (p.M + rows - 1) / rows;
     a.n_tiles = p.N / (kgroups == 1 ? 128 : 32 * (8 / kgroups));
-    a.iters = p.K / (64 * kgroups);  // even: K % 512 == 0
+    a.iters = p.K / (64 * kgroups);
     return p.dtype == DT_BF16 ? launch_dt<DT_BF16>(a, p.bits, kgroups, lc) : launch_dt<DT_F16>(a, p.bits, kgroups, lc);
 }
 

@@ -75,3 +75,24 @@ def test_qmm_routing_between_8_and_32_rows(oracle, M, N):
     for buf in (w, s, b, x, out):
         buf.free()
     assert rel_err(got, exp) <= 5e-2
+
+
+@pytest.mark.parametrize("K", [320, 768, 1152, 11008])
+@pytest.mark.parametrize("M", [40, 300])
+def test_tile_kernel_on_rows_of_whole_64s(oracle, M, K):
+    """Row lengths that are multiples of 64 but not of 512 (768 and 11008 are down-projection widths
+    of real models) run on the tile kernel, with fewer K-groups per workgroup or an odd number of iterations. Against the mma-semantics
+    oracle, 2e-2 as for the prefill configuration."""
+    N, G, bits, dt = 256, 64, 4, DType.BF16
+    print(f"[case] qmm M={M} K={K}", flush=True)
+    c = make_case(5300 + M + K % 101, dt, bits, G, M, N, K)
+    exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    out = GpuBuffer(M * N * dt.size_bytes)
+    ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+    got = unpack_f32(out.read_bytes(), dt)
+    for buf in (w, s, b, x, out):
+        buf.free()
+    assert rel_err(got, exp) <= 2e-2
