@@ -262,6 +262,24 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
     p.w = w; p.scales = s; p.biases = b; p.x = x; p.out = out;
     p.M = 1; p.N = N; p.K = K;
     p.gather = mode; p.route = route; p.T = mode == GATHER_SINGLE ? 1 : T; p.E = E;
+    // Many rows per expert (a prefill through an MoE layer): the GEMV family would stream every
+    // expert's weights once per 8 or 16 of its rows, so the rows go to the tile kernel, grouped by
+    // expert, like the reference's MMA gather kernels (crates/metaltile-std/src/ffai/moe.rs:2256).
+    // Measured crossover: 16 rows per expert, the most one GEMV pass takes (8 experts x 14336x4096:
+    // 16 rows each 97 us GEMV / 84 us tiles, 24 rows 139 / 87, 256 rows 588 / 88; 128 experts x
+    // 2048x768: 24 rows each 231 / 80 us; at 8 rows each the GEMV wins, 51 us against 119).
+    const int gopt = options().gather_grouped;
+    if (mode != GATHER_SINGLE && gopt != 1 && (gopt == 2 || (uint64_t)T > (uint64_t)16 * (E < T ? E : T))) {
+        QmmParams q;
+        q.dtype = dtype; q.bits = bits; q.group_size = G;
+        q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
+        q.M = T; q.N = N; q.K = K;
+        const bool ids = mode == GATHER_INDICES;
+        rc = ensure_scratch(qmm_grouped_scratch_bytes(T, E, ids));
+        if (rc) return rc;
+        rc = launch_qmm_grouped(q, route, ids, T, E, g.scratch_buf, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
     return run_gemv(p, lc);
 }
 
@@ -1123,6 +1141,11 @@ int mtq_set_option(const char* name, int value) {
     if (!strcmp(name, "qmm.by_m")) {
         if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmm.by_m must be 0 (choose), 1 or 2 (off)");
         options().qmm_by_m = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "gather.grouped")) {
+        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "gather.grouped must be 0 (choose), 1 (never) or 2 (always)");
+        options().gather_grouped = value;
         return MTQ_OK;
     }
     if (!strcmp(name, "qmm.tile_rows")) {

@@ -92,6 +92,7 @@ struct Options {
     int qmm_kernel = 0;           // MFMA qmm: 0 auto, 1 both operands through LDS, 2 weights direct to registers
     int qmm_kgroups = 0;          // direct qmm: K-groups per workgroup (0 = choose; 1, 2, 4)
     int qmm_by_m = 0;             // direct qmm: 1 = an XCD keeps its M-tiles' activations and streams all weights
+    int gather_grouped = 0;       // expert-routed rows on the tile kernel: 0 = choose by rows per expert, 1 = never, 2 = always
     int qmm_tile_rows = 0;        // direct qmm: activation rows per tile (0 = choose; 32, 64, 128)
     int qmv_mfma = 0;             // matrix-core qmv: 0 auto, 1 never, 2 whenever the shape fits
     int qmv_mfma_kp = 0;          // matrix-core qmv: K parts per row block
@@ -152,6 +153,12 @@ struct QmmParams {
 int launch_qmm_mfma(const QmmParams& p, const LaunchCtx& lc);
 // 64x128 tiles, weights converted in MFMA operand registers, activations through LDS (qmm_direct.hip).
 int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc);
+// Expert-routed rows on the same kernel (many rows per expert): p holds one expert's shapes (N, K),
+// x [T][K], out [T][N], w / scales / biases the stacked experts. `route` = CSR offsets [E + 1], or one
+// expert id per row when per_row_ids. scratch: qmm_grouped_scratch_bytes() bytes.
+size_t qmm_grouped_scratch_bytes(uint32_t T, uint32_t E, bool sort_rows);
+int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_ids, uint32_t T, uint32_t E, void* scratch,
+                       const LaunchCtx& lc);
 
 // Affine quantise (quantize = true: T[n_elem] -> packed words + scales + biases) and
 // dequantise (packed words + scales + biases -> T[n_elem]) (affine.hip).

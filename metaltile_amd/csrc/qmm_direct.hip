@@ -52,6 +52,12 @@ struct QmmDArgs {
     uint32_t m_tiles, n_tiles, iters;
     uint32_t m_tile_rows;  // 32 (4 K-groups only), 64 or 128
     uint32_t by_m;         // consecutive workgroup ids walk the N-tiles of one M-tile (else the M-tiles of one N-tile)
+    // grouped mode (expert-routed rows): tiles[0] = number of row tiles, then one uint4 per tile
+    // (expert, first row of the tile in the row order, rows in the tile, 0); rowlist maps the row
+    // order to rows of x / out (null: the identity). w / scales / biases are the stacked experts'.
+    const uint32_t* tiles;
+    const uint32_t* rowlist;
+    uint64_t w_expert_bytes, sb_expert_elems;
 };
 
 
@@ -69,7 +75,7 @@ struct QmmDArgs {
 // KG = 1 is the half-size workgroup: 4 waves, all N-waves of one K-group, 32*MB x 128 tile,
 // 64 k per iteration and no partial sums to combine. Two such workgroups share a compute unit
 // and are not in step with each other, so one's LDS traffic runs under the other's MFMAs.
-template <int DT, int BITS, int PD, int MB, bool SBL, int KG>
+template <int DT, int BITS, int PD, int MB, bool SBL, int KG, bool GR = false>
 __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArgs a) {
     constexpr int NW = KG == 1 ? 4 : 8;      // waves
     constexpr int NT = 64 * NW;              // threads
@@ -90,15 +96,32 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
 
     const uint32_t total = a.m_tiles * a.n_tiles;
     uint32_t vid = blockIdx.x;
-    if (total % 8 == 0) vid = (blockIdx.x & 7u) * (total / 8) + (blockIdx.x >> 3);
-    const uint32_t nt = a.by_m ? vid % a.n_tiles : vid / a.m_tiles, mt = a.by_m ? vid / a.n_tiles : vid % a.m_tiles;
-    const uint32_t m0 = mt * DBM, n0 = nt * DBN;
+    if (!GR && total % 8 == 0) vid = (blockIdx.x & 7u) * (total / 8) + (blockIdx.x >> 3);
+    uint32_t nt = a.by_m ? vid % a.n_tiles : vid / a.m_tiles, mt = a.by_m ? vid / a.n_tiles : vid % a.m_tiles;
+    // rows of this tile: row j of the tile is row (row_first + j) of the row order, j < row_count
+    uint32_t row_first = mt * DBM, row_count = a.M > row_first ? min((uint32_t)DBM, a.M - row_first) : 0u;
+    if constexpr (GR) {
+        nt = blockIdx.x % a.n_tiles;
+        mt = blockIdx.x / a.n_tiles;
+        if (mt >= a.tiles[0]) return;  // the grid is sized for the worst routing
+        const uint4 t = ((const uint4*)a.tiles)[1 + mt];
+        row_first = t.y;
+        row_count = t.z;
+        a.w += (size_t)t.x * a.w_expert_bytes;
+        a.scales += (size_t)t.x * a.sb_expert_elems * 2;
+        a.biases += (size_t)t.x * a.sb_expert_elems * 2;
+    }
+    auto row_of = [&](uint32_t j) -> uint32_t {  // j < row_count
+        if constexpr (GR) return a.rowlist ? a.rowlist[row_first + j] : row_first + j;
+        else return row_first + j;
+    };
+    const uint32_t n0 = nt * DBN;
 
     // activations: thread t moves 32 bytes of row t/TPR (bytes [32*(t%TPR), +32) of the iteration's row)
     const uint32_t xr = tid / TPR, xc = tid % TPR;
     uint32_t xoff[XV / 2];
 #pragma unroll
-    for (int i = 0; i < XV / 2; i++) xoff[i] = min(m0 + xr + RS * i, a.M - 1) * (a.K * 2) + xc * 32;
+    for (int i = 0; i < XV / 2; i++) xoff[i] = row_of(min(xr + RS * i, row_count - 1)) * (a.K * 2) + xc * 32;
     // weights: row n0 + 32*wn + fr, codes [64*kg + 32*fh, +32) of the iteration
     const uint32_t wrow = n0 + wn * 32 + fr;  // < N: N is a multiple of the tile width
     const uint32_t woff = wrow * (a.K * BITS / 8) + (kg * 64 + fh * 32) * BITS / 8;
@@ -303,9 +326,8 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
         const uint32_t v = tid + i * NT, lrow = v / VPR, c16 = v % VPR;
-        const uint32_t row = m0 + lrow;
-        if (row < a.M && (DBM * VPR % NT == 0 || lrow < (uint32_t)DBM))
-            *(q_u32x4*)((uint16_t*)a.out + (size_t)row * a.N + n0 + c16 * 8) = *(const q_u32x4*)(otile + lrow * DBN + c16 * 8);
+        if (lrow < row_count)
+            *(q_u32x4*)((uint16_t*)a.out + (size_t)row_of(lrow) * a.N + n0 + c16 * 8) = *(const q_u32x4*)(otile + lrow * DBN + c16 * 8);
     }
 }
 
@@ -318,7 +340,7 @@ static size_t lds_need(uint32_t rows, uint32_t kg, uint32_t gpr, bool sbl) {
     return main_loop > epilogue ? main_loop : epilogue;
 }
 
-template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, const LaunchCtx& lc) {
+template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, const LaunchCtx& lc, bool grouped = false) {
     const void* fn;
     const bool tall = a.m_tile_rows == 128;
     const uint32_t dbn = kgroups == 1 ? 128 : 32 * (8 / kgroups);
@@ -338,6 +360,16 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
     }
 #undef QD_PICK
 #undef QD_PICK3
+    if (grouped) {  // 64-row tiles, 2 or 4 K-groups
+#define QD_G(B, KGv) (sbl ? (const void*)qmm_direct_kernel<DT, B, 2, 2, true, KGv, true> : (const void*)qmm_direct_kernel<DT, B, 2, 2, false, KGv, true>)
+        if (a.m_tile_rows != 64 || (kgroups != 2 && kgroups != 4)) return fail(ERR_UNSUPPORTED, "grouped qmm: tile shape");
+        switch (bits) {
+            case 2: fn = kgroups == 4 ? QD_G(2, 4) : QD_G(2, 2); break;
+            case 4: fn = kgroups == 4 ? QD_G(4, 4) : QD_G(4, 2); break;
+            default: fn = kgroups == 4 ? QD_G(8, 4) : QD_G(8, 2); break;
+        }
+#undef QD_G
+    }
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     void* args[] = {&a};
@@ -408,6 +440,107 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
     a.n_tiles = p.N / (kgroups == 1 ? 128 : 32 * (8 / kgroups));
     a.iters = p.K / (64 * kgroups);
     return p.dtype == DT_BF16 ? launch_dt<DT_BF16>(a, p.bits, kgroups, lc) : launch_dt<DT_F16>(a, p.bits, kgroups, lc);
+}
+
+// ---- expert-routed rows on the tile kernel ---------------------------------------------------
+// Builds the table of row tiles: for every expert, its rows in the row order cut into tiles of
+// `tile_rows`. CSR routing follows the reference's rule (crates/metaltile-std/src/ffai/moe.rs:376-385):
+// row t belongs to the first expert e with t < off[e + 1], rows past every offset to expert 0; so
+// expert e owns [max(off[1..e]), min(off[e + 1], T)) and expert 0 also the tail [max(off), T).
+// With sorted == 1 the offsets are a plain prefix sum over a sorted row list.
+struct TileTabArgs {
+    const uint32_t* off;  // [E + 1]
+    uint32_t* tiles;      // [4 + 4 * max_tiles]
+    uint32_t E, T, tile_rows, max_tiles;
+};
+__global__ __launch_bounds__(64) void gather_tiles_kernel(TileTabArgs a) {
+    if (threadIdx.x != 0) return;  // E is small next to the GEMM that follows: one lane, in order
+    uint32_t n = 0, mx = 0;
+    uint4* tab = (uint4*)a.tiles + 1;
+    auto emit = [&](uint32_t e, uint32_t lo, uint32_t hi) {
+        for (uint32_t r = lo; r < hi && n < a.max_tiles; r += a.tile_rows, n++) tab[n] = make_uint4(e, r, min(a.tile_rows, hi - r), 0u);
+    };
+    for (uint32_t e = 0; e < a.E; e++) {
+        const uint32_t lo = min(mx, a.T), hi = min(a.off[e + 1], a.T);
+        if (hi > lo) emit(e, lo, hi);
+        mx = max(mx, a.off[e + 1]);
+    }
+    if (mx < a.T) emit(0u, mx, a.T);
+    a.tiles[0] = n;
+}
+
+size_t qmm_grouped_scratch_bytes(uint32_t T, uint32_t E, bool sort_rows) {
+    const size_t max_tiles = (size_t)(T + 63) / 64 + E + 1;
+    size_t b = 16 + max_tiles * 16;
+    if (sort_rows) b += ((size_t)2 * T + E + 1 + 3) / 4 * 16;  // sorted row list, inverse permutation, offsets
+    return b;
+}
+
+// x [T][K], out [T][N], stacked w / scales / biases [E][N][...]; route = CSR offsets [E + 1] or,
+// with per_row_ids, one expert id per row (sorted by expert here, on the device).
+int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_ids, uint32_t T, uint32_t E, void* scratch,
+                       const LaunchCtx& lc) {
+    if (p.dtype != DT_F16 && p.dtype != DT_BF16) return fail(ERR_UNSUPPORTED, "grouped qmm: f16 / bf16 only");
+    if (p.bits != 2 && p.bits != 4 && p.bits != 8) return fail(ERR_UNSUPPORTED, "grouped qmm: bits must be 2, 4 or 8");
+    const uint32_t G = p.group_size;
+    if (T == 0 || p.N % 128 || p.K % 128 || G < 32 || (G & (G - 1)) || p.K % G)
+        return fail(ERR_UNSUPPORTED, "grouped qmm: N % 128, K % 128 or group size");
+    if ((uint64_t)T * p.K * 2 >= (1ull << 32) || (uint64_t)p.N * p.K * p.bits / 8 >= (1ull << 32) || (uint64_t)T * p.N * 2 >= (1ull << 34))
+        return fail(ERR_UNSUPPORTED, "grouped qmm: operand too large");
+    if (E > 2048) return fail(ERR_UNSUPPORTED, "grouped qmm: more than 2048 experts");
+    if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.out % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
+        return fail(ERR_UNSUPPORTED, "grouped qmm: operands must be 16-byte aligned");
+    const uint32_t max_tiles = (T + 63) / 64 + E + 1;
+    uint32_t* tiles = (uint32_t*)scratch;
+    const uint32_t* off = route;
+    const uint32_t* rowlist = nullptr;
+    LaunchCtx first = lc, mid = lc, last = lc;
+    first.stop = nullptr;
+    mid.start = mid.stop = nullptr;
+    last.start = nullptr;
+    bool started = false;
+    if (per_row_ids) {
+        uint32_t* sorted = tiles + 4 + (size_t)max_tiles * 4;
+        uint32_t* inv = sorted + T;
+        uint32_t* offs = inv + T;
+        int rc = launch_moe_sort(route, T, 1, E, sorted, inv, offs, first);
+        if (rc) return rc;
+        started = true;
+        off = offs;
+        rowlist = sorted;
+    }
+    TileTabArgs ta{off, tiles, E, T, 64u, max_tiles};
+    void* targs[] = {&ta};
+    hipError_t e = launch_kernel((const void*)gather_tiles_kernel, dim3(1), dim3(64), targs, 0, started ? mid : first);
+    if (e != hipSuccess) return hip_fail(e, "gather tile table kernel launch");
+
+    QmmDArgs a;
+    a.w = (const unsigned char*)p.w;
+    a.scales = (const unsigned char*)p.scales;
+    a.biases = (const unsigned char*)p.biases;
+    a.x = (const unsigned char*)p.x;
+    a.out = p.out;
+    a.M = T;
+    a.N = p.N;
+    a.K = p.K;
+    uint32_t l = 0;
+    while ((1u << l) < G) l++;
+    a.log2g = l;
+    a.gpr = p.K / G;
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    // 64 x 128 tiles; 64 x 64 on 4 K-groups when that still leaves fewer tiles than compute units
+    uint32_t kgroups = ((uint64_t)((T + 63) / 64) * (p.N / 128) * 2 <= (uint64_t)cus && p.K % 256 == 0) ? 4 : 2;
+    a.m_tile_rows = 64;
+    a.m_tiles = max_tiles;
+    a.n_tiles = p.N / (32 * (8 / kgroups));
+    a.iters = p.K / (64 * kgroups);
+    a.by_m = 1;
+    a.tiles = tiles;
+    a.rowlist = rowlist;
+    a.w_expert_bytes = (uint64_t)p.N * p.K * p.bits / 8;
+    a.sb_expert_elems = (uint64_t)p.N * a.gpr;
+    return p.dtype == DT_BF16 ? launch_dt<DT_BF16>(a, p.bits, kgroups, last, true) : launch_dt<DT_F16>(a, p.bits, kgroups, last, true);
 }
 
 }  // namespace mtq

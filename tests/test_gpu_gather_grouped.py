@@ -1,0 +1,115 @@
+"""gather_qmv with many rows per expert: the rows are grouped by expert on the device and run on the
+MFMA tile kernel (the regime of the reference's mt_moe_gather_qmm_mma_* kernels,
+crates/metaltile-std/src/ffai/moe.rs:2256). Checked per expert against the oracle's mma semantics
+(weights rounded to the element dtype first), 2e-2 on max|a-e| / max(|e|, 1), and against exact
+dequantisation at the reference's bf16 bound of 5e-2; both routing views, sorted and unsorted ids,
+an empty expert, ragged last tiles, and the CSR rule that rows past every offset belong to expert 0."""
+import numpy as np
+import pytest
+
+from metaltile_amd import DType, GpuBuffer, _lib, ops, unpack_f32
+from metaltile_amd.synth import make_case
+from tests.parity import rel_err
+
+pytestmark = pytest.mark.gpu
+ODT = {DType.F16: 1, DType.BF16: 2}
+
+
+@pytest.fixture
+def grouped():
+    lib = _lib.load()
+
+    def set_(value):
+        assert lib.mtq_set_option(b"gather.grouped", value) == 0
+
+    yield set_
+    lib.mtq_set_option(b"gather.grouped", 0)
+
+
+def _expected(oracle, c, ids, T, N, K, E, bits, G, dt):
+    """Row t against expert ids[t], mma semantics, computed expert by expert."""
+    exp = np.zeros((T, N), np.float32)
+    wpe, spe = N * K * bits // 32, N * (K // G)
+    x = c.x_f.reshape(T, K)
+    for e in range(E):
+        rows = np.nonzero(ids == e)[0]
+        if rows.size == 0:
+            continue
+        part = oracle.qmm_mma(c.w[e * wpe:(e + 1) * wpe], c.scales_f[e * spe:(e + 1) * spe], c.biases_f[e * spe:(e + 1) * spe],
+                              np.ascontiguousarray(x[rows]).reshape(-1), rows.size, N, K, bits, G, ODT[dt], threads=8)
+        exp[rows] = part.reshape(rows.size, N)
+    return oracle.round_through(exp.reshape(-1), ODT[dt])
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_grouped_gather_both_views(oracle, grouped, bits, dt):
+    E, N, K, G = 5, 256, 512, 64
+    counts = [40, 0, 70, 3, 64]
+    T = sum(counts)
+    c = make_case(7100 + bits, dt, bits, G, T, N, K, E=E)
+    ids_sorted = np.repeat(np.arange(E), counts).astype("<u4")
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype("<u4")
+    rng = np.random.default_rng(3)
+    ids_shuffled = ids_sorted[rng.permutation(T)]
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    exact = oracle.round_through(oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=ids_sorted,
+                                                   f64=True, threads=8).astype(np.float32), ODT[dt])
+    grouped(2)
+    for view, route, fn, ids in (("csr", offsets, ops.gather_qmv_csr, ids_sorted),
+                                 ("indices sorted", ids_sorted, ops.gather_qmv_indices, ids_sorted),
+                                 ("indices shuffled", ids_shuffled, ops.gather_qmv_indices, ids_shuffled)):
+        print(f"[case] grouped gather {view} {dt.name} b{bits}", flush=True)
+        out = GpuBuffer(T * N * dt.size_bytes)
+        r = GpuBuffer.from_bytes(route.tobytes())
+        fn(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+        got = unpack_f32(out.read_bytes(), dt)
+        out.free(); r.free()
+        assert rel_err(got, _expected(oracle, c, ids, T, N, K, E, bits, G, dt)) <= 2e-2, view
+        # (rounding s*q + b of an 8-bit code to a 16-bit element moves it by more than this bound allows
+        # on near-zero outputs: 8-bit cases are held to the mma-semantics oracle only)
+        if ids is ids_sorted and bits <= 4:
+            assert rel_err(got, exact) <= 5e-2, view
+    for buf in (w, s, b, x):
+        buf.free()
+
+
+def test_grouped_gather_csr_tail_rows_go_to_expert_0(oracle, grouped):
+    """Offsets that stop short of T: the reference's rule sends the remaining rows to expert 0."""
+    dt, bits, E, N, K, G = DType.BF16, 4, 3, 128, 256, 64
+    offsets = np.array([0, 10, 10, 75], "<u4")     # expert 1 empty, rows 75..99 past every offset
+    T = 100
+    ids = np.concatenate([np.zeros(10), np.full(65, 2), np.zeros(25)]).astype("<u4")
+    c = make_case(7200, dt, bits, G, T, N, K, E=E)
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    grouped(2)
+    out = GpuBuffer(T * N * 2)
+    r = GpuBuffer.from_bytes(offsets.tobytes())
+    ops.gather_qmv_csr(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+    got = unpack_f32(out.read_bytes(), dt)
+    assert rel_err(got, _expected(oracle, c, ids, T, N, K, E, bits, G, dt)) <= 2e-2
+    for buf in (w, s, b, x, out, r):
+        buf.free()
+
+
+def test_gather_switches_to_the_tile_kernel_by_itself(oracle):
+    """64 rows per expert: chosen without the option; same bounds."""
+    dt, bits, E, N, K, G = DType.BF16, 4, 4, 256, 1024, 64
+    T = 64 * E
+    c = make_case(7300, dt, bits, G, T, N, K, E=E)
+    rng = np.random.default_rng(5)
+    ids = rng.integers(0, E, size=T).astype("<u4")
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    out = GpuBuffer(T * N * 2)
+    r = GpuBuffer.from_bytes(ids.tobytes())
+    ops.gather_qmv_indices(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+    got = unpack_f32(out.read_bytes(), dt)
+    exact = oracle.round_through(oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=ids,
+                                                   f64=True, threads=8).astype(np.float32), 2)
+    assert rel_err(got, exact) <= 5e-2
+    assert rel_err(got, _expected(oracle, c, ids, T, N, K, E, bits, G, dt)) <= 2e-2
+    for buf in (w, s, b, x, out, r):
+        buf.free()
