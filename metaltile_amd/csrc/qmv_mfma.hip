@@ -65,8 +65,8 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     const uint32_t G = p.group_size;
     if (!is_pow2(G) || G < cpc || G > 16u * cpc || p.K % G) return fail(ERR_UNSUPPORTED, "mfma qmv: group size");
     const uint32_t gpr = p.K / G;
-    if (gpr % 4) return fail(ERR_UNSUPPORTED, "mfma qmv: groups per row not a multiple of 4");
-    if ((uintptr_t)p.w % (odd ? 4 : 16) || (uintptr_t)p.x % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
+    if ((uintptr_t)p.w % (odd ? 4 : 16) || (uintptr_t)p.x % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16 ||
+        (rb64 % 16 && !odd) || (p.K * 2) % 16)
         return fail(ERR_UNSUPPORTED, "mfma qmv: operands must be 16-byte aligned");
     const bool gather = p.gather == GATHER_CSR || p.gather == GATHER_INDICES;
     const uint32_t rows = gather ? p.T : (p.gather == GATHER_SINGLE ? 1u : p.M);

@@ -278,9 +278,24 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     auto sbw_load = [&](uint32_t rb, SbRegs& o, uint32_t nudge = 0u) {  // nudge: an opaque zero, see the pass loop
         rb = min(rb, a.nrb - 1);
         const uint32_t row = min(row0 + (rb * a.RBW + rbw) * 4u + (lane & 3u), a.N - 1);
-        const uint32_t src = row * a.gpr + min(g_lo + (lane >> 2) * 4u, a.gpr - 4) + nudge;
-        o.s = *(const uint2*)(sslab + src);
-        o.b = *(const uint2*)(bslab + src);
+        if (a.gpr & 3u) {
+            // rows of scales that are not a whole number of 8-byte vectors (K / G = 14, 18, 22, 45 ...):
+            // element loads, each clamped to the row
+            const uint32_t g0 = g_lo + (lane >> 2) * 4u, base = row * a.gpr + nudge;
+            uint32_t e[4], f[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t idx = base + min(g0 + (uint32_t)j, a.gpr - 1);
+                e[j] = sslab[idx];
+                f[j] = bslab[idx];
+            }
+            o.s = make_uint2(e[0] | (e[1] << 16), e[2] | (e[3] << 16));
+            o.b = make_uint2(f[0] | (f[1] << 16), f[2] | (f[3] << 16));
+        } else {
+            const uint32_t src = row * a.gpr + min(g_lo + (lane >> 2) * 4u, a.gpr - 4) + nudge;
+            o.s = *(const uint2*)(sslab + src);
+            o.b = *(const uint2*)(bslab + src);
+        }
     };
     auto sbw_store = [&](const SbRegs& o) {
         if (lane < a.gpw) {  // gpw / 4 vectors for each of the 4 rows

@@ -93,12 +93,13 @@ def test_large_groups(oracle, M, G, bits, dt):
 
 @pytest.mark.parametrize("dt", [DType.F16, DType.BF16], ids=lambda d: d.name)
 @pytest.mark.parametrize("bits", [2, 3, 4, 6, 8])
-@pytest.mark.parametrize("K", [768, 1280, 3584, 11008, 18944])
+@pytest.mark.parametrize("K", [768, 896, 1152, 1280, 2880, 3584, 11008, 18944])
 @pytest.mark.parametrize("M", [1, 3, 8])
 def test_rows_that_are_not_whole_steps(oracle, M, K, bits, dt):
     """Row lengths of real models that are not a whole number of the kernels' wave-wide steps
     (768, 1280, 11008: the last step is partial) or whose step count has no small divisor
-    (3584 = 7 steps, 18944 = 37: K parts of unequal length)."""
+    (3584 = 7 steps, 18944 = 37: K parts of unequal length), or whose rows of scales are not whole
+    8-byte vectors (896, 1152, 2880: 14, 18, 45 groups)."""
     N, G = 52, 64
     c = make_case(1100 + bits + K % 97 + M, dt, bits, G, M, N, K, bias_rule="midpoint")
     print(f"[case] row length {K} {dt.name} b{bits} M{M}", flush=True)
