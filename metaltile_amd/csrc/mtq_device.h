@@ -294,4 +294,36 @@ template <int DT, int BITS> struct XSlice<DT, BITS, false> {
     }
 };
 
+// Rows of one expert under the reference's CSR rule (crates/metaltile-std/src/ffai/moe.rs:376-385):
+// row t belongs to the first expert e with t < off[e + 1], rows past every offset to expert 0. So
+// expert e owns [max(off[1..e]), min(off[e + 1], T)) and expert 0 also the tail [max(off), T).
+// Called by whole waves with a uniform expert; each wave scans the offsets 64 at a time. An expert
+// whose own offsets already leave it empty returns before the scan: with many experts and few rows
+// most workgroups are such, and a per-workgroup scan of every offset was the whole cost of the launch
+// (256 experts, 8 rows: 408 us, against 27 us for the same routing as per-row ids).
+__device__ __forceinline__ uint32_t csr_expert_rows(const uint32_t* off, uint32_t E, uint32_t T, uint32_t expert, uint32_t lane,
+                                                    uint32_t& lo, uint32_t& n1, uint32_t& lo2) {
+    const uint32_t o_hi = off[expert + 1];
+    lo = n1 = lo2 = 0;
+    if (expert != 0 && o_hi <= off[expert]) return 0;  // hi <= off[e] <= max(off[1..e]): no row
+    uint32_t l = 0, mx = 0;
+    for (uint32_t j0 = 1; j0 <= E; j0 += 64) {
+        const uint32_t j = j0 + lane;
+        const uint32_t o = j <= E ? off[j] : 0u;
+        if (j <= expert) l = max(l, o);
+        mx = max(mx, o);
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) {
+        l = max(l, (uint32_t)__shfl_xor((int)l, d, 64));
+        mx = max(mx, (uint32_t)__shfl_xor((int)mx, d, 64));
+    }
+    const uint32_t hi = min(o_hi, T);
+    lo = l;
+    n1 = hi > lo ? hi - lo : 0;
+    lo2 = min(mx, T);
+    const uint32_t n2 = expert == 0 ? T - lo2 : 0;
+    return n1 + n2;
+}
+
 }  // namespace mtq

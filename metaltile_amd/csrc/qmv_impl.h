@@ -138,18 +138,7 @@ __global__ __launch_bounds__(MAXT) void qmv_kernel(QmvKArgs a) {
         // E(t) = first e with t < off[e+1], else 0
         // (crates/metaltile-std/src/ffai/moe.rs:376-385): for expert e that is
         // t in [max(off[1..e]), off[e+1]); rows past every offset fall to expert 0.
-        uint32_t mx = 0, l = 0;
-        for (uint32_t j = 1; j <= a.E; j++) {
-            uint32_t o = a.route[j];
-            if (j <= expert) l = max(l, o);
-            mx = max(mx, o);
-        }
-        uint32_t hi = min(a.route[expert + 1], a.T);
-        lo = l;
-        n1 = hi > lo ? hi - lo : 0;
-        lo2 = min(mx, a.T);
-        uint32_t n2 = expert == 0 ? a.T - lo2 : 0;
-        cnt = n1 + n2;
+        cnt = csr_expert_rows(a.route, a.E, a.T, expert, lane, lo, n1, lo2);
         if (cnt == 0) return;
     } else if constexpr (MODE == GATHER_INDICES) {
         expert = blockIdx.y;
