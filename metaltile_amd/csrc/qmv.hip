@@ -242,17 +242,20 @@ static int launch_qmv_dot2(const QmvParams& p, const LaunchCtx& lc) {
     const uint32_t tpb = C * rps;
     if (tpb % 64) return fail(ERR_UNSUPPORTED, "fast qmv: workgroup not a whole number of waves");
 
-    if (!gather && p.gather != GATHER_SINGLE && rows > 4) {
-        // more activation rows than one pass holds: run passes of up to 4 rows
+    // Rows per pass: 4, except that a thread's slice of an f32 activation row for 2-bit codes is 64
+    // floats, and two of those no longer fit the register file (2 rows: 35 us against 2 x 5.6).
+    const uint32_t pass_rows = (p.dtype == DT_F32 && p.bits == 2) ? 1u : 4u;
+    if (!gather && p.gather != GATHER_SINGLE && rows > pass_rows) {
+        // more activation rows than one pass holds
         const size_t esz = p.dtype == DT_F32 ? 4 : 2;
-        for (uint32_t m0 = 0; m0 < rows; m0 += 4) {
+        for (uint32_t m0 = 0; m0 < rows; m0 += pass_rows) {
             QmvParams q = p;
-            q.M = rows - m0 < 4 ? rows - m0 : 4;
+            q.M = rows - m0 < pass_rows ? rows - m0 : pass_rows;
             q.x = (const char*)p.x + (size_t)m0 * p.K * esz;
             q.out = (char*)p.out + (size_t)m0 * p.N * esz;
             LaunchCtx l2 = lc;
             if (m0) l2.start = nullptr;
-            if (m0 + 4 < rows) l2.stop = nullptr;
+            if (m0 + pass_rows < rows) l2.stop = nullptr;
             int rc = launch_qmv_fast(q, l2);
             if (rc) return rc;
         }
