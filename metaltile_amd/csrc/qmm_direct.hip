@@ -447,11 +447,12 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
 // `tile_rows`. CSR routing follows the reference's rule (crates/metaltile-std/src/ffai/moe.rs:376-385):
 // row t belongs to the first expert e with t < off[e + 1], rows past every offset to expert 0; so
 // expert e owns [max(off[1..e]), min(off[e + 1], T)) and expert 0 also the tail [max(off), T).
-// With sorted == 1 the offsets are a plain prefix sum over a sorted row list.
+// With tail_to_0 == 0 (offsets from the sort of per-row ids) rows past the last offset are rows
+// whose id names no expert: they get no tile, so their output rows stay untouched.
 struct TileTabArgs {
     const uint32_t* off;  // [E + 1]
     uint32_t* tiles;      // [4 + 4 * max_tiles]
-    uint32_t E, T, tile_rows, max_tiles;
+    uint32_t E, T, tile_rows, max_tiles, tail_to_0;
 };
 __global__ __launch_bounds__(64) void gather_tiles_kernel(TileTabArgs a) {
     if (threadIdx.x != 0) return;  // E is small next to the GEMM that follows: one lane, in order
@@ -465,14 +466,14 @@ __global__ __launch_bounds__(64) void gather_tiles_kernel(TileTabArgs a) {
         if (hi > lo) emit(e, lo, hi);
         mx = max(mx, a.off[e + 1]);
     }
-    if (mx < a.T) emit(0u, mx, a.T);
+    if (a.tail_to_0 && mx < a.T) emit(0u, mx, a.T);
     a.tiles[0] = n;
 }
 
 size_t qmm_grouped_scratch_bytes(uint32_t T, uint32_t E, bool sort_rows) {
     const size_t max_tiles = (size_t)(T + 63) / 64 + E + 1;
     size_t b = 16 + max_tiles * 16;
-    if (sort_rows) b += ((size_t)2 * T + E + 1 + 3) / 4 * 16;  // sorted row list, inverse permutation, offsets
+    if (sort_rows) b += ((size_t)2 * T + E + 2 + 3) / 4 * 16;  // sorted row list, inverse permutation, offsets of E + 1 buckets
     return b;
 }
 
@@ -487,7 +488,7 @@ int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_i
         return fail(ERR_UNSUPPORTED, "grouped qmm: N % 128, K % 128 or group size");
     if ((uint64_t)T * p.K * 2 >= (1ull << 32) || (uint64_t)p.N * p.K * p.bits / 8 >= (1ull << 32) || (uint64_t)T * p.N * 2 >= (1ull << 34))
         return fail(ERR_UNSUPPORTED, "grouped qmm: operand too large");
-    if (E > 2048) return fail(ERR_UNSUPPORTED, "grouped qmm: more than 2048 experts");
+    if (E >= 2048) return fail(ERR_UNSUPPORTED, "grouped qmm: 2048 experts or more");
     if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.out % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
         return fail(ERR_UNSUPPORTED, "grouped qmm: operands must be 16-byte aligned");
     const uint32_t max_tiles = (T + 63) / 64 + E + 1;
@@ -503,13 +504,15 @@ int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_i
         uint32_t* sorted = tiles + 4 + (size_t)max_tiles * 4;
         uint32_t* inv = sorted + T;
         uint32_t* offs = inv + T;
-        int rc = launch_moe_sort(route, T, 1, E, sorted, inv, offs, first);
+        // one bucket more than experts: the sort clamps ids to its last bucket, which so collects the
+        // rows whose id names no expert
+        int rc = launch_moe_sort(route, T, 1, E + 1, sorted, inv, offs, first);
         if (rc) return rc;
         started = true;
         off = offs;
         rowlist = sorted;
     }
-    TileTabArgs ta{off, tiles, E, T, 64u, max_tiles};
+    TileTabArgs ta{off, tiles, E, T, 64u, max_tiles, per_row_ids ? 0u : 1u};
     void* targs[] = {&ta};
     hipError_t e = launch_kernel((const void*)gather_tiles_kernel, dim3(1), dim3(64), targs, 0, started ? mid : first);
     if (e != hipSuccess) return hip_fail(e, "gather tile table kernel launch");

@@ -113,3 +113,29 @@ def test_gather_switches_to_the_tile_kernel_by_itself(oracle):
     assert rel_err(got, _expected(oracle, c, ids, T, N, K, E, bits, G, dt)) <= 2e-2
     for buf in (w, s, b, x, out, r):
         buf.free()
+
+
+def test_grouped_gather_rows_without_an_expert_stay_untouched(oracle, grouped):
+    """Per-row ids >= E name no expert: those output rows are not written (include/mtq.h), also on the
+    tile path."""
+    dt, bits, E, N, K, G = DType.BF16, 4, 3, 128, 256, 64
+    T = 90
+    rng = np.random.default_rng(9)
+    ids = rng.integers(0, E, size=T).astype("<u4")
+    ids[[5, 17, 60]] = [E, E + 7, 0xFFFFFFFF]
+    c = make_case(7400, dt, bits, G, T, N, K, E=E)
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    sentinel = np.full(T * N, 0x7B7B, np.uint16)
+    grouped(2)
+    out = GpuBuffer.from_bytes(sentinel.tobytes())
+    r = GpuBuffer.from_bytes(ids.tobytes())
+    ops.gather_qmv_indices(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+    raw = np.frombuffer(out.read_bytes(), np.uint16).reshape(T, N)
+    got = unpack_f32(raw.tobytes(), dt).reshape(T, N)
+    valid = ids < E
+    assert np.all(raw[~valid] == 0x7B7B)
+    exp = _expected(oracle, c, np.where(valid, ids, E + 1).astype("<u4"), T, N, K, E, bits, G, dt).reshape(T, N)
+    assert rel_err(got[valid].reshape(-1), exp[valid].reshape(-1)) <= 2e-2
+    for buf in (w, s, b, x, out, r):
+        buf.free()
