@@ -123,7 +123,8 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
 #pragma unroll
     for (int i = 0; i < XV / 2; i++) xoff[i] = row_of(min(xr + RS * i, row_count - 1)) * (a.K * 2) + xc * 32;
     // weights: row n0 + 32*wn + fr, codes [64*kg + 32*fh, +32) of the iteration
-    const uint32_t wrow = n0 + wn * 32 + fr;  // < N: N is a multiple of the tile width
+    // the last tile of a ragged N works its missing rows on row N - 1 and stores none of their columns
+    const uint32_t wrow = min(n0 + wn * 32 + fr, a.N - 1);
     const uint32_t woff = wrow * (a.K * BITS / 8) + (kg * 64 + fh * 32) * BITS / 8;
     const uint32_t soff = wrow * a.gpr * 2;
     const uint32_t kofs = kg * 64 + fh * 32;  // k offset of this lane's codes inside an iteration
@@ -206,8 +207,9 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
         const uint32_t vpr = a.gpr / 8, nvec = DBN * vpr;
         for (uint32_t v = tid; v < nvec; v += NT) {
             const uint32_t row = v / vpr, c0 = (v - row * vpr) * 8;
-            const q_u32x4 sv = *(const q_u32x4*)((const uint16_t*)a.scales + (size_t)(n0 + row) * a.gpr + c0);
-            const q_u32x4 bv = *(const q_u32x4*)((const uint16_t*)a.biases + (size_t)(n0 + row) * a.gpr + c0);
+            const uint32_t grow = min(n0 + row, a.N - 1);
+            const q_u32x4 sv = *(const q_u32x4*)((const uint16_t*)a.scales + (size_t)grow * a.gpr + c0);
+            const q_u32x4 bv = *(const q_u32x4*)((const uint16_t*)a.biases + (size_t)grow * a.gpr + c0);
             uint32_t* ds = (uint32_t*)(sbS + row * sbld + c0);
             uint32_t* db = (uint32_t*)(sbB + row * sbld + c0);
             ds[0] = sv.x; ds[1] = sv.y; ds[2] = sv.z; ds[3] = sv.w;
@@ -323,11 +325,20 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
     // all threads store the tile, 16 bytes each, whole rows
     constexpr int VPR = DBN / 8;                    // 16-byte vectors per tile row
     constexpr int VPT = (DBM * VPR + NT - 1) / NT;  // vectors per thread
+    if ((a.N & 7u) == 0) {
 #pragma unroll
-    for (int i = 0; i < VPT; i++) {
-        const uint32_t v = tid + i * NT, lrow = v / VPR, c16 = v % VPR;
-        if (lrow < row_count)
-            *(q_u32x4*)((uint16_t*)a.out + (size_t)row_of(lrow) * a.N + n0 + c16 * 8) = *(const q_u32x4*)(otile + lrow * DBN + c16 * 8);
+        for (int i = 0; i < VPT; i++) {
+            const uint32_t v = tid + i * NT, lrow = v / VPR, col = n0 + (v % VPR) * 8;
+            if (lrow < row_count && col < a.N)
+                *(q_u32x4*)((uint16_t*)a.out + (size_t)row_of(lrow) * a.N + col) = *(const q_u32x4*)(otile + lrow * DBN + (v % VPR) * 8);
+        }
+    } else {
+        // output rows that are not whole 16-byte vectors: element stores, neighbouring lanes on
+        // neighbouring columns
+        for (uint32_t e = tid; e < (uint32_t)(DBM * DBN); e += NT) {
+            const uint32_t lrow = e / DBN, col = n0 + e % DBN;
+            if (lrow < row_count && col < a.N) ((uint16_t*)a.out)[(size_t)row_of(lrow) * a.N + col] = otile[e];
+        }
     }
 }
 
@@ -383,8 +394,8 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
         return fail(ERR_UNSUPPORTED, "direct qmm: f16 / bf16 activations only");
     if (p.bits != 2 && p.bits != 4 && p.bits != 8) return fail(ERR_UNSUPPORTED, "direct qmm: bits must be 2, 4 or 8");
     const uint32_t G = p.group_size;
-    if (p.M == 0 || p.N % 128 || p.K % 64 || G < 32 || (G & (G - 1)) || p.K % G)
-        return fail(ERR_UNSUPPORTED, "direct qmm: N % 128, K % 64 or group size");
+    if (p.M == 0 || p.N == 0 || p.K % 64 || G < 32 || (G & (G - 1)) || p.K % G)
+        return fail(ERR_UNSUPPORTED, "direct qmm: K % 64 or group size");
     if ((uint64_t)p.M * p.K * 2 >= (1ull << 32) || (uint64_t)p.N * p.K * p.bits / 8 >= (1ull << 32))
         return fail(ERR_UNSUPPORTED, "direct qmm: operand larger than 4 GiB");
     if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.out % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
@@ -408,8 +419,8 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
     // half the chip idle, 64 x 64 tiles on 4 K-groups (M = 128: 18.6 us against 26).
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    const uint64_t tall_wide = (uint64_t)((p.M + 127) / 128) * (p.N / 128);
-    const uint64_t short_wide = (uint64_t)((p.M + 63) / 64) * (p.N / 128);
+    const uint64_t tall_wide = (uint64_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
+    const uint64_t short_wide = (uint64_t)((p.M + 63) / 64) * ((p.N + 127) / 128);
     uint32_t rows = 64, kgroups = 2;
     if (tall_wide >= 2 * (uint64_t)cus) { rows = 128; kgroups = 1; }  // two 4-wave workgroups per CU (M = 2048: 72-75 us against 80-84; M = 4096: 160-170 against 180-190)
     else if (tall_wide >= (uint64_t)cus) { rows = 128; kgroups = 2; }
@@ -437,7 +448,8 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
     const uint64_t x_bytes = (uint64_t)p.M * p.K * 2, w_bytes = (uint64_t)p.N * p.K * p.bits / 8;
     a.by_m = options().qmm_by_m == 1 || (options().qmm_by_m == 0 && x_bytes > w_bytes);
     a.m_tiles = (p.M + rows - 1) / rows;
-    a.n_tiles = p.N / (kgroups == 1 ? 128 : 32 * (8 / kgroups));
+    const uint32_t tile_cols = kgroups == 1 ? 128 : 32 * (8 / kgroups);
+    a.n_tiles = (p.N + tile_cols - 1) / tile_cols;  // the last one may hang over N
     a.iters = p.K / (64 * kgroups);
     return p.dtype == DT_BF16 ? launch_dt<DT_BF16>(a, p.bits, kgroups, lc) : launch_dt<DT_F16>(a, p.bits, kgroups, lc);
 }
@@ -484,8 +496,8 @@ int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_i
     if (p.dtype != DT_F16 && p.dtype != DT_BF16) return fail(ERR_UNSUPPORTED, "grouped qmm: f16 / bf16 only");
     if (p.bits != 2 && p.bits != 4 && p.bits != 8) return fail(ERR_UNSUPPORTED, "grouped qmm: bits must be 2, 4 or 8");
     const uint32_t G = p.group_size;
-    if (T == 0 || p.N % 128 || p.K % 128 || G < 32 || (G & (G - 1)) || p.K % G)
-        return fail(ERR_UNSUPPORTED, "grouped qmm: N % 128, K % 128 or group size");
+    if (T == 0 || p.N == 0 || p.K % 128 || G < 32 || (G & (G - 1)) || p.K % G)
+        return fail(ERR_UNSUPPORTED, "grouped qmm: K % 128 or group size");
     if ((uint64_t)T * p.K * 2 >= (1ull << 32) || (uint64_t)p.N * p.K * p.bits / 8 >= (1ull << 32) || (uint64_t)T * p.N * 2 >= (1ull << 34))
         return fail(ERR_UNSUPPORTED, "grouped qmm: operand too large");
     if (E >= 2048) return fail(ERR_UNSUPPORTED, "grouped qmm: 2048 experts or more");
@@ -533,10 +545,10 @@ int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_i
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     // 64 x 128 tiles; 64 x 64 on 4 K-groups when that still leaves fewer tiles than compute units
-    uint32_t kgroups = ((uint64_t)((T + 63) / 64) * (p.N / 128) * 2 <= (uint64_t)cus && p.K % 256 == 0) ? 4 : 2;
+    uint32_t kgroups = ((uint64_t)((T + 63) / 64) * ((p.N + 127) / 128) * 2 <= (uint64_t)cus && p.K % 256 == 0) ? 4 : 2;
     a.m_tile_rows = 64;
     a.m_tiles = max_tiles;
-    a.n_tiles = p.N / (32 * (8 / kgroups));
+    a.n_tiles = (p.N + 32 * (8 / kgroups) - 1) / (32 * (8 / kgroups));
     a.iters = p.K / (64 * kgroups);
     a.by_m = 1;
     a.tiles = tiles;

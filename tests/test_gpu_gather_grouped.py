@@ -139,3 +139,26 @@ def test_grouped_gather_rows_without_an_expert_stay_untouched(oracle, grouped):
     assert rel_err(got[valid].reshape(-1), exp[valid].reshape(-1)) <= 2e-2
     for buf in (w, s, b, x, out, r):
         buf.free()
+
+
+@pytest.mark.parametrize("N", [192, 200])
+def test_grouped_gather_ragged_n(oracle, grouped, N):
+    """Expert matrices whose row count is not a multiple of the tile width."""
+    dt, bits, E, K, G = DType.BF16, 4, 3, 256, 64
+    T = 150
+    rng = np.random.default_rng(10)
+    ids = rng.integers(0, E, size=T).astype("<u4")
+    c = make_case(7500 + N, dt, bits, G, T, N, K, E=E)
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    grouped(2)
+    out = GpuBuffer.from_bytes(np.full(T * N + 1024, 0x7B7B, np.uint16).tobytes())
+    r = GpuBuffer.from_bytes(ids.tobytes())
+    ops.gather_qmv_indices(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+    raw = np.frombuffer(out.read_bytes(), np.uint16)
+    assert np.all(raw[T * N:] == 0x7B7B)
+    got = unpack_f32(raw[:T * N].tobytes(), dt)
+    exp = _expected(oracle, c, ids, T, N, K, E, bits, G, dt)
+    assert rel_err(got, exp.reshape(-1)) <= 2e-2
+    for buf in (w, s, b, x, out, r):
+        buf.free()

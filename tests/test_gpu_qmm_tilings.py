@@ -96,3 +96,32 @@ def test_tile_kernel_on_rows_of_whole_64s(oracle, M, K):
     for buf in (w, s, b, x, out):
         buf.free()
     assert rel_err(got, exp) <= 2e-2
+
+
+@pytest.mark.parametrize("N", [8, 64, 192, 1000, 1001, 2880])
+@pytest.mark.parametrize("tiling", [(0, 0), (128, 1), (128, 2), (64, 2), (64, 4), (32, 4)])
+def test_tile_kernel_on_ragged_n(oracle, options, N, tiling):
+    """Matrices whose row count is not a multiple of the tile width (2880 and odd vocabulary sizes in
+    real models): the last column tile hangs over N, works its missing rows on row N - 1 and stores
+    none of their columns. The output buffer carries a guard band after the last row that must stay
+    untouched. Against the mma-semantics oracle, 2e-2 as for the prefill configuration."""
+    rows, kg = tiling
+    M, K, G, bits, dt = 70, 512, 64, 4, DType.BF16
+    print(f"[case] qmm ragged N={N} tile_rows={rows} kgroups={kg}", flush=True)
+    c = make_case(5600 + N + rows + kg, dt, bits, G, M, N, K)
+    exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    guard = 4096
+    out = GpuBuffer.from_bytes(np.full(M * N + guard, 0x7B7B, np.uint16).tobytes())
+    options("qmm.tile_rows", rows)
+    options("qmm.kgroups", kg)
+    options("qmm.kernel", 2)
+    ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+    raw = np.frombuffer(out.read_bytes(), np.uint16)
+    for buf in (w, s, b, x, out):
+        buf.free()
+    assert np.all(raw[M * N:] == 0x7B7B)
+    got = unpack_f32(raw[:M * N].tobytes(), dt)
+    assert rel_err(got, exp) <= 2e-2
