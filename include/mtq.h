@@ -341,6 +341,7 @@ MTQ_API int mtq_flush_cache(void);
  *   "qmm.by_m"             order in which workgroups walk the tiles: 0 = choose, 1 = the N-tiles of one M-tile
  *                          first, 2 = the M-tiles of one N-tile first
  *   "qmm.splits"           LDS tile kernel: 0 = choose per shape, or the number of K slices per output tile
+ *   "qmm.f32_tiles"        f32 batches on the f32 matrix-core kernel: 0 = choose by rows, 1 = never, 2 = always
  *   "gather.grouped"       gather_qmv with many rows per expert on the tile kernel: 0 = choose, 1 = never, 2 = always
  *   "qvm.wgs"              qvm: workgroups to aim for when K is sliced, 0 = choose
  *   "moe.sort"             expert sort: 0 = choose by size, 1 = always the bitonic network
