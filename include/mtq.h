@@ -133,7 +133,8 @@ MTQ_API int mtq_qmm(int dtype, int bits, uint32_t group_size, const void *w, con
  * Both row views: while experts average at most 16 rows, each expert's rows run on the
  * GEMV kernels (exact w_hat = s*q + b in f32); above that the rows are grouped by expert
  * into 64-row tiles on the MFMA tile kernel, where w_hat is rounded to the element type
- * first, as in the reference's MMA gathers (moe.rs:2256). The grouping tables live in a
+ * first, as in the reference's MMA gathers (moe.rs:2256); MTQ_F32 rows always run grouped, in
+ * 32-row tiles on the f32 matrix-core kernel (f32 rounding only). The grouping tables live in a
  * library-owned buffer (allocated on first use). Option "gather.grouped": 0 this rule,
  * 1 never grouped, 2 always grouped. */
 MTQ_API int mtq_gather_qmv_csr(int dtype, int bits, uint32_t group_size, const void *x,

@@ -291,7 +291,21 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
     // 16 rows each 97 us GEMV / 84 us tiles, 24 rows 139 / 87, 256 rows 588 / 88; 128 experts x
     // 2048x768: 24 rows each 231 / 80 us; at 8 rows each the GEMV wins, 51 us against 119).
     const int gopt = options().gather_grouped;
-    if (mode != GATHER_SINGLE && gopt != 1 && (gopt == 2 || (uint64_t)T > (uint64_t)16 * (E < T ? E : T))) {
+    // f32 rows always go grouped to the f32 matrix-core kernel: the f32 dot kernels take 4 rows per pass
+    // and lose at any routing (128 experts x 256x2048: 64 rows 64 us against 48, 1024 rows 315 against 88;
+    // 8 experts x 4096x4096: 8 rows 212 against 77, 128 rows 940 against 112, host time included).
+    if (dtype == DT_F32 && mode != GATHER_SINGLE && gopt != 1 && options().qmm_f32_tiles != 1) {
+        QmmParams q;
+        q.dtype = dtype; q.bits = bits; q.group_size = G;
+        q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
+        q.M = T; q.N = N; q.K = K;
+        const bool ids = mode == GATHER_INDICES;
+        rc = ensure_scratch(qmm_grouped_scratch_bytes(T, E, ids, 32));
+        if (rc) return rc;
+        rc = launch_qmm_f32_grouped(q, route, ids, T, E, g.scratch_buf, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
+    if (dtype != DT_F32 && mode != GATHER_SINGLE && gopt != 1 && (gopt == 2 || (uint64_t)T > (uint64_t)16 * (E < T ? E : T))) {
         QmmParams q;
         q.dtype = dtype; q.bits = bits; q.group_size = G;
         q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;

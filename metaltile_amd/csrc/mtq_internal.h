@@ -159,9 +159,23 @@ int launch_qmm_f32(const QmmParams& p, const LaunchCtx& lc);
 // Expert-routed rows on the same kernel (many rows per expert): p holds one expert's shapes (N, K),
 // x [T][K], out [T][N], w / scales / biases the stacked experts. `route` = CSR offsets [E + 1], or one
 // expert id per row when per_row_ids. scratch: qmm_grouped_scratch_bytes() bytes.
-size_t qmm_grouped_scratch_bytes(uint32_t T, uint32_t E, bool sort_rows);
+size_t qmm_grouped_scratch_bytes(uint32_t T, uint32_t E, bool sort_rows, uint32_t tile_rows = 64);
 int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_ids, uint32_t T, uint32_t E, void* scratch,
                        const LaunchCtx& lc);
+// The table of row tiles behind both grouped launchers: tiles[0] = count, tiles[1 + i] = (expert,
+// first row in the row order, rows, 0); rowlist maps the row order to rows of x / out (null: identity).
+struct GatherTiles {
+    uint32_t* tiles = nullptr;
+    const uint32_t* rowlist = nullptr;
+    uint32_t max_tiles = 0;
+    LaunchCtx last;
+};
+int build_gather_tiles(const uint32_t* route, bool per_row_ids, uint32_t T, uint32_t E, uint32_t tile_rows, void* scratch,
+                       const LaunchCtx& lc, GatherTiles& out);
+// The same for f32 operands, 32-row tiles on the f32 matrix-core kernel (qmm_f32.hip);
+// scratch: qmm_grouped_scratch_bytes(T, E, per_row_ids, 32).
+int launch_qmm_f32_grouped(const QmmParams& p, const uint32_t* route, bool per_row_ids, uint32_t T, uint32_t E, void* scratch,
+                           const LaunchCtx& lc);
 
 // Affine quantise (quantize = true: T[n_elem] -> packed words + scales + biases) and
 // dequantise (packed words + scales + biases -> T[n_elem]) (affine.hip).

@@ -482,35 +482,28 @@ __global__ __launch_bounds__(64) void gather_tiles_kernel(TileTabArgs a) {
     a.tiles[0] = n;
 }
 
-size_t qmm_grouped_scratch_bytes(uint32_t T, uint32_t E, bool sort_rows) {
-    const size_t max_tiles = (size_t)(T + 63) / 64 + E + 1;
+size_t qmm_grouped_scratch_bytes(uint32_t T, uint32_t E, bool sort_rows, uint32_t tile_rows) {
+    const size_t max_tiles = (size_t)(T + tile_rows - 1) / tile_rows + E + 1;
     size_t b = 16 + max_tiles * 16;
     if (sort_rows) b += ((size_t)2 * T + E + 2 + 3) / 4 * 16;  // sorted row list, inverse permutation, offsets of E + 1 buckets
     return b;
 }
 
-// x [T][K], out [T][N], stacked w / scales / biases [E][N][...]; route = CSR offsets [E + 1] or,
-// with per_row_ids, one expert id per row (sorted by expert here, on the device).
-int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_ids, uint32_t T, uint32_t E, void* scratch,
-                       const LaunchCtx& lc) {
-    if (p.dtype != DT_F16 && p.dtype != DT_BF16) return fail(ERR_UNSUPPORTED, "grouped qmm: f16 / bf16 only");
-    if (p.bits != 2 && p.bits != 4 && p.bits != 8) return fail(ERR_UNSUPPORTED, "grouped qmm: bits must be 2, 4 or 8");
-    const uint32_t G = p.group_size;
-    if (T == 0 || p.N == 0 || p.K % 128 || G < 32 || (G & (G - 1)) || p.K % G)
-        return fail(ERR_UNSUPPORTED, "grouped qmm: K % 128 or group size");
-    if ((uint64_t)T * p.K * 2 >= (1ull << 32) || (uint64_t)p.N * p.K * p.bits / 8 >= (1ull << 32) || (uint64_t)T * p.N * 2 >= (1ull << 34))
-        return fail(ERR_UNSUPPORTED, "grouped qmm: operand too large");
+// Sorts per-row ids by expert where needed and launches the tile table kernel into `scratch`
+// (sized by qmm_grouped_scratch_bytes for the same tile_rows). `out.last` is the launch context for
+// the kernel that consumes the table (it carries the caller's stop event).
+int build_gather_tiles(const uint32_t* route, bool per_row_ids, uint32_t T, uint32_t E, uint32_t tile_rows, void* scratch,
+                       const LaunchCtx& lc, GatherTiles& out) {
     if (E >= 2048) return fail(ERR_UNSUPPORTED, "grouped qmm: 2048 experts or more");
-    if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.out % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
-        return fail(ERR_UNSUPPORTED, "grouped qmm: operands must be 16-byte aligned");
-    const uint32_t max_tiles = (T + 63) / 64 + E + 1;
+    const uint32_t max_tiles = (T + tile_rows - 1) / tile_rows + E + 1;
     uint32_t* tiles = (uint32_t*)scratch;
     const uint32_t* off = route;
     const uint32_t* rowlist = nullptr;
-    LaunchCtx first = lc, mid = lc, last = lc;
+    LaunchCtx first = lc, mid = lc;
+    out.last = lc;
     first.stop = nullptr;
     mid.start = mid.stop = nullptr;
-    last.start = nullptr;
+    out.last.start = nullptr;
     bool started = false;
     if (per_row_ids) {
         uint32_t* sorted = tiles + 4 + (size_t)max_tiles * 4;
@@ -524,10 +517,36 @@ int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_i
         off = offs;
         rowlist = sorted;
     }
-    TileTabArgs ta{off, tiles, E, T, 64u, max_tiles, per_row_ids ? 0u : 1u};
+    TileTabArgs ta{off, tiles, E, T, tile_rows, max_tiles, per_row_ids ? 0u : 1u};
     void* targs[] = {&ta};
     hipError_t e = launch_kernel((const void*)gather_tiles_kernel, dim3(1), dim3(64), targs, 0, started ? mid : first);
     if (e != hipSuccess) return hip_fail(e, "gather tile table kernel launch");
+    out.tiles = tiles;
+    out.rowlist = rowlist;
+    out.max_tiles = max_tiles;
+    return ERR_OK;
+}
+
+// x [T][K], out [T][N], stacked w / scales / biases [E][N][...]; route = CSR offsets [E + 1] or,
+// with per_row_ids, one expert id per row (sorted by expert here, on the device).
+int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_ids, uint32_t T, uint32_t E, void* scratch,
+                       const LaunchCtx& lc) {
+    if (p.dtype != DT_F16 && p.dtype != DT_BF16) return fail(ERR_UNSUPPORTED, "grouped qmm: f16 / bf16 only");
+    if (p.bits != 2 && p.bits != 4 && p.bits != 8) return fail(ERR_UNSUPPORTED, "grouped qmm: bits must be 2, 4 or 8");
+    const uint32_t G = p.group_size;
+    if (T == 0 || p.N == 0 || p.K % 128 || G < 32 || (G & (G - 1)) || p.K % G)
+        return fail(ERR_UNSUPPORTED, "grouped qmm: K % 128 or group size");
+    if ((uint64_t)T * p.K * 2 >= (1ull << 32) || (uint64_t)p.N * p.K * p.bits / 8 >= (1ull << 32) || (uint64_t)T * p.N * 2 >= (1ull << 34))
+        return fail(ERR_UNSUPPORTED, "grouped qmm: operand too large");
+    if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.out % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
+        return fail(ERR_UNSUPPORTED, "grouped qmm: operands must be 16-byte aligned");
+    GatherTiles gt;
+    int rc = build_gather_tiles(route, per_row_ids, T, E, 64u, scratch, lc, gt);
+    if (rc) return rc;
+    const uint32_t max_tiles = gt.max_tiles;
+    uint32_t* tiles = gt.tiles;
+    const uint32_t* rowlist = gt.rowlist;
+    const LaunchCtx& last = gt.last;
 
     QmmDArgs a;
     a.w = (const unsigned char*)p.w;

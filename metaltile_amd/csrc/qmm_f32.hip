@@ -7,8 +7,8 @@
 // w_hat = fma(s, q, b) in f32, products and sums in f32 on v_mfma_f32_32x32x2_f32.
 //
 // Layout of the work. A wave owns a 32-row x (32 * NB)-column block of the output over a slice of
-// K; the four waves of a workgroup take every fourth 64-k step of the same block and meet in LDS at
-// the end. In the 32x32x2 operand layout lane l holds row (or column) l % 32 and k-half l / 32, so
+// K; the NW (4 or 16) waves of a workgroup take every NW-th 64-k step of the same block and meet in
+// LDS at the end. In the 32x32x2 operand layout lane l holds row (or column) l % 32 and k-half l / 32, so
 // a lane reads exactly its own operands from global memory: 32 consecutive f32 of activation row
 // l % 32 (one 128-byte line) and the 32 codes (4 * bits bytes) of weight row l % 32 of each column
 // block, for k in [64 * step + 32 * (l / 32), +32). Nothing passes through LDS in the loop and no
@@ -29,6 +29,10 @@ struct QmmFArgs {
     const float* x;
     float* out;
     uint32_t M, N, K, gpr, log2g, steps, m_tiles, n_tiles, by_m;
+    // expert-routed rows (GR): the table of row tiles, the row order, the experts' strides
+    const uint32_t* tiles;
+    const uint32_t* rowlist;
+    uint64_t w_expert_bytes, sb_expert_elems;
 };
 
 // code j of 32 codes of BITS bits packed LSB-first into BITS words; j is a constant after unrolling
@@ -39,7 +43,7 @@ template <int BITS> __device__ __forceinline__ uint32_t qf_code(const uint32_t* 
     return v & ((1u << BITS) - 1u);
 }
 
-template <int BITS, int NB, int NW>
+template <int BITS, int NB, int NW, bool GR = false>
 __global__ __launch_bounds__(64 * NW) void qmm_f32_kernel(QmmFArgs a) {
     __shared__ float red[NW][NB * 16][64];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -48,11 +52,28 @@ __global__ __launch_bounds__(64 * NW) void qmm_f32_kernel(QmmFArgs a) {
     // workgroup ids congruent mod 8 share an XCD: give each XCD a contiguous run of tiles
     const uint32_t total = a.m_tiles * a.n_tiles;
     uint32_t vid = blockIdx.x;
-    if (total % 8 == 0) vid = (blockIdx.x & 7u) * (total / 8) + (blockIdx.x >> 3);
-    const uint32_t nt = a.by_m ? vid % a.n_tiles : vid / a.m_tiles, mt = a.by_m ? vid / a.n_tiles : vid % a.m_tiles;
+    if (!GR && total % 8 == 0) vid = (blockIdx.x & 7u) * (total / 8) + (blockIdx.x >> 3);
+    uint32_t nt = a.by_m ? vid % a.n_tiles : vid / a.m_tiles, mt = a.by_m ? vid / a.n_tiles : vid % a.m_tiles;
+    // rows of this tile: row j of the tile is row (row_first + j) of the row order, j < row_count
+    uint32_t row_first = mt * 32, row_count = a.M > row_first ? min(32u, a.M - row_first) : 0u;
+    if constexpr (GR) {
+        nt = blockIdx.x % a.n_tiles;
+        mt = blockIdx.x / a.n_tiles;
+        if (mt >= a.tiles[0]) return;  // the grid is sized for the worst routing; the whole workgroup leaves
+        const uint4 t = ((const uint4*)a.tiles)[1 + mt];
+        row_first = t.y;
+        row_count = t.z;
+        a.w += (size_t)t.x * a.w_expert_bytes;
+        a.scales += (size_t)t.x * a.sb_expert_elems;
+        a.biases += (size_t)t.x * a.sb_expert_elems;
+    }
+    auto row_of = [&](uint32_t j) -> uint32_t {  // j < row_count
+        if constexpr (GR) return a.rowlist ? a.rowlist[row_first + j] : row_first + j;
+        else return row_first + j;
+    };
 
     // rows and columns past the edge are worked on the last one and not stored
-    const uint32_t row = min(mt * 32 + fr, a.M - 1);
+    const uint32_t row = row_of(min(fr, row_count - 1));
     const float* xp = a.x + (size_t)row * a.K + 32 * fh;
     const unsigned char* wp[NB];
     const float* sp[NB];
@@ -133,8 +154,8 @@ __global__ __launch_bounds__(64 * NW) void qmm_f32_kernel(QmmFArgs a) {
             float r = red[0][nb * 16 + v][lane];
 #pragma unroll
             for (int u = 1; u < NW; u++) r += red[u][nb * 16 + v][lane];
-            const uint32_t orow = mt * 32 + 8 * (v / 4) + 4 * fh + (v % 4);
-            if (orow < a.M && col < a.N) a.out[(size_t)orow * a.N + col] = r;
+            const uint32_t lrow = 8 * (v / 4) + 4 * fh + (v % 4);
+            if (lrow < row_count && col < a.N) a.out[(size_t)row_of(lrow) * a.N + col] = r;
         }
     }
 }
@@ -161,6 +182,9 @@ int launch_qmm_f32(const QmmParams& p, const LaunchCtx& lc) {
     a.log2g = l;
     a.gpr = p.K / G;
     a.steps = p.K / 64;
+    a.tiles = nullptr;
+    a.rowlist = nullptr;
+    a.w_expert_bytes = a.sb_expert_elems = 0;
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     a.m_tiles = (p.M + 31) / 32;
@@ -194,6 +218,69 @@ int launch_qmm_f32(const QmmParams& p, const LaunchCtx& lc) {
     void* args[] = {&a};
     hipError_t e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles), dim3(64 * nw), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "f32 qmm kernel launch");
+    return ERR_OK;
+}
+
+// x [T][K], out [T][N], stacked w / scales / biases [E][N][...]; route = CSR offsets [E + 1] or, with
+// per_row_ids, one expert id per row (sorted by expert on the device). Rows of one expert share 32-row
+// tiles; replaces, for T = f32, the reference's gather kernels (crates/metaltile-std/src/ffai/moe.rs:358,
+// 2256 and their per-width forms).
+int launch_qmm_f32_grouped(const QmmParams& p, const uint32_t* route, bool per_row_ids, uint32_t T, uint32_t E, void* scratch,
+                           const LaunchCtx& lc) {
+    const uint32_t G = p.group_size;
+    if (p.dtype != DT_F32) return fail(ERR_UNSUPPORTED, "f32 grouped qmm: element type");
+    if (T == 0 || p.N == 0 || p.K == 0 || p.K % 64 || G < 32 || (G & (G - 1)) || p.K % G)
+        return fail(ERR_UNSUPPORTED, "f32 grouped qmm: K % 64 or group size");
+    if (p.bits < 2 || p.bits > 8) return fail(ERR_UNSUPPORTED, "f32 grouped qmm: code width");
+    if ((uintptr_t)p.w % 4 || (uintptr_t)p.x % 16 || (uintptr_t)p.out % 4 || (uintptr_t)p.scales % 4 || (uintptr_t)p.biases % 4)
+        return fail(ERR_UNSUPPORTED, "f32 grouped qmm: operand alignment");
+    if (((uint64_t)p.N * p.K * p.bits / 8) % 4) return fail(ERR_UNSUPPORTED, "f32 grouped qmm: expert stride");
+    GatherTiles gt;
+    int rc = build_gather_tiles(route, per_row_ids, T, E, 32u, scratch, lc, gt);
+    if (rc) return rc;
+    QmmFArgs a;
+    a.w = (const unsigned char*)p.w;
+    a.scales = (const float*)p.scales;
+    a.biases = (const float*)p.biases;
+    a.x = (const float*)p.x;
+    a.out = (float*)p.out;
+    a.M = T;
+    a.N = p.N;
+    a.K = p.K;
+    uint32_t l = 0;
+    while ((1u << l) < G) l++;
+    a.log2g = l;
+    a.gpr = p.K / G;
+    a.steps = p.K / 64;
+    a.tiles = gt.tiles;
+    a.rowlist = gt.rowlist;
+    a.w_expert_bytes = (uint64_t)p.N * p.K * p.bits / 8;
+    a.sb_expert_elems = (uint64_t)p.N * a.gpr;
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    a.m_tiles = gt.max_tiles;
+    const int nb = (uint64_t)((T + 31) / 32) * ((p.N + 63) / 64) >= 2 * (uint64_t)cus ? 2 : 1;
+    a.n_tiles = (p.N + 32 * nb - 1) / (32 * nb);
+    if ((uint64_t)a.m_tiles * a.n_tiles >= (1ull << 31)) return fail(ERR_UNSUPPORTED, "f32 grouped qmm: too many tiles");
+    a.by_m = 1;
+    const void* fn = nullptr;
+#define QF_PICK(B)                                                                                                   \
+    case B:                                                                                                          \
+        fn = nb == 2 ? (const void*)qmm_f32_kernel<B, 2, 4, true> : (const void*)qmm_f32_kernel<B, 1, 4, true>;      \
+        break;
+    switch (p.bits) {
+        QF_PICK(2)
+        QF_PICK(3)
+        QF_PICK(4)
+        QF_PICK(5)
+        QF_PICK(6)
+        QF_PICK(7)
+        QF_PICK(8)
+    }
+#undef QF_PICK
+    void* args[] = {&a};
+    hipError_t e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles), dim3(256), args, 0, gt.last);
+    if (e != hipSuccess) return hip_fail(e, "f32 grouped qmm kernel launch");
     return ERR_OK;
 }
 

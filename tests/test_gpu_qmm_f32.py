@@ -72,3 +72,73 @@ def test_f32_batches_route_by_rows(oracle, f32_tiles):
     assert _run(oracle, 9410, 4, 32, 12, 64, 96, ops.qmm) <= 1e-4
     f32_tiles(1)
     assert _run(oracle, 9411, 4, 64, 12, 64, 1024, ops.qmm) <= 1e-4
+
+
+@pytest.fixture
+def grouped():
+    lib = _lib.load()
+
+    def set_(value):
+        assert lib.mtq_set_option(b"gather.grouped", value) == 0
+
+    yield set_
+    lib.mtq_set_option(b"gather.grouped", 0)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
+def test_f32_grouped_gather_both_views(oracle, grouped, bits):
+    """f32 rows routed to experts, grouped into 32-row tiles: CSR offsets (with an empty expert, an
+    expert of more than one tile and a tail past the last offset, which belongs to expert 0) and shuffled
+    per-row ids (three of them naming no expert: those output rows must stay untouched)."""
+    dt, E, N, K, G = DType.F32, 5, 72, 512, 64
+    counts = [40, 0, 70, 3, 32]
+    T = sum(counts) + 6  # 6 tail rows
+    c = make_case(9500 + bits, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype("<u4")
+    ids_csr = np.concatenate([np.repeat(np.arange(E), counts), np.zeros(6, np.int64)]).astype("<u4")
+    rng = np.random.default_rng(bits)
+    ids = rng.permutation(ids_csr).astype("<u4")
+    bad = np.array([7, 50, 100])
+    ids[bad] = [E, E + 3, 0xFFFFFFFF]
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    grouped(2)
+    for view, route, fn, rows_ids in (("csr", offsets, ops.gather_qmv_csr, ids_csr), ("indices", ids, ops.gather_qmv_indices, ids)):
+        print(f"[case] f32 grouped gather {view} b{bits}", flush=True)
+        valid = rows_ids < E
+        exp = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G,
+                                indices=np.where(valid, rows_ids, 0).astype("<u4"), f64=True, threads=8)
+        exp = np.asarray(exp, np.float32).reshape(T, N)
+        out = GpuBuffer.from_bytes(np.full(T * N + 256, 0x7B7B7B7B, np.uint32).tobytes())
+        r = GpuBuffer.from_bytes(route.tobytes())
+        fn(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+        raw = np.frombuffer(out.read_bytes(), np.uint32)
+        out.free(); r.free()
+        assert np.all(raw[T * N:] == 0x7B7B7B7B), view
+        got = raw[:T * N].view(np.float32).reshape(T, N)
+        assert np.all(raw[:T * N].reshape(T, N)[~valid] == 0x7B7B7B7B), view
+        assert rel_err(got[valid].reshape(-1), exp[valid].reshape(-1)) <= 1e-4, view
+    for buf in (w, s, b, x):
+        buf.free()
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_f32_gather_default_rule(oracle, grouped, mode):
+    """Without the option f32 rows go grouped at any number of rows per expert; with the option at 1 they
+    stay on the dot kernels. Both within the bound."""
+    dt, bits, E, N, K, G = DType.F32, 4, 4, 64, 256, 64
+    grouped(mode)
+    for per in (2, 12):
+        T = per * E
+        c = make_case(9600 + per, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
+        ids = np.repeat(np.arange(E), per).astype("<u4")
+        exp = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=ids, f64=True, threads=8)
+        w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                      GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+        out = GpuBuffer(T * N * 4)
+        r = GpuBuffer.from_bytes(ids.tobytes())
+        ops.gather_qmv_indices(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+        got = np.frombuffer(out.read_bytes(), np.float32)
+        assert rel_err(got, np.asarray(exp, np.float32).reshape(-1)) <= 1e-4
+        for buf in (w, s, b, x, out, r):
+            buf.free()
