@@ -40,10 +40,16 @@ def test_reference_setup_qvm_int4_fast(ctx, oracle, dt, tol):
 
 @pytest.mark.parametrize("dt", [DType.F32, DType.F16, DType.BF16], ids=lambda d: d.name)
 @pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 7, 8])
-@pytest.mark.parametrize("M,N,K,G", [(1, 64, 256, 64), (1, 4096, 4096, 64), (3, 96, 1024, 32), (1, 32, 192, 64)])
+# N = 64, 4096, 96 and 32 take the kernel whose threads own 32 columns; N = 8 and 40 (8-bit: 8 too) are not
+# multiples of 32 and take the one whose threads own one word or one column (their N * bits is a multiple of 32
+# for the even code widths only).
+@pytest.mark.parametrize("M,N,K,G", [(1, 64, 256, 64), (1, 4096, 4096, 64), (3, 96, 1024, 32), (1, 32, 192, 64),
+                                     (2, 40, 256, 64), (1, 8, 128, 32), (1, 1056, 2048, 64)])
 def test_qvm_widths(oracle, dt, bits, M, N, K, G):
     if N * K > 1 << 22 and (bits not in (3, 4, 8) or dt == DType.F16):
         pytest.skip("the 4096 x 4096 case runs for 3-, 4- and 8-bit codes in f32 and bf16")
+    if N * bits % 32:
+        pytest.skip("N * bits must be a multiple of 32")
     print(f"[case] qvm {dt.name} b{bits} g{G} M{M} N{N} K{K}", flush=True)
     rng = np.random.default_rng(bits * 100 + N + K)
     rt = lambda v: oracle.round_through(np.asarray(v, dtype=np.float32), ODT[dt])
