@@ -75,10 +75,18 @@ __device__ __forceinline__ uint4 dequant8(const uint32_t* wr, int i, float s, fl
         for (int d = 0; d < 2; d++)
 #pragma unroll
             for (int j = 0; j < 4; j++) v[4 * d + j] = fmaf((float)((wr[2 * i + d] >> (8 * j)) & 0xFFu), s, b);
-    } else {  // BITS == 2: 16 codes per dword, this call takes half of dword i/2
+    } else if constexpr (BITS == 2) {  // 16 codes per dword, this call takes half of dword i/2
         const uint32_t w = wr[i / 2] >> (16 * (i & 1));
 #pragma unroll
         for (int j = 0; j < 8; j++) v[j] = fmaf((float)((w >> (2 * j)) & 3u), s, b);
+    } else {  // bit-stream widths: code c of the run sits at bit c * BITS of the BITS words, LSB first
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int o = (8 * i + j) * BITS, lo = o >> 5, sh = o & 31;
+            uint32_t q = wr[lo] >> sh;
+            if (sh + BITS > 32) q |= wr[lo + 1] << (32 - sh);
+            v[j] = fmaf((float)(q & ((1u << BITS) - 1u)), s, b);
+        }
     }
     return make_uint4(pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3]), pack2<DT>(v[4], v[5]), pack2<DT>(v[6], v[7]));
 }

@@ -42,7 +42,7 @@ def _expected(oracle, c, ids, T, N, K, E, bits, G, dt):
 
 
 @pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
-@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
 def test_grouped_gather_both_views(oracle, grouped, bits, dt):
     E, N, K, G = 5, 256, 512, 64
     counts = [40, 0, 70, 3, 64]

@@ -125,3 +125,49 @@ def test_tile_kernel_on_ragged_n(oracle, options, N, tiling):
     assert np.all(raw[M * N:] == 0x7B7B)
     got = unpack_f32(raw[:M * N].tobytes(), dt)
     assert rel_err(got, exp) <= 2e-2
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("bits", [3, 5, 6, 7])
+def test_direct_qmm_bit_stream_widths(oracle, options, bits, dt):
+    """3-, 5-, 6- and 7-bit codes on the register-operand tile kernel, every tiling built for them,
+    ragged M and N. Against the mma-semantics oracle, 2e-2 as for the prefill configuration."""
+    M, N, K, G = 200, 200, 1024, 64
+    c = make_case(5700 + bits, dt, bits, G, M, N, K)
+    exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    options("qmm.kernel", 2)
+    for rows, kg in ((0, 0), (128, 1), (64, 1), (64, 2), (64, 4), (32, 4)):
+        print(f"[case] direct qmm {dt.name} b{bits} kgroups={kg} tile_rows={rows}", flush=True)
+        options("qmm.kgroups", kg)
+        options("qmm.tile_rows", rows)
+        out = GpuBuffer.from_bytes(np.full(M * N + 512, 0x7B7B, np.uint16).tobytes())
+        ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+        raw = np.frombuffer(out.read_bytes(), np.uint16)
+        out.free()
+        assert np.all(raw[M * N:] == 0x7B7B)
+        err = rel_err(unpack_f32(raw[:M * N].tobytes(), dt), exp)
+        assert err <= 2e-2, f"kgroups={kg} rows={rows}: rel err {err:.3e}"
+    for buf in (w, s, b, x):
+        buf.free()
+
+
+@pytest.mark.parametrize("bits", [3, 5, 6])
+@pytest.mark.parametrize("M", [512, 2048])
+def test_bit_stream_widths_route_to_tiles(oracle, bits, M):
+    """The default routing at prefill sizes (128-row tiles from 2048 rows at N = 1024)."""
+    N, K, G, dt = 1024, 512, 64, DType.BF16
+    print(f"[case] qmm b{bits} M={M}", flush=True)
+    c = make_case(5800 + bits + M, dt, bits, G, M, N, K)
+    exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    out = GpuBuffer(M * N * dt.size_bytes)
+    ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+    got = unpack_f32(out.read_bytes(), dt)
+    for buf in (w, s, b, x, out):
+        buf.free()
+    assert rel_err(got, exp) <= 2e-2
