@@ -162,7 +162,9 @@ static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s,
     if (M == 0) return ERR_OK;
     if (!w || !s || !b || !x || !out) return fail(ERR_BAD_ARG, "null buffer");
     if (dtype == DT_F32 && options().qmm_f32_tiles != 1) return op_qmv(dtype, bits, G, w, s, b, x, out, M, N, K, lc);
-    if (M >= 17 || (M >= 9 && N >= 8192) || force_mma) {
+    // 7-bit codes have no GEMV kernel of their own (the reference has no 7-bit kernels either): any
+    // number of rows beats the generic kernel on the tile kernel (4096 x 4096: 1 row 28 -> 17 us, 16 rows 236 -> 17).
+    if (M >= 17 || (M >= 9 && N >= 8192) || force_mma || bits == 7) {
         QmmParams q;
         q.dtype = dtype; q.bits = bits; q.group_size = G;
         q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
