@@ -118,9 +118,12 @@ MTQ_API int mtq_qmv(int dtype, int bits, uint32_t group_size, const void *w, con
                     uint32_t K);
 
 /* qmm: same product for any M; routes by M like mt_qmm_for
- * (crates/metaltile-std/src/mlx/quantized.rs:5040-5065): large M runs the
- * LDS-dequant + MFMA tile kernel (replaces mt_qmm_mma / _m16 / _int8 / _int2,
- * quantized.rs:2106, 2408, 2731, 3330), small M the qmv family. */
+ * (crates/metaltile-std/src/mlx/quantized.rs:5040-5065): from 9 rows (from 5 where the
+ * rows are long) the MFMA tile kernel (replaces mt_qmm_mma / _m16 / _int8 / _int2 / _b3 /
+ * _b5 / _b6, quantized.rs:2106, 2408, 2731, 3330, 3560-3900; w_hat rounded to the element
+ * type before the multiply, as there), below that the qmv family (exact w_hat). MTQ_F32
+ * batches run on the f32 matrix cores from 5 rows. Short, wide matrices split K over
+ * workgroups through a library-owned buffer (allocated on first use). */
 MTQ_API int mtq_qmm(int dtype, int bits, uint32_t group_size, const void *w, const void *scales,
                     const void *biases, const void *x, void *out, uint32_t M, uint32_t N,
                     uint32_t K);
@@ -342,6 +345,8 @@ MTQ_API int mtq_flush_cache(void);
  *   "qmm.by_m"             order in which workgroups walk the tiles: 0 = choose, 1 = the N-tiles of one M-tile
  *                          first, 2 = the M-tiles of one N-tile first
  *   "qmm.splits"           LDS tile kernel: 0 = choose per shape, or the number of K slices per output tile
+ *   "qmm.ksplit"           register-operand tile kernel: 0 = choose, 1 = never split K, n = n splits (f32 partial
+ *                          tiles in the library-owned buffer, added in split order by a second kernel)
  *   "qmm.f32_tiles"        f32 batches on the f32 matrix-core kernel: 0 = choose by rows, 1 = never, 2 = always
  *   "gather.grouped"       gather_qmv with many rows per expert on the tile kernel: 0 = choose, 1 = never, 2 = always
  *   "qvm.wgs"              qvm: workgroups to aim for when K is sliced, 0 = choose

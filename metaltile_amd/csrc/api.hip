@@ -147,13 +147,15 @@ static int op_qmv(int dtype, int bits, uint32_t G, const void* w, const void* s,
     return run_gemv(p, lc);
 }
 
+static int ensure_scratch(size_t need);
+
 // Kernel routing by M, the counterpart of mt_qmm_for
 // (crates/metaltile-std/src/mlx/quantized.rs:5040-5065, which sends M = 16 and the multiples
 // of 32 to its MMA kernels). Here the GEMV family takes 8 activation rows per pass over the
-// weights, so it serves up to 8 rows; the MFMA tile kernel takes over from 17 rows (a third
-// pass always loses: N = K = 4096, 20 rows, 17.5 us against 16.0) and, where the matrix has
-// enough column tiles to fill the chip with one row of tiles (N >= 8192), from 9 rows
-// (14336x4096, 12 rows: 22.7 us against 18.0; 4096x14336 stays: 38.6 against 59).
+// weights, so it serves up to 8 rows; from 9 rows the MFMA tile kernel takes over: a second GEMV
+// pass always loses to 32-row tiles once short matrices split K over workgroups (16 rows, GEMV
+// against tiles: 4096 x 14336 50 / 23 us, 2048 x 8192 21 / 11, 1024 x 4096 24 / 11, 14336 x 4096
+// 25 / 15, 128256 x 4096 134 / 98).
 static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s, const void* b,
                   const void* x, void* out, uint32_t M, uint32_t N, uint32_t K, bool force_mma,
                   const LaunchCtx& lc) {
@@ -164,13 +166,23 @@ static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s,
     if (dtype == DT_F32 && options().qmm_f32_tiles != 1) return op_qmv(dtype, bits, G, w, s, b, x, out, M, N, K, lc);
     // 7-bit codes have no GEMV kernel of their own (the reference has no 7-bit kernels either): any
     // number of rows beats the generic kernel on the tile kernel (4096 x 4096: 1 row 28 -> 17 us, 16 rows 236 -> 17).
-    if (M >= 17 || (M >= 9 && N >= 8192) || force_mma || bits == 7) {
+    // 5..8 rows: rows too long for 8 of them in LDS make the GEMV take two passes, and short, wide
+    // matrices leave it few row blocks; the split-K tiles are ahead there (8 rows, GEMV against tiles:
+    // 4096 x 14336 26 / 22 us, 1024 x 4096 14 / 10, 8192 x 28672 107 / 62, 28672 x 8192 56 / 39; but
+    // 14336 x 4096 12 / 14, 128256 x 4096 70 / 84).
+    const bool long_rows = M >= 5 && ((uint64_t)K >= 2 * (uint64_t)N || (K >= 8192 && (uint64_t)N >= 3 * (uint64_t)K));
+    if (M >= 9 || long_rows || force_mma || bits == 7) {
         QmmParams q;
         q.dtype = dtype; q.bits = bits; q.group_size = G;
         q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
         q.M = M; q.N = N; q.K = K;
         if (options().qmm_kernel != 1) {
-            rc = launch_qmm_direct(q, lc);
+            const size_t need = qmm_direct_scratch_bytes(q);  // f32 partial tiles when K is split
+            if (need) {
+                rc = ensure_scratch(need);
+                if (rc) return rc;
+            }
+            rc = launch_qmm_direct(q, lc, need ? g.scratch_buf : nullptr);
             if (rc != ERR_UNSUPPORTED) return rc;
         }
         rc = launch_qmm_mfma(q, lc);
@@ -1184,6 +1196,11 @@ int mtq_set_option(const char* name, int value) {
     if (!strcmp(name, "gather.grouped")) {
         if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "gather.grouped must be 0 (choose), 1 (never) or 2 (always)");
         options().gather_grouped = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmm.ksplit")) {
+        if (value < 0 || value > 64) return fail(ERR_BAD_ARG, "qmm.ksplit must be 0 (choose), 1 (never) or a number of splits up to 64");
+        options().qmm_ksplit = value;
         return MTQ_OK;
     }
     if (!strcmp(name, "qmm.f32_tiles")) {

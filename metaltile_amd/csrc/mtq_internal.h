@@ -93,6 +93,7 @@ struct Options {
     int qmm_kgroups = 0;          // direct qmm: K-groups per workgroup (0 = choose; 1, 2, 4)
     int qmm_by_m = 0;             // direct qmm: 1 = an XCD keeps its M-tiles' activations and streams all weights
     int gather_grouped = 0;       // expert-routed rows on the tile kernel: 0 = choose by rows per expert, 1 = never, 2 = always
+    int qmm_ksplit = 0;           // direct qmm: 0 = choose, 1 = never split K, n = n splits
     int qmm_f32_tiles = 0;        // f32 batches on the f32 matrix cores: 0 = choose by rows, 1 = never, 2 = always
     int qmm_tile_rows = 0;        // direct qmm: activation rows per tile (0 = choose; 32, 64, 128)
     int qmv_mfma = 0;             // matrix-core qmv: 0 auto, 1 never, 2 whenever the shape fits
@@ -153,7 +154,9 @@ struct QmmParams {
 // Tiled MFMA GEMM with weights dequantised into LDS (qmm.hip).
 int launch_qmm_mfma(const QmmParams& p, const LaunchCtx& lc);
 // 64x128 tiles, weights converted in MFMA operand registers, activations through LDS (qmm_direct.hip).
-int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc);
+// scratch: qmm_direct_scratch_bytes(p) bytes (0 when K is not split: then scratch may be null).
+size_t qmm_direct_scratch_bytes(const QmmParams& p);
+int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc, void* scratch);
 // f32 operands on the f32 matrix cores, any code width (qmm_f32.hip).
 int launch_qmm_f32(const QmmParams& p, const LaunchCtx& lc);
 // Expert-routed rows on the same kernel (many rows per expert): p holds one expert's shapes (N, K),

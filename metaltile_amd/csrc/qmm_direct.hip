@@ -43,6 +43,15 @@ static size_t lds_need(uint32_t rows, uint32_t kg, uint32_t gpr, bool sbl) {
     return main_loop > epilogue ? main_loop : epilogue;
 }
 
+// Adds the K splits' partial tiles in split order and rounds to the element type.
+template <int DT> __global__ __launch_bounds__(256) void qmm_split_reduce_kernel(const float* part, void* out, uint32_t total, uint32_t ksplit) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    float r = part[i];
+    for (uint32_t sp = 1; sp < ksplit; sp++) r += part[(size_t)sp * total + i];
+    ((uint16_t*)out)[i] = f32_to_elem_bits<DT>(r);
+}
+
 template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, const LaunchCtx& lc, bool grouped = false) {
     const void* fn = nullptr;
     const bool tall = a.m_tile_rows == 128;
@@ -79,12 +88,34 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     void* args[] = {&a};
+    if (a.ksplit > 1 && !grouped) {
+        LaunchCtx l1 = lc, l2 = lc;
+        l1.stop = nullptr;
+        l2.start = nullptr;
+        e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles, a.ksplit), dim3(kgroups == 1 ? 256 : 512), args, shmem, l1);
+        if (e != hipSuccess) return hip_fail(e, "qmm direct kernel launch");
+        const float* part = a.part;
+        void* out = a.out;
+        uint32_t total = a.M * a.N, ks = a.ksplit;
+        void* rargs[] = {&part, &out, &total, &ks};
+        e = launch_kernel((const void*)qmm_split_reduce_kernel<DT>, dim3((total + 255) / 256), dim3(256), rargs, 0, l2);
+        if (e != hipSuccess) return hip_fail(e, "qmm split reduce kernel launch");
+        return ERR_OK;
+    }
     e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles), dim3(kgroups == 1 ? 256 : 512), args, shmem, lc);
     if (e != hipSuccess) return hip_fail(e, "qmm direct kernel launch");
     return ERR_OK;
 }
 
-int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
+// rows of k-iterations below which a K split is not worth its second launch
+static constexpr uint32_t QMM_SPLIT_MIN_ITERS = 16;
+
+struct QmmDPlan {
+    uint32_t rows, kgroups, ksplit, iters_per_split;
+};
+
+// Checks the shape and picks the tile, the K-groups and the K split.
+static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
     if (p.dtype != DT_F16 && p.dtype != DT_BF16)
         return fail(ERR_UNSUPPORTED, "direct qmm: f16 / bf16 activations only");
     if (p.bits < 2 || p.bits > 8) return fail(ERR_UNSUPPORTED, "direct qmm: bits must be in 2..8");
@@ -96,19 +127,6 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
         return fail(ERR_UNSUPPORTED, "direct qmm: operand larger than 4 GiB");
     if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.out % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
         return fail(ERR_UNSUPPORTED, "direct qmm: operands must be 16-byte aligned");
-    QmmDArgs a;
-    a.w = (const unsigned char*)p.w;
-    a.scales = (const unsigned char*)p.scales;
-    a.biases = (const unsigned char*)p.biases;
-    a.x = (const unsigned char*)p.x;
-    a.out = p.out;
-    a.M = p.M;
-    a.N = p.N;
-    a.K = p.K;
-    uint32_t l = 0;
-    while ((1u << l) < G) l++;
-    a.log2g = l;
-    a.gpr = p.K / G;
     // Tile choice, measured at N = K = 4096: 128 x 128 tiles (each converted weight
     // feeds 4 MFMAs) win once they fill the chip (M >= 1024: 42-47 us against 50);
     // below that 64 x 128 (M = 512: 29 us against 37-42); and when even those leave
@@ -118,7 +136,14 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
     const uint64_t tall_wide = (uint64_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
     const uint64_t short_wide = (uint64_t)((p.M + 63) / 64) * ((p.N + 127) / 128);
     uint32_t rows = 64, kgroups = 2;
-    if (tall_wide >= 2 * (uint64_t)cus) { rows = 128; kgroups = 1; }  // two 4-wave workgroups per CU (M = 2048: 72-75 us against 80-84; M = 4096: 160-170 against 180-190)
+    // Few rows never take a taller tile than they fill, however many column tiles there are: a
+    // 128-row tile for 16 rows streams the weights at a quarter of the rate (128256 x 4096, 16 rows:
+    // 162 us on 128 x 128 tiles, 86 us on 32 x 64; 28672 x 8192: 72 against 38 us). Up to 64 rows the
+    // 64 x 64 tiles on 4 K-groups stay ahead until there are more 128-column tiles than compute
+    // units (28672 x 8192, 32 rows on 64-row tiles: 58 us against 68; 128256 x 4096: 132 against 85).
+    if (p.M <= 32) { rows = 32; kgroups = 4; }
+    else if (p.M <= 64) { rows = 64; kgroups = short_wide <= (uint64_t)cus ? 4 : 2; }
+    else if (tall_wide >= 2 * (uint64_t)cus) { rows = 128; kgroups = 1; }  // two 4-wave workgroups per CU (M = 2048: 72-75 us against 80-84; M = 4096: 160-170 against 180-190)
     else if (tall_wide >= (uint64_t)cus) { rows = 128; kgroups = 2; }
     else if (short_wide * 2 <= (uint64_t)cus) {  // few tiles: halve their width, and their height for up to 32 rows
         rows = p.M <= 32 ? 32 : 64;
@@ -139,6 +164,56 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
         if (options().qmm_tile_rows) return fail(ERR_BAD_ARG, "qmm.tile_rows 32 needs 4 K-groups");
         rows = 64;
     }
+    pl.rows = rows;
+    pl.kgroups = kgroups;
+    // Few tiles and long rows (a down projection at 9..64 rows: 4096 x 14336 gives 64 tiles for 256
+    // compute units): K is cut into splits, one workgroup per (tile, split), whose f32 partial tiles a
+    // second kernel adds in split order.
+    const uint32_t tile_cols = kgroups == 1 ? 128 : 32 * (8 / kgroups);
+    const uint64_t tiles = (uint64_t)((p.M + rows - 1) / rows) * ((p.N + tile_cols - 1) / tile_cols);
+    const uint32_t iters = p.K / (64 * kgroups);
+    uint32_t ks = 1;
+    if (options().qmm_ksplit > 1) ks = (uint32_t)options().qmm_ksplit;
+    else if (options().qmm_ksplit == 0 && tiles * 2 <= (uint64_t)cus && iters >= QMM_SPLIT_MIN_ITERS) {
+        // one workgroup per compute unit, at least 4 iterations each (measured optimum: 4096 x 14336,
+        // 32 rows, 64 tiles: 1 / 2 / 4 / 8 / 16 splits 57 / 34 / 23 / 27 / 32 us; 2048 x 8192, 32 tiles:
+        // 23 / 17 / 12 / 11 / 12 us; 8192 x 28672, 128 tiles: 108 / 63 / 62 / 66 / 80 us)
+        ks = (uint32_t)((uint64_t)cus / tiles);
+        if (ks > iters / 4) ks = iters / 4;
+        if (ks > 16) ks = 16;
+    }
+    if (ks > iters) ks = iters;
+    if (ks < 1) ks = 1;
+    pl.iters_per_split = (iters + ks - 1) / ks;
+    pl.ksplit = (iters + pl.iters_per_split - 1) / pl.iters_per_split;  // no empty split
+    return ERR_OK;
+}
+
+size_t qmm_direct_scratch_bytes(const QmmParams& p) {
+    QmmDPlan pl;
+    if (plan_direct(p, pl) != ERR_OK || pl.ksplit <= 1) return 0;
+    return (size_t)pl.ksplit * p.M * p.N * sizeof(float);
+}
+
+int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc, void* scratch) {
+    QmmDPlan pl;
+    int rc = plan_direct(p, pl);
+    if (rc) return rc;
+    const uint32_t G = p.group_size, rows = pl.rows, kgroups = pl.kgroups;
+    if (pl.ksplit > 1 && !scratch) return fail(ERR_BAD_ARG, "direct qmm: K split without a scratch buffer");
+    QmmDArgs a;
+    a.w = (const unsigned char*)p.w;
+    a.scales = (const unsigned char*)p.scales;
+    a.biases = (const unsigned char*)p.biases;
+    a.x = (const unsigned char*)p.x;
+    a.out = p.out;
+    a.M = p.M;
+    a.N = p.N;
+    a.K = p.K;
+    uint32_t l = 0;
+    while ((1u << l) < G) l++;
+    a.log2g = l;
+    a.gpr = p.K / G;
     a.m_tile_rows = rows;
     // Workgroup ids congruent mod 8 share an XCD and its L2. Whichever operand is smaller is
     // streamed by every XCD and the larger one is split between them (activations larger than the
@@ -149,6 +224,12 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc) {
     const uint32_t tile_cols = kgroups == 1 ? 128 : 32 * (8 / kgroups);
     a.n_tiles = (p.N + tile_cols - 1) / tile_cols;  // the last one may hang over N
     a.iters = p.K / (64 * kgroups);
+    a.ksplit = pl.ksplit;
+    a.iters_per_split = pl.iters_per_split;
+    a.part = (float*)scratch;
+    a.tiles = nullptr;
+    a.rowlist = nullptr;
+    a.w_expert_bytes = a.sb_expert_elems = 0;
     return p.dtype == DT_BF16 ? launch_dt<DT_BF16>(a, p.bits, kgroups, lc) : launch_dt<DT_F16>(a, p.bits, kgroups, lc);
 }
 
@@ -268,6 +349,9 @@ int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_i
     a.n_tiles = (p.N + 32 * (8 / kgroups) - 1) / (32 * (8 / kgroups));
     a.iters = p.K / (64 * kgroups);
     a.by_m = 1;
+    a.ksplit = 1;
+    a.iters_per_split = a.iters;
+    a.part = nullptr;
     a.tiles = tiles;
     a.rowlist = rowlist;
     a.w_expert_bytes = (uint64_t)p.N * p.K * p.bits / 8;

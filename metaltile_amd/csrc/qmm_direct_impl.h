@@ -32,6 +32,10 @@ struct QmmDArgs {
     const uint32_t* tiles;
     const uint32_t* rowlist;
     uint64_t w_expert_bytes, sb_expert_elems;
+    // split K (few tiles, long rows): workgroup (x, y) works iterations [y * iters_per_split, +iters_per_split)
+    // of tile x and writes its f32 partial tile to part[y][M][N]; a second kernel adds the splits in order.
+    uint32_t ksplit, iters_per_split;
+    float* part;
 };
 
 
@@ -90,6 +94,16 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
         else return row_first + j;
     };
     const uint32_t n0 = nt * DBN;
+    uint32_t it_base = 0;  // first iteration of this workgroup's share of K
+    if (!GR && a.ksplit > 1) {
+        it_base = blockIdx.y * a.iters_per_split;
+        a.iters = min(a.iters_per_split, a.iters - it_base);
+        a.x += (size_t)it_base * (DBK * 2);
+        a.w += (size_t)it_base * (DBK * BITS / 8);
+    }
+    // groups of scales / biases this workgroup needs: [sb_g0, sb_g0 + sb_ng), whole 8-element vectors
+    const uint32_t sb_g0 = ((it_base * DBK) >> a.log2g) & ~7u;
+    const uint32_t sb_ng = min(a.gpr - sb_g0, (((((it_base + a.iters) * DBK - 1) >> a.log2g) + 1 - sb_g0) + 7u) & ~7u);
 
     // activations: thread t moves 32 bytes of row t/TPR (bytes [32*(t%TPR), +32) of the iteration's row)
     const uint32_t xr = tid / TPR, xc = tid % TPR;
@@ -139,7 +153,7 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
             }                                                                            \
         }                                                                                \
         if constexpr (!SBL) {                                                            \
-            const uint32_t g_ = (it_ * DBK + kofs) >> a.log2g;                           \
+            const uint32_t g_ = ((it_base + it_) * DBK + kofs) >> a.log2g;               \
             ps[SET] = *(const uint16_t*)(a.scales + soff + (size_t)g_ * 2);              \
             pb[SET] = *(const uint16_t*)(a.biases + soff + (size_t)g_ * 2);              \
         }                                                                                \
@@ -156,7 +170,7 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
 
     auto scale_bias = [&](uint32_t it_, int set, float& s_, float& b_) {
         if constexpr (SBL) {
-            const uint32_t g_ = (min(it_, a.iters - 1) * DBK + kofs) >> a.log2g;
+            const uint32_t g_ = (((it_base + min(it_, a.iters - 1)) * DBK + kofs) >> a.log2g) - sb_g0;
             s_ = elem_bits_to_f32<DT>(sbS[sbrow + g_]);
             b_ = elem_bits_to_f32<DT>(sbB[sbrow + g_]);
         } else {
@@ -180,12 +194,12 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
     if constexpr (SBL) {
         // DBN rows x gpr elements each of scales and biases, 16 bytes per load: vector v of
         // the tile covers elements [8*(v % vpr), +8) of row v / vpr
-        const uint32_t vpr = a.gpr / 8, nvec = DBN * vpr;
+        const uint32_t vpr = sb_ng / 8, nvec = DBN * vpr;
         for (uint32_t v = tid; v < nvec; v += NT) {
             const uint32_t row = v / vpr, c0 = (v - row * vpr) * 8;
             const uint32_t grow = min(n0 + row, a.N - 1);
-            const q_u32x4 sv = *(const q_u32x4*)((const uint16_t*)a.scales + (size_t)grow * a.gpr + c0);
-            const q_u32x4 bv = *(const q_u32x4*)((const uint16_t*)a.biases + (size_t)grow * a.gpr + c0);
+            const q_u32x4 sv = *(const q_u32x4*)((const uint16_t*)a.scales + (size_t)grow * a.gpr + sb_g0 + c0);
+            const q_u32x4 bv = *(const q_u32x4*)((const uint16_t*)a.biases + (size_t)grow * a.gpr + sb_g0 + c0);
             uint32_t* ds = (uint32_t*)(sbS + row * sbld + c0);
             uint32_t* db = (uint32_t*)(sbB + row * sbld + c0);
             ds[0] = sv.x; ds[1] = sv.y; ds[2] = sv.z; ds[3] = sv.w;
@@ -294,9 +308,15 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
                 float r = acc[bi][v];
 #pragma unroll
                 for (int g = 0; g < KG - 1; g++) r += red[g * GRP + ((wn * MB + bi) * 16 + v) * 64 + lane];
-                otile[lrow * DBN + wn * 32 + fr] = f32_to_elem_bits<DT>(r);
+                if (!GR && a.ksplit > 1) {  // this split's f32 partial sums, 32 consecutive columns per half wave
+                    const uint32_t col = n0 + wn * 32 + fr;
+                    if (lrow < row_count && col < a.N) a.part[((size_t)blockIdx.y * a.M + row_first + lrow) * a.N + col] = r;
+                } else {
+                    otile[lrow * DBN + wn * 32 + fr] = f32_to_elem_bits<DT>(r);
+                }
             }
     }
+    if (!GR && a.ksplit > 1) return;  // the whole workgroup: ksplit is a launch constant
     __syncthreads();
     // all threads store the tile, 16 bytes each, whole rows
     constexpr int VPR = DBN / 8;                    // 16-byte vectors per tile row

@@ -24,7 +24,7 @@ def options():
         assert lib.mtq_set_option(name.encode(), value) == 0, name
 
     yield set_
-    for name in ("qmm.kernel", "qmm.kgroups", "qmm.tile_rows", "qmm.by_m"):
+    for name in ("qmm.kernel", "qmm.kgroups", "qmm.tile_rows", "qmm.by_m", "qmm.ksplit"):
         lib.mtq_set_option(name.encode(), 0)
 
 
@@ -171,3 +171,52 @@ def test_bit_stream_widths_route_to_tiles(oracle, bits, M):
     for buf in (w, s, b, x, out):
         buf.free()
     assert rel_err(got, exp) <= 2e-2
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
+def test_direct_qmm_split_k(oracle, options, bits, dt):
+    """K cut into splits whose f32 partial tiles a second kernel adds in order: forced split counts that
+    do and do not divide the iteration count (K = 1792 is 7 iterations of 256 and 14 of 128), ragged M and
+    N, group sizes 32 and 128 (a split may start inside a group), and the automatic choice on a short, wide
+    matrix. Against the mma-semantics oracle, 2e-2 as for the prefill configuration; a guard band after the
+    output must stay untouched."""
+    for (M, N, K, G) in ((20, 200, 1792, 128), (70, 72, 1792, 32)):
+        c = make_case(5900 + bits + M, dt, bits, G, M, N, K)
+        exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
+        exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+        w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                      GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+        options("qmm.kernel", 2)
+        for ks in (0, 1, 2, 3, 5, 7):
+            print(f"[case] split-K qmm {dt.name} b{bits} M{M} N{N} K{K} g{G} ksplit={ks}", flush=True)
+            options("qmm.ksplit", ks)
+            out = GpuBuffer.from_bytes(np.full(M * N + 512, 0x7B7B, np.uint16).tobytes())
+            ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+            raw = np.frombuffer(out.read_bytes(), np.uint16)
+            out.free()
+            assert np.all(raw[M * N:] == 0x7B7B)
+            err = rel_err(unpack_f32(raw[:M * N].tobytes(), dt), exp)
+            assert err <= 2e-2, f"ksplit={ks}: rel err {err:.3e}"
+        for buf in (w, s, b, x):
+            buf.free()
+
+
+def test_split_k_is_deterministic_and_close_to_unsplit(options):
+    """Two runs of a split launch give the same bits (the splits are added in a fixed order), and the
+    split result differs from the unsplit one only by the order of the f32 sums."""
+    dt, bits, G, M, N, K = DType.BF16, 4, 64, 32, 256, 8192
+    c = make_case(5999, dt, bits, G, M, N, K)
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    res = {}
+    for ks in (1, 0, 0):
+        options("qmm.ksplit", ks)
+        out = GpuBuffer(M * N * 2)
+        ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+        res.setdefault(ks, []).append(out.read_bytes())
+        out.free()
+    for buf in (w, s, b, x):
+        buf.free()
+    assert res[0][0] == res[0][1]
+    assert rel_err(unpack_f32(res[0][0], dt), unpack_f32(res[1][0], dt)) <= 1e-2
