@@ -246,19 +246,49 @@ struct TileTabArgs {
     uint32_t E, T, tile_rows, max_tiles, tail_to_0;
 };
 __global__ __launch_bounds__(64) void gather_tiles_kernel(TileTabArgs a) {
-    if (threadIdx.x != 0) return;  // E is small next to the GEMM that follows: one lane, in order
-    uint32_t n = 0, mx = 0;
+    // One wave, 64 experts at a time: lane l takes expert base + l. The rule needs, per expert, the
+    // largest offset before it (a running maximum) and the number of tiles before it (a running sum);
+    // both are wave scans, carried from one batch of 64 to the next, so the table comes out in expert
+    // order exactly as a serial walk would write it, without a chain of dependent loads.
+    const uint32_t lane = threadIdx.x;
+    uint32_t n = 0, mx = 0;  // carried: tiles so far, largest offset so far (wave-uniform)
     uint4* tab = (uint4*)a.tiles + 1;
-    auto emit = [&](uint32_t e, uint32_t lo, uint32_t hi) {
-        for (uint32_t r = lo; r < hi && n < a.max_tiles; r += a.tile_rows, n++) tab[n] = make_uint4(e, r, min(a.tile_rows, hi - r), 0u);
+    auto emit = [&](uint32_t first, uint32_t e, uint32_t lo, uint32_t hi) {
+        uint32_t i = first;
+        for (uint32_t r = lo; r < hi && i < a.max_tiles; r += a.tile_rows, i++) tab[i] = make_uint4(e, r, min(a.tile_rows, hi - r), 0u);
     };
-    for (uint32_t e = 0; e < a.E; e++) {
-        const uint32_t lo = min(mx, a.T), hi = min(a.off[e + 1], a.T);
-        if (hi > lo) emit(e, lo, hi);
-        mx = max(mx, a.off[e + 1]);
+    for (uint32_t base = 0; base < a.E; base += 64) {
+        const uint32_t e = base + lane;
+        const uint32_t o1 = e < a.E ? a.off[e + 1] : 0u;
+        // inclusive running maximum over the lanes
+        uint32_t pm = o1;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t t = __shfl_up(pm, d, 64);
+            if (lane >= (uint32_t)d) pm = max(pm, t);
+        }
+        uint32_t before = __shfl_up(pm, 1, 64);  // largest offset of the earlier lanes of this batch
+        before = lane == 0 ? mx : max(mx, before);
+        const uint32_t lo = min(before, a.T), hi = min(o1, a.T);
+        const uint32_t cnt = (e < a.E && hi > lo) ? (hi - lo + a.tile_rows - 1) / a.tile_rows : 0u;
+        uint32_t ps = cnt;  // inclusive running sum of tile counts
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t t = __shfl_up(ps, d, 64);
+            if (lane >= (uint32_t)d) ps += t;
+        }
+        if (cnt) emit(n + ps - cnt, e, lo, hi);
+        n += __shfl(ps, 63, 64);
+        mx = max(mx, __shfl(pm, 63, 64));
     }
-    if (a.tail_to_0 && mx < a.T) emit(0u, mx, a.T);
-    a.tiles[0] = n;
+    if (lane == 0) {
+        if (a.tail_to_0 && mx < a.T) {
+            const uint32_t cnt = (a.T - mx + a.tile_rows - 1) / a.tile_rows;
+            emit(n, 0u, mx, a.T);
+            n += cnt;
+        }
+        a.tiles[0] = min(n, a.max_tiles);
+    }
 }
 
 size_t qmm_grouped_scratch_bytes(uint32_t T, uint32_t E, bool sort_rows, uint32_t tile_rows) {
