@@ -133,7 +133,7 @@ MTQ_API int mtq_qmm(int dtype, int bits, uint32_t group_size, const void *w, con
  * mt_moe_gather_qmm_int4{,_m8,_m16,_m32} and _b* (crates/metaltile-std/src/ffai/moe.rs:358,
  * 634, 900, 1363, 461-605). w is [E][N][K*bits/32], scales/biases [E][N][K/G],
  * x [T][K], expert_offsets u32[E+1], out [T][N].
- * Both row views: while experts average at most 16 rows, each expert's rows run on the
+ * Both row views: while experts average at most 8 rows, each expert's rows run on the
  * GEMV kernels (exact w_hat = s*q + b in f32); above that the rows are grouped by expert
  * into 64-row tiles on the MFMA tile kernel, where w_hat is rounded to the element type
  * first, as in the reference's MMA gathers (moe.rs:2256); MTQ_F32 rows always run grouped, in

@@ -299,11 +299,11 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
     p.M = 1; p.N = N; p.K = K;
     p.gather = mode; p.route = route; p.T = mode == GATHER_SINGLE ? 1 : T; p.E = E;
     // Many rows per expert (a prefill through an MoE layer): the GEMV family would stream every
-    // expert's weights once per 8 or 16 of its rows, so the rows go to the tile kernel, grouped by
-    // expert, like the reference's MMA gather kernels (crates/metaltile-std/src/ffai/moe.rs:2256).
-    // Measured crossover: 16 rows per expert, the most one GEMV pass takes (8 experts x 14336x4096:
-    // 16 rows each 97 us GEMV / 84 us tiles, 24 rows 139 / 87, 256 rows 588 / 88; 128 experts x
-    // 2048x768: 24 rows each 231 / 80 us; at 8 rows each the GEMV wins, 51 us against 119).
+    // expert's weights once per 8 of its rows, so the rows go to the tile kernel, grouped by expert,
+    // like the reference's MMA gather kernels (crates/metaltile-std/src/ffai/moe.rs:2256). Measured
+    // crossover: 8 rows per expert, the most one GEMV pass takes (GEMV / tiles, us, 10 rows each:
+    // 128 experts x 2048x768 125 / 52, 768x2048 56 / 44, 64 x 1408x2048 51 / 41, 8 x 14336x4096
+    // 118 / 94, 8 x 4096x2048 25 / 28; 6 rows each: 69 / 53, 36 / 44, 38 / 41, 64 / 134, 19 / 28).
     const int gopt = options().gather_grouped;
     // f32 rows always go grouped to the f32 matrix-core kernel: the f32 dot kernels take 4 rows per pass
     // and lose at any routing (128 experts x 256x2048: 64 rows 64 us against 48, 1024 rows 315 against 88;
@@ -319,7 +319,7 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
         rc = launch_qmm_f32_grouped(q, route, ids, T, E, g.scratch_buf, lc);
         if (rc != ERR_UNSUPPORTED) return rc;
     }
-    if (dtype != DT_F32 && mode != GATHER_SINGLE && gopt != 1 && (gopt == 2 || (uint64_t)T > (uint64_t)16 * (E < T ? E : T))) {
+    if (dtype != DT_F32 && mode != GATHER_SINGLE && gopt != 1 && (gopt == 2 || (uint64_t)T > (uint64_t)8 * (E < T ? E : T))) {
         QmmParams q;
         q.dtype = dtype; q.bits = bits; q.group_size = G;
         q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
