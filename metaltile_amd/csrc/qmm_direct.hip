@@ -144,7 +144,16 @@ static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
     if (p.M <= 32) { rows = 32; kgroups = 4; }
     else if (p.M <= 64) { rows = 64; kgroups = short_wide <= (uint64_t)cus ? 4 : 2; }
     else if (tall_wide >= 2 * (uint64_t)cus) { rows = 128; kgroups = 1; }  // two 4-wave workgroups per CU (M = 2048: 72-75 us against 80-84; M = 4096: 160-170 against 180-190)
-    else if (tall_wide >= (uint64_t)cus) { rows = 128; kgroups = 2; }
+    // Between one and two tall tiles per compute unit the 8-wave workgroups (one per compute unit) run
+    // a second, mostly empty round unless the count is an exact multiple; the 4-wave ones share compute
+    // units and do not (1024 rows: 5120 x 5120 100 -> 82 us, 6144 x 4096 79 -> 68, 5120 x 13824 316 -> 233;
+    // 4096 x 4096, exactly 256 tiles, stays: 42.9 against 47.2).
+    else if (tall_wide >= (uint64_t)cus) { rows = 128; kgroups = tall_wide % (uint64_t)cus == 0 ? 2 : 1; }
+    // Long rows with too few 128 x 128 tiles for the chip (a down projection at 256..512 rows): the
+    // tall tile on 4-wave workgroups with K split so that two of them share a compute unit beats the
+    // 64-row tiles (512 rows, 4096 x 14336: 131 -> 95 us; 4096 x 11008: 99 -> 78; 5120 x 13824: 213 -> 114;
+    // 384 rows, 8192 x 28672: 446 -> 305; at K = 4096 it loses, 29 -> 36).
+    else if (p.M >= 256 && p.K >= 8192) { rows = 128; kgroups = 1; }
     else if (short_wide * 2 <= (uint64_t)cus) {  // few tiles: halve their width, and their height for up to 32 rows
         rows = p.M <= 32 ? 32 : 64;
         kgroups = 4;
@@ -174,11 +183,16 @@ static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
     const uint32_t iters = p.K / (64 * kgroups);
     uint32_t ks = 1;
     if (options().qmm_ksplit > 1) ks = (uint32_t)options().qmm_ksplit;
-    else if (options().qmm_ksplit == 0 && tiles * 2 <= (uint64_t)cus && iters >= QMM_SPLIT_MIN_ITERS) {
+    else if (options().qmm_ksplit == 0 && rows == 128 && kgroups == 1 && p.K >= 8192 && tiles < 2 * (uint64_t)cus) {
+        // tall tiles on long rows: splits to about two 4-wave workgroups per compute unit, rounded
+        ks = (uint32_t)((4 * (uint64_t)cus / tiles + 1) / 2);
+        if (ks > 8) ks = 8;
+        if (ks > iters / 16) ks = iters / 16;
+    } else if (options().qmm_ksplit == 0 && tiles * 2 <= (uint64_t)cus && iters >= QMM_SPLIT_MIN_ITERS) {
         // one workgroup per compute unit, at least 4 iterations each (measured optimum: 4096 x 14336,
         // 32 rows, 64 tiles: 1 / 2 / 4 / 8 / 16 splits 57 / 34 / 23 / 27 / 32 us; 2048 x 8192, 32 tiles:
         // 23 / 17 / 12 / 11 / 12 us; 8192 x 28672, 128 tiles: 108 / 63 / 62 / 66 / 80 us)
-        ks = (uint32_t)((uint64_t)cus / tiles);
+        ks = (uint32_t)((kgroups == 1 ? 2 : 1) * (uint64_t)cus / tiles);  // two 4-wave workgroups share a compute unit
         if (ks > iters / 4) ks = iters / 4;
         if (ks > 16) ks = 16;
     }

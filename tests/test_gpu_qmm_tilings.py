@@ -220,3 +220,24 @@ def test_split_k_is_deterministic_and_close_to_unsplit(options):
         buf.free()
     assert res[0][0] == res[0][1]
     assert rel_err(unpack_f32(res[0][0], dt), unpack_f32(res[1][0], dt)) <= 1e-2
+
+
+@pytest.mark.parametrize("M,N", [(300, 256), (1100, 384)])
+def test_tall_tiles_on_long_rows(oracle, M, N):
+    """256 rows and more against rows of 8192 codes: the default choice is the 128-row tile on 4-wave
+    workgroups with K split (300 x 256: 6 tiles, 8 splits), and above one tile per compute unit an
+    inexact multiple also takes the 4-wave form. Against the mma-semantics oracle, 2e-2 as for the prefill
+    configuration."""
+    K, G, bits, dt = 8192, 64, 4, DType.BF16
+    print(f"[case] qmm M={M} N={N} K={K}", flush=True)
+    c = make_case(6100 + M, dt, bits, G, M, N, K)
+    exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    out = GpuBuffer(M * N * dt.size_bytes)
+    ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+    got = unpack_f32(out.read_bytes(), dt)
+    for buf in (w, s, b, x, out):
+        buf.free()
+    assert rel_err(got, exp) <= 2e-2
