@@ -113,21 +113,28 @@ static int run_gemv(const QmvParams& p, const LaunchCtx& lc) {
     return rc;
 }
 
+static int ensure_scratch(size_t need);
+
 // f32 batches: the f32 matrix-core kernel works 32 activation rows per pass over the weights, the
-// f32 dot kernels 4. Measured at 4096 x 4096: 4-bit, 4 rows 16.9 us on the dot kernels against 24.2 us,
-// 8 rows 33.6 against 24.7, 32 rows 133 against 32; 3-bit (5-, 6-, 7-bit alike: no f32 dot kernel), 1 row
-// 33.6 against 23.5, 2 rows 43.6 against 23.6, 32 rows 534 against 32.
-// Returns ERR_UNSUPPORTED when the rows stay with the GEMV family.
+// f32 dot kernels 4. Measured at 4096 x 4096 (tiles with K split over workgroups): 4-bit, 4 rows 16.6 us
+// on the dot kernels against 16, 8 rows 33.6 against 16.4, 32 rows 133 against 24; 3-bit (5-, 6-, 7-bit
+// alike: no f32 dot kernel, so every row count goes to the tiles), 1 row 25-35 against 15.4, 32 rows 534
+// against 24. Returns ERR_UNSUPPORTED when the rows stay with the GEMV family.
 static int try_f32_tiles(int bits, uint32_t G, const void* w, const void* s, const void* b, const void* x, void* out,
                          uint32_t M, uint32_t N, uint32_t K, const LaunchCtx& lc) {
     const int opt = options().qmm_f32_tiles;
     const bool odd = bits == 3 || bits == 5 || bits == 6 || bits == 7;
-    if (opt == 1 || (opt == 0 && M < (odd ? 2u : 5u))) return ERR_UNSUPPORTED;
+    if (opt == 1 || (opt == 0 && !odd && M < 5u)) return ERR_UNSUPPORTED;
     QmmParams q;
     q.dtype = DT_F32; q.bits = bits; q.group_size = G;
     q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
     q.M = M; q.N = N; q.K = K;
-    return launch_qmm_f32(q, lc);
+    const size_t need = qmm_f32_scratch_bytes(q);  // f32 partial tiles when K is split
+    if (need) {
+        int rc = ensure_scratch(need);
+        if (rc) return rc;
+    }
+    return launch_qmm_f32(q, lc, need ? g.scratch_buf : nullptr);
 }
 
 static int op_qmv(int dtype, int bits, uint32_t G, const void* w, const void* s, const void* b,
@@ -146,8 +153,6 @@ static int op_qmv(int dtype, int bits, uint32_t G, const void* w, const void* s,
     p.M = M; p.N = N; p.K = K;
     return run_gemv(p, lc);
 }
-
-static int ensure_scratch(size_t need);
 
 // Kernel routing by M, the counterpart of mt_qmm_for
 // (crates/metaltile-std/src/mlx/quantized.rs:5040-5065, which sends M = 16 and the multiples

@@ -158,7 +158,9 @@ int launch_qmm_mfma(const QmmParams& p, const LaunchCtx& lc);
 size_t qmm_direct_scratch_bytes(const QmmParams& p);
 int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc, void* scratch);
 // f32 operands on the f32 matrix cores, any code width (qmm_f32.hip).
-int launch_qmm_f32(const QmmParams& p, const LaunchCtx& lc);
+// scratch: qmm_f32_scratch_bytes(p) bytes (0 when K is not split: then scratch may be null).
+size_t qmm_f32_scratch_bytes(const QmmParams& p);
+int launch_qmm_f32(const QmmParams& p, const LaunchCtx& lc, void* scratch);
 // Expert-routed rows on the same kernel (many rows per expert): p holds one expert's shapes (N, K),
 // x [T][K], out [T][N], w / scales / biases the stacked experts. `route` = CSR offsets [E + 1], or one
 // expert id per row when per_row_ids. scratch: qmm_grouped_scratch_bytes() bytes.

@@ -33,6 +33,10 @@ struct QmmFArgs {
     const uint32_t* tiles;
     const uint32_t* rowlist;
     uint64_t w_expert_bytes, sb_expert_elems;
+    // split K (few tiles): workgroup (x, y) takes steps [y * steps_per_split, +steps_per_split) and writes
+    // its partial tile to part[y][M][N]; qmm_f32_split_reduce_kernel adds the splits in order
+    uint32_t ksplit, steps_per_split;
+    float* part;
 };
 
 // code j of 32 codes of BITS bits packed LSB-first into BITS words; j is a constant after unrolling
@@ -72,16 +76,21 @@ __global__ __launch_bounds__(64 * NW) void qmm_f32_kernel(QmmFArgs a) {
         else return row_first + j;
     };
 
+    uint32_t step0 = 0;  // first step of this workgroup's share of K
+    if (!GR && a.ksplit > 1) {
+        step0 = blockIdx.y * a.steps_per_split;
+        a.steps = min(a.steps_per_split, a.steps - step0);
+    }
     // rows and columns past the edge are worked on the last one and not stored
     const uint32_t row = row_of(min(fr, row_count - 1));
-    const float* xp = a.x + (size_t)row * a.K + 32 * fh;
+    const float* xp = a.x + (size_t)row * a.K + 32 * fh + (size_t)step0 * 64;
     const unsigned char* wp[NB];
     const float* sp[NB];
     const float* bp[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
         const uint32_t n = min((nt * NB + nb) * 32 + fr, a.N - 1);
-        wp[nb] = a.w + (size_t)n * ((size_t)a.K * BITS / 8) + fh * 4 * BITS;
+        wp[nb] = a.w + (size_t)n * ((size_t)a.K * BITS / 8) + fh * 4 * BITS + (size_t)step0 * (8 * BITS);
         sp[nb] = a.scales + (size_t)n * a.gpr;
         bp[nb] = a.biases + (size_t)n * a.gpr;
     }
@@ -94,7 +103,7 @@ __global__ __launch_bounds__(64 * NW) void qmm_f32_kernel(QmmFArgs a) {
         const float* xs = xp + (size_t)step * 64;
 #pragma unroll
         for (int i = 0; i < 8; i++) px[set][i] = *(const qf_f32x4*)(xs + 4 * i);
-        const uint32_t g = (step * 64 + 32 * fh) >> a.log2g;
+        const uint32_t g = ((step0 + step) * 64 + 32 * fh) >> a.log2g;
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
             const uint32_t* ws = (const uint32_t*)(wp[nb] + (size_t)step * (8 * BITS));
@@ -155,12 +164,44 @@ __global__ __launch_bounds__(64 * NW) void qmm_f32_kernel(QmmFArgs a) {
 #pragma unroll
             for (int u = 1; u < NW; u++) r += red[u][nb * 16 + v][lane];
             const uint32_t lrow = 8 * (v / 4) + 4 * fh + (v % 4);
-            if (lrow < row_count && col < a.N) a.out[(size_t)row_of(lrow) * a.N + col] = r;
+            if (lrow < row_count && col < a.N) {
+                if (!GR && a.ksplit > 1) a.part[((size_t)blockIdx.y * a.M + row_first + lrow) * a.N + col] = r;
+                else a.out[(size_t)row_of(lrow) * a.N + col] = r;
+            }
         }
     }
 }
 
-int launch_qmm_f32(const QmmParams& p, const LaunchCtx& lc) {
+// Adds the K splits' partial tiles in split order.
+__global__ __launch_bounds__(256) void qmm_f32_split_reduce_kernel(const float* part, float* out, uint32_t total, uint32_t ksplit) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    float r = part[i];
+    for (uint32_t sp = 1; sp < ksplit; sp++) r += part[(size_t)sp * total + i];
+    out[i] = r;
+}
+
+// K splits for a shape: tiles of 32 x 32 fewer than the compute units and rows long enough to give
+// every split 16 steps (4096 x 4096, 32 rows: 128 tiles, the MFMA work of 128 compute units).
+static uint32_t f32_ksplit(const QmmParams& p, int cus) {
+    const uint64_t tiles = (uint64_t)((p.M + 31) / 32) * ((p.N + 31) / 32);
+    const uint32_t steps = p.K / 64;
+    if (options().qmm_ksplit == 1 || tiles * 2 > (uint64_t)cus || steps < 32) return 1;
+    uint32_t ks = options().qmm_ksplit > 1 ? (uint32_t)options().qmm_ksplit : (uint32_t)((uint64_t)cus / tiles);
+    if (ks > steps / 16) ks = steps / 16;
+    if (ks > 8) ks = 8;
+    return ks < 1 ? 1 : ks;
+}
+
+size_t qmm_f32_scratch_bytes(const QmmParams& p) {
+    if (p.dtype != DT_F32 || p.K % 64 || p.M == 0 || p.N == 0) return 0;
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    const uint32_t ks = f32_ksplit(p, cus);
+    return ks > 1 ? (size_t)ks * p.M * p.N * sizeof(float) : 0;
+}
+
+int launch_qmm_f32(const QmmParams& p, const LaunchCtx& lc, void* scratch) {
     const uint32_t G = p.group_size;
     if (p.dtype != DT_F32) return fail(ERR_UNSUPPORTED, "f32 qmm: element type");
     if (p.M == 0 || p.N == 0 || p.K == 0 || p.K % 64 || G < 32 || (G & (G - 1)) || p.K % G)
@@ -187,6 +228,11 @@ int launch_qmm_f32(const QmmParams& p, const LaunchCtx& lc) {
     a.w_expert_bytes = a.sb_expert_elems = 0;
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    uint32_t ks = f32_ksplit(p, cus);
+    if (ks > 1 && !scratch) ks = 1;
+    a.steps_per_split = (a.steps + ks - 1) / ks;
+    a.ksplit = (a.steps + a.steps_per_split - 1) / a.steps_per_split;  // no empty split
+    a.part = (float*)scratch;
     a.m_tiles = (p.M + 31) / 32;
     // two column blocks per wave halve the activation traffic; taken once that still leaves two
     // workgroups for every compute unit. Below that, and with rows long enough to give every wave
@@ -194,7 +240,7 @@ int launch_qmm_f32(const QmmParams& p, const LaunchCtx& lc) {
     // SIMD hide each other's load latency (4096 x 4096, 32 rows: 42 us with 4 waves, 32 us with 16;
     // 128 rows: 62 us with 4 waves, 67 us with 16).
     const int nb = (uint64_t)a.m_tiles * ((p.N + 63) / 64) >= 2 * (uint64_t)cus ? 2 : 1;
-    const int nw = (nb == 1 && a.steps >= 32 && (uint64_t)a.m_tiles * ((p.N + 31) / 32) <= (uint64_t)cus) ? 16 : 4;
+    const int nw = (nb == 1 && a.steps_per_split >= 32 && (uint64_t)a.m_tiles * ((p.N + 31) / 32) * a.ksplit <= (uint64_t)cus) ? 16 : 4;
     a.n_tiles = (p.N + 32 * nb - 1) / (32 * nb);
     if ((uint64_t)a.m_tiles * a.n_tiles >= (1ull << 31)) return fail(ERR_UNSUPPORTED, "f32 qmm: too many tiles");
     const uint64_t x_bytes = (uint64_t)p.M * p.K * 4, w_bytes = (uint64_t)p.N * p.K * p.bits / 8;
@@ -216,6 +262,20 @@ int launch_qmm_f32(const QmmParams& p, const LaunchCtx& lc) {
     }
 #undef QF_PICK
     void* args[] = {&a};
+    if (a.ksplit > 1) {
+        LaunchCtx l1 = lc, l2 = lc;
+        l1.stop = nullptr;
+        l2.start = nullptr;
+        hipError_t e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles, a.ksplit), dim3(64 * nw), args, 0, l1);
+        if (e != hipSuccess) return hip_fail(e, "f32 qmm kernel launch");
+        const float* part = a.part;
+        float* out = a.out;
+        uint32_t total = a.M * a.N, nsp = a.ksplit;
+        void* rargs[] = {&part, &out, &total, &nsp};
+        e = launch_kernel((const void*)qmm_f32_split_reduce_kernel, dim3((total + 255) / 256), dim3(256), rargs, 0, l2);
+        if (e != hipSuccess) return hip_fail(e, "f32 qmm split reduce kernel launch");
+        return ERR_OK;
+    }
     hipError_t e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles), dim3(64 * nw), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "f32 qmm kernel launch");
     return ERR_OK;
@@ -252,6 +312,9 @@ int launch_qmm_f32_grouped(const QmmParams& p, const uint32_t* route, bool per_r
     a.log2g = l;
     a.gpr = p.K / G;
     a.steps = p.K / 64;
+    a.ksplit = 1;
+    a.steps_per_split = a.steps;
+    a.part = nullptr;
     a.tiles = gt.tiles;
     a.rowlist = gt.rowlist;
     a.w_expert_bytes = (uint64_t)p.N * p.K * p.bits / 8;

@@ -142,3 +142,18 @@ def test_f32_gather_default_rule(oracle, grouped, mode):
         assert rel_err(got, np.asarray(exp, np.float32).reshape(-1)) <= 1e-4
         for buf in (w, s, b, x, out, r):
             buf.free()
+
+
+@pytest.mark.parametrize("ks", [0, 1, 3, 8])
+def test_f32_tiles_split_k(oracle, f32_tiles, ks):
+    """Few tiles and long rows: K is cut into splits (chosen, off, forced to counts that do and do not divide
+    the 64 steps of K = 4096) whose partial tiles a second kernel adds in order; ragged M and N."""
+    lib = _lib.load()
+    f32_tiles(2)
+    assert lib.mtq_set_option(b"qmm.ksplit", ks) == 0
+    try:
+        for bits, G in ((4, 64), (3, 128)):
+            print(f"[case] f32 tiles split-K ks={ks} b{bits}", flush=True)
+            assert _run(oracle, 9900 + ks + bits, bits, G, 20, 72, 4096, ops.qmm) <= 2e-4
+    finally:
+        lib.mtq_set_option(b"qmm.ksplit", 0)
