@@ -197,7 +197,7 @@ static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
         if (ks > 16) ks = 16;
     }
     if (ks > iters) ks = iters;
-    if (ks < 1) ks = 1;
+    if (ks < 1 || (uint64_t)p.M * p.N >= (1ull << 31)) ks = 1;  // the reduction indexes the output with 32 bits
     pl.iters_per_split = (iters + ks - 1) / ks;
     pl.ksplit = (iters + pl.iters_per_split - 1) / pl.iters_per_split;  // no empty split
     return ERR_OK;

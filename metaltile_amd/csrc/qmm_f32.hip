@@ -186,7 +186,7 @@ __global__ __launch_bounds__(256) void qmm_f32_split_reduce_kernel(const float* 
 static uint32_t f32_ksplit(const QmmParams& p, int cus) {
     const uint64_t tiles = (uint64_t)((p.M + 31) / 32) * ((p.N + 31) / 32);
     const uint32_t steps = p.K / 64;
-    if (options().qmm_ksplit == 1 || tiles * 2 > (uint64_t)cus || steps < 32) return 1;
+    if (options().qmm_ksplit == 1 || tiles * 2 > (uint64_t)cus || steps < 32 || (uint64_t)p.M * p.N >= (1ull << 31)) return 1;
     uint32_t ks = options().qmm_ksplit > 1 ? (uint32_t)options().qmm_ksplit : (uint32_t)((uint64_t)cus / tiles);
     if (ks > steps / 16) ks = steps / 16;
     if (ks > 8) ks = 8;
