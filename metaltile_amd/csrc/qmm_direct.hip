@@ -70,7 +70,18 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
         case 2: QD_PICK(2); break;
         case 4: QD_PICK(4); break;
         case 8: QD_PICK(8); break;
-        default: fn = qmm_direct_pick_odd(DT, bits, kgroups, a.m_tile_rows, sbl, grouped); break;
+        default: fn = qmm_direct_pick_odd(DT, bits, kgroups, a.m_tile_rows, sbl, grouped, a.ksplit > 1); break;
+    }
+    if (a.ksplit > 1 && !grouped && !odd) {  // the K-split instances: the tilings qmm_direct_split_built() names
+#define QD_S3(B, MBv, KGv) (sbl ? (const void*)qmm_direct_kernel<DT, B, 2, MBv, true, KGv, false, true> : (const void*)qmm_direct_kernel<DT, B, 2, MBv, false, KGv, false, true>)
+#define QD_SPLIT(B) fn = kgroups == 4 ? (a.m_tile_rows == 32 ? QD_S3(B, 1, 4) : QD_S3(B, 2, 4)) : QD_S3(B, 4, 1)
+        switch (bits) {
+            case 2: QD_SPLIT(2); break;
+            case 4: QD_SPLIT(4); break;
+            default: QD_SPLIT(8); break;
+        }
+#undef QD_SPLIT
+#undef QD_S3
     }
     if (!fn) return fail(ERR_UNSUPPORTED, "direct qmm: tiling not built for this code width");
 #undef QD_PICK
@@ -109,6 +120,11 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
 
 // rows of k-iterations below which a K split is not worth its second launch
 static constexpr uint32_t QMM_SPLIT_MIN_ITERS = 16;
+
+// Tilings whose K-split instances are built: 32 x 64 and 64 x 64 on 4 K-groups, 128 x 128 on 1.
+static bool qmm_direct_split_built(uint32_t rows, uint32_t kgroups) {
+    return (kgroups == 4 && (rows == 32 || rows == 64)) || (kgroups == 1 && rows == 128);
+}
 
 struct QmmDPlan {
     uint32_t rows, kgroups, ksplit, iters_per_split;
@@ -202,6 +218,7 @@ static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
     }
     if (ks > iters) ks = iters;
     if (ks < 1 || (uint64_t)p.M * p.N >= (1ull << 31)) ks = 1;  // the reduction indexes the output with 32 bits
+    if (!qmm_direct_split_built(rows, kgroups)) ks = 1;
     pl.iters_per_split = (iters + ks - 1) / ks;
     pl.ksplit = (iters + pl.iters_per_split - 1) / pl.iters_per_split;  // no empty split
     return ERR_OK;

@@ -53,7 +53,7 @@ struct QmmDArgs {
 // KG = 1 is the half-size workgroup: 4 waves, all N-waves of one K-group, 32*MB x 128 tile,
 // 64 k per iteration and no partial sums to combine. Two such workgroups share a compute unit
 // and are not in step with each other, so one's LDS traffic runs under the other's MFMAs.
-template <int DT, int BITS, int PD, int MB, bool SBL, int KG, bool GR = false>
+template <int DT, int BITS, int PD, int MB, bool SBL, int KG, bool GR = false, bool SP = false>
 __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArgs a) {
     constexpr int NW = KG == 1 ? 4 : 8;      // waves
     constexpr int NT = 64 * NW;              // threads
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
     };
     const uint32_t n0 = nt * DBN;
     uint32_t it_base = 0;  // first iteration of this workgroup's share of K
-    if (!GR && a.ksplit > 1) {
+    if constexpr (SP) {
         it_base = blockIdx.y * a.iters_per_split;
         a.iters = min(a.iters_per_split, a.iters - it_base);
         a.x += (size_t)it_base * (DBK * 2);
@@ -126,7 +126,9 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
     const uint32_t sbld = a.gpr + 2;  // row stride in elements; (gpr + 2) / 2 dwords is odd for gpr % 4 == 0: rows spread over the banks
     uint16_t* sbS = (uint16_t*)(lds + 2 * DBUF);
     uint16_t* sbB = sbS + DBN * sbld;
-    const uint32_t sbrow = (wn * 32 + fr) * sbld;
+    // this lane's row in the staged window, less the window's first group: indexed with absolute group numbers
+    const int sbrow = (int)((wn * 32 + fr) * sbld) - (int)sb_g0;
+    const uint32_t kofs_abs = it_base * DBK + kofs;  // k of this lane's codes counted from the start of the row
 
 #define QD_LOAD(IT, SET)                                                                 \
     do {                                                                                 \
@@ -153,7 +155,7 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
             }                                                                            \
         }                                                                                \
         if constexpr (!SBL) {                                                            \
-            const uint32_t g_ = ((it_base + it_) * DBK + kofs) >> a.log2g;               \
+            const uint32_t g_ = (it_ * DBK + kofs_abs) >> a.log2g;                       \
             ps[SET] = *(const uint16_t*)(a.scales + soff + (size_t)g_ * 2);              \
             pb[SET] = *(const uint16_t*)(a.biases + soff + (size_t)g_ * 2);              \
         }                                                                                \
@@ -170,7 +172,7 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
 
     auto scale_bias = [&](uint32_t it_, int set, float& s_, float& b_) {
         if constexpr (SBL) {
-            const uint32_t g_ = (((it_base + min(it_, a.iters - 1)) * DBK + kofs) >> a.log2g) - sb_g0;
+            const int g_ = (int)((min(it_, a.iters - 1) * DBK + kofs_abs) >> a.log2g);
             s_ = elem_bits_to_f32<DT>(sbS[sbrow + g_]);
             b_ = elem_bits_to_f32<DT>(sbB[sbrow + g_]);
         } else {
@@ -308,7 +310,7 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
                 float r = acc[bi][v];
 #pragma unroll
                 for (int g = 0; g < KG - 1; g++) r += red[g * GRP + ((wn * MB + bi) * 16 + v) * 64 + lane];
-                if (!GR && a.ksplit > 1) {  // this split's f32 partial sums, 32 consecutive columns per half wave
+                if constexpr (SP) {  // this split's f32 partial sums, 32 consecutive columns per half wave
                     const uint32_t col = n0 + wn * 32 + fr;
                     if (lrow < row_count && col < a.N) a.part[((size_t)blockIdx.y * a.M + row_first + lrow) * a.N + col] = r;
                 } else {
@@ -316,7 +318,7 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
                 }
             }
     }
-    if (!GR && a.ksplit > 1) return;  // the whole workgroup: ksplit is a launch constant
+    if constexpr (SP) return;  // split instances end here: the second kernel rounds and stores
     __syncthreads();
     // all threads store the tile, 16 bytes each, whole rows
     constexpr int VPR = DBN / 8;                    // 16-byte vectors per tile row
@@ -339,6 +341,6 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
 }
 
 // Kernel for 3-, 5-, 6- and 7-bit codes (qmm_direct_odd.hip); null when the combination is not built.
-const void* qmm_direct_pick_odd(int dtype, int bits, uint32_t kgroups, uint32_t tile_rows, bool sbl, bool grouped);
+const void* qmm_direct_pick_odd(int dtype, int bits, uint32_t kgroups, uint32_t tile_rows, bool sbl, bool grouped, bool split);
 
 }  // namespace mtq

@@ -9,11 +9,19 @@
 
 namespace mtq {
 
-template <int DT, int B> static const void* pick_b(uint32_t kgroups, uint32_t tile_rows, bool sbl, bool grouped) {
+template <int DT, int B> static const void* pick_b(uint32_t kgroups, uint32_t tile_rows, bool sbl, bool grouped, bool split) {
 #define QO(MBv, KGv, GRv) (sbl ? (const void*)qmm_direct_kernel<DT, B, 2, MBv, true, KGv, GRv> : (const void*)qmm_direct_kernel<DT, B, 2, MBv, false, KGv, GRv>)
     if (grouped) {
         if (tile_rows != 64) return nullptr;
         return kgroups == 4 ? QO(2, 4, true) : kgroups == 2 ? QO(2, 2, true) : nullptr;
+    }
+    if (split) {  // K-split instances (f32 partial tiles, no store of their own)
+#define QS(MBv, KGv) (sbl ? (const void*)qmm_direct_kernel<DT, B, 2, MBv, true, KGv, false, true> : (const void*)qmm_direct_kernel<DT, B, 2, MBv, false, KGv, false, true>)
+        if (tile_rows == 128 && kgroups == 1) return QS(4, 1);
+        if (tile_rows == 64 && kgroups == 4) return QS(2, 4);
+        if (tile_rows == 32 && kgroups == 4) return QS(1, 4);
+        return nullptr;
+#undef QS
     }
     if (tile_rows == 128 && kgroups == 1) return QO(4, 1, false);
     if (tile_rows == 64 && kgroups == 2) return QO(2, 2, false);
@@ -24,19 +32,19 @@ template <int DT, int B> static const void* pick_b(uint32_t kgroups, uint32_t ti
 #undef QO
 }
 
-template <int DT> static const void* pick_dt(int bits, uint32_t kgroups, uint32_t tile_rows, bool sbl, bool grouped) {
+template <int DT> static const void* pick_dt(int bits, uint32_t kgroups, uint32_t tile_rows, bool sbl, bool grouped, bool split) {
     switch (bits) {
-        case 3: return pick_b<DT, 3>(kgroups, tile_rows, sbl, grouped);
-        case 5: return pick_b<DT, 5>(kgroups, tile_rows, sbl, grouped);
-        case 6: return pick_b<DT, 6>(kgroups, tile_rows, sbl, grouped);
-        case 7: return pick_b<DT, 7>(kgroups, tile_rows, sbl, grouped);
+        case 3: return pick_b<DT, 3>(kgroups, tile_rows, sbl, grouped, split);
+        case 5: return pick_b<DT, 5>(kgroups, tile_rows, sbl, grouped, split);
+        case 6: return pick_b<DT, 6>(kgroups, tile_rows, sbl, grouped, split);
+        case 7: return pick_b<DT, 7>(kgroups, tile_rows, sbl, grouped, split);
         default: return nullptr;
     }
 }
 
-const void* qmm_direct_pick_odd(int dtype, int bits, uint32_t kgroups, uint32_t tile_rows, bool sbl, bool grouped) {
-    return dtype == DT_BF16 ? pick_dt<DT_BF16>(bits, kgroups, tile_rows, sbl, grouped)
-         : dtype == DT_F16 ? pick_dt<DT_F16>(bits, kgroups, tile_rows, sbl, grouped) : nullptr;
+const void* qmm_direct_pick_odd(int dtype, int bits, uint32_t kgroups, uint32_t tile_rows, bool sbl, bool grouped, bool split) {
+    return dtype == DT_BF16 ? pick_dt<DT_BF16>(bits, kgroups, tile_rows, sbl, grouped, split)
+         : dtype == DT_F16 ? pick_dt<DT_F16>(bits, kgroups, tile_rows, sbl, grouped, split) : nullptr;
 }
 
 }  // namespace mtq
