@@ -37,7 +37,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=8, help="distinct MLP weight sets streamed per step")
-    ap.add_argument("--workload", default="qmv", choices=["qmv", "qkv", "qmm", "gather", "quantize", "dequantize", "copy"],
+    ap.add_argument("--workload", default="qmv", choices=["qmv", "qkv", "qmm", "gather", "gather_prefill", "quantize", "dequantize", "copy"],
                     help="qmv is the headline; qmm / gather report the other configurations; "
                          "copy runs only the known-size copy kernel (counter calibration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -283,6 +283,39 @@ def main():
                          "frac": round(nbytes / kern_avg / 1e3 / HBM_PEAK_GBS, 4),
                          "traffic": traffic_from_profiles("gather_bf16_b4_e8"), "avg_launch_us_timed_region": round(kern_avg, 3),
                          "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(float(per.min()), 3)}},
+        })
+        print(json.dumps(out))
+        return
+
+    if a.workload == "gather_prefill":
+        # a prefill through an MoE layer: 2048 rows routed by per-row ids (unsorted) to 8 experts of 4096 x 4096;
+        # the rows run grouped by expert on the MFMA tile kernel (sort + tile table + one tile launch)
+        E, N, K, G, T = 8, 4096, 4096, 64, 2048
+        rng = np.random.default_rng(8100)
+        ids = rng.integers(0, E, size=T).astype("<u4")
+        consts = {"m_total": T, "n_out": N, "k_in": K, "group_size": G}
+        specs, keep = [], []
+        for i in range(2):
+            bufs = {"x": GpuBuffer.from_bytes(m.pack_f32(rng.standard_normal(T * K).astype(np.float32), dt)),
+                    "w": GpuBuffer.from_bytes(rng.integers(0, 2 ** 32, size=E * N * K // 8, dtype=np.uint32).tobytes()),
+                    "scales": GpuBuffer.from_bytes(m.pack_f32(np.full(E * N * (K // G), 0.01, np.float32), dt)),
+                    "biases": GpuBuffer.from_bytes(m.pack_f32(np.full(E * N * (K // G), -0.07, np.float32), dt)),
+                    "indices": GpuBuffer.from_bytes(ids.tobytes()), "out": GpuBuffer(T * N * 2)}
+            keep.append(bufs)
+            specs.append(("mt_moe_gather_qmm_mma_int4", dt, bufs, consts))
+        runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
+        _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+        call_avg = chain_us / (a.steps * len(specs))
+        flop = 2.0 * T * N * K
+        out.update({
+            "metric": "gather_qmv TFLOP/s, 2048 rows over 8 experts (4-bit g64 bf16, N=K=4096, per-row ids)",
+            "value": round(flop * len(specs) * a.steps / wall_us / 1e6, 1), "unit": "TFLOP/s",
+            "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
+            "config": {"workload": "gather_qmv grouped by expert, E=8 N=4096 K=4096, 2048 rows, per-row ids", "calls_per_step": len(specs),
+                       "launches_per_call": 3, "device": info["name"] or info["arch"]},
+            "roofline": {"bound": "mfma", "achieved": round(flop / call_avg / 1e6, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(flop / call_avg / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                         "avg_call_us_timed_region": round(call_avg, 3)},
         })
         print(json.dumps(out))
         return
