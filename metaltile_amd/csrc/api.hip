@@ -330,7 +330,7 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
         q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
         q.M = T; q.N = N; q.K = K;
         const bool ids = mode == GATHER_INDICES;
-        rc = ensure_scratch(qmm_grouped_scratch_bytes(T, E, ids));
+        rc = ensure_scratch(qmm_grouped_scratch_bytes(T, E, ids, 32));  // sized for the smaller tile height: more tiles
         if (rc) return rc;
         rc = launch_qmm_grouped(q, route, ids, T, E, g.scratch_buf, lc);
         if (rc != ERR_UNSUPPORTED) return rc;

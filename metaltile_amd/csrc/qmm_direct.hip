@@ -88,12 +88,15 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
 #undef QD_PICK3
     if (grouped && !odd) {  // 64-row tiles, 2 or 4 K-groups
 #define QD_G(B, KGv) (sbl ? (const void*)qmm_direct_kernel<DT, B, 2, 2, true, KGv, true> : (const void*)qmm_direct_kernel<DT, B, 2, 2, false, KGv, true>)
-        if (a.m_tile_rows != 64 || (kgroups != 2 && kgroups != 4)) return fail(ERR_UNSUPPORTED, "grouped qmm: tile shape");
+#define QD_G1(B) (sbl ? (const void*)qmm_direct_kernel<DT, B, 2, 1, true, 4, true> : (const void*)qmm_direct_kernel<DT, B, 2, 1, false, 4, true>)
+        if (!(a.m_tile_rows == 64 && (kgroups == 2 || kgroups == 4)) && !(a.m_tile_rows == 32 && kgroups == 4))
+            return fail(ERR_UNSUPPORTED, "grouped qmm: tile shape");
         switch (bits) {
-            case 2: fn = kgroups == 4 ? QD_G(2, 4) : QD_G(2, 2); break;
-            case 4: fn = kgroups == 4 ? QD_G(4, 4) : QD_G(4, 2); break;
-            default: fn = kgroups == 4 ? QD_G(8, 4) : QD_G(8, 2); break;
+            case 2: fn = a.m_tile_rows == 32 ? QD_G1(2) : kgroups == 4 ? QD_G(2, 4) : QD_G(2, 2); break;
+            case 4: fn = a.m_tile_rows == 32 ? QD_G1(4) : kgroups == 4 ? QD_G(4, 4) : QD_G(4, 2); break;
+            default: fn = a.m_tile_rows == 32 ? QD_G1(8) : kgroups == 4 ? QD_G(8, 4) : QD_G(8, 2); break;
         }
+#undef QD_G1
 #undef QD_G
     }
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -326,6 +329,18 @@ __global__ __launch_bounds__(64) void gather_tiles_kernel(TileTabArgs a) {
     }
 }
 
+// Row-tile height of a grouped launch: 64, or 32 (on 4 K-groups, K % 256 == 0) for large experts with at
+// most 24 rows each on average, where the 64-row tiles are mostly padding (random routing, 12 / 24 rows per
+// expert, 64- against 32-row tiles: 8 x 14336 x 4096 100 / 99 against 85 / 88 us, 8 x 4096 x 4096 43 / 42
+// against 36 / 43). With more rows, or many small experts, the 32-row tiles lose (every weight is converted
+// once per 32 rows instead of 64: 128 x 2048 x 768, 48 rows each: 75 against 137 us).
+static uint32_t grouped_tile_rows(const QmmParams& p, uint32_t T, uint32_t E) {
+    if (p.K % 256 || (p.bits != 2 && p.bits != 4 && p.bits != 8)) return 64u;
+    if (options().qmm_tile_rows == 32) return 32u;
+    if (options().qmm_tile_rows == 64) return 64u;
+    return ((uint64_t)T <= 24ull * E && (uint64_t)p.N * p.K >= (1ull << 24)) ? 32u : 64u;
+}
+
 size_t qmm_grouped_scratch_bytes(uint32_t T, uint32_t E, bool sort_rows, uint32_t tile_rows) {
     const size_t max_tiles = (size_t)(T + tile_rows - 1) / tile_rows + E + 1;
     size_t b = 16 + max_tiles * 16;
@@ -384,8 +399,10 @@ int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_i
         return fail(ERR_UNSUPPORTED, "grouped qmm: operand too large");
     if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.out % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
         return fail(ERR_UNSUPPORTED, "grouped qmm: operands must be 16-byte aligned");
+    // 32-row tiles (on 4 K-groups) where the experts' rows would leave the 64-row tiles mostly padding
+    const uint32_t tile_rows = grouped_tile_rows(p, T, E);
     GatherTiles gt;
-    int rc = build_gather_tiles(route, per_row_ids, T, E, 64u, scratch, lc, gt);
+    int rc = build_gather_tiles(route, per_row_ids, T, E, tile_rows, scratch, lc, gt);
     if (rc) return rc;
     const uint32_t max_tiles = gt.max_tiles;
     uint32_t* tiles = gt.tiles;
@@ -412,7 +429,8 @@ int launch_qmm_grouped(const QmmParams& p, const uint32_t* route, bool per_row_i
     // 768 x 2048, 10 rows each: 68 us on 4 K-groups, 44 us on 2).
     const uint64_t row_tiles = (uint64_t)(T + 63) / 64 + (E < T ? E : T) / 2;
     uint32_t kgroups = (row_tiles * ((p.N + 127) / 128) * 2 <= (uint64_t)cus && p.K % 256 == 0) ? 4 : 2;
-    a.m_tile_rows = 64;
+    if (tile_rows == 32) kgroups = 4;
+    a.m_tile_rows = tile_rows;
     a.m_tiles = max_tiles;
     a.n_tiles = (p.N + 32 * (8 / kgroups) - 1) / (32 * (8 / kgroups));
     a.iters = p.K / (64 * kgroups);

@@ -162,3 +162,37 @@ def test_grouped_gather_ragged_n(oracle, grouped, N):
     assert rel_err(got, exp.reshape(-1)) <= 2e-2
     for buf in (w, s, b, x, out, r):
         buf.free()
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_grouped_gather_on_32_row_tiles(oracle, grouped, bits):
+    """The grouped launch on 32-row tiles (the choice for few rows per expert on large experts, forced here
+    through the option): uneven counts, an empty expert, shuffled per-row ids and the CSR view."""
+    lib = _lib.load()
+    dt, E, N, K, G = DType.BF16, 5, 200, 512, 64
+    counts = [40, 0, 70, 3, 33]
+    T = sum(counts)
+    c = make_case(7600 + bits, dt, bits, G, T, N, K, E=E)
+    ids_sorted = np.repeat(np.arange(E), counts).astype("<u4")
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype("<u4")
+    ids_shuffled = ids_sorted[np.random.default_rng(4).permutation(T)]
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    grouped(2)
+    assert lib.mtq_set_option(b"qmm.tile_rows", 32) == 0
+    try:
+        for view, route, fn, ids in (("csr", offsets, ops.gather_qmv_csr, ids_sorted),
+                                     ("indices shuffled", ids_shuffled, ops.gather_qmv_indices, ids_shuffled)):
+            print(f"[case] grouped gather, 32-row tiles, {view} b{bits}", flush=True)
+            out = GpuBuffer.from_bytes(np.full(T * N + 256, 0x7B7B, np.uint16).tobytes())
+            r = GpuBuffer.from_bytes(route.tobytes())
+            fn(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+            raw = np.frombuffer(out.read_bytes(), np.uint16)
+            out.free(); r.free()
+            assert np.all(raw[T * N:] == 0x7B7B), view
+            got = unpack_f32(raw[:T * N].tobytes(), dt)
+            assert rel_err(got, _expected(oracle, c, ids, T, N, K, E, bits, G, dt)) <= 2e-2, view
+    finally:
+        lib.mtq_set_option(b"qmm.tile_rows", 0)
+    for buf in (w, s, b, x):
+        buf.free()
