@@ -90,7 +90,9 @@ MTQ_API const char *mtq_last_error(void);
 MTQ_API int mtq_device_name(char *out, size_t cap);
 MTQ_API int mtq_get_device_info(mtq_device_info *out);
 /* Use a caller-owned hipStream_t (passed as void*) for all later launches;
- * NULL restores the library's own stream. */
+ * NULL restores the library's own stream. Waits for the work queued on the stream
+ * being left: several ops share one library-owned scratch buffer, so launches of
+ * such ops must not overlap across streams. */
 MTQ_API int mtq_set_stream(void *hip_stream);
 
 /* ---- buffers ------------------------------------------------------------ */

@@ -52,6 +52,7 @@ struct State {
     void* flush_buf = nullptr;
     void* scratch_buf = nullptr;     // library-owned scratch: normalised rows, qvm partial sums
     size_t scratch_bytes = 0;
+    size_t scratch_held = 0;         // bytes at the front of scratch_buf that the running op keeps for itself
     size_t flush_bytes = 0;
     hipDeviceProp_t prop;
     bool timed_armed = false;    // next typed launch attaches the events
@@ -131,10 +132,11 @@ static int try_f32_tiles(int bits, uint32_t G, const void* w, const void* s, con
     q.M = M; q.N = N; q.K = K;
     const size_t need = qmm_f32_scratch_bytes(q);  // f32 partial tiles when K is split
     if (need) {
-        int rc = ensure_scratch(need);
+        // behind whatever the calling op holds at the front of the buffer (a normalised row)
+        int rc = ensure_scratch(g.scratch_held + need);
         if (rc) return rc;
     }
-    return launch_qmm_f32(q, lc, need ? g.scratch_buf : nullptr);
+    return launch_qmm_f32(q, lc, need ? (char*)g.scratch_buf + g.scratch_held : nullptr);
 }
 
 static int op_qmv(int dtype, int bits, uint32_t G, const void* w, const void* s, const void* b,
@@ -184,10 +186,10 @@ static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s,
         if (options().qmm_kernel != 1) {
             const size_t need = qmm_direct_scratch_bytes(q);  // f32 partial tiles when K is split
             if (need) {
-                rc = ensure_scratch(need);
+                rc = ensure_scratch(g.scratch_held + need);
                 if (rc) return rc;
             }
-            rc = launch_qmm_direct(q, lc, need ? g.scratch_buf : nullptr);
+            rc = launch_qmm_direct(q, lc, need ? (char*)g.scratch_buf + g.scratch_held : nullptr);
             if (rc != ERR_UNSUPPORTED) return rc;
         }
         rc = launch_qmm_mfma(q, lc);
@@ -245,8 +247,18 @@ static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const
     const size_t sz = esize(dtype);
     const uint32_t rows = dtype == DT_F32 ? 1u : 2u;
     const size_t x_bytes = ((size_t)rows * K * sz + 255) & ~(size_t)255;
-    const size_t need = x_bytes + (rows == 2 ? (size_t)2 * N * sz : 0);
-    rc = ensure_scratch(need);
+    const size_t held = (x_bytes + (rows == 2 ? (size_t)2 * N * sz : 0) + 255) & ~(size_t)255;
+    // The qmv that follows may itself want scratch (f32 rows on the tile kernel split K into partial
+    // tiles): size the buffer for both now, so that it is not reallocated under the normalised row, and
+    // let that qmv work behind the held part, so that its partial tiles do not overwrite the row it reads.
+    size_t inner = 0;
+    if (dtype == DT_F32) {
+        QmmParams q;
+        q.dtype = dtype; q.bits = bits; q.group_size = G; q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
+        q.M = rows; q.N = N; q.K = K;
+        inner = qmm_f32_scratch_bytes(q);
+    }
+    rc = ensure_scratch(held + inner);
     if (rc) return rc;
     LaunchCtx first = lc, mid = lc, last = lc;
     first.stop = nullptr;
@@ -254,9 +266,15 @@ static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const
     last.start = nullptr;
     rc = launch_rms_norm(dtype, x, norm_w, eps, g.scratch_buf, K, first);
     if (rc) return rc;
-    if (rows == 1) return op_qmv(dtype, bits, G, w, s, b, g.scratch_buf, out, 1, N, K, last);
+    g.scratch_held = held;
+    if (rows == 1) {
+        rc = op_qmv(dtype, bits, G, w, s, b, g.scratch_buf, out, 1, N, K, last);
+        g.scratch_held = 0;
+        return rc;
+    }
     char* part = (char*)g.scratch_buf + x_bytes;
     rc = op_qmv(dtype, bits, G, w, s, b, g.scratch_buf, part, 2, N, K, mid);
+    g.scratch_held = 0;
     if (rc) return rc;
     return launch_add_rows(dtype, part, part + (size_t)N * sz, out, N, last);
 }
@@ -777,7 +795,11 @@ int mtq_get_device_info(mtq_device_info* out) {
 int mtq_set_stream(void* hip_stream) {
     int rc = need_ready();
     if (rc) return rc;
-    g.stream = hip_stream ? (hipStream_t)hip_stream : g.own_stream;
+    hipStream_t next = hip_stream ? (hipStream_t)hip_stream : g.own_stream;
+    // launches queued on the stream being left may still use the library-owned scratch buffer,
+    // which the next stream's launches would reuse (or regrow) with no ordering between the two
+    if (next != g.stream) MTQ_HIP(hipStreamSynchronize(g.stream));
+    g.stream = next;
     return MTQ_OK;
 }
 
