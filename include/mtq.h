@@ -173,6 +173,17 @@ MTQ_API int mtq_gather_qmv_single(int dtype, int bits, uint32_t group_size, cons
 MTQ_API int mtq_qvm(int dtype, int bits, uint32_t group_size, const void *w, const void *scales, const void *biases,
                     const void *x, void *out, uint32_t M, uint32_t N, uint32_t K);
 
+/* mtq_qvm for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same
+ * arguments, same kernels and bit-identical results as mtq_qvm, but the f32 partial rows go
+ * through a 4 MiB array that is part of the library's code object instead of a library-owned
+ * allocation: the call makes no hipMalloc / hipFree. Shapes whose partial rows
+ * (M * slices * N * 4 bytes, slices = about 512 / (ceil(N / 512) * M) workgroups' worth) exceed
+ * 4 MiB fail with MTQ_ERR_UNSUPPORTED. Every call on a GPU shares that GPU's array: calls that
+ * overlap on one GPU (two streams, two threads) race; calls on one stream are ordered. */
+MTQ_API int mtq_qvm_noalloc(int dtype, int bits, uint32_t group_size, const void *w, const void *scales,
+                            const void *biases, const void *x, void *out, uint32_t M, uint32_t N, uint32_t K);
+
 /* Batched qmv: n_mats (1..4) weight matrices of the same K, code width and group size
  * against ONE activation row, in one launch: outs[j][n] = sum_k w_hat_j[n,k] * x[k].
  * Replaces ffai_batched_qkv_qgemv / _fast (three matrices, one concatenated output:

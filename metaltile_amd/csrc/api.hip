@@ -60,6 +60,15 @@ struct State {
 };
 static State g;
 
+// Scratch of mtq_qvm_noalloc: part of the code object, so it exists on every GPU the library is
+// loaded on without any allocation call. `noalloc_scratch` names the array for the host only as a
+// symbol; its address on a device comes from hipGetSymbolAddress (looked up once per device in
+// mtq_init) and that address is what the launches are given.
+static constexpr size_t kNoallocScratchBytes = (size_t)4 << 20;
+static __device__ __align__(256) unsigned char noalloc_scratch[kNoallocScratchBytes];
+static constexpr int kMaxDevices = 64;
+static void* g_noalloc_ptr[kMaxDevices] = {};
+
 static int need_ready() {
     if (!g.ready) return fail(ERR_NO_DEVICE, "mtq_init has not succeeded (no usable GPU?)");
     return ERR_OK;
@@ -742,6 +751,11 @@ int mtq_init(int device) {
     MTQ_HIP(hipGetDeviceProperties(&g.prop, device));
     if (strncmp(g.prop.gcnArchName, "gfx950", 6) != 0)
         return fail(ERR_NO_DEVICE, std::string("kernels are built for gfx950 only, device is ") + g.prop.gcnArchName);
+    if (device < kMaxDevices && !g_noalloc_ptr[device]) {
+        void* sp = nullptr;
+        MTQ_HIP(hipGetSymbolAddress(&sp, HIP_SYMBOL(noalloc_scratch)));
+        g_noalloc_ptr[device] = sp;
+    }
     MTQ_HIP(hipStreamCreateWithFlags(&g.own_stream, hipStreamNonBlocking));
     MTQ_HIP(hipEventCreate(&g.ev_start));
     MTQ_HIP(hipEventCreate(&g.ev_stop));
@@ -907,6 +921,33 @@ int mtq_qvm(int dtype, int bits, uint32_t group_size, const void* w, const void*
     int rc = need_ready();
     if (rc) return rc;
     return op_qvm(dtype, bits, group_size, w, scales, biases, x, out, M, N, K, make_ctx());
+}
+
+int mtq_qvm_noalloc(int dtype, int bits, uint32_t group_size, const void* w, const void* scales, const void* biases,
+                    const void* x, void* out, uint32_t M, uint32_t N, uint32_t K) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (dtype != DT_F32 && dtype != DT_F16 && dtype != DT_BF16) return fail(ERR_BAD_ARG, "dtype must be MTQ_F32, MTQ_F16 or MTQ_BF16");
+    if (bits < 2 || bits > 8) return fail(ERR_BAD_ARG, "bits must be in 2..8");
+    if (N == 0 || K == 0) return fail(ERR_SHAPE, "N and K must be non-zero");
+    if (group_size == 0 || K % group_size) return fail(ERR_SHAPE, "group_size must be non-zero and divide K");
+    if ((uint64_t)N * bits % 32) return fail(ERR_SHAPE, "N*bits must be a multiple of 32");
+    if (M == 0) return ERR_OK;
+    if (!w || !scales || !biases || !x || !out) return fail(ERR_BAD_ARG, "null buffer");
+    void* sp = g.device >= 0 && g.device < kMaxDevices ? g_noalloc_ptr[g.device] : nullptr;
+    if (!sp) return fail(ERR_UNSUPPORTED, "mtq_qvm_noalloc: no built-in scratch on this device index");
+    const size_t need = qvm_scratch_bytes(bits, group_size, M, N, K);
+    if (need > kNoallocScratchBytes) {
+        char m[200];
+        snprintf(m, sizeof m, "mtq_qvm_noalloc: the partial rows need %zu bytes, the built-in scratch holds %zu; use mtq_qvm",
+                 need, kNoallocScratchBytes);
+        return fail(ERR_UNSUPPORTED, m);
+    }
+    QmvParams p;
+    p.dtype = dtype; p.bits = bits; p.group_size = group_size; p.w = w; p.scales = scales; p.biases = biases; p.x = x; p.out = out;
+    p.M = M; p.N = N; p.K = K;
+    // every partial row the reduction reads is written by the first kernel of this call: nothing to clear
+    return launch_qvm(p, sp, make_ctx());
 }
 
 int mtq_qmv_batched(int dtype, int bits, uint32_t group_size, int n_mats, const void* const* w,

@@ -51,6 +51,12 @@ def qvm(dtype, bits, group_size, w, scales, biases, x, out, M, N, K):
     _lib.check(lib.mtq_qvm(int(dtype), bits, group_size, _p(w), _p(scales), _p(biases), _p(x), _p(out), M, N, K))
 
 
+def qvm_noalloc(dtype, bits, group_size, w, scales, biases, x, out, M, N, K):
+    """qvm through the library's built-in 4 MiB scratch array: no device allocation in the call."""
+    lib = _ensure_init()
+    _lib.check(lib.mtq_qvm_noalloc(int(dtype), bits, group_size, _p(w), _p(scales), _p(biases), _p(x), _p(out), M, N, K))
+
+
 def qmv_batched(dtype, bits, group_size, ws, scales, biases, x, outs, Ns, K):
     """2..4 weight matrices (lists of buffers) against one activation row, one launch."""
     lib = _ensure_init()
