@@ -11,8 +11,18 @@ The timed region is K steps enqueued back to back through the C-ABI's dispatch
 chain (no host wait inside), bracketed by the host clock (`value`) and by one
 pair of HIP events recorded on the launch stream (`roofline`: average launch
 duration = event time / launches). A second, untimed-for-throughput pass
-attaches an event pair to every launch for the per-kernel distribution. The CPU baseline is the oracle restatement of the
-reference's CPU path timed on the host cores on a bounded sample.
+attaches an event pair to every launch for the per-kernel distribution. The CPU
+baseline is the oracle restatement of the reference's CPU path timed on the
+host cores on a bounded sample.
+
+The default run then times, in the same process, the two other figures the
+headline metric and its configurations name and reports them under
+"secondary": qmm at M = 512 (4-bit g64 bf16, N = K = 4096; bound: bf16 MFMA)
+and the Mixtral-style gather_qmv (8 experts of 14336 x 4096, 32 routed rows;
+bound: HBM on the bytes of the experts that are hit), each with its own
+roofline object. `value`, `ms_per_step` and `steps` describe the qmv region
+only. `--workload sweep` reports the 18 cells of the bit-width / group-size
+sweep (f16, 8192 x 8192, batch 1 and 4).
 
 Prints ONE JSON line on stdout.
 """
@@ -37,10 +47,14 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=8, help="distinct MLP weight sets streamed per step")
-    ap.add_argument("--workload", default="qmv", choices=["qmv", "qkv", "qmm", "gather", "gather_prefill", "quantize", "dequantize", "copy"],
-                    help="qmv is the headline; qmm / gather report the other configurations; "
+    ap.add_argument("--workload", default="qmv",
+                    choices=["qmv", "qkv", "qmm", "gather", "gather_prefill", "quantize", "dequantize", "copy", "sweep"],
+                    help="qmv is the headline (its line also carries qmm M=512 and the gather as secondary legs); "
+                         "qmm / gather report those configurations alone; sweep the bit-width / group-size cells; "
                          "copy runs only the known-size copy kernel (counter calibration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-secondary", action="store_true", help="qmv workload: skip the qmm M=512 and gather legs")
+    ap.add_argument("--m", type=int, default=512, help="qmm workload: activation rows")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--hot", action="store_true", help="re-use one weight set (cache-resident) instead of rotating")
     return ap.parse_args()
@@ -59,40 +73,271 @@ def traffic_from_profiles(tag: str):
     return None
 
 
-def cpu_baseline_qmv(seconds: float):
-    """Reference CPU path (qmm_oracle restated in C) on one layer's three matrices."""
-    import numpy as np
-    from oracle import oracle as o
-    from metaltile_amd import DType
-    from metaltile_amd.synth import make_case, qmv_bytes
-    o.build()
-    cores = min(16, os.cpu_count() or 1)
-    shapes = [(14336, 4096), (14336, 4096), (4096, 14336)]
-    cases = [make_case(7000 + i, DType.BF16, 4, 64, 1, n, k) for i, (n, k) in enumerate(shapes)]
-    nbytes = sum(qmv_bytes(n, k, 4, 64, 1, 2) for n, k in shapes)
+# ---------------------------------------------------------------------------
+# CPU baseline: the oracle restatement of the reference's CPU path
+# ---------------------------------------------------------------------------
+
+def _timed_loop(fn, seconds):
     reps, t0 = 0, time.perf_counter()
     while True:
-        for c in cases:
-            o.qmm(c.w, c.scales_f, c.biases_f, c.x_f, 1, c.N, c.K, 4, 64, threads=cores)
+        fn(reps)
         reps += 1
         el = time.perf_counter() - t0
         if el >= seconds:
-            break
-    # the same loop on one thread, as the reference's single-threaded setup() runs it
-    reps1, t1 = 0, time.perf_counter()
-    while True:
-        c = cases[reps1 % len(cases)]
+            return reps, el
+
+
+def cpu_baseline(seconds: float):
+    """Reference CPU path (qmm_oracle / gather oracle restated in C) on bounded samples of the three
+    decode workloads: the Llama MLP matrices (the headline), the f32 4096 x 4096 qmv in full, and
+    the 32 routed rows of the Mixtral-style gather."""
+    import numpy as np
+    from oracle import oracle as o
+    from metaltile_amd import DType
+    from metaltile_amd.synth import make_case, qmv_bytes, top2_routing
+    o.build()
+    host_threads = os.cpu_count() or 1
+    cores = min(16, host_threads)
+    shapes = [(14336, 4096), (14336, 4096), (4096, 14336)]
+    cases = [make_case(7000 + i, DType.BF16, 4, 64, 1, n, k) for i, (n, k) in enumerate(shapes)]
+    nbytes = sum(qmv_bytes(n, k, 4, 64, 1, 2) for n, k in shapes)
+
+    def layer(_):
+        for c in cases:
+            o.qmm(c.w, c.scales_f, c.biases_f, c.x_f, 1, c.N, c.K, 4, 64, threads=cores)
+    reps, el = _timed_loop(layer, seconds * 0.5)
+
+    # the same matrices on one thread, as the reference's single-threaded setup() runs them
+    def one_matrix(i):
+        c = cases[i % len(cases)]
         o.qmm(c.w, c.scales_f, c.biases_f, c.x_f, 1, c.N, c.K, 4, 64, threads=1)
-        reps1 += 1
-        el1 = time.perf_counter() - t1
-        if el1 >= seconds / 3:
-            break
+    reps1, el1 = _timed_loop(one_matrix, seconds * 0.2)
     one = qmv_bytes(14336, 4096, 4, 64, 1, 2) * reps1 / el1 / 1e9
-    return {"value": round(nbytes * reps / el / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+
+    # f32 qmv 4096 x 4096: the reference's own CPU-runnable configuration, whole matrix every pass
+    c0 = make_case(7100, DType.F32, 4, 64, 1, 4096, 4096)
+    b0 = qmv_bytes(4096, 4096, 4, 64, 1, 4)
+    r0, e0 = _timed_loop(lambda _: o.qmm(c0.w, c0.scales_f, c0.biases_f, c0.x_f, 1, 4096, 4096, 4, 64, threads=1), seconds * 0.1)
+    r0m, e0m = _timed_loop(lambda _: o.qmm(c0.w, c0.scales_f, c0.biases_f, c0.x_f, 1, 4096, 4096, 4, 64, threads=cores), seconds * 0.05)
+
+    # gather: 2 experts of 14336 x 4096 (a quarter of the 8), the 32 routed rows dealt to them 16 / 16;
+    # bytes counted as the bench's gather leg counts them (unique-expert bytes + rows in and out)
+    E, N, K, G = 2, 14336, 4096, 64
+    cg = make_case(7200, DType.BF16, 4, G, 16, N, K, E=E)
+    tok, _, offsets = top2_routing(7201, 16, E)
+    xr = cg.x_f.reshape(16, K)[tok].reshape(-1)
+    T = int(tok.size)
+    bg = E * (N * K // 2 + 2 * N * (K // G) * 2) + 16 * K * 2 + T * N * 2 + 4 * (E + 1)
+    rg, eg = _timed_loop(lambda _: o.gather_qmm(xr, cg.w, cg.scales_f, cg.biases_f, T, K, N, E, 4, G,
+                                                expert_offsets=offsets, threads=cores), seconds * 0.15)
+    return {"value": round(nbytes * reps / el / 1e9, 3), "unit": "GB/s", "cores": cores, "host_hardware_threads": host_threads,
+            "kind": "port",
             "sample": f"{reps} passes over one layer (gate, up 14336x4096; down 4096x14336), "
                       f"f32-sequential oracle, {el:.1f} s, row-parallel over {cores} threads; "
                       f"one thread: {one:.3f} GB/s over {reps1} matrices in {el1:.1f} s",
-            "value_one_thread": round(one, 3)}
+            "value_one_thread": round(one, 3),
+            "also": {
+                "qmv_f32_4096x4096": {"value": round(b0 * r0m / e0m / 1e9, 3), "value_one_thread": round(b0 * r0 / e0 / 1e9, 3),
+                                      "unit": "GB/s", "cores": cores,
+                                      "sample": f"whole matrix, {r0} passes on one thread in {e0:.1f} s, {r0m} on {cores} threads in {e0m:.1f} s"},
+                "gather_qmv": {"value": round(bg * rg / eg / 1e9, 3), "unit": "GB/s", "cores": cores,
+                               "sample": f"2 of the 8 experts (14336x4096 each) with {T} routed rows (the full configuration has 32 "
+                                         f"rows on 8 experts: 4 rows per expert against 16 here), gather oracle, {rg} passes in {eg:.1f} s; "
+                                         "bytes = unique-expert bytes + rows, so the CPU's figure falls with the rows per expert"},
+            }}
+
+
+# ---------------------------------------------------------------------------
+# GPU legs
+# ---------------------------------------------------------------------------
+
+def leg_qmv(a, runner, info):
+    import numpy as np
+    import metaltile_amd as m
+    from metaltile_amd import DType, GpuBuffer
+    from metaltile_amd.synth import make_case, qmv_bytes
+    dt = DType.BF16
+    shapes = [(14336, 4096), (14336, 4096), (4096, 14336)]
+    layers = 1 if a.hot else a.layers
+    specs, keep, step_bytes = [], [], 0
+    for layer in range(layers):
+        for j, (n, k) in enumerate(shapes):
+            c = make_case(5000 + layer * 3 + j, dt, 4, 64, 1, n, k)
+            bufs = {"w": GpuBuffer.from_bytes(c.w.tobytes()), "scales": GpuBuffer.from_bytes(c.scales_bytes),
+                    "biases": GpuBuffer.from_bytes(c.biases_bytes), "x": GpuBuffer.from_bytes(c.x_bytes),
+                    "out": GpuBuffer(n * 2)}
+            keep.append(bufs)
+            specs.append(("mt_qmv", dt, bufs, {"k": k, "gs_per_row": k // 64}))
+            step_bytes += qmv_bytes(n, k, 4, 64, 1, 2)
+    launch_bytes = qmv_bytes(14336, 4096, 4, 64, 1, 2)   # == the transposed shape's figure
+    if a.hot:
+        specs = specs * a.layers
+        step_bytes *= a.layers
+    runner.flush_slc()
+    runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
+    # Timed region: K steps enqueued back to back with no host wait and no
+    # per-launch instrumentation; one pair of HIP events on the stream
+    # brackets it (chain_us), the host clock brackets it too (wall_us).
+    _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+    n_per_step = len(specs)
+    kern_avg = chain_us / (a.steps * n_per_step)   # average launch duration over the timed region
+    # Second pass, same launches: each carries its own event pair, giving the
+    # distribution of the kernels' own durations (the pairs cost ~15 us of
+    # host time per launch, so this pass is not the one whose wall clock counts).
+    per, _, _ = runner.dispatch_chain(specs, repeat=min(a.steps, 20), per_kernel=True)
+    per = np.array(per)
+    st = m.BenchStats.from_samples(per.tolist())
+    gbs = step_bytes * a.steps / wall_us / 1e3
+    by_shape, frac_by_shape = {}, {}
+    for j, name in enumerate(["gate_14336x4096", "up_14336x4096", "down_4096x14336"]):
+        sel = per.reshape(-1, n_per_step)[:, j::3]
+        by_shape[name] = round(float(sel.mean()), 3)
+        frac_by_shape[name] = round(launch_bytes / float(sel.mean()) / 1e3 / HBM_PEAK_GBS, 4)
+    achieved = launch_bytes / kern_avg / 1e3
+    for bufs in keep:
+        for b in bufs.values():
+            b.free()
+    return {
+        "metric": "qmv GB/s & % HBM peak (4-bit g64, 4096x14336 bf16); qmm TFLOP/s M=512", "value": round(gbs, 1), "unit": "GB/s",
+        "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
+        "config": {"workload": "qmv 4-bit g64 bf16, Llama-3-8B MLP decode (gate/up 14336x4096 + down 4096x14336), batch 1",
+                   "layers_per_step": a.layers, "launches_per_step": n_per_step, "bytes_per_step": step_bytes,
+                   "weights": "hot (one set re-used)" if a.hot else "cold (rotating sets, > last-level cache)",
+                   "device": info["name"] or info["arch"], "arch": info["arch"], "compute_units": info["compute_units"]},
+        "pct_hbm_peak_whole_job": round(100.0 * gbs / HBM_PEAK_GBS, 2),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_from_profiles("qmv_bf16_b4_llama_mlp"),
+                     "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, 1 row>", "bytes_per_launch": launch_bytes,
+                     "avg_launch_us_timed_region": round(kern_avg, 3),
+                     "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(st.min_us, 3),
+                                           "median_us": round(st.median_us, 3), "p95_us": round(st.p95_us, 3),
+                                           "avg_us_by_shape": by_shape, "frac_by_shape": frac_by_shape}},
+    }
+
+
+def leg_qmm(a, runner, info, M=512):
+    import numpy as np
+    from metaltile_amd import DType, GpuBuffer
+    from metaltile_amd.synth import make_case
+    dt = DType.BF16
+    N, K = 4096, 4096
+    sets = 1 if a.hot else 16
+    specs, keep = [], []
+    for i in range(sets):
+        c = make_case(6000 + i, dt, 4, 64, M, N, K)
+        bufs = {"w": GpuBuffer.from_bytes(c.w.tobytes()), "scales": GpuBuffer.from_bytes(c.scales_bytes),
+                "biases": GpuBuffer.from_bytes(c.biases_bytes), "x": GpuBuffer.from_bytes(c.x_bytes),
+                "out": GpuBuffer(M * N * 2)}
+        keep.append(bufs)
+        specs.append(("mt_qmm_mma", dt, bufs, {"k": K, "n": N, "gs_per_row": K // 64}))
+    flops = 2.0 * M * N * K
+    runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
+    _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+    kern_avg = chain_us / (a.steps * len(specs))
+    per, _, _ = runner.dispatch_chain(specs, repeat=min(a.steps, 20), per_kernel=True)
+    per = np.array(per)
+    tf = flops * len(specs) * a.steps / wall_us / 1e6
+    ach = flops / kern_avg / 1e6
+    for bufs in keep:
+        for b in bufs.values():
+            b.free()
+    return {
+        "metric": f"qmm TFLOP/s M={M} (4-bit g64 bf16, N=K=4096)", "value": round(tf, 1), "unit": "TFLOP/s",
+        "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
+        "config": {"workload": f"qmm 4-bit g64 bf16 prefill, M={M} N=4096 K=4096", "launches_per_step": len(specs),
+                   "device": info["name"] or info["arch"]},
+        "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": traffic_from_profiles("qmm_bf16_b4_m512") if M == 512 else None,
+                     "flop_per_launch": flops, "avg_launch_us_timed_region": round(kern_avg, 3),
+                     "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(float(per.min()), 3)}},
+    }
+
+
+def leg_gather(a, runner, info):
+    import numpy as np
+    import metaltile_amd as m
+    from metaltile_amd import DType, GpuBuffer
+    from metaltile_amd.synth import make_case, top2_routing
+    dt = DType.BF16
+    E, N, K, G, tokens = 8, 14336, 4096, 64, 16
+    c = make_case(8000, dt, 4, G, tokens, N, K, E=E)
+    tok, exp_id, offsets = top2_routing(8001, tokens, E)
+    T = int(tok.size)
+    x_rows = c.x_f.reshape(tokens, K)[tok].reshape(-1)
+    consts = {"k_in": K, "m_out": N, "n_experts": E, "group_size": G}
+    U = int(np.unique(exp_id).size)
+    nbytes = U * (N * K // 2 + 2 * N * (K // G) * 2) + tokens * K * 2 + T * N * 2 + 4 * (E + 1)
+    # four copies of the experts' weights (1.06 GB), visited in turn: every launch reads cold weights
+    specs, keep = [], []
+    for i in range(4):
+        bufs = {"x": GpuBuffer.from_bytes(m.pack_f32(x_rows, dt)), "weight_packed": GpuBuffer.from_bytes(c.w.tobytes()),
+                "scales": GpuBuffer.from_bytes(c.scales_bytes), "biases": GpuBuffer.from_bytes(c.biases_bytes),
+                "expert_offsets": GpuBuffer.from_bytes(offsets.astype("<u4").tobytes()), "out": GpuBuffer(T * N * 2)}
+        keep.append(bufs)
+        specs.append(("mt_moe_gather_qmm_int4", dt, bufs, consts))
+    runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
+    _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+    kern_avg = chain_us / (a.steps * len(specs))
+    per, _, _ = runner.dispatch_chain(specs, repeat=min(a.steps, 20), per_kernel=True)
+    per = np.array(per)
+    for bufs in keep:
+        for b in bufs.values():
+            b.free()
+    return {
+        "metric": "gather_qmv GB/s on unique-expert bytes (8 experts x 14336x4096 4-bit g64 bf16, 16 tokens top-2)",
+        "value": round(nbytes * len(specs) * a.steps / wall_us / 1e3, 1), "unit": "GB/s",
+        "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
+        "config": {"workload": "gather_qmv E=8 N=14336 K=4096, 32 (token,expert) rows", "experts_hit": U,
+                   "launches_per_step": len(specs), "bytes_per_step": nbytes * len(specs),
+                   "weights": "cold (4 rotating copies of the experts)", "device": info["name"] or info["arch"]},
+        "roofline": {"bound": "hbm", "achieved": round(nbytes / kern_avg / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(nbytes / kern_avg / 1e3 / HBM_PEAK_GBS, 4),
+                     "traffic": traffic_from_profiles("gather_bf16_b4_e8"), "bytes_per_launch": nbytes,
+                     "avg_launch_us_timed_region": round(kern_avg, 3),
+                     "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(float(per.min()), 3)}},
+    }
+
+
+def leg_sweep(a, runner, info):
+    """Bit widths {2, 4, 8} x group sizes {32, 64, 128} x batch {1, 4}, W[8192, 8192], f16, through the typed
+    entry point mtq_qmv: per cell the kernels' own durations (GPU timestamps attached to each launch) over
+    rotating weight copies (cold), GB/s on the algorithmic bytes and the fraction of the HBM peak."""
+    import numpy as np
+    from metaltile_amd import DType, GpuBuffer, ops
+    from metaltile_amd.synth import make_case, qmv_bytes
+    dt = DType.F16
+    N = K = 8192
+    cells, worst = {}, None
+    for bits in (2, 4, 8):
+        for G in (32, 64, 128):
+            per_copy = N * K * bits // 8 + 2 * N * (K // G) * 2
+            sets = max(2, -(-(640 << 20) // per_copy))   # more than twice the 256 MB last-level cache in rotation
+            base = make_case(9000 + bits * 10 + G, dt, bits, G, 4, N, K, bias_rule="midpoint")
+            wb, sb, bb = base.w.tobytes(), base.scales_bytes, base.biases_bytes
+            xb, ob = GpuBuffer.from_bytes(base.x_bytes), GpuBuffer(4 * N * 2)
+            copies = [(GpuBuffer.from_bytes(wb), GpuBuffer.from_bytes(sb), GpuBuffer.from_bytes(bb)) for _ in range(sets)]
+            for M in (1, 4):
+                nb = qmv_bytes(N, K, bits, G, M, 2)
+                n_samples = max(sets, min(a.steps, 60))
+                us = []
+                for i in range(a.warmup % 4 + sets + n_samples):
+                    w, s, b = copies[i % sets]
+                    t = ops.timed(ops.qmv, dt, bits, G, w, s, b, xb, ob, M, N, K)
+                    if i >= a.warmup % 4 + sets:
+                        us.append(t)
+                avg, med = float(np.mean(us)), float(np.median(us))
+                frac = nb / avg / 1e3 / HBM_PEAK_GBS
+                cells[f"b{bits}_g{G}_m{M}"] = {"avg_us": round(avg, 2), "median_us": round(med, 2), "GBps": round(nb / avg / 1e3, 1),
+                                               "frac": round(frac, 4), "bytes": nb}
+                if worst is None or frac < worst[1]:
+                    worst = (f"b{bits}_g{G}_m{M}", frac)
+            for c in copies:
+                for buf in c:
+                    buf.free()
+            xb.free()
+            ob.free()
+    return cells, worst
 
 
 def main():
@@ -105,7 +350,7 @@ def main():
     import numpy as np
     import metaltile_amd as m
     from metaltile_amd import DType, GpuBuffer
-    from metaltile_amd.synth import make_case, qmv_bytes, top2_routing
+    from metaltile_amd.synth import make_case, qmv_bytes
 
     runner = m.GpuRunner(0)
     info = runner.device_info()
@@ -123,60 +368,38 @@ def main():
         return
 
     if a.workload == "qmv":
-        shapes = [(14336, 4096), (14336, 4096), (4096, 14336)]
-        layers = 1 if a.hot else a.layers
-        specs, keep, step_bytes = [], [], 0
-        for layer in range(layers):
-            for j, (n, k) in enumerate(shapes):
-                c = make_case(5000 + layer * 3 + j, dt, 4, 64, 1, n, k)
-                bufs = {"w": GpuBuffer.from_bytes(c.w.tobytes()), "scales": GpuBuffer.from_bytes(c.scales_bytes),
-                        "biases": GpuBuffer.from_bytes(c.biases_bytes), "x": GpuBuffer.from_bytes(c.x_bytes),
-                        "out": GpuBuffer(n * 2)}
-                keep.append(bufs)
-                specs.append(("mt_qmv", dt, bufs, {"k": k, "gs_per_row": k // 64}))
-                step_bytes += qmv_bytes(n, k, 4, 64, 1, 2)
-        launch_bytes = qmv_bytes(14336, 4096, 4, 64, 1, 2)   # == the transposed shape's figure
-        if a.hot:
-            specs = specs * a.layers
-            step_bytes *= a.layers
-        runner.flush_slc()
-        runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
-        # Timed region: K steps enqueued back to back with no host wait and no
-        # per-launch instrumentation; one pair of HIP events on the stream
-        # brackets it (chain_us), the host clock brackets it too (wall_us).
-        _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
-        n_per_step = len(specs)
-        kern_avg = chain_us / (a.steps * n_per_step)   # average launch duration over the timed region
-        # Second pass, same launches: each carries its own event pair, giving the
-        # distribution of the kernels' own durations (the pairs cost ~15 us of
-        # host time per launch, so this pass is not the one whose wall clock counts).
-        per, _, _ = runner.dispatch_chain(specs, repeat=min(a.steps, 20), per_kernel=True)
-        per = np.array(per)
-        st = m.BenchStats.from_samples(per.tolist())
-        gbs = step_bytes * a.steps / wall_us / 1e3
-        by_shape = {}
-        for j, name in enumerate(["gate_14336x4096", "up_14336x4096", "down_4096x14336"]):
-            sel = per.reshape(-1, n_per_step)[:, j::3]
-            by_shape[name] = round(float(sel.mean()), 3)
-        achieved = launch_bytes / kern_avg / 1e3
-        out.update({
-            "metric": "qmv GB/s & % HBM peak (4-bit g64, 4096x14336 bf16)", "value": round(gbs, 1), "unit": "GB/s",
-            "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
-            "config": {"workload": "qmv 4-bit g64 bf16, Llama-3-8B MLP decode (gate/up 14336x4096 + down 4096x14336), batch 1",
-                       "layers_per_step": a.layers, "launches_per_step": n_per_step, "bytes_per_step": step_bytes,
-                       "weights": "hot (one set re-used)" if a.hot else "cold (rotating sets, > last-level cache)",
-                       "device": info["name"] or info["arch"], "arch": info["arch"], "compute_units": info["compute_units"]},
-            "pct_hbm_peak_whole_job": round(100.0 * gbs / HBM_PEAK_GBS, 2),
-            "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_from_profiles("qmv_bf16_b4_llama_mlp"),
-                         "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, 1 row>", "bytes_per_launch": launch_bytes,
-                         "avg_launch_us_timed_region": round(kern_avg, 3),
-                         "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(st.min_us, 3),
-                                               "median_us": round(st.median_us, 3), "p95_us": round(st.p95_us, 3),
-                                               "avg_us_by_shape": by_shape}},
-        })
+        out.update(leg_qmv(a, runner, info))
+        if not a.no_secondary:
+            sec = {}
+            for key, leg in (("qmm_m512", lambda: leg_qmm(a, runner, info, 512)), ("gather_c4", lambda: leg_gather(a, runner, info))):
+                r = leg()
+                sec[key] = {"metric": r["metric"], "value": r["value"], "unit": r["unit"],
+                            "ms_per_launch": round(r["roofline"]["avg_launch_us_timed_region"] / 1e3, 6),
+                            "workload": r["config"]["workload"], "roofline": r["roofline"]}
+            out["secondary"] = sec
         if not a.no_cpu:
-            out["cpu_baseline"] = cpu_baseline_qmv(a.cpu_seconds)
+            out["cpu_baseline"] = cpu_baseline(a.cpu_seconds)
+        print(json.dumps(out))
+        return
+
+    if a.workload == "qmm":
+        out.update(leg_qmm(a, runner, info, a.m))
+        print(json.dumps(out))
+        return
+
+    if a.workload == "gather":
+        out.update(leg_gather(a, runner, info))
+        print(json.dumps(out))
+        return
+
+    if a.workload == "sweep":
+        cells, worst = leg_sweep(a, runner, info)
+        c = cells["b4_g64_m1"]
+        out.update({"metric": "qmv GB/s per cell, bits {2,4,8} x group {32,64,128} x batch {1,4}, f16, 8192x8192",
+                    "value": c["GBps"], "unit": "GB/s", "ms_per_step": round(c["avg_us"] / 1e3, 6), "dtype": "f16",
+                    "config": {"workload": "qmv sweep W[8192,8192] f16 (value = the 4-bit g64 batch-1 cell)", "device": info["name"] or info["arch"]},
+                    "roofline": {"bound": "hbm", "achieved": c["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": c["frac"], "traffic": None},
+                    "cells": cells, "worst_cell": {"cell": worst[0], "frac": round(worst[1], 4)}})
         print(json.dumps(out))
         return
 
@@ -214,75 +437,6 @@ def main():
                          "traffic": traffic_from_profiles("qkv_fused_bf16_b4_llama_attn"),
                          "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, 1 row>, 3 matrices per launch",
                          "avg_launch_us_timed_region": round(kern_avg, 3)},
-        })
-        print(json.dumps(out))
-        return
-
-    if a.workload == "qmm":
-        M, N, K = 512, 4096, 4096
-        sets = 1 if a.hot else 16
-        specs, keep = [], []
-        for i in range(sets):
-            c = make_case(6000 + i, dt, 4, 64, M, N, K)
-            bufs = {"w": GpuBuffer.from_bytes(c.w.tobytes()), "scales": GpuBuffer.from_bytes(c.scales_bytes),
-                    "biases": GpuBuffer.from_bytes(c.biases_bytes), "x": GpuBuffer.from_bytes(c.x_bytes),
-                    "out": GpuBuffer(M * N * 2)}
-            keep.append(bufs)
-            specs.append(("mt_qmm_mma", dt, bufs, {"k": K, "n": N, "gs_per_row": K // 64}))
-        flops = 2.0 * M * N * K
-        runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
-        _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
-        kern_avg = chain_us / (a.steps * len(specs))
-        per, _, _ = runner.dispatch_chain(specs, repeat=min(a.steps, 20), per_kernel=True)
-        per = np.array(per)
-        tf = flops * len(specs) * a.steps / wall_us / 1e6
-        ach = flops / kern_avg / 1e6
-        out.update({
-            "metric": "qmm TFLOP/s M=512 (4-bit g64 bf16, N=K=4096)", "value": round(tf, 1), "unit": "TFLOP/s",
-            "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
-            "config": {"workload": "qmm 4-bit g64 bf16 prefill, M=512 N=4096 K=4096", "launches_per_step": len(specs),
-                       "device": info["name"] or info["arch"]},
-            "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic_from_profiles("qmm_bf16_b4_m512"),
-                         "avg_launch_us_timed_region": round(kern_avg, 3),
-                         "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(float(per.min()), 3)}},
-        })
-        print(json.dumps(out))
-        return
-
-    if a.workload == "gather":
-        E, N, K, G, tokens = 8, 14336, 4096, 64, 16
-        c = make_case(8000, dt, 4, G, tokens, N, K, E=E)
-        tok, exp_id, offsets = top2_routing(8001, tokens, E)
-        T = int(tok.size)
-        x_rows = c.x_f.reshape(tokens, K)[tok].reshape(-1)
-        consts = {"k_in": K, "m_out": N, "n_experts": E, "group_size": G}
-        U = int(np.unique(exp_id).size)
-        nbytes = U * (N * K // 2 + 2 * N * (K // G) * 2) + tokens * K * 2 + T * N * 2 + 4 * (E + 1)
-        # four copies of the experts' weights (1.06 GB), visited in turn: every launch reads cold weights
-        specs, keep = [], []
-        for i in range(4):
-            bufs = {"x": GpuBuffer.from_bytes(m.pack_f32(x_rows, dt)), "weight_packed": GpuBuffer.from_bytes(c.w.tobytes()),
-                    "scales": GpuBuffer.from_bytes(c.scales_bytes), "biases": GpuBuffer.from_bytes(c.biases_bytes),
-                    "expert_offsets": GpuBuffer.from_bytes(offsets.astype("<u4").tobytes()), "out": GpuBuffer(T * N * 2)}
-            keep.append(bufs)
-            specs.append(("mt_moe_gather_qmm_int4", dt, bufs, consts))
-        runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
-        _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
-        kern_avg = chain_us / (a.steps * len(specs))
-        per, _, _ = runner.dispatch_chain(specs, repeat=min(a.steps, 20), per_kernel=True)
-        per = np.array(per)
-        out.update({
-            "metric": "gather_qmv GB/s on unique-expert bytes (8 experts x 14336x4096 4-bit g64 bf16, 16 tokens top-2)",
-            "value": round(nbytes * len(specs) * a.steps / wall_us / 1e3, 1), "unit": "GB/s",
-            "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
-            "config": {"workload": "gather_qmv E=8 N=14336 K=4096, 32 (token,expert) rows", "experts_hit": U,
-                       "launches_per_step": len(specs), "bytes_per_step": nbytes * len(specs),
-                       "weights": "cold (4 rotating copies of the experts)", "device": info["name"] or info["arch"]},
-            "roofline": {"bound": "hbm", "achieved": round(nbytes / kern_avg / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(nbytes / kern_avg / 1e3 / HBM_PEAK_GBS, 4),
-                         "traffic": traffic_from_profiles("gather_bf16_b4_e8"), "avg_launch_us_timed_region": round(kern_avg, 3),
-                         "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(float(per.min()), 3)}},
         })
         print(json.dumps(out))
         return

@@ -141,7 +141,10 @@ MTQ_API int mtq_qmm(int dtype, int bits, uint32_t group_size, const void *w, con
  * first, as in the reference's MMA gathers (moe.rs:2256); MTQ_F32 rows always run grouped, in
  * 32-row tiles on the f32 matrix-core kernel (f32 rounding only). The grouping tables live in a
  * library-owned buffer (allocated on first use). Option "gather.grouped": 0 this rule,
- * 1 never grouped, 2 always grouped. */
+ * 1 never grouped, 2 always grouped. Through mtq_dispatch the reference's kernel name decides instead:
+ * mt_moe_gather_qmm_int4{,_m8,_m16,_m32} and mt_moe_gather_qmm_b* multiply by the exact s*q + b in the
+ * reference and stay on the GEMV kernels here at any number of rows per expert (option
+ * "gather.names_exact"); mt_moe_gather_qmm_mma_* round w_hat to T in the reference and follow the rule above. */
 MTQ_API int mtq_gather_qmv_csr(int dtype, int bits, uint32_t group_size, const void *x,
                                const void *w, const void *scales, const void *biases,
                                const uint32_t *expert_offsets, void *out, uint32_t T, uint32_t N,
@@ -346,8 +349,6 @@ MTQ_API int mtq_flush_cache(void);
  *   "qmv.stream_depth"     streaming kernel: 0 = choose per shape, or 4 / 8 loads in flight per thread
  *   "qmv.stream_batches"   streaming kernel: 0 = choose per shape, or 1..16 batches per thread
  *   "qmv.mfma"             matrix-core GEMV kernel: 0 = choose per shape, 1 = never, 2 = wherever it applies
- *   "qmv.mfma_delay"       matrix-core GEMV kernel: pause (x 512 clocks) before the first weight loads, 0..64;
- *                          a measurement aid
  *   "qmv.mfma_kp" / "qmv.mfma_rbw" / "qmv.mfma_nrb" / "qmv.mfma_sets"
  *                          matrix-core GEMV geometry: K parts per row, row blocks side by side and one
  *                          after the other per workgroup, 4-row activation sets per pass; 0 = choose
@@ -362,6 +363,9 @@ MTQ_API int mtq_flush_cache(void);
  *                          tiles in the library-owned buffer, added in split order by a second kernel)
  *   "qmm.f32_tiles"        f32 batches on the f32 matrix-core kernel: 0 = choose by rows, 1 = never, 2 = always
  *   "gather.grouped"       gather_qmv with many rows per expert on the tile kernel: 0 = choose, 1 = never, 2 = always
+ *   "gather.names_exact"   the exact-dequant gather names of mtq_dispatch (mt_moe_gather_qmm_int4, _m8, _m16, _m32, _b3 ..
+ *                          _b8): 0 = always on the GEMV kernels (exact s*q + b, as those reference kernels compute), 1 = grouped
+ *                          on the tile kernel above 8 rows per expert like the typed entry points (w_hat rounded to T first)
  *   "qvm.wgs"              qvm: workgroups to aim for when K is sliced, 0 = choose
  *   "moe.sort"             expert sort: 0 = choose by size, 1 = always the bitonic network
  *   "moe_down.rows"        fused MoE down projection: output rows per workgroup, 0 = choose

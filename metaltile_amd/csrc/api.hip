@@ -319,7 +319,7 @@ static int op_qmv_batched(int dtype, int bits, uint32_t G, int n, const void* co
 
 static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, const void* w,
                      const void* s, const void* b, const uint32_t* route, void* out, uint32_t T,
-                     uint32_t N, uint32_t K, uint32_t E, const LaunchCtx& lc) {
+                     uint32_t N, uint32_t K, uint32_t E, const LaunchCtx& lc, bool exact_only = false) {
     int rc = check_common(dtype, bits, G, N, K);
     if (rc) return rc;
     if (E == 0) return fail(ERR_SHAPE, "n_experts must be non-zero");
@@ -351,7 +351,10 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
         rc = launch_qmm_f32_grouped(q, route, ids, T, E, g.scratch_buf, lc);
         if (rc != ERR_UNSUPPORTED) return rc;
     }
-    if (dtype != DT_F32 && mode != GATHER_SINGLE && gopt != 1 && (gopt == 2 || (uint64_t)T > (uint64_t)8 * (E < T ? E : T))) {
+    // exact_only: the caller named a reference kernel that multiplies by the exact f32 s*q + b
+    // (mt_moe_gather_qmm_int4* / _b*, crates/metaltile-std/src/ffai/moe.rs:358-433); the tile kernel rounds
+    // that value to the element type first, so such a name stays on the GEMV kernels at any routing density.
+    if (dtype != DT_F32 && mode != GATHER_SINGLE && gopt != 1 && (gopt == 2 || (!exact_only && (uint64_t)T > (uint64_t)8 * (E < T ? E : T)))) {
         QmmParams q;
         q.dtype = dtype; q.bits = bits; q.group_size = G;
         q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
@@ -569,7 +572,8 @@ static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, in
             MTQ_NEED(bufs[4], "expert_offsets", (uint64_t)(E + 1) * 4);
             MTQ_NEED(bufs[5], "out", (uint64_t)T * N * sz);
             return op_gather(GATHER_CSR, dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr,
-                             bufs[3].ptr, (const uint32_t*)bufs[4].ptr, bufs[5].ptr, T, N, K, E, lc);
+                             bufs[3].ptr, (const uint32_t*)bufs[4].ptr, bufs[5].ptr, T, N, K, E, lc,
+                             options().gather_names_exact == 0);
         }
         case F_GIDX: {
             uint32_t T = consts[0], N = consts[1], K = consts[2], G = consts[3];
@@ -1234,11 +1238,6 @@ int mtq_set_option(const char* name, int value) {
         options().qmv_mfma_sets = value;
         return MTQ_OK;
     }
-    if (!strcmp(name, "qmv.mfma_delay")) {
-        if (value < 0 || value > 64) return fail(ERR_BAD_ARG, "qmv.mfma_delay must be in 0..64");
-        options().qmv_mfma_delay = value;
-        return MTQ_OK;
-    }
     if (!strcmp(name, "qmv.mfma_kp") || !strcmp(name, "qmv.mfma_rbw") || !strcmp(name, "qmv.mfma_nrb")) {
         if (value < 0 || value > 256) return fail(ERR_BAD_ARG, "qmv.mfma_* must be in 0..256");
         if (name[9] == 'k') options().qmv_mfma_kp = value;
@@ -1264,6 +1263,11 @@ int mtq_set_option(const char* name, int value) {
     if (!strcmp(name, "gather.grouped")) {
         if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "gather.grouped must be 0 (choose), 1 (never) or 2 (always)");
         options().gather_grouped = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "gather.names_exact")) {
+        if (value < 0 || value > 1) return fail(ERR_BAD_ARG, "gather.names_exact must be 0 (exact-dequant names stay exact) or 1 (they may run grouped)");
+        options().gather_names_exact = value;
         return MTQ_OK;
     }
     if (!strcmp(name, "qmm.ksplit")) {

@@ -93,6 +93,7 @@ struct Options {
     int qmm_kgroups = 0;          // direct qmm: K-groups per workgroup (0 = choose; 1, 2, 4)
     int qmm_by_m = 0;             // direct qmm: 1 = an XCD keeps its M-tiles' activations and streams all weights
     int gather_grouped = 0;       // expert-routed rows on the tile kernel: 0 = choose by rows per expert, 1 = never, 2 = always
+    int gather_names_exact = 0;   // name-keyed exact-dequant gathers (mt_moe_gather_qmm_int4*, _b*): 0 = never on the rounding tile kernel, 1 = by rows per expert
     int qmm_ksplit = 0;           // direct qmm: 0 = choose, 1 = never split K, n = n splits
     int qmm_f32_tiles = 0;        // f32 batches on the f32 matrix cores: 0 = choose by rows, 1 = never, 2 = always
     int qmm_tile_rows = 0;        // direct qmm: activation rows per tile (0 = choose; 32, 64, 128)
@@ -101,7 +102,6 @@ struct Options {
     int qmv_mfma_rbw = 0;         // matrix-core qmv: row blocks walked in parallel per workgroup
     int qmv_mfma_nrb = 0;         // matrix-core qmv: row blocks per wave
     int qmv_mfma_sets = 0;        // matrix-core gather: 4-row MFMA sets per pass (0 = choose; 1, 2, 4)
-    int qmv_mfma_delay = 0;       // matrix-core qmv: pause (x512 clocks) before the first weight loads
 };
 Options& options();
 

@@ -232,7 +232,6 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     a.gpw = gpw;
     a.log2g = ilog2(G);
     a.list_cap = list_cap;
-    a.delay = (uint32_t)opt.qmv_mfma_delay;
     QmvMGeom g;
     g.mp = mp;
     g.s = s;

@@ -75,7 +75,6 @@ struct QmvMArgs {
     uint32_t gpr, log2g;
     uint32_t gpw;       // (scale, bias) pairs per row that a wave keeps in LDS: the groups of its K part, whole 4-vectors, <= 64
     uint32_t list_cap;  // capacity of the row list (indices mode)
-    uint32_t delay;     // units of 512 clocks between the small loads and the first weight loads
 };
 
 struct QmvMGeom {
@@ -390,7 +389,6 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         sbw_load(0, sb_now, pzero);
         if constexpr (REFILL) sbw_load(1, sb_next, pzero);
         MTQ_MFMA_KEEP_ORDER();
-        for (uint32_t i = 0; i < a.delay; i++) __builtin_amdgcn_s_sleep(8);
         MTQ_MFMA_KEEP_ORDER();
         uint32_t ring[D][NWD];
 #pragma unroll

@@ -77,13 +77,39 @@ def test_config3_qmm_bf16(oracle, M):
     3.4e-2 on this metric relative to exact dequantisation; the GPU is also
     held to 5e-2 against the exact oracle, the reference's own bf16 bound,
     crates/metaltile-std/tests/qmm_gpu_correctness.rs:2085-2106.)
-    M=2048 is covered by the property test; its oracle takes too long here."""
+    M=2048 has a test of its own below (32 sampled rows: the oracle works row by row)."""
     case = make_case(3000 + M, DType.BF16, 4, 64, M, 4096, 4096)
     got, _ = _check(case, oracle, 2e-2, entry=ops.qmm, mma=True)
     exact = oracle.qmm_f64(case.w, case.scales_f, case.biases_f, case.x_f, M, 4096, 4096, 4, 64, threads=8)
     dev = rel_err(got, exact)
     print(f"deviation from exact dequantisation: {dev:.3e}")
     assert dev <= 1e-1
+
+
+def test_config3_qmm_bf16_m2048_sampled_rows(oracle):
+    """The M = 2048 point of the same configuration. An output row depends on its own activation row only, so 32
+    rows drawn from the 2048 (first and last among them) are checked against the oracle run on those rows alone,
+    at the cost of M = 32: 2e-2 against the mma semantics, 1e-1 against exact dequantisation; every other row must
+    at least be finite and non-trivial."""
+    M, N, K = 2048, 4096, 4096
+    case = make_case(3000 + M, DType.BF16, 4, 64, M, N, K)
+    w, s, b, x = (GpuBuffer.from_bytes(case.w.tobytes()), GpuBuffer.from_bytes(case.scales_bytes),
+                  GpuBuffer.from_bytes(case.biases_bytes), GpuBuffer.from_bytes(case.x_bytes))
+    out = GpuBuffer.from_bytes(b"\xff" * (M * N * 2))
+    ops.qmm(DType.BF16, 4, 64, w, s, b, x, out, M, N, K)
+    got = unpack_f32(out.read_bytes(), DType.BF16).reshape(M, N)
+    for buf in (w, s, b, x, out):
+        buf.free()
+    assert np.isfinite(got).all() and np.all(np.abs(got).max(axis=1) > 0)
+    rng = np.random.default_rng(3)
+    rows = np.unique(np.concatenate([[0, M - 1, 127, 128, 1023, 1024], rng.choice(M, size=26, replace=False)]))
+    xs = np.ascontiguousarray(case.x_f.reshape(M, K)[rows]).reshape(-1)
+    mma = oracle.qmm_mma(case.w, case.scales_f, case.biases_f, xs, rows.size, N, K, 4, 64, 2, threads=8)
+    exact = oracle.qmm_f64(case.w, case.scales_f, case.biases_f, xs, rows.size, N, K, 4, 64, threads=8)
+    e_mma = rel_err(got[rows], oracle.round_through(mma.astype(np.float32), 2))
+    e_exact = rel_err(got[rows], exact)
+    print(f"M=2048, {rows.size} sampled rows: vs mma semantics {e_mma:.3e}, vs exact dequantisation {e_exact:.3e}")
+    assert e_mma <= 2e-2 and e_exact <= 1e-1
 
 
 def test_config4_gather_bf16(oracle):

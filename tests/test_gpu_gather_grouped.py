@@ -196,3 +196,53 @@ def test_grouped_gather_on_32_row_tiles(oracle, grouped, bits):
         lib.mtq_set_option(b"qmm.tile_rows", 0)
     for buf in (w, s, b, x):
         buf.free()
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_names_keep_their_arithmetic(runner, oracle, bits):
+    """Through the name-keyed dispatch, at 20 rows per expert (above the 8 at which the typed entry points switch to
+    the tile kernel): the reference's exact-dequant CSR names (mt_moe_gather_qmm_int4 / _b8, crates/metaltile-std/src/
+    ffai/moe.rs:358-433) are held to the exact oracle at 1e-2, also for 8-bit codes, where rounding s*q + b to bf16
+    first would not pass; the MMA names (mt_moe_gather_qmm_mma_*, moe.rs:2256) are held to the oracle's mma
+    semantics at 2e-2. With option gather.names_exact = 1 the CSR names follow the MMA names."""
+    dt, E, N, K, G = DType.BF16, 4, 256, 1024, 64
+    counts = [20, 20, 20, 20]
+    T = sum(counts)
+    c = make_case(7300 + bits, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
+    ids = np.repeat(np.arange(E), counts).astype("<u4")
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype("<u4")
+    exact = oracle.round_through(oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=ids,
+                                                   f64=True, threads=8).astype(np.float32), ODT[dt])
+    mma = _expected(oracle, c, ids, T, N, K, E, bits, G, dt)
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    off, idx, out = GpuBuffer.from_bytes(offsets.tobytes()), GpuBuffer.from_bytes(ids.tobytes()), GpuBuffer(T * N * 2)
+    csr_name = "mt_moe_gather_qmm_int4" if bits == 4 else "mt_moe_gather_qmm_b8"
+    mma_name = "mt_moe_gather_qmm_mma_int4" if bits == 4 else "mt_moe_gather_qmm_mma_int8"
+    csr_bufs = {"x": x, "weight_packed": w, "scales": s, "biases": b, "expert_offsets": off, "out": out}
+    csr_consts = {"k_in": K, "m_out": N, "n_experts": E, "group_size": G}
+    lib = _lib.load()
+
+    def run(name, bufs, consts):
+        out.zero()
+        runner.dispatch(name, dt, bufs, consts)
+        return unpack_f32(out.read_bytes(), dt)
+
+    got = run(csr_name, csr_bufs, csr_consts)
+    e_exact, e_mma = rel_err(got, exact), rel_err(got, mma)
+    print(f"{csr_name}: vs exact {e_exact:.3e}, vs mma semantics {e_mma:.3e}")
+    assert e_exact <= 1e-2
+    got_m = run(mma_name, {"x": x, "w": w, "scales": s, "biases": b, "indices": idx, "out": out},
+                {"m_total": T, "n_out": N, "k_in": K, "group_size": G})
+    m_exact, m_mma = rel_err(got_m, exact), rel_err(got_m, mma)
+    print(f"{mma_name}: vs exact {m_exact:.3e}, vs mma semantics {m_mma:.3e}")
+    assert m_mma <= 2e-2
+    assert not np.array_equal(got, got_m)      # the two names really ran different arithmetic
+    try:
+        assert lib.mtq_set_option(b"gather.names_exact", 1) == 0
+        got_s = run(csr_name, csr_bufs, csr_consts)
+        assert np.array_equal(got_s, got_m)
+    finally:
+        lib.mtq_set_option(b"gather.names_exact", 0)
+    for buf in (w, s, b, x, off, idx, out):
+        buf.free()
