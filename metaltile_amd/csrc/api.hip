@@ -1281,8 +1281,13 @@ int mtq_set_option(const char* name, int value) {
         return MTQ_OK;
     }
     if (!strcmp(name, "qmm.tile_rows")) {
-        if (value != 0 && value != 32 && value != 64 && value != 128) return fail(ERR_BAD_ARG, "qmm.tile_rows must be 0, 32, 64 or 128");
+        if (value != 0 && value != 32 && value != 64 && value != 128 && value != 256) return fail(ERR_BAD_ARG, "qmm.tile_rows must be 0, 32, 64, 128 or 256");
         options().qmm_tile_rows = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmm.dma")) {
+        if (value < 0 || value > 1) return fail(ERR_BAD_ARG, "qmm.dma must be 0 (where the shape allows) or 1 (never)");
+        options().qmm_dma = value;
         return MTQ_OK;
     }
     if (!strcmp(name, "qmm.splits")) {

@@ -52,8 +52,28 @@ template <int DT> __global__ __launch_bounds__(256) void qmm_split_reduce_kernel
     ((uint16_t*)out)[i] = f32_to_elem_bits<DT>(r);
 }
 
+// Shapes the load-to-LDS instances take: 4-bit codes, 2 K-groups, whole iterations of 128 k, whole 8-element
+// vectors of scales per row, one launch (no K split, no expert routing), and the ring of tiles beside the tile's
+// scales and biases within the 160 KB.
+static bool dma_fits(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr) {
+    if (options().qmm_dma == 1 || bits != 4 || kgroups != 2 || K % 128 || gpr % 8) return false;
+    if (rows != 64 && rows != 128 && rows != 256) return false;
+    return qmm_dma_lds_bytes(rows, gpr) <= 160 * 1024;
+}
+
 template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, const LaunchCtx& lc, bool grouped = false) {
     const void* fn = nullptr;
+    if (!grouped && a.ksplit <= 1 && dma_fits(bits, a.m_tile_rows, kgroups, a.K, a.gpr)) {
+        fn = qmm_dma_pick(DT, a.m_tile_rows);
+        const size_t shmem = qmm_dma_lds_bytes(a.m_tile_rows, a.gpr);
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
+        void* args[] = {&a};
+        e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles), dim3(512), args, shmem, lc);
+        if (e != hipSuccess) return hip_fail(e, "qmm load-to-LDS kernel launch");
+        return ERR_OK;
+    }
+    if (a.m_tile_rows == 256) return fail(ERR_UNSUPPORTED, "direct qmm: 256-row tiles need 4-bit codes, K % 128 == 0 and at most 64 groups per row");
     const bool tall = a.m_tile_rows == 128;
     const uint32_t dbn = kgroups == 1 ? 128 : 32 * (8 / kgroups);
     // scales and biases of the tile's rows in LDS when they fit beside the activation tiles
@@ -181,6 +201,33 @@ static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
         rows = p.M <= 32 ? 32 : 64;
         kgroups = 4;
     }
+    // Shapes the load-to-LDS instances take, with enough 64 x 128 tiles for half the chip: the tile height with
+    // the lowest estimate. A round of tiles (one per compute unit) costs, at K = 4096, 20.6 / 28.0 / 48.5 us on
+    // 64- / 128- / 256-row tiles when at most half the compute units are busy, 16 / 35 / 45 % more when all are
+    // (the clock drops under full matrix load), and another 15 / 10 / 0 % when more rounds follow. Measured at
+    // 4096 x 4096: 384 rows 26.7 -> 22.9 us, 512 rows 28.7 -> 23.8, 768 rows 38.3 -> 31.6, 1024 rows 43.0 -> 37.8,
+    // 1536 rows 68.7 -> 56.8, 2048 rows 79.2 -> 70.6, 4096 rows 152 -> 141; 14336 x 4096: 512 rows 75.3 -> 65.1,
+    // 4096 rows 513 -> 459; 4096 x 8192, 512 rows: 61.1 -> 43.8.
+    if (p.M > 64 && short_wide * 2 > (uint64_t)cus && !options().qmm_tile_rows && !options().qmm_kgroups) {
+        static const uint32_t heights[3] = {64, 128, 256};
+        static const double base[3] = {20.6, 28.0, 48.5}, full[3] = {0.16, 0.35, 0.45}, more[3] = {1.15, 1.10, 1.0};
+        double best = 0.0;
+        // long rows leave room for 64-row tiles only: past two rounds of them the 128-row tiles on 4-wave workgroups
+        // stay ahead (4096 x 8192, 2048 rows: 188 us against 203)
+        const bool short_only = !dma_fits(p.bits, 128, 2, p.K, p.K / G) && short_wide > 2 * (uint64_t)cus;
+        for (int i = 0; i < 3 && !short_only; i++) {
+            if (!dma_fits(p.bits, heights[i], 2, p.K, p.K / G)) continue;
+            const uint64_t tiles = (uint64_t)((p.M + heights[i] - 1) / heights[i]) * ((p.N + 127) / 128);
+            const uint64_t whole = tiles / (uint64_t)cus, rest = tiles % (uint64_t)cus;
+            double est = (double)whole * base[i] * (1.0 + full[i]) * (whole + (rest ? 1 : 0) > 1 ? more[i] : 1.0);
+            if (rest) {
+                double f = ((double)rest / cus - 0.5) * 2.0;
+                f = f < 0.0 ? 0.0 : f;
+                est += base[i] * (1.0 + full[i] * f);
+            }
+            if (best == 0.0 || est < best) { best = est; rows = heights[i]; kgroups = 2; }
+        }
+    }
     if (options().qmm_tile_rows) rows = (uint32_t)options().qmm_tile_rows;
     if (options().qmm_kgroups) kgroups = (uint32_t)options().qmm_kgroups;
     // An iteration covers 64 k per K-group: K must be a multiple of 64 * K-groups (an odd number of
@@ -192,6 +239,8 @@ static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
     }
     // the bit-stream widths are built with 128-row tiles on 1 K-group only
     if (odd_bits && rows == 128 && !options().qmm_kgroups) kgroups = 1;
+    if (rows == 256 && !dma_fits(p.bits, 256, kgroups, p.K, p.K / G))
+        return fail(ERR_BAD_ARG, "qmm.tile_rows 256 needs 4-bit codes, 2 K-groups, K % 128 == 0 and at most 64 groups per row");
     if (rows == 32 && kgroups != 4) {
         if (options().qmm_tile_rows) return fail(ERR_BAD_ARG, "qmm.tile_rows 32 needs 4 K-groups");
         rows = 64;

@@ -1,0 +1,26 @@
+// Instances of the tile kernel whose activation tile is brought in by load-to-LDS instructions (4-bit codes,
+// f16 / bf16, 2 K-groups x 4 column waves): replaces the same reference kernels as qmm_direct.hip (mt_qmm_mma and
+// its _m16 form, crates/metaltile-std/src/mlx/quantized.rs:2106-2405, 2408) with the same arithmetic, on 64 x 128,
+// 128 x 128 and 256 x 128 tiles. A translation unit of its own so that it compiles beside qmm_direct.hip.
+#include "qmm_dma_impl.h"
+
+namespace mtq {
+
+// LDS of one workgroup: the ring of tiles and the scales / biases window, or the epilogue's partial sums and
+// element tile (at most 128 rows at a time).
+size_t qmm_dma_lds_bytes(uint32_t rows, uint32_t gpr) {
+    const uint32_t mb = rows / 32, nbuf = mb == 8 ? 2 : 3, dbn = 128, kg = 2;
+    const size_t main_loop = (size_t)nbuf * mb * kg * 4096 + (size_t)2 * dbn * (gpr + (nbuf != 3 ? 0 : 2)) * 2;
+    const uint32_t epb = mb == 8 ? 4 : mb;
+    const size_t epilogue = (size_t)(kg - 1) * 4 * epb * 16 * 64 * 4 + (size_t)epb * 32 * dbn * 2;
+    return main_loop > epilogue ? main_loop : epilogue;
+}
+
+const void* qmm_dma_pick(int dtype, uint32_t rows) {
+#define QDMA(DTv) (rows == 64 ? (const void*)qmm_dma_kernel<DTv, 2, 2, 8> : rows == 128 ? (const void*)qmm_dma_kernel<DTv, 4, 2, 8> \
+                   : rows == 256 ? (const void*)qmm_dma_kernel<DTv, 8, 2, 8> : nullptr)
+    return dtype == DT_BF16 ? QDMA(DT_BF16) : dtype == DT_F16 ? QDMA(DT_F16) : nullptr;
+#undef QDMA
+}
+
+}  // namespace mtq

@@ -1,0 +1,352 @@
+// The register-operand tile kernel with its activation tile brought in by load-to-LDS instructions
+// (see qmm_direct.hip for the tiling; this header only differs in how the operands travel).
+#pragma once
+#include "qmm_direct_impl.h"
+
+#include <type_traits>
+
+namespace mtq {
+
+typedef uint32_t qm_u32x4 __attribute__((ext_vector_type(4)));
+typedef float qm_f32x2 __attribute__((ext_vector_type(2)));
+
+// f(integral_constant<int, I>) for I = B .. E-1: loop indices that are constant expressions in the body.
+template <int B, int E, class F> __device__ __forceinline__ void qm_static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        qm_static_for<B + 1, E>(f);
+    }
+}
+
+// One 16-byte-per-lane load from global memory straight into LDS: lane l's bytes land at
+// lds_base + 16 * l (lds_base is wave-uniform and goes through M0); the global address is
+// sbase + voff per lane. Counts in vmcnt like any vector memory load.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"   // M0 is a reserved register: naming it as clobbered is the point
+__device__ __forceinline__ void qm_load_to_lds(uint32_t lds_base, uint32_t voff, const void* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sbase) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+// 16 bytes per lane from sbase + voff into registers. The result is valid only after a qm_wait_vm
+// that covers it; until then the registers must not be read or copied.
+__device__ __forceinline__ void qm_load_regs(qm_u32x4& dst, uint32_t voff, const void* sbase) {
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
+}
+// Waits until at most N vector memory loads of this wave are outstanding (they complete in order).
+template <int N> __device__ __forceinline__ void qm_wait_vm() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// The same, and ties the loaded registers to the wait so that no use of them is scheduled above it.
+template <int N> __device__ __forceinline__ void qm_wait_vm_for(qm_u32x4& r) {
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r) : "n"(N) : "memory");
+}
+
+// Four 4-bit codes -> four elements s * q + b rounded to T, as two dwords. e and o hold the even and the odd
+// codes of a weight dword one per byte (e = w & 0x0F0F0F0F, o = (w >> 4) & 0x0F0F0F0F); `half` picks bytes
+// 0, 1 or 2, 3. A byte 0..15 read as an fp8 (E4M3) number is exactly code / 512, so one packed fp8 -> f32
+// convert yields two codes, and with s512 = 512 * s the fused multiply-add rounds the same exact value
+// s * q + b as it would from the integer code.
+template <int DT> __device__ __forceinline__ void qm_dequant4_b4(uint32_t e, uint32_t o, int half, float s512, float b, uint32_t& d0, uint32_t& d1) {
+    const qm_f32x2 fe = half ? __builtin_amdgcn_cvt_pk_f32_fp8((int)e, true) : __builtin_amdgcn_cvt_pk_f32_fp8((int)e, false);
+    const qm_f32x2 fo = half ? __builtin_amdgcn_cvt_pk_f32_fp8((int)o, true) : __builtin_amdgcn_cvt_pk_f32_fp8((int)o, false);
+    d0 = pack2<DT>(fmaf(fe.x, s512, b), fmaf(fo.x, s512, b));
+    d1 = pack2<DT>(fmaf(fe.y, s512, b), fmaf(fo.y, s512, b));
+}
+
+// Same tiling and arguments as qmm_direct_kernel with 8 waves (KG = 2 or 4 K-groups x 8 / KG column waves,
+// 4-bit codes, scales and biases of the tile staged in LDS), same results; what differs:
+//   activations: the (32 * MB) x (64 * KG) tile of an iteration is MB * KG slots of 32 rows x 64 k (4 KB,
+//     16-byte chunks XOR-swizzled so that the fragment reads are conflict free); the eight waves share its
+//     load-to-LDS instructions (MB * KG / 2 each), issued two iterations ahead into a ring of three tiles: no
+//     register, no LDS store instruction and no vector ALU work is spent on staging. A wave waits for its own
+//     share of the next tile before the iteration's barrier, so past the barrier the whole tile is in LDS.
+//   weights: 16 bytes per lane (the 32 codes it converts) straight into registers three iterations ahead;
+//     converted one iteration ahead with the packed fp8 -> f32 convert (two codes per instruction).
+// Every vector memory load of the loop is issued by hand in a fixed order, so the waits are "at most N loads
+// outstanding" with compile-time N.
+// NB is the depth of the ring of activation tiles (0: three, or two for 256-row tiles, whose tile is 64 KB): tile
+// it + NB - 1 is issued during iteration it. Measured at 1024 x 4096 x 4096 the depth does not matter (2 / 3 / 4:
+// 39.3 / 40.0 / 41.5 us): the loop is not waiting for latency.
+// 256-row tiles (MB = 8) keep the scales and biases unpadded, row r rotated by 8 r elements, so that two tiles and the
+// window fill the 160 KB exactly at 64 groups per row; their epilogue runs in two rounds of 128 rows.
+template <int DT, int MB, int KG, int NW, int NB = 0, bool GR = false, bool SP = false>
+__global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
+    static_assert(NW == 8 || NW == 16, "two or four waves per SIMD");
+    static_assert(KG == 2 || KG == 4, "2 or 4 K-groups");
+    static_assert(MB == 1 || MB == 2 || MB == 4 || MB == 8, "32 to 256 rows");
+    constexpr int BITS = 4;
+    constexpr int NT = 64 * NW, NWV = NW / KG;
+    constexpr int DBN = 32 * NWV, DBK = 64 * KG, DBM = 32 * MB;
+    constexpr int NSLOT = MB * KG, SLOT = 4096, TILE = NSLOT * SLOT;
+    constexpr int NBUF = NB ? NB : MB == 8 ? 2 : 3;
+    static_assert(NBUF >= 2 && NBUF <= 6, "ring of 2 to 6 tiles");
+    constexpr int WSN = NBUF < 3 ? 3 : NBUF;   // weight register sets: weights are issued WSN iterations ahead
+    constexpr int IPW = NSLOT * 4 / NW;       // load-to-LDS instructions per wave and iteration
+    static_assert(IPW >= 1 && NSLOT * 4 % NW == 0, "the tile's load instructions divide among the waves");
+    constexpr int NM = 4 * MB;                // MFMAs per wave and iteration
+    constexpr int UN = WSN % 2 ? 2 * WSN : WSN;   // unroll: a multiple of the ring, of the weight sets and of 2 (fragment parity)
+    static_assert(UN % NBUF == 0 && UN % WSN == 0 && UN % 2 == 0, "unroll covers every ring");
+    extern __shared__ __align__(16) unsigned char lds[];  // NBUF tiles, then the scales / biases window
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t kg = wave / NWV, wn = wave % NWV;
+    const uint32_t fr = lane & 31u, fh = lane >> 5;
+
+    const uint32_t total = a.m_tiles * a.n_tiles;
+    uint32_t vid = blockIdx.x;
+    if (!GR && total % 8 == 0) vid = (blockIdx.x & 7u) * (total / 8) + (blockIdx.x >> 3);
+    uint32_t nt = a.by_m ? vid % a.n_tiles : vid / a.m_tiles, mt = a.by_m ? vid / a.n_tiles : vid % a.m_tiles;
+    uint32_t row_first = mt * DBM, row_count = a.M > row_first ? min((uint32_t)DBM, a.M - row_first) : 0u;
+    if constexpr (GR) {
+        nt = blockIdx.x % a.n_tiles;
+        mt = blockIdx.x / a.n_tiles;
+        if (mt >= a.tiles[0]) return;  // the grid is sized for the worst routing
+        const uint4 t = ((const uint4*)a.tiles)[1 + mt];
+        row_first = t.y;
+        row_count = t.z;
+        a.w += (size_t)t.x * a.w_expert_bytes;
+        a.scales += (size_t)t.x * a.sb_expert_elems * 2;
+        a.biases += (size_t)t.x * a.sb_expert_elems * 2;
+    }
+    auto row_of = [&](uint32_t j) -> uint32_t {  // j < row_count
+        if constexpr (GR) return a.rowlist ? a.rowlist[row_first + j] : row_first + j;
+        else return row_first + j;
+    };
+    const uint32_t n0 = nt * DBN;
+    uint32_t it_base = 0;  // first iteration of this workgroup's share of K
+    if constexpr (SP) {
+        it_base = blockIdx.y * a.iters_per_split;
+        a.iters = min(a.iters_per_split, a.iters - it_base);
+        a.x += (size_t)it_base * (DBK * 2);
+        a.w += (size_t)it_base * (DBK * BITS / 8);
+    }
+    const uint32_t ilast = a.iters - 1;
+    // groups of scales / biases this workgroup needs: [sb_g0, sb_g0 + sb_ng), whole 8-element vectors
+    const uint32_t sb_g0 = ((it_base * DBK) >> a.log2g) & ~7u;
+    const uint32_t sb_ng = min(a.gpr - sb_g0, (((((it_base + a.iters) * DBK - 1) >> a.log2g) + 1 - sb_g0) + 7u) & ~7u);
+
+    // ---- per-lane offsets ---------------------------------------------------------------------------
+    // this wave's load-to-LDS instructions: unit q = wave * IPW + i is quarter q % 4 of slot q / 4; slot sl holds
+    // row block sl % MB, k-block sl / MB of the iteration; a quarter is 8 rows x 128 bytes, lane l moving chunk
+    // (l % 8) ^ ((row / 2) % 8) of row 8 * quarter + l / 8
+    uint32_t xoff[IPW];
+#pragma unroll
+    for (int i = 0; i < IPW; i++) {
+        const uint32_t q = wave * IPW + i, sl = q / 4, t = q % 4;
+        const uint32_t rr = 8 * t + (lane >> 3), c = (lane & 7u) ^ ((rr >> 1) & 7u);
+        const uint32_t lrow = min((sl % MB) * 32 + rr, row_count - 1);
+        xoff[i] = row_of(lrow) * (a.K * 2) + (sl / MB) * 128 + c * 16;
+    }
+    // fragment reads: MFMA step j of lane (fr, fh) takes chunk 4 * fh + j of row fr of slot (bi, kg)
+    uint32_t aoff[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) aoff[j] = kg * MB * SLOT + (fr * 8 + ((4 * fh + j) ^ ((fr >> 1) & 7u))) * 16;
+    // weights: row n0 + 32 * wn + fr, codes [64 * kg + 32 * fh, +32) of the iteration; the last tile of a ragged N
+    // works its missing rows on row N - 1 and stores none of their columns
+    const uint32_t wrow = min(n0 + wn * 32 + fr, a.N - 1);
+    const uint32_t woff = wrow * (a.K * BITS / 8) + (kg * 64 + fh * 32) * BITS / 8;
+    const uint32_t kofs_abs = it_base * DBK + kg * 64 + fh * 32;  // k of this lane's codes counted from the start of the row
+    const uint32_t ring = (uint32_t)(uintptr_t)lds;
+
+    // LDS after the tiles: [DBN rows][gpr + 2] scales, then the same for biases
+    // rows padded by two elements, or (256-row tiles: no room for padding) row r rotated by 8 r elements, so that
+    // the 32 rows a wave reads one group of do not all fall into one bank
+    constexpr bool ROT = NBUF != 3;
+    const uint32_t sbld = ROT ? sb_ng : a.gpr + 2;
+    uint16_t* sbS = (uint16_t*)(lds + NBUF * TILE);
+    uint16_t* sbB = sbS + DBN * sbld;
+    const int sbrow = (int)((wn * 32 + fr) * sbld) - (ROT ? 0 : (int)sb_g0);
+    const uint32_t sbrot = ((wn * 32 + fr) * 8) % sbld - sb_g0 + sbld;   // ROT: position of group g is (g + sbrot) mod sbld
+
+    auto issue_x = [&](uint32_t it, int buf) {
+        const unsigned char* src = a.x + (size_t)min(it, ilast) * (DBK * 2);
+#pragma unroll
+        for (int i = 0; i < IPW; i++) qm_load_to_lds(ring + buf * TILE + (wave * IPW + i) * 1024, xoff[i], src);
+    };
+    qm_u32x4 raw[WSN];
+    auto issue_w = [&](uint32_t it, int set) {
+        qm_load_regs(raw[set], woff, a.w + (size_t)min(it, ilast) * (DBK * BITS / 8)); };
+    // 512 * scale and bias of this lane's codes in iteration it (zero past the end: such an iteration adds nothing)
+    auto scale_bias = [&](uint32_t it, float& s512, float& b) {
+        int g = (int)((min(it, ilast) * DBK + kofs_abs) >> a.log2g);
+        if constexpr (ROT) {
+            g += sbrot;                      // in [sbld, 3 sbld)
+            if (g >= 2 * (int)sbld) g -= sbld;
+            g -= sbld;
+        }
+        s512 = elem_bits_to_f32<DT>(sbS[sbrow + g]) * 512.f;
+        b = elem_bits_to_f32<DT>(sbB[sbrow + g]);
+        if (it > ilast) s512 = b = 0.f;
+    };
+
+    f32x16 acc[MB];
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[i][v] = 0.f;
+
+    // ---- prologue ------------------------------------------------------------------------------------
+    // issue order of the loop: iteration it issues W(it + 3), then X(it + 2) x IPW; the iterations before the
+    // first issue W(0), W(1) | W(2), X(0) | W(3)... : here W(0), W(1), W(2), X(0), then (as iteration -1) X(1)
+    qm_static_for<0, WSN>([&](auto i_c) { issue_w(decltype(i_c)::value, decltype(i_c)::value); });
+    qm_static_for<0, NBUF - 1>([&](auto i_c) { issue_x(decltype(i_c)::value, decltype(i_c)::value); });
+    {
+        // DBN rows x sb_ng elements each of scales and biases, 16 bytes per load (ordinary loads: the compiler waits)
+        const uint32_t vpr = sb_ng / 8, nvec = DBN * vpr;
+        for (uint32_t v = tid; v < nvec; v += NT) {
+            const uint32_t row = v / vpr, c0 = (v - row * vpr) * 8;
+            const uint32_t grow = min(n0 + row, a.N - 1);
+            const q_u32x4 sv = *(const q_u32x4*)((const uint16_t*)a.scales + (size_t)grow * a.gpr + sb_g0 + c0);
+            const q_u32x4 bv = *(const q_u32x4*)((const uint16_t*)a.biases + (size_t)grow * a.gpr + sb_g0 + c0);
+            const uint32_t cpos = ROT ? (c0 + row * 8) % sbld : c0;   // whole 8-element vectors move together
+            uint32_t* ds = (uint32_t*)(sbS + row * sbld + cpos);
+            uint32_t* db = (uint32_t*)(sbB + row * sbld + cpos);
+            ds[0] = sv.x; ds[1] = sv.y; ds[2] = sv.z; ds[3] = sv.w;
+            db[0] = bv.x; db[1] = bv.y; db[2] = bv.z; db[3] = bv.w;
+        }
+    }
+    qm_wait_vm<(NBUF - 2) * IPW>();   // everything but X(1)..: the first tile's share and the first weight sets
+    __syncthreads();      // tile 0 and the scales are in LDS
+    uint32_t bq[2][4][4];  // converted fragments: [iteration parity][MFMA step][dword]
+    float sn, bn;          // 512 * scale and bias of the iteration being converted (the next one)
+    {
+        qm_wait_vm_for<(NBUF - 2) * IPW>(raw[0]);
+        float s0, b0;
+        scale_bias(0, s0, b0);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t e = raw[0][j] & 0x0F0F0F0Fu, o = (raw[0][j] >> 4) & 0x0F0F0F0Fu;
+            qm_dequant4_b4<DT>(e, o, 0, s0, b0, bq[0][j][0], bq[0][j][1]);
+            qm_dequant4_b4<DT>(e, o, 1, s0, b0, bq[0][j][2], bq[0][j][3]);
+        }
+        scale_bias(1, sn, bn);
+    }
+    qm_u32x4 af[2][4];  // activation fragments of one 32-row block: [row block parity][MFMA step]
+#pragma unroll
+    for (int j = 0; j < 4; j++) af[0][j] = *(const qm_u32x4*)(lds + aoff[j]);
+
+    const uint32_t iters_up = (a.iters + UN - 1) / UN * UN;
+    for (uint32_t it0 = 0; it0 < iters_up; it0 += UN) {
+        qm_static_for<0, UN>([&](auto u_c) {
+            constexpr int u = decltype(u_c)::value;
+            constexpr int cur = u & 1, nxt = cur ^ 1;
+            constexpr int buf = u % NBUF;
+            const uint32_t it = it0 + u;
+            if (it >= a.iters) return;   // (uniform) the unrolled run reaches past the last iteration
+            // loads: this wave's share of the tile two iterations ahead into the buffer read during the last iteration,
+            // weights three iterations ahead into the set whose weights have been converted
+            if constexpr (NBUF == 2) {
+                // ring of two: the next tile into the buffer read during the last iteration, then the weights
+                issue_x(it + 1, (u + 1) % NBUF);
+                issue_w(it + WSN, u % WSN);
+            } else {
+                issue_w(it + WSN, u % WSN);
+                issue_x(it + NBUF - 1, (u + NBUF - 1) % NBUF);
+            }
+            float sn2, bn2;
+            uint32_t ek = 0, ok = 0;
+            // weights of the next iteration, issued WSN - 1 iterations ago: the loads younger than they are the tiles
+            // of WSN iterations and the weights of WSN - 1 (ring of two: tiles and weights of two iterations)
+            qm_wait_vm_for<(NBUF == 2 ? 2 * IPW + 2 : WSN * IPW + WSN - 1)>(raw[(u + 1) % WSN]);
+            qm_static_for<0, MB>([&](auto bi_c) {
+                constexpr int bi = decltype(bi_c)::value;
+                constexpr int par = bi & 1;
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[par][0]), "+v"(af[par][1]), "+v"(af[par][2]), "+v"(af[par][3])::"memory");
+                if (bi + 1 < MB) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) af[par ^ 1][j] = *(const qm_u32x4*)(lds + buf * TILE + (bi + 1) * SLOT + aoff[j]);
+                }
+                if (bi == 0) scale_bias(it + 2, sn2, bn2);
+                __builtin_amdgcn_sched_barrier(0);
+                qm_static_for<0, 4>([&](auto j_c) {
+                    constexpr int j = decltype(j_c)::value;
+                    constexpr int m = bi * 4 + j;   // MFMA of the iteration
+                    const uint4 bv = make_uint4(bq[cur][j][0], bq[cur][j][1], bq[cur][j][2], bq[cur][j][3]);
+                    const uint4 av = make_uint4(af[par][j].x, af[par][j].y, af[par][j].z, af[par][j].w);
+                    acc[bi] = mfma32<DT>(av, bv, acc[bi]);
+                    // its share of the next iteration's conversion: half fragments [8 m / NM, 8 (m + 1) / NM)
+#pragma unroll
+                    for (int hf = 8 * m / NM; hf < 8 * (m + 1) / NM; hf++) {
+                        const int jj = hf / 2, half = hf % 2;
+                        if (half == 0) {
+                            ek = raw[(u + 1) % WSN][jj] & 0x0F0F0F0Fu;
+                            ok = (raw[(u + 1) % WSN][jj] >> 4) & 0x0F0F0F0Fu;
+                        }
+                        qm_dequant4_b4<DT>(ek, ok, half, sn, bn, bq[nxt][jj][2 * half], bq[nxt][jj][2 * half + 1]);
+                    }
+                });
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            sn = sn2;
+            bn = bn2;
+            // this wave's share of the next tile (issued one iteration ago) is in LDS once at most this iteration's
+            // loads are outstanding; past the barrier every wave's share is
+            // (one less than the steady state allows: the first iterations follow the prologue's order)
+            qm_wait_vm<(NBUF == 2 ? 1 : NBUF == 3 ? IPW + 1 : (NBUF - 2) * (IPW + 1) - 1)>();
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 4; j++) af[0][j] = *(const qm_u32x4*)(lds + ((u + 1) % NBUF) * TILE + aoff[j]);
+        });
+    }
+    qm_wait_vm<0>();   // loads still in flight write into the ring the epilogue is about to reuse
+    __syncthreads();
+
+    // ---- the other K-groups hand their accumulators to K-group 0 through LDS, at most 128 rows at a time ---
+    constexpr int EPB = MB == 8 ? 4 : MB;       // row blocks per round
+    constexpr int GRP = NWV * EPB * 16 * 64;    // floats per K-group and round
+    float* red = (float*)lds;                   // [kg - 1][wn][bi][v][lane]
+    uint16_t* otile = (uint16_t*)(lds + (KG - 1) * GRP * 4);   // the round's rows as [row][DBN columns], behind the partial sums
+    qm_static_for<0, MB / EPB>([&](auto ph_c) {
+        constexpr int ph = decltype(ph_c)::value;
+        if constexpr (ph > 0) __syncthreads();   // the last round's tile has been stored
+        if (kg != 0) {
+#pragma unroll
+            for (int bi = 0; bi < EPB; bi++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) red[(kg - 1) * GRP + ((wn * EPB + bi) * 16 + v) * 64 + lane] = acc[ph * EPB + bi][v];
+        }
+        __syncthreads();
+        // accumulator layout: column j = lane%32, row i = 8*(v/4) + 4*(lane/32) + v%4.
+        // K-group 0 adds, rounds to the element dtype and writes the rows to LDS
+        if (kg == 0) {
+#pragma unroll
+            for (int bi = 0; bi < EPB; bi++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const uint32_t trow = bi * 32 + 8 * (v / 4) + 4 * fh + (v % 4), lrow = ph * EPB * 32 + trow;
+                    float r = acc[ph * EPB + bi][v];
+#pragma unroll
+                    for (int g = 0; g < KG - 1; g++) r += red[g * GRP + ((wn * EPB + bi) * 16 + v) * 64 + lane];
+                    if constexpr (SP) {  // this split's f32 partial sums, 32 consecutive columns per half wave
+                        const uint32_t col = n0 + wn * 32 + fr;
+                        if (lrow < row_count && col < a.N) a.part[((size_t)blockIdx.y * a.M + row_first + lrow) * a.N + col] = r;
+                    } else {
+                        otile[trow * DBN + wn * 32 + fr] = f32_to_elem_bits<DT>(r);
+                    }
+                }
+        }
+        if constexpr (!SP) {  // split instances end with the partial sums: the second kernel rounds and stores
+            __syncthreads();
+            // all threads store the rows, 16 bytes each, whole rows
+            constexpr int VPR = DBN / 8;                         // 16-byte vectors per tile row
+            constexpr int VPT = (EPB * 32 * VPR + NT - 1) / NT;  // vectors per thread
+            if ((a.N & 7u) == 0) {
+#pragma unroll
+                for (int i = 0; i < VPT; i++) {
+                    const uint32_t v = tid + i * NT, trow = v / VPR, lrow = ph * EPB * 32 + trow, col = n0 + (v % VPR) * 8;
+                    if (trow < (uint32_t)(EPB * 32) && lrow < row_count && col < a.N)
+                        *(q_u32x4*)((uint16_t*)a.out + (size_t)row_of(lrow) * a.N + col) = *(const q_u32x4*)(otile + trow * DBN + (v % VPR) * 8);
+                }
+            } else {
+                for (uint32_t e = tid; e < (uint32_t)(EPB * 32 * DBN); e += NT) {
+                    const uint32_t trow = e / DBN, lrow = ph * EPB * 32 + trow, col = n0 + e % DBN;
+                    if (lrow < row_count && col < a.N) ((uint16_t*)a.out)[(size_t)row_of(lrow) * a.N + col] = otile[e];
+                }
+            }
+        }
+    });
+}
+
+}  // namespace mtq

@@ -24,7 +24,7 @@ def options():
         assert lib.mtq_set_option(name.encode(), value) == 0, name
 
     yield set_
-    for name in ("qmm.kernel", "qmm.kgroups", "qmm.tile_rows", "qmm.by_m", "qmm.ksplit"):
+    for name in ("qmm.kernel", "qmm.kgroups", "qmm.tile_rows", "qmm.by_m", "qmm.ksplit", "qmm.dma"):
         lib.mtq_set_option(name.encode(), 0)
 
 
@@ -43,14 +43,17 @@ def test_direct_qmm_every_tiling(oracle, options, bits, dt):
             print(f"[case] direct qmm {dt.name} b{bits} kgroups={kg} tile_rows={rows}", flush=True)
             options("qmm.kgroups", kg)
             options("qmm.tile_rows", rows)
-            for by_m in (1, 2):  # both orders of walking the tiles
+            # both orders of walking the tiles; 4-bit codes on 2 K-groups also with and without the instances
+            # that bring the activation tile in by load-to-LDS instructions
+            for by_m, dma in ((1, 0), (2, 0), (1, 1)):
                 options("qmm.by_m", by_m)
+                options("qmm.dma", dma)
                 out = GpuBuffer(M * N * dt.size_bytes)
                 ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
                 got = unpack_f32(out.read_bytes(), dt)
                 out.free()
                 err = rel_err(got, exp)
-                assert err <= 2e-2, f"kgroups={kg} rows={rows} by_m={by_m}: rel err {err:.3e}"
+                assert err <= 2e-2, f"kgroups={kg} rows={rows} by_m={by_m} dma={dma}: rel err {err:.3e}"
     for buf in (w, s, b, x):
         buf.free()
 
@@ -241,3 +244,58 @@ def test_tall_tiles_on_long_rows(oracle, M, N):
     for buf in (w, s, b, x, out):
         buf.free()
     assert rel_err(got, exp) <= 2e-2
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("M,N,K,G", [(300, 256, 256, 32),      # two iterations; ragged last tiles at every height
+                                     (257, 200, 768, 32),      # six iterations, N % 8 == 0 but N % 128 != 0
+                                     (70, 131, 1024, 128),     # N % 8 != 0: element-wise stores
+                                     (512, 384, 4096, 64),     # 64 groups per row: the 256-row tile's LDS is full to the byte
+                                     (260, 128, 2816, 32)])    # 22 iterations (not a multiple of the unroll), 88 groups per row
+def test_load_to_lds_tiles(oracle, options, dt, M, N, K, G):
+    """The 4-bit instances whose activation tile arrives by load-to-LDS instructions, on 64-, 128- and 256-row
+    tiles, against the oracle's mma semantics (2e-2, as above) and against the register-staged instance of the
+    same tiling (same arithmetic, same order of the partial sums: bit-equal)."""
+    bits = 4
+    c = make_case(5400 + M + K, dt, bits, G, M, N, K)
+    exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    options("qmm.kernel", 2)
+    options("qmm.kgroups", 2)
+    for rows in (64, 128, 256):
+        if rows == 256 and K // G > 64:
+            continue  # two 64 KB tiles leave room for 64 groups per row
+        print(f"[case] load-to-LDS qmm {dt.name} M={M} N={N} K={K} g{G} tile_rows={rows}", flush=True)
+        options("qmm.tile_rows", rows)
+        options("qmm.dma", 0)
+        out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
+        ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+        got_bytes = out.read_bytes()
+        got = unpack_f32(got_bytes, dt)
+        out.free()
+        assert rel_err(got, exp) <= 2e-2, f"rows={rows}"
+        if rows != 256:
+            options("qmm.dma", 1)
+            out = GpuBuffer(M * N * dt.size_bytes)
+            ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+            assert out.read_bytes() == got_bytes, f"rows={rows}: differs from the register-staged instance"
+            out.free()
+    for buf in (w, s, b, x):
+        buf.free()
+
+
+def test_256_row_tiles_refuse_what_they_cannot_take(options):
+    """Forced 256-row tiles on a shape outside their limits (8-bit codes) are refused, not rerouted."""
+    dt, bits, G, M, N, K = DType.BF16, 8, 64, 256, 128, 256
+    c = make_case(5500, dt, bits, G, M, N, K)
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    out = GpuBuffer(M * N * dt.size_bytes)
+    options("qmm.kernel", 2)
+    options("qmm.tile_rows", 256)
+    with pytest.raises(Exception, match="256"):
+        ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+    for buf in (w, s, b, x, out):
+        buf.free()
