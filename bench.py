@@ -48,10 +48,11 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=8, help="distinct MLP weight sets streamed per step")
     ap.add_argument("--workload", default="qmv",
-                    choices=["qmv", "qkv", "qmm", "gather", "gather_prefill", "quantize", "dequantize", "copy", "sweep"],
+                    choices=["qmv", "qkv", "qmm", "gather", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep"],
                     help="qmv is the headline (its line also carries qmm M=512 and the gather as secondary legs); "
                          "qmm / gather report those configurations alone; sweep the bit-width / group-size cells; "
-                         "copy runs only the known-size copy kernel (counter calibration)")
+                         "copy runs only the known-size copy kernel (counter calibration); read times a kernel that only reads the "
+                         "headline launch's bytes (the ceiling for the qmv kernel)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-secondary", action="store_true", help="qmv workload: skip the qmm M=512 and gather legs")
     ap.add_argument("--m", type=int, default=512, help="qmm workload: activation rows")
@@ -364,6 +365,27 @@ def main():
         us = runner.copy_kernel(dst, src, nbytes, repeat=max(a.steps, 1))
         out.update({"metric": "copy kernel GB/s (read+write)", "value": round(2 * nbytes / us / 1e3, 1), "unit": "GB/s",
                     "ms_per_step": us / 1e3, "dtype": "u8", "config": {"workload": f"device copy of {nbytes} B"}})
+        print(json.dumps(out))
+        return
+
+    if a.workload == "read":
+        # the ceiling of the headline kernel: launches that only read as many bytes as one qmv of the headline
+        # shape (weights, scales, biases: 33 MB), over 24 buffers (more than the last-level cache holds)
+        nbytes = qmv_bytes(14336, 4096, 4, 64, 1, 2) // 16 * 16
+        bufs = [GpuBuffer(nbytes) for _ in range(24)]
+        cells = {}
+        for wgs in (512, 1024, 1792, 2048, 3584, 4096, 8192):
+            for nt in (False, True):
+                runner.read_kernel(bufs, nbytes, repeat=2, workgroups=wgs, nontemporal=nt)
+                us = min(runner.read_kernel(bufs, nbytes, repeat=max(a.steps // 10, 2), workgroups=wgs, nontemporal=nt) for _ in range(3))
+                cells[f"wg{wgs}{'_nt' if nt else ''}"] = {"us": round(us, 3), "GBps": round(nbytes / us / 1e3, 1), "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        best = min(cells.values(), key=lambda c: c["us"])
+        out.update({"metric": "read-only kernel GB/s, 33 MB per launch (the headline qmv's bytes), cold buffers, back to back",
+                    "value": best["GBps"], "unit": "GB/s", "ms_per_step": best["us"] / 1e3, "dtype": "u8",
+                    "config": {"workload": f"read {nbytes} B per launch over 24 buffers", "cells": cells},
+                    "roofline": {"bound": "hbm", "achieved": best["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": best["frac"], "traffic": None}})
+        for b in bufs:
+            b.free()
         print(json.dumps(out))
         return
 

@@ -328,6 +328,16 @@ MTQ_API int mtq_dispatch_chain(const mtq_dispatch_spec *specs, int n, int repeat
  * readings are calibrated against. */
 MTQ_API int mtq_copy_kernel(void *dst, const void *src, size_t bytes, int repeat, double *avg_us);
 
+/* Measurement aid, no counterpart in the reference: a kernel that only reads. `repeat` passes over the n_srcs
+ * buffers of `bytes` bytes each (bytes % 16 == 0) are enqueued back to back on the library's stream, one launch per
+ * buffer, `workgroups` (0 = 2048) workgroups of 256 threads with eight 16-byte loads in flight per thread
+ * (nontemporal != 0: loads marked as not to be kept in cache); *avg_us is the average launch duration
+ * over the run, gaps between launches included. `sink` is 4 bytes of device memory that are (in practice) never
+ * written. With more buffers than the last-level cache holds this is the rate at which a launch of that size can
+ * stream HBM at all: the ceiling for a weight-streaming kernel of the same size. */
+MTQ_API int mtq_read_kernel(const void *const *srcs, int n_srcs, size_t bytes, int repeat, int workgroups,
+                            int nontemporal, void *sink, double *avg_us);
+
 /* 1 if mtq_dispatch knows `kernel_name`, else 0. */
 MTQ_API int mtq_kernel_supported(const char *kernel_name);
 /* Number of names mtq_dispatch knows, and the i-th of them (NULL past the end). */
