@@ -330,13 +330,13 @@ MTQ_API int mtq_copy_kernel(void *dst, const void *src, size_t bytes, int repeat
 
 /* Measurement aid, no counterpart in the reference: a kernel that only reads. `repeat` passes over the n_srcs
  * buffers of `bytes` bytes each (bytes % 16 == 0) are enqueued back to back on the library's stream, one launch per
- * buffer, `workgroups` (0 = 2048) workgroups of 256 threads with eight 16-byte loads in flight per thread
- * (nontemporal != 0: loads marked as not to be kept in cache); *avg_us is the average launch duration
+ * buffer, `workgroups` (0 = 2048) workgroups of 256 threads with `in_flight` (1, 2, 4, 8; 0 = 8) 16-byte loads in
+ * flight per thread (nontemporal != 0: loads marked as not to be kept in cache); *avg_us is the average launch duration
  * over the run, gaps between launches included. `sink` is 4 bytes of device memory that are (in practice) never
  * written. With more buffers than the last-level cache holds this is the rate at which a launch of that size can
  * stream HBM at all: the ceiling for a weight-streaming kernel of the same size. */
 MTQ_API int mtq_read_kernel(const void *const *srcs, int n_srcs, size_t bytes, int repeat, int workgroups,
-                            int nontemporal, void *sink, double *avg_us);
+                            int in_flight, int nontemporal, void *sink, double *avg_us);
 
 /* 1 if mtq_dispatch knows `kernel_name`, else 0. */
 MTQ_API int mtq_kernel_supported(const char *kernel_name);

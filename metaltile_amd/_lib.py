@@ -74,7 +74,7 @@ SIGNATURES = {
     "mtq_measure": (C.c_int, [C.c_char_p, C.c_int, _bufp, C.c_int, _u32p, C.c_int, _u32p, _u32p, C.c_int, C.c_int, _dblp]),
     "mtq_dispatch_chain": (C.c_int, [C.POINTER(MtqDispatchSpec), C.c_int, C.c_int, _dblp, _dblp, _dblp]),
     "mtq_copy_kernel": (C.c_int, [_vp, _vp, C.c_size_t, C.c_int, _dblp]),
-    "mtq_read_kernel": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_size_t, C.c_int, C.c_int, C.c_int, _vp, _dblp]),
+    "mtq_read_kernel": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _dblp]),
     "mtq_kernel_supported": (C.c_int, [C.c_char_p]),
     "mtq_kernel_count": (C.c_int, []),
     "mtq_kernel_name": (C.c_char_p, [C.c_int]),

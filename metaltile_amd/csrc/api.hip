@@ -97,8 +97,8 @@ __global__ __launch_bounds__(256) void flush_kernel(uint4* p, size_t n) {
 }
 
 // Reads n 16-byte vectors and keeps nothing: the rate at which a launch of this size can pull bytes out of HBM
-// at all, the ceiling of every weight-streaming kernel of the same size. Eight loads in flight per thread.
-template <bool NT> __global__ __launch_bounds__(256) void read_kernel(const uint4* __restrict__ src, size_t n, uint32_t* sink) {
+// at all, the ceiling of every weight-streaming kernel of the same size. B loads in flight per thread.
+template <bool NT, int B> __global__ __launch_bounds__(256) void read_kernel(const uint4* __restrict__ src, size_t n, uint32_t* sink) {
     const size_t stride = (size_t)gridDim.x * 256;
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     uint4 acc = make_uint4(0, 0, 0, 0);
@@ -111,14 +111,17 @@ template <bool NT> __global__ __launch_bounds__(256) void read_kernel(const uint
             return src[j];
         }
     };
-    for (; i + 7 * stride < n; i += 8 * stride) {
-        uint4 v[8];
+    // batches of up to B loads, all issued before the first is used; none past the end
+    for (; i < n; i += B * stride) {
+        uint4 v[B];
 #pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = ld(i + u * stride);
+        for (int u = 0; u < B; u++) {
+            v[u] = make_uint4(0, 0, 0, 0);
+            if (i + u * stride < n) v[u] = ld(i + u * stride);
+        }
 #pragma unroll
-        for (int u = 0; u < 8; u++) { acc.x ^= v[u].x; acc.y ^= v[u].y; acc.z ^= v[u].z; acc.w ^= v[u].w; }
+        for (int u = 0; u < B; u++) { acc.x ^= v[u].x; acc.y ^= v[u].y; acc.z ^= v[u].z; acc.w ^= v[u].w; }
     }
-    for (; i < n; i += stride) { const uint4 v = ld(i); acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w; }
     // a store the compiler cannot rule out and that in practice never happens
     if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9E3779B9u && (acc.x + acc.y) == 0x7F4A7C15u) *sink = acc.z;
 }
@@ -1187,11 +1190,19 @@ int mtq_dispatch_chain(const mtq_dispatch_spec* specs, int n, int repeat, double
     return MTQ_OK;
 }
 
-int mtq_read_kernel(const void* const* srcs, int n_srcs, size_t bytes, int repeat, int workgroups, int nontemporal, void* sink, double* avg_us) {
+int mtq_read_kernel(const void* const* srcs, int n_srcs, size_t bytes, int repeat, int workgroups, int in_flight, int nontemporal, void* sink, double* avg_us) {
     int rc = need_ready();
     if (rc) return rc;
     if (!srcs || n_srcs < 1 || bytes == 0 || bytes % 16 || repeat < 1 || !sink || workgroups < 0 || workgroups > 65536)
         return fail(ERR_BAD_ARG, "read: need buffers, bytes % 16 == 0, repeat >= 1, a 4-byte sink, 0..65536 workgroups");
+    if (in_flight != 0 && in_flight != 1 && in_flight != 2 && in_flight != 4 && in_flight != 8) return fail(ERR_BAD_ARG, "read: loads in flight per thread must be 0 (= 8), 1, 2, 4 or 8");
+    const void* fn = nullptr;
+    switch (in_flight) {
+        case 1: fn = nontemporal ? (const void*)read_kernel<true, 1> : (const void*)read_kernel<false, 1>; break;
+        case 2: fn = nontemporal ? (const void*)read_kernel<true, 2> : (const void*)read_kernel<false, 2>; break;
+        case 4: fn = nontemporal ? (const void*)read_kernel<true, 4> : (const void*)read_kernel<false, 4>; break;
+        default: fn = nontemporal ? (const void*)read_kernel<true, 8> : (const void*)read_kernel<false, 8>; break;
+    }
     for (int i = 0; i < n_srcs; i++)
         if (!srcs[i] || (uintptr_t)srcs[i] % 16) return fail(ERR_BAD_ARG, "read: null or unaligned buffer");
     const size_t n = bytes / 16;
@@ -1205,7 +1216,7 @@ int mtq_read_kernel(const void* const* srcs, int n_srcs, size_t bytes, int repea
             const uint4* s = (const uint4*)srcs[i];
             uint32_t* k = (uint32_t*)sink;
             void* args[] = {&s, (void*)&n, &k};
-            hipError_t e = launch_kernel(nontemporal ? (const void*)read_kernel<true> : (const void*)read_kernel<false>, dim3(wgs), dim3(256), args, 0, lc);
+            hipError_t e = launch_kernel(fn, dim3(wgs), dim3(256), args, 0, lc);
             if (e != hipSuccess) return hip_fail(e, "read kernel launch");
         }
     MTQ_HIP(hipEventRecord(g.ev_stop, g.stream));

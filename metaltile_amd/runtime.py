@@ -237,13 +237,13 @@ class GpuRunner:
         _lib.check(self._lib.mtq_copy_kernel(dst.ptr, src.ptr, int(nbytes), int(repeat), C.byref(us)))
         return us.value
 
-    def read_kernel(self, srcs, nbytes: int, repeat: int = 1, workgroups: int = 0, nontemporal: bool = False) -> float:
+    def read_kernel(self, srcs, nbytes: int, repeat: int = 1, workgroups: int = 0, in_flight: int = 8, nontemporal: bool = False) -> float:
         """Average duration (us) of a launch that only reads `nbytes` of each buffer in `srcs`, enqueued back to back."""
         us = C.c_double(0.0)
         arr = (C.c_void_p * len(srcs))(*[s.ptr for s in srcs])
         sink = GpuBuffer(16)
         try:
-            _lib.check(self._lib.mtq_read_kernel(arr, len(srcs), int(nbytes), int(repeat), int(workgroups), int(bool(nontemporal)),
+            _lib.check(self._lib.mtq_read_kernel(arr, len(srcs), int(nbytes), int(repeat), int(workgroups), int(in_flight), int(bool(nontemporal)),
                                                  sink.ptr, C.byref(us)))
         finally:
             sink.free()
