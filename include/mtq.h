@@ -328,6 +328,41 @@ MTQ_API int mtq_dispatch_chain(const mtq_dispatch_spec *specs, int n, int repeat
  * readings are calibrated against. */
 MTQ_API int mtq_copy_kernel(void *dst, const void *src, size_t bytes, int repeat, double *avg_us);
 
+/* ---- planning without a device ------------------------------------------- */
+
+/* What a call WOULD launch, computed by the same routing and geometry code as the call itself, with no device, no
+ * mtq_init and no allocation: the counterpart of the reference's host-side checks before encoding a dispatch
+ * (crates/metaltile-runtime/src/dispatch/single_dispatch.rs:142-158, buffer_plan.rs:62-77). Returns what the typed
+ * entry point of `op` would return for these arguments as far as shapes decide it (MTQ_OK, MTQ_ERR_BAD_ARG,
+ * MTQ_ERR_SHAPE, MTQ_ERR_UNSUPPORTED) and fills `info` with every kernel launch in order (name, grid, block, dynamic
+ * LDS bytes) and the library-owned scratch bytes the call would need. M is the activation row count (qmv, qmm, qvm),
+ * T the routed row count and E the expert count of the gathers; unused ones are ignored. The compute-unit count
+ * that some geometries depend on is the current device's, or 256 without one. Options set with mtq_set_option apply. */
+enum mtq_op {
+    MTQ_OP_QMV = 0,
+    MTQ_OP_QMM = 1,             /* mt_qmm*: exact dequantisation, any row count */
+    MTQ_OP_QMM_MMA = 2,         /* mt_qmm_mma*: weights rounded to the element type first */
+    MTQ_OP_QVM = 3,
+    MTQ_OP_GATHER_CSR = 4,
+    MTQ_OP_GATHER_INDICES = 5,
+    MTQ_OP_GATHER_SINGLE = 6,
+    MTQ_OP_RMS_NORM_QMV = 7
+};
+#define MTQ_PLAN_MAX_LAUNCHES 8
+typedef struct mtq_plan_launch {
+    char kernel[192];           /* demangled kernel name with its template arguments */
+    uint32_t grid[3];           /* workgroups */
+    uint32_t block[3];          /* threads per workgroup */
+    size_t lds_bytes;           /* dynamic LDS per workgroup */
+} mtq_plan_launch;
+typedef struct mtq_plan_info {
+    int n_launches;             /* launches the call makes; only the first MTQ_PLAN_MAX_LAUNCHES are described */
+    mtq_plan_launch launch[MTQ_PLAN_MAX_LAUNCHES];
+    size_t scratch_bytes;       /* library-owned device scratch the call needs (0 if none) */
+} mtq_plan_info;
+MTQ_API int mtq_plan(int op, int dtype, int bits, uint32_t group_size, uint32_t M, uint32_t N, uint32_t K, uint32_t E,
+                     uint32_t T, mtq_plan_info *info);
+
 /* Measurement aid, no counterpart in the reference: a kernel that only reads. `repeat` passes over the n_srcs
  * buffers of `bytes` bytes each (bytes % 16 == 0) are enqueued back to back on the library's stream, one launch per
  * buffer, `workgroups` (0 = 2048) workgroups of 256 threads with `in_flight` (1, 2, 4, 8; 0 = 8) 16-byte loads in

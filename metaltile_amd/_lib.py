@@ -32,6 +32,17 @@ class MtqDeviceInfo(C.Structure):
     ]
 
 
+PLAN_MAX_LAUNCHES = 8
+
+
+class MtqPlanLaunch(C.Structure):
+    _fields_ = [("kernel", C.c_char * 192), ("grid", C.c_uint32 * 3), ("block", C.c_uint32 * 3), ("lds_bytes", C.c_size_t)]
+
+
+class MtqPlanInfo(C.Structure):
+    _fields_ = [("n_launches", C.c_int), ("launch", MtqPlanLaunch * PLAN_MAX_LAUNCHES), ("scratch_bytes", C.c_size_t)]
+
+
 _u32 = C.c_uint32
 _vp = C.c_void_p
 _u32p = C.POINTER(C.c_uint32)
@@ -74,6 +85,7 @@ SIGNATURES = {
     "mtq_measure": (C.c_int, [C.c_char_p, C.c_int, _bufp, C.c_int, _u32p, C.c_int, _u32p, _u32p, C.c_int, C.c_int, _dblp]),
     "mtq_dispatch_chain": (C.c_int, [C.POINTER(MtqDispatchSpec), C.c_int, C.c_int, _dblp, _dblp, _dblp]),
     "mtq_copy_kernel": (C.c_int, [_vp, _vp, C.c_size_t, C.c_int, _dblp]),
+    "mtq_plan": (C.c_int, [C.c_int, C.c_int, C.c_int, _u32, _u32, _u32, _u32, _u32, _u32, C.POINTER(MtqPlanInfo)]),
     "mtq_read_kernel": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _dblp]),
     "mtq_kernel_supported": (C.c_int, [C.c_char_p]),
     "mtq_kernel_count": (C.c_int, []),

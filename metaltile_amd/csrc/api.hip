@@ -5,6 +5,8 @@
 #include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
+#include <cxxabi.h>
+#include <dlfcn.h>
 #include <time.h>
 
 #include <cstdio>
@@ -31,8 +33,54 @@ int hip_fail(hipError_t e, const char* what) {
     return e == hipErrorNoDevice || e == hipErrorInvalidDevice ? ERR_NO_DEVICE : ERR_HIP;
 }
 
+// What mtq_plan records instead of launching.
+struct PlanRecorder {
+    bool on = false;
+    int n = 0;                 // launches seen (may exceed the slots of the caller's struct)
+    size_t scratch = 0;        // most library-owned scratch any step asked for
+    mtq_plan_info* out = nullptr;
+};
+static PlanRecorder g_plan;
+bool planning() { return g_plan.on; }
+void plan_note_scratch(size_t bytes) {
+    if (bytes > g_plan.scratch) g_plan.scratch = bytes;
+}
+
+hipError_t set_max_dynamic_lds(const void* fn, size_t bytes) {
+    if (g_plan.on) return hipSuccess;
+    return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+// Name of a kernel from the address of its host-side stub, without asking the runtime (which needs a device).
+static void kernel_name_of(const void* fn, char* out, size_t cap) {
+    Dl_info di;
+    if (dladdr(fn, &di) && di.dli_sname) {
+        int st = 0;
+        char* dm = abi::__cxa_demangle(di.dli_sname, nullptr, nullptr, &st);
+        std::string s = st == 0 && dm ? dm : di.dli_sname;
+        free(dm);
+        const std::string stub = "__device_stub__";
+        const size_t k = s.find(stub);
+        if (k != std::string::npos) s.erase(k, stub.size());
+        snprintf(out, cap, "%s", s.c_str());
+    } else {
+        snprintf(out, cap, "kernel@%p", fn);
+    }
+}
+
 hipError_t launch_kernel(const void* fn, dim3 grid, dim3 block, void** args, size_t shmem,
                          const LaunchCtx& lc) {
+    if (g_plan.on) {
+        if (g_plan.out && g_plan.n < MTQ_PLAN_MAX_LAUNCHES) {
+            mtq_plan_launch& l = g_plan.out->launch[g_plan.n];
+            kernel_name_of(fn, l.kernel, sizeof(l.kernel));
+            l.grid[0] = grid.x; l.grid[1] = grid.y; l.grid[2] = grid.z;
+            l.block[0] = block.x; l.block[1] = block.y; l.block[2] = block.z;
+            l.lds_bytes = shmem;
+        }
+        g_plan.n++;
+        return hipSuccess;
+    }
     if (lc.start || lc.stop)
         return hipExtLaunchKernel(fn, grid, block, args, shmem, lc.stream, lc.start, lc.stop, 0);
     return hipLaunchKernel(fn, grid, block, args, shmem, lc.stream);
@@ -239,6 +287,10 @@ static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s,
 
 // Library-owned device scratch (normalised rows, qvm partial sums): grown on demand, never shrunk.
 static int ensure_scratch(size_t need) {
+    if (g_plan.on) {  // mtq_plan has put a stand-in address into scratch_buf; nothing is allocated
+        plan_note_scratch(need);
+        return ERR_OK;
+    }
     if (g.scratch_bytes >= need) return ERR_OK;
     if (g.scratch_buf) {
         MTQ_HIP(hipStreamSynchronize(g.stream));  // earlier launches may still use the old buffer
@@ -1225,6 +1277,41 @@ int mtq_read_kernel(const void* const* srcs, int n_srcs, size_t bytes, int repea
     MTQ_HIP(hipEventElapsedTime(&ms, g.ev_start, g.ev_stop));
     if (avg_us) *avg_us = (double)ms * 1000.0 / ((double)repeat * n_srcs);
     return MTQ_OK;
+}
+
+int mtq_plan(int op, int dtype, int bits, uint32_t group_size, uint32_t M, uint32_t N, uint32_t K, uint32_t E, uint32_t T,
+             mtq_plan_info* info) {
+    if (!info) return fail(ERR_BAD_ARG, "plan: info must not be null");
+    memset(info, 0, sizeof(*info));
+    if (op < MTQ_OP_QMV || op > MTQ_OP_RMS_NORM_QMV) return fail(ERR_BAD_ARG, "plan: unknown op");
+    // Stand-in operand addresses: distinct, 256-byte aligned, never dereferenced (no launch happens).
+    auto at = [](int i) { return (void*)(uintptr_t)(0x100000000ull + ((uint64_t)i << 36)); };
+    const void *w = at(1), *s = at(2), *b = at(3), *x = at(4), *aux = at(6), *aux2 = at(7);
+    void* out = at(5);
+    void* const real_scratch = g.scratch_buf;
+    const size_t real_held = g.scratch_held;
+    g.scratch_buf = at(8);
+    g_plan = PlanRecorder{};
+    g_plan.on = true;
+    g_plan.out = info;
+    LaunchCtx lc;  // null stream, no events: nothing is enqueued
+    int rc;
+    switch (op) {
+        case MTQ_OP_QMV: rc = op_qmv(dtype, bits, group_size, w, s, b, x, out, M, N, K, lc); break;
+        case MTQ_OP_QMM: rc = op_qmm(dtype, bits, group_size, w, s, b, x, out, M, N, K, false, lc); break;
+        case MTQ_OP_QMM_MMA: rc = op_qmm(dtype, bits, group_size, w, s, b, x, out, M, N, K, true, lc); break;
+        case MTQ_OP_QVM: rc = op_qvm(dtype, bits, group_size, w, s, b, x, out, M, N, K, lc); break;
+        case MTQ_OP_GATHER_CSR: rc = op_gather(GATHER_CSR, dtype, bits, group_size, x, w, s, b, (const uint32_t*)aux, out, T, N, K, E, lc); break;
+        case MTQ_OP_GATHER_INDICES: rc = op_gather(GATHER_INDICES, dtype, bits, group_size, x, w, s, b, (const uint32_t*)aux, out, T, N, K, E, lc); break;
+        case MTQ_OP_GATHER_SINGLE: rc = op_gather(GATHER_SINGLE, dtype, bits, group_size, x, w, s, b, (const uint32_t*)aux, out, 1, N, K, E, lc); break;
+        default: rc = op_rms_norm_qmv(dtype, bits, group_size, x, aux, w, s, b, out, (const float*)aux2, N, K, lc); break;
+    }
+    info->n_launches = g_plan.n;
+    info->scratch_bytes = g_plan.scratch;
+    g_plan = PlanRecorder{};
+    g.scratch_buf = real_scratch;
+    g.scratch_held = real_held;
+    return rc;
 }
 
 int mtq_copy_kernel(void* dst, const void* src, size_t bytes, int repeat, double* avg_us) {

@@ -259,7 +259,7 @@ int launch_moe_sort(const uint32_t* indices, uint32_t n_tokens, uint32_t k, uint
         SortArgs a{indices, sort_token_idx, inv_perm, expert_offsets, (uint32_t)n64, 0, k, n_experts};
         const size_t shmem = (size_t)17 * n_experts * 4;
         if (shmem > 48 * 1024) {
-            hipError_t e = hipFuncSetAttribute((const void*)moe_count_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+            hipError_t e = set_max_dynamic_lds((const void*)moe_count_sort_kernel, (size_t)shmem);
             if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
         }
         void* args[] = {&a};
@@ -273,7 +273,7 @@ int launch_moe_sort(const uint32_t* indices, uint32_t n_tokens, uint32_t k, uint
     SortArgs a{indices, sort_token_idx, inv_perm, expert_offsets, (uint32_t)n64, n_pad, k, n_experts};
     const size_t shmem = (size_t)n_pad * 4;
     if (shmem > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)moe_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        hipError_t e = set_max_dynamic_lds((const void*)moe_sort_kernel, (size_t)shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     }
     void* args[] = {&a};

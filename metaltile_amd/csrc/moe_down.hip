@@ -165,7 +165,7 @@ int launch_moe_down_swiglu(int dtype, uint32_t group_size, uint32_t n_slots, con
         default: return fail(ERR_BAD_ARG, "unknown dtype");
     }
     if (shmem > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        hipError_t e = set_max_dynamic_lds(fn, (size_t)shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     }
     void* args[] = {&a};

@@ -43,6 +43,13 @@ struct LaunchCtx {
 
 hipError_t launch_kernel(const void* fn, dim3 grid, dim3 block, void** args, size_t shmem,
                          const LaunchCtx& lc);
+// Raises a kernel's dynamic LDS limit (needed above 48 KB).
+hipError_t set_max_dynamic_lds(const void* fn, size_t bytes);
+// Planning (mtq_plan): the routing and geometry code runs as for a real call, but launch_kernel and
+// set_max_dynamic_lds only record what they are given and nothing touches a device. Code that would allocate
+// device scratch of its own asks planning() first and reports the bytes with plan_note_scratch instead.
+bool planning();
+void plan_note_scratch(size_t bytes);
 
 // How the x/out rows of a GEMV-family launch are selected.
 enum GatherMode : int {

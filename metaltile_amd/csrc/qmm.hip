@@ -251,6 +251,10 @@ struct QmmScratch {
 static QmmScratch g_scratch;
 
 static int ensure_scratch(size_t partial_bytes, size_t tiles, hipStream_t stream) {
+    if (planning()) {
+        plan_note_scratch(partial_bytes + (tiles < 1024 ? 1024 : tiles) * sizeof(uint32_t));
+        return ERR_OK;
+    }
     if (g_scratch.partial_bytes < partial_bytes) {
         if (g_scratch.partials) {
             MTQ_HIP(hipStreamSynchronize(stream));
@@ -283,7 +287,7 @@ template <int DT> static int launch_qmm_dt(QmmKArgs& a, int bits, const LaunchCt
         case 4: fn = (const void*)qmm_kernel<DT, 4>; break;
         default: fn = (const void*)qmm_kernel<DT, 8>; break;
     }
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS);
+    hipError_t e = set_max_dynamic_lds(fn, (size_t)QLDS);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     void* args[] = {&a};
     e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles * a.splits), dim3(256), args, QLDS, lc);

@@ -66,7 +66,7 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
     if (!grouped && a.ksplit <= 1 && dma_fits(bits, a.m_tile_rows, kgroups, a.K, a.gpr)) {
         fn = qmm_dma_pick(DT, a.m_tile_rows);
         const size_t shmem = qmm_dma_lds_bytes(a.m_tile_rows, a.gpr);
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        hipError_t e = set_max_dynamic_lds(fn, (size_t)shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
         void* args[] = {&a};
         e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles), dim3(512), args, shmem, lc);
@@ -119,7 +119,7 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
 #undef QD_G1
 #undef QD_G
     }
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    hipError_t e = set_max_dynamic_lds(fn, (size_t)shmem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     void* args[] = {&a};
     if (a.ksplit > 1 && !grouped) {

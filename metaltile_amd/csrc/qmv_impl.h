@@ -615,8 +615,7 @@ template <int DT, int BITS, int MB, int RT, int MODE, int MAXT, int SBI>
 static int qmv_launch_inst(QmvKArgs& a, const QmvGeom& g, const LaunchCtx& lc) {
     auto fn = qmv_kernel<DT, BITS, MB, RT, MODE, MAXT, SBI>;
     if (g.shmem > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)g.shmem);
+        hipError_t e = set_max_dynamic_lds((const void*)fn, (size_t)g.shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     }
     void* args[] = {&a};
@@ -678,7 +677,7 @@ static int qmv_stream_launch_sbi(QmvSArgs& a, const QmvSGeom& g, const LaunchCtx
         default: fn = (const void*)qmv_stream_kernel<DT, BITS, MB, D, MODE, MAXT, 4>; break;
     }
     if (g.shmem > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.shmem);
+        hipError_t e = set_max_dynamic_lds(fn, (size_t)g.shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     }
     void* args[] = {&a};
@@ -698,7 +697,7 @@ static int qmv_stream_norm_launch_d(QmvSArgs& a, const QmvSGeom& g, const Launch
         default: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 4, true>; break;
     }
     if (g.shmem > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.shmem);
+        hipError_t e = set_max_dynamic_lds(fn, (size_t)g.shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     }
     void* args[] = {&a};

@@ -547,7 +547,7 @@ int qmv_mfma_launch_one(QmvMArgs& a, const QmvMGeom& g, const LaunchCtx& lc) {
     const void* fn = a.nrb > 1 ? (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT, true>
                                : (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT, false>;
     if (g.shmem > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.shmem);
+        hipError_t e = set_max_dynamic_lds(fn, (size_t)g.shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     }
     void* args[] = {&a};

@@ -130,3 +130,17 @@ def timed(fn, *args, **kw) -> float:
 
 def sync():
     _lib.check(_ensure_init().mtq_sync())
+
+
+PLAN_OPS = {"qmv": 0, "qmm": 1, "qmm_mma": 2, "qvm": 3, "gather_csr": 4, "gather_indices": 5, "gather_single": 6, "rms_norm_qmv": 7}
+
+
+def plan(op: str, dtype, bits: int, group_size: int, M: int = 1, N: int = 0, K: int = 0, E: int = 1, T: int = 0):
+    """What the call would launch, without a device (mtq_plan): (rc, [(kernel, grid, block, lds_bytes)], scratch_bytes).
+    rc is the code the typed entry point would return as far as shapes decide it; no exception is raised."""
+    lib = _lib.load()
+    info = _lib.MtqPlanInfo()
+    rc = lib.mtq_plan(PLAN_OPS[op], int(dtype), bits, group_size, M, N, K, E, T, info)
+    launches = [(l.kernel.decode(), tuple(l.grid), tuple(l.block), int(l.lds_bytes))
+                for l in info.launch[:min(info.n_launches, _lib.PLAN_MAX_LAUNCHES)]]
+    return rc, launches, int(info.scratch_bytes), info.n_launches

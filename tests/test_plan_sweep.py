@@ -1,0 +1,142 @@
+"""Routing and launch geometry without a GPU: mtq_plan runs the same code as the typed entry points and records
+what they would launch. A sweep over a few thousand shapes checks every recorded launch against the limits of the
+part (1024 threads per workgroup, 160 KB of LDS, grid dimensions), that every valid shape is served (the generic
+kernel stands behind every specialised one), that argument validation is reached without a device, and pins the
+kernels the benchmark configurations are routed to.
+
+Counterpart of the reference's host-side checks before a dispatch is encoded
+(crates/metaltile-runtime/src/dispatch/single_dispatch.rs:142-158, buffer_plan.rs:62-77).
+"""
+import itertools
+
+import pytest
+
+from metaltile_amd import DType, ops
+
+OK, BAD_ARG, SHAPE, UNSUPPORTED = 0, -2, -3, -7
+LDS_MAX = 160 * 1024
+
+
+def check_launches(tag, launches, n_launches, rows=1):
+    # exact-dequant batches run as passes of up to 4 (f32 dot kernels) or 8 / 16 rows over the weights
+    assert 1 <= n_launches <= max(8, rows // 4 + 2), f"{tag}: {n_launches} launches"
+    assert len(launches) == min(n_launches, 8)
+    for kernel, grid, block, lds in launches:
+        threads = block[0] * block[1] * block[2]
+        assert kernel.startswith(("void mtq::", "mtq::")), f"{tag}: kernel name {kernel!r}"
+        assert 1 <= threads <= 1024 and threads % 64 == 0, f"{tag}: {kernel} block {block}"
+        assert 1 <= grid[0] < 2 ** 31 and 1 <= grid[1] <= 65535 and 1 <= grid[2] <= 65535, f"{tag}: {kernel} grid {grid}"
+        assert grid[0] * grid[1] * grid[2] < 2 ** 32, f"{tag}: {kernel} grid {grid}"
+        assert lds <= LDS_MAX, f"{tag}: {kernel} asks for {lds} B of LDS"
+
+
+def valid(bits, G, N, K):
+    return N > 0 and K > 0 and G > 0 and K % G == 0 and (K * bits) % 32 == 0
+
+
+# row lengths of the models named in the benchmark configurations and their neighbours, and awkward ones
+KS = [64, 96, 128, 320, 576, 768, 1024, 1152, 1408, 2048, 2816, 3584, 4096, 5120, 6144, 8192, 11008, 13824, 14336, 18944, 28672]
+NS = [1, 7, 64, 100, 131, 333, 768, 1000, 2048, 4096, 5120, 14336, 28672, 128256]
+MS = [1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 33, 64, 65, 100, 128, 256, 300, 512, 640, 1024, 1536, 2048, 3000, 4096]
+
+
+def test_qmv_qmm_sweep():
+    """Every valid (dtype, bits, group, M, N, K) is served by some kernel within the part's limits."""
+    n = 0
+    for dt in (DType.F32, DType.F16, DType.BF16):
+        for bits, G in itertools.product((2, 3, 4, 5, 6, 8), (32, 64, 128)):
+            for K in KS:
+                if not valid(bits, G, 1, K):
+                    continue
+                for N in (NS if K in (4096, 14336, 576, 11008) else (100, 4096, 14336)):
+                    for M in (MS if (K, N) in ((4096, 4096), (14336, 4096), (4096, 14336), (11008, 4096)) else (1, 4, 16, 300)):
+                        if M * K * 4 >= 2 ** 32 or M * N * 4 >= 2 ** 32:
+                            continue
+                        for op in ("qmv", "qmm", "qmm_mma") if M > 1 else ("qmv",):
+                            if op == "qmv" and M > 8:
+                                continue
+                            tag = f"{op} {dt.name} b{bits} g{G} M{M} N{N} K{K}"
+                            rc, launches, scratch, nl = ops.plan(op, dt, bits, G, M, N, K)
+                            assert rc == OK, f"{tag}: rc {rc}"
+                            check_launches(tag, launches, nl, M)
+                            assert scratch < 2 ** 34, tag
+                            n += 1
+    assert n > 3000
+
+
+def test_gather_and_fused_sweep():
+    n = 0
+    for dt in (DType.F16, DType.BF16, DType.F32):
+        for bits, G in ((4, 64), (8, 64), (2, 32), (3, 64), (6, 128)):
+            for N, K in ((14336, 4096), (4096, 14336), (768, 2048), (2048, 768), (1408, 2048), (100, 576)):
+                if not valid(bits, G, N, K):
+                    continue
+                for E, T in ((8, 32), (8, 2048), (128, 8192), (64, 1), (2047, 4096), (2048, 64), (1, 300), (8, 0)):
+                    for op in ("gather_csr", "gather_indices"):
+                        tag = f"{op} {dt.name} b{bits} g{G} N{N} K{K} E{E} T{T}"
+                        rc, launches, scratch, nl = ops.plan(op, dt, bits, G, 1, N, K, E, T)
+                        assert rc == OK, f"{tag}: rc {rc}"
+                        if T:
+                            check_launches(tag, launches, nl)
+                        else:
+                            assert nl == 0
+                        n += 1
+                rc, launches, _, nl = ops.plan("gather_single", dt, bits, G, 1, N, K, 8)
+                assert rc == OK
+                check_launches(f"gather_single {dt.name} b{bits} N{N} K{K}", launches, nl)
+                rc, launches, _, nl = ops.plan("rms_norm_qmv", dt, bits, G, 1, N, K)
+                assert rc == OK
+                check_launches(f"rms_norm_qmv {dt.name} b{bits} N{N} K{K}", launches, nl)
+                if (N * bits) % 32 == 0:
+                    for M in (1, 2, 8):
+                        rc, launches, scratch, nl = ops.plan("qvm", dt, bits, G, M, N, K)
+                        assert rc == OK
+                        check_launches(f"qvm {dt.name} b{bits} M{M} N{N} K{K}", launches, nl)
+                n += 3
+    assert n > 500
+
+
+def test_validation_without_a_device():
+    P = lambda op, *a, **k: ops.plan(op, *a, **k)[0]
+    assert P("qmv", 7, 4, 64, 1, 4096, 4096) == BAD_ARG          # no such dtype
+    assert P("qmv", DType.BF16, 9, 64, 1, 4096, 4096) == BAD_ARG  # bits
+    assert P("qmv", DType.BF16, 1, 64, 1, 4096, 4096) == BAD_ARG
+    assert P("qmv", DType.BF16, 4, 64, 1, 0, 4096) == SHAPE       # N == 0
+    assert P("qmv", DType.BF16, 4, 64, 1, 4096, 0) == SHAPE
+    assert P("qmv", DType.BF16, 4, 0, 1, 4096, 4096) == SHAPE     # group size
+    assert P("qmv", DType.BF16, 4, 96, 1, 4096, 4096) == SHAPE    # K % G
+    assert P("qmm", DType.BF16, 3, 4, 16, 64, 4) == SHAPE         # K * bits % 32
+    assert P("gather_csr", DType.BF16, 4, 64, 1, 4096, 4096, 0, 8) == SHAPE   # no experts
+    assert P("qvm", DType.BF16, 3, 64, 1, 100, 4096) == SHAPE     # N * bits % 32
+    assert P("qmv", DType.BF16, 4, 64, 0, 4096, 4096) == OK       # no rows: nothing to do
+    assert ops.plan("qmv", DType.BF16, 4, 64, 0, 4096, 4096)[3] == 0
+
+
+def test_benchmark_configurations_are_routed_as_documented():
+    def kernels(op, *a, **k):
+        rc, launches, _, _ = ops.plan(op, *a, **k)
+        assert rc == OK
+        return [l[0] for l in launches], launches
+
+    ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 14336, 4096)
+    assert "qmv_stream_kernel<2, 4, 1," in ks[0] and ls[0][1][0] * 8 == 14336   # 8 rows per workgroup
+    ks, _ = kernels("qmv", DType.BF16, 4, 64, 1, 4096, 14336)
+    assert "qmv_stream_kernel<2, 4, 1," in ks[0]
+    ks, _ = kernels("qmv", DType.F32, 4, 64, 1, 4096, 4096)
+    assert "qmv_stream_kernel<0, 4" in ks[0] or "qmv_kernel<0, 4" in ks[0]
+    for M, mb in ((512, 2), (1024, 4), (2048, 8)):     # 64-, 128-, 256-row load-to-LDS tiles
+        ks, ls = kernels("qmm_mma", DType.BF16, 4, 64, M, 4096, 4096)
+        assert f"qmm_dma_kernel<2, {mb}, 2, 8," in ks[0], ks
+        assert ls[0][1][0] == 256 and ls[0][2][0] == 512
+    ks, ls = kernels("qmm_mma", DType.BF16, 4, 64, 32, 4096, 4096)
+    assert "qmm_direct_kernel<2, 4, 2, 1," in ks[0]    # 32-row tiles
+    ks, _ = kernels("qmm_mma", DType.BF16, 8, 64, 512, 4096, 4096)
+    assert "qmm_direct_kernel<2, 8," in ks[0]          # other code widths stay on the register-staged tiles
+    ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 32)
+    assert "qmv_mfma_kernel<2, 4," in ks[0]
+    ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 4096, 4096, 8, 2048)
+    assert "moe_count_sort_kernel" in ks[0] and "gather_tiles_kernel" in ks[1] and "qmm_direct_kernel" in ks[2]
+    for bits, M in itertools.product((2, 4, 8), (1, 4)):   # the sweep configuration's cells
+        for G in (32, 64, 128):
+            ks, _ = kernels("qmv", DType.F16, bits, G, M, 8192, 8192)
+            assert "generic" not in ks[0], (bits, G, M, ks)
