@@ -48,7 +48,10 @@ uint32_t window_pairs(uint32_t kp_count, uint32_t spp, uint32_t cpc, uint32_t lo
 
 int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     if (p.dtype != DT_F16 && p.dtype != DT_BF16) return fail(ERR_UNSUPPORTED, "mfma qmv: f16/bf16 only");
-    const bool odd = p.bits == 3 || p.bits == 5 || p.bits == 6;
+    // 2-bit codes in groups of 32: a 16-byte lane chunk (64 codes) would straddle two groups, so the lanes take
+    // 8 bytes (32 codes) each, like the widths whose chunk is 32 codes of the bit stream
+    const bool half2 = p.bits == 2 && p.group_size == 32;
+    const bool odd = p.bits == 3 || p.bits == 5 || p.bits == 6 || half2;
     if (!(p.bits == 2 || p.bits == 4 || p.bits == 8 || odd))
         return fail(ERR_UNSUPPORTED, "mfma qmv: bits");
     if (p.N == 0 || p.K == 0) return fail(ERR_UNSUPPORTED, "mfma qmv: empty");
@@ -240,8 +243,8 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     g.shmem = lds_bytes(R, nchp * cpc, nch, gpr, rows_wg, KP * RBW, gpw, KP, list_cap);
     g.grid = dim3((p.N + rows_wg - 1) / rows_wg, gather ? p.E : 1, 1);
     if (odd)
-        return p.dtype == DT_F16 ? qmv_mfma_launch_dtype_odd<DT_F16>(a, p.bits, p.gather, g, lc)
-                                 : qmv_mfma_launch_dtype_odd<DT_BF16>(a, p.bits, p.gather, g, lc);
+        return p.dtype == DT_F16 ? qmv_mfma_launch_dtype_odd<DT_F16>(a, half2 ? 22 : p.bits, p.gather, g, lc)
+                                 : qmv_mfma_launch_dtype_odd<DT_BF16>(a, half2 ? 22 : p.bits, p.gather, g, lc);
     switch (p.dtype) {
         case DT_F16: return qmv_mfma_launch_dtype<DT_F16>(a, p.bits, p.gather, g, lc);
         default: return qmv_mfma_launch_dtype<DT_BF16>(a, p.bits, p.gather, g, lc);

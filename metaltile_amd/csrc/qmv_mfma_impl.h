@@ -107,13 +107,17 @@ template <int DT> __device__ __forceinline__ m_f32x4 mfma4(m_u32x2 a, m_u32x2 b,
 // two 4-bit planes (PLANES = 2), high nibbles first; the accumulator is scaled by
 // 16 between the planes, so sum = 16*sum(hi*x) + sum(lo*x) and the offset to
 // remove is MAGIC*(16+1) per activation.
+// BITS = 22 stands for 2-bit codes taken 32 at a time (8 bytes per lane instead of 16): the form for groups of 32
+// codes, which a 64-code chunk would straddle.
 template <int DT, int BITS> struct MfmaCodec {
-    static constexpr bool kPow2 = (32 % BITS) == 0;
+    static constexpr bool kHalf2 = BITS == 22;
+    static constexpr int CBITS = kHalf2 ? 2 : BITS;       // bits per code
+    static constexpr bool kPow2 = (32 % CBITS) == 0;
     static constexpr int PLANES = (DT == DT_BF16 && BITS == 8) ? 2 : 1;
     static constexpr float kMagic = (DT == DT_BF16 ? 128.0f : 1024.0f) * (PLANES == 2 ? 17.0f : 1.0f);
-    static constexpr int PF = kPow2 ? 32 / BITS : 0;     // codes per dword (power-of-two widths)
-    static constexpr int NWD = kPow2 ? 4 : BITS;
-    static constexpr int CPC = kPow2 ? 4 * PF : 32;
+    static constexpr int PF = kPow2 ? 32 / CBITS : 0;    // codes per dword (power-of-two widths)
+    static constexpr int NWD = kHalf2 ? 2 : kPow2 ? 4 : BITS;
+    static constexpr int CPC = kPow2 ? NWD * PF : 32;
     static constexpr int CB = NWD * 4;                    // chunk bytes
     __host__ __device__ static constexpr int src(int o) {
         if (!kPow2) return o;
@@ -132,11 +136,11 @@ template <int DT, int BITS> struct MfmaCodec {
                     pw[CPC / 2 + wi * 2 + j] = ((w[wi] >> (8 * j)) & 0x000F000Fu) | kor;
                 }
         } else if constexpr (kPow2) {
-            constexpr uint32_t MASK = ((1u << BITS) - 1u) * 0x00010001u;
+            constexpr uint32_t MASK = ((1u << CBITS) - 1u) * 0x00010001u;
 #pragma unroll
-            for (int wi = 0; wi < 4; wi++)
+            for (int wi = 0; wi < NWD; wi++)
 #pragma unroll
-                for (int j = 0; j < PF / 2; j++) pw[wi * (PF / 2) + j] = ((w[wi] >> (BITS * j)) & MASK) | kor;
+                for (int j = 0; j < PF / 2; j++) pw[wi * (PF / 2) + j] = ((w[wi] >> (CBITS * j)) & MASK) | kor;
         } else {
             constexpr uint32_t M1 = (1u << BITS) - 1u;
 #pragma unroll
@@ -156,7 +160,10 @@ template <int DT, int BITS> struct MfmaCodec {
         typedef uint32_t v4 __attribute__((ext_vector_type(4), aligned(4)));
         typedef uint32_t v3 __attribute__((ext_vector_type(3), aligned(4)));
         typedef uint32_t v2 __attribute__((ext_vector_type(2), aligned(4)));
-        if constexpr (NWD == 3) {
+        if constexpr (NWD == 2) {
+            const v2 t = __builtin_nontemporal_load((const v2*)p);
+            w[0] = t.x; w[1] = t.y;
+        } else if constexpr (NWD == 3) {
             const v3 t = __builtin_nontemporal_load((const v3*)p);
             w[0] = t.x; w[1] = t.y; w[2] = t.z;
         } else {
@@ -601,6 +608,7 @@ template <int DT> int qmv_mfma_launch_dtype_odd(QmvMArgs& a, int bits, int mode,
         case 3: return qmv_mfma_launch_mode<DT, 3>(a, mode, g, lc);
         case 5: return qmv_mfma_launch_mode<DT, 5>(a, mode, g, lc);
         case 6: return qmv_mfma_launch_mode<DT, 6>(a, mode, g, lc);
+        case 22: return qmv_mfma_launch_mode<DT, 22>(a, mode, g, lc);   // 2-bit codes in 8-byte chunks (groups of 32)
         default: return fail(ERR_UNSUPPORTED, "mfma qmv: code width");
     }
 }

@@ -135,3 +135,40 @@ def test_gather_rows_that_are_not_whole_steps(oracle, K):
         out.free(); r.free()
     for buf in (w, s, b, x):
         buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.F16, DType.BF16], ids=lambda d: d.name)
+@pytest.mark.parametrize("M,N,K", [(2, 100, 1024), (3, 64, 2080), (4, 256, 8192), (8, 40, 1024), (6, 33, 544)])
+def test_2bit_groups_of_32_on_the_matrix_core_kernel(oracle, M, N, K, dt):
+    """2-bit codes with groups of 32: a 16-byte lane chunk holds 64 codes (two groups), so the matrix-core
+    kernel takes them 32 codes (8 bytes) per lane; rows that are not whole 512-code steps included. Batches
+    and both gather views against the f64-accumulated oracle, 1e-2 as above."""
+    bits, G = 2, 32
+    c = make_case(900 + M + K, dt, bits, G, M, N, K, bias_rule="midpoint")
+    print(f"[case] qmv {dt.name} b2 g32 M{M} N{N} K{K}", flush=True)
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
+    ops.qmv(dt, bits, G, w, s, b, x, out, M, N, K)
+    got = unpack_f32(out.read_bytes(), dt)
+    assert rel_err(got, _expected(oracle, c)) <= TOL[dt]
+    for buf in (w, s, b, x, out):
+        buf.free()
+    # the same rows routed to 3 experts (one empty)
+    E = 3
+    counts = [M - 1, 0, 1]
+    cg = make_case(950 + M + K, dt, bits, G, M, N, K, E=E, bias_rule="midpoint")
+    indices = np.repeat(np.arange(E), counts).astype("<u4")
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype("<u4")
+    exp = oracle.gather_qmm(cg.x_f, cg.w, cg.scales_f, cg.biases_f, M, K, N, E, bits, G, indices=indices, f64=True, threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(cg.w.tobytes()), GpuBuffer.from_bytes(cg.scales_bytes),
+                  GpuBuffer.from_bytes(cg.biases_bytes), GpuBuffer.from_bytes(cg.x_bytes))
+    for view, route, fn in (("csr", offsets, ops.gather_qmv_csr), ("indices", indices, ops.gather_qmv_indices)):
+        r = GpuBuffer.from_bytes(route.tobytes())
+        out = GpuBuffer(M * N * dt.size_bytes)
+        fn(dt, bits, G, x, w, s, b, r, out, M, N, K, E)
+        assert rel_err(unpack_f32(out.read_bytes(), dt), exp) <= TOL[dt], view
+        out.free(); r.free()
+    for buf in (w, s, b, x):
+        buf.free()
