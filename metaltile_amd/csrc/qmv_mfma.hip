@@ -141,7 +141,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     const uint32_t list_cap = p.gather == GATHER_INDICES ? p.T : 0;
     uint32_t RBW = 1, nrb = 1;
     for (;; s /= 2) {
-        const uint32_t maxt = (s >= 4 || (s >= 2 && p.bits != 4 && p.bits != 8)) ? 512u : 1024u;
+        const uint32_t maxt = s >= 2 ? 512u : 1024u;
         if (64u * KP > maxt) {
             if (s > 1) continue;
             return fail(ERR_UNSUPPORTED, "mfma qmv: too many K parts");

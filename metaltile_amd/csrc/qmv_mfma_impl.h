@@ -434,8 +434,11 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         const uint32_t xl_set = (uint32_t)NP * a.nchp * MP * 16u;  // bytes from one row set to the next
         const uint32_t part_g0 = (kp * a.spp * 16u * (uint32_t)CPC) >> a.log2g;  // this wave's K part: whole groups
         const uint32_t part_ng = min(a.gpr, ((kp * a.spp + spp_eff) * 16u * (uint32_t)CPC) >> a.log2g) - part_g0;
-        auto turn = [&](auto issue_tag) {
+        // SE: row sets the pass works on. A pass of a gather whose expert has at most MP rows left skips the
+        // second set's operand reads, MFMAs and scale terms (its rows are not live and are never stored).
+        auto turn = [&](auto issue_tag, auto sets_tag) {
             constexpr bool ISSUE = decltype(issue_tag)::value;
+            constexpr int SE = decltype(sets_tag)::value;
             const uint32_t row_local = (rb * a.RBW + rbw) * 4u + r;
             {
                 const bool wrap = sg0 + D >= sppD;
@@ -449,7 +452,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                     // operands from LDS
                     m_u32x4 av[S][NP];
 #pragma unroll
-                    for (int s = 0; s < S; s++) {
+                    for (int s = 0; s < SE; s++) {
 #pragma unroll
                         for (int p = 0; p < NP; p++)
                             av[s][p] = *(const m_u32x4*)(xl_lane + (sgc * ((uint32_t)NP * 16u * MP * 16u) + (uint32_t)s * xl_set) + p * (16 * MP * 16));
@@ -467,7 +470,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                         for (int m = 0; m < CPC / 4; m++) {  // MFMA m of the chunk: codes 4m .. 4m+3 of its operand sequence
                             const m_u32x2 b = {pw[pl * (CPC / 2) + 2 * m], pw[pl * (CPC / 2) + 2 * m + 1]};
 #pragma unroll
-                            for (int s = 0; s < S; s++) {
+                            for (int s = 0; s < SE; s++) {
                                 const m_u32x4 piece = av[s][m / 2];
                                 const m_u32x2 aop = (m & 1) ? m_u32x2{piece.z, piece.w} : m_u32x2{piece.x, piece.y};
                                 const m_f32x4 zero = {0.f, 0.f, 0.f, 0.f};
@@ -476,13 +479,13 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                         }
                         if (pl + 1 < Codec::PLANES) {
 #pragma unroll
-                            for (int s = 0; s < S; s++)
+                            for (int s = 0; s < SE; s++)
 #pragma unroll
                                 for (int i = 0; i < MP; i++) acc[s][i] *= 16.0f;  // only the live rows are read later
                         }
                     }
 #pragma unroll
-                    for (int s = 0; s < S; s++)
+                    for (int s = 0; s < SE; s++)
 #pragma unroll
                         for (int i = 0; i < MP; i++) {
                             tot[s][i] = fmaf(sb.x, acc[s][i], tot[s][i]);
@@ -494,7 +497,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                         const uint32_t g = part_g0 + gi;
                         const float bq = SB[sb_row + g].y;
 #pragma unroll
-                        for (int s = 0; s < S; s++) {
+                        for (int s = 0; s < SE; s++) {
                             const float* xg = XG + ((size_t)s * a.gpr + g) * MP;
 #pragma unroll
                             for (int i = 0; i < MP; i++) tot[s][i] = fmaf(bq, xg[i], tot[s][i]);
@@ -502,7 +505,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                     }
                     // lanes of one weight row (same r, all q) add up: q spans lane bits 2..5
 #pragma unroll
-                    for (int s = 0; s < S; s++)
+                    for (int s = 0; s < SE; s++)
 #pragma unroll
                         for (int i = 0; i < MP; i++) {
                             float v = tot[s][i];
@@ -527,8 +530,13 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
             }
         };
         const uint32_t n_turns = a.nrb * (sppD / D);
-        for (uint32_t it = 0; it + 1 < n_turns; it++) turn(std::true_type{});
-        turn(std::false_type{});
+        if (S > 1 && live <= (uint32_t)MP) {
+            for (uint32_t it = 0; it + 1 < n_turns; it++) turn(std::true_type{}, std::integral_constant<int, 1>{});
+            turn(std::false_type{}, std::integral_constant<int, 1>{});
+        } else {
+            for (uint32_t it = 0; it + 1 < n_turns; it++) turn(std::true_type{}, std::integral_constant<int, S>{});
+            turn(std::false_type{}, std::integral_constant<int, S>{});
+        }
         __syncthreads();
 
         // ---- add the K parts and store ----------------------------------------
@@ -549,10 +557,14 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
 
 template <int DT, int BITS, int MP, int S, int MODE>
 int qmv_mfma_launch_one(QmvMArgs& a, const QmvMGeom& g, const LaunchCtx& lc) {
-    constexpr int MAXT = (S >= 4 || (S >= 2 && BITS != 4 && BITS != 8)) ? 512 : 1024;
+    // Two row sets (8 rows per pass) at 1024 threads leave 128 registers per lane and the kernel spills; at 512
+    // threads it has 256 and keeps eight weight loads in flight per lane instead of four: the same bytes in flight
+    // per compute unit from half the waves.
+    constexpr int MAXT = S >= 2 ? 512 : 1024;
+    constexpr int D = (S == 2 && (BITS == 4 || BITS == 8)) ? 8 : 4;
     if (g.tpb > (uint32_t)MAXT) return fail(ERR_UNSUPPORTED, "mfma qmv: workgroup too large for this row count");
-    const void* fn = a.nrb > 1 ? (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT, true>
-                               : (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT, false>;
+    const void* fn = a.nrb > 1 ? (const void*)qmv_mfma_kernel<DT, BITS, MP, S, D, MODE, MAXT, true>
+                               : (const void*)qmv_mfma_kernel<DT, BITS, MP, S, D, MODE, MAXT, false>;
     if (g.shmem > 48 * 1024) {
         hipError_t e = set_max_dynamic_lds(fn, (size_t)g.shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
