@@ -63,8 +63,8 @@ static bool dma_fits(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint
 
 template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, const LaunchCtx& lc, bool grouped = false) {
     const void* fn = nullptr;
-    if (!grouped && a.ksplit <= 1 && dma_fits(bits, a.m_tile_rows, kgroups, a.K, a.gpr)) {
-        fn = qmm_dma_pick(DT, a.m_tile_rows);
+    if (a.ksplit <= 1 && dma_fits(bits, a.m_tile_rows, kgroups, a.K, a.gpr) && (!grouped || a.m_tile_rows == 64)) {
+        fn = qmm_dma_pick(DT, a.m_tile_rows, grouped);
         const size_t shmem = qmm_dma_lds_bytes(a.m_tile_rows, a.gpr);
         hipError_t e = set_max_dynamic_lds(fn, (size_t)shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");

@@ -16,7 +16,12 @@ size_t qmm_dma_lds_bytes(uint32_t rows, uint32_t gpr) {
     return main_loop > epilogue ? main_loop : epilogue;
 }
 
-const void* qmm_dma_pick(int dtype, uint32_t rows) {
+const void* qmm_dma_pick(int dtype, uint32_t rows, bool grouped) {
+    if (grouped) {  // rows routed to experts: 64-row tiles cut from each expert's rows
+        if (rows != 64) return nullptr;
+        return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 0, true>
+             : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 0, true> : nullptr;
+    }
 #define QDMA(DTv) (rows == 64 ? (const void*)qmm_dma_kernel<DTv, 2, 2, 8> : rows == 128 ? (const void*)qmm_dma_kernel<DTv, 4, 2, 8> \
                    : rows == 256 ? (const void*)qmm_dma_kernel<DTv, 8, 2, 8> : nullptr)
     return dtype == DT_BF16 ? QDMA(DT_BF16) : dtype == DT_F16 ? QDMA(DT_F16) : nullptr;

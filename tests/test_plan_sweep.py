@@ -135,7 +135,7 @@ def test_benchmark_configurations_are_routed_as_documented():
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 32)
     assert "qmv_mfma_kernel<2, 4," in ks[0]
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 4096, 4096, 8, 2048)
-    assert "moe_count_sort_kernel" in ks[0] and "gather_tiles_kernel" in ks[1] and "qmm_direct_kernel" in ks[2]
+    assert "moe_count_sort_kernel" in ks[0] and "gather_tiles_kernel" in ks[1] and "qmm_dma_kernel<2, 2, 2, 8, 0, true" in ks[2]
     for bits, M in itertools.product((2, 4, 8), (1, 4)):   # the sweep configuration's cells
         for G in (32, 64, 128):
             ks, _ = kernels("qmv", DType.F16, bits, G, M, 8192, 8192)
