@@ -1440,7 +1440,7 @@ int mtq_set_option(const char* name, int value) {
         return MTQ_OK;
     }
     if (!strcmp(name, "qmm.dma")) {
-        if (value < 0 || value > 1) return fail(ERR_BAD_ARG, "qmm.dma must be 0 (where the shape allows) or 1 (never)");
+        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmm.dma must be 0 (where the shape allows), 1 (never) or 2 (always with windowed scales)");
         options().qmm_dma = value;
         return MTQ_OK;
     }

@@ -55,17 +55,23 @@ template <int DT> __global__ __launch_bounds__(256) void qmm_split_reduce_kernel
 // Shapes the load-to-LDS instances take: 4-bit codes, 2 K-groups, whole iterations of 128 k, whole 8-element
 // vectors of scales per row, one launch (no K split, no expert routing), and the ring of tiles beside the tile's
 // scales and biases within the 160 KB.
-static bool dma_fits(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr) {
-    if (options().qmm_dma == 1 || bits != 4 || kgroups != 2 || K % 128 || gpr % 8) return false;
-    if (rows != 64 && rows != 128 && rows != 256) return false;
-    return qmm_dma_lds_bytes(rows, gpr) <= 160 * 1024;
+// Returns 0 (not taken), 1 (the tile's whole rows of scales and biases in LDS) or 2 (two windows of 32 groups,
+// refilled along K: rows too long for 1; groups of 64 or 128 codes).
+static int dma_mode(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr) {
+    if (options().qmm_dma == 1 || bits != 4 || kgroups != 2 || K % 128 || gpr % 8) return 0;
+    if (rows != 64 && rows != 128 && rows != 256) return 0;
+    if (options().qmm_dma != 2 && qmm_dma_lds_bytes(rows, gpr, false) <= 160 * 1024) return 1;
+    const uint32_t G = K / gpr;
+    return (G == 64 || G == 128) && gpr >= 32 ? 2 : 0;
 }
+static bool dma_fits(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr) { return dma_mode(bits, rows, kgroups, K, gpr) != 0; }
 
 template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, const LaunchCtx& lc, bool grouped = false) {
     const void* fn = nullptr;
     if (a.ksplit <= 1 && dma_fits(bits, a.m_tile_rows, kgroups, a.K, a.gpr) && (!grouped || a.m_tile_rows == 64)) {
-        fn = qmm_dma_pick(DT, a.m_tile_rows, grouped);
-        const size_t shmem = qmm_dma_lds_bytes(a.m_tile_rows, a.gpr);
+        const bool windowed = dma_mode(bits, a.m_tile_rows, kgroups, a.K, a.gpr) == 2;
+        fn = qmm_dma_pick(DT, a.m_tile_rows, grouped, windowed);
+        const size_t shmem = qmm_dma_lds_bytes(a.m_tile_rows, a.gpr, windowed);
         hipError_t e = set_max_dynamic_lds(fn, (size_t)shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
         void* args[] = {&a};

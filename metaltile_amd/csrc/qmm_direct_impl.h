@@ -344,7 +344,9 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
 const void* qmm_direct_pick_odd(int dtype, int bits, uint32_t kgroups, uint32_t tile_rows, bool sbl, bool grouped, bool split);
 // The instances with load-to-LDS activation tiles (qmm_dma.hip): 4-bit codes, 2 K-groups, 64 / 128 / 256 rows, K a
 // multiple of 128, whole 8-element vectors of scales per row; nullptr for other tile heights.
-const void* qmm_dma_pick(int dtype, uint32_t tile_rows, bool grouped);
-size_t qmm_dma_lds_bytes(uint32_t tile_rows, uint32_t gpr);
+// `windowed`: the scales and biases as two windows of 32 groups refilled along K (groups of 64 or 128 codes) instead of
+// the tile's whole rows.
+const void* qmm_dma_pick(int dtype, uint32_t tile_rows, bool grouped, bool windowed);
+size_t qmm_dma_lds_bytes(uint32_t tile_rows, uint32_t gpr, bool windowed);
 
 }  // namespace mtq

@@ -8,19 +8,31 @@ namespace mtq {
 
 // LDS of one workgroup: the ring of tiles and the scales / biases window, or the epilogue's partial sums and
 // element tile (at most 128 rows at a time).
-size_t qmm_dma_lds_bytes(uint32_t rows, uint32_t gpr) {
+size_t qmm_dma_lds_bytes(uint32_t rows, uint32_t gpr, bool windowed) {
     const uint32_t mb = rows / 32, nbuf = mb == 8 ? 2 : 3, dbn = 128, kg = 2;
-    const size_t main_loop = (size_t)nbuf * mb * kg * 4096 + (size_t)2 * dbn * (gpr + (nbuf != 3 ? 0 : 2)) * 2;
+    // scales and biases: the tile's whole rows, or two windows of 32 groups
+    const size_t sb = windowed ? 32768 : (size_t)2 * dbn * (gpr + (nbuf != 3 ? 0 : 2)) * 2;
+    const size_t main_loop = (size_t)nbuf * mb * kg * 4096 + sb;
     const uint32_t epb = mb == 8 ? 4 : mb;
     const size_t epilogue = (size_t)(kg - 1) * 4 * epb * 16 * 64 * 4 + (size_t)epb * 32 * dbn * 2;
     return main_loop > epilogue ? main_loop : epilogue;
 }
 
-const void* qmm_dma_pick(int dtype, uint32_t rows, bool grouped) {
+const void* qmm_dma_pick(int dtype, uint32_t rows, bool grouped, bool windowed) {
     if (grouped) {  // rows routed to experts: 64-row tiles cut from each expert's rows
         if (rows != 64) return nullptr;
+        if (windowed)
+            return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 0, true, false, true>
+                 : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 0, true, false, true> : nullptr;
         return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 0, true>
              : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 0, true> : nullptr;
+    }
+    if (windowed) {
+#define QDMAW(DTv) (rows == 64 ? (const void*)qmm_dma_kernel<DTv, 2, 2, 8, 0, false, false, true>                                \
+                    : rows == 128 ? (const void*)qmm_dma_kernel<DTv, 4, 2, 8, 0, false, false, true>                              \
+                    : rows == 256 ? (const void*)qmm_dma_kernel<DTv, 8, 2, 8, 0, false, false, true> : nullptr)
+        return dtype == DT_BF16 ? QDMAW(DT_BF16) : dtype == DT_F16 ? QDMAW(DT_F16) : nullptr;
+#undef QDMAW
     }
 #define QDMA(DTv) (rows == 64 ? (const void*)qmm_dma_kernel<DTv, 2, 2, 8> : rows == 128 ? (const void*)qmm_dma_kernel<DTv, 4, 2, 8> \
                    : rows == 256 ? (const void*)qmm_dma_kernel<DTv, 8, 2, 8> : nullptr)

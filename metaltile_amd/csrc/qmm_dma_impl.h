@@ -26,6 +26,10 @@ template <int B, int E, class F> __device__ __forceinline__ void qm_static_for(F
 __device__ __forceinline__ void qm_load_to_lds(uint32_t lds_base, uint32_t voff, const void* sbase) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sbase) : "memory", "m0");
 }
+// The same with 4 bytes per lane: lane l's dword lands at lds_base + 4 * l.
+__device__ __forceinline__ void qm_load_to_lds_b32(uint32_t lds_base, uint32_t voff, const void* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_base), "v"(voff), "s"(sbase) : "memory", "m0");
+}
 #pragma clang diagnostic pop
 // 16 bytes per lane from sbase + voff into registers. The result is valid only after a qm_wait_vm
 // that covers it; until then the registers must not be read or copied.
@@ -70,7 +74,12 @@ template <int DT> __device__ __forceinline__ void qm_dequant4_b4(uint32_t e, uin
 // 39.3 / 40.0 / 41.5 us): the loop is not waiting for latency.
 // 256-row tiles (MB = 8) keep the scales and biases unpadded, row r rotated by 8 r elements, so that two tiles and the
 // window fill the 160 KB exactly at 64 groups per row; their epilogue runs in two rounds of 128 rows.
-template <int DT, int MB, int KG, int NW, int NB = 0, bool GR = false, bool SP = false>
+// WIN: rows too long for their scales and biases to sit in LDS whole (K / G groups x 128 columns x 4 bytes). They
+// are kept as two windows of 32 groups (16 KB each: [scales | biases][128 columns][32 groups], 16-byte chunks
+// XOR-swizzled by column pair); while the loop reads one window, every wave brings 256 bytes of the next one in per
+// iteration with a 4-byte-per-lane load-to-LDS (64 pieces = 8 iterations of the G / 4 a window lasts, so groups of
+// 64 and 128 codes), as one more hand-counted load per iteration. The LDS footprint no longer depends on K.
+template <int DT, int MB, int KG, int NW, int NB = 0, bool GR = false, bool SP = false, bool WIN = false>
 __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     static_assert(NW == 8 || NW == 16, "two or four waves per SIMD");
     static_assert(KG == 2 || KG == 4, "2 or 4 K-groups");
@@ -81,6 +90,8 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     constexpr int NSLOT = MB * KG, SLOT = 4096, TILE = NSLOT * SLOT;
     constexpr int NBUF = NB ? NB : MB == 8 ? 2 : 3;
     static_assert(NBUF >= 2 && NBUF <= 6, "ring of 2 to 6 tiles");
+    static_assert(!WIN || (KG == 2 && NW == 8 && !SP && NBUF <= 3), "windows: 128-k iterations, 8 waves, whole rows");
+    constexpr int NSB = WIN ? 1 : 0;           // window loads per wave and iteration
     constexpr int WSN = NBUF < 3 ? 3 : NBUF;   // weight register sets: weights are issued WSN iterations ahead
     constexpr int IPW = NSLOT * 4 / NW;       // load-to-LDS instructions per wave and iteration
     static_assert(IPW >= 1 && NSLOT * 4 % NW == 0, "the tile's load instructions divide among the waves");
@@ -159,6 +170,23 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     uint16_t* sbB = sbS + DBN * sbld;
     const int sbrow = (int)((wn * 32 + fr) * sbld) - (ROT ? 0 : (int)sb_g0);
     const uint32_t sbrot = ((wn * 32 + fr) * 8) % sbld - sb_g0 + sbld;   // ROT: position of group g is (g + sbrot) mod sbld
+    // WIN: windows at the same place; this lane's column inside a window and its swizzle
+    const unsigned char* sbW = lds + NBUF * TILE;
+    const uint32_t wcol = wn * 32 + fr, wswz = (wcol >> 1) & 3u;
+    const uint32_t log2p = a.log2g - 2;        // iterations a window lasts: 32 groups x G codes / 128
+    // piece `pid` (256 bytes, LDS order) of window `wi`: where this lane's dword comes from
+    auto issue_sb = [&](uint32_t it) {
+        if constexpr (WIN) {
+            const uint32_t t = (it + 2) & ((1u << log2p) - 1u), wi = ((it + 2) >> log2p) + 1;
+            const uint32_t pid = (t * 8u + wave) & 63u;
+            const uint32_t off = pid * 256u + 4u * lane;          // byte inside the window
+            const uint32_t isb = off >> 13, rem = off & 8191u, col = rem >> 6, cpos = (rem >> 4) & 3u, dw = (rem >> 2) & 3u;
+            const uint32_t c = cpos ^ ((col >> 1) & 3u);
+            const uint32_t grp = min(wi * 32u + c * 8u, a.gpr - 8u) + dw * 2u;
+            const uint32_t voff = (min(n0 + col, a.N - 1) * a.gpr + grp) * 2u;
+            qm_load_to_lds_b32(ring + NBUF * TILE + (wi & 1u) * 16384u + pid * 256u, voff, isb ? a.biases : a.scales);
+        }
+    };
 
     auto issue_x = [&](uint32_t it, int buf) {
         const unsigned char* src = a.x + (size_t)min(it, ilast) * (DBK * 2);
@@ -171,6 +199,14 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     // 512 * scale and bias of this lane's codes in iteration it (zero past the end: such an iteration adds nothing)
     auto scale_bias = [&](uint32_t it, float& s512, float& b) {
         int g = (int)((min(it, ilast) * DBK + kofs_abs) >> a.log2g);
+        if constexpr (WIN) {
+            const uint32_t gl = (uint32_t)g & 31u;
+            const unsigned char* p = sbW + (((uint32_t)g >> 5) & 1u) * 16384u + wcol * 64u + (((gl >> 3) ^ wswz) << 4) + ((gl & 7u) << 1);
+            s512 = elem_bits_to_f32<DT>(*(const uint16_t*)p) * 512.f;
+            b = elem_bits_to_f32<DT>(*(const uint16_t*)(p + 8192));
+            if (it > ilast) s512 = b = 0.f;
+            return;
+        }
         if constexpr (ROT) {
             g += sbrot;                      // in [sbld, 3 sbld)
             if (g >= 2 * (int)sbld) g -= sbld;
@@ -192,7 +228,16 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     // first issue W(0), W(1) | W(2), X(0) | W(3)... : here W(0), W(1), W(2), X(0), then (as iteration -1) X(1)
     qm_static_for<0, WSN>([&](auto i_c) { issue_w(decltype(i_c)::value, decltype(i_c)::value); });
     qm_static_for<0, NBUF - 1>([&](auto i_c) { issue_x(decltype(i_c)::value, decltype(i_c)::value); });
-    {
+    if constexpr (WIN) {
+        // windows 0 and 1, 16 bytes per load: 2 windows x (scales, biases) x 128 columns x 4 chunks
+        for (uint32_t v = tid; v < 2048u; v += NT) {
+            const uint32_t win = v >> 10, isb = (v >> 9) & 1u, col = (v >> 2) & 127u, c = v & 3u;
+            const uint32_t grp = min(win * 32u + c * 8u, a.gpr - 8u);
+            const q_u32x4 val = *(const q_u32x4*)((const uint16_t*)(isb ? a.biases : a.scales) + (size_t)min(n0 + col, a.N - 1) * a.gpr + grp);
+            uint32_t* d = (uint32_t*)(lds + NBUF * TILE + win * 16384u + isb * 8192u + col * 64u + ((c ^ ((col >> 1) & 3u)) << 4));
+            d[0] = val.x; d[1] = val.y; d[2] = val.z; d[3] = val.w;
+        }
+    } else {
         // DBN rows x sb_ng elements each of scales and biases, 16 bytes per load (ordinary loads: the compiler waits)
         const uint32_t vpr = sb_ng / 8, nvec = DBN * vpr;
         for (uint32_t v = tid; v < nvec; v += NT) {
@@ -238,18 +283,20 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
             // loads: this wave's share of the tile two iterations ahead into the buffer read during the last iteration,
             // weights three iterations ahead into the set whose weights have been converted
             if constexpr (NBUF == 2) {
-                // ring of two: the next tile into the buffer read during the last iteration, then the weights
+                // ring of two: (window piece,) the next tile into the buffer read during the last iteration, then the weights
+                issue_sb(it);
                 issue_x(it + 1, (u + 1) % NBUF);
                 issue_w(it + WSN, u % WSN);
             } else {
                 issue_w(it + WSN, u % WSN);
+                issue_sb(it);
                 issue_x(it + NBUF - 1, (u + NBUF - 1) % NBUF);
             }
             float sn2, bn2;
             uint32_t ek = 0, ok = 0;
             // weights of the next iteration, issued WSN - 1 iterations ago: the loads younger than they are the tiles
             // of WSN iterations and the weights of WSN - 1 (ring of two: tiles and weights of two iterations)
-            qm_wait_vm_for<(NBUF == 2 ? 2 * IPW + 2 : WSN * IPW + WSN - 1)>(raw[(u + 1) % WSN]);
+            qm_wait_vm_for<(NBUF == 2 ? 2 * IPW + 2 + 2 * NSB : WSN * IPW + WSN - 1 + WSN * NSB)>(raw[(u + 1) % WSN]);
             qm_static_for<0, MB>([&](auto bi_c) {
                 constexpr int bi = decltype(bi_c)::value;
                 constexpr int par = bi & 1;
@@ -284,7 +331,7 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
             // this wave's share of the next tile (issued one iteration ago) is in LDS once at most this iteration's
             // loads are outstanding; past the barrier every wave's share is
             // (one less than the steady state allows: the first iterations follow the prologue's order)
-            qm_wait_vm<(NBUF == 2 ? 1 : NBUF == 3 ? IPW + 1 : (NBUF - 2) * (IPW + 1) - 1)>();
+            qm_wait_vm<(NBUF == 2 ? 1 : NBUF == 3 ? IPW + 1 + NSB : (NBUF - 2) * (IPW + 1) - 1)>();
             __syncthreads();
 #pragma unroll
             for (int j = 0; j < 4; j++) af[0][j] = *(const qm_u32x4*)(lds + ((u + 1) % NBUF) * TILE + aoff[j]);

@@ -299,3 +299,40 @@ def test_256_row_tiles_refuse_what_they_cannot_take(options):
         ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
     for buf in (w, s, b, x, out):
         buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("M,N,K,G", [(300, 256, 8192, 64),     # 128 groups per row: 4 windows of 32
+                                     (130, 200, 14336, 64),    # 224 groups: 7 windows, 112 iterations, ragged N
+                                     (257, 131, 8192, 128),    # groups of 128: a window lasts 32 iterations; N % 8 != 0
+                                     (512, 128, 4096, 64),     # 64 groups: whole rows fit, windows forced (2 windows)
+                                     (64, 128, 2560, 64)])     # 40 groups: the last window is partial (20 iterations)
+def test_load_to_lds_tiles_with_windowed_scales(oracle, options, dt, M, N, K, G):
+    """Rows too long for their scales and biases to sit in LDS whole: two windows of 32 groups refilled along K by
+    load-to-LDS instructions. Forced (qmm.dma = 2) on every tile height, against the oracle's mma semantics (2e-2)
+    and bit-equal to the register-staged instance of the same tiling."""
+    bits = 4
+    c = make_case(5600 + M + K, dt, bits, G, M, N, K)
+    exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    options("qmm.kernel", 2)
+    options("qmm.kgroups", 2)
+    for rows in (64, 128, 256):
+        print(f"[case] windowed load-to-LDS qmm {dt.name} M={M} N={N} K={K} g{G} tile_rows={rows}", flush=True)
+        options("qmm.tile_rows", rows)
+        options("qmm.dma", 2)
+        out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
+        ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+        got_bytes = out.read_bytes()
+        out.free()
+        assert rel_err(unpack_f32(got_bytes, dt), exp) <= 2e-2, f"rows={rows}"
+        if rows != 256:
+            options("qmm.dma", 1)
+            out = GpuBuffer(M * N * dt.size_bytes)
+            ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+            assert out.read_bytes() == got_bytes, f"rows={rows}: differs from the register-staged instance"
+            out.free()
+    for buf in (w, s, b, x):
+        buf.free()
