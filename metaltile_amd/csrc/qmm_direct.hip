@@ -60,7 +60,7 @@ template <int DT> __global__ __launch_bounds__(256) void qmm_split_reduce_kernel
 static int dma_mode(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr) {
     if (options().qmm_dma == 1 || bits != 4 || kgroups != 2 || K % 128 || gpr % 8) return 0;
     if (rows != 64 && rows != 128 && rows != 256) return 0;
-    if (options().qmm_dma != 2 && qmm_dma_lds_bytes(rows, gpr, false) <= 160 * 1024) return 1;
+    if (options().qmm_dma != 2 && qmm_dma_lds_bytes(rows, gpr, false, false) <= 160 * 1024) return 1;
     const uint32_t G = K / gpr;
     return (G == 64 || G == 128) && gpr >= 32 ? 2 : 0;
 }
@@ -70,13 +70,42 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
     const void* fn = nullptr;
     if (a.ksplit <= 1 && dma_fits(bits, a.m_tile_rows, kgroups, a.K, a.gpr) && (!grouped || a.m_tile_rows == 64)) {
         const bool windowed = dma_mode(bits, a.m_tile_rows, kgroups, a.K, a.gpr) == 2;
-        fn = qmm_dma_pick(DT, a.m_tile_rows, grouped, windowed);
-        const size_t shmem = qmm_dma_lds_bytes(a.m_tile_rows, a.gpr, windowed);
+        int dev = 0, cus = 256;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        const bool shallow = grouped || (uint64_t)a.m_tiles * a.n_tiles > (uint64_t)cus;
+        fn = qmm_dma_pick(DT, a.m_tile_rows, grouped, windowed, shallow);
+        const size_t shmem = qmm_dma_lds_bytes(a.m_tile_rows, a.gpr, windowed, shallow);
         hipError_t e = set_max_dynamic_lds(fn, (size_t)shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
         void* args[] = {&a};
         e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles), dim3(512), args, shmem, lc);
         if (e != hipSuccess) return hip_fail(e, "qmm load-to-LDS kernel launch");
+        return ERR_OK;
+    }
+    // The same transport on the 4-K-group tilings of few rows (32 x 64 and 64 x 64 tiles, plain, K-split or grouped
+    // by expert): bit-equal results; 4096 x 14336, 16 / 32 / 64 / 128 rows 23.7 / 24.8 / 29.0 / 46.5 -> 16.0 / 17.6 /
+    // 22.9 / 34.0 us, 14336 x 4096 15.4 / 15.9 / 21.5 / 28.8 -> 13.9 / 14.3 / 19.0 / 27.0, 4096 x 4096 128 / 256 rows
+    // 17.1 / 20.9 -> 16.3 / 17.1 (64 rows and fewer: the same within 1 %).
+    if (options().qmm_dma != 1 && bits == 4 && kgroups == 4 && (a.m_tile_rows == 32 || a.m_tile_rows == 64) && a.K % 256 == 0 &&
+        a.gpr % 8 == 0 && qmm_dma4_lds_bytes(a.m_tile_rows, a.gpr) <= 160 * 1024 && !(grouped && a.ksplit > 1)) {
+        const bool split = a.ksplit > 1;
+        fn = qmm_dma4_pick(DT, a.m_tile_rows, split, grouped);
+        const size_t shmem = qmm_dma4_lds_bytes(a.m_tile_rows, a.gpr);
+        hipError_t e = set_max_dynamic_lds(fn, (size_t)shmem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
+        void* args[] = {&a};
+        LaunchCtx l1 = lc, l2 = lc;
+        if (split) { l1.stop = nullptr; l2.start = nullptr; }
+        e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles, split ? a.ksplit : 1), dim3(512), args, shmem, l1);
+        if (e != hipSuccess) return hip_fail(e, "qmm load-to-LDS kernel launch");
+        if (split) {
+            const float* part = a.part;
+            void* out = a.out;
+            uint32_t total = a.M * a.N, ks = a.ksplit;
+            void* rargs[] = {&part, &out, &total, &ks};
+            e = launch_kernel((const void*)qmm_split_reduce_kernel<DT>, dim3((total + 255) / 256), dim3(256), rargs, 0, l2);
+            if (e != hipSuccess) return hip_fail(e, "qmm split reduce kernel launch");
+        }
         return ERR_OK;
     }
     if (a.m_tile_rows == 256) return fail(ERR_UNSUPPORTED, "direct qmm: 256-row tiles need 4-bit codes, K % 128 == 0 and at most 64 groups per row");

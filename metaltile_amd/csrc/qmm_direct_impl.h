@@ -346,7 +346,12 @@ const void* qmm_direct_pick_odd(int dtype, int bits, uint32_t kgroups, uint32_t 
 // multiple of 128, whole 8-element vectors of scales per row; nullptr for other tile heights.
 // `windowed`: the scales and biases as two windows of 32 groups refilled along K (groups of 64 or 128 codes) instead of
 // the tile's whole rows.
-const void* qmm_dma_pick(int dtype, uint32_t tile_rows, bool grouped, bool windowed);
-size_t qmm_dma_lds_bytes(uint32_t tile_rows, uint32_t gpr, bool windowed);
+// `shallow` (64-row tiles): a ring of two tiles instead of three, two workgroups per compute unit; grouped launches
+// always take it.
+const void* qmm_dma_pick(int dtype, uint32_t tile_rows, bool grouped, bool windowed, bool shallow);
+size_t qmm_dma_lds_bytes(uint32_t tile_rows, uint32_t gpr, bool windowed, bool shallow);
+// The same on 4 K-groups (32 x 64 and 64 x 64 tiles, K a multiple of 256), plain or K-split.
+const void* qmm_dma4_pick(int dtype, uint32_t tile_rows, bool split, bool grouped);
+size_t qmm_dma4_lds_bytes(uint32_t tile_rows, uint32_t gpr);
 
 }  // namespace mtq

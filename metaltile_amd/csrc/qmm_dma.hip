@@ -8,8 +8,12 @@ namespace mtq {
 
 // LDS of one workgroup: the ring of tiles and the scales / biases window, or the epilogue's partial sums and
 // element tile (at most 128 rows at a time).
-size_t qmm_dma_lds_bytes(uint32_t rows, uint32_t gpr, bool windowed) {
-    const uint32_t mb = rows / 32, nbuf = mb == 8 ? 2 : 3, dbn = 128, kg = 2;
+size_t qmm_dma_lds_bytes(uint32_t rows, uint32_t gpr, bool windowed, bool shallow) {
+    // `shallow`: 64-row tiles with a ring of two, so that two workgroups share a compute unit (64 KB each at 64
+    // groups per row): for launches of more tiles than compute units, where one workgroup's prologue and epilogue
+    // then run beside the other's loop (8 x 14336 x 4096 grouped by expert, 100 rows each: 199 -> 187 us; one
+    // round of tiles is faster on the ring of three: 4096 x 4096, 512 rows 24.9 against 26.3 us)
+    const uint32_t mb = rows / 32, nbuf = (mb == 8 || (mb == 2 && shallow)) ? 2 : 3, dbn = 128, kg = 2;
     // scales and biases: the tile's whole rows, or two windows of 32 groups
     const size_t sb = windowed ? 32768 : (size_t)2 * dbn * (gpr + (nbuf != 3 ? 0 : 2)) * 2;
     const size_t main_loop = (size_t)nbuf * mb * kg * 4096 + sb;
@@ -18,26 +22,55 @@ size_t qmm_dma_lds_bytes(uint32_t rows, uint32_t gpr, bool windowed) {
     return main_loop > epilogue ? main_loop : epilogue;
 }
 
-const void* qmm_dma_pick(int dtype, uint32_t rows, bool grouped, bool windowed) {
+const void* qmm_dma_pick(int dtype, uint32_t rows, bool grouped, bool windowed, bool shallow) {
+    if (!grouped && rows == 64 && !shallow) {
+        if (windowed)
+            return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 0, false, false, true>
+                 : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 0, false, false, true> : nullptr;
+        return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8> : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8> : nullptr;
+    }
     if (grouped) {  // rows routed to experts: 64-row tiles cut from each expert's rows
         if (rows != 64) return nullptr;
         if (windowed)
-            return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 0, true, false, true>
-                 : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 0, true, false, true> : nullptr;
-        return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 0, true>
-             : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 0, true> : nullptr;
+            return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 2, true, false, true>
+                 : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 2, true, false, true> : nullptr;
+        return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 2, true>
+             : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 2, true> : nullptr;
     }
     if (windowed) {
-#define QDMAW(DTv) (rows == 64 ? (const void*)qmm_dma_kernel<DTv, 2, 2, 8, 0, false, false, true>                                \
+#define QDMAW(DTv) (rows == 64 ? (const void*)qmm_dma_kernel<DTv, 2, 2, 8, 2, false, false, true>                                \
                     : rows == 128 ? (const void*)qmm_dma_kernel<DTv, 4, 2, 8, 0, false, false, true>                              \
                     : rows == 256 ? (const void*)qmm_dma_kernel<DTv, 8, 2, 8, 0, false, false, true> : nullptr)
         return dtype == DT_BF16 ? QDMAW(DT_BF16) : dtype == DT_F16 ? QDMAW(DT_F16) : nullptr;
 #undef QDMAW
     }
-#define QDMA(DTv) (rows == 64 ? (const void*)qmm_dma_kernel<DTv, 2, 2, 8> : rows == 128 ? (const void*)qmm_dma_kernel<DTv, 4, 2, 8> \
+#define QDMA(DTv) (rows == 64 ? (const void*)qmm_dma_kernel<DTv, 2, 2, 8, 2> : rows == 128 ? (const void*)qmm_dma_kernel<DTv, 4, 2, 8> \
                    : rows == 256 ? (const void*)qmm_dma_kernel<DTv, 8, 2, 8> : nullptr)
     return dtype == DT_BF16 ? QDMA(DT_BF16) : dtype == DT_F16 ? QDMA(DT_F16) : nullptr;
 #undef QDMA
+}
+
+// 4 K-groups x 2 column waves (32 x 64 and 64 x 64 tiles, 256 k per iteration): the tilings of few rows, also as
+// K-split instances that write f32 partial tiles.
+size_t qmm_dma4_lds_bytes(uint32_t rows, uint32_t gpr) {
+    const uint32_t mb = rows / 32, dbn = 64, kg = 4;
+    const size_t main_loop = (size_t)3 * mb * kg * 4096 + (size_t)2 * dbn * (gpr + 2) * 2;
+    const size_t epilogue = (size_t)(kg - 1) * 2 * mb * 16 * 64 * 4 + (size_t)mb * 32 * dbn * 2;
+    return main_loop > epilogue ? main_loop : epilogue;
+}
+
+const void* qmm_dma4_pick(int dtype, uint32_t rows, bool split, bool grouped) {
+    if (grouped) {
+        if (split || (rows != 32 && rows != 64)) return nullptr;
+        if (dtype == DT_BF16) return rows == 32 ? (const void*)qmm_dma_kernel<DT_BF16, 1, 4, 8, 0, true> : (const void*)qmm_dma_kernel<DT_BF16, 2, 4, 8, 0, true>;
+        if (dtype == DT_F16) return rows == 32 ? (const void*)qmm_dma_kernel<DT_F16, 1, 4, 8, 0, true> : (const void*)qmm_dma_kernel<DT_F16, 2, 4, 8, 0, true>;
+        return nullptr;
+    }
+#define QDMA4(DTv) (split ? (rows == 32 ? (const void*)qmm_dma_kernel<DTv, 1, 4, 8, 0, false, true> : (const void*)qmm_dma_kernel<DTv, 2, 4, 8, 0, false, true>) \
+                          : (rows == 32 ? (const void*)qmm_dma_kernel<DTv, 1, 4, 8> : (const void*)qmm_dma_kernel<DTv, 2, 4, 8>))
+    if (rows != 32 && rows != 64) return nullptr;
+    return dtype == DT_BF16 ? QDMA4(DT_BF16) : dtype == DT_F16 ? QDMA4(DT_F16) : nullptr;
+#undef QDMA4
 }
 
 }  // namespace mtq

@@ -336,3 +336,37 @@ def test_load_to_lds_tiles_with_windowed_scales(oracle, options, dt, M, N, K, G)
             out.free()
     for buf in (w, s, b, x):
         buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("M,N,K,G", [(20, 200, 1024, 64), (64, 131, 2048, 32), (33, 128, 4096, 64), (50, 64, 768, 32)])
+def test_load_to_lds_tiles_on_4_kgroups(oracle, options, dt, M, N, K, G):
+    """The tilings of few rows (32 x 64 and 64 x 64 tiles on 4 K-groups, 256 k per iteration) with load-to-LDS
+    activation tiles, unsplit and with K split over 1, 2 and 3 workgroups (f32 partial tiles added by the reduce
+    kernel): the oracle's mma semantics (2e-2) and bit-equal to the register-staged instances."""
+    bits = 4
+    c = make_case(5700 + M + K, dt, bits, G, M, N, K)
+    exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    options("qmm.kernel", 2)
+    options("qmm.kgroups", 4)
+    for rows in (32, 64):
+        for ksplit in (1, 2, 3):
+            if ksplit > K // 256:
+                continue
+            print(f"[case] load-to-LDS qmm on 4 K-groups {dt.name} M={M} N={N} K={K} g{G} tile_rows={rows} ksplit={ksplit}", flush=True)
+            options("qmm.tile_rows", rows)
+            options("qmm.ksplit", ksplit)
+            res = {}
+            for dma in (0, 1):
+                options("qmm.dma", dma)
+                out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
+                ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+                res[dma] = out.read_bytes()
+                out.free()
+            assert rel_err(unpack_f32(res[0], dt), exp) <= 2e-2, f"rows={rows} ksplit={ksplit}"
+            assert res[0] == res[1], f"rows={rows} ksplit={ksplit}: differs from the register-staged instance"
+    for buf in (w, s, b, x):
+        buf.free()

@@ -129,13 +129,14 @@ def test_benchmark_configurations_are_routed_as_documented():
         assert f"qmm_dma_kernel<2, {mb}, 2, 8," in ks[0], ks
         assert ls[0][1][0] == 256 and ls[0][2][0] == 512
     ks, ls = kernels("qmm_mma", DType.BF16, 4, 64, 32, 4096, 4096)
-    assert "qmm_direct_kernel<2, 4, 2, 1," in ks[0]    # 32-row tiles
+    assert "qmm_dma_kernel<2, 1, 4, 8," in ks[0]       # 32-row tiles on 4 K-groups, K split: a reduce kernel follows
+    assert "qmm_split_reduce_kernel" in ks[1]
     ks, _ = kernels("qmm_mma", DType.BF16, 8, 64, 512, 4096, 4096)
     assert "qmm_direct_kernel<2, 8," in ks[0]          # other code widths stay on the register-staged tiles
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 32)
     assert "qmv_mfma_kernel<2, 4," in ks[0]
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 4096, 4096, 8, 2048)
-    assert "moe_count_sort_kernel" in ks[0] and "gather_tiles_kernel" in ks[1] and "qmm_dma_kernel<2, 2, 2, 8, 0, true" in ks[2]
+    assert "moe_count_sort_kernel" in ks[0] and "gather_tiles_kernel" in ks[1] and "qmm_dma_kernel<2, 2, 2, 8, 2, true" in ks[2]
     for bits, M in itertools.product((2, 4, 8), (1, 4)):   # the sweep configuration's cells
         for G in (32, 64, 128):
             ks, _ = kernels("qmv", DType.F16, bits, G, M, 8192, 8192)
