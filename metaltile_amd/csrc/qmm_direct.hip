@@ -58,9 +58,10 @@ template <int DT> __global__ __launch_bounds__(256) void qmm_split_reduce_kernel
 // Returns 0 (not taken), 1 (the tile's whole rows of scales and biases in LDS) or 2 (two windows of 32 groups,
 // refilled along K: rows too long for 1; groups of 64 or 128 codes).
 static int dma_mode(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr) {
-    if (options().qmm_dma == 1 || bits != 4 || kgroups != 2 || K % 128 || gpr % 8) return 0;
+    if (options().qmm_dma == 1 || bits != 4 || kgroups != 2 || K % 128 || gpr % 2) return 0;
     if (rows != 64 && rows != 128 && rows != 256) return 0;
-    if (options().qmm_dma != 2 && qmm_dma_lds_bytes(rows, gpr, false, false) <= 160 * 1024) return 1;
+    // whole rows are staged as 8-group vectors; the windows take them two groups at a time (K = 11008 at g64: 172 groups)
+    if (options().qmm_dma != 2 && gpr % 8 == 0 && qmm_dma_lds_bytes(rows, gpr, false, false) <= 160 * 1024) return 1;
     const uint32_t G = K / gpr;
     return (G == 64 || G == 128) && gpr >= 32 ? 2 : 0;
 }
@@ -243,7 +244,10 @@ static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
     // 4096 x 4096: 384 rows 26.7 -> 22.9 us, 512 rows 28.7 -> 23.8, 768 rows 38.3 -> 31.6, 1024 rows 43.0 -> 37.8,
     // 1536 rows 68.7 -> 56.8, 2048 rows 79.2 -> 70.6, 4096 rows 152 -> 141; 14336 x 4096: 512 rows 75.3 -> 65.1,
     // 4096 rows 513 -> 459; 4096 x 8192, 512 rows: 61.1 -> 43.8.
-    if (p.M > 64 && short_wide * 2 > (uint64_t)cus && !options().qmm_tile_rows && !options().qmm_kgroups) {
+    // (long rows that leave even the 64-row tiles short of one per compute unit keep the K-split tall tiles chosen
+    // above: 300 rows, 4096 x 11008 63 us against 68, 4096 x 14336 79 against 81)
+    const bool underfilled_long = p.M >= 256 && p.K > 8192 && short_wide < (uint64_t)cus;   // (at K = 8192 the 64-row tiles win: 300 rows 38 us against 49)
+    if (p.M > 64 && short_wide * 2 > (uint64_t)cus && !underfilled_long && !options().qmm_tile_rows && !options().qmm_kgroups) {
         static const uint32_t heights[3] = {64, 128, 256};
         static const double base[3] = {20.6, 28.0, 48.5}, full[3] = {0.16, 0.35, 0.45}, more[3] = {1.15, 1.10, 1.0};
         double best = 0.0;

@@ -182,7 +182,8 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
             const uint32_t off = pid * 256u + 4u * lane;          // byte inside the window
             const uint32_t isb = off >> 13, rem = off & 8191u, col = rem >> 6, cpos = (rem >> 4) & 3u, dw = (rem >> 2) & 3u;
             const uint32_t c = cpos ^ ((col >> 1) & 3u);
-            const uint32_t grp = min(wi * 32u + c * 8u, a.gpr - 8u) + dw * 2u;
+            // two groups per dword; past the row's last group the load is clamped onto it (those positions are never read)
+            const uint32_t grp = min(wi * 32u + c * 8u + dw * 2u, a.gpr - 2u);
             const uint32_t voff = (min(n0 + col, a.N - 1) * a.gpr + grp) * 2u;
             qm_load_to_lds_b32(ring + NBUF * TILE + (wi & 1u) * 16384u + pid * 256u, voff, isb ? a.biases : a.scales);
         }
@@ -229,13 +230,13 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     qm_static_for<0, WSN>([&](auto i_c) { issue_w(decltype(i_c)::value, decltype(i_c)::value); });
     qm_static_for<0, NBUF - 1>([&](auto i_c) { issue_x(decltype(i_c)::value, decltype(i_c)::value); });
     if constexpr (WIN) {
-        // windows 0 and 1, 16 bytes per load: 2 windows x (scales, biases) x 128 columns x 4 chunks
-        for (uint32_t v = tid; v < 2048u; v += NT) {
-            const uint32_t win = v >> 10, isb = (v >> 9) & 1u, col = (v >> 2) & 127u, c = v & 3u;
-            const uint32_t grp = min(win * 32u + c * 8u, a.gpr - 8u);
-            const q_u32x4 val = *(const q_u32x4*)((const uint16_t*)(isb ? a.biases : a.scales) + (size_t)min(n0 + col, a.N - 1) * a.gpr + grp);
-            uint32_t* d = (uint32_t*)(lds + NBUF * TILE + win * 16384u + isb * 8192u + col * 64u + ((c ^ ((col >> 1) & 3u)) << 4));
-            d[0] = val.x; d[1] = val.y; d[2] = val.z; d[3] = val.w;
+        // windows 0 and 1, a dword (two groups) per load: 2 windows x (scales, biases) x 128 columns x 16 dwords; rows
+        // need not be whole 8-group vectors (K / G even is enough), loads past a row's end are clamped onto its last dword
+        for (uint32_t v = tid; v < 8192u; v += NT) {
+            const uint32_t win = v >> 12, isb = (v >> 11) & 1u, col = (v >> 4) & 127u, c = (v >> 2) & 3u, dw = v & 3u;
+            const uint32_t grp = min(win * 32u + c * 8u + dw * 2u, a.gpr - 2u);
+            const uint32_t val = *(const uint32_t*)((const uint16_t*)(isb ? a.biases : a.scales) + (size_t)min(n0 + col, a.N - 1) * a.gpr + grp);
+            *(uint32_t*)(lds + NBUF * TILE + win * 16384u + isb * 8192u + col * 64u + ((c ^ ((col >> 1) & 3u)) << 4) + dw * 4u) = val;
         }
     } else {
         // DBN rows x sb_ng elements each of scales and biases, 16 bytes per load (ordinary loads: the compiler waits)

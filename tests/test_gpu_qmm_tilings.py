@@ -306,7 +306,8 @@ def test_256_row_tiles_refuse_what_they_cannot_take(options):
                                      (130, 200, 14336, 64),    # 224 groups: 7 windows, 112 iterations, ragged N
                                      (257, 131, 8192, 128),    # groups of 128: a window lasts 32 iterations; N % 8 != 0
                                      (512, 128, 4096, 64),     # 64 groups: whole rows fit, windows forced (2 windows)
-                                     (64, 128, 2560, 64)])     # 40 groups: the last window is partial (20 iterations)
+                                     (64, 128, 2560, 64),      # 40 groups: the last window is partial (20 iterations)
+                                     (96, 128, 11008, 64)])    # 172 groups: not whole 8-group vectors, 6 windows (the last of 12 groups)
 def test_load_to_lds_tiles_with_windowed_scales(oracle, options, dt, M, N, K, G):
     """Rows too long for their scales and biases to sit in LDS whole: two windows of 32 groups refilled along K by
     load-to-LDS instructions. Forced (qmm.dma = 2) on every tile height, against the oracle's mma semantics (2e-2)
