@@ -400,11 +400,13 @@ MTQ_API int mtq_flush_cache(void);
  *   "qmm.kernel"           0 = choose per shape, 1 = tile kernel with both operands through LDS, 2 = tile
  *                          kernel with the weights converted in registers
  *   "qmm.kgroups"          register-operand tile kernel: K-groups per workgroup, 0 = choose, or 1 / 2 / 4
- *   "qmm.tile_rows"        activation rows per tile, 0 = choose, or 32 (4 K-groups only) / 64 / 128 / 256 (4-bit codes
- *                          on 2 K-groups only)
- *   "qmm.dma"              tile instances that bring the activation tile in by load-to-LDS instructions (4-bit codes):
- *                          0 = where the shape allows, 1 = never (the register-staged instances; same results bit for
- *                          bit), 2 = with the scales and biases in windows even where whole rows fit
+ *   "qmm.tile_rows"        activation rows per tile, 0 = choose, or 32 (4 K-groups only) / 64 / 128 / 256 (4- and 8-bit
+ *                          codes on 2 K-groups only)
+ *   "qmm.dma"              tile instances that bring the activation tile in by load-to-LDS instructions (4- and 8-bit
+ *                          codes): 0 = where the shape allows and it pays (8-bit codes: rows of 8192 codes and more, or
+ *                          launches that fill the chip), 1 = never (the register-staged instances; same results bit for
+ *                          bit), 2 = with the scales and biases in windows even where whole rows fit, 3 = wherever the
+ *                          shape allows
  *   "qmm.by_m"             order in which workgroups walk the tiles: 0 = choose, 1 = the N-tiles of one M-tile
  *                          first, 2 = the M-tiles of one N-tile first
  *   "qmm.splits"           LDS tile kernel: 0 = choose per shape, or the number of K slices per output tile

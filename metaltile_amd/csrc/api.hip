@@ -1440,7 +1440,8 @@ int mtq_set_option(const char* name, int value) {
         return MTQ_OK;
     }
     if (!strcmp(name, "qmm.dma")) {
-        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmm.dma must be 0 (where the shape allows), 1 (never) or 2 (always with windowed scales)");
+        if (value < 0 || value > 3)
+            return fail(ERR_BAD_ARG, "qmm.dma must be 0 (where it pays), 1 (never), 2 (always with windowed scales) or 3 (wherever the shape allows)");
         options().qmm_dma = value;
         return MTQ_OK;
     }

@@ -104,7 +104,7 @@ struct Options {
     int qmm_ksplit = 0;           // direct qmm: 0 = choose, 1 = never split K, n = n splits
     int qmm_f32_tiles = 0;        // f32 batches on the f32 matrix cores: 0 = choose by rows, 1 = never, 2 = always
     int qmm_tile_rows = 0;        // direct qmm: activation rows per tile (0 = choose; 32, 64, 128, 256)
-    int qmm_dma = 0;              // direct qmm: activation tiles by load-to-LDS instructions: 0 = where the shape allows, 1 = never, 2 = with the scales in windows even where whole rows fit
+    int qmm_dma = 0;              // direct qmm: activation tiles by load-to-LDS instructions: 0 = where it pays, 1 = never, 2 = with the scales in windows even where whole rows fit, 3 = wherever the shape allows
     int qmv_mfma = 0;             // matrix-core qmv: 0 auto, 1 never, 2 whenever the shape fits
     int qmv_mfma_kp = 0;          // matrix-core qmv: K parts per row block
     int qmv_mfma_rbw = 0;         // matrix-core qmv: row blocks walked in parallel per workgroup

@@ -52,29 +52,35 @@ template <int DT> __global__ __launch_bounds__(256) void qmm_split_reduce_kernel
     ((uint16_t*)out)[i] = f32_to_elem_bits<DT>(r);
 }
 
-// Shapes the load-to-LDS instances take: 4-bit codes, 2 K-groups, whole iterations of 128 k, whole 8-element
+// Shapes the load-to-LDS instances take: 4- or 8-bit codes, 2 K-groups, whole iterations of 128 k, whole 8-element
 // vectors of scales per row, one launch (no K split, no expert routing), and the ring of tiles beside the tile's
 // scales and biases within the 160 KB.
 // Returns 0 (not taken), 1 (the tile's whole rows of scales and biases in LDS) or 2 (two windows of 32 groups,
 // refilled along K: rows too long for 1; groups of 64 or 128 codes).
 static int dma_mode(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr) {
-    if (options().qmm_dma == 1 || bits != 4 || kgroups != 2 || K % 128 || gpr % 2) return 0;
+    if (options().qmm_dma == 1 || (bits != 4 && bits != 8) || kgroups != 2 || K % 128 || gpr % 2) return 0;
     if (rows != 64 && rows != 128 && rows != 256) return 0;
     // whole rows are staged as 8-group vectors; the windows take them two groups at a time (K = 11008 at g64: 172 groups)
     if (options().qmm_dma != 2 && gpr % 8 == 0 && qmm_dma_lds_bytes(rows, gpr, false, false) <= 160 * 1024) return 1;
     const uint32_t G = K / gpr;
+    if (bits == 8 && rows == 256) return 0;   // that instance does not fit the register file
     return (G == 64 || G == 128) && gpr >= 32 ? 2 : 0;
 }
 static bool dma_fits(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr) { return dma_mode(bits, rows, kgroups, K, gpr) != 0; }
 
 template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, const LaunchCtx& lc, bool grouped = false) {
     const void* fn = nullptr;
-    if (a.ksplit <= 1 && dma_fits(bits, a.m_tile_rows, kgroups, a.K, a.gpr) && (!grouped || a.m_tile_rows == 64)) {
+    // 8-bit codes on short rows gain nothing where the launch leaves compute units idle (14336 x 4096, 128 rows:
+    // 36.3 against 34.3 us) or on the 4-K-group tiles (4096 x 4096, 16 / 64 rows 11.6 / 15.3 against 10.9 / 14.6;
+    // 4096 x 14336 20.2 / 28.7 against 31.6 / 37.4): those stay on the register-staged instances
+    const bool b8_short = bits == 8 && a.K < 8192 && options().qmm_dma < 2;
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (a.ksplit <= 1 && dma_fits(bits, a.m_tile_rows, kgroups, a.K, a.gpr) && (!grouped || a.m_tile_rows == 64) &&
+        !(b8_short && !grouped && a.m_tile_rows != 256 && (uint64_t)a.m_tiles * a.n_tiles < (uint64_t)cus)) {
         const bool windowed = dma_mode(bits, a.m_tile_rows, kgroups, a.K, a.gpr) == 2;
-        int dev = 0, cus = 256;
-        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         const bool shallow = grouped || (uint64_t)a.m_tiles * a.n_tiles > (uint64_t)cus;
-        fn = qmm_dma_pick(DT, a.m_tile_rows, grouped, windowed, shallow);
+        fn = qmm_dma_pick(bits, DT, a.m_tile_rows, grouped, windowed, shallow);
         const size_t shmem = qmm_dma_lds_bytes(a.m_tile_rows, a.gpr, windowed, shallow);
         hipError_t e = set_max_dynamic_lds(fn, (size_t)shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
@@ -87,10 +93,10 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
     // by expert): bit-equal results; 4096 x 14336, 16 / 32 / 64 / 128 rows 23.7 / 24.8 / 29.0 / 46.5 -> 16.0 / 17.6 /
     // 22.9 / 34.0 us, 14336 x 4096 15.4 / 15.9 / 21.5 / 28.8 -> 13.9 / 14.3 / 19.0 / 27.0, 4096 x 4096 128 / 256 rows
     // 17.1 / 20.9 -> 16.3 / 17.1 (64 rows and fewer: the same within 1 %).
-    if (options().qmm_dma != 1 && bits == 4 && kgroups == 4 && (a.m_tile_rows == 32 || a.m_tile_rows == 64) && a.K % 256 == 0 &&
+    if (options().qmm_dma != 1 && (bits == 4 || bits == 8) && !b8_short && kgroups == 4 && (a.m_tile_rows == 32 || a.m_tile_rows == 64) && a.K % 256 == 0 &&
         a.gpr % 8 == 0 && qmm_dma4_lds_bytes(a.m_tile_rows, a.gpr) <= 160 * 1024 && !(grouped && a.ksplit > 1)) {
         const bool split = a.ksplit > 1;
-        fn = qmm_dma4_pick(DT, a.m_tile_rows, split, grouped);
+        fn = qmm_dma4_pick(bits, DT, a.m_tile_rows, split, grouped);
         const size_t shmem = qmm_dma4_lds_bytes(a.m_tile_rows, a.gpr);
         hipError_t e = set_max_dynamic_lds(fn, (size_t)shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
@@ -109,7 +115,7 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
         }
         return ERR_OK;
     }
-    if (a.m_tile_rows == 256) return fail(ERR_UNSUPPORTED, "direct qmm: 256-row tiles need 4-bit codes, K % 128 == 0 and at most 64 groups per row");
+    if (a.m_tile_rows == 256) return fail(ERR_UNSUPPORTED, "direct qmm: 256-row tiles need 4- or 8-bit codes, K % 128 == 0 and rows whose scales fit LDS (or, 4-bit codes, groups of 64 or 128 codes)");
     const bool tall = a.m_tile_rows == 128;
     const uint32_t dbn = kgroups == 1 ? 128 : 32 * (8 / kgroups);
     // scales and biases of the tile's rows in LDS when they fit beside the activation tiles
@@ -279,7 +285,7 @@ static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
     // the bit-stream widths are built with 128-row tiles on 1 K-group only
     if (odd_bits && rows == 128 && !options().qmm_kgroups) kgroups = 1;
     if (rows == 256 && !dma_fits(p.bits, 256, kgroups, p.K, p.K / G))
-        return fail(ERR_BAD_ARG, "qmm.tile_rows 256 needs 4-bit codes, 2 K-groups, K % 128 == 0 and at most 64 groups per row");
+        return fail(ERR_BAD_ARG, "qmm.tile_rows 256 needs 4- or 8-bit codes, 2 K-groups, K % 128 == 0 and rows whose scales fit LDS (or, 4-bit codes, groups of 64 or 128 codes)");
     if (rows == 32 && kgroups != 4) {
         if (options().qmm_tile_rows) return fail(ERR_BAD_ARG, "qmm.tile_rows 32 needs 4 K-groups");
         rows = 64;

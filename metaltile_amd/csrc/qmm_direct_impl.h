@@ -342,16 +342,16 @@ __global__ __launch_bounds__(KG == 1 ? 256 : 512) void qmm_direct_kernel(QmmDArg
 
 // Kernel for 3-, 5-, 6- and 7-bit codes (qmm_direct_odd.hip); null when the combination is not built.
 const void* qmm_direct_pick_odd(int dtype, int bits, uint32_t kgroups, uint32_t tile_rows, bool sbl, bool grouped, bool split);
-// The instances with load-to-LDS activation tiles (qmm_dma.hip): 4-bit codes, 2 K-groups, 64 / 128 / 256 rows, K a
+// The instances with load-to-LDS activation tiles (qmm_dma.hip, qmm_dma_b8.hip): 4- and 8-bit codes, 2 K-groups, 64 / 128 / 256 rows, K a
 // multiple of 128, whole 8-element vectors of scales per row; nullptr for other tile heights.
 // `windowed`: the scales and biases as two windows of 32 groups refilled along K (groups of 64 or 128 codes) instead of
 // the tile's whole rows.
 // `shallow` (64-row tiles): a ring of two tiles instead of three, two workgroups per compute unit; grouped launches
 // always take it.
-const void* qmm_dma_pick(int dtype, uint32_t tile_rows, bool grouped, bool windowed, bool shallow);
+const void* qmm_dma_pick(int bits, int dtype, uint32_t tile_rows, bool grouped, bool windowed, bool shallow);
 size_t qmm_dma_lds_bytes(uint32_t tile_rows, uint32_t gpr, bool windowed, bool shallow);
 // The same on 4 K-groups (32 x 64 and 64 x 64 tiles, K a multiple of 256), plain or K-split.
-const void* qmm_dma4_pick(int dtype, uint32_t tile_rows, bool split, bool grouped);
+const void* qmm_dma4_pick(int bits, int dtype, uint32_t tile_rows, bool split, bool grouped);
 size_t qmm_dma4_lds_bytes(uint32_t tile_rows, uint32_t gpr);
 
 }  // namespace mtq

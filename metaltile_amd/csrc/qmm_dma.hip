@@ -1,8 +1,9 @@
-// Instances of the tile kernel whose activation tile is brought in by load-to-LDS instructions (4-bit codes,
+// Instances of the tile kernel whose activation tile is brought in by load-to-LDS instructions (4-bit codes here, 8-bit
+// ones in qmm_dma_b8.hip;
 // f16 / bf16, 2 K-groups x 4 column waves): replaces the same reference kernels as qmm_direct.hip (mt_qmm_mma and
 // its _m16 form, crates/metaltile-std/src/mlx/quantized.rs:2106-2405, 2408) with the same arithmetic, on 64 x 128,
 // 128 x 128 and 256 x 128 tiles. A translation unit of its own so that it compiles beside qmm_direct.hip.
-#include "qmm_dma_impl.h"
+#include "qmm_dma_picks.h"
 
 namespace mtq {
 
@@ -22,32 +23,11 @@ size_t qmm_dma_lds_bytes(uint32_t rows, uint32_t gpr, bool windowed, bool shallo
     return main_loop > epilogue ? main_loop : epilogue;
 }
 
-const void* qmm_dma_pick(int dtype, uint32_t rows, bool grouped, bool windowed, bool shallow) {
-    if (!grouped && rows == 64 && !shallow) {
-        if (windowed)
-            return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 0, false, false, true>
-                 : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 0, false, false, true> : nullptr;
-        return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8> : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8> : nullptr;
-    }
-    if (grouped) {  // rows routed to experts: 64-row tiles cut from each expert's rows
-        if (rows != 64) return nullptr;
-        if (windowed)
-            return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 2, true, false, true>
-                 : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 2, true, false, true> : nullptr;
-        return dtype == DT_BF16 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 2, true>
-             : dtype == DT_F16 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 2, true> : nullptr;
-    }
-    if (windowed) {
-#define QDMAW(DTv) (rows == 64 ? (const void*)qmm_dma_kernel<DTv, 2, 2, 8, 2, false, false, true>                                \
-                    : rows == 128 ? (const void*)qmm_dma_kernel<DTv, 4, 2, 8, 0, false, false, true>                              \
-                    : rows == 256 ? (const void*)qmm_dma_kernel<DTv, 8, 2, 8, 0, false, false, true> : nullptr)
-        return dtype == DT_BF16 ? QDMAW(DT_BF16) : dtype == DT_F16 ? QDMAW(DT_F16) : nullptr;
-#undef QDMAW
-    }
-#define QDMA(DTv) (rows == 64 ? (const void*)qmm_dma_kernel<DTv, 2, 2, 8, 2> : rows == 128 ? (const void*)qmm_dma_kernel<DTv, 4, 2, 8> \
-                   : rows == 256 ? (const void*)qmm_dma_kernel<DTv, 8, 2, 8> : nullptr)
-    return dtype == DT_BF16 ? QDMA(DT_BF16) : dtype == DT_F16 ? QDMA(DT_F16) : nullptr;
-#undef QDMA
+const void* qmm_dma_pick_b8(int dtype, uint32_t rows, bool grouped, bool windowed, bool shallow);
+const void* qmm_dma4_pick_b8(int dtype, uint32_t rows, bool split, bool grouped);
+
+const void* qmm_dma_pick(int bits, int dtype, uint32_t rows, bool grouped, bool windowed, bool shallow) {
+    return bits == 8 ? qmm_dma_pick_b8(dtype, rows, grouped, windowed, shallow) : qmm_dma_pick_t<4>(dtype, rows, grouped, windowed, shallow);
 }
 
 // 4 K-groups x 2 column waves (32 x 64 and 64 x 64 tiles, 256 k per iteration): the tilings of few rows, also as
@@ -59,18 +39,8 @@ size_t qmm_dma4_lds_bytes(uint32_t rows, uint32_t gpr) {
     return main_loop > epilogue ? main_loop : epilogue;
 }
 
-const void* qmm_dma4_pick(int dtype, uint32_t rows, bool split, bool grouped) {
-    if (grouped) {
-        if (split || (rows != 32 && rows != 64)) return nullptr;
-        if (dtype == DT_BF16) return rows == 32 ? (const void*)qmm_dma_kernel<DT_BF16, 1, 4, 8, 0, true> : (const void*)qmm_dma_kernel<DT_BF16, 2, 4, 8, 0, true>;
-        if (dtype == DT_F16) return rows == 32 ? (const void*)qmm_dma_kernel<DT_F16, 1, 4, 8, 0, true> : (const void*)qmm_dma_kernel<DT_F16, 2, 4, 8, 0, true>;
-        return nullptr;
-    }
-#define QDMA4(DTv) (split ? (rows == 32 ? (const void*)qmm_dma_kernel<DTv, 1, 4, 8, 0, false, true> : (const void*)qmm_dma_kernel<DTv, 2, 4, 8, 0, false, true>) \
-                          : (rows == 32 ? (const void*)qmm_dma_kernel<DTv, 1, 4, 8> : (const void*)qmm_dma_kernel<DTv, 2, 4, 8>))
-    if (rows != 32 && rows != 64) return nullptr;
-    return dtype == DT_BF16 ? QDMA4(DT_BF16) : dtype == DT_F16 ? QDMA4(DT_F16) : nullptr;
-#undef QDMA4
+const void* qmm_dma4_pick(int bits, int dtype, uint32_t rows, bool split, bool grouped) {
+    return bits == 8 ? qmm_dma4_pick_b8(dtype, rows, split, grouped) : qmm_dma4_pick_t<4>(dtype, rows, split, grouped);
 }
 
 }  // namespace mtq

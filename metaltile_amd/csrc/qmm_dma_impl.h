@@ -45,6 +45,9 @@ template <int N> __device__ __forceinline__ void qm_wait_vm() {
 template <int N> __device__ __forceinline__ void qm_wait_vm_for(qm_u32x4& r) {
     asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r) : "n"(N) : "memory");
 }
+template <int N> __device__ __forceinline__ void qm_wait_vm_for2(qm_u32x4& r0, qm_u32x4& r1) {
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(r0), "+v"(r1) : "n"(N) : "memory");
+}
 
 // Four 4-bit codes -> four elements s * q + b rounded to T, as two dwords. e and o hold the even and the odd
 // codes of a weight dword one per byte (e = w & 0x0F0F0F0F, o = (w >> 4) & 0x0F0F0F0F); `half` picks bytes
@@ -79,12 +82,16 @@ template <int DT> __device__ __forceinline__ void qm_dequant4_b4(uint32_t e, uin
 // XOR-swizzled by column pair); while the loop reads one window, every wave brings 256 bytes of the next one in per
 // iteration with a 4-byte-per-lane load-to-LDS (64 pieces = 8 iterations of the G / 4 a window lasts, so groups of
 // 64 and 128 codes), as one more hand-counted load per iteration. The LDS footprint no longer depends on K.
-template <int DT, int MB, int KG, int NW, int NB = 0, bool GR = false, bool SP = false, bool WIN = false>
+// BITS: 4, or 8 (a lane's 32 codes are then 32 bytes: two 16-byte loads per iteration, bytes converted with the
+// byte-select converts; everything else alike).
+template <int DT, int MB, int KG, int NW, int NB = 0, bool GR = false, bool SP = false, bool WIN = false, int BITS = 4>
 __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     static_assert(NW == 8 || NW == 16, "two or four waves per SIMD");
     static_assert(KG == 2 || KG == 4, "2 or 4 K-groups");
     static_assert(MB == 1 || MB == 2 || MB == 4 || MB == 8, "32 to 256 rows");
-    constexpr int BITS = 4;
+    static_assert(BITS == 4 || BITS == 8, "4- or 8-bit codes");
+    constexpr int NWL = BITS / 4;              // 16-byte weight loads per lane and iteration
+    constexpr float KSCALE = BITS == 4 ? 512.f : 1.f;   // 4-bit codes are read as fp8 = code / 512
     constexpr int NT = 64 * NW, NWV = NW / KG;
     constexpr int DBN = 32 * NWV, DBK = 64 * KG, DBM = 32 * MB;
     constexpr int NSLOT = MB * KG, SLOT = 4096, TILE = NSLOT * SLOT;
@@ -194,16 +201,41 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
 #pragma unroll
         for (int i = 0; i < IPW; i++) qm_load_to_lds(ring + buf * TILE + (wave * IPW + i) * 1024, xoff[i], src);
     };
-    qm_u32x4 raw[WSN];
+    qm_u32x4 raw[WSN][NWL];
     auto issue_w = [&](uint32_t it, int set) {
-        qm_load_regs(raw[set], woff, a.w + (size_t)min(it, ilast) * (DBK * BITS / 8)); };
+        const unsigned char* src = a.w + (size_t)min(it, ilast) * (DBK * BITS / 8);
+        qm_load_regs(raw[set][0], woff, src);
+        if constexpr (NWL == 2) qm_load_regs(raw[set][1], woff, src + 16);
+    };
+    // waits until at most N loads are outstanding and ties a weight set to the wait
+    auto wait_w = [&](auto n_c, int set) {
+        constexpr int N = decltype(n_c)::value;
+        if constexpr (NWL == 2) qm_wait_vm_for2<N>(raw[set][0], raw[set][NWL - 1]);
+        else qm_wait_vm_for<N>(raw[set][0]);
+    };
+    // half fragment hf (4 codes) of weight set `set` -> two dwords of elements
+    uint32_t ek = 0, ok = 0;
+    auto convert_half = [&](int set, int hf, float sc, float bi, uint32_t& d0, uint32_t& d1) {
+        if constexpr (BITS == 4) {
+            const int jj = hf / 2, half = hf % 2;
+            if (half == 0) {
+                ek = raw[set][0][jj] & 0x0F0F0F0Fu;
+                ok = (raw[set][0][jj] >> 4) & 0x0F0F0F0Fu;
+            }
+            qm_dequant4_b4<DT>(ek, ok, half, sc, bi, d0, d1);
+        } else {
+            const uint32_t w8 = raw[set][hf / 4][hf % 4];
+            d0 = pack2<DT>(fmaf((float)(w8 & 0xFFu), sc, bi), fmaf((float)((w8 >> 8) & 0xFFu), sc, bi));
+            d1 = pack2<DT>(fmaf((float)((w8 >> 16) & 0xFFu), sc, bi), fmaf((float)(w8 >> 24), sc, bi));
+        }
+    };
     // 512 * scale and bias of this lane's codes in iteration it (zero past the end: such an iteration adds nothing)
     auto scale_bias = [&](uint32_t it, float& s512, float& b) {
         int g = (int)((min(it, ilast) * DBK + kofs_abs) >> a.log2g);
         if constexpr (WIN) {
             const uint32_t gl = (uint32_t)g & 31u;
             const unsigned char* p = sbW + (((uint32_t)g >> 5) & 1u) * 16384u + wcol * 64u + (((gl >> 3) ^ wswz) << 4) + ((gl & 7u) << 1);
-            s512 = elem_bits_to_f32<DT>(*(const uint16_t*)p) * 512.f;
+            s512 = elem_bits_to_f32<DT>(*(const uint16_t*)p) * KSCALE;
             b = elem_bits_to_f32<DT>(*(const uint16_t*)(p + 8192));
             if (it > ilast) s512 = b = 0.f;
             return;
@@ -213,7 +245,7 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
             if (g >= 2 * (int)sbld) g -= sbld;
             g -= sbld;
         }
-        s512 = elem_bits_to_f32<DT>(sbS[sbrow + g]) * 512.f;
+        s512 = elem_bits_to_f32<DT>(sbS[sbrow + g]) * KSCALE;
         b = elem_bits_to_f32<DT>(sbB[sbrow + g]);
         if (it > ilast) s512 = b = 0.f;
     };
@@ -258,15 +290,11 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     uint32_t bq[2][4][4];  // converted fragments: [iteration parity][MFMA step][dword]
     float sn, bn;          // 512 * scale and bias of the iteration being converted (the next one)
     {
-        qm_wait_vm_for<(NBUF - 2) * IPW>(raw[0]);
+        wait_w(std::integral_constant<int, (NBUF - 2) * IPW>{}, 0);
         float s0, b0;
         scale_bias(0, s0, b0);
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint32_t e = raw[0][j] & 0x0F0F0F0Fu, o = (raw[0][j] >> 4) & 0x0F0F0F0Fu;
-            qm_dequant4_b4<DT>(e, o, 0, s0, b0, bq[0][j][0], bq[0][j][1]);
-            qm_dequant4_b4<DT>(e, o, 1, s0, b0, bq[0][j][2], bq[0][j][3]);
-        }
+        for (int hf = 0; hf < 8; hf++) convert_half(0, hf, s0, b0, bq[0][hf / 2][2 * (hf % 2)], bq[0][hf / 2][2 * (hf % 2) + 1]);
         scale_bias(1, sn, bn);
     }
     qm_u32x4 af[2][4];  // activation fragments of one 32-row block: [row block parity][MFMA step]
@@ -294,10 +322,9 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
                 issue_x(it + NBUF - 1, (u + NBUF - 1) % NBUF);
             }
             float sn2, bn2;
-            uint32_t ek = 0, ok = 0;
             // weights of the next iteration, issued WSN - 1 iterations ago: the loads younger than they are the tiles
             // of WSN iterations and the weights of WSN - 1 (ring of two: tiles and weights of two iterations)
-            qm_wait_vm_for<(NBUF == 2 ? 2 * IPW + 2 + 2 * NSB : WSN * IPW + WSN - 1 + WSN * NSB)>(raw[(u + 1) % WSN]);
+            wait_w(std::integral_constant<int, (NBUF == 2 ? 2 * IPW + 2 * NWL + 2 * NSB : WSN * (IPW + NSB) + (WSN - 1) * NWL)>{}, (u + 1) % WSN);
             qm_static_for<0, MB>([&](auto bi_c) {
                 constexpr int bi = decltype(bi_c)::value;
                 constexpr int par = bi & 1;
@@ -316,14 +343,8 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
                     acc[bi] = mfma32<DT>(av, bv, acc[bi]);
                     // its share of the next iteration's conversion: half fragments [8 m / NM, 8 (m + 1) / NM)
 #pragma unroll
-                    for (int hf = 8 * m / NM; hf < 8 * (m + 1) / NM; hf++) {
-                        const int jj = hf / 2, half = hf % 2;
-                        if (half == 0) {
-                            ek = raw[(u + 1) % WSN][jj] & 0x0F0F0F0Fu;
-                            ok = (raw[(u + 1) % WSN][jj] >> 4) & 0x0F0F0F0Fu;
-                        }
-                        qm_dequant4_b4<DT>(ek, ok, half, sn, bn, bq[nxt][jj][2 * half], bq[nxt][jj][2 * half + 1]);
-                    }
+                    for (int hf = 8 * m / NM; hf < 8 * (m + 1) / NM; hf++)
+                        convert_half((u + 1) % WSN, hf, sn, bn, bq[nxt][hf / 2][2 * (hf % 2)], bq[nxt][hf / 2][2 * (hf % 2) + 1]);
                 });
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -332,7 +353,7 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
             // this wave's share of the next tile (issued one iteration ago) is in LDS once at most this iteration's
             // loads are outstanding; past the barrier every wave's share is
             // (one less than the steady state allows: the first iterations follow the prologue's order)
-            qm_wait_vm<(NBUF == 2 ? 1 : NBUF == 3 ? IPW + 1 + NSB : (NBUF - 2) * (IPW + 1) - 1)>();
+            qm_wait_vm<(NBUF == 2 ? NWL : NBUF == 3 ? IPW + NWL + NSB : (NBUF - 2) * (IPW + NWL) - 1)>();
             __syncthreads();
 #pragma unroll
             for (int j = 0; j < 4; j++) af[0][j] = *(const qm_u32x4*)(lds + ((u + 1) % NBUF) * TILE + aoff[j]);

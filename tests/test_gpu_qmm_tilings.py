@@ -252,12 +252,12 @@ def test_tall_tiles_on_long_rows(oracle, M, N):
                                      (70, 131, 1024, 128),     # N % 8 != 0: element-wise stores
                                      (512, 384, 4096, 64),     # 64 groups per row: the 256-row tile's LDS is full to the byte
                                      (260, 128, 2816, 32)])    # 22 iterations (not a multiple of the unroll), 88 groups per row
-def test_load_to_lds_tiles(oracle, options, dt, M, N, K, G):
-    """The 4-bit instances whose activation tile arrives by load-to-LDS instructions, on 64-, 128- and 256-row
-    tiles, against the oracle's mma semantics (2e-2, as above) and against the register-staged instance of the
-    same tiling (same arithmetic, same order of the partial sums: bit-equal)."""
-    bits = 4
-    c = make_case(5400 + M + K, dt, bits, G, M, N, K)
+@pytest.mark.parametrize("bits", [4, 8])
+def test_load_to_lds_tiles(oracle, options, dt, M, N, K, G, bits):
+    """The 4- and 8-bit instances whose activation tile arrives by load-to-LDS instructions, on 64-, 128- and
+    256-row tiles, against the oracle's mma semantics (2e-2, as above) and against the register-staged instance of
+    the same tiling (same arithmetic, same order of the partial sums: bit-equal)."""
+    c = make_case(5400 + M + K + bits, dt, bits, G, M, N, K)
     exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
     exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
     w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
@@ -267,9 +267,9 @@ def test_load_to_lds_tiles(oracle, options, dt, M, N, K, G):
     for rows in (64, 128, 256):
         if rows == 256 and K // G > 64:
             continue  # two 64 KB tiles leave room for 64 groups per row
-        print(f"[case] load-to-LDS qmm {dt.name} M={M} N={N} K={K} g{G} tile_rows={rows}", flush=True)
+        print(f"[case] load-to-LDS qmm {dt.name} b{bits} M={M} N={N} K={K} g{G} tile_rows={rows}", flush=True)
         options("qmm.tile_rows", rows)
-        options("qmm.dma", 0)
+        options("qmm.dma", 3)
         out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
         ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
         got_bytes = out.read_bytes()
@@ -287,7 +287,7 @@ def test_load_to_lds_tiles(oracle, options, dt, M, N, K, G):
 
 
 def test_256_row_tiles_refuse_what_they_cannot_take(options):
-    """Forced 256-row tiles on a shape outside their limits (8-bit codes) are refused, not rerouted."""
+    """Forced 256-row tiles on a shape outside their limits (4 groups per row) are refused, not rerouted."""
     dt, bits, G, M, N, K = DType.BF16, 8, 64, 256, 128, 256
     c = make_case(5500, dt, bits, G, M, N, K)
     w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
@@ -308,20 +308,21 @@ def test_256_row_tiles_refuse_what_they_cannot_take(options):
                                      (512, 128, 4096, 64),     # 64 groups: whole rows fit, windows forced (2 windows)
                                      (64, 128, 2560, 64),      # 40 groups: the last window is partial (20 iterations)
                                      (96, 128, 11008, 64)])    # 172 groups: not whole 8-group vectors, 6 windows (the last of 12 groups)
-def test_load_to_lds_tiles_with_windowed_scales(oracle, options, dt, M, N, K, G):
+@pytest.mark.parametrize("bits", [4, 8])
+def test_load_to_lds_tiles_with_windowed_scales(oracle, options, dt, M, N, K, G, bits):
     """Rows too long for their scales and biases to sit in LDS whole: two windows of 32 groups refilled along K by
-    load-to-LDS instructions. Forced (qmm.dma = 2) on every tile height, against the oracle's mma semantics (2e-2)
-    and bit-equal to the register-staged instance of the same tiling."""
-    bits = 4
-    c = make_case(5600 + M + K, dt, bits, G, M, N, K)
+    load-to-LDS instructions. Forced (qmm.dma = 2) on every tile height (8-bit codes: 64 and 128 rows, the 256-row
+    instance does not fit the register file), against the oracle's mma semantics (2e-2) and bit-equal to the
+    register-staged instance of the same tiling."""
+    c = make_case(5600 + M + K + bits, dt, bits, G, M, N, K)
     exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
     exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
     w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
                   GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
     options("qmm.kernel", 2)
     options("qmm.kgroups", 2)
-    for rows in (64, 128, 256):
-        print(f"[case] windowed load-to-LDS qmm {dt.name} M={M} N={N} K={K} g{G} tile_rows={rows}", flush=True)
+    for rows in (64, 128, 256) if bits == 4 else (64, 128):
+        print(f"[case] windowed load-to-LDS qmm {dt.name} b{bits} M={M} N={N} K={K} g{G} tile_rows={rows}", flush=True)
         options("qmm.tile_rows", rows)
         options("qmm.dma", 2)
         out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
@@ -341,12 +342,12 @@ def test_load_to_lds_tiles_with_windowed_scales(oracle, options, dt, M, N, K, G)
 
 @pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
 @pytest.mark.parametrize("M,N,K,G", [(20, 200, 1024, 64), (64, 131, 2048, 32), (33, 128, 4096, 64), (50, 64, 768, 32)])
-def test_load_to_lds_tiles_on_4_kgroups(oracle, options, dt, M, N, K, G):
+@pytest.mark.parametrize("bits", [4, 8])
+def test_load_to_lds_tiles_on_4_kgroups(oracle, options, dt, M, N, K, G, bits):
     """The tilings of few rows (32 x 64 and 64 x 64 tiles on 4 K-groups, 256 k per iteration) with load-to-LDS
     activation tiles, unsplit and with K split over 1, 2 and 3 workgroups (f32 partial tiles added by the reduce
     kernel): the oracle's mma semantics (2e-2) and bit-equal to the register-staged instances."""
-    bits = 4
-    c = make_case(5700 + M + K, dt, bits, G, M, N, K)
+    c = make_case(5700 + M + K + bits, dt, bits, G, M, N, K)
     exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
     exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
     w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
@@ -357,17 +358,17 @@ def test_load_to_lds_tiles_on_4_kgroups(oracle, options, dt, M, N, K, G):
         for ksplit in (1, 2, 3):
             if ksplit > K // 256:
                 continue
-            print(f"[case] load-to-LDS qmm on 4 K-groups {dt.name} M={M} N={N} K={K} g{G} tile_rows={rows} ksplit={ksplit}", flush=True)
+            print(f"[case] load-to-LDS qmm on 4 K-groups {dt.name} b{bits} M={M} N={N} K={K} g{G} tile_rows={rows} ksplit={ksplit}", flush=True)
             options("qmm.tile_rows", rows)
             options("qmm.ksplit", ksplit)
             res = {}
-            for dma in (0, 1):
+            for dma in (3, 1):
                 options("qmm.dma", dma)
                 out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
                 ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
                 res[dma] = out.read_bytes()
                 out.free()
-            assert rel_err(unpack_f32(res[0], dt), exp) <= 2e-2, f"rows={rows} ksplit={ksplit}"
-            assert res[0] == res[1], f"rows={rows} ksplit={ksplit}: differs from the register-staged instance"
+            assert rel_err(unpack_f32(res[3], dt), exp) <= 2e-2, f"rows={rows} ksplit={ksplit}"
+            assert res[3] == res[1], f"rows={rows} ksplit={ksplit}: differs from the register-staged instance"
     for buf in (w, s, b, x):
         buf.free()

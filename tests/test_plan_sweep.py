@@ -132,7 +132,9 @@ def test_benchmark_configurations_are_routed_as_documented():
     assert "qmm_dma_kernel<2, 1, 4, 8," in ks[0]       # 32-row tiles on 4 K-groups, K split: a reduce kernel follows
     assert "qmm_split_reduce_kernel" in ks[1]
     ks, _ = kernels("qmm_mma", DType.BF16, 8, 64, 512, 4096, 4096)
-    assert "qmm_direct_kernel<2, 8," in ks[0]          # other code widths stay on the register-staged tiles
+    assert "qmm_dma_kernel<2, 2, 2, 8," in ks[0] and ks[0].rstrip(">(mtq::QmmDArgs)").endswith(", 8")   # 8-bit codes: the same tiles
+    ks, _ = kernels("qmm_mma", DType.BF16, 6, 64, 512, 4096, 4096)
+    assert "qmm_direct_kernel<2, 6," in ks[0]          # other code widths stay on the register-staged tiles
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 32)
     assert "qmv_mfma_kernel<2, 4," in ks[0]
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 4096, 4096, 8, 2048)
