@@ -68,6 +68,24 @@ static int dma_mode(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint3
 }
 static bool dma_fits(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr) { return dma_mode(bits, rows, kgroups, K, gpr) != 0; }
 
+// K-split load-to-LDS instances on 2 K-groups (64 x 128 and 128 x 128 tiles): every split stages its own share of
+// the tile's scales and biases, whole 8-group vectors, beside the ring of three tiles. Returns the LDS bytes, or 0
+// where the shape is not taken.
+static size_t dma_split_lds(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr, uint32_t iters_per_split, uint32_t ksplit) {
+    if (options().qmm_dma == 1 || (bits != 4 && bits != 8) || kgroups != 2 || K % 128 || gpr % 8 || ksplit < 2) return 0;
+    if (rows != 64 && rows != 128) return 0;
+    const uint32_t G = K / gpr, iters = K / 128;
+    uint32_t most = 0;   // the kernel's own count of groups per split, at its largest
+    for (uint32_t sp = 0; sp < ksplit; sp++) {
+        const uint32_t it0 = sp * iters_per_split, its = iters - it0 < iters_per_split ? iters - it0 : iters_per_split;
+        const uint32_t g0 = (it0 * 128 / G) & ~7u, ng_all = ((((it0 + its) * 128 - 1) / G + 1 - g0) + 7u) & ~7u;
+        const uint32_t ng = ng_all < gpr - g0 ? ng_all : gpr - g0;
+        most = ng > most ? ng : most;
+    }
+    const size_t need = qmm_dma_split_lds_bytes(rows, most);
+    return need <= 160 * 1024 ? need : 0;
+}
+
 template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, const LaunchCtx& lc, bool grouped = false) {
     const void* fn = nullptr;
     // 8-bit codes on short rows gain nothing where the launch leaves compute units idle (14336 x 4096, 128 rows:
@@ -76,6 +94,24 @@ template <int DT> static int launch_dt(QmmDArgs& a, int bits, uint32_t kgroups, 
     const bool b8_short = bits == 8 && a.K < 8192 && options().qmm_dma < 2;
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (const size_t shmem = grouped ? 0 : dma_split_lds(bits, a.m_tile_rows, kgroups, a.K, a.gpr, a.iters_per_split, a.ksplit)) {
+        fn = qmm_dma_split_pick(bits, DT, a.m_tile_rows);
+        hipError_t e = set_max_dynamic_lds(fn, shmem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
+        void* args[] = {&a};
+        LaunchCtx l1 = lc, l2 = lc;
+        l1.stop = nullptr;
+        l2.start = nullptr;
+        e = launch_kernel(fn, dim3(a.m_tiles * a.n_tiles, a.ksplit), dim3(512), args, shmem, l1);
+        if (e != hipSuccess) return hip_fail(e, "qmm load-to-LDS kernel launch");
+        const float* part = a.part;
+        void* out = a.out;
+        uint32_t total = a.M * a.N, ks = a.ksplit;
+        void* rargs[] = {&part, &out, &total, &ks};
+        e = launch_kernel((const void*)qmm_split_reduce_kernel<DT>, dim3((total + 255) / 256), dim3(256), rargs, 0, l2);
+        if (e != hipSuccess) return hip_fail(e, "qmm split reduce kernel launch");
+        return ERR_OK;
+    }
     if (a.ksplit <= 1 && dma_fits(bits, a.m_tile_rows, kgroups, a.K, a.gpr) && (!grouped || a.m_tile_rows == 64) &&
         !(b8_short && !grouped && a.m_tile_rows != 256 && (uint64_t)a.m_tiles * a.n_tiles < (uint64_t)cus)) {
         const bool windowed = dma_mode(bits, a.m_tile_rows, kgroups, a.K, a.gpr) == 2;
@@ -273,6 +309,23 @@ static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
             if (best == 0.0 || est < best) { best = est; rows = heights[i]; kgroups = 2; }
         }
     }
+    // Long rows and too few 128 x 128 tiles for the chip (a down projection at 100..512 rows): the load-to-LDS tall
+    // tile with K split so that every compute unit has one workgroup. us, the choice above -> this one:
+    // 4096 x 14336, 128 / 256 / 384 / 512 rows 36.3 / 60.7 / 82.0 / 97.4 -> 31.7 / 47.3 / 75.5 / 80.7 (8-bit codes
+    // 44.5 / 72.7 / 96.7 / 116.9 -> 39.1 / 56.1 / 86.8 / 92.7); 4096 x 8192, 256 / 384 / 512 rows 39.8 / 43.4 / 50.9 ->
+    // 31.3 / 40.4 / 48.4 (128 rows lose, 22.0 -> 24.3); 5120 x 13824, 128 / 256 / 384 rows 47.9 / 70.7 / 92.2 -> 37.4 /
+    // 55.6 / 75.9; 8192 x 28672 (a split's scales fit LDS from 4 splits on), 128 / 256 rows 163.5 / 184.4 -> 84.7 / 156.7.
+    uint32_t dma_ks = 0;
+    if (!options().qmm_tile_rows && !options().qmm_kgroups && options().qmm_ksplit == 0 && p.K >= 8192 &&
+        (p.M > 128 || (p.M > 96 && p.K > 8192)) && tall_wide * 2 <= (uint64_t)cus && (uint64_t)p.M * p.N < (1ull << 31)) {
+        uint32_t ks = (uint32_t)((uint64_t)cus / tall_wide);
+        ks = ks > 8 ? 8 : ks;
+        for (int attempt = 0; attempt < 2 && !dma_ks && ks <= 8; attempt++, ks *= 2) {
+            const uint32_t its = p.K / 128, ips = (its + ks - 1) / ks, eff = (its + ips - 1) / ips;
+            if (eff >= 2 && dma_split_lds(p.bits, 128, 2, p.K, p.K / G, ips, eff)) dma_ks = ks;
+        }
+        if (dma_ks) { rows = 128; kgroups = 2; }
+    }
     if (options().qmm_tile_rows) rows = (uint32_t)options().qmm_tile_rows;
     if (options().qmm_kgroups) kgroups = (uint32_t)options().qmm_kgroups;
     // An iteration covers 64 k per K-group: K must be a multiple of 64 * K-groups (an odd number of
@@ -300,12 +353,13 @@ static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
     const uint32_t iters = p.K / (64 * kgroups);
     uint32_t ks = 1;
     if (options().qmm_ksplit > 1) ks = (uint32_t)options().qmm_ksplit;
+    else if (dma_ks) ks = dma_ks;
     else if (options().qmm_ksplit == 0 && rows == 128 && kgroups == 1 && p.K >= 8192 && tiles < 2 * (uint64_t)cus) {
         // tall tiles on long rows: splits to about two 4-wave workgroups per compute unit, rounded
         ks = (uint32_t)((4 * (uint64_t)cus / tiles + 1) / 2);
         if (ks > 8) ks = 8;
         if (ks > iters / 16) ks = iters / 16;
-    } else if (options().qmm_ksplit == 0 && tiles * 2 <= (uint64_t)cus && iters >= QMM_SPLIT_MIN_ITERS) {
+    } else if (options().qmm_ksplit == 0 && kgroups != 2 && tiles * 2 <= (uint64_t)cus && iters >= QMM_SPLIT_MIN_ITERS) {
         // one workgroup per compute unit, at least 4 iterations each (measured optimum: 4096 x 14336,
         // 32 rows, 64 tiles: 1 / 2 / 4 / 8 / 16 splits 57 / 34 / 23 / 27 / 32 us; 2048 x 8192, 32 tiles:
         // 23 / 17 / 12 / 11 / 12 us; 8192 x 28672, 128 tiles: 108 / 63 / 62 / 66 / 80 us)
@@ -315,9 +369,12 @@ static int plan_direct(const QmmParams& p, QmmDPlan& pl) {
     }
     if (ks > iters) ks = iters;
     if (ks < 1 || (uint64_t)p.M * p.N >= (1ull << 31)) ks = 1;  // the reduction indexes the output with 32 bits
-    if (!qmm_direct_split_built(rows, kgroups)) ks = 1;
     pl.iters_per_split = (iters + ks - 1) / ks;
     pl.ksplit = (iters + pl.iters_per_split - 1) / pl.iters_per_split;  // no empty split
+    if (!qmm_direct_split_built(rows, kgroups) && !dma_split_lds(p.bits, rows, kgroups, p.K, p.K / G, pl.iters_per_split, pl.ksplit)) {
+        pl.ksplit = 1;
+        pl.iters_per_split = iters;
+    }
     return ERR_OK;
 }
 

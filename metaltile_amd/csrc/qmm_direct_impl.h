@@ -351,6 +351,8 @@ const void* qmm_direct_pick_odd(int dtype, int bits, uint32_t kgroups, uint32_t 
 const void* qmm_dma_pick(int bits, int dtype, uint32_t tile_rows, bool grouped, bool windowed, bool shallow);
 size_t qmm_dma_lds_bytes(uint32_t tile_rows, uint32_t gpr, bool windowed, bool shallow);
 // The same on 4 K-groups (32 x 64 and 64 x 64 tiles, K a multiple of 256), plain or K-split.
+size_t qmm_dma_split_lds_bytes(uint32_t tile_rows, uint32_t groups);
+const void* qmm_dma_split_pick(int bits, int dtype, uint32_t tile_rows);
 const void* qmm_dma4_pick(int bits, int dtype, uint32_t tile_rows, bool split, bool grouped);
 size_t qmm_dma4_lds_bytes(uint32_t tile_rows, uint32_t gpr);
 

@@ -24,10 +24,24 @@ size_t qmm_dma_lds_bytes(uint32_t rows, uint32_t gpr, bool windowed, bool shallo
 }
 
 const void* qmm_dma_pick_b8(int dtype, uint32_t rows, bool grouped, bool windowed, bool shallow);
+const void* qmm_dma_split_pick_b8(int dtype, uint32_t rows);
 const void* qmm_dma4_pick_b8(int dtype, uint32_t rows, bool split, bool grouped);
 
 const void* qmm_dma_pick(int bits, int dtype, uint32_t rows, bool grouped, bool windowed, bool shallow) {
     return bits == 8 ? qmm_dma_pick_b8(dtype, rows, grouped, windowed, shallow) : qmm_dma_pick_t<4>(dtype, rows, grouped, windowed, shallow);
+}
+
+// K-split instances on 2 K-groups: `groups` = the most groups of scales one split's share of a row spans (whole
+// 8-group vectors)
+size_t qmm_dma_split_lds_bytes(uint32_t rows, uint32_t groups) {
+    const uint32_t mb = rows / 32, dbn = 128, kg = 2;
+    const size_t main_loop = (size_t)3 * mb * kg * 4096 + (size_t)2 * dbn * (groups + 2) * 2;
+    const size_t epilogue = (size_t)(kg - 1) * 4 * mb * 16 * 64 * 4;
+    return main_loop > epilogue ? main_loop : epilogue;
+}
+
+const void* qmm_dma_split_pick(int bits, int dtype, uint32_t rows) {
+    return bits == 8 ? qmm_dma_split_pick_b8(dtype, rows) : qmm_dma_split_pick_t<4>(dtype, rows);
 }
 
 // 4 K-groups x 2 column waves (32 x 64 and 64 x 64 tiles, 256 k per iteration): the tilings of few rows, also as

@@ -8,6 +8,7 @@ namespace mtq {
 const void* qmm_dma_pick_b8(int dtype, uint32_t rows, bool grouped, bool windowed, bool shallow) {
     return qmm_dma_pick_t<8>(dtype, rows, grouped, windowed, shallow);
 }
+const void* qmm_dma_split_pick_b8(int dtype, uint32_t rows) { return qmm_dma_split_pick_t<8>(dtype, rows); }
 const void* qmm_dma4_pick_b8(int dtype, uint32_t rows, bool split, bool grouped) { return qmm_dma4_pick_t<8>(dtype, rows, split, grouped); }
 
 }  // namespace mtq

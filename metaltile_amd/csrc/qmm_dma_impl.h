@@ -172,7 +172,7 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     // rows padded by two elements, or (256-row tiles: no room for padding) row r rotated by 8 r elements, so that
     // the 32 rows a wave reads one group of do not all fall into one bank
     constexpr bool ROT = NBUF != 3;
-    const uint32_t sbld = ROT ? sb_ng : a.gpr + 2;
+    const uint32_t sbld = ROT ? sb_ng : sb_ng + 2;   // (a K split stages its own share of the groups only)
     uint16_t* sbS = (uint16_t*)(lds + NBUF * TILE);
     uint16_t* sbB = sbS + DBN * sbld;
     const int sbrow = (int)((wn * 32 + fr) * sbld) - (ROT ? 0 : (int)sb_g0);

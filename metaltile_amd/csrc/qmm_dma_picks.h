@@ -34,6 +34,15 @@ template <int BITS> const void* qmm_dma_pick_t(int dtype, uint32_t rows, bool gr
 }
 
 
+// K-split instances of the 64 x 128 and 128 x 128 tiles (f32 partial tiles, a ring of three, whole groups of the split's
+// share of the rows in LDS)
+template <int BITS> const void* qmm_dma_split_pick_t(int dtype, uint32_t rows) {
+    if (rows != 64 && rows != 128) return nullptr;
+    if (dtype == DT_BF16) return rows == 64 ? (const void*)qmm_dma_kernel<DT_BF16, 2, 2, 8, 0, false, true, false, BITS> : (const void*)qmm_dma_kernel<DT_BF16, 4, 2, 8, 0, false, true, false, BITS>;
+    if (dtype == DT_F16) return rows == 64 ? (const void*)qmm_dma_kernel<DT_F16, 2, 2, 8, 0, false, true, false, BITS> : (const void*)qmm_dma_kernel<DT_F16, 4, 2, 8, 0, false, true, false, BITS>;
+    return nullptr;
+}
+
 template <int BITS> const void* qmm_dma4_pick_t(int dtype, uint32_t rows, bool split, bool grouped) {
     if (grouped) {
         if (split || (rows != 32 && rows != 64)) return nullptr;

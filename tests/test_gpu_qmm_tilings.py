@@ -372,3 +372,39 @@ def test_load_to_lds_tiles_on_4_kgroups(oracle, options, dt, M, N, K, G, bits):
             assert res[3] == res[1], f"rows={rows} ksplit={ksplit}: differs from the register-staged instance"
     for buf in (w, s, b, x):
         buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M,N,K,G", [(130, 200, 4096, 64),     # 32 iterations, ragged tiles both ways
+                                     (257, 131, 2048, 32),     # N % 8 != 0
+                                     (64, 128, 14336, 64),     # 112 iterations, 224 groups: whole rows would not fit beside 128-row tiles
+                                     (300, 256, 3072, 128)])   # 24 groups: splits share 8-group vectors of scales
+def test_load_to_lds_tiles_with_k_split(oracle, options, dt, M, N, K, G, bits):
+    """64 x 128 and 128 x 128 load-to-LDS tiles with K split over 2, 3 and 5 workgroups (f32 partial tiles added in
+    split order by the reduce kernel; every split stages its own share of the scales): the oracle's mma semantics
+    (2e-2), and the unsplit instance's result to within the rounding of the element type (the sums are the same
+    terms added in another order)."""
+    c = make_case(5800 + M + K + bits, dt, bits, G, M, N, K)
+    exp = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, ODT[dt], threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    options("qmm.kernel", 2)
+    options("qmm.kgroups", 2)
+    for rows in (64, 128):
+        options("qmm.tile_rows", rows)
+        got = {}
+        for ksplit in (1, 2, 3, 5):
+            print(f"[case] K-split load-to-LDS qmm {dt.name} b{bits} M={M} N={N} K={K} g{G} tile_rows={rows} ksplit={ksplit}", flush=True)
+            options("qmm.ksplit", ksplit)
+            out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
+            ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+            got[ksplit] = unpack_f32(out.read_bytes(), dt)
+            out.free()
+            assert rel_err(got[ksplit], exp) <= 2e-2, f"rows={rows} ksplit={ksplit}"
+            if ksplit > 1:
+                scale = float(np.abs(got[1]).max())
+                assert float(np.abs(got[ksplit] - got[1]).max()) <= (2.0 ** -7 if dt == DType.BF16 else 2.0 ** -10) * scale * 2
+    for buf in (w, s, b, x):
+        buf.free()

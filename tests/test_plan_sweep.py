@@ -133,6 +133,9 @@ def test_benchmark_configurations_are_routed_as_documented():
     assert "qmm_split_reduce_kernel" in ks[1]
     ks, _ = kernels("qmm_mma", DType.BF16, 8, 64, 512, 4096, 4096)
     assert "qmm_dma_kernel<2, 2, 2, 8," in ks[0] and ks[0].rstrip(">(mtq::QmmDArgs)").endswith(", 8")   # 8-bit codes: the same tiles
+    for bits in (4, 8):     # a down projection at 512 rows: 128 tall tiles, K split in two so that every compute unit has one
+        ks, ls = kernels("qmm_mma", DType.BF16, bits, 64, 512, 4096, 14336)
+        assert "qmm_dma_kernel<2, 4, 2, 8, 0, false, true, false" in ks[0] and ls[0][1][:2] == (128, 2) and "qmm_split_reduce_kernel" in ks[1]
     ks, _ = kernels("qmm_mma", DType.BF16, 6, 64, 512, 4096, 4096)
     assert "qmm_direct_kernel<2, 6," in ks[0]          # other code widths stay on the register-staged tiles
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 32)
