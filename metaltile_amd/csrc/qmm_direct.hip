@@ -69,16 +69,18 @@ static int dma_mode(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint3
 static bool dma_fits(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr) { return dma_mode(bits, rows, kgroups, K, gpr) != 0; }
 
 // K-split load-to-LDS instances on 2 K-groups (64 x 128 and 128 x 128 tiles): every split stages its own share of
-// the tile's scales and biases, whole 8-group vectors, beside the ring of three tiles. Returns the LDS bytes, or 0
+// the tile's scales and biases (whole 8-group vectors, or pairs of groups where rows are not whole vectors) beside the
+// ring of three tiles. Returns the LDS bytes, or 0
 // where the shape is not taken.
 static size_t dma_split_lds(int bits, uint32_t rows, uint32_t kgroups, uint32_t K, uint32_t gpr, uint32_t iters_per_split, uint32_t ksplit) {
-    if (options().qmm_dma == 1 || (bits != 4 && bits != 8) || kgroups != 2 || K % 128 || gpr % 8 || ksplit < 2) return 0;
+    if (options().qmm_dma == 1 || (bits != 4 && bits != 8) || kgroups != 2 || K % 128 || gpr % 2 || ksplit < 2) return 0;
     if (rows != 64 && rows != 128) return 0;
     const uint32_t G = K / gpr, iters = K / 128;
     uint32_t most = 0;   // the kernel's own count of groups per split, at its largest
     for (uint32_t sp = 0; sp < ksplit; sp++) {
         const uint32_t it0 = sp * iters_per_split, its = iters - it0 < iters_per_split ? iters - it0 : iters_per_split;
-        const uint32_t g0 = (it0 * 128 / G) & ~7u, ng_all = ((((it0 + its) * 128 - 1) / G + 1 - g0) + 7u) & ~7u;
+        const uint32_t al = gpr % 8 ? 1u : 7u;
+        const uint32_t g0 = (it0 * 128 / G) & ~al, ng_all = ((((it0 + its) * 128 - 1) / G + 1 - g0) + al) & ~al;
         const uint32_t ng = ng_all < gpr - g0 ? ng_all : gpr - g0;
         most = ng > most ? ng : most;
     }

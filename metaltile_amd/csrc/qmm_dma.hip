@@ -32,10 +32,10 @@ const void* qmm_dma_pick(int bits, int dtype, uint32_t rows, bool grouped, bool 
 }
 
 // K-split instances on 2 K-groups: `groups` = the most groups of scales one split's share of a row spans (whole
-// 8-group vectors)
+// 8-group vectors, or whole dwords where a row is not whole vectors)
 size_t qmm_dma_split_lds_bytes(uint32_t rows, uint32_t groups) {
     const uint32_t mb = rows / 32, dbn = 128, kg = 2;
-    const size_t main_loop = (size_t)3 * mb * kg * 4096 + (size_t)2 * dbn * (groups + 2) * 2;
+    const size_t main_loop = (size_t)3 * mb * kg * 4096 + (size_t)2 * dbn * (((groups + 3) & ~3u) + 2) * 2;
     const size_t epilogue = (size_t)(kg - 1) * 4 * mb * 16 * 64 * 4;
     return main_loop > epilogue ? main_loop : epilogue;
 }

@@ -141,9 +141,11 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
         a.w += (size_t)it_base * (DBK * BITS / 8);
     }
     const uint32_t ilast = a.iters - 1;
-    // groups of scales / biases this workgroup needs: [sb_g0, sb_g0 + sb_ng), whole 8-element vectors
-    const uint32_t sb_g0 = ((it_base * DBK) >> a.log2g) & ~7u;
-    const uint32_t sb_ng = min(a.gpr - sb_g0, (((((it_base + a.iters) * DBK - 1) >> a.log2g) + 1 - sb_g0) + 7u) & ~7u);
+    // groups of scales / biases this workgroup needs: [sb_g0, sb_g0 + sb_ng), whole 8-element vectors (rows that are
+    // not whole vectors, K-split instances only: whole dwords, two groups)
+    const uint32_t sb_al = (a.gpr & 7u) ? 1u : 7u;
+    const uint32_t sb_g0 = ((it_base * DBK) >> a.log2g) & ~sb_al;
+    const uint32_t sb_ng = min(a.gpr - sb_g0, (((((it_base + a.iters) * DBK - 1) >> a.log2g) + 1 - sb_g0) + sb_al) & ~sb_al);
 
     // ---- per-lane offsets ---------------------------------------------------------------------------
     // this wave's load-to-LDS instructions: unit q = wave * IPW + i is quarter q % 4 of slot q / 4; slot sl holds
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     // rows padded by two elements, or (256-row tiles: no room for padding) row r rotated by 8 r elements, so that
     // the 32 rows a wave reads one group of do not all fall into one bank
     constexpr bool ROT = NBUF != 3;
-    const uint32_t sbld = ROT ? sb_ng : sb_ng + 2;   // (a K split stages its own share of the groups only)
+    const uint32_t sbld = ROT ? sb_ng : ((sb_ng + 3u) & ~3u) + 2;   // (a K split stages its own share of the groups only)
     uint16_t* sbS = (uint16_t*)(lds + NBUF * TILE);
     uint16_t* sbB = sbS + DBN * sbld;
     const int sbrow = (int)((wn * 32 + fr) * sbld) - (ROT ? 0 : (int)sb_g0);
@@ -269,6 +271,15 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
             const uint32_t grp = min(win * 32u + c * 8u + dw * 2u, a.gpr - 2u);
             const uint32_t val = *(const uint32_t*)((const uint16_t*)(isb ? a.biases : a.scales) + (size_t)min(n0 + col, a.N - 1) * a.gpr + grp);
             *(uint32_t*)(lds + NBUF * TILE + win * 16384u + isb * 8192u + col * 64u + ((c ^ ((col >> 1) & 3u)) << 4) + dw * 4u) = val;
+        }
+    } else if (!ROT && (a.gpr & 7u)) {
+        // rows of scales that are not whole 16-byte vectors: a dword (two groups) per load
+        const uint32_t dpr = sb_ng / 2, ndw = DBN * dpr;
+        for (uint32_t v = tid; v < ndw; v += NT) {
+            const uint32_t row = v / dpr, c0 = (v - row * dpr) * 2;
+            const uint32_t grow = min(n0 + row, a.N - 1);
+            *(uint32_t*)(sbS + row * sbld + c0) = *(const uint32_t*)((const uint16_t*)a.scales + (size_t)grow * a.gpr + sb_g0 + c0);
+            *(uint32_t*)(sbB + row * sbld + c0) = *(const uint32_t*)((const uint16_t*)a.biases + (size_t)grow * a.gpr + sb_g0 + c0);
         }
     } else {
         // DBN rows x sb_ng elements each of scales and biases, 16 bytes per load (ordinary loads: the compiler waits)

@@ -379,7 +379,8 @@ def test_load_to_lds_tiles_on_4_kgroups(oracle, options, dt, M, N, K, G, bits):
 @pytest.mark.parametrize("M,N,K,G", [(130, 200, 4096, 64),     # 32 iterations, ragged tiles both ways
                                      (257, 131, 2048, 32),     # N % 8 != 0
                                      (64, 128, 14336, 64),     # 112 iterations, 224 groups: whole rows would not fit beside 128-row tiles
-                                     (300, 256, 3072, 128)])   # 24 groups: splits share 8-group vectors of scales
+                                     (300, 256, 3072, 128),    # 24 groups: splits share 8-group vectors of scales
+                                     (96, 136, 11008, 64)])    # 172 groups: rows of scales are not whole vectors (staged by dwords)
 def test_load_to_lds_tiles_with_k_split(oracle, options, dt, M, N, K, G, bits):
     """64 x 128 and 128 x 128 load-to-LDS tiles with K split over 2, 3 and 5 workgroups (f32 partial tiles added in
     split order by the reduce kernel; every split stages its own share of the scales): the oracle's mma semantics
