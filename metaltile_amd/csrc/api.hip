@@ -226,12 +226,36 @@ static int try_f32_tiles(int bits, uint32_t G, const void* w, const void* s, con
     return launch_qmm_f32(q, lc, need ? (char*)g.scratch_buf + g.scratch_held : nullptr);
 }
 
+
+// Batches of 5..16 rows on the 16-row matrix-core GEMV where the shape allows and it is the fastest kernel;
+// ERR_UNSUPPORTED otherwise. `exact`: the caller's alternative is the GEMV family (passes of up to 8 rows, the
+// same exact-dequant arithmetic); else it is the tile kernel.
+static int try_wide(int dtype, int bits, uint32_t G, const void* w, const void* s, const void* b, const void* x,
+                    void* out, uint32_t M, uint32_t N, uint32_t K, bool exact, const LaunchCtx& lc) {
+    if (M < 5 || M > 16 || options().qmv_wide == 1) return ERR_UNSUPPORTED;
+    QmmParams q;
+    q.dtype = dtype; q.bits = bits; q.group_size = G;
+    q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
+    q.M = M; q.N = N; q.K = K;
+    if (!qmv_wide_takes(q)) return ERR_UNSUPPORTED;
+    (void)exact;
+    if (options().qmv_wide != 2) return ERR_UNSUPPORTED;
+    const size_t need = qmv_wide_scratch_bytes(q);
+    if (need) {
+        int rc = ensure_scratch(g.scratch_held + need);
+        if (rc) return rc;
+    }
+    return launch_qmv_wide(q, lc, need ? (char*)g.scratch_buf + g.scratch_held : nullptr);
+}
+
 static int op_qmv(int dtype, int bits, uint32_t G, const void* w, const void* s, const void* b,
                   const void* x, void* out, uint32_t M, uint32_t N, uint32_t K, const LaunchCtx& lc) {
     int rc = check_common(dtype, bits, G, N, K);
     if (rc) return rc;
     if (M == 0) return ERR_OK;
     if (!w || !s || !b || !x || !out) return fail(ERR_BAD_ARG, "null buffer");
+    rc = try_wide(dtype, bits, G, w, s, b, x, out, M, N, K, true, lc);
+    if (rc != ERR_UNSUPPORTED) return rc;
     if (dtype == DT_F32) {
         rc = try_f32_tiles(bits, G, w, s, b, x, out, M, N, K, lc);
         if (rc != ERR_UNSUPPORTED) return rc;
@@ -264,6 +288,10 @@ static int op_qmm(int dtype, int bits, uint32_t G, const void* w, const void* s,
     // matrices leave it few row blocks; the split-K tiles are ahead there (8 rows, GEMV against tiles:
     // 4096 x 14336 26 / 22 us, 1024 x 4096 14 / 10, 8192 x 28672 107 / 62, 28672 x 8192 56 / 39; but
     // 14336 x 4096 12 / 14, 128256 x 4096 70 / 84).
+    if (!force_mma) {
+        rc = try_wide(dtype, bits, G, w, s, b, x, out, M, N, K, false, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
     const bool long_rows = M >= 5 && ((uint64_t)K >= 2 * (uint64_t)N || (K >= 8192 && (uint64_t)N >= 3 * (uint64_t)K));
     if (M >= 9 || long_rows || force_mma || bits == 7) {
         QmmParams q;
@@ -1385,6 +1413,21 @@ int mtq_set_option(const char* name, int value) {
     if (!strcmp(name, "qmv.mfma")) {
         if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmv.mfma must be 0 (auto), 1 (off) or 2 (prefer)");
         options().qmv_mfma = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmv.wide_kp")) {
+        if (value < 0 || value > 16 || (value & (value - 1))) return fail(ERR_BAD_ARG, "qmv.wide_kp must be 0, 1, 2, 4, 8 or 16");
+        options().qmv_wide_kp = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmv.wide_nb")) {
+        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmv.wide_nb must be 0, 1 or 2");
+        options().qmv_wide_nb = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmv.wide")) {
+        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmv.wide must be 0 (choose), 1 (never) or 2 (wherever the shape allows)");
+        options().qmv_wide = value;
         return MTQ_OK;
     }
     if (!strcmp(name, "qmv.mfma_sets")) {

@@ -110,6 +110,9 @@ struct Options {
     int qmv_mfma_rbw = 0;         // matrix-core qmv: row blocks walked in parallel per workgroup
     int qmv_mfma_nrb = 0;         // matrix-core qmv: row blocks per wave
     int qmv_mfma_sets = 0;        // matrix-core gather: 4-row MFMA sets per pass (0 = choose; 1, 2, 4)
+    int qmv_wide_kp = 0;          // 16-row matrix-core GEMV: waves sharing a row block (0 = choose; 1, 2, 4, 8, 16)
+    int qmv_wide_nb = 0;          // 16-row matrix-core GEMV: row blocks per wave (0 = choose; 1, 2)
+    int qmv_wide = 0;             // 16-row matrix-core GEMV for batches of 5..16 rows: 0 = choose per shape, 1 = never, 2 = wherever the shape allows
 };
 Options& options();
 
@@ -165,6 +168,11 @@ int launch_qmm_mfma(const QmmParams& p, const LaunchCtx& lc);
 // scratch: qmm_direct_scratch_bytes(p) bytes (0 when K is not split: then scratch may be null).
 size_t qmm_direct_scratch_bytes(const QmmParams& p);
 int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc, void* scratch);
+// 16-row matrix-core GEMV (qmv_wide.hip): 4-bit codes, f16 / bf16, at most 16 rows, K % 512 == 0.
+// scratch: qmv_wide_scratch_bytes(p) bytes (0 when K is not split: then scratch may be null).
+bool qmv_wide_takes(const QmmParams& p);
+size_t qmv_wide_scratch_bytes(const QmmParams& p);
+int launch_qmv_wide(const QmmParams& p, const LaunchCtx& lc, void* scratch);
 // f32 operands on the f32 matrix cores, any code width (qmm_f32.hip).
 // scratch: qmm_f32_scratch_bytes(p) bytes (0 when K is not split: then scratch may be null).
 size_t qmm_f32_scratch_bytes(const QmmParams& p);

@@ -1,0 +1,68 @@
+"""The 16-row matrix-core GEMV (qmv_wide_kernel: 4-bit codes, f16 / bf16, batches of up to 16 rows on the
+16x16x32 MFMA), forced through the library's option on shapes that exercise every branch of its geometry, against
+the f64-accumulated oracle of the exact-dequant form (out = sum_g s * sum q x + b * sum x, the arithmetic of the
+reference's mt_qmm, crates/metaltile-std/src/mlx/quantized.rs:1330-1500). Tolerance on max|a-e|/max(|e|,1): 1e-2
+for f16 / bf16, the benchmark configurations' bound."""
+import numpy as np
+import pytest
+
+from metaltile_amd import DType, GpuBuffer, _lib, ops, unpack_f32
+from metaltile_amd.synth import make_case
+from tests.parity import rel_err
+
+pytestmark = pytest.mark.gpu
+ODT = {DType.F16: 1, DType.BF16: 2}
+
+
+@pytest.fixture
+def wide():
+    lib = _lib.load()
+    assert lib.mtq_set_option(b"qmv.wide", 2) == 0
+
+    def geometry(kp, nb):
+        assert lib.mtq_set_option(b"qmv.wide_kp", kp) == 0 and lib.mtq_set_option(b"qmv.wide_nb", nb) == 0
+
+    yield geometry
+    for name in (b"qmv.wide", b"qmv.wide_kp", b"qmv.wide_nb"):
+        lib.mtq_set_option(name, 0)
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("M,N,K,G", [(16, 512, 1024, 64),     # two turns per row block, every wave of two workgroups busy
+                                     (5, 100, 512, 64),       # one turn (odd total), ragged last row block, rows 5..15 repeated
+                                     (9, 4100, 1536, 32),     # three turns, groups of 32: a group per MFMA; 257 row blocks
+                                     (13, 333, 2048, 128),    # groups of 128: 8-byte scale loads
+                                     (16, 40, 5120, 64),      # ten turns: K split in two slices of five (f32 partial rows)
+                                     (7, 8200, 14336, 64),    # 28 turns in four slices of seven; several row blocks per wave
+                                     (12, 70000, 512, 128)])  # 4375 row blocks: waves walk up to two blocks of one turn each
+@pytest.mark.parametrize("kp,nb", [(0, 0), (1, 2), (4, 1), (16, 2)], ids=lambda v: str(v))
+def test_wide_gemv(oracle, wide, dt, M, N, K, G, kp, nb):
+    """kp, nb: waves that share a row block (each with a run of the turns; their sums meet in LDS) and row blocks
+    per wave, chosen by the library (0, 0) or forced."""
+    bits = 4
+    wide(kp, nb)
+    c = make_case(6100 + M + N % 97, dt, bits, G, M, N, K, bias_rule="midpoint")
+    print(f"[case] wide qmv {dt.name} g{G} M{M} N{N} K{K} kp={kp} nb={nb}", flush=True)
+    exp = oracle.qmm_f64(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, bits, G, threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
+    ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
+    got = unpack_f32(out.read_bytes(), dt)
+    assert rel_err(got, exp) <= 1e-2
+    for buf in (w, s, b, x, out):
+        buf.free()
+
+
+def test_wide_gemv_is_the_kernel_that_ran(wide):
+    """The forced route is the wide kernel (a K split adds its reduce kernel), and shapes outside its limits fall
+    through to the other kernels instead of failing."""
+    rc, launches, scratch, n = ops.plan("qmm", DType.BF16, 4, 64, 16, 8192, 4096)
+    assert rc == 0 and n == 1 and "qmv_wide_kernel<2, 64, " in launches[0][0] and launches[0][2][0] == 1024
+    rc, launches, scratch, n = ops.plan("qmm", DType.F16, 4, 32, 9, 8192, 8192)
+    assert rc == 0 and n == 2 and "qmv_wide_kernel<1, 32, 1>" in launches[0][0] and "qmv_wide_reduce_kernel" in launches[1][0]
+    assert launches[0][1][1] == 2 and scratch >= 2 * 9 * 8192 * 4
+    for args in ((DType.BF16, 8, 64, 16, 8192, 4096), (DType.BF16, 4, 64, 16, 8192, 4352), (DType.BF16, 4, 64, 17, 8192, 4096)):
+        rc, launches, _, n = ops.plan("qmm", *args)
+        assert rc == 0 and all("qmv_wide" not in l[0] for l in launches)
