@@ -22,7 +22,9 @@ and the Mixtral-style gather_qmv (8 experts of 14336 x 4096, 32 routed rows;
 bound: HBM on the bytes of the experts that are hit), each with its own
 roofline object. `value`, `ms_per_step` and `steps` describe the qmv region
 only. `--workload sweep` reports the 18 cells of the bit-width / group-size
-sweep (f16, 8192 x 8192, batch 1 and 4).
+sweep (f16, 8192 x 8192, batch 1 and 4); `--workload batch` a decode batch of
+`--rows` rows (default 16) against one large matrix (`--shape`, default the
+128256 x 4096 lm-head), by the exact-dequant kernel name mt_qmm.
 
 Prints ONE JSON line on stdout.
 """
@@ -48,7 +50,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=8, help="distinct MLP weight sets streamed per step")
     ap.add_argument("--workload", default="qmv",
-                    choices=["qmv", "qkv", "qmm", "gather", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep"],
+                    choices=["qmv", "qkv", "qmm", "batch", "gather", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep"],
                     help="qmv is the headline (its line also carries qmm M=512 and the gather as secondary legs); "
                          "qmm / gather report those configurations alone; sweep the bit-width / group-size cells; "
                          "copy runs only the known-size copy kernel (counter calibration); read times a kernel that only reads the "
@@ -56,6 +58,8 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-secondary", action="store_true", help="qmv workload: skip the qmm M=512 and gather legs")
     ap.add_argument("--m", type=int, default=512, help="qmm workload: activation rows")
+    ap.add_argument("--rows", type=int, default=16, help="batch workload: activation rows (a decode batch)")
+    ap.add_argument("--shape", default="128256x4096", help="batch workload: weight matrix N x K")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--hot", action="store_true", help="re-use one weight set (cache-resident) instead of rotating")
     return ap.parse_args()
@@ -255,6 +259,45 @@ def leg_qmm(a, runner, info, M=512):
     }
 
 
+def leg_batch(a, runner, info):
+    """A decode batch of a few rows against one large matrix (the lm-head of Llama-3: 128256 x 4096), by the
+    exact-dequant kernel name mt_qmm: bound by the weight stream, so reported against the HBM roofline."""
+    import numpy as np
+    from metaltile_amd import DType, GpuBuffer, pack_f32
+    dt = DType.BF16
+    N, K = (int(v) for v in a.shape.split("x"))
+    M, G = a.rows, 64
+    rng = np.random.default_rng(7)
+    sets = 1 if a.hot else 4
+    specs, keep = [], []
+    for i in range(sets):
+        bufs = {"w": GpuBuffer.from_bytes(rng.integers(0, 2 ** 32, size=N * K // 8, dtype=np.uint32).tobytes()),
+                "scales": GpuBuffer.from_bytes(pack_f32((0.02 * np.abs(rng.standard_normal(N * K // G)) + 1e-3).astype(np.float32), dt)),
+                "biases": GpuBuffer.from_bytes(pack_f32((-0.1 + 0.01 * rng.standard_normal(N * K // G)).astype(np.float32), dt)),
+                "x": GpuBuffer.from_bytes(pack_f32(rng.standard_normal(M * K).astype(np.float32), dt)),
+                "out": GpuBuffer(M * N * 2)}
+        keep.append(bufs)
+        specs.append(("mt_qmm", dt, bufs, {"k": K, "n": N, "gs_per_row": K // G}))
+    nbytes = N * K // 2 + 2 * N * (K // G) * 2 + M * K * 2 + M * N * 2
+    runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
+    _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+    kern_avg = chain_us / (a.steps * len(specs))
+    for bufs in keep:
+        for b in bufs.values():
+            b.free()
+    gbs = nbytes * len(specs) * a.steps / wall_us / 1e3
+    ach = nbytes / kern_avg / 1e3
+    return {
+        "metric": f"qmm GB/s, {M} rows (4-bit g64 bf16, {N}x{K})", "value": round(gbs, 1), "unit": "GB/s",
+        "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
+        "config": {"workload": f"mt_qmm 4-bit g64 bf16, {M} rows x {N}x{K}", "launches_per_step": len(specs),
+                   "device": info["name"] or info["arch"]},
+        "roofline": {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": nbytes,
+                     "avg_launch_us_timed_region": round(kern_avg, 3)},
+    }
+
+
 def leg_gather(a, runner, info):
     import numpy as np
     import metaltile_amd as m
@@ -406,6 +449,11 @@ def main():
 
     if a.workload == "qmm":
         out.update(leg_qmm(a, runner, info, a.m))
+        print(json.dumps(out))
+        return
+
+    if a.workload == "batch":
+        out.update(leg_batch(a, runner, info))
         print(json.dumps(out))
         return
 

@@ -238,8 +238,15 @@ static int try_wide(int dtype, int bits, uint32_t G, const void* w, const void* 
     q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
     q.M = M; q.N = N; q.K = K;
     if (!qmv_wide_takes(q)) return ERR_UNSUPPORTED;
-    (void)exact;
-    if (options().qmv_wide != 2) return ERR_UNSUPPORTED;
+    // Every workgroup stages its 16 rows of activations (128 KB at K = 4096), which pays once a compute unit streams
+    // several times that in weights. us, 5 / 8 / 12 / 16 rows, the other kernels (GEMV passes of up to 8 rows | tiles)
+    // against this one: 128256 x 4096 67 69 118 133 | 90 91 92 93 -> 63 62 63 66; 57344 x 4096 32 33 60 66 | 43 44 44
+    // 46 -> 31 32 33 34; 28672 x 8192 53 54 81 109 | 46 46 46 47 -> 33 34 35 36; 32768 x 4096 21 22 37 41 | 26 27 27 27
+    // -> 20 20 21 22; 14336 x 4096 13 14 24 27 | 13 13 13 14 -> 13 14 15 15; 4096 x 4096 7.5 8.1 10.6 12.8 | 9.3 9.5 9.9
+    // 10.0 -> 10.4 11.2 12.0 12.8.
+    const uint64_t codes = (uint64_t)N * K;
+    const bool pays = exact && M >= 9 ? codes >= (1ull << 25) : codes >= 100000000ull;
+    if (options().qmv_wide != 2 && !pays) return ERR_UNSUPPORTED;
     const size_t need = qmv_wide_scratch_bytes(q);
     if (need) {
         int rc = ensure_scratch(g.scratch_held + need);

@@ -96,16 +96,14 @@ template <int DT> __device__ __forceinline__ float qw_elem(uint32_t dw, int odd)
     else return f16_bits_to_f32(odd ? (dw >> 16) : (dw & 0xFFFFu));
 }
 
-template <int DT, int G, int NB> __global__ __launch_bounds__(1024) void qmv_wide_kernel(QmvWArgs a) {
+template <int DT, int G, int NB, int SETS> __global__ __launch_bounds__(1024) void qmv_wide_kernel(QmvWArgs a) {
     static_assert(G == 32 || G == 64 || G == 128, "group size");
     static_assert(NB == 1 || NB == 2, "row blocks per wave");
+    static_assert(SETS >= 1 && SETS <= 3, "a wave works on at most 4 * SETS turns");
     constexpr int NW = 16;
     constexpr int GPT = 512 / G;       // groups per turn
-    constexpr int SBW = GPT / 2;       // dwords of packed scales (and of biases) per turn and weight row
+    constexpr int DPT = GPT / 2;       // dwords of packed scales (and of biases) per turn and weight row
     constexpr int UPG = G / 32;        // MFMAs per group
-    constexpr int SBE = SBW == 2 ? 2 : 4;   // dwords per scale load (8 or 16 bytes), loads per row and turn
-    constexpr int SV = SBW / SBE;
-    typedef typename std::conditional<SBW == 2, qw_u32x2, qw_u32x4>::type SBV;
     constexpr int MAXG = G == 32 ? 9 : G == 64 ? 5 : 3;   // groups a wave stages at most: a slice is at most 4608 codes
     constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
     extern __shared__ __align__(16) unsigned char lds[];
@@ -120,50 +118,56 @@ template <int DT, int G, int NB> __global__ __launch_bounds__(1024) void qmv_wid
 
     // KP waves share a set of NB row blocks, each taking a run of the slice's turns
     const uint32_t kp = wave & (a.kp - 1u), wr = wave >> a.log2kp;
-    const uint32_t t0 = min(kp * a.tpk, turns), t1 = min(t0 + a.tpk, turns);
+    const uint32_t t0 = min(kp * a.tpk, turns), t1 = min(t0 + a.tpk, turns), cnt = t1 - t0;   // cnt <= 4 * SETS (host)
     const uint32_t rb0 = (blockIdx.x * (NW >> a.log2kp) + wr) * NB;
-    // The waves start at different turns of their run and wrap around: were they all at the same turn, a workgroup's
-    // loads of a moment would all have the same address bits 8..10 (rows are a power of two apart), i.e. fall on few
-    // of the memory's channels.
-    const uint32_t cnt = t1 - t0, tfirst = t0 + (cnt ? (wr + blockIdx.x) % cnt : 0u);
-    uint32_t row[NB], woff[NB], soff[NB];   // byte offsets of this lane's weights and scales in turn 0 of the slice
+    uint32_t row[NB], woff[NB];   // woff: byte offset of this lane's weights in turn 0 of the slice
 #pragma unroll
     for (int i = 0; i < NB; i++) {   // row blocks past the matrix work on its last row and store nothing
         row[i] = (rb0 + i) * 16u + j;
-        const uint32_t rc = min(row[i], a.N - 1u);
-        woff[i] = rc * (a.K / 2u) + q * 16u;
-        soff[i] = rc * a.gpr * 2u;
+        woff[i] = min(row[i], a.N - 1u) * (a.K / 2u) + q * 16u;
     }
-    const unsigned char* wbase = a.w + k0 / 2u;                                    // + 256 bytes per turn
-    const unsigned char* sbase = (const unsigned char*)(a.scales + k0 / (uint32_t)G);   // + 2 GPT bytes per turn
-    const unsigned char* bbase = (const unsigned char*)(a.biases + k0 / (uint32_t)G);
+    const unsigned char* wbase = a.w + k0 / 2u;   // + 256 bytes per turn
 
-    // ---- the first turn's scales, biases and weights: in flight while the activations are staged -----------------
-    // Every load of the stream is issued by hand, in a fixed order (a turn's scales and biases, then its weights
-    // step by step), and waited for with "at most N loads outstanding": the compiler would sink the loads to the
-    // end of a turn and wait for all of them at its top.
-    qw_u32x4 ring[NB][4];
-    SBV sbs[2][NB][SV], sbb[2][NB][SV];   // scales and biases of the even and of the odd turns (counted from t0)
+    // ---- scales and biases of the wave's whole run, read once ------------------------------------------------------
+    // A row's scales are 16 bytes per turn of one 128-byte line; read turn by turn, the line had left the L2 by the
+    // next turn and was fetched from memory again (4.8 x the bytes). The four lanes of a weight row take the turns
+    // q, q + 4, q + 8 of the run (one 128-byte line per instruction and row); at turn n the lanes fetch the pairs from
+    // lane quarter n % 4, register set n / 4, with ds_bpermute.
+    uint32_t sreg[NB][SETS][DPT], breg[NB][SETS][DPT];
 #pragma unroll
     for (int i = 0; i < NB; i++) {
+        const size_t e0 = (size_t)min(row[i], a.N - 1u) * a.gpr + k0 / (uint32_t)G;
+#pragma unroll
+        for (int st = 0; st < SETS; st++) {
+            const uint32_t n = min(4u * st + q, cnt ? cnt - 1u : 0u);   // a turn past the run: any valid address, never used
+            const size_t e = e0 + (size_t)min(t0 + n, turns - 1u) * GPT;
+            if constexpr (DPT == 2) {
+                const qw_u32x2 sv = *(const qw_u32x2*)(a.scales + e), bv = *(const qw_u32x2*)(a.biases + e);
+                sreg[i][st][0] = sv.x; sreg[i][st][1] = sv.y; breg[i][st][0] = bv.x; breg[i][st][1] = bv.y;
+            } else {
+#pragma unroll
+                for (int h = 0; h < DPT / 4; h++) {
+                    const qw_u32x4 sv = *(const qw_u32x4*)(a.scales + e + 8 * h), bv = *(const qw_u32x4*)(a.biases + e + 8 * h);
+                    sreg[i][st][4 * h] = sv.x; sreg[i][st][4 * h + 1] = sv.y; sreg[i][st][4 * h + 2] = sv.z; sreg[i][st][4 * h + 3] = sv.w;
+                    breg[i][st][4 * h] = bv.x; breg[i][st][4 * h + 1] = bv.y; breg[i][st][4 * h + 2] = bv.z; breg[i][st][4 * h + 3] = bv.w;
+                }
+            }
+        }
+    }
+
+    // ---- the first turn's weights: in flight while the activations are staged --------------------------------------
+    // The weight loads of the stream are issued by hand, in a fixed order, and waited for with "at most N loads
+    // outstanding": the compiler would sink the loads to the end of a turn and wait for all of them at its top.
+    // The loop below is the only code that touches registers with loads in flight, and every turn issues its loads
+    // (those of a wave's last turn, for a turn that does not exist, all read the slice's first bytes): a register
+    // allocator that had to join several copies of the turn would move such registers about while their loads fly.
+    qw_u32x4 ring[NB][4];
+#pragma unroll
+    for (int i = 0; i < NB; i++)
 #pragma unroll
         for (int d = 0; d < 4; d++) ring[i][d] = qw_u32x4{0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int h = 0; h < SV; h++) { sbs[0][i][h] = SBV{}; sbb[0][i][h] = SBV{}; sbs[1][i][h] = SBV{}; sbb[1][i][h] = SBV{}; }
-    }
-    auto issue_sb = [&](auto par_c, uint32_t t, bool real) {
-        constexpr int P = decltype(par_c)::value;
-#pragma unroll
-        for (int i = 0; i < NB; i++)
-#pragma unroll
-            for (int h = 0; h < SV; h++) {
-                qw_load<0>(sbs[P][i][h], real ? soff[i] + h * 16u : 0u, sbase + t * (uint32_t)(GPT * 2));
-                qw_load<0>(sbb[P][i][h], real ? soff[i] + h * 16u : 0u, bbase + t * (uint32_t)(GPT * 2));
-            }
-    };
     {
-        const uint32_t tc = min(tfirst, turns - 1u);   // a wave without turns loads a valid address and uses nothing
-        issue_sb(std::integral_constant<int, 0>{}, tc, true);
+        const uint32_t tc = min(t0, turns - 1u);   // a wave without turns loads a valid address and uses nothing
         qw_static_for<0, 4>([&](auto d_c) {
             constexpr int d = decltype(d_c)::value;
 #pragma unroll
@@ -207,6 +211,14 @@ template <int DT, int G, int NB> __global__ __launch_bounds__(1024) void qmv_wid
         }
     }
     __syncthreads();
+    // (the compiler's own wait for the scales and biases belongs here, not inside the loop, where it would wait for
+    // the loop's loads as well)
+#pragma unroll
+    for (int i = 0; i < NB; i++)
+#pragma unroll
+        for (int st = 0; st < SETS; st++)
+#pragma unroll
+            for (int k = 0; k < DPT; k++) { qw_tie(sreg[i][st][k]); qw_tie(breg[i][st][k]); }
 
     // ---- stream ---------------------------------------------------------------------------------------------------
     const uint32_t kor = magic_or_vgpr<DT>();
@@ -218,37 +230,24 @@ template <int DT, int G, int NB> __global__ __launch_bounds__(1024) void qmv_wid
     for (int i = 0; i < NB; i++)
 #pragma unroll
         for (int r = 0; r < 4; r++) tot[i][r] = 0.f;
-    // One turn: 512 codes of every row block of the wave; the next turn's loads go out as this one's registers are
-    // consumed. Loads outstanding at the top of a turn, oldest first: its scales and biases (LS), its weights (LW).
-    // Scales and biases live in two sets of registers used in turn: a set is read while the other is loaded, so
-    // the loop is written two turns at a time and is the only code that touches registers with loads in flight
-    // (a register allocator that has to join several copies of the turn would move such registers about). Hence
-    // every turn issues loads (a wave's last ones, for a turn that does not exist, all read the slice's first 16
-    // bytes) and an odd number of turns ends with a turn whose scales and biases are multiplied by zero.
-    constexpr int LS = NB * SV * 2, LW = NB * 4;
-    auto turn = [&](auto par_c, uint32_t t, uint32_t tn, bool has_next, bool live) {
-        constexpr int P = decltype(par_c)::value;
-        const float livef = live ? 1.0f : 0.0f;
+    // One turn: 512 codes of every row block of the wave. The registers of two steps are reloaded for the next turn
+    // together, behind steps 1 and 3, so that both 64-byte halves of a 128-byte line are asked for at the same time
+    // (asked for a quarter turn apart, most lines were fetched from memory twice: the loads are marked as read
+    // once). Loads outstanding at the top of a turn: its weights, 4 NB; when step d's are needed, the younger ones
+    // are the rest of the turn's and the next turn's issued so far: 3 NB at steps 0 and 2, 2 NB at steps 1 and 3.
+    for (uint32_t n = 0; n < cnt; n++) {
+        const uint32_t t = t0 + n;
+        const bool has_next = n + 1u < cnt;
+        const uint32_t tn = has_next ? t + 1u : t;
         const unsigned char* xl_t = xl_lane + t * 16384u;
         const unsigned char* xg_t = xg_lane + t * (uint32_t)(GPT * 64);
+        const int src_lane4 = (int)((j + 16u * (n & 3u)) * 4u);   // the lane that holds this turn's scales and biases of row j
+        uint32_t m4 = (n & 4u) ? ~0u : 0u, m8 = (n & 8u) ? ~0u : 0u;   // register set n / 4: all-ones masks for sets 1 and 2
+        asm volatile("" : "+s"(m4), "+s"(m8));
         qw_f32x4 acc[NB];
         qw_static_for<0, 4>([&](auto d_c) {
             constexpr int d = decltype(d_c)::value;
-            // step d's weights: younger than they are the rest of the turn's weights, the next turn's scales and
-            // biases and its weights issued so far
-            if constexpr (d == 0) {
-                qw_wait<LW - NB>();
-#pragma unroll
-                for (int i = 0; i < NB; i++)
-#pragma unroll
-                    for (int h = 0; h < SV; h++) { qw_tie(sbs[P][i][h]); qw_tie(sbb[P][i][h]); }
-                issue_sb(std::integral_constant<int, P ^ 1>{}, tn, has_next);
-            } else {
-                // the next turn's weights go out two steps at a time (behind steps 1 and 3), so that both 64-byte
-                // halves of a 128-byte line are asked for together: asked for a quarter turn apart, most lines
-                // were fetched from memory twice
-                qw_wait<(d == 2 ? 3 * NB : 2 * NB) + LS>();
-            }
+            qw_wait<(d % 2 ? 2 : 3) * NB>();
             uint32_t v[NB][4];
 #pragma unroll
             for (int i = 0; i < NB; i++) {
@@ -262,7 +261,7 @@ template <int DT, int G, int NB> __global__ __launch_bounds__(1024) void qmv_wid
                 const auto b23 = __builtin_amdgcn_permlane16_swap(a02[1], a13[1], false, false);
                 v[i][0] = b01[0]; v[i][1] = b01[1]; v[i][2] = b23[0]; v[i][3] = b23[1];
             }
-            if constexpr (d == 1 || d == 3) {
+            if constexpr (d % 2 == 1) {
 #pragma unroll
                 for (int i = 0; i < NB; i++) qw_load_once<(d - 1) * 64>(ring[i][d - 1], has_next ? woff[i] : 0u, wbase + tn * 256u);
 #pragma unroll
@@ -283,8 +282,21 @@ template <int DT, int G, int NB> __global__ __launch_bounds__(1024) void qmv_wid
                     const qw_f32x4 xg = *(const qw_f32x4*)(xg_t + gi * 64);
 #pragma unroll
                     for (int i = 0; i < NB; i++) {
-                        const float sv = qw_elem<DT>(sbs[P][i][(gi / 2) / SBE][(gi / 2) % SBE], gi % 2) * livef;
-                        const float bv = qw_elem<DT>(sbb[P][i][(gi / 2) / SBE][(gi / 2) % SBE], gi % 2) * livef;
+                        // (bitwise selection under masks the optimiser cannot see through: a conditional selection
+                        // between array elements becomes an indexed read, and the arrays then live in scratch memory)
+                        uint32_t sp = sreg[i][0][gi / 2], bp = breg[i][0][gi / 2];
+                        if constexpr (SETS > 1) {
+                            sp = (sp & ~m4) | (sreg[i][1][gi / 2] & m4);
+                            bp = (bp & ~m4) | (breg[i][1][gi / 2] & m4);
+                        }
+                        if constexpr (SETS > 2) {
+                            sp = (sp & ~m8) | (sreg[i][2][gi / 2] & m8);
+                            bp = (bp & ~m8) | (breg[i][2][gi / 2] & m8);
+                        }
+                        // (an odd group's pair was fetched for the even group before it; the compiler keeps it)
+                        const uint32_t spl = (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane4, (int)sp);
+                        const uint32_t bpl = (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane4, (int)bp);
+                        const float sv = qw_elem<DT>(spl, gi % 2), bv = qw_elem<DT>(bpl, gi % 2);
                         const float bm = fmaf(-MAGIC, sv, bv);
 #pragma unroll
                         for (int r = 0; r < 4; r++) tot[i][r] = fmaf(bm, xg[r], fmaf(sv, acc[i][r], tot[i][r]));
@@ -292,15 +304,6 @@ template <int DT, int G, int NB> __global__ __launch_bounds__(1024) void qmv_wid
                 }
             }
         });
-    };
-    {
-        uint32_t cur = tfirst;
-        for (uint32_t n = 0; n < cnt; n += 2u) {
-            const uint32_t n1 = cur + 1u == t1 ? t0 : cur + 1u, n2 = n1 + 1u == t1 ? t0 : n1 + 1u;
-            turn(std::integral_constant<int, 0>{}, cur, n1, n + 1u < cnt, true);
-            turn(std::integral_constant<int, 1>{}, n1, n2, n + 2u < cnt, n + 1u < cnt);   // (past an odd count: a turn that adds nothing)
-            cur = n2;
-        }
     }
     qw_wait<0>();   // the last turn's loads, or those of a wave without turns
 
@@ -343,7 +346,7 @@ template <int DT> __global__ __launch_bounds__(256) void qmv_wide_reduce_kernel(
 }
 
 struct QmvWPlan {
-    uint32_t kslice, ksplit, nb, kp, log2kp, tpk, grid_x;
+    uint32_t kslice, ksplit, nb, kp, log2kp, tpk, sets, grid_x;
     size_t lds;
 };
 
@@ -361,8 +364,7 @@ static bool plan_wide(const QmmParams& p, QmvWPlan& pl) {
     const uint32_t max_turns = (160u * 1024u) / per_turn;
     const uint32_t turns = p.K / 512u;
     uint32_t ks = (turns + max_turns - 1) / max_turns;
-    uint32_t tps = (turns + ks - 1) / ks;
-    if ((tps & 1u) && tps > 1u && tps < max_turns) tps++;   // the loop works two turns at a time
+    const uint32_t tps = (turns + ks - 1) / ks;
     ks = (turns + tps - 1) / tps;
     pl.kslice = tps * 512u;
     pl.ksplit = ks;
@@ -374,7 +376,7 @@ static bool plan_wide(const QmmParams& p, QmvWPlan& pl) {
     pl.nb = (nrb + 15u) / 16u > want + want / 4u && G != 32 ? 2u : 1u;   // (two row blocks of 32-code groups do not fit the registers)
     pl.kp = 1;
     pl.log2kp = 0;
-    while (pl.nb == 1u && pl.kp < 16u && pl.kp * 2u <= tps && (nrb * pl.kp + 15u) / 16u < want) {
+    while (pl.nb == 1u && pl.kp < 16u && pl.kp * 2u <= tps && (nrb * pl.kp * 2u + 15u) / 16u <= want) {
         pl.kp *= 2u;
         pl.log2kp++;
     }
@@ -385,8 +387,17 @@ static bool plan_wide(const QmmParams& p, QmvWPlan& pl) {
         while ((1u << pl.log2kp) < pl.kp) pl.log2kp++;
     }
     if (options().qmv_wide_nb) pl.nb = G == 32 ? 1u : (uint32_t)options().qmv_wide_nb;
+    // A wave keeps the scales and biases of its whole run of turns in registers, a set per 4 turns: at most 3 sets
+    // (2 with two row blocks per wave, 1 for groups of 32 codes, whose turns hold twice the groups).
+    const uint32_t max_sets = G == 32 ? 1u : 3u;
+    while (pl.kp < 16u && (tps + pl.kp - 1) / pl.kp > 4u * max_sets) {
+        pl.kp *= 2u;
+        pl.log2kp++;
+    }
     pl.tpk = (tps + pl.kp - 1) / pl.kp;
-    if ((pl.tpk & 1u) && pl.tpk > 1u) pl.tpk++;
+    pl.sets = (pl.tpk + 3u) / 4u;
+    if (pl.sets > max_sets) return false;
+    if (pl.nb == 2u && pl.sets > 2u) pl.nb = 1;
     if (pl.kp > 1u && pl.lds < (size_t)16 * pl.nb * 1024) pl.lds = (size_t)16 * pl.nb * 1024;   // the K parts' sums, a KB per wave and row block
     const uint32_t per_wg = 16u * pl.nb / pl.kp;
     pl.grid_x = (nrb + per_wg - 1) / per_wg;
@@ -424,11 +435,14 @@ int launch_qmv_wide(const QmmParams& p, const LaunchCtx& lc, void* scratch) {
     a.log2kp = pl.log2kp;
     a.tpk = pl.tpk;
     const void* fn = nullptr;
-#define QW_PICK2(DTv, NBv) (p.group_size == 32 ? (const void*)qmv_wide_kernel<DTv, 32, 1> : p.group_size == 64 ? (const void*)qmv_wide_kernel<DTv, 64, NBv> : (const void*)qmv_wide_kernel<DTv, 128, NBv>)
+#define QW_PICK3(DTv, Gv, NBv) (pl.sets == 1 ? (const void*)qmv_wide_kernel<DTv, Gv, NBv, 1> : pl.sets == 2 ? (const void*)qmv_wide_kernel<DTv, Gv, NBv, 2> : NBv == 1 ? (const void*)qmv_wide_kernel<DTv, Gv, 1, 3> : nullptr)
+#define QW_PICK2(DTv, NBv) (p.group_size == 32 ? (const void*)qmv_wide_kernel<DTv, 32, 1, 1> : p.group_size == 64 ? QW_PICK3(DTv, 64, NBv) : QW_PICK3(DTv, 128, NBv))
 #define QW_PICK(DTv) (pl.nb == 2 ? QW_PICK2(DTv, 2) : QW_PICK2(DTv, 1))
     fn = p.dtype == DT_BF16 ? QW_PICK(DT_BF16) : QW_PICK(DT_F16);
 #undef QW_PICK
 #undef QW_PICK2
+#undef QW_PICK3
+    if (!fn) return fail(ERR_UNSUPPORTED, "wide qmv: geometry not built");
     hipError_t e = set_max_dynamic_lds(fn, pl.lds);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
     void* args[] = {&a};

@@ -61,8 +61,8 @@ def test_wide_gemv_is_the_kernel_that_ran(wide):
     rc, launches, scratch, n = ops.plan("qmm", DType.BF16, 4, 64, 16, 8192, 4096)
     assert rc == 0 and n == 1 and "qmv_wide_kernel<2, 64, " in launches[0][0] and launches[0][2][0] == 1024
     rc, launches, scratch, n = ops.plan("qmm", DType.F16, 4, 32, 9, 8192, 8192)
-    assert rc == 0 and n == 2 and "qmv_wide_kernel<1, 32, 1>" in launches[0][0] and "qmv_wide_reduce_kernel" in launches[1][0]
-    assert launches[0][1][1] == 2 and scratch >= 2 * 9 * 8192 * 4
+    assert rc == 0 and n == 2 and "qmv_wide_kernel<1, 32, 1, 1>" in launches[0][0] and "qmv_wide_reduce_kernel" in launches[1][0]
+    assert launches[0][1][1] == 2 and scratch >= 2 * 9 * 8192 * 4   # groups of 32: a wave keeps at most 4 turns of scales in registers
     for args in ((DType.BF16, 8, 64, 16, 8192, 4096), (DType.BF16, 4, 64, 16, 8192, 4352), (DType.BF16, 4, 64, 17, 8192, 4096)):
         rc, launches, _, n = ops.plan("qmm", *args)
         assert rc == 0 and all("qmv_wide" not in l[0] for l in launches)
