@@ -16,6 +16,12 @@ pytestmark = pytest.mark.gpu
 ODT = {DType.F16: 1, DType.BF16: 2}
 
 
+def cold():
+    """Empties the caches: the kernels whose loads are issued and waited for by hand must not depend on data
+    arriving early (a wait that is one load short passes on warm caches)."""
+    assert _lib.load().mtq_flush_cache() == 0
+
+
 @pytest.fixture
 def options():
     lib = _lib.load()
@@ -271,6 +277,7 @@ def test_load_to_lds_tiles(oracle, options, dt, M, N, K, G, bits):
         options("qmm.tile_rows", rows)
         options("qmm.dma", 3)
         out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
+        cold()
         ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
         got_bytes = out.read_bytes()
         got = unpack_f32(got_bytes, dt)
@@ -279,6 +286,7 @@ def test_load_to_lds_tiles(oracle, options, dt, M, N, K, G, bits):
         if rows != 256:
             options("qmm.dma", 1)
             out = GpuBuffer(M * N * dt.size_bytes)
+            cold()
             ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
             assert out.read_bytes() == got_bytes, f"rows={rows}: differs from the register-staged instance"
             out.free()
@@ -326,6 +334,7 @@ def test_load_to_lds_tiles_with_windowed_scales(oracle, options, dt, M, N, K, G,
         options("qmm.tile_rows", rows)
         options("qmm.dma", 2)
         out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
+        cold()
         ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
         got_bytes = out.read_bytes()
         out.free()
@@ -333,6 +342,7 @@ def test_load_to_lds_tiles_with_windowed_scales(oracle, options, dt, M, N, K, G,
         if rows != 256:
             options("qmm.dma", 1)
             out = GpuBuffer(M * N * dt.size_bytes)
+            cold()
             ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
             assert out.read_bytes() == got_bytes, f"rows={rows}: differs from the register-staged instance"
             out.free()
@@ -365,6 +375,7 @@ def test_load_to_lds_tiles_on_4_kgroups(oracle, options, dt, M, N, K, G, bits):
             for dma in (3, 1):
                 options("qmm.dma", dma)
                 out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
+                cold()
                 ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
                 res[dma] = out.read_bytes()
                 out.free()
@@ -400,6 +411,7 @@ def test_load_to_lds_tiles_with_k_split(oracle, options, dt, M, N, K, G, bits):
             print(f"[case] K-split load-to-LDS qmm {dt.name} b{bits} M={M} N={N} K={K} g{G} tile_rows={rows} ksplit={ksplit}", flush=True)
             options("qmm.ksplit", ksplit)
             out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
+            cold()
             ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
             got[ksplit] = unpack_f32(out.read_bytes(), dt)
             out.free()

@@ -48,6 +48,7 @@ def test_wide_gemv(oracle, wide, dt, M, N, K, G, kp, nb):
     w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
                   GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
     out = GpuBuffer.from_bytes(b"\xff" * (M * N * dt.size_bytes))
+    assert _lib.load().mtq_flush_cache() == 0   # cold operands: hand-counted waits must not rely on data arriving early
     ops.qmm(dt, bits, G, w, s, b, x, out, M, N, K)
     got = unpack_f32(out.read_bytes(), dt)
     assert rel_err(got, exp) <= 1e-2
