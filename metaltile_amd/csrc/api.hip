@@ -367,6 +367,19 @@ static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const
     QmvParams p;
     p.dtype = dtype; p.bits = bits; p.group_size = G; p.w = w; p.scales = s; p.biases = b; p.x = x; p.out = out;
     p.N = N; p.K = K;
+    // 4-bit f16 / bf16: the norm applied as the matrix-core GEMV stages its row (two staged rows share one set of 4;
+    // no per-workgroup renormalisation beyond the sum of squares). us, streaming kernel -> this: 14336 x 4096 12.6 ->
+    // 10.6, 6144 x 4096 8.1 -> 7.3; it loses on short matrices and long rows (4096 x 4096 6.2 -> 6.4, 4096 x 14336 13.7 -> 14.1).
+    const bool norm_on_mfma = options().qmv_norm_mfma == 2 ||
+                              (options().qmv_norm_mfma == 0 && K <= 8192 && (uint64_t)N * K >= 24000000ull);
+    if (bits == 4 && dtype != DT_F32 && norm_on_mfma) {
+        QmvParams pm = p;
+        pm.M = 1;
+        pm.norm_w = norm_w;
+        pm.norm_eps = eps;
+        rc = launch_qmv_mfma(pm, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
     rc = launch_qmv_norm(p, norm_w, eps, lc);
     if (rc != ERR_UNSUPPORTED) return rc;
     // scratch: the normalised row(s), then for 16-bit types the two partial outputs
@@ -1420,6 +1433,11 @@ int mtq_set_option(const char* name, int value) {
     if (!strcmp(name, "qmv.mfma")) {
         if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmv.mfma must be 0 (auto), 1 (off) or 2 (prefer)");
         options().qmv_mfma = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmv.norm_mfma")) {
+        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmv.norm_mfma must be 0 (choose), 1 (never) or 2 (wherever the shape allows)");
+        options().qmv_norm_mfma = value;
         return MTQ_OK;
     }
     if (!strcmp(name, "qmv.wide_kp")) {

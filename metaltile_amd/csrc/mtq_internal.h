@@ -57,6 +57,7 @@ enum GatherMode : int {
     GATHER_CSR = 1,      // rows sorted by expert, expert_offsets[E+1]
     GATHER_INDICES = 2,  // indices[T] gives the expert of each row
     GATHER_SINGLE = 3,   // one row against slab expert_index[0]
+    GATHER_NORM = 4,     // matrix-core GEMV only: one row, RMS-normalised as it is staged (QmvParams::norm_w, norm_eps)
 };
 
 struct QmvParams {
@@ -73,6 +74,8 @@ struct QmvParams {
     const uint32_t* route = nullptr;  // expert_offsets / indices / expert_index
     uint32_t T = 0;                   // rows (gather modes)
     uint32_t E = 1;                   // experts
+    const void* norm_w = nullptr;     // matrix-core GEMV: weights of an RMS norm applied to the one row of x first
+    const float* norm_eps = nullptr;  // its epsilon (device memory)
 };
 
 // Several weight matrices with the same K, code width and group size against one
@@ -110,6 +113,7 @@ struct Options {
     int qmv_mfma_rbw = 0;         // matrix-core qmv: row blocks walked in parallel per workgroup
     int qmv_mfma_nrb = 0;         // matrix-core qmv: row blocks per wave
     int qmv_mfma_sets = 0;        // matrix-core gather: 4-row MFMA sets per pass (0 = choose; 1, 2, 4)
+    int qmv_norm_mfma = 0;        // RMS norm fused into the matrix-core GEMV (4-bit f16 / bf16): 0 = choose, 1 = never, 2 = wherever the shape allows
     int qmv_wide_kp = 0;          // 16-row matrix-core GEMV: waves sharing a row block (0 = choose; 1, 2, 4, 8, 16)
     int qmv_wide_nb = 0;          // 16-row matrix-core GEMV: row blocks per wave (0 = choose; 1, 2)
     int qmv_wide = 0;             // 16-row matrix-core GEMV for batches of 5..16 rows: 0 = choose per shape, 1 = never, 2 = wherever the shape allows

@@ -72,7 +72,10 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
         (rb64 % 16 && !odd) || (p.K * 2) % 16)
         return fail(ERR_UNSUPPORTED, "mfma qmv: operands must be 16-byte aligned");
     const bool gather = p.gather == GATHER_CSR || p.gather == GATHER_INDICES;
-    const uint32_t rows = gather ? p.T : (p.gather == GATHER_SINGLE ? 1u : p.M);
+    const bool norm = p.norm_w != nullptr;   // one row, staged as two (rounded value and remainder)
+    if (norm && (p.gather != GATHER_NONE || p.M != 1 || p.bits != 4 || !p.norm_eps || (uintptr_t)p.norm_w % 16))
+        return fail(ERR_UNSUPPORTED, "mfma qmv: the fused norm takes one row of 4-bit codes");
+    const uint32_t rows = gather ? p.T : (p.gather == GATHER_SINGLE ? 1u : (norm ? 2u : p.M));
     if (rows == 0) return ERR_OK;
     const Options& opt = options();
 
@@ -235,6 +238,9 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     a.gpw = gpw;
     a.log2g = ilog2(G);
     a.list_cap = list_cap;
+    a.norm_w = p.norm_w;
+    a.norm_eps = p.norm_eps;
+    const int mode = norm ? (int)GATHER_NORM : p.gather;
     QmvMGeom g;
     g.mp = mp;
     g.s = s;
@@ -243,11 +249,11 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     g.shmem = lds_bytes(R, nchp * cpc, nch, gpr, rows_wg, KP * RBW, gpw, KP, list_cap);
     g.grid = dim3((p.N + rows_wg - 1) / rows_wg, gather ? p.E : 1, 1);
     if (odd)
-        return p.dtype == DT_F16 ? qmv_mfma_launch_dtype_odd<DT_F16>(a, half2 ? 22 : p.bits, p.gather, g, lc)
-                                 : qmv_mfma_launch_dtype_odd<DT_BF16>(a, half2 ? 22 : p.bits, p.gather, g, lc);
+        return p.dtype == DT_F16 ? qmv_mfma_launch_dtype_odd<DT_F16>(a, half2 ? 22 : p.bits, mode, g, lc)
+                                 : qmv_mfma_launch_dtype_odd<DT_BF16>(a, half2 ? 22 : p.bits, mode, g, lc);
     switch (p.dtype) {
-        case DT_F16: return qmv_mfma_launch_dtype<DT_F16>(a, p.bits, p.gather, g, lc);
-        default: return qmv_mfma_launch_dtype<DT_BF16>(a, p.bits, p.gather, g, lc);
+        case DT_F16: return qmv_mfma_launch_dtype<DT_F16>(a, p.bits, mode, g, lc);
+        default: return qmv_mfma_launch_dtype<DT_BF16>(a, p.bits, mode, g, lc);
     }
 }
 

@@ -75,6 +75,8 @@ struct QmvMArgs {
     uint32_t gpr, log2g;
     uint32_t gpw;       // (scale, bias) pairs per row that a wave keeps in LDS: the groups of its K part, whole 4-vectors, <= 64
     uint32_t list_cap;  // capacity of the row list (indices mode)
+    const void* norm_w;     // GATHER_NORM: the norm's weights [K] and its epsilon
+    const float* norm_eps;
 };
 
 struct QmvMGeom {
@@ -206,6 +208,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     float* RED = (float*)(SB + (size_t)sb_zero + 1);                 // [KP][rows_wg][R]
     uint32_t* rowlist = (uint32_t*)(RED + (size_t)a.KP * rows_wg * R);
     __shared__ uint32_t s_meta[4];
+    __shared__ float s_sq[16];
 
     const uint32_t tid = threadIdx.x, TPB = blockDim.x;
     const uint32_t lane = tid & 63u, wave = tid >> 6;
@@ -240,8 +243,36 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         expert = min(a.route[0], a.E - 1);  // an out-of-range id must not fault the GPU
         cnt = 1;
     }
+    // GATHER_NORM: x' = (x * norm_w) * rsqrt(mean(x^2) + eps) in f32 (crates/metaltile-std/src/ffai/rms_norm_qgemv.rs:64-77,
+    // 104-106) is staged as two rows, its value rounded to the element type and the rounded remainder (16 significant
+    // bits in all), whose dot products are added at the end: rounding x' alone costs 3.5e-2 on the parity metric.
+    float inv_rms = 1.0f;
+    if constexpr (MODE == GATHER_NORM) {
+        cnt = 2;
+        float ss = 0.f;
+        for (uint32_t c = tid; c < a.nch; c += TPB) {
+            const m_u32x4* src = (const m_u32x4*)((const uint16_t*)a.x + (size_t)c * CPC);
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const m_u32x4 v = src[p];
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const float lo_ = DT == DT_BF16 ? bf16_bits_to_f32(v[k] & 0xFFFFu) : f16_bits_to_f32(v[k] & 0xFFFFu);
+                    const float hi_ = DT == DT_BF16 ? bf16_bits_to_f32(v[k] >> 16) : f16_bits_to_f32(v[k] >> 16);
+                    ss = fmaf(lo_, lo_, fmaf(hi_, hi_, ss));
+                }
+            }
+        }
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        if (lane == 0) s_sq[wave] = ss;
+        __syncthreads();
+        ss = 0.f;
+        for (uint32_t wv = 0; wv < TPB / 64u; wv++) ss += s_sq[wv];
+        inv_rms = rsqrtf(ss / (float)a.K + a.norm_eps[0]);
+    }
     auto batch_row = [&](uint32_t j) -> uint32_t {
         if (j >= cnt) return NOROW;
+        if constexpr (MODE == GATHER_NORM) return 0u;
         if constexpr (MODE == GATHER_CSR) return j < n1 ? lo + j : lo2 + (j - n1);
         else if constexpr (MODE == GATHER_INDICES) return rowlist[j];
         else return j;
@@ -335,6 +366,7 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         // cores compute from their LDS slots lands in output rows nobody stores.
         const uint32_t ntask = live * a.nchp;  // chunks past the row's end are staged as zeros
         uint32_t raw[NP * 4];
+        uint32_t nraw[MODE == GATHER_NORM ? NP * 4 : 1];   // the norm's weights for the chunk
         bool row_live;
         auto x_load = [&](uint32_t task) {
             const uint32_t i = task / a.nchp, c = task - i * a.nchp;
@@ -347,6 +379,14 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                 const m_u32x4 v = src[p];
                 raw[4 * p] = v.x; raw[4 * p + 1] = v.y; raw[4 * p + 2] = v.z; raw[4 * p + 3] = v.w;
             }
+            if constexpr (MODE == GATHER_NORM) {
+                const m_u32x4* nsrc = (const m_u32x4*)((const uint16_t*)a.norm_w + (size_t)min(c, a.nch - 1) * CPC);
+#pragma unroll
+                for (int p = 0; p < NP; p++) {
+                    const m_u32x4 v = nsrc[p];
+                    nraw[4 * p] = v.x; nraw[4 * p + 1] = v.y; nraw[4 * p + 2] = v.z; nraw[4 * p + 3] = v.w;
+                }
+            }
         };
         const uint32_t cpg = (1u << a.log2g) / (uint32_t)CPC;  // chunks per group: a power of two, at most 16
         auto x_store = [&](uint32_t task) {
@@ -354,6 +394,23 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
             if (!row_live) {
 #pragma unroll
                 for (int j = 0; j < NP * 4; j++) raw[j] = 0u;
+            }
+            if constexpr (MODE == GATHER_NORM) {   // row 0: x' rounded; row 1: what the rounding left
+#pragma unroll
+                for (int j = 0; j < NP * 4; j++) {
+                    uint32_t o2[2];
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const uint32_t xb = h ? raw[j] >> 16 : raw[j] & 0xFFFFu, wb = h ? nraw[j] >> 16 : nraw[j] & 0xFFFFu;
+                        const float xf = DT == DT_BF16 ? bf16_bits_to_f32(xb) : f16_bits_to_f32(xb);
+                        const float wf = DT == DT_BF16 ? bf16_bits_to_f32(wb) : f16_bits_to_f32(wb);
+                        const float xn = (xf * wf) * inv_rms;
+                        const uint32_t hb = f32_to_elem_bits<DT>(xn);
+                        const float hf = DT == DT_BF16 ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb);
+                        o2[h] = i == 0 ? hb : (uint32_t)f32_to_elem_bits<DT>(xn - hf);
+                    }
+                    raw[j] = o2[0] | (o2[1] << 16);
+                }
             }
             float sum = 0.f;
 #pragma unroll
@@ -542,6 +599,16 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
         // ---- add the K parts and store ----------------------------------------
         uint32_t stid = tid;
         if constexpr (MODE == GATHER_CSR || MODE == GATHER_INDICES) asm volatile("" : "+v"(stid));
+        if constexpr (MODE == GATHER_NORM) {   // one output row: the sum of the two staged rows' dot products
+            for (uint32_t rl = stid; rl < rows_wg; rl += TPB) {
+                const uint32_t row = row0 + rl;
+                if (row >= a.N) continue;
+                float v = 0.f;
+                for (uint32_t k2 = 0; k2 < a.KP; k2++) v += RED[((size_t)k2 * rows_wg + rl) * R] + RED[((size_t)k2 * rows_wg + rl) * R + 1];
+                store_elem<DT>(a.out, row, v);
+            }
+            return;
+        }
         for (uint32_t idx = stid; idx < rows_wg * live; idx += TPB) {
             const uint32_t i = idx / rows_wg, rl = idx - i * rows_wg;
             const uint32_t row = row0 + rl;
@@ -602,6 +669,9 @@ int qmv_mfma_launch_mode(QmvMArgs& a, int mode, const QmvMGeom& g, const LaunchC
         case GATHER_NONE: return qmv_mfma_launch_rows<DT, BITS, GATHER_NONE>(a, g, lc);
         case GATHER_CSR: return qmv_mfma_launch_rows<DT, BITS, GATHER_CSR>(a, g, lc);
         case GATHER_INDICES: return qmv_mfma_launch_rows<DT, BITS, GATHER_INDICES>(a, g, lc);
+        case GATHER_NORM:
+            if constexpr (BITS == 4) return qmv_mfma_launch_one<DT, 4, 2, 1, GATHER_NORM>(a, g, lc);
+            else return fail(ERR_UNSUPPORTED, "mfma qmv: the fused norm is built for 4-bit codes");
         default: return qmv_mfma_launch_rows<DT, BITS, GATHER_SINGLE>(a, g, lc);
     }
 }

@@ -92,3 +92,36 @@ def test_fused_equals_norm_then_qmv_f32(oracle):
     assert rel_err(a, p) <= 1e-5
     for buf in (w, s, b, xb, nwb, epsb, o1, o2):
         buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.F16, DType.BF16], ids=lambda d: d.name)
+@pytest.mark.parametrize("N,K,G", [(4096, 4096, 64), (1000, 2048, 64), (333, 8192, 128), (14336, 4096, 64), (100, 14336, 64), (64, 1024, 32)])
+def test_norm_fused_into_the_matrix_core_gemv(oracle, dt, N, K, G):
+    """The same operation with the norm applied as the matrix-core GEMV stages its row (4-bit codes; forced with
+    qmv.norm_mfma = 2), against the oracle at the bound of the other fused kernel."""
+    from metaltile_amd import _lib
+    lib = _lib.load()
+    bits = 4
+    print(f"[case] rms_norm_qmv on the matrix-core GEMV {dt.name} g{G} N{N} K{K}", flush=True)
+    c = make_case(1400 + N, dt, bits, G, 1, N, K, bias_rule="midpoint")
+    rng = np.random.default_rng(N + K)
+    nw = oracle.round_through((1.0 + 0.2 * rng.standard_normal(K)).astype(np.float32), ODT[dt])
+    eps = np.float32(1e-5)
+    _, exp64, _ = oracle.rms_norm_qgemv(c.w, c.scales_f, c.biases_f, c.x_f, nw, K, G, N, bits, eps)
+    exp = oracle.round_through(exp64.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    nwb, epsb = GpuBuffer.from_bytes(pack_f32(nw, dt)), GpuBuffer.from_bytes(eps.tobytes())
+    out = GpuBuffer.from_bytes(b"\xff" * (N * dt.size_bytes))
+    assert lib.mtq_set_option(b"qmv.norm_mfma", 2) == 0
+    try:
+        rc, launches, _, n = ops.plan("rms_norm_qmv", dt, bits, G, 1, N, K)
+        assert rc == 0 and n == 1 and "qmv_mfma_kernel" in launches[0][0], launches
+        ops.rms_norm_qmv(dt, bits, G, x, nwb, w, s, b, out, epsb, N, K)
+    finally:
+        lib.mtq_set_option(b"qmv.norm_mfma", 0)
+    got = unpack_f32(out.read_bytes(N * dt.size_bytes), dt)
+    assert np.isfinite(got).all()
+    assert rel_err(got, exp) <= TOL[dt]
+    for buf in (w, s, b, x, nwb, epsb, out):
+        buf.free()
