@@ -25,7 +25,7 @@ HIPFLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
 ]
-SOURCES = ["api.hip", "qmv.hip", "qmv_f32.hip", "qmv_f16.hip", "qmv_bf16.hip", "qmv_mfma.hip", "qmv_mfma_f16.hip", "qmv_mfma_bf16.hip", "qmv_mfma_f16_odd.hip", "qmv_mfma_bf16_odd.hip", "qmv_wide.hip", "generic.hip", "qmm.hip", "qmm_direct.hip", "qmm_direct_odd.hip", "qmm_dma.hip", "qmm_dma_b8.hip", "qmm_f32.hip", "affine.hip", "norm.hip", "moe.hip", "moe_down.hip", "qvm.hip"]
+SOURCES = ["api.hip", "qmv.hip", "qmv_f32.hip", "qmv_f16.hip", "qmv_bf16.hip", "qmv_mfma.hip", "qmv_mfma_f16.hip", "qmv_mfma_bf16.hip", "qmv_mfma_f16_odd.hip", "qmv_mfma_bf16_odd.hip", "qmv_wide.hip", "qmv_wide_gather.hip", "generic.hip", "qmm.hip", "qmm_direct.hip", "qmm_direct_odd.hip", "qmm_dma.hip", "qmm_dma_b8.hip", "qmm_f32.hip", "affine.hip", "norm.hip", "moe.hip", "moe_down.hip", "qvm.hip"]
 
 
 def _headers():

@@ -484,6 +484,10 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
     // exact_only: the caller named a reference kernel that multiplies by the exact f32 s*q + b
     // (mt_moe_gather_qmm_int4* / _b*, crates/metaltile-std/src/ffai/moe.rs:358-433); the tile kernel rounds
     // that value to the element type first, so such a name stays on the GEMV kernels at any routing density.
+    if (dtype != DT_F32 && mode != GATHER_SINGLE && options().gather_wide == 2) {
+        rc = launch_qmv_wide_gather(p, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
     if (dtype != DT_F32 && mode != GATHER_SINGLE && gopt != 1 && (gopt == 2 || (!exact_only && (uint64_t)T > (uint64_t)8 * (E < T ? E : T)))) {
         QmmParams q;
         q.dtype = dtype; q.bits = bits; q.group_size = G;
@@ -493,6 +497,16 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
         rc = ensure_scratch(qmm_grouped_scratch_bytes(T, E, ids, 32));  // sized for the smaller tile height: more tiles
         if (rc) return rc;
         rc = launch_qmm_grouped(q, route, ids, T, E, g.scratch_buf, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
+    // More than 4 rows per expert on large experts, below the tile kernel's crossover or under a name that must stay
+    // exact: the 16-row matrix-core GEMV, 16 rows of an expert per pass. 8 experts x 14336 x 4096, rows by random ids,
+    // us, 8-row passes of the GEMV family -> this: 64 rows 113 -> 64, 128 rows 199 -> 118, 256 rows 359 -> 171 (the tiles,
+    // rounded weights: 80 and 98 at 128 and 256 rows). It loses below (16 rows 54 -> 60, 32 rows 58 -> 62: a workgroup
+    // stages 16 rows whatever the expert has) and on small experts.
+    if (dtype != DT_F32 && mode != GATHER_SINGLE && options().gather_wide == 0 && (uint64_t)N * K >= (1ull << 24) &&
+        (uint64_t)T > (uint64_t)4 * (E < T ? E : T)) {
+        rc = launch_qmv_wide_gather(p, lc);
         if (rc != ERR_UNSUPPORTED) return rc;
     }
     return run_gemv(p, lc);
@@ -1480,6 +1494,11 @@ int mtq_set_option(const char* name, int value) {
     if (!strcmp(name, "qmm.by_m")) {
         if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmm.by_m must be 0 (choose), 1 or 2 (off)");
         options().qmm_by_m = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "gather.wide")) {
+        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "gather.wide must be 0 (choose), 1 (never) or 2 (wherever the shape allows)");
+        options().gather_wide = value;
         return MTQ_OK;
     }
     if (!strcmp(name, "gather.grouped")) {

@@ -116,6 +116,7 @@ struct Options {
     int qmv_norm_mfma = 0;        // RMS norm fused into the matrix-core GEMV (4-bit f16 / bf16): 0 = choose, 1 = never, 2 = wherever the shape allows
     int qmv_wide_kp = 0;          // 16-row matrix-core GEMV: waves sharing a row block (0 = choose; 1, 2, 4, 8, 16)
     int qmv_wide_nb = 0;          // 16-row matrix-core GEMV: row blocks per wave (0 = choose; 1, 2)
+    int gather_wide = 0;          // expert-routed rows on the 16-row matrix-core GEMV: 0 = choose, 1 = never, 2 = wherever the shape allows
     int qmv_wide = 0;             // 16-row matrix-core GEMV for batches of 5..16 rows: 0 = choose per shape, 1 = never, 2 = wherever the shape allows
 };
 Options& options();
@@ -177,6 +178,8 @@ int launch_qmm_direct(const QmmParams& p, const LaunchCtx& lc, void* scratch);
 bool qmv_wide_takes(const QmmParams& p);
 size_t qmv_wide_scratch_bytes(const QmmParams& p);
 int launch_qmv_wide(const QmmParams& p, const LaunchCtx& lc, void* scratch);
+// The same kernel on expert-routed rows (p.gather = GATHER_CSR / GATHER_INDICES), 16 rows of an expert per pass.
+int launch_qmv_wide_gather(const QmvParams& p, const LaunchCtx& lc);
 // f32 operands on the f32 matrix cores, any code width (qmm_f32.hip).
 // scratch: qmm_f32_scratch_bytes(p) bytes (0 when K is not split: then scratch may be null).
 size_t qmm_f32_scratch_bytes(const QmmParams& p);
