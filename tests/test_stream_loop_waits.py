@@ -1,0 +1,69 @@
+"""The 16-row matrix-core GEMV issues its weight loads by hand and waits for them with hand-counted
+`s_waitcnt vmcnt(N)`. That only pipelines if the compiler adds no wait of its own inside the stream loop: one
+`vmcnt` wait it inserts there (for a register whose load it still believes pending, or for a spilled value it
+reloads) also waits for every load in flight, silently, with correct results. This test compiles the kernel's two
+translation units to assembly (no GPU needed) and checks, for every instance, that inside the loop that holds the
+MFMAs the only `vmcnt` waits are the four written by hand and that nothing there touches scratch memory."""
+import concurrent.futures
+import os
+import re
+import shutil
+import subprocess
+import tempfile
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "..", "metaltile_amd", "csrc")
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+
+
+def _assembly(src, out):
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I" + os.path.join(HERE, "..", "include"), "--cuda-device-only", "-S", os.path.join(CSRC, src), "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    return open(out).read().split("\n")
+
+
+def _stream_loops(lines):
+    """(kernel symbol, hand-written vmcnt waits, all vmcnt waits, scratch accesses, MFMAs) of each kernel's MFMA loop."""
+    starts = [(i, l.split(":")[0]) for i, l in enumerate(lines) if l.startswith("_ZN3mtq15qmv_wide_kernel") and "; @" in l]
+    starts.append((len(lines), ""))
+    for (s0, name), (s1, _) in zip(starts, starts[1:]):
+        body = lines[s0:s1]
+        found = None
+        for i, l in enumerate(body):
+            if "Inner Loop Header" not in l:
+                continue
+            k = i
+            while k >= 0 and not re.match(r"^\.LBB\d+_\d+:", body[k]):
+                k -= 1
+            label = body[k].split(":")[0]
+            j, mine, every, scratch, mfma = k + 1, 0, 0, 0, 0
+            while j < len(body) and not re.search(r"s_cbranch\w+ " + re.escape(label) + r"\b", body[j]):
+                if "s_waitcnt vmcnt" in body[j]:
+                    every += 1
+                    mine += "ASMSTART" in body[j - 1]
+                scratch += "scratch_" in body[j]
+                mfma += "v_mfma" in body[j]
+                j += 1
+            if mfma:
+                found = (name, mine, every, scratch, mfma)
+        assert found, f"{name}: no loop with MFMAs"
+        yield found
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc is needed to produce the assembly")
+def test_only_hand_counted_waits_in_the_stream_loop():
+    with tempfile.TemporaryDirectory() as tmp:
+        with concurrent.futures.ThreadPoolExecutor(max_workers=2) as ex:
+            outs = list(ex.map(lambda s: _assembly(s, os.path.join(tmp, s + ".s")), ["qmv_wide.hip", "qmv_wide_gather.hip"]))
+    n = 0
+    for lines in outs:
+        for name, mine, every, scratch, mfma in _stream_loops(lines):
+            assert mine == 4 and every == 4, f"{name}: {every} vmcnt waits in the stream loop, {mine} of them hand-written"
+            assert scratch == 0, f"{name}: {scratch} scratch accesses in the stream loop"
+            assert mfma in (16, 32), name
+            n += 1
+    assert n >= 40
