@@ -56,6 +56,7 @@ static bool wide_geometry(uint32_t G, uint32_t tps, uint32_t nrb, uint32_t want,
     pl.sets = (pl.tpk + 3u) / 4u;
     if (pl.sets > max_sets) return false;
     if (pl.nb == 2u && pl.sets > 2u) pl.nb = 1;
+    if (pl.nb == 2u && pl.sets == 1u && G == 128) pl.nb = 1;   // (that instance does not fit 128 registers; runs of at most 4 turns on very many rows)
     if (pl.kp > 1u && pl.lds < (size_t)16 * pl.nb * 1024) pl.lds = (size_t)16 * pl.nb * 1024;   // the K parts' sums, a KB per wave and row block
     const uint32_t per_wg = 16u * pl.nb / pl.kp;
     pl.grid_x = (nrb + per_wg - 1) / per_wg;
@@ -118,7 +119,7 @@ int launch_qmv_wide(const QmmParams& p, const LaunchCtx& lc, void* scratch) {
     a.T = p.M;
     a.E = 1;
     const void* fn = nullptr;
-#define QW_PICK3(DTv, Gv, NBv) (pl.sets == 1 ? (const void*)qmv_wide_kernel<DTv, Gv, NBv, 1> : pl.sets == 2 ? (const void*)qmv_wide_kernel<DTv, Gv, NBv, 2> : NBv == 1 ? (const void*)qmv_wide_kernel<DTv, Gv, 1, 3> : nullptr)
+#define QW_PICK3(DTv, Gv, NBv) (pl.sets == 1 ? (const void*)qmv_wide_kernel<DTv, Gv, (Gv == 128 ? 1 : NBv), 1> : pl.sets == 2 ? (const void*)qmv_wide_kernel<DTv, Gv, NBv, 2> : NBv == 1 ? (const void*)qmv_wide_kernel<DTv, Gv, 1, 3> : nullptr)
 #define QW_PICK2(DTv, NBv) (p.group_size == 32 ? (const void*)qmv_wide_kernel<DTv, 32, 1, 1> : p.group_size == 64 ? QW_PICK3(DTv, 64, NBv) : QW_PICK3(DTv, 128, NBv))
 #define QW_PICK(DTv) (pl.nb == 2 ? QW_PICK2(DTv, 2) : QW_PICK2(DTv, 1))
     fn = p.dtype == DT_BF16 ? QW_PICK(DT_BF16) : QW_PICK(DT_F16);

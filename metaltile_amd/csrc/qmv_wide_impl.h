@@ -172,11 +172,17 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
     const uint32_t t0 = min(kp * a.tpk, turns), t1 = min(t0 + a.tpk, turns), cnt = t1 - t0;   // cnt <= 4 * SETS (host)
     const uint32_t rb0 = (blockIdx.x * (NW >> a.log2kp) + wr) * NB;
     const uint32_t n_pass = GATHER ? (nrows + 15u) / 16u : 1u;
-    uint32_t row[NB], woff[NB];   // woff: byte offset of this lane's weights in turn 0 of the slice
+    // A weight load covers whole 128-byte lines: eight lanes share a row's line, so one instruction takes the line of
+    // rows 0 .. 7 of the block (woff[i][0]) and a second that of rows 8 .. 15 (woff[i][1]); lane (j, q) holds piece
+    // q + 4 (j / 8) of row j % 8 (or 8 + j % 8). (Four lanes to a row, 64 bytes of 16 lines per instruction, the same
+    // bytes streamed at 5.2 - 5.5 TB/s in a read-only kernel of this shape; whole lines at 6.3 - 6.5.)
+    uint32_t row[NB], woff[NB][2];   // woff: byte offsets of this lane's two loads in turn 0 of the slice
 #pragma unroll
     for (int i = 0; i < NB; i++) {   // row blocks past the matrix work on its last row and store nothing
         row[i] = (rb0 + i) * 16u + j;
-        woff[i] = min(row[i], a.N - 1u) * (a.K / 2u) + q * 16u;
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+            woff[i][h] = min((rb0 + i) * 16u + 8u * h + (j & 7u), a.N - 1u) * (a.K / 2u) + (q + 4u * (j >> 3)) * 16u;
     }
     const unsigned char* wbase = a.w + k0 / 2u;   // + 256 bytes per turn
 
@@ -185,12 +191,27 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
     // next turn and was fetched from memory again (4.8 x the bytes). The four lanes of a weight row take the turns
     // q, q + 4, q + 8 of the run (one 128-byte line per instruction and row); at turn n the lanes fetch the pairs from
     // lane quarter n % 4, register set n / 4, with ds_bpermute.
+    // With 16 bytes per turn (groups of 64 codes) and two sets, the first two are read as the weights are: eight lanes
+    // to a row, pieces q + 4 (j / 8) of rows j % 8 and 8 + j % 8, whole lines per instruction; the half rows change
+    // places behind the barrier below.
+    constexpr bool PAIRED = DPT == 4 && SETS >= 2;
     uint32_t sreg[NB][SETS][DPT], breg[NB][SETS][DPT];
 #pragma unroll
     for (int i = 0; i < NB; i++) {
-        const size_t e0 = (size_t)min(row[i], a.N - 1u) * a.gpr + k0 / (uint32_t)G;
+        [[maybe_unused]] const size_t e0 = (size_t)min(row[i], a.N - 1u) * a.gpr + k0 / (uint32_t)G;
+        if constexpr (PAIRED) {
 #pragma unroll
-        for (int st = 0; st < SETS; st++) {
+            for (int h = 0; h < 2; h++) {
+                const size_t eh = (size_t)min((rb0 + i) * 16u + 8u * h + (j & 7u), a.N - 1u) * a.gpr + k0 / (uint32_t)G;
+                const uint32_t n = min(q + 4u * (j >> 3), cnt ? cnt - 1u : 0u);
+                const size_t e = eh + (size_t)min(t0 + n, turns - 1u) * GPT;
+                const qw_u32x4 sv = *(const qw_u32x4*)(a.scales + e), bv = *(const qw_u32x4*)(a.biases + e);
+                sreg[i][h][0] = sv.x; sreg[i][h][1] = sv.y; sreg[i][h][2] = sv.z; sreg[i][h][3] = sv.w;
+                breg[i][h][0] = bv.x; breg[i][h][1] = bv.y; breg[i][h][2] = bv.z; breg[i][h][3] = bv.w;
+            }
+        }
+#pragma unroll
+        for (int st = PAIRED ? 2 : 0; st < SETS; st++) {
             const uint32_t n = min(4u * st + q, cnt ? cnt - 1u : 0u);   // a turn past the run: any valid address, never used
             const size_t e = e0 + (size_t)min(t0 + n, turns - 1u) * GPT;
             if constexpr (DPT == 2) {
@@ -225,7 +246,7 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
         qw_static_for<0, 4>([&](auto d_c) {
             constexpr int d = decltype(d_c)::value;
 #pragma unroll
-            for (int i = 0; i < NB; i++) qw_load_once<d * 64>(ring[i][d], woff[i], wbase + tc * 256u);
+            for (int i = 0; i < NB; i++) qw_load_once<(d / 2) * 128>(ring[i][d], woff[i][d % 2], wbase + tc * 256u);
         });
     }
 
@@ -277,6 +298,21 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
         for (int st = 0; st < SETS; st++)
 #pragma unroll
             for (int k = 0; k < DPT; k++) { qw_tie(sreg[i][st][k]); qw_tie(breg[i][st][k]); }
+    if (PAIRED && pass == 0u) {
+        // set 0 = turn q, set 1 = turn 4 + q of row j: lanes j >= 8 take set 0 from the second load of lane j - 8,
+        // lanes j < 8 take set 1 from the first load of lane j + 8
+        constexpr int ROR8 = 0x128;
+#pragma unroll
+        for (int i = 0; i < NB; i++)
+#pragma unroll
+            for (int k = 0; k < DPT; k++) {
+                const uint32_t s0 = sreg[i][0][k], s1 = sreg[i][1][k], b0 = breg[i][0][k], b1 = breg[i][1][k];
+                sreg[i][0][k] = (uint32_t)__builtin_amdgcn_update_dpp((int)s0, (int)s1, ROR8, 0xF, 0xC, false);
+                sreg[i][1][k] = (uint32_t)__builtin_amdgcn_update_dpp((int)s1, (int)s0, ROR8, 0xF, 0x3, false);
+                breg[i][0][k] = (uint32_t)__builtin_amdgcn_update_dpp((int)b0, (int)b1, ROR8, 0xF, 0xC, false);
+                breg[i][1][k] = (uint32_t)__builtin_amdgcn_update_dpp((int)b1, (int)b0, ROR8, 0xF, 0x3, false);
+            }
+    }
 
     // ---- stream ---------------------------------------------------------------------------------------------------
     const uint32_t kor = magic_or_vgpr<DT>();
@@ -288,11 +324,10 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
     for (int i = 0; i < NB; i++)
 #pragma unroll
         for (int r = 0; r < 4; r++) tot[i][r] = 0.f;
-    // One turn: 512 codes of every row block of the wave. The registers of two steps are reloaded for the next turn
-    // together, behind steps 1 and 3, so that both 64-byte halves of a 128-byte line are asked for at the same time
-    // (asked for a quarter turn apart, most lines were fetched from memory twice: the loads are marked as read
-    // once). Loads outstanding at the top of a turn: its weights, 4 NB; when step d's are needed, the younger ones
-    // are the rest of the turn's and the next turn's issued so far: 3 NB at steps 0 and 2, 2 NB at steps 1 and 3.
+    // One turn: 512 codes of every row block of the wave, in four steps of 128. ring[i][2 p] and ring[i][2 p + 1] hold
+    // line p of the turn (steps 2 p and 2 p + 1) for rows 0 .. 7 and 8 .. 15 of block i; both are reloaded for the next
+    // turn behind step 2 p + 1. Loads outstanding at the top of a turn: its weights, 4 NB; when line p is needed, the
+    // younger ones are the other line's, of this turn (p = 0) or the next (p = 1): 2 NB.
     for (uint32_t n = 0; n < cnt; n++) {
         const uint32_t t = t0 + n;
         const bool has_next = n + 1u < cnt;
@@ -305,14 +340,36 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
         qw_f32x4 acc[NB];
         qw_static_for<0, 4>([&](auto d_c) {
             constexpr int d = decltype(d_c)::value;
-            qw_wait<(d % 2 ? 2 : 3) * NB>();
+            if constexpr (d % 2 == 0) {
+                qw_wait<2 * NB>();
+#pragma unroll
+                for (int i = 0; i < NB; i++) { qw_tie(ring[i][d]); qw_tie(ring[i][d + 1]); }
+            }
             uint32_t v[NB][4];
 #pragma unroll
             for (int i = 0; i < NB; i++) {
-                qw_tie(ring[i][d]);
+                // The step's 64 bytes of row j: lanes j < 8 hold the line's first half of their own row in the first
+                // register and the first half of row j + 8 in the second; lanes j >= 8 hold the second half of row
+                // j - 8 and of their own. Each half row changes places with the lane 8 further on (a rotation by 8
+                // within the 16 lanes, written to half of them).
+                qw_u32x4 w4;
+                {
+                    const qw_u32x4 ra = ring[i][d & ~1], rb = ring[i][d | 1];
+                    constexpr int ROR8 = 0x128;
+                    if constexpr (d % 2 == 0) {   // first half: lanes j >= 8 take it from the second register of lane j - 8
+                        w4.x = (uint32_t)__builtin_amdgcn_update_dpp((int)ra.x, (int)rb.x, ROR8, 0xF, 0xC, false);
+                        w4.y = (uint32_t)__builtin_amdgcn_update_dpp((int)ra.y, (int)rb.y, ROR8, 0xF, 0xC, false);
+                        w4.z = (uint32_t)__builtin_amdgcn_update_dpp((int)ra.z, (int)rb.z, ROR8, 0xF, 0xC, false);
+                        w4.w = (uint32_t)__builtin_amdgcn_update_dpp((int)ra.w, (int)rb.w, ROR8, 0xF, 0xC, false);
+                    } else {                      // second half: lanes j < 8 take it from the first register of lane j + 8
+                        w4.x = (uint32_t)__builtin_amdgcn_update_dpp((int)rb.x, (int)ra.x, ROR8, 0xF, 0x3, false);
+                        w4.y = (uint32_t)__builtin_amdgcn_update_dpp((int)rb.y, (int)ra.y, ROR8, 0xF, 0x3, false);
+                        w4.z = (uint32_t)__builtin_amdgcn_update_dpp((int)rb.z, (int)ra.z, ROR8, 0xF, 0x3, false);
+                        w4.w = (uint32_t)__builtin_amdgcn_update_dpp((int)rb.w, (int)ra.w, ROR8, 0xF, 0x3, false);
+                    }
+                }
                 // 4 x 4 transpose of the step's dwords among the lanes j, j + 16, j + 32, j + 48: before, dword u of
                 // lane quarter q is codes [32 q + 8 u, +8) of the step; after, codes [32 u + 8 q, +8)
-                const qw_u32x4 w4 = ring[i][d];
                 const auto a02 = __builtin_amdgcn_permlane32_swap(w4.x, w4.z, false, false);
                 const auto a13 = __builtin_amdgcn_permlane32_swap(w4.y, w4.w, false, false);
                 const auto b01 = __builtin_amdgcn_permlane16_swap(a02[0], a13[0], false, false);
@@ -321,9 +378,10 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
             }
             if constexpr (d % 2 == 1) {
 #pragma unroll
-                for (int i = 0; i < NB; i++) qw_load_once<(d - 1) * 64>(ring[i][d - 1], has_next ? woff[i] : 0u, wbase + tn * 256u);
-#pragma unroll
-                for (int i = 0; i < NB; i++) qw_load_once<d * 64>(ring[i][d], has_next ? woff[i] : 0u, wbase + tn * 256u);
+                for (int i = 0; i < NB; i++) {
+                    qw_load_once<(d / 2) * 128>(ring[i][d - 1], has_next ? woff[i][0] : 0u, wbase + tn * 256u);
+                    qw_load_once<(d / 2) * 128>(ring[i][d], has_next ? woff[i][1] : 0u, wbase + tn * 256u);
+                }
             }
 #pragma unroll
             for (int u = 0; u < 4; u++) {
@@ -390,9 +448,10 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
             const uint32_t orow = batch_row(row_base + m);
 #pragma unroll
             for (int i = 0; i < NB; i++) {
-                if (row[i] >= a.N) continue;
-                if (!GATHER && gridDim.y > 1) a.part[((size_t)blockIdx.y * a.M + orow) * a.N + row[i]] = tot[i][r];
-                else ((uint16_t*)a.out)[(size_t)orow * a.N + row[i]] = f32_to_elem_bits<DT>(tot[i][r]);
+                const uint32_t wrow = (rb0 + i) * 16u + j;   // (worked out again: one register fewer across the stream)
+                if (wrow >= a.N) continue;
+                if (!GATHER && gridDim.y > 1) a.part[((size_t)blockIdx.y * a.M + orow) * a.N + wrow] = tot[i][r];
+                else ((uint16_t*)a.out)[(size_t)orow * a.N + wrow] = f32_to_elem_bits<DT>(tot[i][r]);
             }
         }
     }
