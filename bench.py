@@ -46,8 +46,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    # (a step is 0.2 ms: the card's clocks settle over the first ~20 ms of load, so the default warm-up is that long)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--layers", type=int, default=8, help="distinct MLP weight sets streamed per step")
     ap.add_argument("--workload", default="qmv",
                     choices=["qmv", "qkv", "qmm", "batch", "gather", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep"],

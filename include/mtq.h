@@ -401,7 +401,7 @@ MTQ_API int mtq_flush_cache(void);
  *                          0 = where it is faster than the streaming kernel's fused form, 1 = never, 2 = wherever the
  *                          shape allows
  *   "gather.wide"          expert-routed rows on the 16-row matrix-core GEMV (4-bit g64 f16 / bf16, K <= 4608): 0 = where
- *                          it is the fastest kernel (large experts, more than 4 rows per expert, below the tile
+ *                          it is the fastest kernel (large experts, at least 4 rows per expert, below the tile
  *                          kernel's crossover or under an exact-dequant name), 1 = never, 2 = wherever the shape allows
  *   "qmv.wide"             16-row matrix-core GEMV for batches of 5..16 rows (4-bit codes, f16 / bf16, K % 512 == 0):
  *                          0 = where it is the fastest kernel, 1 = never, 2 = wherever the shape allows

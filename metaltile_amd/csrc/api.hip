@@ -240,12 +240,13 @@ static int try_wide(int dtype, int bits, uint32_t G, const void* w, const void* 
     if (!qmv_wide_takes(q)) return ERR_UNSUPPORTED;
     // Every workgroup stages its 16 rows of activations (128 KB at K = 4096), which pays once a compute unit streams
     // several times that in weights. us, 5 / 8 / 12 / 16 rows, the other kernels (GEMV passes of up to 8 rows | tiles)
-    // against this one: 128256 x 4096 67 69 118 133 | 90 91 92 93 -> 63 62 63 66; 57344 x 4096 32 33 60 66 | 43 44 44
-    // 46 -> 31 32 33 34; 28672 x 8192 53 54 81 109 | 46 46 46 47 -> 33 34 35 36; 32768 x 4096 21 22 37 41 | 26 27 27 27
-    // -> 20 20 21 22; 14336 x 4096 13 14 24 27 | 13 13 13 14 -> 13 14 15 15; 4096 x 4096 7.5 8.1 10.6 12.8 | 9.3 9.5 9.9
-    // 10.0 -> 10.4 11.2 12.0 12.8.
+    // against this one: 128256 x 4096 69 66 116 131 | 88 89 90 92 -> 54 53 55 55; 57344 x 4096 31 32 56 62 | 42 43 43
+    // 44 -> 26 27 28 29; 28672 x 8192 50 52 77 103 | 45 45 45 45 -> 29 30 31 32; 32768 x 4096 21 22 38 43 | 27 27 27 28
+    // -> 17.5 18.3 19.5 20.3; 8192 x 8192 19 22 32 42 | 17.4 16.9 17.1 17.4 -> 14.8 15.6 17.2 18.3; 14336 x 4096 13.1 13.6
+    // 23 27 | 13.5 13.4 13.6 13.7 -> 12.3 12.9 13.8 14.7; 4096 x 14336 23 25 38 50 | 15.2 15.4 15.9 16.0 -> 14.8 15.1 16.2
+    // 17.4; 4096 x 4096 7.6 8.3 10.7 12.6 | 9.4 9.6 9.9 10.1 -> 10.1 10.7 11.4 12.1.
     const uint64_t codes = (uint64_t)N * K;
-    const bool pays = exact && M >= 9 ? codes >= (1ull << 25) : codes >= 100000000ull;
+    const bool pays = M <= 8 ? codes >= 50000000ull : exact ? codes >= (1ull << 25) : codes >= 100000000ull;
     if (options().qmv_wide != 2 && !pays) return ERR_UNSUPPORTED;
     const size_t need = qmv_wide_scratch_bytes(q);
     if (need) {
@@ -499,13 +500,13 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
         rc = launch_qmm_grouped(q, route, ids, T, E, g.scratch_buf, lc);
         if (rc != ERR_UNSUPPORTED) return rc;
     }
-    // More than 4 rows per expert on large experts, below the tile kernel's crossover or under a name that must stay
+    // From 4 rows per expert on large experts, below the tile kernel's crossover or under a name that must stay
     // exact: the 16-row matrix-core GEMV, 16 rows of an expert per pass. 8 experts x 14336 x 4096, rows by random ids,
-    // us, 8-row passes of the GEMV family -> this: 64 rows 113 -> 64, 128 rows 199 -> 118, 256 rows 359 -> 171 (the tiles,
-    // rounded weights: 80 and 98 at 128 and 256 rows). It loses below (16 rows 54 -> 60, 32 rows 58 -> 62: a workgroup
-    // stages 16 rows whatever the expert has) and on small experts.
+    // us, 8-row passes of the GEMV family -> this: 32 rows 58.6 -> 54.5 (CSR 63 -> 60), 64 rows 113 -> 56, 128 rows
+    // 197 -> 105, 256 rows 345 -> 152 (the tiles, rounded weights: 82 and 99 at 128 and 256 rows). It loses below (16 rows
+    // 53 -> 54.5: a workgroup stages 16 rows whatever the expert has) and on small experts.
     if (dtype != DT_F32 && mode != GATHER_SINGLE && options().gather_wide == 0 && (uint64_t)N * K >= (1ull << 24) &&
-        (uint64_t)T > (uint64_t)4 * (E < T ? E : T)) {
+        (uint64_t)T >= (uint64_t)4 * (E < T ? E : T)) {
         rc = launch_qmv_wide_gather(p, lc);
         if (rc != ERR_UNSUPPORTED) return rc;
     }

@@ -138,7 +138,9 @@ def test_benchmark_configurations_are_routed_as_documented():
         assert "qmm_dma_kernel<2, 4, 2, 8, 0, false, true, false" in ks[0] and ls[0][1][:2] == (128, 2) and "qmm_split_reduce_kernel" in ks[1]
     ks, _ = kernels("qmm_mma", DType.BF16, 6, 64, 512, 4096, 4096)
     assert "qmm_direct_kernel<2, 6," in ks[0]          # other code widths stay on the register-staged tiles
-    ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 32)
+    ks, ls = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 32)   # 4 rows per expert: the routed 16-row GEMV
+    assert "qmv_wide_kernel<2, 64, 2, 2, 2>" in ks[0] and ls[0][1][:2] == (28, 8) and ls[0][2][0] == 1024
+    ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 16)           # 2 rows per expert: 8-row passes
     assert "qmv_mfma_kernel<2, 4," in ks[0]
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 4096, 4096, 8, 2048)
     assert "moe_count_sort_kernel" in ks[0] and "gather_tiles_kernel" in ks[1] and "qmm_dma_kernel<2, 2, 2, 8, 2, true" in ks[2]
