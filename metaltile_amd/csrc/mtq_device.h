@@ -326,4 +326,56 @@ __device__ __forceinline__ uint32_t csr_expert_rows(const uint32_t* off, uint32_
     return n1 + n2;
 }
 
+// Gathers with fewer rows than experts launch one grid row per activation row instead of one per expert (most
+// experts are not hit, and a workgroup that only finds that out holds its compute unit's LDS and wave slots while its
+// loads of the routing come back: 8 experts of 14336 x 4096 with one row took 17 us, the same bytes as one matrix 8).
+// Grid row `slot` serves the slot-th expert, in ascending order, that has a row; 0xFFFFFFFF if there are fewer.
+// The same in every lane. CSR view, the reference's rule E(t) = first e with t < off[e + 1], else 0
+// (crates/metaltile-std/src/ffai/moe.rs:376-385): expert e has rows iff min(off[e + 1], T) > min(max(off[1 .. e]), T),
+// and expert 0 also takes the rows past every offset.
+__device__ __forceinline__ uint32_t csr_slot_expert(const uint32_t* off, uint32_t E, uint32_t T, uint32_t slot, uint32_t lane) {
+    uint32_t mx = 0;
+    for (uint32_t j0 = 1; j0 <= E; j0 += 64) mx = max(mx, j0 + lane <= E ? off[j0 + lane] : 0u);
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, d, 64));
+    const bool tail = min(mx, T) < T;
+    uint32_t seen = 0, carry = 0;   // carry: max(off[1 .. e0])
+    for (uint32_t e0 = 0; e0 < E; e0 += 64) {
+        const uint32_t e = e0 + lane;
+        const uint32_t o_hi = e < E ? off[e + 1] : 0u;
+        uint32_t incl = o_hi;   // inclusive prefix maximum over the lanes
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = (uint32_t)__shfl_up((int)incl, d, 64);
+            if (lane >= (uint32_t)d) incl = max(incl, up);
+        }
+        uint32_t before = (uint32_t)__shfl_up((int)incl, 1, 64);
+        before = max(lane ? before : 0u, carry);
+        const bool hit = e < E && (min(o_hi, T) > min(before, T) || (e == 0 && tail));
+        unsigned long long m = __ballot(hit);
+        const uint32_t c = (uint32_t)__popcll(m);
+        if (slot < seen + c) {
+            for (uint32_t i = seen; i < slot; i++) m &= m - 1ull;
+            return e0 + (uint32_t)__ffsll((long long)m) - 1u;
+        }
+        seen += c;
+        carry = max(carry, (uint32_t)__shfl((int)incl, 63, 64));
+    }
+    return 0xFFFFFFFFu;
+}
+// Per-row ids (at most 64 rows): the slot-th smallest id below E that a row names.
+__device__ __forceinline__ uint32_t ids_slot_expert(const uint32_t* ids, uint32_t E, uint32_t T, uint32_t slot, uint32_t lane) {
+    uint32_t v = lane < T ? ids[lane] : 0xFFFFFFFFu;
+    if (v >= E) v = 0xFFFFFFFFu;
+    uint32_t cur = 0xFFFFFFFFu;
+    for (uint32_t i = 0; i <= slot; i++) {
+        uint32_t c = (i == 0 || v > cur) ? v : 0xFFFFFFFFu;   // ids above the last one found
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) c = min(c, (uint32_t)__shfl_xor((int)c, d, 64));
+        if (c == 0xFFFFFFFFu) return c;
+        cur = c;
+    }
+    return cur;
+}
+
 }  // namespace mtq

@@ -238,6 +238,9 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     a.gpw = gpw;
     a.log2g = ilog2(G);
     a.list_cap = list_cap;
+    // fewer rows than experts: a grid row per row, each finding the expert it serves (at most T experts have rows)
+    const bool by_slot = (p.gather == GATHER_CSR || p.gather == GATHER_INDICES) && p.T < p.E && p.T <= 32;
+    a.by_slot = by_slot ? 1u : 0u;
     a.norm_w = p.norm_w;
     a.norm_eps = p.norm_eps;
     const int mode = norm ? (int)GATHER_NORM : p.gather;
@@ -247,7 +250,7 @@ int launch_qmv_mfma(const QmvParams& p, const LaunchCtx& lc) {
     g.tpb = 64u * KP * RBW;
     const uint32_t rows_wg = 4 * RBW * nrb;
     g.shmem = lds_bytes(R, nchp * cpc, nch, gpr, rows_wg, KP * RBW, gpw, KP, list_cap);
-    g.grid = dim3((p.N + rows_wg - 1) / rows_wg, gather ? p.E : 1, 1);
+    g.grid = dim3((p.N + rows_wg - 1) / rows_wg, by_slot ? p.T : gather ? p.E : 1, 1);
     if (odd)
         return p.dtype == DT_F16 ? qmv_mfma_launch_dtype_odd<DT_F16>(a, half2 ? 22 : p.bits, mode, g, lc)
                                  : qmv_mfma_launch_dtype_odd<DT_BF16>(a, half2 ? 22 : p.bits, mode, g, lc);

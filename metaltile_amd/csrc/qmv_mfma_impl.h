@@ -75,6 +75,7 @@ struct QmvMArgs {
     uint32_t gpr, log2g;
     uint32_t gpw;       // (scale, bias) pairs per row that a wave keeps in LDS: the groups of its K part, whole 4-vectors, <= 64
     uint32_t list_cap;  // capacity of the row list (indices mode)
+    uint32_t by_slot;   // gathers: blockIdx.y counts the experts that have rows (fewer rows than experts), not all experts
     const void* norm_w;     // GATHER_NORM: the norm's weights [K] and its epsilon
     const float* norm_eps;
 };
@@ -220,11 +221,19 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     uint32_t expert = 0, cnt = a.M, lo = 0, n1 = a.M, lo2 = 0;
     if constexpr (MODE == GATHER_CSR) {
         expert = blockIdx.y;
+        if (a.by_slot) {
+            expert = __builtin_amdgcn_readfirstlane(csr_slot_expert(a.route, a.E, a.T, blockIdx.y, lane));   // (the same in every lane: a scalar)
+            if (expert == NOROW) return;
+        }
         // E(t) = first e with t < off[e+1], else 0 (crates/metaltile-std/src/ffai/moe.rs:376-385)
         cnt = csr_expert_rows(a.route, a.E, a.T, expert, lane, lo, n1, lo2);
         if (cnt == 0) return;
     } else if constexpr (MODE == GATHER_INDICES) {
         expert = blockIdx.y;
+        if (a.by_slot) {
+            expert = __builtin_amdgcn_readfirstlane(ids_slot_expert(a.route, a.E, a.T, blockIdx.y, lane));
+            if (expert == NOROW) return;
+        }
         if (tid < 64) {
             uint32_t n = 0;
             for (uint32_t t0 = 0; t0 < a.T; t0 += 64) {

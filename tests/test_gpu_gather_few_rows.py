@@ -1,0 +1,89 @@
+"""gather_qmv with fewer rows than experts (a decode step of a mixture-of-experts layer: one or two tokens, top-k):
+the launch has one grid row per activation row and each grid row finds the expert it serves on the device, instead
+of one grid row per expert most of which find no row. Both routing views against the gather oracle
+(crates/metaltile-std/src/ffai/moe.rs:3577-3622), 1e-2 on max|a-e| / max(|e|, 1) for f16 / bf16; more than 64
+experts (the scan walks them in chunks of 64), rows that name the same expert, CSR offsets that leave rows past the
+last offset to expert 0 (moe.rs:376-385), offsets that step back, and ids that name no expert."""
+import numpy as np
+import pytest
+
+from metaltile_amd import DType, GpuBuffer, _lib, ops, unpack_f32
+from metaltile_amd.synth import make_case
+from tests.parity import rel_err
+
+pytestmark = pytest.mark.gpu
+ODT = {DType.F16: 1, DType.BF16: 2}
+
+
+def _offsets(ids, E):
+    return np.concatenate([[0], np.cumsum(np.bincount(ids, minlength=E))]).astype("<u4")
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("E,ids", [(8, [3]), (8, [1, 6]), (8, [0, 7]), (8, [2, 2, 5]), (8, [0, 1, 2, 3, 4, 5, 6]),
+                                   (130, [0, 63, 64, 65, 128, 129]), (130, [129]), (70, [64, 64, 64, 69]),
+                                   (40, list(range(4, 36)))],
+                         ids=lambda v: str(v) if isinstance(v, int) else "-".join(map(str, v[:6])))
+def test_fewer_rows_than_experts(oracle, dt, E, ids):
+    bits, G, N, K = 4, 64, 264, 1024
+    T = len(ids)
+    idn = np.array(ids, dtype="<u4")
+    c = make_case(8400 + E + T, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
+    exp = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=idn, f64=True, threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt]).reshape(T, N)
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    for view, route, fn in (("csr", _offsets(idn, E), ops.gather_qmv_csr), ("indices", idn, ops.gather_qmv_indices)):
+        print(f"[case] few-row gather {view} {dt.name} E{E} ids={ids}", flush=True)
+        rc, launches, _, n = ops.plan("gather_" + view, dt, bits, G, 1, N, K, E, T)
+        assert rc == 0 and n == 1 and "qmv_mfma_kernel" in launches[0][0] and launches[0][1][1] == T, launches
+        out, r = GpuBuffer.from_bytes(b"\xff" * (T * N * dt.size_bytes)), GpuBuffer.from_bytes(route.tobytes())
+        fn(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+        got = unpack_f32(out.read_bytes(), dt).reshape(T, N)
+        assert rel_err(got.reshape(-1), exp.reshape(-1)) <= 1e-2, view
+        out.free(); r.free()
+    for buf in (w, s, b, x):
+        buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+def test_fewer_rows_than_experts_odd_routing(oracle, dt):
+    """Offsets that end short (the last rows go to expert 0), offsets that step back (a later, smaller offset gives its
+    expert no row), and per-row ids that name no expert (those output rows keep their bytes)."""
+    bits, G, N, K, E, T = 4, 64, 132, 512, 9, 5
+    c = make_case(8500, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+
+    def run_csr(off, ids_equiv, label):
+        exp = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=np.array(ids_equiv, dtype="<u4"),
+                                f64=True, threads=8)
+        exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+        via_offsets = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G,
+                                        expert_offsets=np.array(off, dtype="<u4"), f64=True, threads=8)
+        assert np.array_equal(oracle.round_through(via_offsets.astype(np.float32), ODT[dt]), exp), label   # the rule, as the oracle reads it
+        print(f"[case] few-row gather csr {dt.name} {label} off={off}", flush=True)
+        out, r = GpuBuffer(T * N * dt.size_bytes), GpuBuffer.from_bytes(np.array(off, dtype="<u4").tobytes())
+        ops.gather_qmv_csr(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+        assert rel_err(unpack_f32(out.read_bytes(), dt), exp) <= 1e-2, label
+        out.free(); r.free()
+
+    #        e: 0  1  2  3  4  5  6  7  8
+    run_csr([0, 0, 0, 2, 2, 2, 2, 3, 3, 3], [2, 2, 6, 0, 0], "tail to expert 0")
+    run_csr([0, 1, 1, 3, 2, 2, 4, 4, 4, 5], [0, 2, 2, 5, 8], "an offset that steps back")
+    ids = np.array([7, E + 1, 7, 0xFFFFFFFF, 2], dtype="<u4")
+    exp = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=np.array([7, 0, 7, 0, 2], dtype="<u4"),
+                            f64=True, threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt]).reshape(T, N)
+    print(f"[case] few-row gather indices {dt.name} nameless ids", flush=True)
+    out, r = GpuBuffer.from_bytes(b"\xab" * (T * N * dt.size_bytes)), GpuBuffer.from_bytes(ids.tobytes())
+    ops.gather_qmv_indices(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+    raw = out.read_bytes()
+    got = unpack_f32(raw, dt).reshape(T, N)
+    rb = N * dt.size_bytes
+    for t in (1, 3):
+        assert raw[t * rb:(t + 1) * rb] == b"\xab" * rb
+    for t in (0, 2, 4):
+        assert rel_err(got[t], exp[t]) <= 1e-2
+    for buf in (w, s, b, x, out, r):
+        buf.free()
