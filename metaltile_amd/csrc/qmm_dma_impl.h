@@ -371,6 +371,13 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
         });
     }
     qm_wait_vm<0>();   // loads still in flight write into the ring the epilogue is about to reuse
+    // (The last weight loads are issued for iterations that do not exist and nothing reads them: to the compiler their
+    // registers are free from the loop's end on, and a value put there ahead of the wait would be overwritten when the
+    // load lands. Naming the registers behind the wait keeps them taken until then.)
+#pragma unroll
+    for (int ws = 0; ws < WSN; ws++)
+#pragma unroll
+        for (int k = 0; k < NWL; k++) asm volatile("" ::"v"(raw[ws][k]));
     __syncthreads();
 
     // ---- the other K-groups hand their accumulators to K-group 0 through LDS, at most 128 rows at a time ---

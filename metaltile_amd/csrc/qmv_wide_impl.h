@@ -422,6 +422,13 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
         });
     }
     qw_wait<0>();   // the last turn's loads, or those of a wave without turns
+    // (Nothing reads what those loads bring, so to the compiler their registers are free from the loop's end on, and it
+    // may put other values there ahead of the wait, for the loads to overwrite when they land. Naming the registers
+    // behind the wait keeps them taken until then.)
+#pragma unroll
+    for (int i = 0; i < NB; i++)
+#pragma unroll
+        for (int d = 0; d < 4; d++) qw_tie(ring[i][d]);
 
     // ---- the K parts of a row block meet in LDS (over the staged activations, which are done with) ---------------
     if (a.kp > 1u) {

@@ -3,7 +3,9 @@
 `vmcnt` wait it inserts there (for a register whose load it still believes pending, or for a spilled value it
 reloads) also waits for every load in flight, silently, with correct results. This test compiles the kernel's two
 translation units to assembly (no GPU needed) and checks, for every instance, that inside the loop that holds the
-MFMAs the only `vmcnt` waits are the two written by hand and that nothing there touches scratch memory."""
+MFMAs the only `vmcnt` waits are the two written by hand and that nothing there touches scratch memory; and that
+between the loop's end and the wait for its last loads (which nothing reads: dead registers to the compiler) nothing is
+written to a register one of those loads is still on its way to."""
 import concurrent.futures
 import os
 import re
@@ -26,8 +28,39 @@ def _assembly(src, out):
     return open(out).read().split("\n")
 
 
+def _regs(operand):
+    m = re.match(r"v\[(\d+):(\d+)\]", operand)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.match(r"v(\d+)$", operand)
+    return {int(m.group(1))} if m else set()
+
+
+def _early_writes(body, loop_end):
+    """The last turn's loads are still in flight when the loop ends and nothing reads them: to the compiler their
+    registers are free. A value written to one of them before the wait is overwritten when the load lands."""
+    ring = set()
+    for i, l in enumerate(body):
+        if "ASMSTART" in body[i - 1] and "global_load_dword" in l:
+            ring |= _regs(l.split()[1].rstrip(","))
+    assert ring
+    hits = []
+    for i in range(loop_end + 1, len(body)):
+        l = body[i]
+        if "s_waitcnt vmcnt(0)" in l and "ASMSTART" in body[i - 1]:
+            return hits
+        t = l.split()
+        if not t or t[0].startswith((";", ".", "s_", "ds_write", "global_store", "scratch_store", "buffer_store", "v_cmp")) or len(t) < 2:
+            continue
+        if _regs(t[1].rstrip(",")) & ring:
+            hits.append(l.strip())
+    raise AssertionError("no hand-written vmcnt(0) behind the stream loop")
+
+
 def _stream_loops(lines):
-    """(kernel symbol, hand-written vmcnt waits, all vmcnt waits, scratch accesses, MFMAs) of each kernel's MFMA loop."""
+    """(kernel symbol, hand-written vmcnt waits, all vmcnt waits, scratch accesses, MFMAs, early writes) of each kernel's
+    MFMA loop; early writes: instructions between the loop's end and the hand-written vmcnt(0) behind it that write a
+    register some hand-issued load targets."""
     starts = [(i, l.split(":")[0]) for i, l in enumerate(lines) if l.startswith("_ZN3mtq15qmv_wide_kernel") and "; @" in l]
     starts.append((len(lines), ""))
     for (s0, name), (s1, _) in zip(starts, starts[1:]):
@@ -48,10 +81,10 @@ def _stream_loops(lines):
                 scratch += "scratch_" in body[j]
                 mfma += "v_mfma" in body[j]
                 j += 1
-            if mfma:
-                found = (name, mine, every, scratch, mfma)
+            if mfma and j < len(body):   # (a loop whose back edge is not a conditional branch to its header is not the stream loop)
+                found = (name, mine, every, scratch, mfma, j)
         assert found, f"{name}: no loop with MFMAs"
-        yield found
+        yield found[:5] + (_early_writes(body, found[5]),)
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc is needed to produce the assembly")
@@ -61,9 +94,10 @@ def test_only_hand_counted_waits_in_the_stream_loop():
             outs = list(ex.map(lambda s: _assembly(s, os.path.join(tmp, s + ".s")), ["qmv_wide.hip", "qmv_wide_gather.hip"]))
     n = 0
     for lines in outs:
-        for name, mine, every, scratch, mfma in _stream_loops(lines):
+        for name, mine, every, scratch, mfma, early in _stream_loops(lines):
             assert mine == 2 and every == 2, f"{name}: {every} vmcnt waits in the stream loop, {mine} of them hand-written"
             assert scratch == 0, f"{name}: {scratch} scratch accesses in the stream loop"
+            assert not early, f"{name}: registers with loads in flight are written before the wait behind the loop: {early[:3]}"
             assert mfma in (16, 32), name
             n += 1
     assert n >= 40
