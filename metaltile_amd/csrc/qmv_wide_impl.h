@@ -235,6 +235,11 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
         for (int d = 0; d < 4; d++) ring[i][d] = qw_u32x4{0u, 0u, 0u, 0u};
     for (uint32_t pass = 0; pass < n_pass; pass++) {
     const uint32_t row_base = pass * 16u, live = min(16u, nrows - row_base);   // activation rows of this pass
+    // (With several passes, addresses that do not change from pass to pass - of the staged operands, of the K parts'
+    // sums, of the final stores - are worked out ahead of the pass loop and live across every stream in registers there
+    // are none left for: each wave spills them. They are worked out from the lane's coordinates plus a zero that the
+    // optimiser cannot tell from a value that changes with the pass.)
+    const uint32_t pz = GATHER ? pass & (a.log2kp >> 16) : 0u;
     // ---- the first turn's weights: in flight while the activations are staged --------------------------------------
     // The weight loads of the stream are issued by hand, in a fixed order, and waited for with "at most N loads
     // outstanding": the compiler would sink the loads to the end of a turn and wait for all of them at its top.
@@ -317,8 +322,8 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
     // ---- stream ---------------------------------------------------------------------------------------------------
     const uint32_t kor = magic_or_vgpr<DT>();
     const uint32_t msk = 0x000F000Fu;
-    const unsigned char* xl_lane = lds + (q * 16u + j) * 16u;
-    const unsigned char* xg_lane = (const unsigned char*)(XG + 4u * q);
+    const unsigned char* xl_lane = lds + (q * 16u + j + pz) * 16u;
+    const unsigned char* xg_lane = (const unsigned char*)(XG + 4u * (q + pz));
     float tot[NB][4];
 #pragma unroll
     for (int i = 0; i < NB; i++)
@@ -437,25 +442,26 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
 #pragma unroll
         for (int i = 0; i < NB; i++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) red[((wave * NB + i) * 4u + r) * 64u + lane] = tot[i][r];
+            for (int r = 0; r < 4; r++) red[((wave * NB + i) * 4u + r) * 64u + lane + pz] = tot[i][r];
         __syncthreads();
         if (kp == 0u)
         for (uint32_t o = 1; o < a.kp; o++)
 #pragma unroll
             for (int i = 0; i < NB; i++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) tot[i][r] += red[(((wave + o) * NB + i) * 4u + r) * 64u + lane];
+                for (int r = 0; r < 4; r++) tot[i][r] += red[(((wave + o) * NB + i) * 4u + r) * 64u + lane + pz];
     }
     // activation rows 4 q .. 4 q + 3 of the pass, weight row `row`
     if (kp == 0u) {
+        const uint32_t jp = j + pz, qp = q + pz;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const uint32_t m = 4u * q + r;
+            const uint32_t m = 4u * qp + r;
             if (m >= live) continue;
             const uint32_t orow = batch_row(row_base + m);
 #pragma unroll
             for (int i = 0; i < NB; i++) {
-                const uint32_t wrow = (rb0 + i) * 16u + j;   // (worked out again: one register fewer across the stream)
+                const uint32_t wrow = (rb0 + i) * 16u + jp;   // (worked out again: one register fewer across the stream)
                 if (wrow >= a.N) continue;
                 if (!GATHER && gridDim.y > 1) a.part[((size_t)blockIdx.y * a.M + orow) * a.N + wrow] = tot[i][r];
                 else ((uint16_t*)a.out)[(size_t)orow * a.N + wrow] = f32_to_elem_bits<DT>(tot[i][r]);
