@@ -151,14 +151,23 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     // this wave's load-to-LDS instructions: unit q = wave * IPW + i is quarter q % 4 of slot q / 4; slot sl holds
     // row block sl % MB, k-block sl / MB of the iteration; a quarter is 8 rows x 128 bytes, lane l moving chunk
     // (l % 8) ^ ((row / 2) % 8) of row 8 * quarter + l / 8
-    uint32_t xoff[IPW];
-#pragma unroll
-    for (int i = 0; i < IPW; i++) {
+    auto x_offset = [&](int i) -> uint32_t {
         const uint32_t q = wave * IPW + i, sl = q / 4, t = q % 4;
         const uint32_t rr = 8 * t + (lane >> 3), c = (lane & 7u) ^ ((rr >> 1) & 7u);
         const uint32_t lrow = min((sl % MB) * 32 + rr, row_count - 1);
-        xoff[i] = row_of(lrow) * (a.K * 2) + (sl / MB) * 128 + c * 16;
-    }
+        return row_of(lrow) * (a.K * 2) + (sl / MB) * 128 + c * 16;
+    };
+    // 256-row tiles with windows have no register to spare (three of these offsets were spilled and reloaded inside
+    // the loop, each reload with the compiler's wait for every load in flight): a wave's instructions 4 .. 7 there move
+    // the row block after that of instructions 0 .. 3, 32 rows on, which in a full tile is the same lane offsets from
+    // a base 32 rows on. Only those four are kept; a ragged last tile (rows clamped per lane) works its offsets out
+    // again at every use.
+    constexpr bool LEAN = MB == 8 && WIN && !GR && IPW == 8;
+    constexpr int NXO = LEAN ? 4 : IPW;
+    const bool full_tile = row_count == (uint32_t)DBM;
+    uint32_t xoff[NXO];
+#pragma unroll
+    for (int i = 0; i < NXO; i++) xoff[i] = x_offset(i);
     // fragment reads: MFMA step j of lane (fr, fh) takes chunk 4 * fh + j of row fr of slot (bi, kg)
     uint32_t aoff[4];
 #pragma unroll
@@ -201,7 +210,16 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     auto issue_x = [&](uint32_t it, int buf) {
         const unsigned char* src = a.x + (size_t)min(it, ilast) * (DBK * 2);
 #pragma unroll
-        for (int i = 0; i < IPW; i++) qm_load_to_lds(ring + buf * TILE + (wave * IPW + i) * 1024, xoff[i], src);
+        for (int i = 0; i < NXO; i++) qm_load_to_lds(ring + buf * TILE + (wave * IPW + i) * 1024, xoff[i], src);
+        if constexpr (LEAN) {
+            if (full_tile) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) qm_load_to_lds(ring + buf * TILE + (wave * IPW + 4 + i) * 1024, xoff[i], src + (size_t)32 * a.K * 2);
+            } else {
+#pragma unroll
+                for (int i = 4; i < 8; i++) qm_load_to_lds(ring + buf * TILE + (wave * IPW + i) * 1024, x_offset(i), src);
+            }
+        }
     };
     qm_u32x4 raw[WSN][NWL];
     auto issue_w = [&](uint32_t it, int set) {
