@@ -142,6 +142,12 @@ def test_benchmark_configurations_are_routed_as_documented():
     assert "qmv_wide_kernel<2, 64, 2, 2, 2>" in ks[0] and ls[0][1][:2] == (28, 8) and ls[0][2][0] == 1024
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 16)           # 2 rows per expert: 8-row passes
     assert "qmv_mfma_kernel<2, 4," in ks[0]
+    for view in ("gather_csr", "gather_indices"):      # fewer rows than experts: a grid row per row, not per expert
+        for T, E in ((1, 8), (2, 8), (7, 8), (8, 128), (32, 128)):
+            ks, ls = kernels(view, DType.BF16, 4, 64, 1, 14336, 4096, E, T)
+            assert "qmv_mfma_kernel<2, 4," in ks[0] and ls[0][1][1] == T, (view, T, E, ls)
+        ks, ls = kernels(view, DType.BF16, 4, 64, 1, 2048, 768, 128, 33)   # (more than 32 rows: a grid row per expert)
+        assert ls[0][1][1] == 128
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 4096, 4096, 8, 2048)
     assert "moe_count_sort_kernel" in ks[0] and "gather_tiles_kernel" in ks[1] and "qmm_dma_kernel<2, 2, 2, 8, 2, true" in ks[2]
     for bits, M in itertools.product((2, 4, 8), (1, 4)):   # the sweep configuration's cells
