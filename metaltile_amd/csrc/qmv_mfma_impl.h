@@ -636,11 +636,20 @@ int qmv_mfma_launch_one(QmvMArgs& a, const QmvMGeom& g, const LaunchCtx& lc) {
     // Two row sets (8 rows per pass) at 1024 threads leave 128 registers per lane and the kernel spills; at 512
     // threads it has 256 and keeps eight weight loads in flight per lane instead of four: the same bytes in flight
     // per compute unit from half the waves.
+    // A wave's steps per row block are walked in whole rings: with 4 steps (rows of 2048 4-bit codes) a ring of eight
+    // is half padding, loads included (128 experts of 256 x 2048, 8 rows each: 17.9 -> 23.2 us). The deep ring is taken
+    // where it pads no more than the ring of four does, and for 4-bit codes only (8-bit, 8 rows, 4096 x 4096: 10.2 us
+    // on the ring of eight, 9.2 on that of four; larger matrices alike).
     constexpr int MAXT = S >= 2 ? 512 : 1024;
-    constexpr int D = (S == 2 && (BITS == 4 || BITS == 8)) ? 8 : 4;
+    constexpr bool DEEP = S == 2 && BITS == 4;
     if (g.tpb > (uint32_t)MAXT) return fail(ERR_UNSUPPORTED, "mfma qmv: workgroup too large for this row count");
-    const void* fn = a.nrb > 1 ? (const void*)qmv_mfma_kernel<DT, BITS, MP, S, D, MODE, MAXT, true>
-                               : (const void*)qmv_mfma_kernel<DT, BITS, MP, S, D, MODE, MAXT, false>;
+    const void* fn = a.nrb > 1 ? (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT, true>
+                               : (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 4, MODE, MAXT, false>;
+    if constexpr (DEEP) {
+        if ((a.spp + 7u) / 8u * 8u == (a.spp + 3u) / 4u * 4u)
+            fn = a.nrb > 1 ? (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 8, MODE, MAXT, true>
+                           : (const void*)qmv_mfma_kernel<DT, BITS, MP, S, 8, MODE, MAXT, false>;
+    }
     if (g.shmem > 48 * 1024) {
         hipError_t e = set_max_dynamic_lds(fn, (size_t)g.shmem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(max dynamic LDS)");
