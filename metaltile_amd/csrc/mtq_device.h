@@ -363,6 +363,38 @@ __device__ __forceinline__ uint32_t csr_slot_expert(const uint32_t* off, uint32_
     }
     return 0xFFFFFFFFu;
 }
+// Both of the above from one read of the offsets, for at most 64 experts (lane e holds off[e + 1]; everything else is
+// exchanged between lanes): which expert this grid row serves (`sel` is the expert, or with by_slot the slot) and its
+// rows. Returns the expert's row count and sets expert (0xFFFFFFFF: a slot past the experts that have rows), lo, n1,
+// lo2 as csr_expert_rows does. One trip to memory instead of three or four ahead of the first activation load.
+__device__ __forceinline__ uint32_t csr_route64(const uint32_t* off, uint32_t E, uint32_t T, uint32_t sel, bool by_slot, uint32_t lane,
+                                                uint32_t& expert, uint32_t& lo, uint32_t& n1, uint32_t& lo2) {
+    const uint32_t o_hi = lane < E ? off[lane + 1] : 0u;
+    uint32_t incl = o_hi;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t up = (uint32_t)__shfl_up((int)incl, d, 64);
+        if (lane >= (uint32_t)d) incl = max(incl, up);
+    }
+    uint32_t before = (uint32_t)__shfl_up((int)incl, 1, 64);   // max(off[1 .. e])
+    if (lane == 0) before = 0;
+    const uint32_t mx = (uint32_t)__shfl((int)incl, 63, 64);
+    lo = n1 = lo2 = 0;
+    expert = sel;
+    if (by_slot) {
+        const bool hit = lane < E && (min(o_hi, T) > min(before, T) || (lane == 0 && min(mx, T) < T));
+        unsigned long long m = __ballot(hit);
+        if (sel >= (uint32_t)__popcll(m)) { expert = 0xFFFFFFFFu; return 0; }
+        for (uint32_t i = 0; i < sel; i++) m &= m - 1ull;
+        expert = (uint32_t)__ffsll((long long)m) - 1u;
+    }
+    const uint32_t l = (uint32_t)__shfl((int)before, (int)expert, 64), oh = (uint32_t)__shfl((int)o_hi, (int)expert, 64);
+    const uint32_t hi = min(oh, T);
+    lo = l;
+    n1 = hi > lo ? hi - lo : 0;
+    lo2 = min(mx, T);
+    return n1 + (expert == 0 ? T - lo2 : 0u);
+}
 // Per-row ids (at most 64 rows): the slot-th smallest id below E that a row names.
 __device__ __forceinline__ uint32_t ids_slot_expert(const uint32_t* ids, uint32_t E, uint32_t T, uint32_t slot, uint32_t lane) {
     uint32_t v = lane < T ? ids[lane] : 0xFFFFFFFFu;

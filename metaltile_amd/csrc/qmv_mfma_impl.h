@@ -221,12 +221,17 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
     uint32_t expert = 0, cnt = a.M, lo = 0, n1 = a.M, lo2 = 0;
     if constexpr (MODE == GATHER_CSR) {
         expert = blockIdx.y;
-        if (a.by_slot) {
-            expert = __builtin_amdgcn_readfirstlane(csr_slot_expert(a.route, a.E, a.T, blockIdx.y, lane));   // (the same in every lane: a scalar)
-            if (expert == NOROW) return;
-        }
         // E(t) = first e with t < off[e+1], else 0 (crates/metaltile-std/src/ffai/moe.rs:376-385)
-        cnt = csr_expert_rows(a.route, a.E, a.T, expert, lane, lo, n1, lo2);
+        if (a.E <= 64u) {
+            cnt = csr_route64(a.route, a.E, a.T, blockIdx.y, a.by_slot != 0u, lane, expert, lo, n1, lo2);
+            expert = __builtin_amdgcn_readfirstlane(expert);   // (the same in every lane: a scalar)
+        } else {
+            if (a.by_slot) {
+                expert = __builtin_amdgcn_readfirstlane(csr_slot_expert(a.route, a.E, a.T, blockIdx.y, lane));
+                if (expert == NOROW) return;
+            }
+            cnt = csr_expert_rows(a.route, a.E, a.T, expert, lane, lo, n1, lo2);
+        }
         if (cnt == 0) return;
     } else if constexpr (MODE == GATHER_INDICES) {
         expert = blockIdx.y;

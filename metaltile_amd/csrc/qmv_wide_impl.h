@@ -132,7 +132,12 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
     uint32_t expert = 0, nrows = a.M, lo = 0, n1 = a.M, lo2 = 0;
     if constexpr (MODE == GATHER_CSR) {
         expert = blockIdx.y;
-        nrows = csr_expert_rows(a.route, a.E, a.T, expert, lane, lo, n1, lo2);
+        if (a.E <= 64u) {
+            uint32_t same;
+            nrows = csr_route64(a.route, a.E, a.T, expert, false, lane, same, lo, n1, lo2);   // (one read of the offsets)
+        } else {
+            nrows = csr_expert_rows(a.route, a.E, a.T, expert, lane, lo, n1, lo2);
+        }
         // (the same in every lane: kept in scalar registers, the vector ones are all spoken for)
         nrows = __builtin_amdgcn_readfirstlane(nrows);
         lo = __builtin_amdgcn_readfirstlane(lo);
