@@ -108,6 +108,7 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
     a.rows_per_wg = best_d * best_nb * rps;
     a.nb = best_nb;
     a.E = p.E;
+    a.T = p.T;
     a.norm_w = norm_w;
     a.eps = eps;
     a.nmat = 0;
@@ -130,7 +131,8 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
     g.sbi = per_thread <= 1 ? 1 : per_thread <= 2 ? 2 : 4;
     g.tpb = tpb;
     g.shmem = (size_t)a.rows_per_wg * gpr * 8 + (size_t)a.rows_per_wg * rows * a.wpr * 4;
-    g.grid = dim3((p.N + a.rows_per_wg - 1) / a.rows_per_wg, batch ? (uint32_t)batch->n : 1u, 1);
+    const bool routed = p.gather == GATHER_CSR || p.gather == GATHER_INDICES;   // a grid row per activation row
+    g.grid = dim3((p.N + a.rows_per_wg - 1) / a.rows_per_wg, batch ? (uint32_t)batch->n : routed ? p.T : 1u, 1);
     if (norm_w) {
         g.shmem += 16 * sizeof(float);  // one partial sum of squares per wave
         switch (p.dtype) {
@@ -196,6 +198,14 @@ int launch_qmv_norm(const QmvParams& p0, const void* norm_w, const float* eps, c
 
 static int launch_qmv_dot2(const QmvParams& p, const LaunchCtx& lc);
 
+// Routed rows the one-row streaming kernel takes: one row (two when the streaming kernel is asked for by option),
+// fewer than the experts, at most 64 experts (the routing is read by one wave-wide load), 4-bit codes.
+static bool qmv_few_routed_rows(const QmvParams& p) {
+    const uint32_t most = options().qmv_kernel == 2 ? 2u : 1u;
+    return (p.gather == GATHER_CSR || p.gather == GATHER_INDICES) && p.T >= 1 && p.T <= most && p.T < p.E && p.E <= 64 && p.bits == 4 &&
+           options().qmv_kernel != 1;
+}
+
 int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {
     // The matrix-core kernel wins as soon as more than one activation row shares
     // the weight stream (and for every gather); a single row is as fast on the
@@ -205,6 +215,13 @@ int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {
                       p.bits == 3 || p.bits == 5 || p.bits == 6;
     const int mode = options().qmv_mfma;
     bool tried_mfma = false;
+    // One routed row: the one-row streaming kernel, each grid row once per row of the expert it finds. 8 experts of
+    // 14336 x 4096, us, matrix-core GEMV -> this: 1 row 14.9 -> 10.6 (the plain one-row launch on one expert: 8.3; the
+    // routing sits ahead of the first weight load); 2 rows on 2 experts 17.6 -> 18.1, so those stay where they were.
+    if (qmv_few_routed_rows(p) && mode != 2) {
+        int rc = launch_qmv_dot2(p, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
     if (mode == 2 || (mode == 0 && many)) {
         int rc = launch_qmv_mfma(p, lc);
         if (rc != ERR_UNSUPPORTED) return rc;
@@ -230,9 +247,10 @@ static int launch_qmv_dot2(const QmvParams& p, const LaunchCtx& lc) {
     if (!is_pow2(G) || G * 2 < cpc || p.K % G) return fail(ERR_UNSUPPORTED, "fast qmv: group size");
     const uint32_t C = p.K / cpc;
     const bool gather = p.gather == GATHER_CSR || p.gather == GATHER_INDICES;
-    const uint32_t rows = gather ? p.T : (p.gather == GATHER_SINGLE ? 1u : p.M);
+    const bool few = qmv_few_routed_rows(p);   // worked one row at a time
+    const uint32_t rows = few ? 1u : gather ? p.T : (p.gather == GATHER_SINGLE ? 1u : p.M);
     if (rows == 0) return ERR_OK;  // nothing to compute
-    const uint32_t maxt = (gather || rows > 1) ? 512u : 1024u;
+    const uint32_t maxt = ((gather && !few) || rows > 1) ? 512u : 1024u;
     if (C > maxt) return fail(ERR_UNSUPPORTED, "fast qmv: row too long for one workgroup");
     if (!(C % 64 == 0 || (C < 64 && is_pow2(C)))) return fail(ERR_UNSUPPORTED, "fast qmv: chunk count");
     if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16) return fail(ERR_UNSUPPORTED, "fast qmv: w and x must be 16-byte aligned");
@@ -262,9 +280,9 @@ static int launch_qmv_dot2(const QmvParams& p, const LaunchCtx& lc) {
         return ERR_OK;
     }
 
-    if (!gather && options().qmv_kernel != 1) {
+    if ((!gather || few) && options().qmv_kernel != 1) {
         int rc = launch_qmv_stream(p, C, rps, tpb, rows, lc);
-        if (rc != ERR_UNSUPPORTED) return rc;
+        if (rc != ERR_UNSUPPORTED || few) return rc;
     }
 
     QmvGeom g;

@@ -336,6 +336,7 @@ struct QmvSArgs {
     uint32_t rows_per_wg;    // multiple of D*rps
     uint32_t nb;             // batches of D rows per thread
     uint32_t E;
+    uint32_t T;              // routed modes: activation rows (fewer than experts; blockIdx.y counts the experts that have rows)
     // Batched launch (several weight matrices against the same activations, blockIdx.y
     // = matrix): per-matrix operands; nmat = 0 for a plain launch.
     uint32_t nmat;
@@ -463,10 +464,34 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
     const uint32_t rows_here = min(a.rows_per_wg, Nm - rb);      // >= 1 by construction of the grid
     const uint32_t k0 = c * CPC;
 
-    uint32_t expert = 0;
+    // Routed rows (one or two rows on at most 64 experts: a decode step of one token through a mixture-of-experts
+    // layer): grid row blockIdx.y serves the blockIdx.y-th expert that has a row and runs the whole kernel once per row
+    // of that expert - one row each when a token's experts are distinct, as top-k routing makes them.
+    constexpr bool ROUTED = MODE == GATHER_CSR || MODE == GATHER_INDICES;
+    uint32_t expert = 0, n_pass = 1, r_lo = 0, r_n1 = 1, r_lo2 = 0;
+    unsigned long long r_mask = 0;
     if constexpr (MODE == GATHER_SINGLE) expert = min(a.route[0], a.E - 1);
+    if constexpr (MODE == GATHER_CSR) {
+        n_pass = csr_route64(a.route, a.E, a.T, blockIdx.y, true, lane, expert, r_lo, r_n1, r_lo2);
+        if (n_pass == 0) return;
+        expert = __builtin_amdgcn_readfirstlane(expert);
+    }
+    if constexpr (MODE == GATHER_INDICES) {
+        expert = __builtin_amdgcn_readfirstlane(ids_slot_expert(a.route, a.E, a.T, blockIdx.y, lane));
+        if (expert == 0xFFFFFFFFu) return;
+        r_mask = __ballot(lane < a.T && a.route[lane] == expert);
+        n_pass = (uint32_t)__popcll(r_mask);
+    }
     const size_t slab_rows = (size_t)expert * Nm;
     const u32x4* wbase = Wm + (slab_rows + rb) * a.C + c;
+    for (uint32_t pass = 0; pass < (ROUTED ? n_pass : 1u); pass++) {
+    uint32_t trow = 0;   // the activation row (and output row) of this pass
+    if constexpr (MODE == GATHER_CSR) trow = pass < r_n1 ? r_lo + pass : r_lo2 + (pass - r_n1);
+    if constexpr (MODE == GATHER_INDICES) {
+        unsigned long long m = r_mask;
+        for (uint32_t i = 0; i < pass; i++) m &= m - 1ull;
+        trow = (uint32_t)__ffsll((long long)m) - 1u;
+    }
 
     // ---- loads, smallest first ----------------------------------------------
     const size_t sb0 = (slab_rows + rb) * a.gpr;
@@ -488,7 +513,7 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
     uint4 xraw[MB][XS::NRAW];
 #pragma unroll
     for (int mb = 0; mb < MBR; mb++) {
-        const uint32_t t = mb < (int)a.M ? mb : 0;
+        const uint32_t t = ROUTED ? trow : (mb < (int)a.M ? mb : 0);
         xs[mb].load_raw(a.x, (size_t)t * a.K + k0, xraw[mb]);
     }
     uint4 nraw[NORM ? XS::NRAW : 1];
@@ -603,8 +628,10 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
         if (mb >= a.M) continue;
         float sum = 0.f;
         for (uint32_t wi = 0; wi < a.wpr; wi++) sum += part[o * a.wpr + wi];
-        store_elem<DT>(Om, (size_t)mb * Nm + rb + rl, sum);
+        store_elem<DT>(Om, (size_t)(ROUTED ? trow : mb) * Nm + rb + rl, sum);
     }
+    if (ROUTED && pass + 1 < n_pass) __syncthreads();   // the next row stages into the same LDS
+    }   // pass
 }
 
 // ---------------------------------------------------------------------------
@@ -738,7 +765,11 @@ template <int DT> int qmv_stream_launch_dtype(QmvSArgs& a, int bits, int mode, c
             default: return qmv_stream_launch_mode<DT, 8, GATHER_NONE>(a, g, lc);
         }
     }
-    if (g.mb != 1) return fail(ERR_UNSUPPORTED, "stream qmv: single-expert mode takes one row");
+    if (g.mb != 1) return fail(ERR_UNSUPPORTED, "stream qmv: the expert modes take one row at a time");
+    if (mode == GATHER_CSR || mode == GATHER_INDICES) {   // (4-bit codes: the width mixture-of-experts weights come in)
+        if (bits != 4) return fail(ERR_UNSUPPORTED, "stream qmv: routed rows take 4-bit codes");
+        return mode == GATHER_CSR ? qmv_stream_launch_mode<DT, 4, GATHER_CSR>(a, g, lc) : qmv_stream_launch_mode<DT, 4, GATHER_INDICES>(a, g, lc);
+    }
     switch (bits) {
         case 2: return qmv_stream_launch_mode<DT, 2, GATHER_SINGLE>(a, g, lc);
         case 4: return qmv_stream_launch_mode<DT, 4, GATHER_SINGLE>(a, g, lc);

@@ -20,15 +20,16 @@ def _offsets(ids, E):
 
 
 @pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
-@pytest.mark.parametrize("E,ids", [(8, [3]), (8, [1, 6]), (8, [0, 7]), (8, [2, 2, 5]), (8, [0, 1, 2, 3, 4, 5, 6]),
+@pytest.mark.parametrize("E,ids", [(8, [3]), (8, [1, 6]), (8, [0, 7]), (8, [4, 4]), (64, [0, 63]), (8, [2, 2, 5]), (8, [0, 1, 2, 3, 4, 5, 6]),
                                    (130, [0, 63, 64, 65, 128, 129]), (130, [129]), (70, [64, 64, 64, 69]),
                                    (40, list(range(4, 36)))],
                          ids=lambda v: str(v) if isinstance(v, int) else "-".join(map(str, v[:6])))
-def test_fewer_rows_than_experts(oracle, dt, E, ids):
-    bits, G, N, K = 4, 64, 264, 1024
+@pytest.mark.parametrize("K", [1024, 2048])
+def test_fewer_rows_than_experts(oracle, dt, E, ids, K):
+    bits, G, N = 4, 64, 264
     T = len(ids)
     idn = np.array(ids, dtype="<u4")
-    c = make_case(8400 + E + T, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
+    c = make_case(8400 + E + T + K, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
     exp = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=idn, f64=True, threads=8)
     exp = oracle.round_through(exp.astype(np.float32), ODT[dt]).reshape(T, N)
     w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
@@ -36,7 +37,9 @@ def test_fewer_rows_than_experts(oracle, dt, E, ids):
     for view, route, fn in (("csr", _offsets(idn, E), ops.gather_qmv_csr), ("indices", idn, ops.gather_qmv_indices)):
         print(f"[case] few-row gather {view} {dt.name} E{E} ids={ids}", flush=True)
         rc, launches, _, n = ops.plan("gather_" + view, dt, bits, G, 1, N, K, E, T)
-        assert rc == 0 and n == 1 and "qmv_mfma_kernel" in launches[0][0] and launches[0][1][1] == T, launches
+        # one row on at most 64 experts: the one-row streaming kernel (rows of whole waves of 16-byte chunks)
+        kernel = "qmv_stream_kernel" if T == 1 and E <= 64 and K >= 2048 else "qmv_mfma_kernel"
+        assert rc == 0 and n == 1 and kernel in launches[0][0] and launches[0][1][1] == T, launches
         out, r = GpuBuffer.from_bytes(b"\xff" * (T * N * dt.size_bytes)), GpuBuffer.from_bytes(route.tobytes())
         fn(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
         got = unpack_f32(out.read_bytes(), dt).reshape(T, N)
@@ -86,4 +89,62 @@ def test_fewer_rows_than_experts_odd_routing(oracle, dt):
     for t in (0, 2, 4):
         assert rel_err(got[t], exp[t]) <= 1e-2
     for buf in (w, s, b, x, out, r):
+        buf.free()
+
+
+@pytest.fixture
+def prefer_streaming():
+    lib = _lib.load()
+    assert lib.mtq_set_option(b"qmv.kernel", 2) == 0
+    yield
+    lib.mtq_set_option(b"qmv.kernel", 0)
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+def test_two_rows_on_the_one_row_kernel(oracle, dt, prefer_streaming):
+    """The one-row streaming kernel serves routed rows one at a time, each grid row once per row of its expert. It is
+    chosen for one row; asked for by option it takes two, which is what runs its second pass: offsets that end short,
+    offsets that step back, an id that names no expert, the same expert for both rows, two experts."""
+    bits, G, N, K, E, T = 4, 64, 132, 2048, 9, 2
+    c = make_case(8600, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+
+    def expect(ids_equiv):
+        e = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=np.array(ids_equiv, dtype="<u4"),
+                              f64=True, threads=8)
+        return oracle.round_through(e.astype(np.float32), ODT[dt]).reshape(T, N)
+
+    #                      e: 0  1  2  3  4  5  6  7  8
+    for off, ids_equiv, label in (([0, 0, 0, 0, 1, 1, 1, 1, 1, 1], [3, 0], "tail to expert 0"),
+                                  ([0, 0, 0, 0, 0, 0, 0, 0, 0, 0], [0, 0], "every row in the tail"),
+                                  ([0, 0, 2, 1, 1, 1, 1, 1, 1, 1], [1, 1], "an offset that steps back"),
+                                  ([0, 0, 1, 1, 1, 1, 1, 2, 2, 2], [1, 6], "two experts"),
+                                  ([0, 0, 0, 0, 0, 0, 0, 0, 0, 2], [8, 8], "both rows on the last expert")):
+        via_offsets = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G,
+                                        expert_offsets=np.array(off, dtype="<u4"), f64=True, threads=8)
+        exp = expect(ids_equiv)
+        assert np.array_equal(oracle.round_through(via_offsets.astype(np.float32), ODT[dt]).reshape(T, N), exp), label
+        print(f"[case] two-row gather csr {dt.name} {label} off={off}", flush=True)
+        _, launches, _, _ = ops.plan("gather_csr", dt, bits, G, 1, N, K, E, T)
+        assert "qmv_stream_kernel" in launches[0][0] and launches[0][1][1] == T, launches
+        out, r = GpuBuffer(T * N * dt.size_bytes), GpuBuffer.from_bytes(np.array(off, dtype="<u4").tobytes())
+        ops.gather_qmv_csr(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+        assert rel_err(unpack_f32(out.read_bytes(), dt), exp.reshape(-1)) <= 1e-2, label
+        out.free(); r.free()
+    rb = N * dt.size_bytes
+    for ids, kept in (([E + 1, 4], 0), ([6, 0xFFFFFFFF], 1), ([5, 5], None), ([7, 2], None)):
+        print(f"[case] two-row gather indices {dt.name} ids={ids}", flush=True)
+        exp = expect([i if i < E else 0 for i in ids])
+        out, r = GpuBuffer.from_bytes(b"\xab" * (T * rb)), GpuBuffer.from_bytes(np.array(ids, dtype="<u4").tobytes())
+        ops.gather_qmv_indices(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+        raw = out.read_bytes()
+        got = unpack_f32(raw, dt).reshape(T, N)
+        for t in range(T):
+            if t == kept:
+                assert raw[t * rb:(t + 1) * rb] == b"\xab" * rb, ids
+            else:
+                assert rel_err(got[t], exp[t]) <= 1e-2, ids
+        out.free(); r.free()
+    for buf in (w, s, b, x):
         buf.free()

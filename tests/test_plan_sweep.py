@@ -145,7 +145,8 @@ def test_benchmark_configurations_are_routed_as_documented():
     for view in ("gather_csr", "gather_indices"):      # fewer rows than experts: a grid row per row, not per expert
         for T, E in ((1, 8), (2, 8), (7, 8), (8, 128), (32, 128)):
             ks, ls = kernels(view, DType.BF16, 4, 64, 1, 14336, 4096, E, T)
-            assert "qmv_mfma_kernel<2, 4," in ks[0] and ls[0][1][1] == T, (view, T, E, ls)
+            kernel = "qmv_stream_kernel<2, 4, 1," if T == 1 and E <= 64 else "qmv_mfma_kernel<2, 4,"   # one row: the one-row kernel
+            assert kernel in ks[0] and ls[0][1][1] == T, (view, T, E, ls)
         ks, ls = kernels(view, DType.BF16, 4, 64, 1, 2048, 768, 128, 33)   # (more than 32 rows: a grid row per expert)
         assert ls[0][1][1] == 128
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 4096, 4096, 8, 2048)
