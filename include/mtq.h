@@ -210,6 +210,21 @@ MTQ_API int mtq_rms_norm_qmv(int dtype, int bits, uint32_t group_size, const voi
                              const void *w, const void *scales, const void *biases, void *out, const float *eps_buf,
                              uint32_t N, uint32_t K);
 
+/* Gated RMSNorm fused into a 4-bit qmv (the tail of a gated-delta-net layer): with y f32 [hv, dv], z T [hv, dv],
+ * norm_weight T [dv], inner[r, d] = y[r, d] * inv_rms[r] * norm_weight[d] * silu(z[r, d]),
+ * inv_rms[r] = 1 / sqrt(mean_d(y[r]^2) + eps_buf[0]), silu(v) = v / (1 + exp(-v)), and
+ * out[n] = sum_i w_hat[n, i] * inner_flat[i] over i = r * dv + d in [0, hv * dv). y is f32 for every dtype;
+ * eps_buf is a DEVICE pointer to one f32. Replaces ffai_gated_rms_norm_qgemv_int4_fast
+ * (crates/metaltile-std/src/ffai/gated_rms_norm_qgemv.rs:88-291), whose invariants (hv * dv % 512 == 0,
+ * N % 8 == 0, group_size 64, dv % 32 == 0, hv even, hv * dv <= 8192) are not required here: any hv, dv >= 1 with
+ * group_size dividing hv * dv. inner is an f32 value as in the reference (never rounded to T); the f16 / bf16 kernels
+ * carry it as a rounded value plus a rounded remainder (16 significant bits). One launch for f16 / bf16 when hv * dv is a
+ * multiple of 2048 (at most 32768) and dv is 32 .. 2048 in powers of two; otherwise inner is written to a library-owned
+ * buffer first (allocated on first use, grown on demand) and an ordinary qmv follows. */
+MTQ_API int mtq_gated_rms_norm_qmv(int dtype, uint32_t group_size, const float *y, const void *z, const void *norm_weight,
+                                   const float *eps_buf, const void *w, const void *scales, const void *biases, void *out,
+                                   uint32_t hv, uint32_t dv, uint32_t N);
+
 /* ---- MoE routing around gather_qmv -------------------------------------------------- */
 
 /* Top-k experts per token row and their softmax weights. logits T[n_rows, n_experts] ->
@@ -397,6 +412,9 @@ MTQ_API int mtq_flush_cache(void);
  *   "qmv.mfma_kp" / "qmv.mfma_rbw" / "qmv.mfma_nrb" / "qmv.mfma_sets"
  *                          matrix-core GEMV geometry: K parts per row, row blocks side by side and one
  *                          after the other per workgroup, 4-row activation sets per pass; 0 = choose
+ *   "qmv.gated_fused"      mtq_gated_rms_norm_qmv as one launch of the streaming kernel (hv * dv a multiple of 2048 up to
+ *                          32768, dv = 32 .. 2048 in powers of two): 0 = for f16 / bf16, 1 = never (the activation is staged
+ *                          in the library's buffer), 2 = wherever the shape allows
  *   "qmv.norm_mfma"        mtq_rms_norm_qmv with the norm applied inside the matrix-core GEMV (4-bit codes, f16 / bf16):
  *                          0 = where it is faster than the streaming kernel's fused form, 1 = never, 2 = wherever the
  *                          shape allows

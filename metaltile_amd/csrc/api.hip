@@ -357,6 +357,49 @@ static int op_qvm(int dtype, int bits, uint32_t G, const void* w, const void* s,
     return launch_qvm(p, g.scratch_buf, lc);
 }
 
+// A qmv whose activation row some first launch writes into library-owned scratch: `stage(dst, ctx)` enqueues
+// that launch (one row of K for f32; for f16 / bf16 two rows, the rounded values and the rounded remainders, so
+// that the row carries 16 significant bits), an ordinary qmv follows, and for two rows the sum of their outputs.
+template <class Stage>
+static int qmv_of_staged_row(int dtype, int bits, uint32_t G, const void* w, const void* s, const void* b, void* out,
+                             uint32_t N, uint32_t K, const LaunchCtx& lc, Stage&& stage) {
+    int rc;
+    // scratch: the normalised row(s), then for 16-bit types the two partial outputs
+    const size_t sz = esize(dtype);
+    const uint32_t rows = dtype == DT_F32 ? 1u : 2u;
+    const size_t x_bytes = ((size_t)rows * K * sz + 255) & ~(size_t)255;
+    const size_t held = (x_bytes + (rows == 2 ? (size_t)2 * N * sz : 0) + 255) & ~(size_t)255;
+    // The qmv that follows may itself want scratch (f32 rows on the tile kernel split K into partial
+    // tiles): size the buffer for both now, so that it is not reallocated under the normalised row, and
+    // let that qmv work behind the held part, so that its partial tiles do not overwrite the row it reads.
+    size_t inner = 0;
+    if (dtype == DT_F32) {
+        QmmParams q;
+        q.dtype = dtype; q.bits = bits; q.group_size = G; q.w = w; q.scales = s; q.biases = b; q.x = g.scratch_buf; q.out = out;
+        q.M = rows; q.N = N; q.K = K;
+        inner = qmm_f32_scratch_bytes(q);
+    }
+    rc = ensure_scratch(held + inner);
+    if (rc) return rc;
+    LaunchCtx first = lc, mid = lc, last = lc;
+    first.stop = nullptr;
+    mid.start = mid.stop = nullptr;
+    last.start = nullptr;
+    rc = stage(g.scratch_buf, first);
+    if (rc) return rc;
+    g.scratch_held = held;
+    if (rows == 1) {
+        rc = op_qmv(dtype, bits, G, w, s, b, g.scratch_buf, out, 1, N, K, last);
+        g.scratch_held = 0;
+        return rc;
+    }
+    char* part = (char*)g.scratch_buf + x_bytes;
+    rc = op_qmv(dtype, bits, G, w, s, b, g.scratch_buf, part, 2, N, K, mid);
+    g.scratch_held = 0;
+    if (rc) return rc;
+    return launch_add_rows(dtype, part, part + (size_t)N * sz, out, N, last);
+}
+
 // RMSNorm fused into qmv: inside the streaming kernel when the row fits it, else the
 // row is normalised into a library-owned buffer and an ordinary qmv follows.
 static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const void* norm_w, const void* w,
@@ -383,40 +426,38 @@ static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const
     }
     rc = launch_qmv_norm(p, norm_w, eps, lc);
     if (rc != ERR_UNSUPPORTED) return rc;
-    // scratch: the normalised row(s), then for 16-bit types the two partial outputs
-    const size_t sz = esize(dtype);
-    const uint32_t rows = dtype == DT_F32 ? 1u : 2u;
-    const size_t x_bytes = ((size_t)rows * K * sz + 255) & ~(size_t)255;
-    const size_t held = (x_bytes + (rows == 2 ? (size_t)2 * N * sz : 0) + 255) & ~(size_t)255;
-    // The qmv that follows may itself want scratch (f32 rows on the tile kernel split K into partial
-    // tiles): size the buffer for both now, so that it is not reallocated under the normalised row, and
-    // let that qmv work behind the held part, so that its partial tiles do not overwrite the row it reads.
-    size_t inner = 0;
-    if (dtype == DT_F32) {
-        QmmParams q;
-        q.dtype = dtype; q.bits = bits; q.group_size = G; q.w = w; q.scales = s; q.biases = b; q.x = x; q.out = out;
-        q.M = rows; q.N = N; q.K = K;
-        inner = qmm_f32_scratch_bytes(q);
+    return qmv_of_staged_row(dtype, bits, G, w, s, b, out, N, K, lc, [&](void* dst, const LaunchCtx& ctx) {
+        return launch_rms_norm(dtype, x, norm_w, eps, dst, K, ctx);
+    });
+}
+
+// Gated RMSNorm + 4-bit qmv (crates/metaltile-std/src/ffai/gated_rms_norm_qgemv.rs:88-291): the gated, normalised
+// rows of y (hv rows of dv, flat: the GEMV's activation of hv * dv) are written into library-owned scratch, an
+// ordinary qmv follows. The reference stages that activation in f32 and never rounds it to the element type;
+// the two-row form of the staged qmv keeps 16 significant bits of it for f16 / bf16.
+static int op_gated_rms_norm_qmv(int dtype, uint32_t G, const float* y, const void* z, const void* norm_w, const float* eps,
+                                 const void* w, const void* s, const void* b, void* out, uint32_t hv, uint32_t dv, uint32_t N,
+                                 const LaunchCtx& lc) {
+    if (hv == 0 || dv == 0) return fail(ERR_SHAPE, "hv and dv must be non-zero");
+    if ((uint64_t)hv * dv > 0xFFFFFFFFull) return fail(ERR_SHAPE, "hv * dv must fit 32 bits");
+    const uint32_t K = hv * dv;
+    int rc = check_common(dtype, 4, G, N, K);
+    if (rc) return rc;
+    if (!y || !z || !norm_w || !eps || !w || !s || !b || !out) return fail(ERR_BAD_ARG, "null buffer");
+    // One launch: the streaming kernel gates and normalises the slice each thread holds. us per call, staged (three
+    // launches; two for f32) -> one launch, dv 128: bf16 hv 16, 2048 rows 7.8 -> 5.6 (the plain qmv of that matrix: 3.3);
+    // hv 32, 1024 rows 10.3 -> 5.6; hv 32, 4096 rows 9.3 -> 8.3; hv 64, 8192 rows 14.3 -> 14.0. f32 stays staged (6.3 -> 6.9,
+    // 7.9 -> 11.5, 16.3 -> 19.3): its one-row streaming kernel is the slower one to begin with.
+    if (options().qmv_gated_fused == 2 || (options().qmv_gated_fused == 0 && dtype != DT_F32)) {
+        QmvParams p;
+        p.dtype = dtype; p.bits = 4; p.group_size = G; p.w = w; p.scales = s; p.biases = b; p.x = y; p.out = out;
+        p.N = N; p.K = K;
+        rc = launch_qmv_gated_norm(p, z, norm_w, eps, dv, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
     }
-    rc = ensure_scratch(held + inner);
-    if (rc) return rc;
-    LaunchCtx first = lc, mid = lc, last = lc;
-    first.stop = nullptr;
-    mid.start = mid.stop = nullptr;
-    last.start = nullptr;
-    rc = launch_rms_norm(dtype, x, norm_w, eps, g.scratch_buf, K, first);
-    if (rc) return rc;
-    g.scratch_held = held;
-    if (rows == 1) {
-        rc = op_qmv(dtype, bits, G, w, s, b, g.scratch_buf, out, 1, N, K, last);
-        g.scratch_held = 0;
-        return rc;
-    }
-    char* part = (char*)g.scratch_buf + x_bytes;
-    rc = op_qmv(dtype, bits, G, w, s, b, g.scratch_buf, part, 2, N, K, mid);
-    g.scratch_held = 0;
-    if (rc) return rc;
-    return launch_add_rows(dtype, part, part + (size_t)N * sz, out, N, last);
+    return qmv_of_staged_row(dtype, 4, G, w, s, b, out, N, K, lc, [&](void* dst, const LaunchCtx& ctx) {
+        return launch_gated_rms_norm(dtype, y, z, norm_w, eps, dst, hv, dv, ctx);
+    });
 }
 
 // Fused projections: one launch when the shape fits the streaming kernel, else one qmv per matrix.
@@ -517,7 +558,7 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
 // name-keyed dispatch table
 // ---------------------------------------------------------------------------
 
-enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_NORMQ, F_ROUTER, F_PERMUTE, F_UNPERMUTE, F_MOEDOWN, F_QVM, F_QVM_FAST };
+enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_NORMQ, F_GNORMQ, F_ROUTER, F_PERMUTE, F_UNPERMUTE, F_MOEDOWN, F_QVM, F_QVM_FAST };
 
 struct KernelDesc {
     const char* name;
@@ -577,6 +618,8 @@ static const KernelDesc kTable[] = {
     // x, norm_weight, weight, scales, biases, output, eps_buf | in_dim, group_size
     {"ffai_rms_norm_qgemv", F_NORMQ, 4, 7, 2}, {"ffai_rms_norm_qgemv_fast", F_NORMQ, 4, 7, 2},
     {"ffai_rms_norm_qgemv_int8_fast", F_NORMQ, 8, 7, 2},
+    // y (f32), z, norm_weight, eps_buf, q_weight, q_scales, q_biases, out | hv, dv, out_dim, group_size
+    {"ffai_gated_rms_norm_qgemv_int4_fast", F_GNORMQ, 4, 8, 4},
     // router_logits, indices_out, weights_out | n_experts, k, norm_topk_prob
     {"mt_moe_router_topk", F_ROUTER, 0, 3, 3},
     // tokens, sort_token_idx, permuted | hidden
@@ -814,6 +857,23 @@ static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, in
             MTQ_NEED(bufs[6], "eps_buf", 4);
             return op_rms_norm_qmv(dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, bufs[4].ptr,
                                    bufs[5].ptr, (const float*)bufs[6].ptr, N, K, lc);
+        }
+        case F_GNORMQ: {
+            const uint32_t hv = consts[0], dv = consts[1], N = consts[2], G = consts[3];
+            const uint64_t K = (uint64_t)hv * dv;
+            if (K == 0 || N == 0) return fail(ERR_SHAPE, "hv, dv and out_dim must be non-zero");
+            if (K > 0xFFFFFFFFull) return fail(ERR_SHAPE, "hv * dv must fit 32 bits");
+            if (G == 0 || K % G) return fail(ERR_SHAPE, "group_size must divide hv * dv");
+            MTQ_NEED(bufs[0], "y", K * 4);   // f32 whatever the element type
+            MTQ_NEED(bufs[1], "z", K * sz);
+            MTQ_NEED(bufs[2], "norm_weight", (uint64_t)dv * sz);
+            MTQ_NEED(bufs[3], "eps_buf", 4);
+            MTQ_NEED(bufs[4], "q_weight", (uint64_t)N * K / 2);
+            MTQ_NEED(bufs[5], "q_scales", (uint64_t)N * (K / G) * sz);
+            MTQ_NEED(bufs[6], "q_biases", (uint64_t)N * (K / G) * sz);
+            MTQ_NEED(bufs[7], "out", (uint64_t)N * sz);
+            return op_gated_rms_norm_qmv(dtype, G, (const float*)bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, (const float*)bufs[3].ptr,
+                                         bufs[4].ptr, bufs[5].ptr, bufs[6].ptr, bufs[7].ptr, hv, dv, N, lc);
         }
         case F_BQKV:
         case F_B4: {
@@ -1105,6 +1165,14 @@ int mtq_qmv_batched(int dtype, int bits, uint32_t group_size, int n_mats, const 
     int rc = need_ready();
     if (rc) return rc;
     return op_qmv_batched(dtype, bits, group_size, n_mats, w, scales, biases, x, outs, N, K, make_ctx());
+}
+
+int mtq_gated_rms_norm_qmv(int dtype, uint32_t group_size, const float* y, const void* z, const void* norm_weight,
+                           const float* eps_buf, const void* w, const void* scales, const void* biases, void* out, uint32_t hv,
+                           uint32_t dv, uint32_t N) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return op_gated_rms_norm_qmv(dtype, group_size, y, z, norm_weight, eps_buf, w, scales, biases, out, hv, dv, N, make_ctx());
 }
 
 int mtq_rms_norm_qmv(int dtype, int bits, uint32_t group_size, const void* x, const void* norm_weight, const void* w,
@@ -1448,6 +1516,11 @@ int mtq_set_option(const char* name, int value) {
     if (!strcmp(name, "qmv.mfma")) {
         if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmv.mfma must be 0 (auto), 1 (off) or 2 (prefer)");
         options().qmv_mfma = value;
+        return MTQ_OK;
+    }
+    if (!strcmp(name, "qmv.gated_fused")) {
+        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmv.gated_fused must be 0 (choose), 1 (never) or 2 (wherever the shape allows)");
+        options().qmv_gated_fused = value;
         return MTQ_OK;
     }
     if (!strcmp(name, "qmv.norm_mfma")) {

@@ -113,6 +113,7 @@ struct Options {
     int qmv_mfma_rbw = 0;         // matrix-core qmv: row blocks walked in parallel per workgroup
     int qmv_mfma_nrb = 0;         // matrix-core qmv: row blocks per wave
     int qmv_mfma_sets = 0;        // matrix-core gather: 4-row MFMA sets per pass (0 = choose; 1, 2, 4)
+    int qmv_gated_fused = 0;      // gated RMS norm inside the streaming kernel: 0 = choose, 1 = never (stage the row), 2 = wherever the shape allows
     int qmv_norm_mfma = 0;        // RMS norm fused into the matrix-core GEMV (4-bit f16 / bf16): 0 = choose, 1 = never, 2 = wherever the shape allows
     int qmv_wide_kp = 0;          // 16-row matrix-core GEMV: waves sharing a row block (0 = choose; 1, 2, 4, 8, 16)
     int qmv_wide_nb = 0;          // 16-row matrix-core GEMV: row blocks per wave (0 = choose; 1, 2)
@@ -130,9 +131,13 @@ int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc);
 // RMSNorm of the activation row fused into the streaming qmv (eps: device f32).
 // ERR_UNSUPPORTED when the shape does not fit: the caller normalises into scratch first.
 int launch_qmv_norm(const QmvParams& p, const void* norm_w, const float* eps, const LaunchCtx& lc);
+int launch_qmv_gated_norm(const QmvParams& p, const void* gate_z, const void* norm_w, const float* eps, uint32_t dv,
+                          const LaunchCtx& lc);
 // Standalone x'[k] = x[k] * norm_w[k] * rsqrt(mean(x^2) + eps): one f32 row, or for f16 / bf16
 // two rows of K elements (rounded value, rounded remainder).
 int launch_rms_norm(int dtype, const void* x, const void* norm_w, const float* eps, void* out, uint32_t K, const LaunchCtx& lc);
+int launch_gated_rms_norm(int dtype, const float* y, const void* z, const void* norm_w, const float* eps, void* out,
+                          uint32_t hv, uint32_t dv, const LaunchCtx& lc);
 // MoE routing (moe.hip)
 int launch_moe_router_topk(int dtype, const void* logits, uint32_t* indices, void* weights, uint32_t n_rows,
                            uint32_t n_experts, uint32_t k, uint32_t norm_topk_prob, const LaunchCtx& lc);

@@ -39,7 +39,8 @@ static int num_cus() {
 // shape is better served by the one-shot kernel.
 static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint32_t tpb, uint32_t rows,
                              const LaunchCtx& lc, const QmvBatch* batch = nullptr,
-                             const void* norm_w = nullptr, const float* eps = nullptr) {
+                             const void* norm_w = nullptr, const float* eps = nullptr, const void* gate_z = nullptr,
+                             uint32_t dv = 0) {
     const uint32_t G = p.group_size, gpr = p.K / G;
     if (C % 64 || gpr % 4 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)
         return fail(ERR_UNSUPPORTED, "stream qmv: geometry");
@@ -111,6 +112,8 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
     a.T = p.T;
     a.norm_w = norm_w;
     a.eps = eps;
+    a.gate_z = gate_z;
+    a.dv = dv;
     a.nmat = 0;
     if (batch) {
         a.nmat = (uint32_t)batch->n;
@@ -194,6 +197,28 @@ int launch_qmv_norm(const QmvParams& p0, const void* norm_w, const float* eps, c
     uint32_t rps = 1;
     while (C * rps < 256 && C * rps * 2 <= 1024) rps *= 2;
     return launch_qmv_stream(p, C, rps, C * rps, 1, lc, nullptr, norm_w, eps);
+}
+
+// The gated form of the fused norm (4-bit codes): p.x is the f32 activation y [hv, dv], K = hv * dv. A thread's chunk of
+// 32 values must lie within one row of dv, and the dv / 32 threads of a row must be neighbours within a wave.
+int launch_qmv_gated_norm(const QmvParams& p0, const void* gate_z, const void* norm_w, const float* eps, uint32_t dv,
+                          const LaunchCtx& lc) {
+    QmvParams p = p0;
+    p.gather = GATHER_NONE;
+    p.M = 1;
+    p.bits = 4;
+    const uint32_t cpc = 32;
+    if (p.K == 0 || p.N == 0 || dv == 0 || p.K % dv || dv % cpc || !is_pow2(dv / cpc) || dv / cpc > 64)
+        return fail(ERR_UNSUPPORTED, "gated norm + qmv: dv must be 32 times a power of two up to 2048");
+    const uint32_t G = p.group_size;
+    if (!is_pow2(G) || G * 2 < cpc || p.K % G) return fail(ERR_UNSUPPORTED, "gated norm + qmv: group size");
+    const uint32_t C = p.K / cpc;
+    if (C > 1024 || C % 64) return fail(ERR_UNSUPPORTED, "gated norm + qmv: row geometry");
+    if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)norm_w % 16 || (uintptr_t)gate_z % 16)
+        return fail(ERR_UNSUPPORTED, "gated norm + qmv: w, y, z and norm_weight must be 16-byte aligned");
+    uint32_t rps = 1;
+    while (C * rps < 256 && C * rps * 2 <= 1024) rps *= 2;
+    return launch_qmv_stream(p, C, rps, C * rps, 1, lc, nullptr, norm_w, eps, gate_z, dv);
 }
 
 static int launch_qmv_dot2(const QmvParams& p, const LaunchCtx& lc);

@@ -348,6 +348,9 @@ struct QmvSArgs {
     // Fused RMSNorm (NORM kernels): per-element norm weights T[K] and a device f32 holding eps.
     const void* norm_w;
     const float* eps;
+    // Fused gated RMSNorm (NORM = 2): x is f32 [K / dv, dv] whatever the element type, gate_z T[K], norm_w T[dv].
+    const void* gate_z;
+    uint32_t dv;
 };
 
 typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
@@ -395,7 +398,7 @@ template <int DT> __device__ __forceinline__ float raw_sumsq(uint4 v) {
     return s;
 }
 // (x * w) * inv of one vector, as the element-type value `hi` nearest to it and (16-bit
-// types) the rounded remainder `lo`: hi + lo carries 16 significant bits of the f32 product.
+// types) the rounded, scaled remainder `lo` (RemSplit): hi + lo / kRemScale carries 16 significant bits of the f32 product.
 template <int DT> __device__ __forceinline__ void raw_normed(uint4 xv, uint4 wv, float inv, uint4& hi, uint4& lo) {
     const uint32_t x[4] = {xv.x, xv.y, xv.z, xv.w};
     const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
@@ -409,9 +412,46 @@ template <int DT> __device__ __forceinline__ void raw_normed(uint4 xv, uint4 wv,
             auto up = [](uint32_t b) { return DT == DT_BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b); };
             const float v0 = up(x[j] & 0xFFFFu) * up(w[j] & 0xFFFFu) * inv;
             const float v1 = up(x[j] >> 16) * up(w[j] >> 16) * inv;
-            const uint32_t h0 = f32_to_elem_bits<DT>(v0), h1 = f32_to_elem_bits<DT>(v1);
+            uint32_t h0, h1, l0, l1;
+            RemSplit<DT>::split(v0, h0, l0);
+            RemSplit<DT>::split(v1, h1, l1);
             h[j] = h0 | (h1 << 16);
-            l[j] = (uint32_t)f32_to_elem_bits<DT>(v0 - up(h0)) | ((uint32_t)f32_to_elem_bits<DT>(v1 - up(h1)) << 16);
+            l[j] = l0 | (l1 << 16);
+        }
+    }
+    hi = make_uint4(h[0], h[1], h[2], h[3]);
+    lo = make_uint4(l[0], l[1], l[2], l[3]);
+}
+
+// One vector of the gated, normalised activation: element e = y[e] * inv * w[e] * silu(z[e]) in f32
+// (crates/metaltile-std/src/ffai/gated_rms_norm_qgemv.rs:138-149), y in f32 (two vectors of 4 for a 16-bit vector of
+// 8, one for an f32 vector of 4), z and w of the element type; split into `hi` and `lo` as in raw_normed.
+template <int DT> __device__ __forceinline__ void raw_gated(const uint4* yv, uint4 zv, uint4 wv, float inv, uint4& hi, uint4& lo) {
+    const uint32_t z[4] = {zv.x, zv.y, zv.z, zv.w};
+    const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
+    // (the hardware's exponential and reciprocal, about 1 ulp each: a full-precision quotient is a dozen instructions per
+    // element, and every workgroup gates its whole slice before its first dot product)
+    auto gated = [&](float y, float zf, float wf) { return y * inv * wf * (zf * __builtin_amdgcn_rcpf(1.0f + __expf(0.0f - zf))); };
+    uint32_t h[4], l[4];
+    if constexpr (DT == DT_F32) {
+        const uint32_t y[4] = {yv[0].x, yv[0].y, yv[0].z, yv[0].w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            h[j] = __float_as_uint(gated(__uint_as_float(y[j]), __uint_as_float(z[j]), __uint_as_float(w[j])));
+            l[j] = 0;
+        }
+    } else {
+        const uint32_t y[8] = {yv[0].x, yv[0].y, yv[0].z, yv[0].w, yv[1].x, yv[1].y, yv[1].z, yv[1].w};
+        auto up = [](uint32_t b) { return DT == DT_BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b); };
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float v0 = gated(__uint_as_float(y[2 * j]), up(z[j] & 0xFFFFu), up(w[j] & 0xFFFFu));
+            const float v1 = gated(__uint_as_float(y[2 * j + 1]), up(z[j] >> 16), up(w[j] >> 16));
+            uint32_t h0, h1, l0, l1;
+            RemSplit<DT>::split(v0, h0, l0);
+            RemSplit<DT>::split(v1, h1, l1);
+            h[j] = h0 | (h1 << 16);
+            l[j] = l0 | (l1 << 16);
         }
     }
     hi = make_uint4(h[0], h[1], h[2], h[3]);
@@ -423,7 +463,11 @@ template <int DT> __device__ __forceinline__ void raw_normed(uint4 xv, uint4 wv,
 // every workgroup recomputing the row's sum of squares from the slice its threads hold.
 // The dot2 path takes 16-bit operands: for f16 / bf16 the f32 x' is carried as two rows,
 // its rounded value and the rounded remainder (MB = 2), whose dots are added.
-template <int DT, int BITS, int MB, int D, int MODE, int MAXT, int SBI, bool NORM = false>
+// NORM = 2: the gated form (crates/metaltile-std/src/ffai/gated_rms_norm_qgemv.rs:120-151). The activation is hv rows
+// of dv f32 values y, each row normalised by its own sum of squares and gated by silu(z): a thread's chunk lies within
+// one such row (dv a multiple of the chunk), the row's dv / CPC threads are neighbours in a wave, so the sum of squares
+// is a segmented lane reduction and needs no LDS.
+template <int DT, int BITS, int MB, int D, int MODE, int MAXT, int SBI, int NORM = 0>
 __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
     static_assert(!NORM || (MB == (DT == DT_F32 ? 1 : 2) && MODE == GATHER_NONE), "the fused norm takes one plain activation row");
     constexpr int MBR = NORM ? 1 : MB;  // activation rows as the caller sees them
@@ -511,10 +555,18 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
     MTQ_KEEP_LOAD_ORDER();
     XS xs[MB];
     uint4 xraw[MB][XS::NRAW];
+    uint4 yraw[NORM == 2 ? CPC / 4 : 1];
+    if constexpr (NORM == 2) {
+        const uint4* yp = (const uint4*)((const float*)a.x + k0);
 #pragma unroll
-    for (int mb = 0; mb < MBR; mb++) {
-        const uint32_t t = ROUTED ? trow : (mb < (int)a.M ? mb : 0);
-        xs[mb].load_raw(a.x, (size_t)t * a.K + k0, xraw[mb]);
+        for (int i = 0; i < CPC / 4; i++) yraw[i] = yp[i];
+        xs[0].load_raw(a.gate_z, k0, xraw[0]);
+    } else {
+#pragma unroll
+        for (int mb = 0; mb < MBR; mb++) {
+            const uint32_t t = ROUTED ? trow : (mb < (int)a.M ? mb : 0);
+            xs[mb].load_raw(a.x, (size_t)t * a.K + k0, xraw[mb]);
+        }
     }
     uint4 nraw[NORM ? XS::NRAW : 1];
     float eps = 0.f;
@@ -522,7 +574,7 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
         // issued ahead of the weight stream: loads return in order, so a late load of eps
         // would wait for the whole first ring
         eps = a.eps[0];
-        xs[0].load_raw(a.norm_w, k0, nraw);
+        xs[0].load_raw(a.norm_w, NORM == 2 ? k0 % a.dv : k0, nraw);
     }
     MTQ_KEEP_LOAD_ORDER();
     u32x4 ring[D];
@@ -546,7 +598,22 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
             dst[1] = make_float4(sv[2], bv[2] - MAGIC * sv[2], sv[3], bv[3] - MAGIC * sv[3]);
         }
     }
-    if constexpr (NORM) {
+    if constexpr (NORM == 2) {
+        float ssq = 0.f;
+#pragma unroll
+        for (int i = 0; i < CPC / 4; i++) ssq += raw_sumsq<DT_F32>(yraw[i]);
+        ssq = seg_allreduce(ssq, (int)(a.dv / CPC));
+        const float inv = 1.0f / sqrtf(ssq / (float)a.dv + eps);
+        constexpr int YPV = (CPC / 4) / XS::NRAW;   // y vectors per vector of the element type
+#pragma unroll
+        for (int i = 0; i < XS::NRAW; i++) {
+            uint4 hi, lo;
+            raw_gated<DT>(&yraw[i * YPV], xraw[0][i], nraw[i], inv, hi, lo);
+            xraw[0][i] = hi;
+            if constexpr (MB == 2) xraw[1][i] = lo;
+        }
+    }
+    if constexpr (NORM == 1) {
         // threads of the first row slot hold the whole activation row between them
         float ssq = 0.f;
         if (rsub == 0) {
@@ -557,7 +624,7 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
         if (lane == 0) ssq_part[tid >> 6] = ssq;
     }
     __syncthreads();
-    if constexpr (NORM) {
+    if constexpr (NORM == 1) {
         float tot = 0.f;
         for (uint32_t wv = 0; wv < (TPB >> 6); wv++) tot += ssq_part[wv];
         const float inv = 1.0f / sqrtf(tot / (float)a.K + eps);
@@ -597,7 +664,7 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
                 v += p1.x * d23 + p1.y * xs[mb].xsum[1];
                 acc[d][mb] = v;
             }
-            if constexpr (NORM && MB == 2) acc[d][0] += acc[d][1];
+            if constexpr (NORM != 0 && MB == 2) acc[d][0] += acc[d][1] * (1.0f / RemSplit<DT>::kRemScale);
             if constexpr (decltype(issue_next)::value) {
                 const uint32_t rn = min((j + D) * a.rps + rsub, rows_here - 1);
                 ring[d] = __builtin_nontemporal_load(wbase + (size_t)rn * a.C);
@@ -713,15 +780,15 @@ static int qmv_stream_launch_sbi(QmvSArgs& a, const QmvSGeom& g, const LaunchCtx
     return ERR_OK;
 }
 
-// Fused-RMSNorm instances: one activation row, 4- or 8-bit codes.
-template <int DT, int BITS, int D>
+// Fused-RMSNorm instances: one activation row, 4- or 8-bit codes (NORMK = 1); the gated form, 4-bit codes (NORMK = 2).
+template <int DT, int BITS, int D, int NORMK = 1>
 static int qmv_stream_norm_launch_d(QmvSArgs& a, const QmvSGeom& g, const LaunchCtx& lc) {
     constexpr int MBN = DT == DT_F32 ? 1 : 2;  // 16-bit types carry the normalised row as value + remainder
     const void* fn;
     switch (g.sbi) {
-        case 1: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 1, true>; break;
-        case 2: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 2, true>; break;
-        default: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 4, true>; break;
+        case 1: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 1, NORMK>; break;
+        case 2: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 2, NORMK>; break;
+        default: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 4, NORMK>; break;
     }
     if (g.shmem > 48 * 1024) {
         hipError_t e = set_max_dynamic_lds(fn, (size_t)g.shmem);
@@ -735,6 +802,10 @@ static int qmv_stream_norm_launch_d(QmvSArgs& a, const QmvSGeom& g, const Launch
 
 template <int DT> int qmv_stream_norm_launch_dtype(QmvSArgs& a, int bits, const QmvSGeom& g, const LaunchCtx& lc) {
     if (g.mb != 1 || (g.d != 4 && g.d != 8)) return fail(ERR_UNSUPPORTED, "norm + qmv: no kernel instance for this geometry");
+    if (a.gate_z) {
+        if (bits != 4 || g.d != 4) return fail(ERR_UNSUPPORTED, "gated norm + qmv: 4-bit codes, ring of four");
+        return qmv_stream_norm_launch_d<DT, 4, 4, 2>(a, g, lc);
+    }
     if (bits == 4) return g.d == 4 ? qmv_stream_norm_launch_d<DT, 4, 4>(a, g, lc) : qmv_stream_norm_launch_d<DT, 4, 8>(a, g, lc);
     if (bits == 8) return g.d == 4 ? qmv_stream_norm_launch_d<DT, 8, 4>(a, g, lc) : qmv_stream_norm_launch_d<DT, 8, 8>(a, g, lc);
     return fail(ERR_UNSUPPORTED, "norm + qmv: 4- or 8-bit codes");

@@ -419,9 +419,9 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                         const float xf = DT == DT_BF16 ? bf16_bits_to_f32(xb) : f16_bits_to_f32(xb);
                         const float wf = DT == DT_BF16 ? bf16_bits_to_f32(wb) : f16_bits_to_f32(wb);
                         const float xn = (xf * wf) * inv_rms;
-                        const uint32_t hb = f32_to_elem_bits<DT>(xn);
-                        const float hf = DT == DT_BF16 ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb);
-                        o2[h] = i == 0 ? hb : (uint32_t)f32_to_elem_bits<DT>(xn - hf);
+                        uint32_t hb, lb;
+                        RemSplit<DT>::split(xn, hb, lb);   // (the f16 remainder scaled into the normal range)
+                        o2[h] = i == 0 ? hb : lb;
                     }
                     raw[j] = o2[0] | (o2[1] << 16);
                 }
@@ -618,7 +618,8 @@ __global__ __launch_bounds__(MAXT) void qmv_mfma_kernel(QmvMArgs a) {
                 const uint32_t row = row0 + rl;
                 if (row >= a.N) continue;
                 float v = 0.f;
-                for (uint32_t k2 = 0; k2 < a.KP; k2++) v += RED[((size_t)k2 * rows_wg + rl) * R] + RED[((size_t)k2 * rows_wg + rl) * R + 1];
+                for (uint32_t k2 = 0; k2 < a.KP; k2++)
+                    v += RED[((size_t)k2 * rows_wg + rl) * R] + RED[((size_t)k2 * rows_wg + rl) * R + 1] * (1.0f / RemSplit<DT>::kRemScale);
                 store_elem<DT>(a.out, row, v);
             }
             return;

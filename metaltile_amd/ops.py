@@ -73,6 +73,14 @@ def rms_norm_qmv(dtype, bits, group_size, x, norm_weight, w, scales, biases, out
                                     _p(out), _p(eps_buf), N, K))
 
 
+def gated_rms_norm_qmv(dtype, group_size, y, z, norm_weight, eps_buf, w, scales, biases, out, hv, dv, N):
+    """out = qmv(w_hat, flat(rms_norm(y[r]) * norm_weight * silu(z[r]) for r in range(hv))), 4-bit codes; y is f32
+    [hv, dv] for every dtype, eps_buf a device buffer holding one f32."""
+    lib = _ensure_init()
+    _lib.check(lib.mtq_gated_rms_norm_qmv(int(dtype), group_size, _p(y), _p(z), _p(norm_weight), _p(eps_buf), _p(w), _p(scales),
+                                          _p(biases), _p(out), hv, dv, N))
+
+
 def moe_router_topk(dtype, router_logits, indices_out, weights_out, n_rows, n_experts, k, norm_topk_prob=1):
     lib = _ensure_init()
     _lib.check(lib.mtq_moe_router_topk(int(dtype), _p(router_logits), _p(indices_out), _p(weights_out), n_rows, n_experts, k,

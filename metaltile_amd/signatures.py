@@ -6,7 +6,7 @@ out / output, crates/metaltile-macros/src/legacy/sig_parser.rs:43-48,85).
 Sources: crates/metaltile-std/src/mlx/quantized.rs:8-16, 343-352, 4273-4285;
 ffai/dequant_gemv.rs:52-62; ffai/dequant_gemv_expert_indexed.rs:58-68;
 ffai/moe.rs:358-370, 2256-2268; mlx/quantized.rs:3575-3581, 3629-3635 (affine
-quantise / dequantise).
+quantise / dequantise); ffai/gated_rms_norm_qgemv.rs:90-103.
 """
 from __future__ import annotations
 
@@ -73,6 +73,9 @@ _add("ffai_batched_4_qgemv_fast", 4,
      ("out_a", "out_b", "out_c", "out_d", "in_dim", "group_size"), ("a_out", "b_out", "c_out", "d_out"))
 for _n, _b in (("ffai_rms_norm_qgemv", 4), ("ffai_rms_norm_qgemv_fast", 4), ("ffai_rms_norm_qgemv_int8_fast", 8)):
     _add(_n, _b, ("x", "norm_weight", "weight", "scales", "biases", "output", "eps_buf"), ("in_dim", "group_size"), ("output",))
+_add("ffai_gated_rms_norm_qgemv_int4_fast", 4,
+     ("y", "z", "norm_weight", "eps_buf", "q_weight", "q_scales", "q_biases", "out"),
+     ("hv", "dv", "out_dim", "group_size"), ("out",))
 _add("mt_moe_router_topk", 0, ("router_logits", "indices_out", "weights_out"), ("n_experts", "k", "norm_topk_prob"),
      ("indices_out", "weights_out"))
 _add("mt_moe_permute", 0, ("tokens", "sort_token_idx", "permuted"), ("hidden",), ("permuted",))

@@ -27,6 +27,10 @@
  *   rms_norm_qgemv    numpy restatement (dequant matrix @ normalised row), unit norm
  *                     weights with a constant row (inv_rms in closed form), scale
  *                     invariance in x, eps -> large limit.
+ *   gated_rms_norm_qgemv  numpy f64 restatement with the library's logistic function; one row with a constant
+ *                     gate == that gate x the (pinned) rms_norm_qgemv; z = 0 -> zero output; silu(ln 3) = 0.75 ln 3;
+ *                     scaling one row of y leaves the output unchanged at eps = 0 (the sums of squares are per
+ *                     row); norm weights repeat per row (index d, not r * dv + d).
  *   qvm               numpy f64 `x @ dequant(W)` on the [K, N] layout, and qvm(W) == qmv of the
  *                     transposed, repacked matrix.
  *   moe routing       numpy stable argsort + library softmax, the reference tests' tie-break,
@@ -440,6 +444,45 @@ MTQ_ORACLE_API void mtq_oracle_rms_norm_qgemv(const uint32_t *weight, const floa
         double acc64 = 0.0;
         for (size_t d = 0; d < in_dim; d++) {
             float w_real = (float)extract_code(rw, d, bits) * rs[d / group_size] + rb[d / group_size];
+            acc += w_real * nx[d];
+            acc64 += (double)w_real * (double)nx[d];
+        }
+        out[row] = acc;
+        if (out_f64) out_f64[row] = acc64;
+    }
+    free(nx);
+}
+
+/* Fused gated RMSNorm + 4-bit GEMV: inner[r * dv + d] = y[r, d] * inv_rms[r] * norm_weight[d] * silu(z[r, d]) with
+ * inv_rms[r] = 1 / sqrt(sum_d(y[r, d]^2) / dv + eps) and silu(v) = v / (1 + exp(-v)), all in f32 and in that order,
+ * then the f32-sequential dequant dot over in_dim = hv * dv.
+ * Reference: crates/metaltile-std/src/ffai/gated_rms_norm_qgemv.rs:322-366 (CPU form) and :120-151 (kernel).
+ * `inner` (hv * dv floats, may be NULL) receives the gated, normalised activation. When out_f64 is not NULL the dot
+ * is also accumulated in f64 from the same f32 `inner` and f32 weights. */
+MTQ_ORACLE_API void mtq_oracle_gated_rms_norm_qgemv(const uint32_t *weight, const float *scales, const float *biases,
+                                                    const float *y, const float *z, const float *norm_weight, size_t hv,
+                                                    size_t dv, size_t group_size, size_t out_dim, float eps, float *out,
+                                                    double *out_f64, float *inner) {
+    size_t in_dim = hv * dv, wpr = in_dim / 8, ng = in_dim / group_size;
+    float *nx = (float *)malloc(in_dim * sizeof(float));
+    for (size_t r = 0; r < hv; r++) {
+        const float *yr = y + r * dv, *zr = z + r * dv;
+        float ssq = 0.0f;
+        for (size_t d = 0; d < dv; d++) ssq += yr[d] * yr[d];
+        float inv_rms = 1.0f / sqrtf(ssq / (float)dv + eps);
+        for (size_t d = 0; d < dv; d++) {
+            float gate = zr[d] / (1.0f + expf(-zr[d]));
+            nx[r * dv + d] = yr[d] * inv_rms * norm_weight[d] * gate;
+        }
+    }
+    if (inner) memcpy(inner, nx, in_dim * sizeof(float));
+    for (size_t row = 0; row < out_dim; row++) {
+        const uint32_t *rw = weight + row * wpr;
+        const float *rs = scales + row * ng, *rb = biases + row * ng;
+        float acc = 0.0f;
+        double acc64 = 0.0;
+        for (size_t d = 0; d < in_dim; d++) {
+            float w_real = (float)extract_code(rw, d, 4) * rs[d / group_size] + rb[d / group_size];
             acc += w_real * nx[d];
             acc64 += (double)w_real * (double)nx[d];
         }

@@ -185,6 +185,19 @@ def rms_norm_qgemv(w, scales, biases, x, norm_weight, in_dim, group_size, out_di
     return out, out64, normed
 
 
+def gated_rms_norm_qgemv(w, scales, biases, y, z, norm_weight, hv, dv, group_size, out_dim, eps):
+    """4-bit codes; y, z [hv, dv], norm_weight [dv]. Returns (out f32 sequential, out f64-accumulated, the gated,
+    normalised activation f32 [hv * dv])."""
+    w, scales, biases, y, z, norm_weight = _u32(w), _f32(scales), _f32(biases), _f32(y), _f32(z), _f32(norm_weight)
+    assert y.size == hv * dv and z.size == hv * dv and norm_weight.size == dv
+    out = np.empty(out_dim, dtype=np.float32)
+    out64 = np.empty(out_dim, dtype=np.float64)
+    inner = np.empty(hv * dv, dtype=np.float32)
+    lib().mtq_oracle_gated_rms_norm_qgemv(_p(w), _p(scales), _p(biases), _p(y), _p(z), _p(norm_weight), _sz(hv), _sz(dv),
+                                          _sz(group_size), _sz(out_dim), C.c_float(eps), _p(out), _p(out64), _p(inner))
+    return out, out64, inner
+
+
 def qvm(w, scales, biases, x, m, n, k, bits, group_size):
     """W [K, N] packed along N, scales / biases [K/G, N]. Returns (f32 sequential, f64-accumulated), each [m, n]."""
     w, scales, biases, x = _u32(w), _f32(scales), _f32(biases), _f32(x)

@@ -248,6 +248,105 @@ def test_rms_norm_qgemv_against_numpy_and_closed_forms(oracle, bits):
     assert np.max(np.abs(d64 * 1e3 - plain)) < 1e-4 * max(1.0, np.max(np.abs(plain)))
 
 
+def test_gated_rms_norm_qgemv_against_numpy_and_closed_forms(oracle):
+    """Fused gated RMSNorm + 4-bit GEMV (crates/metaltile-std/src/ffai/gated_rms_norm_qgemv.rs:322-366): (a) equals a
+    library matmul of the independently unpacked weight matrix with a numpy-gated, numpy-normalised activation (the
+    gate through the library's logistic function); (b) one row whose gate is the same everywhere is that gate times
+    the pinned RMSNorm GEMV; (c) z = 0 gives zero; (d) silu(ln 3) = 0.75 ln 3; (e) scaling ONE row of y leaves the
+    output unchanged at eps = 0 (a sum of squares over all rows, or a division by hv * dv, breaks this); (f) the norm
+    weights repeat per row (indexing them by r * dv + d instead of d breaks (a) already: they differ along d)."""
+    from scipy.special import expit
+    rng = np.random.default_rng(515)
+    hv, dv, n, g = 4, 96, 12, 64
+    k = hv * dv
+    codes, s, b, _ = _rand_case(rng, n, k, 4, g, 1)
+    w = oracle.pack_codes(codes, 4)
+    y = (rng.standard_normal((hv, dv)) * np.array([0.3, 1.0, 2.5, 7.0])[:, None]).astype(np.float32)
+    z = (1.5 * rng.standard_normal((hv, dv))).astype(np.float32)
+    nw = (1.0 + 0.2 * rng.standard_normal(dv)).astype(np.float32)
+    eps = np.float32(1e-5)
+    out32, out64, inner = oracle.gated_rms_norm_qgemv(w, s, b, y, z, nw, hv, dv, g, n, eps)
+    # (a) numpy in f64 throughout
+    yd, zd, nwd = y.astype(np.float64), z.astype(np.float64), nw.astype(np.float64)
+    inv = 1.0 / np.sqrt(np.mean(yd * yd, axis=1, keepdims=True) + float(eps))
+    ref_inner = (yd * inv * nwd[None, :] * (zd * expit(zd))).reshape(-1)
+    wd = oracle.np_dequant(w, s, b, n, k, 4, g).astype(np.float64).reshape(n, k)
+    ref = wd @ ref_inner
+    assert np.max(np.abs(inner - ref_inner)) < 1e-5 * max(1.0, np.max(np.abs(ref_inner)))
+    assert np.max(np.abs(out64 - ref)) < 1e-4 and np.max(np.abs(out32 - ref)) < 1e-3
+    assert np.max(np.abs(ref)) > 0.3
+    # (b) one row, constant gate: silu(z0) x rms_norm_qgemv
+    z0 = np.float32(0.8)
+    y1 = rng.standard_normal(k).astype(np.float32)
+    nwk = (1.0 + 0.2 * rng.standard_normal(k)).astype(np.float32)
+    _, g64, _ = oracle.gated_rms_norm_qgemv(w, s, b, y1, np.full(k, z0, np.float32), nwk, 1, k, g, n, eps)
+    _, r64, _ = oracle.rms_norm_qgemv(w, s, b, y1, nwk, k, g, n, 4, eps)
+    assert np.max(np.abs(g64 - r64 * float(z0) * float(expit(np.float64(z0))))) < 1e-4
+    # (c) closed gates
+    o32, o64, _ = oracle.gated_rms_norm_qgemv(w, s, b, y, np.zeros_like(z), nw, hv, dv, g, n, eps)
+    assert not o32.any() and not o64.any()
+    # (d) silu(ln 3) = ln 3 / (1 + 1/3)
+    _, _, one = oracle.gated_rms_norm_qgemv(w, s, b, np.ones_like(y), np.full_like(z, np.log(3.0)), np.ones_like(nw), hv, dv, g, n,
+                                            np.float32(0.0))
+    assert np.max(np.abs(one - 0.75 * np.log(3.0))) < 1e-6
+    # (e) per-row scale invariance at eps = 0
+    y4 = y.copy()
+    y4[2] *= 4.0
+    _, a64, _ = oracle.gated_rms_norm_qgemv(w, s, b, y, z, nw, hv, dv, g, n, np.float32(0.0))
+    _, b64, _ = oracle.gated_rms_norm_qgemv(w, s, b, y4, z, nw, hv, dv, g, n, np.float32(0.0))
+    assert np.max(np.abs(a64 - b64)) < 1e-5
+
+
+def _ref_source(n, seed, scale, off):
+    """The deterministic generator of the reference's test (gated_rms_norm_qgemv.rs:308-318): xorshift64 on a u64,
+    ((s % 20000) as f32 / 20000 - 0.5) * scale + off in f32."""
+    out = np.empty(n, dtype=np.float32)
+    s, m = seed, (1 << 64) - 1
+    for i in range(n):
+        s ^= (s << 13) & m
+        s ^= s >> 7
+        s ^= (s << 17) & m
+        out[i] = (np.float32(s % 20000) / np.float32(20000.0) - np.float32(0.5)) * np.float32(scale) + np.float32(off)
+    return out
+
+
+def _ref_quantize_int4_rows(rows, g):
+    """The reference test's per-row quantiser (gated_rms_norm_qgemv.rs:283-305): scale = (max - min) / 15 (1 for a flat
+    group), bias = min, q = round((v - min) / scale) clamped to 0..15, half away from zero."""
+    n, k = rows.shape
+    grp = rows.reshape(n, k // g, g)
+    mn, mx = grp.min(axis=2), grp.max(axis=2)
+    rng_ = mx - mn
+    scale = np.where(np.abs(rng_) < 1e-10, np.float32(1.0), rng_ / np.float32(15.0)).astype(np.float32)
+    t = (grp - mn[:, :, None]) / scale[:, :, None]
+    q = np.clip(np.floor(t + np.float32(0.5)), 0, 15).astype(np.uint8)   # t >= 0: half away from zero == floor(t + 0.5)
+    return q.reshape(n, k), scale.reshape(-1), mn.astype(np.float32).reshape(-1)
+
+
+def test_gated_rms_norm_qgemv_on_the_reference_test_setup(oracle):
+    """The reference's own test (gated_rms_norm_qgemv.rs:372-432: hv 4, dv 128, out_dim 512, g 64, eps 1e-5, inputs from
+    its xorshift generator and its per-row quantiser) holds no numbers, only generators: restated here, with the
+    expectation composed of pieces pinned elsewhere (the gated, normalised activation from numpy, the dot from the
+    pinned plain GEMV oracle), as the reference states the kernel's contract (:62-72)."""
+    from scipy.special import expit
+    hv, dv, n, g = 4, 128, 512, 64
+    k = hv * dv
+    y = _ref_source(k, 0xA1, 2.0, 0.1)
+    z = oracle.round_through(_ref_source(k, 0xD4, 1.5, 0.0), 2)
+    nw = oracle.round_through(_ref_source(dv, 0xB2, 0.4, 1.0), 2)
+    assert abs(float(y.mean()) - 0.1) < 0.05 and 1.9 < float(y.max() - y.min()) <= 2.0   # the generator's range
+    codes, s, b = _ref_quantize_int4_rows(_ref_source(n * k, 0xC3, 3.0, 0.0).reshape(n, k), g)
+    s, b = oracle.round_through(s, 2), oracle.round_through(b, 2)
+    w = oracle.pack_codes(codes, 4)
+    out32, out64, inner = oracle.gated_rms_norm_qgemv(w, s, b, y, z, nw, hv, dv, g, n, np.float32(1e-5))
+    yd, zd = y.astype(np.float64).reshape(hv, dv), z.astype(np.float64).reshape(hv, dv)
+    ref_inner = (yd / np.sqrt(np.mean(yd * yd, axis=1, keepdims=True) + 1e-5) * nw.astype(np.float64)[None, :] * zd * expit(zd)).reshape(-1)
+    assert np.max(np.abs(inner - ref_inner)) < 1e-5
+    plain = oracle.qmm_f64(w, s, b, ref_inner.astype(np.float32), 1, n, k, 4, g).reshape(-1)
+    assert np.max(np.abs(out64 - plain)) < 1e-3 and np.max(np.abs(out32 - plain)) < 5e-3   # the reference's f32 band: 5e-3
+    assert np.max(np.abs(plain)) > 1.0
+
+
 def _np_topk(logits, k, mode):
     """Independent restatement: stable descending argsort + library softmax."""
     from scipy.special import softmax
