@@ -65,20 +65,24 @@ template <int DT> __device__ __forceinline__ uint16_t f32_to_elem_bits(float v) 
 }
 
 // An f32 value carried as two 16-bit operands: `hi`, the element-type value nearest to it, and `lo`, the rounded
-// remainder times kRemScale, so that hi + lo / kRemScale holds 16 significant bits of v. The f16 remainder is scaled by
-// 2^11 (it then has the magnitude of v instead of 2^-11 of it) and an f16 value below the smallest normal goes to the
-// remainder whole: the 16-bit dot instructions do not keep f16 subnormals, while the f32 sums of the same operands
-// (the bias term of the split dot) do, and the two then differ by 1024 x scale x the flushed values.
+// remainder times kRemScale, so that hi + lo / kRemScale holds 16 significant bits of v (the f16 remainder is scaled by
+// 2^11: it then has the magnitude of v and stays a normal number with all its bits where v is small).
+// The value, and each half once converted, pass through an empty asm: every later use must see the same bits. The
+// optimiser otherwise materialises f16(a * b) more than once, with different roundings - contracted into a
+// mixed-precision FMA (one rounding of the exact product) for one use, converted from the rounded f32 product (two
+// roundings) for another. The two differ by one f16 ulp when the f32 product lands on an f16 tie, about once in 8192
+// values; when the dot operand and the f32 sum of the same row (the bias term of the split dot) got different copies,
+// the output was off by 1024 x scale x ulp, the same sign in every output row: 0.11 on the parity metric for one data
+// set in three of the gated norm, nothing for the others.
 template <int DT> struct RemSplit {
     static constexpr float kRemScale = DT == DT_F16 ? 2048.0f : 1.0f;
     static __device__ __forceinline__ float up(uint32_t b) { return DT == DT_BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b); }
     static __device__ __forceinline__ void split(float v, uint32_t& hi, uint32_t& lo) {
-        if constexpr (DT == DT_F16) {
-            hi = fabsf(v) < 6.103515625e-05f ? 0u : (uint32_t)f32_to_elem_bits<DT>(v);
-        } else {
-            hi = f32_to_elem_bits<DT>(v);
-        }
+        asm volatile("" : "+v"(v));
+        hi = f32_to_elem_bits<DT>(v);
+        asm volatile("" : "+v"(hi));
         lo = f32_to_elem_bits<DT>((v - up(hi)) * kRemScale);
+        asm volatile("" : "+v"(lo));
     }
 };
 
