@@ -169,3 +169,21 @@ def test_empty_and_invalid_inputs():
     with pytest.raises(MtqError) as ei:
         ops.qmv(DType.F32, 4, 64, 0, bs, bb, bx, out, 1, 64, 512)              # null pointer
     assert ei.value.code == -2
+
+
+@pytest.mark.parametrize("M,entry", [(1, ops.qmv), (4, ops.qmv), (16, ops.qmv), (64, ops.qmm)], ids=["m1", "m4", "m16", "m64"])
+@pytest.mark.parametrize("scale", [3e-5, 1e-6])
+def test_f16_activations_below_the_smallest_normal(oracle, M, entry, scale):
+    """f16 activations in the subnormal range (|x| < 6.1e-5) count in full, as they do in the reference's f32
+    arithmetic: the split dot adds MAGIC x scale x sum(x) on one side and takes it off on the other, so a kernel that
+    dropped such an operand on one side only would be wrong by two orders of magnitude. Outputs are of the order of
+    the activations, so the bound is relative to the largest expected output: 5e-3 (the f16 rounding of the output
+    itself is 1.4e-3 there)."""
+    dt, N, K, G = DType.F16, 512, 4096, 64
+    print(f"[case] f16 activations x {scale:g}, M={M}", flush=True)
+    c = make_case(9, dt, 4, G, M, N, K, bias_rule="midpoint")
+    x = oracle.round_through((c.x_f * np.float32(scale)).astype(np.float32), 1)
+    assert np.count_nonzero(np.abs(x) < 6.1e-5) > x.size // 2 and np.count_nonzero(x) > x.size // 2
+    exp = oracle.qmm_f64(c.w, c.scales_f, c.biases_f, x, M, N, K, 4, G).reshape(-1)
+    got = _run(dt, 4, G, c.w, c.scales_f, c.biases_f, x, M, N, K, entry=entry)
+    assert np.max(np.abs(got - exp)) <= 5e-3 * np.max(np.abs(exp))
