@@ -199,6 +199,18 @@ MTQ_API int mtq_qmv_batched(int dtype, int bits, uint32_t group_size, int n_mats
                             const void *const *scales, const void *const *biases, const void *x,
                             void *const *outs, const uint32_t *N, uint32_t K);
 
+/* The same over M activation rows (a prefill step's Q / K / V or four projections): x T[M, K], outs[j] T[M, N[j]],
+ * row m of every output the GEMV of activation row m, 1..4 matrices. Replaces ffai_batched_qkv_qmm_fast
+ * (crates/metaltile-std/src/ffai/batched_qkv_qmm.rs:49-68) and ffai_batched_4_qmm_fast
+ * (crates/metaltile-std/src/ffai/batched_4_qmm.rs:61-85), whose row count is the grid's second dimension (under those
+ * names here: the rows `x` holds) and whose constraints (K % 512 == 0, N % 8 == 0, group 64, 4-bit) are not required.
+ * One mtq_qmm per matrix, in order, with mtq_qmm's routing and arithmetic: outputs are bit-equal to single calls.
+ * Dispatched under the reference names the matrices run on the qmv family at every M, which keeps those kernels'
+ * exact-dequant arithmetic (as the `mt_qmm*` names do). w / scales / biases / outs / N are HOST arrays of device pointers / row counts. */
+MTQ_API int mtq_qmm_batched(int dtype, int bits, uint32_t group_size, int n_mats, const void *const *w,
+                            const void *const *scales, const void *const *biases, const void *x,
+                            void *const *outs, const uint32_t *N, uint32_t M, uint32_t K);
+
 /* RMSNorm fused into qmv: out[n] = sum_k w_hat[n,k] * (x[k] * norm_weight[k] * inv_rms),
  * inv_rms = 1 / sqrt(mean(x^2) + eps_buf[0]); eps_buf is a DEVICE pointer to one f32, as in the
  * reference. Replaces ffai_rms_norm_qgemv / _fast (4-bit) and ffai_rms_norm_qgemv_int8_fast

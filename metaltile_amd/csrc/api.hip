@@ -489,6 +489,35 @@ static int op_qmv_batched(int dtype, int bits, uint32_t G, int n, const void* co
     return ERR_OK;
 }
 
+// Several weight matrices against the same M activation rows (the prefill siblings of the batched GEMV,
+// crates/metaltile-std/src/ffai/batched_qkv_qmm.rs:49-68, batched_4_qmm.rs:61-85): row m of every output is the
+// GEMV of activation row m. One qmm per matrix, in order on the caller's stream; at prefill sizes a launch is
+// long against its fixed cost, so one grid over all the matrices would buy nothing.
+static int op_qmm_batched(int dtype, int bits, uint32_t G, int n, const void* const* w, const void* const* s,
+                          const void* const* b, const void* x, void* const* outs, const uint32_t* N, uint32_t M, uint32_t K,
+                          bool exact, const LaunchCtx& lc) {
+    if (n < 1 || n > 4 || !w || !s || !b || !outs || !N) return fail(ERR_BAD_ARG, "batched qmm: 1..4 matrices, non-null arrays");
+    for (int j = 0; j < n; j++) {
+        int rc = check_common(dtype, bits, G, N[j], K);
+        if (rc) return rc;
+    }
+    if (M == 0) return ERR_OK;
+    if (!x) return fail(ERR_BAD_ARG, "null buffer");
+    for (int j = 0; j < n; j++)
+        if (!w[j] || !s[j] || !b[j] || !outs[j]) return fail(ERR_BAD_ARG, "null buffer");
+    for (int j = 0; j < n; j++) {
+        LaunchCtx l2 = lc;
+        if (j) l2.start = nullptr;
+        if (j + 1 < n) l2.stop = nullptr;
+        // exact: the caller named a reference kernel, whose rows are GEMVs on the exact f32 s*q + b (as mt_qmm's are):
+        // the GEMV family at every M; else mtq_qmm's routing, which takes batches to the tiles and their rounded weights
+        int rc = exact ? op_qmv(dtype, bits, G, w[j], s[j], b[j], x, outs[j], M, N[j], K, l2)
+                       : op_qmm(dtype, bits, G, w[j], s[j], b[j], x, outs[j], M, N[j], K, false, l2);
+        if (rc) return rc;
+    }
+    return ERR_OK;
+}
+
 static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, const void* w,
                      const void* s, const void* b, const uint32_t* route, void* out, uint32_t T,
                      uint32_t N, uint32_t K, uint32_t E, const LaunchCtx& lc, bool exact_only = false) {
@@ -558,7 +587,7 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
 // name-keyed dispatch table
 // ---------------------------------------------------------------------------
 
-enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_NORMQ, F_GNORMQ, F_ROUTER, F_PERMUTE, F_UNPERMUTE, F_MOEDOWN, F_QVM, F_QVM_FAST };
+enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_BQKV_QMM, F_B4_QMM, F_NORMQ, F_GNORMQ, F_ROUTER, F_PERMUTE, F_UNPERMUTE, F_MOEDOWN, F_QVM, F_QVM_FAST };
 
 struct KernelDesc {
     const char* name;
@@ -615,6 +644,10 @@ static const KernelDesc kTable[] = {
     {"ffai_batched_qkv_qgemv", F_BQKV, 4, 11, 5}, {"ffai_batched_qkv_qgemv_fast", F_BQKV, 4, 11, 5},
     // x, (w, scales, biases) x 4, a_out .. d_out | out_a .. out_d, in_dim, group_size
     {"ffai_batched_4_qgemv_fast", F_B4, 4, 17, 6},
+    // x, (w, scales, biases) x 3, q_buf, k_buf, v_buf | out_q, out_k, out_v, in_dim, group_size (M rows: from x)
+    {"ffai_batched_qkv_qmm_fast", F_BQKV_QMM, 4, 13, 5},
+    // x, (w, scales, biases) x 4, a_buf .. d_buf | out_a .. out_d, in_dim, group_size
+    {"ffai_batched_4_qmm_fast", F_B4_QMM, 4, 17, 6},
     // x, norm_weight, weight, scales, biases, output, eps_buf | in_dim, group_size
     {"ffai_rms_norm_qgemv", F_NORMQ, 4, 7, 2}, {"ffai_rms_norm_qgemv_fast", F_NORMQ, 4, 7, 2},
     {"ffai_rms_norm_qgemv_int8_fast", F_NORMQ, 8, 7, 2},
@@ -857,6 +890,32 @@ static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, in
             MTQ_NEED(bufs[6], "eps_buf", 4);
             return op_rms_norm_qmv(dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, bufs[4].ptr,
                                    bufs[5].ptr, (const float*)bufs[6].ptr, N, K, lc);
+        }
+        case F_BQKV_QMM:
+        case F_B4_QMM: {
+            // the reference takes the number of rows from the grid; here it is what x holds
+            const int n = d.fam == F_BQKV_QMM ? 3 : 4;
+            const uint32_t K = consts[n], G = consts[n + 1];
+            if (K == 0 || G == 0 || K % G) return fail(ERR_SHAPE, "group_size must divide in_dim");
+            if (bufs[0].bytes % ((uint64_t)K * sz)) return fail(ERR_BUFFER_SIZE, "'x' must hold whole rows of in_dim");
+            const uint64_t M = bufs[0].bytes / ((uint64_t)K * sz);
+            if (M > 0xFFFFFFFFull) return fail(ERR_SHAPE, "too many rows");
+            const void *w[4], *s[4], *b[4];
+            void* outs[4];
+            uint32_t N[4];
+            for (int j = 0; j < n; j++) {
+                N[j] = consts[j];
+                if (N[j] == 0) return fail(ERR_SHAPE, "every out_* must be non-zero");
+                MTQ_NEED(bufs[1 + 3 * j], "w_*", (uint64_t)N[j] * K * bits / 8);
+                MTQ_NEED(bufs[2 + 3 * j], "scales_*", (uint64_t)N[j] * (K / G) * sz);
+                MTQ_NEED(bufs[3 + 3 * j], "biases_*", (uint64_t)N[j] * (K / G) * sz);
+                MTQ_NEED(bufs[1 + 3 * n + j], "*_buf", M * N[j] * sz);
+                w[j] = bufs[1 + 3 * j].ptr;
+                s[j] = bufs[2 + 3 * j].ptr;
+                b[j] = bufs[3 + 3 * j].ptr;
+                outs[j] = bufs[1 + 3 * n + j].ptr;
+            }
+            return op_qmm_batched(dtype, d.bits, G, n, w, s, b, bufs[0].ptr, outs, N, (uint32_t)M, K, true, lc);
         }
         case F_GNORMQ: {
             const uint32_t hv = consts[0], dv = consts[1], N = consts[2], G = consts[3];
@@ -1165,6 +1224,13 @@ int mtq_qmv_batched(int dtype, int bits, uint32_t group_size, int n_mats, const 
     int rc = need_ready();
     if (rc) return rc;
     return op_qmv_batched(dtype, bits, group_size, n_mats, w, scales, biases, x, outs, N, K, make_ctx());
+}
+
+int mtq_qmm_batched(int dtype, int bits, uint32_t group_size, int n_mats, const void* const* w, const void* const* scales,
+                    const void* const* biases, const void* x, void* const* outs, const uint32_t* N, uint32_t M, uint32_t K) {
+    int rc = need_ready();
+    if (rc) return rc;
+    return op_qmm_batched(dtype, bits, group_size, n_mats, w, scales, biases, x, outs, N, M, K, false, make_ctx());
 }
 
 int mtq_gated_rms_norm_qmv(int dtype, uint32_t group_size, const float* y, const void* z, const void* norm_weight,

@@ -66,6 +66,15 @@ def qmv_batched(dtype, bits, group_size, ws, scales, biases, x, outs, Ns, K):
                                    (C.c_uint32 * n)(*Ns), K))
 
 
+def qmm_batched(dtype, bits, group_size, ws, scales, biases, x, outs, Ns, M, K):
+    """1..4 weight matrices (lists of buffers) against the same M activation rows; outs[j] is [M, Ns[j]]."""
+    lib = _ensure_init()
+    n = len(ws)
+    arr = lambda bufs: (C.c_void_p * n)(*[_p(b) for b in bufs])
+    _lib.check(lib.mtq_qmm_batched(int(dtype), bits, group_size, n, arr(ws), arr(scales), arr(biases), _p(x), arr(outs),
+                                   (C.c_uint32 * n)(*Ns), M, K))
+
+
 def rms_norm_qmv(dtype, bits, group_size, x, norm_weight, w, scales, biases, out, eps_buf, N, K):
     """out = qmv(w_hat, rms_norm(x) * norm_weight); eps_buf is a device buffer holding one f32."""
     lib = _ensure_init()

@@ -6,7 +6,7 @@ out / output, crates/metaltile-macros/src/legacy/sig_parser.rs:43-48,85).
 Sources: crates/metaltile-std/src/mlx/quantized.rs:8-16, 343-352, 4273-4285;
 ffai/dequant_gemv.rs:52-62; ffai/dequant_gemv_expert_indexed.rs:58-68;
 ffai/moe.rs:358-370, 2256-2268; mlx/quantized.rs:3575-3581, 3629-3635 (affine
-quantise / dequantise); ffai/gated_rms_norm_qgemv.rs:90-103.
+quantise / dequantise); ffai/gated_rms_norm_qgemv.rs:90-103; ffai/batched_qkv_qmm.rs:49-68; ffai/batched_4_qmm.rs:61-85.
 """
 from __future__ import annotations
 
@@ -71,6 +71,12 @@ _add("ffai_batched_4_qgemv_fast", 4,
      ("x", "w_a", "scales_a", "biases_a", "w_b", "scales_b", "biases_b", "w_c", "scales_c", "biases_c",
       "w_d", "scales_d", "biases_d", "a_out", "b_out", "c_out", "d_out"),
      ("out_a", "out_b", "out_c", "out_d", "in_dim", "group_size"), ("a_out", "b_out", "c_out", "d_out"))
+_add("ffai_batched_qkv_qmm_fast", 4, _QKV[:-1] + ("q_buf", "k_buf", "v_buf"),
+     ("out_q", "out_k", "out_v", "in_dim", "group_size"), ("q_buf", "k_buf", "v_buf"))
+_add("ffai_batched_4_qmm_fast", 4,
+     ("x", "w_a", "scales_a", "biases_a", "w_b", "scales_b", "biases_b", "w_c", "scales_c", "biases_c",
+      "w_d", "scales_d", "biases_d", "a_buf", "b_buf", "c_buf", "d_buf"),
+     ("out_a", "out_b", "out_c", "out_d", "in_dim", "group_size"), ("a_buf", "b_buf", "c_buf", "d_buf"))
 for _n, _b in (("ffai_rms_norm_qgemv", 4), ("ffai_rms_norm_qgemv_fast", 4), ("ffai_rms_norm_qgemv_int8_fast", 8)):
     _add(_n, _b, ("x", "norm_weight", "weight", "scales", "biases", "output", "eps_buf"), ("in_dim", "group_size"), ("output",))
 _add("ffai_gated_rms_norm_qgemv_int4_fast", 4,
