@@ -302,6 +302,18 @@ MTQ_API int mtq_affine_quantize(int dtype, int bits, uint32_t group_size, const 
 MTQ_API int mtq_affine_dequantize(int dtype, int bits, uint32_t group_size, const void *w,
                                   const void *scales, const void *biases, void *out, size_t n_elem);
 
+/* Dequantising gather (a quantized embedding table): out[t, d] = scales[id, d / group_size] * code[id, d] +
+ * biases[id, d / group_size] rounded to T, id = indices[t]; weight u32[vocab, hidden * bits / 32] (each row a bit
+ * stream, element d at bits [d * bits, (d + 1) * bits)), scales / biases T[vocab, hidden / group_size], indices
+ * u32[n_tokens], out T[n_tokens, hidden]. Replaces dequant_gather_int{2,3,4,5,6,8}
+ * (crates/metaltile-std/src/ffai/dequant_gather.rs:45-100; under those names vocab is what `weight` holds and n_tokens
+ * what `indices` holds). An id >= vocab names no row: that output row keeps its bytes (the reference reads past the
+ * table). hidden and group_size multiples of 8 (4-, 8-bit), 16 (2-bit) or 32 (other widths), group_size / that a
+ * power of two; hidden a multiple of group_size. */
+MTQ_API int mtq_dequant_gather(int dtype, int bits, uint32_t group_size, const void *weight, const void *scales,
+                               const void *biases, const uint32_t *indices, void *out, uint32_t n_tokens,
+                               uint32_t hidden, uint32_t vocab);
+
 /* ---- name-keyed dispatch (the reference's binding convention) ----------- */
 
 /* Replaces Context::dispatch_with_grid (crates/metaltile-runtime/src/context.rs:269-283)

@@ -72,6 +72,7 @@ SIGNATURES = {
     "mtq_qvm_noalloc": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "mtq_qmv_batched": (C.c_int, [C.c_int, C.c_int, _u32, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
                                   C.POINTER(C.c_void_p), _vp, C.POINTER(C.c_void_p), _u32p, _u32]),
+    "mtq_dequant_gather": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "mtq_qmm_batched": (C.c_int, [C.c_int, C.c_int, _u32, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
                                   C.POINTER(C.c_void_p), _vp, C.POINTER(C.c_void_p), _u32p, _u32, _u32]),
     "mtq_rms_norm_qmv": (C.c_int, [C.c_int, C.c_int, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32]),

@@ -42,6 +42,11 @@ struct AffineArgs {
     uint32_t group_size;
     uint32_t lanes_per_group;  // G / EPL, a power of two
     uint32_t log2g;            // G is EPL * lanes_per_group: a power of two as well
+    // Gathering dequantise (a quantized embedding table): output row t is table row row_ids[t]; rows of
+    // lanes_per_row lanes; ids from n_rows on name no row and their output rows keep their bytes.
+    const uint32_t* row_ids;
+    uint32_t lanes_per_row;
+    uint32_t n_rows;
 };
 
 template <int BITS> struct AffineGeom {
@@ -167,7 +172,9 @@ __global__ __launch_bounds__(256) void affine_quantize_kernel(AffineArgs a) {
     }
 }
 
-template <int DT, int BITS>
+// GATHER: crates/metaltile-std/src/ffai/dequant_gather.rs:45-93 (one thread per element there; a lane's run of
+// elements here, the same bit stream and the same q * scale + bias).
+template <int DT, int BITS, bool GATHER = false>
 __global__ __launch_bounds__(256) void affine_dequantize_kernel(AffineArgs a) {
 #pragma clang fp contract(off)
     constexpr int EPL = AffineGeom<BITS>::EPL, NW = AffineGeom<BITS>::NW, U = AffineUnroll<BITS>::U;
@@ -180,7 +187,13 @@ __global__ __launch_bounds__(256) void affine_dequantize_kernel(AffineArgs a) {
     for (int u = 0; u < U; u++) {
         t[u] = ((uint64_t)blockIdx.x * U + u) * 256u + threadIdx.x;
         live[u] = t[u] < n_lanes;
-        const uint64_t tc = live[u] ? t[u] : n_lanes - 1;
+        uint64_t tc = live[u] ? t[u] : n_lanes - 1;
+        if constexpr (GATHER) {   // from the output lane to the lane of the table that holds its codes
+            const uint64_t row = tc / a.lanes_per_row;
+            const uint32_t id = a.row_ids[row];
+            live[u] = live[u] && id < a.n_rows;
+            tc = (uint64_t)(id < a.n_rows ? id : 0u) * a.lanes_per_row + (tc - row * a.lanes_per_row);
+        }
         const uint32_t* src = (const uint32_t*)a.in + tc * NW;
         if constexpr (NW == 2) {
             const uint2 w2 = *(const uint2*)src;
@@ -243,6 +256,65 @@ template <int DT> static int launch_bits(bool quantize, int bits, AffineArgs& a,
     }
 }
 
+template <int DT, int BITS> static int launch_gather_one(AffineArgs& a, uint32_t hidden, const LaunchCtx& lc) {
+    constexpr int EPL = AffineGeom<BITS>::EPL;
+    if (a.group_size % EPL || hidden % EPL) return fail(ERR_UNSUPPORTED, "dequant gather: group_size and hidden must be multiples of the lane's run (8, 16 or 32 elements)");
+    a.lanes_per_group = a.group_size / EPL;
+    if (a.lanes_per_group & (a.lanes_per_group - 1)) return fail(ERR_UNSUPPORTED, "dequant gather: group_size / run must be a power of two");
+    a.log2g = 0;
+    while ((1u << a.log2g) < a.group_size) a.log2g++;
+    a.lanes_per_row = hidden / EPL;
+    const uint64_t lanes = a.n_elem / EPL;
+    const uint64_t per_block = 256ull * AffineUnroll<BITS>::U;
+    const uint64_t blocks = (lanes + per_block - 1) / per_block;
+    if (blocks > 0x7FFFFFFFull) return fail(ERR_SHAPE, "dequant gather: too many elements for one launch");
+    void* args[] = {&a};
+    hipError_t e = launch_kernel((const void*)affine_dequantize_kernel<DT, BITS, true>, dim3((uint32_t)blocks), dim3(256), args, 0, lc);
+    if (e != hipSuccess) return hip_fail(e, "dequant gather kernel launch");
+    return ERR_OK;
+}
+
+template <int DT> static int launch_gather_bits(int bits, AffineArgs& a, uint32_t hidden, const LaunchCtx& lc) {
+    switch (bits) {
+        case 2: return launch_gather_one<DT, 2>(a, hidden, lc);
+        case 3: return launch_gather_one<DT, 3>(a, hidden, lc);
+        case 4: return launch_gather_one<DT, 4>(a, hidden, lc);
+        case 5: return launch_gather_one<DT, 5>(a, hidden, lc);
+        case 6: return launch_gather_one<DT, 6>(a, hidden, lc);
+        case 7: return launch_gather_one<DT, 7>(a, hidden, lc);
+        default: return launch_gather_one<DT, 8>(a, hidden, lc);
+    }
+}
+
+// out[t, :] = dequantised row ids[t] of a table [vocab, hidden] in the packed format (weight rows of hidden * bits / 32
+// words, scales / biases rows of hidden / group_size).
+int launch_dequant_gather(int dtype, int bits, uint32_t group_size, const void* weight, const void* scales, const void* biases,
+                          const uint32_t* ids, void* out, uint32_t n_tokens, uint32_t hidden, uint32_t vocab, const LaunchCtx& lc) {
+    if (bits < 2 || bits > 8) return fail(ERR_BAD_ARG, "bits must be in 2..8");
+    if (hidden == 0 || vocab == 0) return fail(ERR_SHAPE, "hidden and vocab must be non-zero");
+    if (group_size == 0 || hidden % group_size) return fail(ERR_SHAPE, "group_size must be non-zero and divide hidden");
+    if ((uint64_t)hidden * bits % 32) return fail(ERR_SHAPE, "hidden*bits must be a multiple of 32");
+    if (n_tokens == 0) return ERR_OK;
+    if (!weight || !scales || !biases || !ids || !out) return fail(ERR_BAD_ARG, "null buffer");
+    if ((uintptr_t)weight % 16 || (uintptr_t)out % 16) return fail(ERR_UNSUPPORTED, "dequant gather: buffers must be 16-byte aligned");
+    AffineArgs a;
+    a.in = weight;
+    a.out = out;
+    a.scales = const_cast<void*>(scales);
+    a.biases = const_cast<void*>(biases);
+    a.n_elem = (uint64_t)n_tokens * hidden;
+    a.group_size = group_size;
+    a.lanes_per_group = 1;
+    a.row_ids = ids;
+    a.n_rows = vocab;
+    switch (dtype) {
+        case DT_F32: return launch_gather_bits<DT_F32>(bits, a, hidden, lc);
+        case DT_F16: return launch_gather_bits<DT_F16>(bits, a, hidden, lc);
+        case DT_BF16: return launch_gather_bits<DT_BF16>(bits, a, hidden, lc);
+        default: return fail(ERR_BAD_ARG, "unknown dtype");
+    }
+}
+
 int launch_affine(bool quantize, int dtype, int bits, uint32_t group_size, const void* in, void* out,
                   void* scales, void* biases, uint64_t n_elem, const LaunchCtx& lc) {
     if (bits < 2 || bits > 8) return fail(ERR_BAD_ARG, "bits must be in 2..8");
@@ -258,6 +330,9 @@ int launch_affine(bool quantize, int dtype, int bits, uint32_t group_size, const
     a.n_elem = n_elem;
     a.group_size = group_size;
     a.lanes_per_group = 1;
+    a.row_ids = nullptr;
+    a.lanes_per_row = 0;
+    a.n_rows = 0;
     switch (dtype) {
         case DT_F32: return launch_bits<DT_F32>(quantize, bits, a, lc);
         case DT_F16: return launch_bits<DT_F16>(quantize, bits, a, lc);

@@ -587,7 +587,7 @@ static int op_gather(int mode, int dtype, int bits, uint32_t G, const void* x, c
 // name-keyed dispatch table
 // ---------------------------------------------------------------------------
 
-enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_BQKV, F_B4, F_BQKV_QMM, F_B4_QMM, F_NORMQ, F_GNORMQ, F_ROUTER, F_PERMUTE, F_UNPERMUTE, F_MOEDOWN, F_QVM, F_QVM_FAST };
+enum Family { F_QMV, F_QMM, F_QMM_MMA, F_QB, F_DGEMV, F_EXPERT, F_GCSR, F_GIDX, F_AQ, F_ADQ, F_DGATHER, F_BQKV, F_B4, F_BQKV_QMM, F_B4_QMM, F_NORMQ, F_GNORMQ, F_ROUTER, F_PERMUTE, F_UNPERMUTE, F_MOEDOWN, F_QVM, F_QVM_FAST };
 
 struct KernelDesc {
     const char* name;
@@ -640,6 +640,10 @@ static const KernelDesc kTable[] = {
     {"mt_moe_gather_qmm_mma_int8", F_GIDX, 8, 6, 4}, {"mt_moe_gather_qmm_mma_b3", F_GIDX, 3, 6, 4},
     {"mt_moe_gather_qmm_mma_b5", F_GIDX, 5, 6, 4}, {"mt_moe_gather_qmm_mma_b6", F_GIDX, 6, 6, 4},
     {"mt_moe_gather_qmm_mma_b8", F_GIDX, 8, 6, 4},
+    // weight, scales, biases, indices, out | hidden, group_size
+    {"dequant_gather_int2", F_DGATHER, 2, 5, 2}, {"dequant_gather_int3", F_DGATHER, 3, 5, 2},
+    {"dequant_gather_int4", F_DGATHER, 4, 5, 2}, {"dequant_gather_int5", F_DGATHER, 5, 5, 2},
+    {"dequant_gather_int6", F_DGATHER, 6, 5, 2}, {"dequant_gather_int8", F_DGATHER, 8, 5, 2},
     // x, (w, scales, biases) x 3, out | out_q, out_k, out_v, in_dim, group_size
     {"ffai_batched_qkv_qgemv", F_BQKV, 4, 11, 5}, {"ffai_batched_qkv_qgemv_fast", F_BQKV, 4, 11, 5},
     // x, (w, scales, biases) x 4, a_out .. d_out | out_a .. out_d, in_dim, group_size
@@ -890,6 +894,21 @@ static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, in
             MTQ_NEED(bufs[6], "eps_buf", 4);
             return op_rms_norm_qmv(dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, bufs[4].ptr,
                                    bufs[5].ptr, (const float*)bufs[6].ptr, N, K, lc);
+        }
+        case F_DGATHER: {
+            // the table's row count is what `weight` holds; the token count what `indices` holds
+            const uint32_t H = consts[0], G = consts[1];
+            if (H == 0 || G == 0 || H % G) return fail(ERR_SHAPE, "group_size must divide hidden");
+            if ((uint64_t)H * bits % 32) return fail(ERR_SHAPE, "hidden*bits must be a multiple of 32");
+            const uint64_t row_bytes = (uint64_t)H * bits / 8;
+            const uint64_t vocab = bufs[0].bytes / row_bytes, T = bufs[3].bytes / 4;
+            if (vocab == 0) return fail(ERR_BUFFER_SIZE, "buffer 'weight' holds less than one row");
+            if (vocab > 0xFFFFFFFFull || T > 0xFFFFFFFFull) return fail(ERR_SHAPE, "too many rows");
+            MTQ_NEED(bufs[1], "scales", vocab * (H / G) * sz);
+            MTQ_NEED(bufs[2], "biases", vocab * (H / G) * sz);
+            MTQ_NEED(bufs[4], "out", T * H * sz);
+            return launch_dequant_gather(dtype, d.bits, G, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, (const uint32_t*)bufs[3].ptr,
+                                         bufs[4].ptr, (uint32_t)T, H, (uint32_t)vocab, lc);
         }
         case F_BQKV_QMM:
         case F_B4_QMM: {
@@ -1224,6 +1243,14 @@ int mtq_qmv_batched(int dtype, int bits, uint32_t group_size, int n_mats, const 
     int rc = need_ready();
     if (rc) return rc;
     return op_qmv_batched(dtype, bits, group_size, n_mats, w, scales, biases, x, outs, N, K, make_ctx());
+}
+
+int mtq_dequant_gather(int dtype, int bits, uint32_t group_size, const void* weight, const void* scales, const void* biases,
+                       const uint32_t* indices, void* out, uint32_t n_tokens, uint32_t hidden, uint32_t vocab) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (dtype != DT_F32 && dtype != DT_F16 && dtype != DT_BF16) return fail(ERR_BAD_ARG, "dtype must be MTQ_F32, MTQ_F16 or MTQ_BF16");
+    return launch_dequant_gather(dtype, bits, group_size, weight, scales, biases, indices, out, n_tokens, hidden, vocab, make_ctx());
 }
 
 int mtq_qmm_batched(int dtype, int bits, uint32_t group_size, int n_mats, const void* const* w, const void* const* scales,

@@ -214,5 +214,7 @@ int launch_qmm_f32_grouped(const QmmParams& p, const uint32_t* route, bool per_r
 // dequantise (packed words + scales + biases -> T[n_elem]) (affine.hip).
 int launch_affine(bool quantize, int dtype, int bits, uint32_t group_size, const void* in, void* out,
                   void* scales, void* biases, uint64_t n_elem, const LaunchCtx& lc);
+int launch_dequant_gather(int dtype, int bits, uint32_t group_size, const void* weight, const void* scales, const void* biases,
+                          const uint32_t* ids, void* out, uint32_t n_tokens, uint32_t hidden, uint32_t vocab, const LaunchCtx& lc);
 
 }  // namespace mtq

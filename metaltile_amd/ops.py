@@ -135,6 +135,13 @@ def affine_dequantize(dtype, bits, group_size, w, scales, biases, out, n_elem):
     _lib.check(lib.mtq_affine_dequantize(int(dtype), bits, group_size, _p(w), _p(scales), _p(biases), _p(out), n_elem))
 
 
+def dequant_gather(dtype, bits, group_size, weight, scales, biases, indices, out, n_tokens, hidden, vocab):
+    """out[t, :] = dequantised row indices[t] of the packed table [vocab, hidden]."""
+    lib = _ensure_init()
+    _lib.check(lib.mtq_dequant_gather(int(dtype), bits, group_size, _p(weight), _p(scales), _p(biases), _p(indices), _p(out),
+                                      n_tokens, hidden, vocab))
+
+
 def timed(fn, *args, **kw) -> float:
     """Run one op with GPU timestamps attached to its kernel; returns microseconds."""
     lib = _ensure_init()

@@ -6,7 +6,7 @@ out / output, crates/metaltile-macros/src/legacy/sig_parser.rs:43-48,85).
 Sources: crates/metaltile-std/src/mlx/quantized.rs:8-16, 343-352, 4273-4285;
 ffai/dequant_gemv.rs:52-62; ffai/dequant_gemv_expert_indexed.rs:58-68;
 ffai/moe.rs:358-370, 2256-2268; mlx/quantized.rs:3575-3581, 3629-3635 (affine
-quantise / dequantise); ffai/gated_rms_norm_qgemv.rs:90-103; ffai/batched_qkv_qmm.rs:49-68; ffai/batched_4_qmm.rs:61-85.
+quantise / dequantise); ffai/gated_rms_norm_qgemv.rs:90-103; ffai/batched_qkv_qmm.rs:49-68; ffai/batched_4_qmm.rs:61-85; ffai/dequant_gather.rs:47-55.
 """
 from __future__ import annotations
 
@@ -64,6 +64,8 @@ for _b in (2, 3, 4, 5, 6, 8):
     _add(f"mt_affine_quantize_int{_b}", _b, ("w", "out", "scales", "biases"), ("group_size",),
          ("out", "scales", "biases"))
     _add(f"mt_affine_dequantize_int{_b}", _b, ("w", "scales", "biases", "out"), ("group_size",), ("out",))
+for _b in (2, 3, 4, 5, 6, 8):
+    _add(f"dequant_gather_int{_b}", _b, ("weight", "scales", "biases", "indices", "out"), ("hidden", "group_size"), ("out",))
 _QKV = ("x", "w_q", "scales_q", "biases_q", "w_k", "scales_k", "biases_k", "w_v", "scales_v", "biases_v", "out")
 for _n in ("ffai_batched_qkv_qgemv", "ffai_batched_qkv_qgemv_fast"):
     _add(_n, 4, _QKV, ("out_q", "out_k", "out_v", "in_dim", "group_size"), ("out",))

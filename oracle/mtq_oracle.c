@@ -31,6 +31,8 @@
  *                     gate == that gate x the (pinned) rms_norm_qgemv; z = 0 -> zero output; silu(ln 3) = 0.75 ln 3;
  *                     scaling one row of y leaves the output unchanged at eps = 0 (the sums of squares are per
  *                     row); norm weights repeat per row (index d, not r * dv + d).
+ *   dequant_gather    (oracle.py: the pinned dequantiser over the table and a numpy row take) brute-force bit
+ *                     extraction per element on the reference test's table generator.
  *   qvm               numpy f64 `x @ dequant(W)` on the [K, N] layout, and qvm(W) == qmv of the
  *                     transposed, repacked matrix.
  *   moe routing       numpy stable argsort + library softmax, the reference tests' tie-break,

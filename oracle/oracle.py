@@ -273,6 +273,14 @@ def affine_dequantize(w, scales, biases, n_elem: int, group_size: int, bits: int
     return out
 
 
+def dequant_gather(weight, scales, biases, indices, vocab: int, hidden: int, group_size: int, bits: int) -> np.ndarray:
+    """out[t, :] = row indices[t] of the dequantised table [vocab, hidden]: the affine dequantiser over the whole table
+    (each row a bit stream of hidden codes, groups along the row) and a row take. Reference:
+    crates/metaltile-std/src/ffai/dequant_gather.rs:148-185 (its CPU form), :56-93 (kernel)."""
+    table = affine_dequantize(weight, scales, biases, vocab * hidden, group_size, bits).reshape(vocab, hidden)
+    return table[np.asarray(indices, dtype=np.int64)]
+
+
 def bench_stats(samples) -> dict:
     s = np.ascontiguousarray(samples, dtype=np.float64)
     out = np.empty(7, dtype=np.float64)

@@ -347,6 +347,27 @@ def test_gated_rms_norm_qgemv_on_the_reference_test_setup(oracle):
     assert np.max(np.abs(plain)) > 1.0
 
 
+@pytest.mark.parametrize("bits,hidden,g", [(2, 256, 64), (4, 256, 64), (8, 256, 64), (3, 64, 32), (5, 64, 32), (6, 64, 32)])
+def test_dequant_gather_brute_force_on_the_reference_table(oracle, bits, hidden, g):
+    """The reference test's table (crates/metaltile-std/src/ffai/dequant_gather.rs:187-215: 8 rows from its bit-stream
+    generator, scales 0.02 + (i % 7) * 0.01, biases ((i % 5) - 2) * 0.05, rows 3 0 7 1 4 4): every output element
+    against the code re-derived from the generator's formula (not read back from the packed words) times its group's
+    scale plus bias; a repeated row, and a row order that is not the table's."""
+    vocab, ids = 8, np.array([3, 0, 7, 1, 4, 4], dtype=np.uint32)
+    ng = hidden // g
+    w = oracle.synth_bitstream_w(vocab, hidden, bits)
+    s = (0.02 + (np.arange(vocab * ng) % 7) * 0.01).astype(np.float32)
+    b = (((np.arange(vocab * ng) % 5).astype(np.float32) - 2.0) * 0.05).astype(np.float32)
+    out = oracle.dequant_gather(w, s, b, ids, vocab, hidden, g, bits)
+    assert out.shape == (ids.size, hidden)
+    for t, r in enumerate(ids.tolist()):
+        for d in range(hidden):
+            code = (((r * hidden + d) * 2654435761 + d) & 0xFFFFFFFF) & ((1 << bits) - 1)
+            want = np.float32(code) * s[r * ng + d // g] + b[r * ng + d // g]
+            assert out[t, d] == want, (t, d)
+    assert np.array_equal(out[4], out[5]) and not np.array_equal(out[0], out[1])
+
+
 def _np_topk(logits, k, mode):
     """Independent restatement: stable descending argsort + library softmax."""
     from scipy.special import softmax
