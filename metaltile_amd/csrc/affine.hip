@@ -189,10 +189,11 @@ __global__ __launch_bounds__(256) void affine_dequantize_kernel(AffineArgs a) {
         live[u] = t[u] < n_lanes;
         uint64_t tc = live[u] ? t[u] : n_lanes - 1;
         if constexpr (GATHER) {   // from the output lane to the lane of the table that holds its codes
-            const uint64_t row = tc / a.lanes_per_row;
+            const uint32_t tc32 = (uint32_t)tc;   // (the host keeps the lane count below 2^32: a 64-bit quotient costs four times this one)
+            const uint32_t row = tc32 / a.lanes_per_row;
             const uint32_t id = a.row_ids[row];
             live[u] = live[u] && id < a.n_rows;
-            tc = (uint64_t)(id < a.n_rows ? id : 0u) * a.lanes_per_row + (tc - row * a.lanes_per_row);
+            tc = (uint64_t)(id < a.n_rows ? id : 0u) * a.lanes_per_row + (tc32 - row * a.lanes_per_row);
         }
         const uint32_t* src = (const uint32_t*)a.in + tc * NW;
         if constexpr (NW == 2) {
@@ -267,7 +268,7 @@ template <int DT, int BITS> static int launch_gather_one(AffineArgs& a, uint32_t
     const uint64_t lanes = a.n_elem / EPL;
     const uint64_t per_block = 256ull * AffineUnroll<BITS>::U;
     const uint64_t blocks = (lanes + per_block - 1) / per_block;
-    if (blocks > 0x7FFFFFFFull) return fail(ERR_SHAPE, "dequant gather: too many elements for one launch");
+    if (blocks > 0x7FFFFFFFull || lanes > 0xFFFFFFFFull) return fail(ERR_SHAPE, "dequant gather: too many elements for one launch");
     void* args[] = {&a};
     hipError_t e = launch_kernel((const void*)affine_dequantize_kernel<DT, BITS, true>, dim3((uint32_t)blocks), dim3(256), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "dequant gather kernel launch");
