@@ -231,7 +231,7 @@ MTQ_API int mtq_rms_norm_qmv(int dtype, int bits, uint32_t group_size, const voi
  * N % 8 == 0, group_size 64, dv % 32 == 0, hv even, hv * dv <= 8192) are not required here: any hv, dv >= 1 with
  * group_size dividing hv * dv. inner is an f32 value as in the reference (never rounded to T); the f16 / bf16 kernels
  * carry it as a rounded value plus a rounded remainder (16 significant bits). One launch for f16 / bf16 when hv * dv is a
- * multiple of 2048 (at most 32768) and dv is 32 .. 2048 in powers of two; otherwise inner is written to a library-owned
+ * multiple of 2048 (at most 16384) and dv is 32 .. 2048 in powers of two; otherwise inner is written to a library-owned
  * buffer first (allocated on first use, grown on demand) and an ordinary qmv follows. */
 MTQ_API int mtq_gated_rms_norm_qmv(int dtype, uint32_t group_size, const float *y, const void *z, const void *norm_weight,
                                    const float *eps_buf, const void *w, const void *scales, const void *biases, void *out,
@@ -437,7 +437,7 @@ MTQ_API int mtq_flush_cache(void);
  *                          matrix-core GEMV geometry: K parts per row, row blocks side by side and one
  *                          after the other per workgroup, 4-row activation sets per pass; 0 = choose
  *   "qmv.gated_fused"      mtq_gated_rms_norm_qmv as one launch of the streaming kernel (hv * dv a multiple of 2048 up to
- *                          32768, dv = 32 .. 2048 in powers of two): 0 = for f16 / bf16, 1 = never (the activation is staged
+ *                          16384, dv = 32 .. 2048 in powers of two): 0 = for f16 / bf16, 1 = never (the activation is staged
  *                          in the library's buffer), 2 = wherever the shape allows
  *   "qmv.norm_mfma"        mtq_rms_norm_qmv with the norm applied inside the matrix-core GEMV (4-bit codes, f16 / bf16):
  *                          0 = where it is faster than the streaming kernel's fused form, 1 = never, 2 = wherever the

@@ -445,8 +445,8 @@ static int op_gated_rms_norm_qmv(int dtype, uint32_t G, const float* y, const vo
     if (rc) return rc;
     if (!y || !z || !norm_w || !eps || !w || !s || !b || !out) return fail(ERR_BAD_ARG, "null buffer");
     // One launch: the streaming kernel gates and normalises the slice each thread holds. us per call, staged (three
-    // launches; two for f32) -> one launch, dv 128: bf16 hv 16, 2048 rows 7.8 -> 5.6 (the plain qmv of that matrix: 3.3);
-    // hv 32, 1024 rows 10.3 -> 5.6; hv 32, 4096 rows 9.3 -> 8.3; hv 64, 8192 rows 14.3 -> 14.0. f32 stays staged (6.3 -> 6.9,
+    // launches; two for f32) -> one launch, dv 128: bf16 hv 16, 2048 rows 7.7 -> 5.1 (the plain qmv of that matrix: 3.3);
+    // hv 32, 1024 rows 10.3 -> 5.7; hv 32, 4096 rows 9.3 -> 8.0; hv 64, 8192 rows 14.8 -> 14.5. f32 stays staged (6.3 -> 6.9,
     // 7.9 -> 11.5, 16.3 -> 19.3): its one-row streaming kernel is the slower one to begin with.
     if (options().qmv_gated_fused == 2 || (options().qmv_gated_fused == 0 && dtype != DT_F32)) {
         QmvParams p;

@@ -138,6 +138,7 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
     g.grid = dim3((p.N + a.rows_per_wg - 1) / a.rows_per_wg, batch ? (uint32_t)batch->n : routed ? p.T : 1u, 1);
     if (norm_w) {
         g.shmem += 16 * sizeof(float);  // one partial sum of squares per wave
+        if (gate_z && rps == 4 && p.dtype != DT_F32) g.shmem += 16 + (size_t)C * 4 * 16 * 2;   // the gated halves, dealt over the row slots
         switch (p.dtype) {
             case DT_F32: return qmv_stream_norm_launch_dtype<DT_F32>(a, p.bits, g, lc);
             case DT_F16: return qmv_stream_norm_launch_dtype<DT_F16>(a, p.bits, g, lc);
@@ -213,11 +214,11 @@ int launch_qmv_gated_norm(const QmvParams& p0, const void* gate_z, const void* n
     const uint32_t G = p.group_size;
     if (!is_pow2(G) || G * 2 < cpc || p.K % G) return fail(ERR_UNSUPPORTED, "gated norm + qmv: group size");
     const uint32_t C = p.K / cpc;
-    if (C > 1024 || C % 64) return fail(ERR_UNSUPPORTED, "gated norm + qmv: row geometry");
+    if (C > 512 || C % 64) return fail(ERR_UNSUPPORTED, "gated norm + qmv: row geometry");
     if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)norm_w % 16 || (uintptr_t)gate_z % 16)
         return fail(ERR_UNSUPPORTED, "gated norm + qmv: w, y, z and norm_weight must be 16-byte aligned");
     uint32_t rps = 1;
-    while (C * rps < 256 && C * rps * 2 <= 1024) rps *= 2;
+    while (C * rps < 256 && C * rps * 2 <= 512) rps *= 2;
     return launch_qmv_stream(p, C, rps, C * rps, 1, lc, nullptr, norm_w, eps, gate_z, dv);
 }
 

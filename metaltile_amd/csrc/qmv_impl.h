@@ -467,9 +467,14 @@ template <int DT> __device__ __forceinline__ void raw_gated(const uint4* yv, uin
 // of dv f32 values y, each row normalised by its own sum of squares and gated by silu(z): a thread's chunk lies within
 // one such row (dv a multiple of the chunk), the row's dv / CPC threads are neighbours in a wave, so the sum of squares
 // is a segmented lane reduction and needs no LDS.
+// NORM = 3: the same with four row slots per workgroup (rows of 2048 values in 256 threads): the four threads that
+// hold the same chunk gate a quarter of it each (one vector of 8) and pass the halves through LDS behind the barrier
+// the staging needs anyway, instead of each gating all 32 values ahead of its first dot product.
 template <int DT, int BITS, int MB, int D, int MODE, int MAXT, int SBI, int NORM = 0>
 __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
     static_assert(!NORM || (MB == (DT == DT_F32 ? 1 : 2) && MODE == GATHER_NONE), "the fused norm takes one plain activation row");
+    static_assert(NORM != 3 || (DT != DT_F32 && BITS == 4), "the dealt gate: 16-bit types, 4-bit codes");
+    constexpr bool GATED = NORM == 2 || NORM == 3;
     constexpr int MBR = NORM ? 1 : MB;  // activation rows as the caller sees them
     static_assert(D == 4 || D == 8, "ring depth");
     typedef XSlice<DT, BITS> XS;
@@ -555,12 +560,13 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
     MTQ_KEEP_LOAD_ORDER();
     XS xs[MB];
     uint4 xraw[MB][XS::NRAW];
-    uint4 yraw[NORM == 2 ? CPC / 4 : 1];
-    if constexpr (NORM == 2) {
+    uint4 yraw[GATED ? CPC / 4 : 1];
+    if constexpr (GATED) {
         const uint4* yp = (const uint4*)((const float*)a.x + k0);
 #pragma unroll
         for (int i = 0; i < CPC / 4; i++) yraw[i] = yp[i];
-        xs[0].load_raw(a.gate_z, k0, xraw[0]);
+        if constexpr (NORM == 3) xraw[0][0] = ((const uint4*)((const uint16_t*)a.gate_z + k0))[rsub];   // this row slot's quarter
+        else xs[0].load_raw(a.gate_z, k0, xraw[0]);
     } else {
 #pragma unroll
         for (int mb = 0; mb < MBR; mb++) {
@@ -574,7 +580,8 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
         // issued ahead of the weight stream: loads return in order, so a late load of eps
         // would wait for the whole first ring
         eps = a.eps[0];
-        xs[0].load_raw(a.norm_w, NORM == 2 ? k0 % a.dv : k0, nraw);
+        if constexpr (NORM == 3) nraw[0] = ((const uint4*)((const uint16_t*)a.norm_w + k0 % a.dv))[rsub];
+        else xs[0].load_raw(a.norm_w, NORM == 2 ? k0 % a.dv : k0, nraw);
     }
     MTQ_KEEP_LOAD_ORDER();
     u32x4 ring[D];
@@ -597,6 +604,26 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
             dst[0] = make_float4(sv[0], bv[0] - MAGIC * sv[0], sv[1], bv[1] - MAGIC * sv[1]);
             dst[1] = make_float4(sv[2], bv[2] - MAGIC * sv[2], sv[3], bv[3] - MAGIC * sv[3]);
         }
+    }
+    uint4* gx = (uint4*)(((uintptr_t)(ssq_part + 16) + 15) & ~(uintptr_t)15);   // NORM = 3: [C][4] value vectors, then [C][4] remainders
+    if constexpr (NORM == 3) {
+        float ssq = 0.f;
+#pragma unroll
+        for (int i = 0; i < CPC / 4; i++) ssq += raw_sumsq<DT_F32>(yraw[i]);
+        ssq = seg_allreduce(ssq, (int)(a.dv / CPC));
+        const float inv = 1.0f / sqrtf(ssq / (float)a.dv + eps);
+        // this row slot's two vectors of y, loaded again (picking them out of yraw by rsub is an indexed read of a
+        // register array, which goes through scratch memory)
+        uint4 yq[2];
+        {
+            const uint4* yp = (const uint4*)((const float*)a.x + k0) + 2u * rsub;
+            yq[0] = yp[0];
+            yq[1] = yp[1];
+        }
+        uint4 hi, lo;
+        raw_gated<DT>(yq, xraw[0][0], nraw[0], inv, hi, lo);
+        gx[c * 4u + rsub] = hi;
+        gx[(a.C + c) * 4u + rsub] = lo;
     }
     if constexpr (NORM == 2) {
         float ssq = 0.f;
@@ -624,6 +651,13 @@ __global__ __launch_bounds__(MAXT) void qmv_stream_kernel(QmvSArgs a) {
         if (lane == 0) ssq_part[tid >> 6] = ssq;
     }
     __syncthreads();
+    if constexpr (NORM == 3) {
+#pragma unroll
+        for (int i = 0; i < XS::NRAW; i++) {
+            xraw[0][i] = gx[c * 4u + i];
+            xraw[1][i] = gx[(a.C + c) * 4u + i];
+        }
+    }
     if constexpr (NORM == 1) {
         float tot = 0.f;
         for (uint32_t wv = 0; wv < (TPB >> 6); wv++) tot += ssq_part[wv];
@@ -781,14 +815,14 @@ static int qmv_stream_launch_sbi(QmvSArgs& a, const QmvSGeom& g, const LaunchCtx
 }
 
 // Fused-RMSNorm instances: one activation row, 4- or 8-bit codes (NORMK = 1); the gated form, 4-bit codes (NORMK = 2).
-template <int DT, int BITS, int D, int NORMK = 1>
+template <int DT, int BITS, int D, int NORMK = 1, int MAXT = 1024>
 static int qmv_stream_norm_launch_d(QmvSArgs& a, const QmvSGeom& g, const LaunchCtx& lc) {
     constexpr int MBN = DT == DT_F32 ? 1 : 2;  // 16-bit types carry the normalised row as value + remainder
     const void* fn;
     switch (g.sbi) {
-        case 1: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 1, NORMK>; break;
-        case 2: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 2, NORMK>; break;
-        default: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, 1024, 4, NORMK>; break;
+        case 1: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, MAXT, 1, NORMK>; break;
+        case 2: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, MAXT, 2, NORMK>; break;
+        default: fn = (const void*)qmv_stream_kernel<DT, BITS, MBN, D, GATHER_NONE, MAXT, 4, NORMK>; break;
     }
     if (g.shmem > 48 * 1024) {
         hipError_t e = set_max_dynamic_lds(fn, (size_t)g.shmem);
@@ -804,7 +838,12 @@ template <int DT> int qmv_stream_norm_launch_dtype(QmvSArgs& a, int bits, const 
     if (g.mb != 1 || (g.d != 4 && g.d != 8)) return fail(ERR_UNSUPPORTED, "norm + qmv: no kernel instance for this geometry");
     if (a.gate_z) {
         if (bits != 4 || g.d != 4) return fail(ERR_UNSUPPORTED, "gated norm + qmv: 4-bit codes, ring of four");
-        return qmv_stream_norm_launch_d<DT, 4, 4, 2>(a, g, lc);
+        if constexpr (DT != DT_F32) {
+            if (a.rps == 4) return qmv_stream_norm_launch_d<DT, 4, 4, 3, 512>(a, g, lc);   // the gate dealt over the four row slots
+        }
+        // (workgroups of at most 512 threads: with the register budget of 1024 the gate's 32 values spill)
+        if (g.tpb > 512) return fail(ERR_UNSUPPORTED, "gated norm + qmv: rows of at most 16384 values");
+        return qmv_stream_norm_launch_d<DT, 4, 4, 2, 512>(a, g, lc);
     }
     if (bits == 4) return g.d == 4 ? qmv_stream_norm_launch_d<DT, 4, 4>(a, g, lc) : qmv_stream_norm_launch_d<DT, 4, 8>(a, g, lc);
     if (bits == 8) return g.d == 4 ? qmv_stream_norm_launch_d<DT, 8, 4>(a, g, lc) : qmv_stream_norm_launch_d<DT, 8, 8>(a, g, lc);
