@@ -48,8 +48,9 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
     const Options& opt = options();
     double best = 1e30;
     uint32_t best_d = 0, best_nb = 0;
+    const bool routed_rows = p.gather == GATHER_CSR || p.gather == GATHER_INDICES;
     for (uint32_t d : {4u, 8u}) {
-        if (d == 8 && rows != 1) continue;
+        if (d == 8 && (rows != 1 || routed_rows)) continue;
         if (opt.qmv_stream_depth && (uint32_t)opt.qmv_stream_depth != d) continue;
         for (uint32_t nb = 1; nb <= 16; nb++) {
             if (opt.qmv_stream_batches && (uint32_t)opt.qmv_stream_batches != nb) continue;

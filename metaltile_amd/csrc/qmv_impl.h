@@ -835,7 +835,7 @@ static int qmv_stream_norm_launch_d(QmvSArgs& a, const QmvSGeom& g, const Launch
 }
 
 template <int DT> int qmv_stream_norm_launch_dtype(QmvSArgs& a, int bits, const QmvSGeom& g, const LaunchCtx& lc) {
-    if (g.mb != 1 || (g.d != 4 && g.d != 8)) return fail(ERR_UNSUPPORTED, "norm + qmv: no kernel instance for this geometry");
+    if (g.mb != 1 || g.d != 4) return fail(ERR_UNSUPPORTED, "norm + qmv: no kernel instance for this geometry");
     if (a.gate_z) {
         if (bits != 4 || g.d != 4) return fail(ERR_UNSUPPORTED, "gated norm + qmv: 4-bit codes, ring of four");
         if constexpr (DT != DT_F32) {
@@ -845,8 +845,8 @@ template <int DT> int qmv_stream_norm_launch_dtype(QmvSArgs& a, int bits, const 
         if (g.tpb > 512) return fail(ERR_UNSUPPORTED, "gated norm + qmv: rows of at most 16384 values");
         return qmv_stream_norm_launch_d<DT, 4, 4, 2, 512>(a, g, lc);
     }
-    if (bits == 4) return g.d == 4 ? qmv_stream_norm_launch_d<DT, 4, 4>(a, g, lc) : qmv_stream_norm_launch_d<DT, 4, 8>(a, g, lc);
-    if (bits == 8) return g.d == 4 ? qmv_stream_norm_launch_d<DT, 8, 4>(a, g, lc) : qmv_stream_norm_launch_d<DT, 8, 8>(a, g, lc);
+    if (bits == 4) return qmv_stream_norm_launch_d<DT, 4, 4>(a, g, lc);   // (the host plans the norm on the ring of four only)
+    if (bits == 8) return qmv_stream_norm_launch_d<DT, 8, 4>(a, g, lc);
     return fail(ERR_UNSUPPORTED, "norm + qmv: 4- or 8-bit codes");
 }
 
@@ -862,7 +862,8 @@ static int qmv_stream_launch_mode(QmvSArgs& a, const QmvSGeom& g, const LaunchCt
             }
         }
     } else if (g.d == 8 && g.mb == 1) {
-        return qmv_stream_launch_sbi<DT, BITS, 1, 8, MODE, 1024>(a, g, lc);
+        // (routed rows keep the ring of four: with eight loads in flight their instances spill)
+        if constexpr (MODE != GATHER_CSR && MODE != GATHER_INDICES) return qmv_stream_launch_sbi<DT, BITS, 1, 8, MODE, 1024>(a, g, lc);
     }
     return fail(ERR_UNSUPPORTED, "stream qmv: no kernel instance for this geometry");
 }
