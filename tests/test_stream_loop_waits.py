@@ -126,3 +126,27 @@ def test_tile_kernels_wait_only_where_written():
             assert not any("scratch_" in l for l in region), f"{name}: scratch memory touched between the MFMAs"
             n += 1
     assert n >= 60
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc is needed to produce the assembly")
+def test_one_row_streaming_instances_keep_their_values_in_registers():
+    """The one-row streaming GEMV is a single pass of loads, dots and a reduction: a value spilled to scratch memory is
+    reloaded in the middle of it, and the compiler's wait for that reload waits for every weight load in flight. Every
+    bf16 instance that serves one or two activation rows - plain, single-expert, routed, with the RMS norm or the gated
+    norm inside - must have a scratch size of zero (the routed instances on a ring of eight loads and the first form of
+    the dealt gate did not, at a cost of up to 2 us per launch; 2-bit codes on three and four rows still spill and are
+    not planned for)."""
+    with tempfile.TemporaryDirectory() as tmp:
+        lines = _assembly("qmv_bf16.hip", os.path.join(tmp, "qmv_bf16.s"))
+    seen = 0
+    for i, l in enumerate(lines):
+        m = re.match(r"^_ZN3mtq17qmv_stream_kernelILi2ELi(\d)ELi(\d)ELi(\d)ELi(\d)ELi(\d+)ELi(\d)ELi(\d)EEEvNS_8QmvSArgsE:", l)
+        if not m:
+            continue
+        bits, mb, depth, mode, maxt, sbi, norm = map(int, m.groups())
+        if mb > 2:
+            continue
+        size = next(int(x.split(":")[1]) for x in lines[i:] if "; ScratchSize:" in x)
+        assert size == 0, f"qmv_stream_kernel<bf16, {bits}-bit, {mb} rows, ring {depth}, mode {mode}, {maxt}, {sbi}, norm {norm}>: {size} bytes of scratch"
+        seen += 1
+    assert seen >= 30
