@@ -226,11 +226,11 @@ int launch_qmv_gated_norm(const QmvParams& p0, const void* gate_z, const void* n
 static int launch_qmv_dot2(const QmvParams& p, const LaunchCtx& lc);
 
 // Routed rows the one-row streaming kernel takes: one row (two when the streaming kernel is asked for by option),
-// fewer than the experts, at most 64 experts (the routing is read by one wave-wide load), 4-bit codes.
+// fewer than the experts, at most 64 experts (the routing is read by one wave-wide load), 4-bit codes, f16 / bf16.
 static bool qmv_few_routed_rows(const QmvParams& p) {
     const uint32_t most = options().qmv_kernel == 2 ? 2u : 1u;
     return (p.gather == GATHER_CSR || p.gather == GATHER_INDICES) && p.T >= 1 && p.T <= most && p.T < p.E && p.E <= 64 && p.bits == 4 &&
-           options().qmv_kernel != 1;
+           p.dtype != DT_F32 && options().qmv_kernel != 1;   // (f32 rows stay where they were: measured for f16 / bf16 only)
 }
 
 int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {
