@@ -51,7 +51,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--layers", type=int, default=8, help="distinct MLP weight sets streamed per step")
     ap.add_argument("--workload", default="qmv",
-                    choices=["qmv", "qkv", "qmm", "batch", "gather", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep"],
+                    choices=["qmv", "qkv", "gated_norm", "qmm", "batch", "gather", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep"],
                     help="qmv is the headline (its line also carries qmm M=512 and the gather as secondary legs); "
                          "qmm / gather report those configurations alone; sweep the bit-width / group-size cells; "
                          "copy runs only the known-size copy kernel (counter calibration); read times a kernel that only reads the "
@@ -507,6 +507,43 @@ def main():
                          "frac": round(achieved / HBM_PEAK_GBS, 4),
                          "traffic": traffic_from_profiles("qkv_fused_bf16_b4_llama_attn"),
                          "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, 1 row>, 3 matrices per launch",
+                         "avg_launch_us_timed_region": round(kern_avg, 3)},
+        })
+        print(json.dumps(out))
+        return
+
+    if a.workload == "gated_norm":
+        # The gated-RMSNorm + out-projection tail of a gated-delta-net layer (the reference's bench shape:
+        # hv 16, dv 128, 2048 output rows), one launch per layer, rotating over `layers` weight sets.
+        hv, dv, N, G = 16, 128, 2048, 64
+        K = hv * dv
+        rng = np.random.default_rng(77)
+        specs, keep = [], []
+        for layer in range(a.layers):
+            c = make_case(7100 + layer, dt, 4, G, 1, N, K)
+            bufs = {"y": GpuBuffer.from_bytes(rng.standard_normal(K).astype(np.float32).tobytes()),
+                    "z": GpuBuffer.from_bytes(m.pack_f32(rng.standard_normal(K).astype(np.float32), dt)),
+                    "norm_weight": GpuBuffer.from_bytes(m.pack_f32((1.0 + 0.1 * rng.standard_normal(dv)).astype(np.float32), dt)),
+                    "eps_buf": GpuBuffer.from_bytes(np.float32(1e-5).tobytes()),
+                    "q_weight": GpuBuffer.from_bytes(c.w.tobytes()), "q_scales": GpuBuffer.from_bytes(c.scales_bytes),
+                    "q_biases": GpuBuffer.from_bytes(c.biases_bytes), "out": GpuBuffer(N * 2)}
+            keep.append(bufs)
+            specs.append(("ffai_gated_rms_norm_qgemv_int4_fast", dt, bufs, {"hv": hv, "dv": dv, "out_dim": N, "group_size": G}))
+        launch_bytes = qmv_bytes(N, K, 4, G, 1, 2) - K * 2 + K * 4 + K * 2 + dv * 2   # y in f32, z, the norm weights
+        runner.flush_slc()
+        runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
+        _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+        kern_avg = chain_us / (a.steps * len(specs))
+        gbs = launch_bytes * len(specs) * a.steps / wall_us / 1e3
+        achieved = launch_bytes / kern_avg / 1e3
+        out.update({
+            "metric": "gated RMSNorm + qmv GB/s (4-bit g64 bf16, hv 16 x dv 128 -> 2048 rows)", "value": round(gbs, 1), "unit": "GB/s",
+            "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
+            "config": {"workload": "ffai_gated_rms_norm_qgemv_int4_fast 4-bit g64 bf16, hv 16, dv 128, out_dim 2048, batch 1",
+                       "launches_per_step": len(specs), "bytes_per_launch": launch_bytes, "device": info["name"] or info["arch"]},
+            "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                         "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, gated norm dealt over four row slots>",
                          "avg_launch_us_timed_region": round(kern_avg, 3)},
         })
         print(json.dumps(out))
