@@ -24,7 +24,9 @@ roofline object. `value`, `ms_per_step` and `steps` describe the qmv region
 only. `--workload sweep` reports the 18 cells of the bit-width / group-size
 sweep (f16, 8192 x 8192, batch 1 and 4); `--workload batch` a decode batch of
 `--rows` rows (default 16) against one large matrix (`--shape`, default the
-128256 x 4096 lm-head), by the exact-dequant kernel name mt_qmm.
+128256 x 4096 lm-head), by the exact-dequant kernel name mt_qmm; `--workload
+qkv` / `gated_norm` the fused one-launch decode pieces (Q + K + V projections;
+gated RMSNorm + out projection at the reference's bench shape).
 
 Prints ONE JSON line on stdout.
 """
