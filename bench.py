@@ -156,6 +156,67 @@ def cpu_baseline(seconds: float):
 
 
 # ---------------------------------------------------------------------------
+# The timed region of every GPU leg
+# ---------------------------------------------------------------------------
+
+WAKE_MS = 40.0       # sustained full-grid load before a leg (the card's clocks settle over ~20 ms of load)
+MIN_WARM_MS = 30.0   # the leg's own chain runs at least this long, untimed, whatever --warmup says
+MFMA_FLOP_PER_CLK_CU = 4096.0   # dense bf16: 2.5 PFLOP/s published = 4096 flop/clk/CU x 256 CUs x 2400 MHz
+
+
+def timed_chain(a, runner, specs, flush=True):
+    """Clock-pinning phase, warm-up, then EXACTLY a.steps timed passes over `specs`.
+
+    Follows the reference's protocol (crates/metaltile-std/src/runner.rs:245-284, 444-475, 635-649): a cache flush
+    of 16 read-modify-write dispatches, then sustained load so that the timed region does not sit inside the clock
+    ramp of a card coming out of idle -- here sized by time, not by count: WAKE_MS of flush dispatches, the
+    --warmup steps, and as many further untimed steps as the chain needs to have run for MIN_WARM_MS. The shader
+    clock is read by a one-wave probe right before and right after the timed region.
+    Returns (wall_us, chain_us, clock dict)."""
+    if flush:
+        runner.flush_slc()
+    wake_ms, wake_n = runner.wake_clocks(WAKE_MS)
+    warm_steps = max(a.warmup, 1)
+    _, _, us = runner.dispatch_chain(specs, repeat=warm_steps, per_kernel=False, stream_events=True)
+    warm_us, last_us, last_steps = us, us, warm_steps
+    for _ in range(8):   # (the first steps of a process run long: estimate the rate afresh from each batch)
+        if warm_us >= MIN_WARM_MS * 1e3:
+            break
+        extra = min(int((MIN_WARM_MS * 1e3 - warm_us) / max(last_us / last_steps, 1e-3)) + 1, 20000)
+        _, _, last_us = runner.dispatch_chain(specs, repeat=extra, per_kernel=False, stream_events=True)
+        last_steps = extra
+        warm_us += last_us
+        warm_steps += extra
+    c0 = runner.clock_probe()
+    _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+    c1 = runner.clock_probe()
+    clock = {"sclk_mhz": round(0.5 * (c0["sclk_mhz"] + c1["sclk_mhz"]), 1),
+             "sclk_mhz_before": round(c0["sclk_mhz"], 1), "sclk_mhz_after": round(c1["sclk_mhz"], 1),
+             "cycle_counter_mhz": round(0.5 * (c0["counter_mhz"] + c1["counter_mhz"]), 2),
+             "method": f"one wave, {c1['valu_ops']} dependent v_add_u32 (4 clk each) against the {c1['wall_clock_mhz']:.0f} MHz "
+                       f"constant-rate counter, {c1['probe_us']:.1f} us, on the launch stream right before / after the timed region",
+             "pinning": {"flush_dispatches": 16, "wake_ms": round(wake_ms, 1), "wake_dispatches": wake_n,
+                         "untimed_steps": warm_steps, "untimed_ms": round(warm_us / 1e3, 2)}}
+    return wall_us, chain_us, clock
+
+
+def hbm_peak_basis(info):
+    """What the HBM peak is divided by: the published figure, with the runtime's own attributes beside it."""
+    b = {"peak_GBps": HBM_PEAK_GBS, "basis": "published MI355X HBM3E peak (8 stacks x 1024 bit x 8 Gb/s)"}
+    if info.get("memory_clock_khz") and info.get("memory_bus_bits"):
+        b["runtime_memory_clock_mhz"] = round(info["memory_clock_khz"] / 1e3, 1)
+        b["runtime_memory_bus_bits"] = info["memory_bus_bits"]
+    return b
+
+
+def mfma_peak_basis(info, clock):
+    cus = info.get("compute_units") or 256
+    return {"peak_TFLOPs": MFMA_BF16_PEAK_TFLOPS,
+            "basis": "published MI355X dense bf16 peak = 4096 flop/clk/CU x 256 CUs x 2400 MHz",
+            "peak_at_measured_clock_TFLOPs": round(MFMA_FLOP_PER_CLK_CU * cus * clock["sclk_mhz"] / 1e6, 1)}
+
+
+# ---------------------------------------------------------------------------
 # GPU legs
 # ---------------------------------------------------------------------------
 
@@ -181,12 +242,7 @@ def leg_qmv(a, runner, info):
     if a.hot:
         specs = specs * a.layers
         step_bytes *= a.layers
-    runner.flush_slc()
-    runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
-    # Timed region: K steps enqueued back to back with no host wait and no
-    # per-launch instrumentation; one pair of HIP events on the stream
-    # brackets it (chain_us), the host clock brackets it too (wall_us).
-    _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+    wall_us, chain_us, clock = timed_chain(a, runner, specs)
     n_per_step = len(specs)
     kern_avg = chain_us / (a.steps * n_per_step)   # average launch duration over the timed region
     # Second pass, same launches: each carries its own event pair, giving the
@@ -216,7 +272,7 @@ def leg_qmv(a, runner, info):
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_from_profiles("qmv_bf16_b4_llama_mlp"),
                      "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, 1 row>", "bytes_per_launch": launch_bytes,
-                     "avg_launch_us_timed_region": round(kern_avg, 3),
+                     "avg_launch_us_timed_region": round(kern_avg, 3), "clock": clock, "peak_basis": hbm_peak_basis(info),
                      "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(st.min_us, 3),
                                            "median_us": round(st.median_us, 3), "p95_us": round(st.p95_us, 3),
                                            "avg_us_by_shape": by_shape, "frac_by_shape": frac_by_shape}},
@@ -239,8 +295,7 @@ def leg_qmm(a, runner, info, M=512):
         keep.append(bufs)
         specs.append(("mt_qmm_mma", dt, bufs, {"k": K, "n": N, "gs_per_row": K // 64}))
     flops = 2.0 * M * N * K
-    runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
-    _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+    wall_us, chain_us, clock = timed_chain(a, runner, specs)
     kern_avg = chain_us / (a.steps * len(specs))
     per, _, _ = runner.dispatch_chain(specs, repeat=min(a.steps, 20), per_kernel=True)
     per = np.array(per)
@@ -258,7 +313,9 @@ def leg_qmm(a, runner, info, M=512):
                      "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": traffic_from_profiles("qmm_bf16_b4_m512") if M == 512 else None,
                      "flop_per_launch": flops, "avg_launch_us_timed_region": round(kern_avg, 3),
-                     "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(float(per.min()), 3)}},
+                     "clock": clock, "peak_basis": mfma_peak_basis(info, clock),
+                     "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "median_us": round(float(np.median(per)), 3),
+                                           "min_us": round(float(per.min()), 3)}},
     }
 
 
@@ -282,8 +339,7 @@ def leg_batch(a, runner, info):
         keep.append(bufs)
         specs.append(("mt_qmm", dt, bufs, {"k": K, "n": N, "gs_per_row": K // G}))
     nbytes = N * K // 2 + 2 * N * (K // G) * 2 + M * K * 2 + M * N * 2
-    runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
-    _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+    wall_us, chain_us, clock = timed_chain(a, runner, specs)
     kern_avg = chain_us / (a.steps * len(specs))
     for bufs in keep:
         for b in bufs.values():
@@ -297,7 +353,7 @@ def leg_batch(a, runner, info):
                    "device": info["name"] or info["arch"]},
         "roofline": {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": nbytes,
-                     "avg_launch_us_timed_region": round(kern_avg, 3)},
+                     "avg_launch_us_timed_region": round(kern_avg, 3), "clock": clock},
     }
 
 
@@ -323,8 +379,7 @@ def leg_gather(a, runner, info):
                 "expert_offsets": GpuBuffer.from_bytes(offsets.astype("<u4").tobytes()), "out": GpuBuffer(T * N * 2)}
         keep.append(bufs)
         specs.append(("mt_moe_gather_qmm_int4", dt, bufs, consts))
-    runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
-    _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+    wall_us, chain_us, clock = timed_chain(a, runner, specs)
     kern_avg = chain_us / (a.steps * len(specs))
     per, _, _ = runner.dispatch_chain(specs, repeat=min(a.steps, 20), per_kernel=True)
     per = np.array(per)
@@ -341,8 +396,9 @@ def leg_gather(a, runner, info):
         "roofline": {"bound": "hbm", "achieved": round(nbytes / kern_avg / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(nbytes / kern_avg / 1e3 / HBM_PEAK_GBS, 4),
                      "traffic": traffic_from_profiles("gather_bf16_b4_e8"), "bytes_per_launch": nbytes,
-                     "avg_launch_us_timed_region": round(kern_avg, 3),
-                     "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(float(per.min()), 3)}},
+                     "avg_launch_us_timed_region": round(kern_avg, 3), "clock": clock, "peak_basis": hbm_peak_basis(info),
+                     "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "median_us": round(float(np.median(per)), 3),
+                                           "min_us": round(float(per.min()), 3)}},
     }
 
 
@@ -365,6 +421,7 @@ def leg_sweep(a, runner, info):
             xb, ob = GpuBuffer.from_bytes(base.x_bytes), GpuBuffer(4 * N * 2)
             copies = [(GpuBuffer.from_bytes(wb), GpuBuffer.from_bytes(sb), GpuBuffer.from_bytes(bb)) for _ in range(sets)]
             for M in (1, 4):
+                runner.wake_clocks(WAKE_MS)
                 nb = qmv_bytes(N, K, bits, G, M, 2)
                 n_samples = max(sets, min(a.steps, 60))
                 us = []
@@ -493,9 +550,7 @@ def main():
             specs.append(("ffai_batched_qkv_qgemv_fast", dt, bufs,
                           {"out_q": Ns[0], "out_k": Ns[1], "out_v": Ns[2], "in_dim": K, "group_size": 64}))
         launch_bytes = sum(qmv_bytes(n, K, 4, 64, 1, 2) for n in Ns) - 2 * K * 2   # x is read once
-        runner.flush_slc()
-        runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
-        _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+        wall_us, chain_us, clock = timed_chain(a, runner, specs)
         kern_avg = chain_us / (a.steps * len(specs))
         gbs = launch_bytes * len(specs) * a.steps / wall_us / 1e3
         achieved = launch_bytes / kern_avg / 1e3
@@ -509,7 +564,7 @@ def main():
                          "frac": round(achieved / HBM_PEAK_GBS, 4),
                          "traffic": traffic_from_profiles("qkv_fused_bf16_b4_llama_attn"),
                          "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, 1 row>, 3 matrices per launch",
-                         "avg_launch_us_timed_region": round(kern_avg, 3)},
+                         "avg_launch_us_timed_region": round(kern_avg, 3), "clock": clock},
         })
         print(json.dumps(out))
         return
@@ -532,9 +587,7 @@ def main():
             keep.append(bufs)
             specs.append(("ffai_gated_rms_norm_qgemv_int4_fast", dt, bufs, {"hv": hv, "dv": dv, "out_dim": N, "group_size": G}))
         launch_bytes = qmv_bytes(N, K, 4, G, 1, 2) - K * 2 + K * 4 + K * 2 + dv * 2   # y in f32, z, the norm weights
-        runner.flush_slc()
-        runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
-        _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+        wall_us, chain_us, clock = timed_chain(a, runner, specs)
         kern_avg = chain_us / (a.steps * len(specs))
         gbs = launch_bytes * len(specs) * a.steps / wall_us / 1e3
         achieved = launch_bytes / kern_avg / 1e3
@@ -546,7 +599,7 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                          "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, gated norm dealt over four row slots>",
-                         "avg_launch_us_timed_region": round(kern_avg, 3)},
+                         "avg_launch_us_timed_region": round(kern_avg, 3), "clock": clock},
         })
         print(json.dumps(out))
         return
@@ -567,8 +620,7 @@ def main():
                     "indices": GpuBuffer.from_bytes(ids.tobytes()), "out": GpuBuffer(T * N * 2)}
             keep.append(bufs)
             specs.append(("mt_moe_gather_qmm_mma_int4", dt, bufs, consts))
-        runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
-        _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+        wall_us, chain_us, clock = timed_chain(a, runner, specs)
         call_avg = chain_us / (a.steps * len(specs))
         flop = 2.0 * T * N * K
         out.update({
@@ -579,7 +631,7 @@ def main():
                        "launches_per_call": 3, "device": info["name"] or info["arch"]},
             "roofline": {"bound": "mfma", "achieved": round(flop / call_avg / 1e6, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(flop / call_avg / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                         "avg_call_us_timed_region": round(call_avg, 3)},
+                         "avg_call_us_timed_region": round(call_avg, 3), "clock": clock},
         })
         print(json.dumps(out))
         return
@@ -603,8 +655,7 @@ def main():
             keep.append(bufs)
             specs.append((f"mt_affine_{a.workload}_int{bits}", dt, bufs, {"group_size": G}))
         nbytes = n * 2 + n * bits // 8 + 2 * (n // G) * 2
-        runner.dispatch_chain(specs, repeat=a.warmup, per_kernel=False)
-        _, wall_us, chain_us = runner.dispatch_chain(specs, repeat=a.steps, per_kernel=False, stream_events=True)
+        wall_us, chain_us, clock = timed_chain(a, runner, specs)
         kern_avg = chain_us / (a.steps * len(specs))
         out.update({
             "metric": f"affine {a.workload} GB/s (4-bit g64 bf16, 14336x4096 elements)",
@@ -614,7 +665,7 @@ def main():
                        "bytes_per_launch": nbytes, "device": info["name"] or info["arch"]},
             "roofline": {"bound": "hbm", "achieved": round(nbytes / kern_avg / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(nbytes / kern_avg / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
-                         "avg_launch_us_timed_region": round(kern_avg, 3)},
+                         "avg_launch_us_timed_region": round(kern_avg, 3), "clock": clock},
         })
         print(json.dumps(out))
         return

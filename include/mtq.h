@@ -361,12 +361,6 @@ typedef struct mtq_dispatch_spec {
 MTQ_API int mtq_dispatch_chain(const mtq_dispatch_spec *specs, int n, int repeat,
                                double *per_kernel_us, double *wall_us, double *stream_us);
 
-/* Plain device-to-device copy kernel of `bytes` (a multiple of 16), enqueued
- * `repeat` times; avg_us (may be NULL) receives the mean GPU duration. No
- * counterpart in the reference: it is the known-size kernel hardware-counter
- * readings are calibrated against. */
-MTQ_API int mtq_copy_kernel(void *dst, const void *src, size_t bytes, int repeat, double *avg_us);
-
 /* ---- planning without a device ------------------------------------------- */
 
 /* What a call WOULD launch, computed by the same routing and geometry code as the call itself, with no device, no
@@ -402,16 +396,6 @@ typedef struct mtq_plan_info {
 MTQ_API int mtq_plan(int op, int dtype, int bits, uint32_t group_size, uint32_t M, uint32_t N, uint32_t K, uint32_t E,
                      uint32_t T, mtq_plan_info *info);
 
-/* Measurement aid, no counterpart in the reference: a kernel that only reads. `repeat` passes over the n_srcs
- * buffers of `bytes` bytes each (bytes % 16 == 0) are enqueued back to back on the library's stream, one launch per
- * buffer, `workgroups` (0 = 2048) workgroups of 256 threads with `in_flight` (1, 2, 4, 8; 0 = 8) 16-byte loads in
- * flight per thread (nontemporal != 0: loads marked as not to be kept in cache); *avg_us is the average launch duration
- * over the run, gaps between launches included. `sink` is 4 bytes of device memory that are (in practice) never
- * written. With more buffers than the last-level cache holds this is the rate at which a launch of that size can
- * stream HBM at all: the ceiling for a weight-streaming kernel of the same size. */
-MTQ_API int mtq_read_kernel(const void *const *srcs, int n_srcs, size_t bytes, int repeat, int workgroups,
-                            int in_flight, int nontemporal, void *sink, double *avg_us);
-
 /* 1 if mtq_dispatch knows `kernel_name`, else 0. */
 MTQ_API int mtq_kernel_supported(const char *kernel_name);
 /* Number of names mtq_dispatch knows, and the i-th of them (NULL past the end). */
@@ -422,9 +406,10 @@ MTQ_API const char *mtq_kernel_name(int i);
  * the reference kernel its selector would pick for M rows. */
 MTQ_API const char *mtq_qmm_for(int dtype, uint32_t m);
 
-/* Replaces GpuRunner::flush_slc (crates/metaltile-std/src/runner.rs:455-475): read-modify-
- * write a scratch region larger than the last-level cache so the next launch
- * starts cold. */
+/* Replaces GpuRunner::flush_slc (crates/metaltile-std/src/runner.rs:444-475): 16 read-modify-
+ * write dispatches (the reference's SLC_FLUSH_DISPATCHES, runner.rs:245) over a scratch region
+ * three times the size of the last-level cache, the last four of which touch every byte of it, so
+ * that the next launch starts cold and follows sustained full-grid load. Waits for the dispatches. */
 MTQ_API int mtq_flush_cache(void);
 
 /* Tuning knobs (no counterpart in the reference). Known names:

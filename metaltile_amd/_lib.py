@@ -35,6 +35,11 @@ class MtqDeviceInfo(C.Structure):
 PLAN_MAX_LAUNCHES = 8
 
 
+class MtqClockSample(C.Structure):
+    _fields_ = [("sclk_mhz", C.c_double), ("counter_mhz", C.c_double), ("probe_us", C.c_double),
+                ("wall_clock_mhz", C.c_double), ("valu_ops", C.c_uint64)]
+
+
 class MtqPlanLaunch(C.Structure):
     _fields_ = [("kernel", C.c_char * 192), ("grid", C.c_uint32 * 3), ("block", C.c_uint32 * 3), ("lds_bytes", C.c_size_t)]
 
@@ -49,7 +54,7 @@ _u32p = C.POINTER(C.c_uint32)
 _dblp = C.POINTER(C.c_double)
 _bufp = C.POINTER(MtqBuf)
 
-# name -> (restype, argtypes); every symbol include/mtq.h declares
+# name -> (restype, argtypes); every symbol include/mtq.h and include/mtq_measure.h declare
 SIGNATURES = {
     "mtq_init": (C.c_int, [C.c_int]),
     "mtq_shutdown": (C.c_int, []),
@@ -96,6 +101,8 @@ SIGNATURES = {
     "mtq_kernel_name": (C.c_char_p, [C.c_int]),
     "mtq_qmm_for": (C.c_char_p, [C.c_int, _u32]),
     "mtq_flush_cache": (C.c_int, []),
+    "mtq_wake_clocks": (C.c_int, [C.c_double, _dblp, C.POINTER(C.c_int)]),
+    "mtq_clock_probe": (C.c_int, [C.POINTER(MtqClockSample)]),
     "mtq_set_option": (C.c_int, [C.c_char_p, C.c_int]),
     "mtq_timed_begin": (C.c_int, []),
     "mtq_timed_last_us": (C.c_int, [_dblp]),

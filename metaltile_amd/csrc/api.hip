@@ -15,6 +15,7 @@
 #include <vector>
 
 #include "../../include/mtq.h"
+#include "../../include/mtq_measure.h"
 #include "mtq_internal.h"
 
 namespace mtq {
@@ -102,6 +103,7 @@ struct State {
     size_t scratch_bytes = 0;
     size_t scratch_held = 0;         // bytes at the front of scratch_buf that the running op keeps for itself
     size_t flush_bytes = 0;
+    uint64_t* probe_buf = nullptr;   // four u64 written by the clock probe
     hipDeviceProp_t prop;
     bool timed_armed = false;    // next typed launch attaches the events
     bool timed_pending = false;  // events attached, not yet read
@@ -143,6 +145,35 @@ __global__ __launch_bounds__(256) void flush_kernel(uint4* p, size_t n) {
         p[i] = v;
     }
 }
+
+// One wave, a chain of dependent adds between two readings of the constant-rate counter: the chain issues one add per
+// four shader clocks whatever else the chip does, so its length on the constant-rate counter gives the shader clock.
+#define MTQ_ADD16 "v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n" \
+                  "v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n" \
+                  "v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n" \
+                  "v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n v_add_u32 %0, %0, %0\n"
+static constexpr uint32_t kProbeAddsPerTurn = 512;
+__global__ __launch_bounds__(64) void clock_probe_kernel(uint64_t* out, uint32_t turns) {
+    uint32_t v = threadIdx.x | 1u;
+    const uint64_t r0 = wall_clock64();
+    const uint64_t c0 = clock64();
+    for (uint32_t i = 0; i < turns; i++) {
+        asm volatile(MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16
+                     MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16
+                     MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16
+                     MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16 MTQ_ADD16
+                     : "+v"(v));
+    }
+    const uint64_t c1 = clock64();
+    const uint64_t r1 = wall_clock64();
+    if (threadIdx.x == 0) {
+        out[0] = r1 - r0;
+        out[1] = c1 - c0;
+        out[2] = (uint64_t)turns * kProbeAddsPerTurn;
+        out[3] = v;
+    }
+}
+#undef MTQ_ADD16
 
 // Reads n 16-byte vectors and keeps nothing: the rate at which a launch of this size can pull bytes out of HBM
 // at all, the ceiling of every weight-streaming kernel of the same size. B loads in flight per thread.
@@ -1057,6 +1088,7 @@ int mtq_shutdown(void) {
     if (!g.ready) return MTQ_OK;
     (void)hipStreamSynchronize(g.stream);
     if (g.flush_buf) (void)hipFree(g.flush_buf);
+    if (g.probe_buf) (void)hipFree(g.probe_buf);
     if (g.scratch_buf) (void)hipFree(g.scratch_buf);
     g.scratch_buf = nullptr;
     g.scratch_bytes = 0;
@@ -1563,19 +1595,75 @@ int mtq_copy_kernel(void* dst, const void* src, size_t bytes, int repeat, double
     return MTQ_OK;
 }
 
-int mtq_flush_cache(void) {
-    int rc = need_ready();
-    if (rc) return rc;
-    const size_t want = (size_t)768 << 20;  // > 256 MB last-level cache + 8 x 4 MB L2
+static int ensure_flush_buf() {
+    const size_t want = (size_t)768 << 20;  // three times the 256 MB last-level cache (+ 8 x 4 MB L2)
     if (!g.flush_buf) {
         MTQ_HIP(hipMalloc(&g.flush_buf, want));
         MTQ_HIP(hipMemsetAsync(g.flush_buf, 0, want, g.stream));
         g.flush_bytes = want;
     }
-    hipLaunchKernelGGL(flush_kernel, dim3(2048), dim3(256), 0, g.stream, (uint4*)g.flush_buf,
-                       g.flush_bytes / sizeof(uint4));
-    MTQ_HIP(hipGetLastError());
+    return MTQ_OK;
+}
+
+// Read-modify-write dispatch number `turn` over a quarter of the flush region: four consecutive turns touch all of it.
+static hipError_t enqueue_flush_quarter(unsigned turn) {
+    const size_t quarter = g.flush_bytes / 4 / sizeof(uint4);
+    hipLaunchKernelGGL(flush_kernel, dim3(2048), dim3(256), 0, g.stream, (uint4*)g.flush_buf + (size_t)(turn % 4) * quarter, quarter);
+    return hipGetLastError();
+}
+
+int mtq_flush_cache(void) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if ((rc = ensure_flush_buf())) return rc;
+    for (unsigned i = 0; i < 16; i++) MTQ_HIP(enqueue_flush_quarter(i));   // the reference's SLC_FLUSH_DISPATCHES
     MTQ_HIP(hipStreamSynchronize(g.stream));
+    return MTQ_OK;
+}
+
+int mtq_wake_clocks(double min_gpu_ms, double* gpu_ms, int* dispatches) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (!(min_gpu_ms >= 0.0) || min_gpu_ms > 2000.0) return fail(ERR_BAD_ARG, "wake: 0 <= min_gpu_ms <= 2000");
+    if ((rc = ensure_flush_buf())) return rc;
+    double total = 0.0;
+    int n = 0;
+    // batches of 16 dispatches, each batch between two events on the stream; the host only waits at a batch's end
+    while (n < 4096 && (n == 0 || total < min_gpu_ms)) {
+        MTQ_HIP(hipEventRecord(g.ev_start, g.stream));
+        for (unsigned i = 0; i < 16; i++, n++) MTQ_HIP(enqueue_flush_quarter((unsigned)n));
+        MTQ_HIP(hipEventRecord(g.ev_stop, g.stream));
+        MTQ_HIP(hipEventSynchronize(g.ev_stop));
+        float ms = 0.f;
+        MTQ_HIP(hipEventElapsedTime(&ms, g.ev_start, g.ev_stop));
+        total += (double)ms;
+    }
+    if (gpu_ms) *gpu_ms = total;
+    if (dispatches) *dispatches = n;
+    return MTQ_OK;
+}
+
+int mtq_clock_probe(mtq_clock_sample* out) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (!out) return fail(ERR_BAD_ARG, "clock probe: out must not be null");
+    if (!g.probe_buf) MTQ_HIP(hipMalloc((void**)&g.probe_buf, 4 * sizeof(uint64_t)));
+    int wall_khz = 0;
+    MTQ_HIP(hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, g.device));
+    if (wall_khz <= 0) return fail(ERR_HIP, "clock probe: the runtime reports no constant-rate counter");
+    const uint32_t turns = 24;   // 12288 adds: about 20 us at 2.4 GHz
+    hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, g.stream, g.probe_buf, turns);
+    MTQ_HIP(hipGetLastError());
+    uint64_t h[4] = {};
+    MTQ_HIP(hipMemcpyAsync(h, g.probe_buf, sizeof(h), hipMemcpyDeviceToHost, g.stream));
+    MTQ_HIP(hipStreamSynchronize(g.stream));
+    if (h[0] == 0) return fail(ERR_HIP, "clock probe: the constant-rate counter did not advance");
+    const double us = (double)h[0] / ((double)wall_khz * 1e-3);
+    out->probe_us = us;
+    out->wall_clock_mhz = (double)wall_khz * 1e-3;
+    out->valu_ops = h[2];
+    out->sclk_mhz = 4.0 * (double)h[2] / us;
+    out->counter_mhz = (double)h[1] / us;
     return MTQ_OK;
 }
 

@@ -252,5 +252,19 @@ class GpuRunner:
     def flush_slc(self) -> None:
         _lib.check(self._lib.mtq_flush_cache())
 
+    def wake_clocks(self, min_gpu_ms: float = 40.0):
+        """Sustained full-grid load for at least `min_gpu_ms` of GPU time (the reference's `wake_dvfs`,
+        crates/metaltile-std/src/runner.rs:280-284, sized by time). Returns (GPU ms spent, dispatches)."""
+        ms, n = C.c_double(0.0), C.c_int(0)
+        _lib.check(self._lib.mtq_wake_clocks(float(min_gpu_ms), C.byref(ms), C.byref(n)))
+        return ms.value, n.value
+
+    def clock_probe(self) -> dict:
+        """One reading of the shader clock behind whatever is queued on the library's stream."""
+        s = _lib.MtqClockSample()
+        _lib.check(self._lib.mtq_clock_probe(C.byref(s)))
+        return {"sclk_mhz": s.sclk_mhz, "counter_mhz": s.counter_mhz, "probe_us": s.probe_us,
+                "wall_clock_mhz": s.wall_clock_mhz, "valu_ops": int(s.valu_ops)}
+
     def sync(self) -> None:
         _lib.check(self._lib.mtq_sync())
