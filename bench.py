@@ -53,11 +53,13 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--layers", type=int, default=8, help="distinct MLP weight sets streamed per step")
     ap.add_argument("--workload", default="qmv",
-                    choices=["qmv", "qkv", "gated_norm", "qmm", "batch", "gather", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep"],
+                    choices=["qmv", "qkv", "gated_norm", "qmm", "batch", "gather", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep", "rows_probe"],
                     help="qmv is the headline (its line also carries qmm M=512 and the gather as secondary legs); "
                          "qmm / gather report those configurations alone; sweep the bit-width / group-size cells; "
                          "copy runs only the known-size copy kernel (counter calibration); read times a kernel that only reads the "
-                         "headline launch's bytes (the ceiling for the qmv kernel)")
+                         "headline launch's bytes (the ceiling for the qmv kernel); rows_probe times a second make of the headline "
+                         "kernel (one wave per four rows, no LDS, no barrier, matrix cores) with parts switched off, beside the shipped "
+                         "kernel and the read-only launch on the same buffers, and prints its per-wave timeline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-secondary", action="store_true", help="qmv workload: skip the qmm M=512 and gather legs")
     ap.add_argument("--m", type=int, default=512, help="qmm workload: activation rows")
@@ -444,6 +446,100 @@ def leg_sweep(a, runner, info):
     return cells, worst
 
 
+def leg_rows_probe(a, runner, info):
+    """The 14336 x 4096 launch of the headline on the same 24 cold operand sets, in one process: mt_qmv on the streaming
+    kernel (LDS-staged scales, dot2) and as shipped (the wave-per-four-rows kernel), a launch that only reads the same
+    weights, and the wave-per-four-rows kernel through its measurement entry point in full, without its arithmetic and
+    with its weight loads only; then that kernel's per-wave timeline (constant-rate counter, 10 ns)."""
+    import numpy as np
+    from metaltile_amd import DType, GpuBuffer
+    from metaltile_amd.synth import make_case, qmv_bytes
+    dt, N, K = DType.BF16, 14336, 4096
+    sets, specs = [], []
+    for i in range(24):
+        c = make_case(5100 + i, dt, 4, 64, 1, N, K)
+        bufs = {"w": GpuBuffer.from_bytes(c.w.tobytes()), "scales": GpuBuffer.from_bytes(c.scales_bytes),
+                "biases": GpuBuffer.from_bytes(c.biases_bytes), "x": GpuBuffer.from_bytes(c.x_bytes), "out": GpuBuffer(N * 2)}
+        sets.append(bufs)
+        specs.append(("mt_qmv", dt, bufs, {"k": K, "gs_per_row": K // 64}))
+    nbytes = qmv_bytes(N, K, 4, 64, 1, 2)
+    tup = [(b["w"], b["scales"], b["biases"], b["x"], b["out"]) for b in sets]
+    reps = max(a.steps, 1)
+    cells = {}
+
+    def cell(name, us):
+        cells[name] = {"us": round(us, 3), "GBps": round(nbytes / us / 1e3, 1), "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+    runner.flush_slc()
+    runner.wake_clocks(WAKE_MS)
+    # three rounds over the five launches, so that every one is timed early and late in the run; the minimum of the
+    # rounds' averages is reported (each average is over reps x 24 back-to-back launches)
+    from metaltile_amd import _lib
+    lib = _lib.load()
+    rounds = {k: [] for k in ("mt_qmv_streaming_kernel", "mt_qmv_shipped", "read_only", "probe_full", "probe_no_arithmetic", "probe_weight_loads_only")}
+    wbytes = N * K // 2 // 16 * 16
+    for _ in range(3):
+        for key, opt in (("mt_qmv_streaming_kernel", 2), ("mt_qmv_shipped", 0)):   # (shipped: the wave-per-four-rows kernel at this shape)
+            _lib.check(lib.mtq_set_option(b"qmv.kernel", opt))
+            try:
+                runner.dispatch_chain(specs, repeat=max(reps // 2, 40), per_kernel=False)
+                _, _, us = runner.dispatch_chain(specs, repeat=reps, per_kernel=False, stream_events=True)
+            finally:
+                lib.mtq_set_option(b"qmv.kernel", 0)
+            rounds[key].append(us / (reps * len(specs)))
+        runner.read_kernel([b["w"] for b in sets], wbytes, repeat=max(reps // 2, 40), workgroups=1792, in_flight=1, nontemporal=True)
+        rounds["read_only"].append(runner.read_kernel([b["w"] for b in sets], wbytes, repeat=reps, workgroups=1792, in_flight=1, nontemporal=True))
+        for mode, key in ((0, "probe_full"), (1, "probe_no_arithmetic"), (2, "probe_weight_loads_only")):
+            runner.probe_qmv_rows(tup, N, mode=mode, repeat=max(reps // 2, 40))
+            rounds[key].append(runner.probe_qmv_rows(tup, N, mode=mode, repeat=reps))
+    for k, v in rounds.items():
+        cell(k, min(v))
+    cells["read_only"]["note"] = f"weights only, {wbytes} B per launch; fraction on the full launch's {nbytes} B for comparison"
+
+    # timeline of one stamped launch inside a chain
+    waves = N // 4
+    timeline = {}
+    names = ["wave started", "all loads issued", "activations in operand order", "first row done", "all rows done", "stored"]
+    for mode, key in ((0, "probe_full"), (1, "probe_no_arithmetic")):
+        st = GpuBuffer(waves * 6 * 8)
+        runner.probe_qmv_rows(tup, N, mode=mode, repeat=40, stamps=st)
+        t = st.read_array(np.uint64).reshape(waves, 6).astype(np.int64)
+        t = (t - t[:, 0].min()) / 100.0   # us on the 100 MHz counter
+        timeline[key] = {nm: {q: round(float(np.quantile(t[:, i], f)), 2) for q, f in (("min", 0.0), ("p10", 0.1), ("median", 0.5), ("p90", 0.9), ("max", 1.0))}
+                         for i, nm in enumerate(names)}
+        done = np.sort(t[:, 5])
+        timeline[key]["waves_stored_by_us"] = {f"{x:.1f}": int(np.searchsorted(done, x)) for x in np.arange(1.0, 9.01, 0.5)}
+        st.free()
+    # parity of the probe's product against the shipped kernel on set 0
+    sets[0]["out"].upload(np.full(N, 0xABAB, np.uint16))
+    runner.probe_qmv_rows(tup[:1], N, mode=0, repeat=1)
+    got = m_unpack(sets[0]["out"].read_bytes())
+    _lib.check(lib.mtq_set_option(b"qmv.kernel", 2))
+    try:
+        runner.dispatch_chain(specs[:1], repeat=1, per_kernel=False)
+    finally:
+        lib.mtq_set_option(b"qmv.kernel", 0)
+    ref = m_unpack(sets[0]["out"].read_bytes())
+    dev = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1.0)))
+    for b in sets:
+        for v in b.values():
+            v.free()
+    c = cells["probe_full"]
+    return {"metric": "qmv GB/s, 14336x4096 4-bit g64 bf16: the wave-per-four-rows kernel with parts switched off, beside the streaming kernel and a read-only launch", "value": c["GBps"], "unit": "GB/s",
+            "ms_per_step": c["us"] / 1e3, "dtype": "bf16",
+            "config": {"workload": "one 14336x4096 launch per step, 24 cold operand sets in rotation; cells = min over 3 rounds of the average launch duration",
+                       "bytes_per_launch": nbytes, "waves": waves, "device": info["name"] or info["arch"]},
+            "roofline": {"bound": "hbm", "achieved": c["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": c["frac"], "traffic": None},
+            "cells": cells, "rounds_us": {k: [round(x, 3) for x in v] for k, v in rounds.items()},
+            "probe_vs_streaming_kernel_max_rel_dev": dev, "timeline_us": timeline}
+
+
+def m_unpack(b):
+    import metaltile_amd as m
+    from metaltile_amd import DType
+    return m.unpack_f32(b, DType.BF16).astype("float64")
+
+
 def main():
     a = parse_args()
     if a.gpus != 1:
@@ -504,6 +600,11 @@ def main():
             out["secondary"] = sec
         if not a.no_cpu:
             out["cpu_baseline"] = cpu_baseline(a.cpu_seconds)
+        print(json.dumps(out))
+        return
+
+    if a.workload == "rows_probe":
+        out.update(leg_rows_probe(a, runner, info))
         print(json.dumps(out))
         return
 

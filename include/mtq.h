@@ -413,7 +413,8 @@ MTQ_API const char *mtq_qmm_for(int dtype, uint32_t m);
 MTQ_API int mtq_flush_cache(void);
 
 /* Tuning knobs (no counterpart in the reference). Known names:
- *   "qmv.kernel"           0 = choose per shape (default), 1 = one-shot kernel, 2 = streaming kernel
+ *   "qmv.kernel"           0 = choose per shape (default), 1 = one-shot kernel, 2 = streaming kernel, 3 = the wave-per-four-rows
+ *                          kernel wherever it applies (one row of 4096 4-bit codes in groups of 64, f16 / bf16)
  *   "qmv.rows_per_thread"  one-shot kernel: 0 = choose per shape, or 4 / 7 / 8
  *   "qmv.stream_depth"     streaming kernel: 0 = choose per shape, or 4 / 8 loads in flight per thread
  *   "qmv.stream_batches"   streaming kernel: 0 = choose per shape, or 1..16 batches per thread

@@ -59,6 +59,20 @@ MTQ_API int mtq_copy_kernel(void *dst, const void *src, size_t bytes, int repeat
 MTQ_API int mtq_read_kernel(const void *const *srcs, int n_srcs, size_t bytes, int repeat, int workgroups,
                             int in_flight, int nontemporal, void *sink, double *avg_us);
 
+/* The wave-per-four-rows make of the headline GEMV (4-bit codes, groups of 64, bf16, rows of K = 4096 codes, N a multiple
+ * of 16) with parts switched off: one wave per four weight rows, every load issued at once, no LDS, no barrier, the dot products
+ * on the matrix cores (metaltile_amd/csrc/qmv_rows.hip, the kernel mtq_qmv runs at this shape). `sets` is n_sets x 5 device pointers (w, scales, biases, x,
+ * out of one operand set, laid out as for mtq_qmv); `repeat` passes over the sets are enqueued back to back and
+ * *avg_us (may be NULL) receives the average launch duration, gaps included. mode 0 computes the product (out is the
+ * same as mtq_qmv's up to the order of the f32 sums), 1 leaves the arithmetic out (loads, the lane reduction and the
+ * stores stay), 2 only loads the weights. With `stamps` (device memory, N / 4 x MTQ_ROWS_PROBE_STAMPS u64, or NULL)
+ * one more launch on set 0 follows in the same chain, in front of n_sets - 1 plain ones, whose waves write readings of
+ * the constant-rate counter: wave started, all loads issued, activations in operand order, first row done, all rows
+ * done, results stored. */
+#define MTQ_ROWS_PROBE_STAMPS 6
+MTQ_API int mtq_probe_qmv_rows(const void *const *sets, int n_sets, uint32_t N, int mode, int repeat, uint64_t *stamps,
+                               double *avg_us);
+
 #ifdef __cplusplus
 }
 #endif

@@ -103,6 +103,7 @@ SIGNATURES = {
     "mtq_flush_cache": (C.c_int, []),
     "mtq_wake_clocks": (C.c_int, [C.c_double, _dblp, C.POINTER(C.c_int)]),
     "mtq_clock_probe": (C.c_int, [C.POINTER(MtqClockSample)]),
+    "mtq_probe_qmv_rows": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, _u32, C.c_int, C.c_int, _vp, _dblp]),
     "mtq_set_option": (C.c_int, [C.c_char_p, C.c_int]),
     "mtq_timed_begin": (C.c_int, []),
     "mtq_timed_last_us": (C.c_int, [_dblp]),

@@ -25,7 +25,9 @@ HIPFLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
 ]
-SOURCES = ["api.hip", "qmv.hip", "qmv_f32.hip", "qmv_f16.hip", "qmv_bf16.hip", "qmv_mfma.hip", "qmv_mfma_f16.hip", "qmv_mfma_bf16.hip", "qmv_mfma_f16_odd.hip", "qmv_mfma_bf16_odd.hip", "qmv_wide.hip", "qmv_wide_gather.hip", "generic.hip", "qmm.hip", "qmm_direct.hip", "qmm_direct_odd.hip", "qmm_dma.hip", "qmm_dma_b8.hip", "qmm_f32.hip", "affine.hip", "norm.hip", "moe.hip", "moe_down.hip", "qvm.hip"]
+# per-source additions: the wave-per-four-rows GEMV keeps its matrix-core results in ordinary vector registers (no accumulator-register copies)
+EXTRA_FLAGS = {"qmv_rows.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+SOURCES = ["api.hip", "qmv.hip", "qmv_f32.hip", "qmv_f16.hip", "qmv_bf16.hip", "qmv_mfma.hip", "qmv_mfma_f16.hip", "qmv_mfma_bf16.hip", "qmv_mfma_f16_odd.hip", "qmv_mfma_bf16_odd.hip", "qmv_wide.hip", "qmv_wide_gather.hip", "generic.hip", "qmm.hip", "qmm_direct.hip", "qmm_direct_odd.hip", "qmm_dma.hip", "qmm_dma_b8.hip", "qmm_f32.hip", "affine.hip", "norm.hip", "moe.hip", "moe_down.hip", "qvm.hip", "qmv_rows.hip"]
 
 
 def _headers():
@@ -46,7 +48,7 @@ def _compile(src, force):
     path = os.path.join(CSRC, src)
     if not force and not _stale(obj, [path] + _headers()):
         return obj, ""
-    cmd = [HIPCC] + HIPFLAGS + (["-x", "hip"] if src.endswith(".cpp") else []) + ["-c", path, "-o", obj]
+    cmd = [HIPCC] + HIPFLAGS + EXTRA_FLAGS.get(src, []) + (["-x", "hip"] if src.endswith(".cpp") else []) + ["-c", path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass does not know the device-only feature flag; that note is noise
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)

@@ -1535,6 +1535,36 @@ int mtq_read_kernel(const void* const* srcs, int n_srcs, size_t bytes, int repea
     return MTQ_OK;
 }
 
+int mtq_probe_qmv_rows(const void* const* sets, int n_sets, uint32_t N, int mode, int repeat, uint64_t* stamps, double* avg_us) {
+    int rc = need_ready();
+    if (rc) return rc;
+    if (!sets || n_sets < 1 || N == 0 || N % 16 || mode < 0 || mode > 2 || repeat < 1)
+        return fail(ERR_BAD_ARG, "rows probe: need operand sets, N a multiple of 16, mode 0..2, repeat >= 1");
+    for (int i = 0; i < 5 * n_sets; i++)
+        if (!sets[i] || (uintptr_t)sets[i] % 16) return fail(ERR_BAD_ARG, "rows probe: null or unaligned operand");
+    LaunchCtx lc;
+    lc.stream = g.stream;
+    auto one = [&](int i, uint64_t* st) {
+        const void* const* p = sets + 5 * i;
+        return launch_rows_probe(p[0], p[1], p[2], p[3], (void*)p[4], N, mode, st, lc);
+    };
+    MTQ_HIP(hipEventRecord(g.ev_start, g.stream));
+    for (int r = 0; r < repeat; r++)
+        for (int i = 0; i < n_sets; i++)
+            if ((rc = one(i, nullptr))) return rc;
+    MTQ_HIP(hipEventRecord(g.ev_stop, g.stream));
+    if (stamps) {
+        if ((rc = one(0, stamps))) return rc;
+        for (int i = 1; i < n_sets; i++)
+            if ((rc = one(i, nullptr))) return rc;
+    }
+    MTQ_HIP(hipStreamSynchronize(g.stream));
+    float ms = 0.f;
+    MTQ_HIP(hipEventElapsedTime(&ms, g.ev_start, g.ev_stop));
+    if (avg_us) *avg_us = (double)ms * 1000.0 / ((double)repeat * n_sets);
+    return MTQ_OK;
+}
+
 int mtq_plan(int op, int dtype, int bits, uint32_t group_size, uint32_t M, uint32_t N, uint32_t K, uint32_t E, uint32_t T,
              mtq_plan_info* info) {
     if (!info) return fail(ERR_BAD_ARG, "plan: info must not be null");
@@ -1690,7 +1720,7 @@ int mtq_set_option(const char* name, int value) {
         return MTQ_OK;
     }
     if (!strcmp(name, "qmv.kernel")) {
-        if (value < 0 || value > 2) return fail(ERR_BAD_ARG, "qmv.kernel must be 0 (auto), 1 (one-shot) or 2 (streaming)");
+        if (value < 0 || value > 3) return fail(ERR_BAD_ARG, "qmv.kernel must be 0 (auto), 1 (one-shot), 2 (streaming) or 3 (wave per four rows)");
         options().qmv_kernel = value;
         return MTQ_OK;
     }

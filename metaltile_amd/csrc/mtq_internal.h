@@ -95,7 +95,7 @@ struct Options {
     int qvm_wgs = 0;              // qvm: target workgroup count (0 = 1024)
     int moe_down_rows = 0;        // fused MoE down projection: rows per workgroup (0 = automatic)
     int qmv_rows_per_thread = 0;  // one-shot kernel: weight rows per thread
-    int qmv_kernel = 0;           // 0 auto, 1 one-shot only, 2 prefer streaming
+    int qmv_kernel = 0;           // 0 auto, 1 one-shot only, 2 prefer streaming, 3 the wave-per-four-rows kernel wherever it applies
     int qmv_stream_depth = 0;     // streaming kernel: ring depth (4 / 8)
     int qmv_stream_batches = 0;   // streaming kernel: batches per thread
     int qmm_splits = 0;           // MFMA qmm: K splits per tile (0 = choose per shape)
@@ -209,6 +209,13 @@ int build_gather_tiles(const uint32_t* route, bool per_row_ids, uint32_t T, uint
 // scratch: qmm_grouped_scratch_bytes(T, E, per_row_ids, 32).
 int launch_qmm_f32_grouped(const QmmParams& p, const uint32_t* route, bool per_row_ids, uint32_t T, uint32_t E, void* scratch,
                            const LaunchCtx& lc);
+
+// One wave per four rows of 4096 4-bit codes in groups of 64, f16 / bf16, one activation row (qmv_rows.hip).
+bool qmv_rows_takes(const QmvParams& p);
+int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc);
+// The same kernel as a measurement aid (bf16; mode 0 / 1 / 2 = full / no arithmetic / weight loads only; stamps may be null).
+int launch_rows_probe(const void* w, const void* s, const void* b, const void* x, void* out, uint32_t N, int mode, uint64_t* stamps,
+                      const LaunchCtx& lc);
 
 // Affine quantise (quantize = true: T[n_elem] -> packed words + scales + biases) and
 // dequantise (packed words + scales + biases -> T[n_elem]) (affine.hip).

@@ -1,0 +1,243 @@
+// qmv_rows_kernel: the 4-bit, group-of-64 GEMV for rows of 4096 codes, f16 / bf16, one activation row (mt_qmv,
+// crates/metaltile-std/src/mlx/quantized.rs:8-308, at the Llama MLP gate / up shape), in a make where nothing is shared
+// between waves. One wave owns four consecutive weight rows and issues every load it will ever make at once
+// (activations, scales, biases, 8 x 16 bytes of weights per lane); there is no LDS staging, no barrier and no loop.
+//   * lane l holds chunks l and 64 + l of a row (16 bytes = 32 codes each: one wave-wide load is 1 KB of one row) and the
+//     64 activations that go with them, in registers, in the order the nibble masks deliver the codes;
+//   * the dot products run on the matrix cores: v_mfma_f32_4x4x4_16b_{bf16,f16} is sixteen independent 4x4x4 products,
+//     and in block b lane 4b + i supplies row i of A (its own activations) and lane 4b + j column j of B (its own codes),
+//     so the diagonal element D[j][j], register j % 4 of lane 4b + j, is that lane's own partial dot product: 7 vector
+//     instructions per weight dword (4 mask-or, 3 shifts) and 2 matrix instructions, against 11 (4 of them double-length
+//     dot2) on the vector ALU;
+//   * a chunk lies in one group, so its eight matrix instructions are followed by one multiply with the group's scale
+//     (each lane loads the two scales of its own chunks); the bias term is sum_g (b_g - MAGIC s_g) * sum(x_g) with lane
+//     g holding the activation sum of group g, exchanged between lanes once per wave;
+//   * four rows are summed over the wave with lane swaps and stored by four lanes.
+// Arithmetic as everywhere in the GEMV family: exact codes times element-type activations, f32 sums, s * dot + b * sum(x).
+// The same source gives the measurement entry point mtq_probe_qmv_rows (include/mtq_measure.h): MODE switches parts off
+// (1: no arithmetic, only loads, reduction and stores; 2: weight loads only), and a stamped launch writes per-wave
+// readings of the constant-rate counter at six points of a wave's life.
+#include <hip/hip_runtime.h>
+
+#include "../../include/mtq.h"
+#include "../../include/mtq_measure.h"
+#include "mtq_device.h"
+#include "mtq_internal.h"
+
+namespace mtq {
+
+typedef uint32_t rp_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned rp_u32x2 __attribute__((ext_vector_type(2)));
+typedef short rp_s16x4 __attribute__((ext_vector_type(4)));
+typedef float rp_f32x4 __attribute__((ext_vector_type(4)));
+
+struct QmvRowsArgs {
+    const rp_u32x4* w;
+    const uint16_t* s;
+    const uint16_t* b;
+    const uint16_t* x;
+    uint16_t* out;
+    uint32_t N;
+    uint64_t* stamps;   // [N / 4][MTQ_ROWS_PROBE_STAMPS] or null
+};
+
+#define RP_KEEP_ORDER() do { asm volatile("" ::: "memory"); __builtin_amdgcn_sched_barrier(0); } while (0)
+
+typedef _Float16 rp_f16x4 __attribute__((ext_vector_type(4)));
+template <int DT> __device__ __forceinline__ rp_f32x4 rp_mfma(rp_u32x2 a, rp_u32x2 b, rp_f32x4 c) {
+    if constexpr (DT == DT_BF16) return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(rp_s16x4, a), __builtin_bit_cast(rp_s16x4, b), c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(rp_f16x4, a), __builtin_bit_cast(rp_f16x4, b), c, 0, 0, 0);
+}
+// a 16-bit element (zero-extended) as f32
+template <int DT> __device__ __forceinline__ float rp_up(uint32_t h) {
+    if constexpr (DT == DT_BF16) return __uint_as_float(h << 16);
+    else return f16_bits_to_f32(h);
+}
+// register (lane % 4) of a block's result: the lane's own product
+__device__ __forceinline__ float rp_diag(rp_f32x4 v, bool b0, bool b1) {
+    const float lo = b0 ? v.y : v.x, hi = b0 ? v.w : v.z;
+    return b1 ? hi : lo;
+}
+__device__ __forceinline__ float rp_swap32_add(float a, float b) {
+    rp_u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r.x) + __uint_as_float(r.y);
+}
+__device__ __forceinline__ float rp_swap16_add(float a, float b) {
+    rp_u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r.x) + __uint_as_float(r.y);
+}
+template <bool TL> __device__ __forceinline__ void rp_stamp(uint64_t (&st)[MTQ_ROWS_PROBE_STAMPS], int i) {
+    if constexpr (TL) {
+        RP_KEEP_ORDER();
+        st[i] = wall_clock64();
+        RP_KEEP_ORDER();
+    }
+}
+
+template <int DT, int MODE, bool TL>
+__global__ __launch_bounds__(256) void qmv_rows_kernel(QmvRowsArgs a) {
+    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
+    constexpr int GPR = 64, C = 128, R = 4;
+    uint64_t st[MTQ_ROWS_PROBE_STAMPS];
+    rp_stamp<TL>(st, 0);                                  // wave started
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t gw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const uint32_t r0 = gw * R;
+    if (r0 >= a.N) return;
+    __builtin_amdgcn_s_setprio(3);
+    uint4 xraw[2][4];
+    if constexpr (MODE != 2) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint4* xv = (const uint4*)(a.x + ((size_t)i * 64 + lane) * 32);
+#pragma unroll
+            for (int v = 0; v < 4; v++) xraw[i][v] = xv[v];
+        }
+    }
+    RP_KEEP_ORDER();
+    uint32_t s0[R], s1[R], bb[R];
+    if constexpr (MODE != 2) {
+        const uint16_t* sp = a.s + (size_t)r0 * GPR + (lane >> 1);
+        const uint16_t* bp = a.b + (size_t)r0 * GPR + lane;
+#pragma unroll
+        for (int r = 0; r < R; r++) { s0[r] = sp[r * GPR]; s1[r] = sp[r * GPR + 32]; bb[r] = bp[r * GPR]; }
+    }
+    RP_KEEP_ORDER();
+    const rp_u32x4* wbase = a.w + (size_t)r0 * C + lane;
+    rp_u32x4 wv[R][2];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        wv[r][0] = __builtin_nontemporal_load(wbase + r * C);
+        wv[r][1] = __builtin_nontemporal_load(wbase + r * C + 64);
+    }
+    RP_KEEP_ORDER();
+    __builtin_amdgcn_s_setprio(0);
+    rp_stamp<TL>(st, 1);                                  // every load issued
+    const bool j0 = lane & 1u, j1 = lane & 2u;
+    uint32_t xp[2][16];
+    float gsum = 0.f;
+    uint32_t kor = DT == DT_BF16 ? 0x43004300u : 0x64006400u;   // (2^7, 2^7) in bf16, (2^10, 2^10) in f16: a code OR-ed into the mantissa is MAGIC + q
+    asm volatile("" : "+v"(kor));
+    if constexpr (MODE == 0) {
+        rp_u32x2 ones;
+        ones.x = ones.y = DT == DT_BF16 ? 0x3F803F80u : 0x3C003C00u;
+        float xsum[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            rp_f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const uint4 v = xraw[i][d];   // activations 8 d .. 8 d + 7 of the chunk; pairs (j, j + 4) match the masks
+                xp[i][4 * d + 0] = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+                xp[i][4 * d + 1] = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+                xp[i][4 * d + 2] = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+                xp[i][4 * d + 3] = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+                rp_u32x2 a0, a1;
+                a0.x = v.x; a0.y = v.y; a1.x = v.z; a1.y = v.w;
+                sacc = rp_mfma<DT>(a0, ones, sacc);
+                sacc = rp_mfma<DT>(a1, ones, sacc);
+            }
+            xsum[i] = rp_diag(sacc, j0, j1);
+        }
+        // group g = chunks 2g and 2g + 1: lanes 2 (g % 32) and + 1 of chunk set g / 32; lane g keeps the sum of group g
+        const uint32_t gl = (lane & 31u) * 8u;
+        const float t0 = __int_as_float(__builtin_amdgcn_ds_bpermute((int)gl, __float_as_int(xsum[0]))) +
+                         __int_as_float(__builtin_amdgcn_ds_bpermute((int)gl + 4, __float_as_int(xsum[0])));
+        const float t1 = __int_as_float(__builtin_amdgcn_ds_bpermute((int)gl, __float_as_int(xsum[1]))) +
+                         __int_as_float(__builtin_amdgcn_ds_bpermute((int)gl + 4, __float_as_int(xsum[1])));
+        gsum = lane < 32 ? t0 : t1;
+    }
+    rp_stamp<TL>(st, 2);                                  // activations in operand order
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if constexpr (MODE == 0) {
+            const float sf0 = rp_up<DT>(s0[r]), sf1 = rp_up<DT>(s1[r]);
+            rp_f32x4 d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    const uint32_t w = wv[r][i][q];
+                    rp_u32x2 b0, b1, a0, a1;
+                    b0.x = (w & 0x000F000Fu) | kor;
+                    b0.y = ((w >> 4) & 0x000F000Fu) | kor;
+                    b1.x = ((w >> 8) & 0x000F000Fu) | kor;
+                    b1.y = ((w >> 12) & 0x000F000Fu) | kor;
+                    a0.x = xp[i][4 * q + 0]; a0.y = xp[i][4 * q + 1];
+                    a1.x = xp[i][4 * q + 2]; a1.y = xp[i][4 * q + 3];
+                    if (i == 0) { d0 = rp_mfma<DT>(a0, b0, d0); d0 = rp_mfma<DT>(a1, b1, d0); }
+                    else { d1 = rp_mfma<DT>(a0, b0, d1); d1 = rp_mfma<DT>(a1, b1, d1); }
+                }
+            }
+            acc[r] = fmaf(sf1, rp_diag(d1, j0, j1), sf0 * rp_diag(d0, j0, j1));
+        } else {
+            uint32_t f = wv[r][0][0] ^ wv[r][0][1] ^ wv[r][0][2] ^ wv[r][0][3] ^ wv[r][1][0] ^ wv[r][1][1] ^ wv[r][1][2] ^ wv[r][1][3];
+            float t = __uint_as_float(f & 0x3FFFFFFFu);
+            if constexpr (MODE == 1)
+                t += rp_up<DT>(s0[r]) + rp_up<DT>(s1[r]) + rp_up<DT>(bb[r]) + __uint_as_float(xraw[0][0].x << 16);
+            acc[r] = t;
+        }
+        if (r == 0) rp_stamp<TL>(st, 3);                  // first row done
+    }
+    if constexpr (MODE == 0) {
+        // (b - MAGIC s) of group `lane` times that group's activation sum; the group's scale is held by lane 2 (lane % 32)
+        const uint32_t src = (lane & 31u) * 8u;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const float sa = rp_up<DT>((uint32_t)__builtin_amdgcn_ds_bpermute((int)src, (int)s0[r]));
+            const float sb = rp_up<DT>((uint32_t)__builtin_amdgcn_ds_bpermute((int)src, (int)s1[r]));
+            acc[r] = fmaf(rp_up<DT>(bb[r]) - MAGIC * (lane < 32 ? sa : sb), gsum, acc[r]);
+        }
+    }
+    rp_stamp<TL>(st, 4);                                  // all rows done
+    float tot = rp_swap16_add(rp_swap32_add(acc[0], acc[1]), rp_swap32_add(acc[2], acc[3]));
+    tot += dpp_f32<0xB1>(tot);
+    tot += dpp_f32<0x4E>(tot);
+    tot += dpp_f32<0x141>(tot);
+    tot += dpp_f32<0x140>(tot);
+    // 16-lane row r of the wave now holds the total of row {0, 2, 1, 3}[r]
+    const uint32_t slot = ((lane >> 4) & 1u) * 2u + (lane >> 5);
+    if ((lane & 15u) == 0) a.out[r0 + slot] = f32_to_elem_bits<DT>(tot);
+    rp_stamp<TL>(st, 5);                                  // stored
+    if constexpr (TL) {
+        if (lane == 0)
+            for (int i = 0; i < MTQ_ROWS_PROBE_STAMPS; i++) a.stamps[(size_t)gw * MTQ_ROWS_PROBE_STAMPS + i] = st[i];
+    }
+}
+
+template <int DT> static const void* qmv_rows_fn(int mode, bool tl) {
+    switch (mode) {
+        case 0: return tl ? (const void*)qmv_rows_kernel<DT, 0, true> : (const void*)qmv_rows_kernel<DT, 0, false>;
+        case 1: return tl ? (const void*)qmv_rows_kernel<DT, 1, true> : (const void*)qmv_rows_kernel<DT, 1, false>;
+        default: return tl ? (const void*)qmv_rows_kernel<DT, 2, true> : (const void*)qmv_rows_kernel<DT, 2, false>;
+    }
+}
+
+static int launch_rows(int dtype, const void* w, const void* s, const void* b, const void* x, void* out, uint32_t N, int mode,
+                       uint64_t* stamps, const LaunchCtx& lc) {
+    QmvRowsArgs a{(const rp_u32x4*)w, (const uint16_t*)s, (const uint16_t*)b, (const uint16_t*)x, (uint16_t*)out, N, stamps};
+    void* args[] = {&a};
+    const void* fn = dtype == DT_BF16 ? qmv_rows_fn<DT_BF16>(mode, stamps != nullptr) : qmv_rows_fn<DT_F16>(mode, stamps != nullptr);
+    hipError_t e = launch_kernel(fn, dim3((N + 15) / 16), dim3(256), args, 0, lc);
+    if (e != hipSuccess) return hip_fail(e, "qmv rows kernel launch");
+    return ERR_OK;
+}
+
+bool qmv_rows_takes(const QmvParams& p) {
+    return p.gather == GATHER_NONE && p.M == 1 && p.bits == 4 && p.group_size == 64 && p.K == 4096 && p.N % 4 == 0 && p.N >= 4 &&
+           (p.dtype == DT_F16 || p.dtype == DT_BF16) && (uintptr_t)p.w % 16 == 0 && (uintptr_t)p.x % 16 == 0 &&
+           (uintptr_t)p.scales % 2 == 0 && (uintptr_t)p.biases % 2 == 0 && (uintptr_t)p.out % 2 == 0;
+}
+
+int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
+    if (!qmv_rows_takes(p)) return fail(ERR_UNSUPPORTED, "qmv rows kernel: one row of 4096 4-bit codes in groups of 64, f16 / bf16, N % 4 == 0");
+    return launch_rows(p.dtype, p.w, p.scales, p.biases, p.x, p.out, p.N, 0, nullptr, lc);
+}
+
+int launch_rows_probe(const void* w, const void* s, const void* b, const void* x, void* out, uint32_t N, int mode, uint64_t* stamps,
+                      const LaunchCtx& lc) {
+    return launch_rows(DT_BF16, w, s, b, x, out, N, mode, stamps, lc);
+}
+
+}  // namespace mtq

@@ -266,5 +266,14 @@ class GpuRunner:
         return {"sclk_mhz": s.sclk_mhz, "counter_mhz": s.counter_mhz, "probe_us": s.probe_us,
                 "wall_clock_mhz": s.wall_clock_mhz, "valu_ops": int(s.valu_ops)}
 
+    def probe_qmv_rows(self, sets, N: int, mode: int = 0, repeat: int = 1, stamps: Optional[GpuBuffer] = None) -> float:
+        """Average launch duration (us) of the wave-per-four-rows make of the 4-bit g64 bf16 GEMV (K = 4096) over
+        `sets` = [(w, scales, biases, x, out) GpuBuffers, ...], enqueued back to back `repeat` times."""
+        flat = [b.ptr for s in sets for b in s]
+        arr = (C.c_void_p * len(flat))(*flat)
+        us = C.c_double(0.0)
+        _lib.check(self._lib.mtq_probe_qmv_rows(arr, len(sets), int(N), int(mode), int(repeat), stamps.ptr if stamps else None, C.byref(us)))
+        return us.value
+
     def sync(self) -> None:
         _lib.check(self._lib.mtq_sync())

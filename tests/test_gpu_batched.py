@@ -11,6 +11,7 @@ kernel serves, must be bit-equal to the single-matrix launch on the same operand
 import numpy as np
 import pytest
 
+from metaltile_amd import _lib
 from metaltile_amd import DType, GpuBuffer, ops, unpack_f32
 from metaltile_amd.synth import make_case
 from tests.parity import rel_err
@@ -61,8 +62,15 @@ def test_batched_matches_single_and_oracle(oracle, dt, bits, G, K, Ns):
         assert np.isfinite(got).all()
         assert rel_err(got, _expected(oracle, c, cases[0].x_f, dt)) <= TOL[dt]
         if bits in (2, 4, 8):
+            # the batched launch is the streaming kernel: the single launch on that kernel (a row of 4096 4-bit codes
+            # would otherwise take the wave-per-four-rows kernel, whose f32 sums meet in another order)
             single = GpuBuffer(N * esz)
-            ops.qmv(dt, bits, G, d[0], d[1], d[2], x, single, 1, N, K)
+            lib = _lib.load()
+            assert lib.mtq_set_option(b"qmv.kernel", 2) == 0
+            try:
+                ops.qmv(dt, bits, G, d[0], d[1], d[2], x, single, 1, N, K)
+            finally:
+                lib.mtq_set_option(b"qmv.kernel", 0)
             assert single.read_bytes(N * esz) == raw, "batched launch must reproduce the single launch bit for bit"
             single.free()
     for b in [x] + outs + [t for d in dev for t in d]:

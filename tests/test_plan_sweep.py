@@ -119,7 +119,12 @@ def test_benchmark_configurations_are_routed_as_documented():
         return [l[0] for l in launches], launches
 
     ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 14336, 4096)
-    assert "qmv_stream_kernel<2, 4, 1," in ks[0] and ls[0][1][0] * 8 == 14336   # 8 rows per workgroup
+    assert "qmv_rows_kernel<2, 0, false>" in ks[0] and ls[0][1][0] * 16 == 14336   # 4 waves x 4 rows per workgroup
+    ks, _ = kernels("qmv", DType.F16, 4, 64, 1, 4100, 4096)
+    assert "qmv_rows_kernel<1, 0, false>" in ks[0]
+    for args in ((DType.BF16, 4, 64, 1, 4098, 4096), (DType.BF16, 4, 32, 1, 4096, 4096), (DType.BF16, 4, 64, 2, 4096, 4096),
+                 (DType.BF16, 8, 64, 1, 4096, 4096), (DType.BF16, 4, 64, 1, 512, 4096)):
+        assert "qmv_rows_kernel" not in kernels("qmv", *args)[0][0]          # what that kernel does not take
     ks, _ = kernels("qmv", DType.BF16, 4, 64, 1, 4096, 14336)
     assert "qmv_stream_kernel<2, 4, 1," in ks[0]
     ks, _ = kernels("qmv", DType.F32, 4, 64, 1, 4096, 4096)
