@@ -203,7 +203,8 @@ MTQ_API int mtq_qmv_batched(int dtype, int bits, uint32_t group_size, int n_mats
  * row m of every output the GEMV of activation row m, 1..4 matrices. Replaces ffai_batched_qkv_qmm_fast
  * (crates/metaltile-std/src/ffai/batched_qkv_qmm.rs:49-68) and ffai_batched_4_qmm_fast
  * (crates/metaltile-std/src/ffai/batched_4_qmm.rs:61-85), whose row count is the grid's second dimension (under those
- * names here: the rows `x` holds) and whose constraints (K % 512 == 0, N % 8 == 0, group 64, 4-bit) are not required.
+ * names here too when mtq_dispatch is given a grid other than the all-ones placeholder, and `x` may then hold more rows;
+ * without one: the rows `x` holds) and whose constraints (K % 512 == 0, N % 8 == 0, group 64, 4-bit) are not required.
  * One mtq_qmm per matrix, in order, with mtq_qmm's routing and arithmetic: outputs are bit-equal to single calls.
  * Dispatched under the reference names the matrices run on the qmv family at every M, which keeps those kernels'
  * exact-dequant arithmetic (as the `mt_qmm*` names do). w / scales / biases / outs / N are HOST arrays of device pointers / row counts. */
@@ -323,7 +324,9 @@ MTQ_API int mtq_dequant_gather(int dtype, int bits, uint32_t group_size, const v
  * parameters in signature order, `consts` its constexprs in signature order
  * (crates/metaltile-std/src/run_kernel.rs:183-188, 210-234). grid/tpg describe
  * the Metal launch and are accepted for compatibility; the HIP launch is
- * derived from name, dtype, constexprs and buffer lengths. Buffers shorter
+ * derived from name, dtype, constexprs and buffer lengths (one exception: the
+ * ffai_batched_*_qmm_fast names take their row count from grid[1], as the
+ * reference does). Buffers shorter
  * than the op needs fail with MTQ_ERR_BUFFER_SIZE. Blocks until the kernel has
  * finished; *elapsed_us (may be NULL) receives its GPU duration. An unknown
  * name fails with MTQ_ERR_UNKNOWN_KERNEL so a caller can fall back. */

@@ -740,7 +740,7 @@ static int need_bytes(const mtq_buf& b, const char* param, uint64_t expected) {
 // Validates the bound buffers against the shape implied by (name, dtype,
 // constexprs, buffer lengths) and enqueues the kernel.
 static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, int n_bufs,
-                         const uint32_t* consts, int n_consts, const LaunchCtx& lc) {
+                         const uint32_t* consts, int n_consts, const LaunchCtx& lc, const uint32_t* grid = nullptr) {
     if (dtype != DT_F32 && dtype != DT_F16 && dtype != DT_BF16) return fail(ERR_BAD_ARG, "dtype must be MTQ_F32, MTQ_F16 or MTQ_BF16");
     if (n_bufs != d.n_bufs || n_consts != d.n_consts || !bufs || !consts) {
         char m[200];
@@ -943,12 +943,21 @@ static int dispatch_desc(const KernelDesc& d, int dtype, const mtq_buf* bufs, in
         }
         case F_BQKV_QMM:
         case F_B4_QMM: {
-            // the reference takes the number of rows from the grid; here it is what x holds
+            // The reference takes the number of rows from the grid's second dimension (its grid is [max_out / 8, M, 1],
+            // crates/metaltile-std/src/ffai/batched_qkv_qmm.rs:46-70): a grid that is more than the all-ones placeholder
+            // decides, and x may then be longer than M rows (a buffer allocated for the longest sequence). Without one
+            // the row count is what x holds.
             const int n = d.fam == F_BQKV_QMM ? 3 : 4;
             const uint32_t K = consts[n], G = consts[n + 1];
             if (K == 0 || G == 0 || K % G) return fail(ERR_SHAPE, "group_size must divide in_dim");
-            if (bufs[0].bytes % ((uint64_t)K * sz)) return fail(ERR_BUFFER_SIZE, "'x' must hold whole rows of in_dim");
-            const uint64_t M = bufs[0].bytes / ((uint64_t)K * sz);
+            uint64_t M;
+            if (grid && grid[1] >= 1 && (grid[0] > 1 || grid[1] > 1)) {
+                M = grid[1];
+                MTQ_NEED(bufs[0], "x", M * K * sz);
+            } else {
+                if (bufs[0].bytes % ((uint64_t)K * sz)) return fail(ERR_BUFFER_SIZE, "'x' must hold whole rows of in_dim");
+                M = bufs[0].bytes / ((uint64_t)K * sz);
+            }
             if (M > 0xFFFFFFFFull) return fail(ERR_SHAPE, "too many rows");
             const void *w[4], *s[4], *b[4];
             void* outs[4];
@@ -1387,7 +1396,7 @@ int mtq_dispatch(const char* kernel_name, int dtype, const mtq_buf* bufs, int n_
     lc.stream = g.stream;
     lc.start = g.ev_start;
     lc.stop = g.ev_stop;
-    rc = dispatch_desc(*d, dtype, bufs, n_bufs, consts, n_consts, lc);
+    rc = dispatch_desc(*d, dtype, bufs, n_bufs, consts, n_consts, lc, grid);
     if (rc) return rc;
     MTQ_HIP(hipStreamSynchronize(g.stream));
     if (elapsed_us) {
@@ -1412,7 +1421,7 @@ int mtq_measure(const char* kernel_name, int dtype, const mtq_buf* bufs, int n_b
     LaunchCtx plain;
     plain.stream = g.stream;
     for (int i = 0; i < warmup; i++) {
-        rc = dispatch_desc(*d, dtype, bufs, n_bufs, consts, n_consts, plain);
+        rc = dispatch_desc(*d, dtype, bufs, n_bufs, consts, n_consts, plain, grid);
         if (rc) return rc;
     }
     MTQ_HIP(hipStreamSynchronize(g.stream));
@@ -1420,7 +1429,7 @@ int mtq_measure(const char* kernel_name, int dtype, const mtq_buf* bufs, int n_b
     timed.start = g.ev_start;
     timed.stop = g.ev_stop;
     for (int i = 0; i < iters; i++) {
-        rc = dispatch_desc(*d, dtype, bufs, n_bufs, consts, n_consts, timed);
+        rc = dispatch_desc(*d, dtype, bufs, n_bufs, consts, n_consts, timed, grid);
         if (rc) return rc;
         MTQ_HIP(hipEventSynchronize(g.ev_stop));
         float ms = 0.f;

@@ -229,8 +229,12 @@ static int launch_qmv_dot2(const QmvParams& p, const LaunchCtx& lc);
 // fewer than the experts, at most 64 experts (the routing is read by one wave-wide load), 4-bit codes, f16 / bf16.
 static bool qmv_few_routed_rows(const QmvParams& p) {
     const uint32_t most = options().qmv_kernel == 2 ? 2u : 1u;
+    // (and only rows the streaming kernel can tile: whole waves of 16-byte chunks, scales in whole 4-vectors, 16-byte aligned;
+    // other rows keep the gather instances of the one-shot and matrix-core kernels)
+    const bool tiles = p.group_size && p.K % 2048 == 0 && p.K % p.group_size == 0 && (p.K / p.group_size) % 4 == 0 &&
+                       (uintptr_t)p.scales % 16 == 0 && (uintptr_t)p.biases % 16 == 0;
     return (p.gather == GATHER_CSR || p.gather == GATHER_INDICES) && p.T >= 1 && p.T <= most && p.T < p.E && p.E <= 64 && p.bits == 4 &&
-           p.dtype != DT_F32 && options().qmv_kernel != 1;   // (f32 rows stay where they were: measured for f16 / bf16 only)
+           p.dtype != DT_F32 && options().qmv_kernel != 1 && tiles;   // (f32 rows stay where they were: measured for f16 / bf16 only)
 }
 
 int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {

@@ -72,7 +72,7 @@ static bool plan_wide(const QmmParams& p, QmvWPlan& pl) {
     if ((uint64_t)p.M * p.N >= (1ull << 31) || (uint64_t)p.N * p.K / 2 >= (1ull << 32)) return false;
     const uint32_t cus = (uint32_t)wide_cus();
     const uint32_t per_turn = wide_bytes_per_turn(G);
-    const uint32_t max_turns = (160u * 1024u) / per_turn;
+    const uint32_t max_turns = (160u * 1024u - 64u) / per_turn;   // (64 bytes left for the kernel's statically allocated row counter)
     const uint32_t turns = p.K / 512u;
     uint32_t ks = (turns + max_turns - 1) / max_turns;
     const uint32_t tps = (turns + ks - 1) / ks;
@@ -160,7 +160,7 @@ int launch_qmv_wide_gather(const QmvParams& p, const LaunchCtx& lc) {
     if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16) return fail(ERR_UNSUPPORTED, "wide gather: alignment");
     if ((uint64_t)p.N * p.K / 2 >= (1ull << 32) || (uint64_t)p.E >= 65536) return fail(ERR_UNSUPPORTED, "wide gather: size");
     const uint32_t per_turn = wide_bytes_per_turn(G), turns = p.K / 512u;
-    if (turns > (160u * 1024u) / per_turn) return fail(ERR_UNSUPPORTED, "wide gather: rows too long for one slice");
+    if (turns > (160u * 1024u - 64u) / per_turn) return fail(ERR_UNSUPPORTED, "wide gather: rows too long for one slice");
     QmvWPlan pl;
     pl.kslice = p.K;
     pl.ksplit = 1;
@@ -169,7 +169,8 @@ int launch_qmv_wide_gather(const QmvParams& p, const LaunchCtx& lc) {
     const uint32_t cus = (uint32_t)wide_cus(), want = cus / e_eff > 0 ? cus / e_eff : 1u;
     if (!wide_geometry(G, turns, (p.N + 15u) / 16u, want, pl)) return fail(ERR_UNSUPPORTED, "wide gather: geometry");
     if (p.gather == GATHER_INDICES) pl.lds += (size_t)p.T * 4;
-    if (pl.lds > 160 * 1024) return fail(ERR_UNSUPPORTED, "wide gather: the row list does not fit LDS");
+    // (the kernel's statically allocated row counter shares the 160 KB with the dynamic part)
+    if (pl.lds + 64 > 160 * 1024) return fail(ERR_UNSUPPORTED, "wide gather: the row list does not fit LDS");
     const void* fn = qmv_wide_gather_pick(p.dtype, p.gather, pl.nb, pl.sets);
     if (!fn) return fail(ERR_UNSUPPORTED, "wide gather: geometry not built");
     QmvWArgs a;

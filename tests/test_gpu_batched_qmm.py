@@ -71,6 +71,32 @@ def test_reference_like_4way_qmm(ctx, oracle, dt):
         assert got.size == exp.size and np.any(got != 0.0)
         assert _ref_err(got, exp.reshape(-1)) <= REF_TOL[dt], tag
 
+@pytest.mark.parametrize("dt", [DType.F16, DType.BF16], ids=lambda d: d.name)
+def test_row_count_comes_from_the_grid(ctx, oracle, dt):
+    """The reference takes M from the grid's second dimension (crates/metaltile-std/src/ffai/batched_qkv_qmm.rs:46-70): a
+    caller that binds buffers allocated for a longer sequence gets exactly grid[1] rows; the rows past them keep their
+    bytes. With the all-ones placeholder grid the row count is what x holds."""
+    K, G, Ns, M, cap = 512, 64, (16, 8, 8), 3, 7
+    x, mats = _ref_mats(oracle, dt, cap, K, G, Ns, (0x22, 0x33, 0x44))
+    bufs = {"x": pack_f32(x, dt)}
+    consts = {"in_dim": K, "group_size": G}
+    for tag, (w, s, b, _), N in zip("qkv", mats, Ns):
+        bufs[f"w_{tag}"], bufs[f"scales_{tag}"], bufs[f"biases_{tag}"] = w.tobytes(), pack_f32(s, dt), pack_f32(b, dt)
+        bufs[f"{tag}_buf"] = b"\xab" * (cap * N * dt.size_bytes)
+        consts[f"out_{tag}"] = N
+    res = ctx.dispatch_with_grid("ffai_batched_qkv_qmm_fast", dt, bufs, consts, (-(-max(Ns) // 8), M, 3), (64, 1, 1))
+    for tag, (_, _, _, exp), N in zip("qkv", mats, Ns):
+        raw = res.outputs[f"{tag}_buf"]
+        assert raw[M * N * dt.size_bytes:] == b"\xab" * ((cap - M) * N * dt.size_bytes), "rows past grid[1] must stay untouched"
+        got = unpack_f32(raw[:M * N * dt.size_bytes], dt)
+        assert _ref_err(got, exp[:M].reshape(-1)) <= REF_TOL[dt], tag
+    res = ctx.dispatch_with_grid("ffai_batched_qkv_qmm_fast", dt, bufs, consts, (1, 1, 1), (64, 1, 1))   # no grid: all 7 rows
+    for tag, (_, _, _, exp) in zip("qkv", mats):
+        assert _ref_err(unpack_f32(res.outputs[f"{tag}_buf"], dt), exp.reshape(-1)) <= REF_TOL[dt], tag
+    with pytest.raises(MtqError) as e:   # more rows asked for than x holds
+        ctx.dispatch_with_grid("ffai_batched_qkv_qmm_fast", dt, bufs, consts, (2, cap + 1, 3), (64, 1, 1))
+    assert e.value.code == -4
+
 
 @pytest.mark.parametrize("dt", [DType.F32, DType.F16, DType.BF16], ids=lambda d: d.name)
 @pytest.mark.parametrize("M,K,Ns", [(2, 2048, (2048, 512, 512)), (8, 4096, (4096, 1024, 1024)), (37, 1024, (520, 8, 136)),

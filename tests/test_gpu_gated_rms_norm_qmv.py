@@ -59,7 +59,8 @@ def _case(oracle, dt, hv, dv, N, G, seed):
 @pytest.mark.parametrize("dt", [DType.F32, DType.F16, DType.BF16], ids=lambda d: d.name)
 @pytest.mark.parametrize("hv,dv,N,G", [(16, 128, 2048, 64), (32, 128, 4096, 64), (4, 128, 512, 64), (1, 512, 64, 64), (3, 96, 40, 32),
                                        (5, 128, 1000, 128), (64, 128, 333, 64), (2, 36, 8, 8), (16, 256, 4096, 64), (1, 2048, 100, 64),
-                                       (64, 32, 64, 32), (8, 512, 256, 128), (3, 2048, 17, 64), (32, 1024, 24, 64)])
+                                       (64, 32, 64, 32), (8, 512, 256, 128), (3, 2048, 17, 64), (32, 1024, 24, 64),
+                                       (8, 2048, 48, 64), (80, 128, 40, 64), (112, 128, 24, 64)])   # K = 16384 (512 threads), 10240, 14336
 def test_shapes(oracle, dt, hv, dv, N, G):
     print(f"[case] gated_rms_norm_qmv {dt.name} hv{hv} dv{dv} g{G} N{N}", flush=True)
     K, eps = hv * dv, np.float32(1e-5)

@@ -148,3 +148,33 @@ def test_two_rows_on_the_one_row_kernel(oracle, dt, prefer_streaming):
         out.free(); r.free()
     for buf in (w, s, b, x):
         buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("K", [1024, 1536, 2048])
+def test_one_routed_row_on_rows_the_streaming_kernel_cannot_tile(oracle, dt, K):
+    """One routed row: rows of whole waves of 16-byte chunks (K = 2048) take the one-row streaming kernel; shorter or
+    ragged rows (K = 1024, 1536) must land on a gather instance of the tiled kernels, not on the one-wave-per-output
+    fallback, and give the same answer either way."""
+    bits, G, N, E, T = 4, 64, 264, 8, 1
+    c = make_case(8700 + K, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    for view in ("csr", "indices"):
+        rc, launches, _, _ = ops.plan("gather_" + view, dt, bits, G, 1, N, K, E=E, T=T)
+        assert rc == 0
+        name = launches[0][0]
+        assert "generic" not in name, name
+        assert ("qmv_stream_kernel" in name) == (K == 2048), name
+    ids = np.array([5], dtype="<u4")
+    exp = oracle.round_through(oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=ids, f64=True, threads=8)
+                               .astype(np.float32), ODT[dt])
+    out, r = GpuBuffer(T * N * dt.size_bytes), GpuBuffer.from_bytes(ids.tobytes())
+    ops.gather_qmv_indices(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+    assert rel_err(unpack_f32(out.read_bytes(), dt), exp) <= 1e-2
+    off = GpuBuffer.from_bytes(np.array([0, 0, 0, 0, 0, 0, 1, 1, 1], dtype="<u4").tobytes())   # the row belongs to expert 5
+    out.zero()
+    ops.gather_qmv_csr(dt, bits, G, x, w, s, b, off, out, T, N, K, E)
+    assert rel_err(unpack_f32(out.read_bytes(), dt), exp) <= 1e-2
+    for buf in (w, s, b, x, out, r, off):
+        buf.free()
