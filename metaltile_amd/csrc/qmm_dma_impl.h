@@ -2,6 +2,7 @@
 // (see qmm_direct.hip for the tiling; this header only differs in how the operands travel).
 #pragma once
 #include "qmm_direct_impl.h"
+#include "vm_schedule.h"
 
 #include <type_traits>
 
@@ -61,6 +62,50 @@ template <int DT> __device__ __forceinline__ void qm_dequant4_b4(uint32_t e, uin
     d1 = pack2<DT>(fmaf(fe.y, s512, b), fmaf(fo.y, s512, b));
 }
 
+// The loop's vector-memory schedule and the waits that follow from it. Per iteration `it` a wave issues, in this order,
+//   ring of three or more tiles: the weights of iteration it + WSN (NWL loads), its piece of the next scale window (NSB),
+//                                its share of tile it + NBUF - 1 (IPW load-to-LDS instructions);
+//   ring of two:                 the window piece, its share of tile it + 1, then the weights of iteration it + WSN;
+// it needs the weights of iteration it + 1 before it converts them (next_weights) and its share of tile it + 1 before
+// the iteration's barrier (next_tile). The prologue issues the first WSN weight sets, then the first NBUF - 1 tiles,
+// and needs tile 0 and weight set 0 (first). holds() replays that order and checks every N against it.
+template <int NBUF, int WSN, int IPW, int NWL, int NSB> struct QmmDmaWaits {
+    static constexpr int next_weights = NBUF == 2 ? 2 * IPW + 2 * NWL + 2 * NSB : WSN * (IPW + NSB) + (WSN - 1) * NWL;
+    static constexpr int next_tile = NBUF == 2 ? NWL : NBUF == 3 ? IPW + NWL + NSB : (NBUF - 2) * (IPW + NWL) - 1;
+    static constexpr int first = (NBUF - 2) * IPW;
+    enum { W = 1, X = 2, S = 3 };
+    static constexpr bool holds() {
+        VmQueue q;
+        for (int i = 0; i < WSN; i++) q.issue(vm_tag(W, i), NWL);
+        for (int i = 0; i < NBUF - 1; i++) q.issue(vm_tag(X, i), IPW);
+        q.wait(first);
+        if (!q.landed(vm_tag(X, 0)) || !q.landed(vm_tag(W, 0))) return false;
+        for (int it = 0; it < 4 * (WSN > NBUF ? WSN : NBUF) + 4; it++) {
+            if (NBUF == 2) {
+                q.issue(vm_tag(S, it), NSB);
+                q.issue(vm_tag(X, it + 1), IPW);
+                q.issue(vm_tag(W, it + WSN), NWL);
+            } else {
+                q.issue(vm_tag(W, it + WSN), NWL);
+                q.issue(vm_tag(S, it), NSB);
+                q.issue(vm_tag(X, it + NBUF - 1), IPW);
+            }
+            const int w_exact = q.younger_than(vm_tag(W, it + 1)), x_exact = q.younger_than(vm_tag(X, it + 1));
+            q.wait(next_weights);
+            if (!q.landed(vm_tag(W, it + 1))) return false;   // the conversion would read weights still in flight
+            q.wait(next_tile);
+            if (!q.landed(vm_tag(X, it + 1))) return false;   // the barrier would release a tile still in flight
+            // steady state: exactly what the schedule allows (rings deeper than three are allowed one less: their first
+            // iterations follow the prologue's order)
+            if (it >= WSN && next_weights != w_exact) return false;
+            if (it >= NBUF && x_exact - next_tile > (NBUF > 3 ? 1 : 0)) return false;
+            // a piece of a scale window is read two iterations after it was issued at the earliest
+            if (NSB && it >= 2 && !q.landed(vm_tag(S, it - 2))) return false;
+        }
+        return true;
+    }
+};
+
 // Same tiling and arguments as qmm_direct_kernel with 8 waves (KG = 2 or 4 K-groups x 8 / KG column waves,
 // 4-bit codes, scales and biases of the tile staged in LDS), same results; what differs:
 //   activations: the (32 * MB) x (64 * KG) tile of an iteration is MB * KG slots of 32 rows x 64 k (4 KB,
@@ -105,6 +150,8 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
     constexpr int NM = 4 * MB;                // MFMAs per wave and iteration
     constexpr int UN = WSN % 2 ? 2 * WSN : WSN;   // unroll: a multiple of the ring, of the weight sets and of 2 (fragment parity)
     static_assert(UN % NBUF == 0 && UN % WSN == 0 && UN % 2 == 0, "unroll covers every ring");
+    typedef QmmDmaWaits<NBUF, WSN, IPW, NWL, NSB> Waits;
+    static_assert(Waits::holds(), "a hand-counted vmcnt wait does not match the order in which the loop issues its loads");
     extern __shared__ __align__(16) unsigned char lds[];  // NBUF tiles, then the scales / biases window
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -314,12 +361,12 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
             db[0] = bv.x; db[1] = bv.y; db[2] = bv.z; db[3] = bv.w;
         }
     }
-    qm_wait_vm<(NBUF - 2) * IPW>();   // everything but X(1)..: the first tile's share and the first weight sets
+    qm_wait_vm<Waits::first>();   // everything but X(1)..: the first tile's share and the first weight sets
     __syncthreads();      // tile 0 and the scales are in LDS
     uint32_t bq[2][4][4];  // converted fragments: [iteration parity][MFMA step][dword]
     float sn, bn;          // 512 * scale and bias of the iteration being converted (the next one)
     {
-        wait_w(std::integral_constant<int, (NBUF - 2) * IPW>{}, 0);
+        wait_w(std::integral_constant<int, Waits::first>{}, 0);
         float s0, b0;
         scale_bias(0, s0, b0);
 #pragma unroll
@@ -353,7 +400,7 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
             float sn2, bn2;
             // weights of the next iteration, issued WSN - 1 iterations ago: the loads younger than they are the tiles
             // of WSN iterations and the weights of WSN - 1 (ring of two: tiles and weights of two iterations)
-            wait_w(std::integral_constant<int, (NBUF == 2 ? 2 * IPW + 2 * NWL + 2 * NSB : WSN * (IPW + NSB) + (WSN - 1) * NWL)>{}, (u + 1) % WSN);
+            wait_w(std::integral_constant<int, Waits::next_weights>{}, (u + 1) % WSN);
             qm_static_for<0, MB>([&](auto bi_c) {
                 constexpr int bi = decltype(bi_c)::value;
                 constexpr int par = bi & 1;
@@ -382,7 +429,7 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
             // this wave's share of the next tile (issued one iteration ago) is in LDS once at most this iteration's
             // loads are outstanding; past the barrier every wave's share is
             // (one less than the steady state allows: the first iterations follow the prologue's order)
-            qm_wait_vm<(NBUF == 2 ? NWL : NBUF == 3 ? IPW + NWL + NSB : (NBUF - 2) * (IPW + NWL) - 1)>();
+            qm_wait_vm<Waits::next_tile>();
             __syncthreads();
 #pragma unroll
             for (int j = 0; j < 4; j++) af[0][j] = *(const qm_u32x4*)(lds + ((u + 1) % NBUF) * TILE + aoff[j]);

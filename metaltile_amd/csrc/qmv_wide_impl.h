@@ -24,6 +24,7 @@
 // blockIdx.y picks the slice and f32 partial rows go to a scratch buffer that a second kernel adds up) is walked
 // in turns of 512 codes; weights are loaded a turn ahead, the scales and biases of a wave's whole run once.
 #include "mtq_device.h"
+#include "vm_schedule.h"
 #include "mtq_internal.h"
 
 #include <type_traits>
@@ -87,6 +88,26 @@ template <int OFF> __device__ __forceinline__ void qw_load(qw_u32x2& dst, uint32
     asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3" : "+v"(dst) : "v"(voff), "s"(sbase), "n"(OFF) : "memory");
 }
 // Waits until at most N vector memory loads of this wave are outstanding (they complete in order).
+// The stream loop's vector-memory schedule and the one wait count that follows from it. A turn's weights are two
+// lines (steps 0-1 and 2-3) of 2 NB loads each; the prologue issues both lines of the first turn; turn n waits for its
+// line 0, issues line 0 of turn n + 1 behind step 1, waits for its line 1 and issues line 1 of turn n + 1 behind step 3.
+// Whenever a line is needed the loads younger than it are exactly the other line's: 2 NB. holds() replays that order.
+template <int NB> struct QmvWideWaits {
+    static constexpr int line = 2 * NB;
+    static constexpr bool holds() {
+        VmQueue q;
+        q.issue(vm_tag(0, 0), 2 * NB);
+        q.issue(vm_tag(1, 0), 2 * NB);
+        for (int n = 0; n < 12; n++)
+            for (int p = 0; p < 2; p++) {
+                if (q.younger_than(vm_tag(p, n)) != line) return false;   // neither too early nor later than need be
+                q.wait(line);
+                if (!q.landed(vm_tag(p, n))) return false;
+                q.issue(vm_tag(p, n + 1), 2 * NB);
+            }
+        return true;
+    }
+};
 template <int N> __device__ __forceinline__ void qw_wait() {
     static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -233,6 +254,7 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
         }
     }
 
+    static_assert(QmvWideWaits<NB>::holds(), "the hand-counted vmcnt wait does not match the order in which the stream loop issues its loads");
     qw_u32x4 ring[NB][4];
 #pragma unroll
     for (int i = 0; i < NB; i++)
@@ -351,7 +373,7 @@ template <int DT, int G, int NB, int SETS, int MODE = GATHER_NONE> __global__ __
         qw_static_for<0, 4>([&](auto d_c) {
             constexpr int d = decltype(d_c)::value;
             if constexpr (d % 2 == 0) {
-                qw_wait<2 * NB>();
+                qw_wait<QmvWideWaits<NB>::line>();
 #pragma unroll
                 for (int i = 0; i < NB; i++) { qw_tie(ring[i][d]); qw_tie(ring[i][d + 1]); }
             }

@@ -20,6 +20,22 @@ CSRC = os.path.join(HERE, "..", "metaltile_amd", "csrc")
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
 
+def _units_including(header):
+    """Every translation unit that instantiates the kernels of `header` (directly or through another header): an
+    instance added in a new file is scanned without this test being told about it."""
+    def includes(path, seen):
+        out = set()
+        for m in re.finditer(r'#include\s+"([^"]+)"', open(path).read()):
+            name = os.path.basename(m.group(1))
+            if name not in seen and os.path.exists(os.path.join(CSRC, name)):
+                seen.add(name)
+                out |= {name} | includes(os.path.join(CSRC, name), seen)
+        return out
+    units = sorted(f for f in os.listdir(CSRC) if f.endswith(".hip") and header in includes(os.path.join(CSRC, f), set()))
+    assert units, header
+    return units
+
+
 def _assembly(src, out):
     cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
            "-I" + os.path.join(HERE, "..", "include"), "--cuda-device-only", "-S", os.path.join(CSRC, src), "-o", out]
@@ -91,7 +107,9 @@ def _stream_loops(lines):
 def test_only_hand_counted_waits_in_the_stream_loop():
     with tempfile.TemporaryDirectory() as tmp:
         with concurrent.futures.ThreadPoolExecutor(max_workers=2) as ex:
-            outs = list(ex.map(lambda s: _assembly(s, os.path.join(tmp, s + ".s")), ["qmv_wide.hip", "qmv_wide_gather.hip"]))
+            units = _units_including("qmv_wide_impl.h")
+            assert {"qmv_wide.hip", "qmv_wide_gather.hip"} <= set(units)
+            outs = list(ex.map(lambda s: _assembly(s, os.path.join(tmp, s + ".s")), units))
     n = 0
     for lines in outs:
         for name, mine, every, scratch, mfma, early in _stream_loops(lines):
@@ -111,7 +129,9 @@ def test_tile_kernels_wait_only_where_written():
     is a wait for every load in flight)."""
     with tempfile.TemporaryDirectory() as tmp:
         with concurrent.futures.ThreadPoolExecutor(max_workers=2) as ex:
-            outs = list(ex.map(lambda s: _assembly(s, os.path.join(tmp, s + ".s")), ["qmm_dma.hip", "qmm_dma_b8.hip"]))
+            units = _units_including("qmm_dma_impl.h")
+            assert {"qmm_dma.hip", "qmm_dma_b8.hip"} <= set(units)
+            outs = list(ex.map(lambda s: _assembly(s, os.path.join(tmp, s + ".s")), units))
     n = 0
     for lines in outs:
         starts = [(i, l.split(":")[0]) for i, l in enumerate(lines) if l.startswith("_ZN3mtq14qmm_dma_kernel") and "; @" in l]
@@ -150,3 +170,40 @@ def test_one_row_streaming_instances_keep_their_values_in_registers():
         assert size == 0, f"qmv_stream_kernel<bf16, {bits}-bit, {mb} rows, ring {depth}, mode {mode}, {maxt}, {sbi}, norm {norm}>: {size} bytes of scratch"
         seen += 1
     assert seen >= 30
+
+
+def test_the_schedule_model_behind_the_static_asserts():
+    """Both hand-waited kernels hold their vmcnt counts against a compile-time replay of their own issue order
+    (csrc/vm_schedule.h: QmmDmaWaits, QmvWideWaits). The replay's queue is checked here on the host compiler, with
+    cases it must accept and cases it must reject, and every schedule the library instantiates must hold."""
+    src = r"""
+#include "vm_schedule.h"
+using namespace mtq;
+constexpr bool accepts() {
+    VmQueue q;
+    q.issue(vm_tag(1, 0), 2); q.issue(vm_tag(1, 1), 2); q.issue(vm_tag(2, 0), 3);
+    if (q.younger_than(vm_tag(1, 0)) != 5 || q.younger_than(vm_tag(1, 1)) != 3 || q.younger_than(vm_tag(2, 0)) != 0) return false;
+    if (q.younger_than(vm_tag(3, 0)) != -1 || q.landed(vm_tag(1, 0))) return false;
+    q.wait(5);                                    // the two oldest loads have landed
+    if (!q.landed(vm_tag(1, 0)) || q.landed(vm_tag(1, 1))) return false;
+    q.wait(6);                                    // a weaker wait later takes nothing back
+    if (!q.landed(vm_tag(1, 0))) return false;
+    q.wait(0);
+    return q.landed(vm_tag(2, 0)) && !q.landed(vm_tag(3, 0));
+}
+static_assert(accepts(), "queue model");
+// one load too many allowed in flight: the load that is needed may be the one still outstanding
+constexpr bool too_weak() { VmQueue q; q.issue(vm_tag(1, 0), 1); q.issue(vm_tag(1, 1), 4); q.wait(5); return q.landed(vm_tag(1, 0)); }
+static_assert(!too_weak(), "a wait that is too weak must be seen");
+int main() { return 0; }
+"""
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "q.cpp")
+        open(path, "w").write(src)
+        r = subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-I", CSRC, path], capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-2000:]
+    # the kernels carry the static_asserts (a build of the library is their test)
+    for header, name in (("qmm_dma_impl.h", "QmmDmaWaits"), ("qmv_wide_impl.h", "QmvWideWaits")):
+        text = open(os.path.join(CSRC, header)).read()
+        assert re.search(r"static_assert\(\s*(Waits|" + name + r"<[^>]*>)::holds\(\)", text), header
+        assert "qm_wait_vm<(" not in text and "qw_wait<2" not in text, f"{header}: a wait count written as a literal expression"
