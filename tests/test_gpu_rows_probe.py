@@ -8,8 +8,8 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dt_name", ["BF16", "F16"])
-@pytest.mark.parametrize("N", [4, 20, 1028, 14336])
-def test_rows_kernel_through_mtq_qmv(oracle, dt_name, N):
+@pytest.mark.parametrize("N,K", [(4, 4096), (20, 4096), (1028, 4096), (14336, 4096), (1, 14336), (19, 14336), (1030, 14336), (4096, 14336)])
+def test_rows_kernel_through_mtq_qmv(oracle, dt_name, N, K):
     """The same kernel as the product path of mtq_qmv (forced with qmv.kernel = 3 below its automatic size), ragged last
     workgroups included, behind a cache flush, against the f64 oracle and bit for bit against the streaming kernel's
     neighbour rows that it must not touch."""
@@ -18,15 +18,14 @@ def test_rows_kernel_through_mtq_qmv(oracle, dt_name, N):
     from metaltile_amd.synth import make_case
     from tests.parity import rel_err
     dt = getattr(DType, dt_name)
-    K = 4096
-    c = make_case(3200 + N, dt, 4, 64, 1, N, K)
+    c = make_case(3200 + N + K, dt, 4, 64, 1, N, K)
     bw, bs, bb, bx = (GpuBuffer.from_bytes(v) for v in (c.w.tobytes(), c.scales_bytes, c.biases_bytes, c.x_bytes))
     out = GpuBuffer.from_bytes(np.full(N + 8, 0xABAB, np.uint16).tobytes())
     from metaltile_amd import _lib
     lib = _lib.load()
     assert lib.mtq_set_option(b"qmv.kernel", 3) == 0
     try:
-        assert "qmv_rows_kernel" in ops.plan("qmv", dt, 4, 64, 1, N, K)[1][0][0]
+        assert ("qmv_rows_kernel" if K == 4096 else "qmv_rows_long_kernel") in ops.plan("qmv", dt, 4, 64, 1, N, K)[1][0][0]
         m.GpuRunner(0).flush_slc()
         ops.qmv(dt, 4, 64, bw, bs, bb, bx, out, 1, N, K)
     finally:
