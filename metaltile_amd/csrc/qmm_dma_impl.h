@@ -347,18 +347,31 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
             *(uint32_t*)(sbB + row * sbld + c0) = *(const uint32_t*)((const uint16_t*)a.biases + (size_t)grow * a.gpr + sb_g0 + c0);
         }
     } else {
-        // DBN rows x sb_ng elements each of scales and biases, 16 bytes per load (ordinary loads: the compiler waits)
+        // DBN rows x sb_ng elements each of scales and biases, 16 bytes per load (ordinary loads: the compiler waits).
+        // Two vectors of each per thread are loaded before the first is stored: the usual tile (128 columns x 64 groups on
+        // 512 threads) is then one trip to memory behind the weight and activation loads above, not two in a row.
         const uint32_t vpr = sb_ng / 8, nvec = DBN * vpr;
-        for (uint32_t v = tid; v < nvec; v += NT) {
-            const uint32_t row = v / vpr, c0 = (v - row * vpr) * 8;
-            const uint32_t grow = min(n0 + row, a.N - 1);
-            const q_u32x4 sv = *(const q_u32x4*)((const uint16_t*)a.scales + (size_t)grow * a.gpr + sb_g0 + c0);
-            const q_u32x4 bv = *(const q_u32x4*)((const uint16_t*)a.biases + (size_t)grow * a.gpr + sb_g0 + c0);
-            const uint32_t cpos = ROT ? (c0 + row * 8) % sbld : c0;   // whole 8-element vectors move together
-            uint32_t* ds = (uint32_t*)(sbS + row * sbld + cpos);
-            uint32_t* db = (uint32_t*)(sbB + row * sbld + cpos);
-            ds[0] = sv.x; ds[1] = sv.y; ds[2] = sv.z; ds[3] = sv.w;
-            db[0] = bv.x; db[1] = bv.y; db[2] = bv.z; db[3] = bv.w;
+        for (uint32_t v0 = 0; v0 < nvec; v0 += 2 * NT) {
+            q_u32x4 sv[2], bv[2];
+            uint32_t row[2], c0[2];
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const uint32_t v = min(v0 + u * NT + tid, nvec - 1);
+                row[u] = v / vpr;
+                c0[u] = (v - row[u] * vpr) * 8;
+                const uint32_t grow = min(n0 + row[u], a.N - 1);
+                sv[u] = *(const q_u32x4*)((const uint16_t*)a.scales + (size_t)grow * a.gpr + sb_g0 + c0[u]);
+                bv[u] = *(const q_u32x4*)((const uint16_t*)a.biases + (size_t)grow * a.gpr + sb_g0 + c0[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                if (v0 + u * NT + tid >= nvec) continue;
+                const uint32_t cpos = ROT ? (c0[u] + row[u] * 8) % sbld : c0[u];   // whole 8-element vectors move together
+                uint32_t* ds = (uint32_t*)(sbS + row[u] * sbld + cpos);
+                uint32_t* db = (uint32_t*)(sbB + row[u] * sbld + cpos);
+                ds[0] = sv[u].x; ds[1] = sv[u].y; ds[2] = sv[u].z; ds[3] = sv[u].w;
+                db[0] = bv[u].x; db[1] = bv[u].y; db[2] = bv[u].z; db[3] = bv[u].w;
+            }
         }
     }
     qm_wait_vm<Waits::first>();   // everything but X(1)..: the first tile's share and the first weight sets
