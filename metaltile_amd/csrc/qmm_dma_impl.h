@@ -458,40 +458,58 @@ __global__ __launch_bounds__(64 * NW) void qmm_dma_kernel(QmmDArgs a) {
         for (int k = 0; k < NWL; k++) asm volatile("" ::"v"(raw[ws][k]));
     __syncthreads();
 
-    // ---- the other K-groups hand their accumulators to K-group 0 through LDS, at most 128 rows at a time ---
+    // ---- the K-groups add their accumulators through LDS, at most 128 rows at a time ------------------------------
+    // A wave's accumulators of a round are U = 4 EPB units of four registers (unit u = row block u / 4, rows
+    // 8 (u % 4) + 4 (lane / 32) + 0 .. 3 of it, column lane % 32). Unit u is summed by K-group u % KG: every other
+    // K-group hands it over with one 16-byte LDS store, the owner adds the KG values in K-group order (its own in its
+    // place: the sum is ((k0 + k1) + k2) + k3 whoever owns it), rounds and writes the four elements into the tile of
+    // rows that leaves in whole 16-byte pieces. All eight waves share the adding, rounding and LDS traffic, and the
+    // partial sums move 16 bytes per instruction.
     constexpr int EPB = MB == 8 ? 4 : MB;       // row blocks per round
-    constexpr int GRP = NWV * EPB * 16 * 64;    // floats per K-group and round
-    float* red = (float*)lds;                   // [kg - 1][wn][bi][v][lane]
+    constexpr int GRP = NWV * EPB * 16 * 64;    // floats per handing-over K-group and round
+    constexpr int U = 4 * EPB;
+    typedef float qm_f32x4 __attribute__((ext_vector_type(4)));
+    qm_f32x4* red4 = (qm_f32x4*)lds;            // [KG - 1 senders][wn][U][lane]
     uint16_t* otile = (uint16_t*)(lds + (KG - 1) * GRP * 4);   // the round's rows as [row][DBN columns], behind the partial sums
     qm_static_for<0, MB / EPB>([&](auto ph_c) {
         constexpr int ph = decltype(ph_c)::value;
         if constexpr (ph > 0) __syncthreads();   // the last round's tile has been stored
-        if (kg != 0) {
-#pragma unroll
-            for (int bi = 0; bi < EPB; bi++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) red[(kg - 1) * GRP + ((wn * EPB + bi) * 16 + v) * 64 + lane] = acc[ph * EPB + bi][v];
-        }
+        qm_static_for<0, U>([&](auto u_c) {
+            constexpr int u = decltype(u_c)::value;
+            constexpr int owner = u % KG, bi = ph * EPB + u / 4, v0 = 4 * (u % 4);
+            if (kg != (uint32_t)owner) {         // (uniform per wave)
+                const uint32_t slot = kg < (uint32_t)owner ? kg : kg - 1u;
+                const qm_f32x4 t = {acc[bi][v0], acc[bi][v0 + 1], acc[bi][v0 + 2], acc[bi][v0 + 3]};
+                red4[((slot * NWV + wn) * U + u) * 64 + lane] = t;
+            }
+        });
         __syncthreads();
-        // accumulator layout: column j = lane%32, row i = 8*(v/4) + 4*(lane/32) + v%4.
-        // K-group 0 adds, rounds to the element dtype and writes the rows to LDS
-        if (kg == 0) {
+        // accumulator layout: column j = lane%32, row i = 8*(v/4) + 4*(lane/32) + v%4
+        qm_static_for<0, U>([&](auto u_c) {
+            constexpr int u = decltype(u_c)::value;
+            constexpr int owner = u % KG, bl = u / 4, bi = ph * EPB + bl, v0 = 4 * (u % 4);
+            if (kg == (uint32_t)owner) {
+                qm_f32x4 r = {0.f, 0.f, 0.f, 0.f};
+                qm_static_for<0, KG>([&](auto j_c) {
+                    constexpr int j = decltype(j_c)::value;
+                    qm_f32x4 val;
+                    if constexpr (j == owner) val = qm_f32x4{acc[bi][v0], acc[bi][v0 + 1], acc[bi][v0 + 2], acc[bi][v0 + 3]};
+                    else val = red4[(((j < owner ? j : j - 1) * NWV + wn) * U + u) * 64 + lane];
+                    if constexpr (j == 0) r = val;
+                    else r = r + val;
+                });
 #pragma unroll
-            for (int bi = 0; bi < EPB; bi++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const uint32_t trow = bi * 32 + 8 * (v / 4) + 4 * fh + (v % 4), lrow = ph * EPB * 32 + trow;
-                    float r = acc[ph * EPB + bi][v];
-#pragma unroll
-                    for (int g = 0; g < KG - 1; g++) r += red[g * GRP + ((wn * EPB + bi) * 16 + v) * 64 + lane];
+                for (int vv = 0; vv < 4; vv++) {
+                    const uint32_t trow = bl * 32 + 8 * (u % 4) + 4 * fh + vv, lrow = ph * EPB * 32 + trow;
                     if constexpr (SP) {  // this split's f32 partial sums, 32 consecutive columns per half wave
                         const uint32_t col = n0 + wn * 32 + fr;
-                        if (lrow < row_count && col < a.N) a.part[((size_t)blockIdx.y * a.M + row_first + lrow) * a.N + col] = r;
+                        if (lrow < row_count && col < a.N) a.part[((size_t)blockIdx.y * a.M + row_first + lrow) * a.N + col] = r[vv];
                     } else {
-                        otile[trow * DBN + wn * 32 + fr] = f32_to_elem_bits<DT>(r);
+                        otile[trow * DBN + wn * 32 + fr] = f32_to_elem_bits<DT>(r[vv]);
                     }
                 }
-        }
+            }
+        });
         if constexpr (!SP) {  // split instances end with the partial sums: the second kernel rounds and stores
             __syncthreads();
             // all threads store the rows, 16 bytes each, whole rows
