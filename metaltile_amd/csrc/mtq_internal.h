@@ -210,8 +210,10 @@ int build_gather_tiles(const uint32_t* route, bool per_row_ids, uint32_t T, uint
 int launch_qmm_f32_grouped(const QmmParams& p, const uint32_t* route, bool per_row_ids, uint32_t T, uint32_t E, void* scratch,
                            const LaunchCtx& lc);
 
-// One wave per four rows of 4096 4-bit codes in groups of 64, f16 / bf16, one activation row (qmv_rows.hip).
+// The wave-per-row kernels (qmv_rows.hip): one activation row, f16 / bf16; rows of 4096 4-bit codes in groups of 64 (one wave per
+// four rows), or 2- / 4-bit codes in groups of 32 / 64 / 128 on rows of 8192, 14336 (4-bit) or 16384 (2-bit) codes (one wave per row).
 bool qmv_rows_takes(const QmvParams& p);
+bool qmv_rows_preferred(const QmvParams& p);
 int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc);
 // The same kernel as a measurement aid (bf16; mode 0 / 1 / 2 = full / no arithmetic / weight loads only; stamps may be null).
 int launch_rows_probe(const void* w, const void* s, const void* b, const void* x, void* out, uint32_t N, int mode, uint64_t* stamps,

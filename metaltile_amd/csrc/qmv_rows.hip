@@ -206,48 +206,97 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(QmvRowsArgs a) {
     }
 }
 
-// ---- long rows: K = CH x 2048 codes with CH > 2 (the down projection's 14336) ----------------------------------------
+// ---- one wave per row, activations shared by the workgroup: other row lengths, group sizes and 2-bit codes -----------
 // The same ownership (lane l holds chunks l, 64 + l, ... of a row, the diagonal of the 4x4x4 blocks, scales loaded per
-// lane, one shot of loads) with two things changed by the row length. A lane's share of the activations is 32 CH values
-// (112 registers at CH = 7), so a wave owns one row, and a workgroup of sixteen waves owns sixteen - one workgroup per
-// compute unit at 4096 rows, every load of the launch issued in its first microsecond. And the activations are put
-// into operand order once per workgroup, not once per wave: thread t prepares chunk t (32 values and their sum) into
-// LDS while the weights are in flight, and after the one barrier of the kernel every lane reads its CH chunks from
-// there (laid out by 16-byte quarter, so that consecutive lanes read consecutive 16 bytes). Measured in one run on
-// 4096 x 14336 bf16: streaming kernel 8.60 us, this with two rows per wave on eight waves 8.34, as here 8.27. (The same
-// sharing for rows of 4096 codes gains nothing over one preparation per wave: 8.00 against 7.95 us.)
-template <int DT, int CH>
-__global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsArgs a) {
-    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
-    constexpr int C = 64 * CH, GPR = 32 * CH;          // chunks and groups per row
-    constexpr int GPL = 4;                              // groups per lane in the bias term: lanes below GPR / 4 take four each
-    static_assert(GPR % GPL == 0 && GPR / GPL <= 64 && C <= 1024, "one thread per chunk, four groups per lane");
-    __shared__ __align__(16) uint32_t xp_lds[4][C][4];  // [16-byte quarter][chunk][4 dwords]: the chunk's pairs 4 q .. 4 q + 3
-    __shared__ __align__(16) float xs_lds[C];           // sum of each chunk's activations
+// lane, one shot of loads), with what longer rows change. A lane's share of the activations grows with the row (112
+// registers for 14336 4-bit codes), so a wave owns one row and a workgroup of sixteen waves owns sixteen - one workgroup
+// per compute unit at 4096 rows, every load of the launch issued in its first microsecond. And the activations are put
+// into operand order once per workgroup, not once per wave: thread t prepares chunk t (its values and their sums) into
+// LDS while the weights are in flight, and after the one barrier of the kernel every lane takes its operands from there
+// (laid out by 16-byte quarter, so that consecutive lanes read consecutive 16 bytes). Measured in one run on
+// 4096 x 14336 bf16: streaming kernel 8.60 us, this with two rows per wave on eight waves 8.34, as here 8.11. (The same
+// sharing for rows of 4096 4-bit codes gains nothing over one preparation per wave: 8.00 against 7.95 us.)
+//
+// A chunk is 16 bytes: CPC = 32 4-bit or 64 2-bit codes. Groups of 32, 64 or 128 codes: the two halves of a chunk are
+// accumulated apart and each takes the scale of its own group (the same one unless 2-bit codes come in groups of 32).
+// 2-bit codes are made operands without moving them: a masked pair of crumbs (i, i + 8) of a weight dword, left at
+// its bit position 2 p inside the two 16-bit halves and OR-ed into the mantissa of 2^(MB - 2 p) (MB = 10 mantissa bits
+// for f16, 7 for bf16), is the pair (2^(MB - 2p) + q_i, 2^(MB - 2p) + q_(i+8)) exactly: five positions fit an f16
+// mantissa and three a bf16 one, so a dword's eight pairs cost 8 mask-or and one shift (f16) or two (bf16) instead of
+// eight shifts. The offset each pair carries depends on its position; sum(offset_k x_k) over a half chunk is worked out
+// once per workgroup by the same matrix instruction with the OR-constants as its second operand, and leaves with the
+// bias term: out = sum_h s_h dot_h + sum_g (b_g X_g - s_g XM_g), X the plain and XM the offset-weighted activation sums.
+struct QmvRowsLArgs {
+    const rp_u32x4* w;
+    const uint16_t* s;
+    const uint16_t* b;
+    const uint16_t* x;
+    uint16_t* out;
+    uint32_t N;
+};
+
+// position class of pair i of a 2-bit weight dword and the shift that brings it there
+template <int DT> __host__ __device__ constexpr int rp_crumb_class(int i) { return DT == DT_F16 ? (i < 5 ? i : i - 5) : i % 3; }
+template <int DT> __host__ __device__ constexpr int rp_crumb_shift(int i) { return DT == DT_F16 ? (i < 5 ? 0 : 10) : 6 * (i / 3); }
+// the OR-constant of class p: 2^(MB - 2 p) in both halves (f16: exponent bias 15, 10 mantissa bits; bf16: 127, 7)
+template <int DT> __host__ __device__ constexpr uint32_t rp_crumb_kor(int p) {
+    const uint32_t h = DT == DT_F16 ? (uint32_t)(15 + 10 - 2 * p) << 10 : (uint32_t)(127 + 7 - 2 * p) << 7;
+    return h | (h << 16);
+}
+
+template <int DT, int BITS, int CH, int LOG2G>
+__global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) {
+    static_assert(BITS == 2 || BITS == 4, "2- or 4-bit codes");
+    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;   // 4-bit codes: one offset for every pair
+    constexpr int CPC = 128 / BITS;        // codes per chunk
+    constexpr int Q = CPC / 8;             // 16-byte quarters of a chunk's activations in operand order (4 pair dwords each)
+    constexpr int C = 64 * CH;             // chunks per row
+    constexpr int K = C * CPC;
+    constexpr int GPR = K >> LOG2G;        // groups per row
+    constexpr int GPL = GPR > 128 ? 4 : GPR > 64 ? 2 : 1;   // groups a lane owns in the bias term (lanes below GPR / GPL)
+    constexpr int SPG = (1 << LOG2G) / (CPC / 2);            // half chunks per group
+    constexpr int NH = (1 << LOG2G) < CPC ? 2 : 1;           // groups a chunk spans: its halves are then accumulated and scaled apart
+    static_assert(C <= 1024, "one thread per chunk");
+    static_assert(LOG2G >= 5 && LOG2G <= 7 && GPR % GPL == 0 && GPR / GPL <= 64 && SPG >= 1, "groups of 32, 64 or 128 codes, at most 256 per row");
+    __shared__ __align__(16) uint32_t xp_lds[Q][C][4];   // [quarter][chunk][4 pair dwords]
+    __shared__ __align__(16) float xs_lds[2 * C];        // activation sum of each half chunk
+    __shared__ __align__(16) float xm_lds[BITS == 2 ? 2 * C : 4];   // 2-bit codes: the sum weighted with the pairs' offsets
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t r0 = blockIdx.x * 16u + wave;
     const bool live = r0 < a.N;
-    const uint32_t rr = live ? r0 : 0u;                  // idle waves of the last workgroup still prepare their chunks
+    const uint32_t rr = live ? r0 : 0u;    // idle waves of the last workgroup still prepare their chunks
     __builtin_amdgcn_s_setprio(3);
     // this thread's chunk of the activations
-    uint4 xraw[4];
+    uint4 xraw[Q];
     if (tid < (uint32_t)C) {
-        const uint4* xv = (const uint4*)(a.x + (size_t)tid * 32);
+        const uint4* xv = (const uint4*)(a.x + (size_t)tid * CPC);
 #pragma unroll
-        for (int v = 0; v < 4; v++) xraw[v] = xv[v];
+        for (int v = 0; v < Q; v++) xraw[v] = xv[v];
     }
     RP_KEEP_ORDER();
-    // scales of this lane's CH chunks (groups 32 i + lane / 2), and for the bias term scales and biases of groups 4 lane .. + 3
-    uint32_t sc[CH];
-    uint2 sv, bv;
+    // scales of the two halves of this lane's CH chunks, and for the bias term scales and biases of groups GPL lane .. + GPL - 1
+    uint32_t sc[CH][NH];
+    uint32_t sw[2] = {0u, 0u}, bw[2] = {0u, 0u};   // GPL elements each, two per dword
     const uint32_t gl = min(lane, (uint32_t)(GPR / GPL - 1));
     {
         const uint16_t* sp = a.s + (size_t)rr * GPR;
         const uint16_t* bp = a.b + (size_t)rr * GPR;
 #pragma unroll
-        for (int i = 0; i < CH; i++) sc[i] = sp[32 * i + (lane >> 1)];
-        sv = ((const uint2*)sp)[gl];
-        bv = ((const uint2*)bp)[gl];
+        for (int i = 0; i < CH; i++) {
+            const uint32_t k0 = (uint32_t)(i * 64 + (int)lane) * CPC;
+            sc[i][0] = sp[k0 >> LOG2G];
+            if constexpr (NH == 2) sc[i][1] = sp[(k0 + CPC / 2) >> LOG2G];
+        }
+        if constexpr (GPL == 4) {
+            const uint2 sv = ((const uint2*)sp)[gl], bv = ((const uint2*)bp)[gl];
+            sw[0] = sv.x; sw[1] = sv.y; bw[0] = bv.x; bw[1] = bv.y;
+        } else if constexpr (GPL == 2) {
+            sw[0] = ((const uint32_t*)sp)[gl];
+            bw[0] = ((const uint32_t*)bp)[gl];
+        } else {
+            sw[0] = sp[gl];
+            bw[0] = bp[gl];
+        }
     }
     RP_KEEP_ORDER();
     const rp_u32x4* wbase = a.w + (size_t)rr * C + lane;
@@ -257,61 +306,148 @@ __global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsArgs a) {
     RP_KEEP_ORDER();
     __builtin_amdgcn_s_setprio(0);
     const bool j0 = lane & 1u, j1 = lane & 2u;
-    uint32_t kor = DT == DT_BF16 ? 0x43004300u : 0x64006400u;
-    asm volatile("" : "+v"(kor));
+    // OR-constants in registers the optimiser cannot see through (an and-or then has one literal operand, its mask)
+    uint32_t kor[BITS == 2 ? (DT == DT_F16 ? 5 : 3) : 1];
+    if constexpr (BITS == 4) kor[0] = DT == DT_BF16 ? 0x43004300u : 0x64006400u;
+    else {
+#pragma unroll
+        for (int p = 0; p < (DT == DT_F16 ? 5 : 3); p++) kor[p] = rp_crumb_kor<DT>(p);
+    }
+#pragma unroll
+    for (int p = 0; p < (int)(sizeof(kor) / 4); p++) asm volatile("" : "+v"(kor[p]));
     // ---- the chunk into operand order, into LDS ------------------------------------------------------------------
     if (tid < (uint32_t)C) {
         rp_u32x2 ones;
         ones.x = ones.y = DT == DT_BF16 ? 0x3F803F80u : 0x3C003C00u;
-        rp_f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+        rp_f32x4 sx[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, sm[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        if constexpr (BITS == 4) {
 #pragma unroll
-        for (int d = 0; d < 4; d++) {
-            const uint4 v = xraw[d];
-            uint4 o;
-            o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
-            o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
-            o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
-            o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
-            *(uint4*)xp_lds[d][tid] = o;
-            rp_u32x2 a0, a1;
-            a0.x = v.x; a0.y = v.y; a1.x = v.z; a1.y = v.w;
-            sacc = rp_mfma<DT>(a0, ones, sacc);
-            sacc = rp_mfma<DT>(a1, ones, sacc);
+            for (int d = 0; d < 4; d++) {       // weight dword d: activations 8 d .. 8 d + 7, pairs (j, j + 4)
+                const uint4 v = xraw[d];
+                uint4 o;
+                o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+                o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+                o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+                o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+                *(uint4*)xp_lds[d][tid] = o;
+                rp_u32x2 a0, a1;
+                a0.x = o.x; a0.y = o.y; a1.x = o.z; a1.y = o.w;
+                sx[d / 2] = rp_mfma<DT>(a0, ones, sx[d / 2]);
+                sx[d / 2] = rp_mfma<DT>(a1, ones, sx[d / 2]);
+            }
+        } else {
+#pragma unroll
+            for (int d = 0; d < 4; d++) {       // weight dword d: activations 16 d .. 16 d + 15, pairs (i, i + 8)
+                const uint4 lo = xraw[2 * d], hi = xraw[2 * d + 1];
+                uint4 o[2];
+                o[0].x = __builtin_amdgcn_perm(hi.x, lo.x, 0x05040100u);
+                o[0].y = __builtin_amdgcn_perm(hi.x, lo.x, 0x07060302u);
+                o[0].z = __builtin_amdgcn_perm(hi.y, lo.y, 0x05040100u);
+                o[0].w = __builtin_amdgcn_perm(hi.y, lo.y, 0x07060302u);
+                o[1].x = __builtin_amdgcn_perm(hi.z, lo.z, 0x05040100u);
+                o[1].y = __builtin_amdgcn_perm(hi.z, lo.z, 0x07060302u);
+                o[1].z = __builtin_amdgcn_perm(hi.w, lo.w, 0x05040100u);
+                o[1].w = __builtin_amdgcn_perm(hi.w, lo.w, 0x07060302u);
+                *(uint4*)xp_lds[2 * d][tid] = o[0];
+                *(uint4*)xp_lds[2 * d + 1][tid] = o[1];
+                const uint32_t pw[8] = {o[0].x, o[0].y, o[0].z, o[0].w, o[1].x, o[1].y, o[1].z, o[1].w};
+#pragma unroll
+                for (int m = 0; m < 4; m++) {   // pairs 2 m, 2 m + 1
+                    rp_u32x2 av, kv;
+                    av.x = pw[2 * m]; av.y = pw[2 * m + 1];
+                    kv.x = kor[rp_crumb_class<DT>(2 * m)]; kv.y = kor[rp_crumb_class<DT>(2 * m + 1)];
+                    sx[d / 2] = rp_mfma<DT>(av, ones, sx[d / 2]);
+                    sm[d / 2] = rp_mfma<DT>(av, kv, sm[d / 2]);
+                }
+            }
         }
-        xs_lds[tid] = rp_diag(sacc, j0, j1);
+        xs_lds[2 * tid] = rp_diag(sx[0], j0, j1);
+        xs_lds[2 * tid + 1] = rp_diag(sx[1], j0, j1);
+        if constexpr (BITS == 2) {
+            xm_lds[2 * tid] = rp_diag(sm[0], j0, j1);
+            xm_lds[2 * tid + 1] = rp_diag(sm[1], j0, j1);
+        }
     }
     __syncthreads();
     if (!live) return;
-    // bias term: sum over this lane's four groups (a group is two neighbouring chunks) of (b - MAGIC s) * sum(x)
+    // bias term: over this lane's GPL groups, b X - s XM (4-bit codes: XM = MAGIC X). A group is SPG half chunks, so the
+    // lane's groups are a run of GPL SPG consecutive half-chunk sums.
     float t = 0.f;
     if (lane < (uint32_t)(GPR / GPL)) {
-        const float4 s0 = *(const float4*)&xs_lds[8 * gl], s1 = *(const float4*)&xs_lds[8 * gl + 4];
-        const float gsum[GPL] = {s0.x + s0.y, s0.z + s0.w, s1.x + s1.y, s1.z + s1.w};
-        const uint32_t sw[2] = {sv.x, sv.y}, bw[2] = {bv.x, bv.y};
+        constexpr int RUN = GPL * SPG;
+        float xs[RUN], xm[RUN];
+        if constexpr (RUN % 4 == 0) {
+#pragma unroll
+            for (int h = 0; h < RUN / 4; h++) {
+                const float4 v = *(const float4*)&xs_lds[lane * RUN + 4 * h];
+                xs[4 * h] = v.x; xs[4 * h + 1] = v.y; xs[4 * h + 2] = v.z; xs[4 * h + 3] = v.w;
+                if constexpr (BITS == 2) {
+                    const float4 m = *(const float4*)&xm_lds[lane * RUN + 4 * h];
+                    xm[4 * h] = m.x; xm[4 * h + 1] = m.y; xm[4 * h + 2] = m.z; xm[4 * h + 3] = m.w;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int h = 0; h < RUN; h++) {
+                xs[h] = xs_lds[lane * RUN + h];
+                if constexpr (BITS == 2) xm[h] = xm_lds[lane * RUN + h];
+            }
+        }
 #pragma unroll
         for (int v = 0; v < GPL; v++) {
+            float X = 0.f, XM = 0.f;
+#pragma unroll
+            for (int h = 0; h < SPG; h++) {
+                X += xs[v * SPG + h];
+                if constexpr (BITS == 2) XM += xm[v * SPG + h];
+            }
+            if constexpr (BITS == 4) XM = MAGIC * X;
             const float sf = rp_up<DT>((sw[v >> 1] >> (16 * (v & 1))) & 0xFFFFu), bf = rp_up<DT>((bw[v >> 1] >> (16 * (v & 1))) & 0xFFFFu);
-            t = fmaf(bf - MAGIC * sf, gsum[v], t);
+            t = fmaf(bf, X, t);
+            t = fmaf(0.f - sf, XM, t);
         }
     }
 #pragma unroll
     for (int i = 0; i < CH; i++) {
-        rp_f32x4 d0 = {0.f, 0.f, 0.f, 0.f};
+        rp_f32x4 dh[NH];
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const uint4 xo = *(const uint4*)xp_lds[q][i * 64 + lane];
-            const uint32_t w = wv[i][q];
-            rp_u32x2 b0, b1, a0, a1;
-            b0.x = (w & 0x000F000Fu) | kor;
-            b0.y = ((w >> 4) & 0x000F000Fu) | kor;
-            b1.x = ((w >> 8) & 0x000F000Fu) | kor;
-            b1.y = ((w >> 12) & 0x000F000Fu) | kor;
-            a0.x = xo.x; a0.y = xo.y;
-            a1.x = xo.z; a1.y = xo.w;
-            d0 = rp_mfma<DT>(a0, b0, d0);
-            d0 = rp_mfma<DT>(a1, b1, d0);
+        for (int h = 0; h < NH; h++) dh[h] = rp_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const uint32_t w = wv[i][d];
+            constexpr int HSH = NH == 2 ? 1 : 2;   // dword d adds to half d >> HSH
+            if constexpr (BITS == 4) {
+                const uint4 xo = *(const uint4*)xp_lds[d][i * 64 + lane];
+                rp_u32x2 b0, b1, a0, a1;
+                b0.x = (w & 0x000F000Fu) | kor[0];
+                b0.y = ((w >> 4) & 0x000F000Fu) | kor[0];
+                b1.x = ((w >> 8) & 0x000F000Fu) | kor[0];
+                b1.y = ((w >> 12) & 0x000F000Fu) | kor[0];
+                a0.x = xo.x; a0.y = xo.y;
+                a1.x = xo.z; a1.y = xo.w;
+                dh[d >> HSH] = rp_mfma<DT>(a0, b0, dh[d >> HSH]);
+                dh[d >> HSH] = rp_mfma<DT>(a1, b1, dh[d >> HSH]);
+            } else {
+                const uint4 xo0 = *(const uint4*)xp_lds[2 * d][i * 64 + lane], xo1 = *(const uint4*)xp_lds[2 * d + 1][i * 64 + lane];
+                const uint32_t xa[8] = {xo0.x, xo0.y, xo0.z, xo0.w, xo1.x, xo1.y, xo1.z, xo1.w};
+                uint32_t pq[8];
+#pragma unroll
+                for (int pi = 0; pi < 8; pi++) {
+                    constexpr uint32_t M2 = 0x00030003u;
+                    const int p = rp_crumb_class<DT>(pi), sh = rp_crumb_shift<DT>(pi);
+                    pq[pi] = ((w >> sh) & (M2 << (2 * p))) | kor[p];
+                }
+#pragma unroll
+                for (int m = 0; m < 4; m++) {
+                    rp_u32x2 av, bvv;
+                    av.x = xa[2 * m]; av.y = xa[2 * m + 1];
+                    bvv.x = pq[2 * m]; bvv.y = pq[2 * m + 1];
+                    dh[d >> HSH] = rp_mfma<DT>(av, bvv, dh[d >> HSH]);
+                }
+            }
         }
-        t = fmaf(rp_up<DT>(sc[i]), rp_diag(d0, j0, j1), t);
+#pragma unroll
+        for (int h = 0; h < NH; h++) t = fmaf(rp_up<DT>(sc[i][h]), rp_diag(dh[h], j0, j1), t);
     }
     t += __shfl_xor(t, 32, 64);
     t += dpp_f32<0xB1>(t);
@@ -340,19 +476,53 @@ static int launch_rows(int dtype, const void* w, const void* s, const void* b, c
     return ERR_OK;
 }
 
+// chunks of 16 bytes per lane and row for the one-row-per-wave kernel, or 0 if it has no instance for the shape
+static int rows_long_ch(const QmvParams& p) {
+    if (p.bits != 2 && p.bits != 4) return 0;
+    const uint32_t G = p.group_size, cpc = 128u / (uint32_t)p.bits;
+    if (G != 32 && G != 64 && G != 128) return 0;
+    if (p.K % (64u * cpc) || p.K / G > 256u || (p.K / G) % 4u) return 0;
+    const uint32_t ch = p.K / (64u * cpc);
+    if (p.bits == 4 && (ch == 4 || ch == 7)) return (int)ch;     // 8192, 14336 codes
+    if (p.bits == 2 && (ch == 2 || ch == 4)) return (int)ch;     // 8192, 16384 codes
+    return 0;
+}
+
 bool qmv_rows_takes(const QmvParams& p) {
-    const bool shape = (p.K == 4096 && p.N % 4 == 0 && p.N >= 4) || (p.K == 14336 && p.N >= 1);
-    return p.gather == GATHER_NONE && p.M == 1 && p.bits == 4 && p.group_size == 64 && shape &&
-           (p.dtype == DT_F16 || p.dtype == DT_BF16) && (uintptr_t)p.w % 16 == 0 && (uintptr_t)p.x % 16 == 0 &&
-           (uintptr_t)p.scales % 8 == 0 && (uintptr_t)p.biases % 8 == 0 && (uintptr_t)p.out % 2 == 0;
+    if (p.gather != GATHER_NONE || p.M != 1 || (p.dtype != DT_F16 && p.dtype != DT_BF16) || p.N == 0) return false;
+    if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.scales % 8 || (uintptr_t)p.biases % 8 || (uintptr_t)p.out % 2) return false;
+    if (p.bits == 4 && p.group_size == 64 && p.K == 4096) return p.N % 4 == 0;   // one wave per four rows
+    return rows_long_ch(p) != 0;
+}
+
+// Where these kernels are the fastest the library has (measured against the streaming kernel in one run, f16 / bf16, us):
+// 14336 x 4096 4-bit g64 8.11 -> 7.86; 4096 x 14336 8.60 -> 8.11 on one machine, 8.63 -> 8.73 on another; 8192 x 8192:
+// 2-bit g32 / g64 / g128 8.98 / 8.55 / 8.41 -> 6.65 / 6.16 / 6.03, 4-bit 9.63 / 9.47 / 9.27 -> 8.53 / 7.90 / 7.78.
+// Small matrices stay where they were (a workgroup here is sixteen rows: few rows leave compute units idle).
+bool qmv_rows_preferred(const QmvParams& p) { return qmv_rows_takes(p) && p.N >= 1024; }
+
+template <int DT, int LOG2G> static const void* rows_long_fn_g(int bits, int ch) {
+    if (bits == 4) {
+        if (ch == 4) return (const void*)qmv_rows_long_kernel<DT, 4, 4, LOG2G>;
+        if constexpr (LOG2G >= 6) return (const void*)qmv_rows_long_kernel<DT, 4, 7, LOG2G>;   // (14336 codes in groups of 32: 448 groups per row)
+        return nullptr;
+    }
+    if (ch == 2) return (const void*)qmv_rows_long_kernel<DT, 2, 2, LOG2G>;
+    if constexpr (LOG2G >= 6) return (const void*)qmv_rows_long_kernel<DT, 2, 4, LOG2G>;       // (16384 codes in groups of 32: 512)
+    return nullptr;
+}
+template <int DT> static const void* rows_long_fn(int bits, int ch, uint32_t G) {
+    return G == 32 ? rows_long_fn_g<DT, 5>(bits, ch) : G == 64 ? rows_long_fn_g<DT, 6>(bits, ch) : rows_long_fn_g<DT, 7>(bits, ch);
 }
 
 int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
-    if (!qmv_rows_takes(p)) return fail(ERR_UNSUPPORTED, "qmv rows kernel: one row of 4096 or 14336 4-bit codes in groups of 64, f16 / bf16");
-    if (p.K == 4096) return launch_rows(p.dtype, p.w, p.scales, p.biases, p.x, p.out, p.N, 0, nullptr, lc);
-    QmvRowsArgs a{(const rp_u32x4*)p.w, (const uint16_t*)p.scales, (const uint16_t*)p.biases, (const uint16_t*)p.x, (uint16_t*)p.out, p.N, nullptr};
+    if (!qmv_rows_takes(p)) return fail(ERR_UNSUPPORTED, "qmv rows kernels: one activation row, 2- or 4-bit codes, f16 / bf16, rows of 4096, 8192, 14336 or 16384 codes");
+    if (p.bits == 4 && p.group_size == 64 && p.K == 4096) return launch_rows(p.dtype, p.w, p.scales, p.biases, p.x, p.out, p.N, 0, nullptr, lc);
+    const int ch = rows_long_ch(p);
+    QmvRowsLArgs a{(const rp_u32x4*)p.w, (const uint16_t*)p.scales, (const uint16_t*)p.biases, (const uint16_t*)p.x, (uint16_t*)p.out, p.N};
     void* args[] = {&a};
-    const void* fn = p.dtype == DT_BF16 ? (const void*)qmv_rows_long_kernel<DT_BF16, 7> : (const void*)qmv_rows_long_kernel<DT_F16, 7>;
+    const void* fn = p.dtype == DT_BF16 ? rows_long_fn<DT_BF16>(p.bits, ch, p.group_size) : rows_long_fn<DT_F16>(p.bits, ch, p.group_size);
+    if (!fn) return fail(ERR_UNSUPPORTED, "qmv rows kernels: no instance for this row length and group size");
     hipError_t e = launch_kernel(fn, dim3((p.N + 15) / 16), dim3(1024), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "qmv long rows kernel launch");
     return ERR_OK;

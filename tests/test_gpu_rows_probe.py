@@ -65,3 +65,51 @@ def test_rows_probe_matches_oracle(oracle, N):
         runner.probe_qmv_rows([bufs], N, mode=3)
     for b in bufs:
         b.free()
+
+
+@pytest.mark.parametrize("dt_name", ["F16", "BF16"])
+@pytest.mark.parametrize("bits,G,N,K", [(2, 32, 50, 8192), (2, 64, 1, 8192), (2, 128, 8192, 8192), (2, 64, 33, 16384), (2, 32, 8192, 8192),
+                                        (4, 32, 50, 8192), (4, 64, 8192, 8192), (4, 128, 17, 8192), (4, 128, 40, 14336)])
+def test_one_row_per_wave_kernel_other_widths_and_groups(oracle, dt_name, bits, G, N, K):
+    """The one-row-per-wave kernel on the shapes it takes beyond the two of the headline: 2-bit codes (made operands in
+    place, with an offset that depends on the crumb's position) and 4-bit codes in groups of 32 / 64 / 128 on rows of
+    8192, 14336 and 16384 codes, forced with qmv.kernel = 3, ragged last workgroups, behind a cache flush, against the
+    f64 oracle on full-range codes."""
+    import metaltile_amd as m
+    from metaltile_amd import DType, GpuBuffer, ops, _lib
+    from metaltile_amd.synth import make_case
+    from tests.parity import rel_err
+    dt = getattr(DType, dt_name)
+    c = make_case(3300 + bits * 7 + G + N + K, dt, bits, G, 1, N, K, bias_rule="midpoint")
+    bw, bs, bb, bx = (GpuBuffer.from_bytes(v) for v in (c.w.tobytes(), c.scales_bytes, c.biases_bytes, c.x_bytes))
+    out = GpuBuffer.from_bytes(np.full(N + 8, 0xABAB, np.uint16).tobytes())
+    lib = _lib.load()
+    assert lib.mtq_set_option(b"qmv.kernel", 3) == 0
+    try:
+        name = ops.plan("qmv", dt, bits, G, 1, N, K)[1][0][0]
+        assert "qmv_rows_long_kernel" in name, name
+        m.GpuRunner(0).flush_slc()
+        ops.qmv(dt, bits, G, bw, bs, bb, bx, out, 1, N, K)
+    finally:
+        lib.mtq_set_option(b"qmv.kernel", 0)
+    raw = out.read_array(np.uint16)
+    assert np.all(raw[N:] == 0xABAB)
+    got = m.unpack_f32(raw[:N].tobytes(), dt)
+    exp = oracle.qmm_f64(c.w, c.scales_f, c.biases_f, c.x_f, 1, N, K, bits, G)
+    assert rel_err(got, exp) <= 1e-2
+    for b in (bw, bs, bb, bx, out):
+        b.free()
+
+
+def test_shapes_the_one_row_per_wave_kernel_refuses():
+    """Rows whose groups do not fit its bias-term ownership (more than 256 groups per row), other widths and other row
+    lengths fall through to the kernels that served them before, also when the option asks for it."""
+    from metaltile_amd import DType, ops, _lib
+    lib = _lib.load()
+    assert lib.mtq_set_option(b"qmv.kernel", 3) == 0
+    try:
+        for bits, G, K in ((4, 32, 14336), (8, 64, 8192), (4, 64, 11008), (2, 16, 8192), (4, 64, 2048), (3, 64, 8192)):
+            rc, launches, _, _ = ops.plan("qmv", DType.F16, bits, G, 1, 4096, K)
+            assert rc == 0 and "qmv_rows" not in launches[0][0], (bits, G, K, launches[0][0])
+    finally:
+        lib.mtq_set_option(b"qmv.kernel", 0)

@@ -179,3 +179,30 @@ def test_dynamic_m_helpers_match_reference_values():
     assert len(p) == 32 * 4 * 2 and p[:16] == x and not any(p[16:])
     with pytest.raises(ValueError):
         d.pad_x_rows_bytes(x, 3, 4, 2)
+
+
+def test_two_bit_operand_constants_are_exact():
+    """The one-row-per-wave GEMV makes a pair of 2-bit codes an MFMA operand by masking it in place and OR-ing it into
+    the mantissa of a power of two chosen by its bit position (csrc/qmv_rows.hip: rp_crumb_class / _shift / _kor). The
+    same constants, restated here, must give exactly offset + code in both halves for every pair of every dword."""
+    def cls(dt, i): return (i if i < 5 else i - 5) if dt == "f16" else i % 3
+    def sh(dt, i): return (0 if i < 5 else 10) if dt == "f16" else 6 * (i // 3)
+    def kor(dt, p):
+        h = ((15 + 10 - 2 * p) << 10) if dt == "f16" else ((127 + 7 - 2 * p) << 7)
+        return h | (h << 16)
+    def val(dt, h):
+        if dt == "f16":
+            return float(np.array([h], dtype=np.uint16).view(np.float16)[0])
+        return float(np.array([h << 16], dtype=np.uint32).view(np.float32)[0])
+    src = open(os.path.join(ROOT, "metaltile_amd", "csrc", "qmv_rows.hip")).read()
+    assert "DT == DT_F16 ? (i < 5 ? i : i - 5) : i % 3" in src and "DT == DT_F16 ? (i < 5 ? 0 : 10) : 6 * (i / 3)" in src
+    assert "(uint32_t)(15 + 10 - 2 * p) << 10 : (uint32_t)(127 + 7 - 2 * p) << 7" in src
+    rng = np.random.default_rng(1)
+    for dt, mant in (("f16", 10), ("bf16", 7)):
+        for w in [0, 0xFFFFFFFF, 0xAAAAAAAA, 0x55555555] + [int(v) for v in rng.integers(0, 2 ** 32, size=500)]:
+            for i in range(8):
+                p = cls(dt, i)
+                v = ((w >> sh(dt, i)) & (0x00030003 << (2 * p))) | kor(dt, p)
+                magic = 2.0 ** (mant - 2 * p)
+                assert val(dt, v & 0xFFFF) == magic + ((w >> (2 * i)) & 3)
+                assert val(dt, v >> 16) == magic + ((w >> (2 * (i + 8))) & 3)
