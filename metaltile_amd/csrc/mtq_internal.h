@@ -215,6 +215,11 @@ int launch_qmm_f32_grouped(const QmmParams& p, const uint32_t* route, bool per_r
 bool qmv_rows_takes(const QmvParams& p);
 bool qmv_rows_preferred(const QmvParams& p);
 int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc);
+// Two to four activation rows (qmv_rows_few.hip): one wave per four weight rows; 4096 or 8192 4-bit codes or 8192 2-bit codes per
+// row, groups of 32 / 64 / 128, f16 / bf16.
+bool qmv_rows_few_takes(const QmvParams& p);
+bool qmv_rows_few_preferred(const QmvParams& p);
+int launch_qmv_rows_few(const QmvParams& p, const LaunchCtx& lc);
 // The same kernel as a measurement aid (bf16; mode 0 / 1 / 2 = full / no arithmetic / weight loads only; stamps may be null).
 int launch_rows_probe(const void* w, const void* s, const void* b, const void* x, void* out, uint32_t N, int mode, uint64_t* stamps,
                       const LaunchCtx& lc);

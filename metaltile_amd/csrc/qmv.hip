@@ -255,6 +255,10 @@ int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {
         int rc = launch_qmv_rows(p, lc);
         if (rc != ERR_UNSUPPORTED) return rc;
     }
+    if (mode != 2 && ((options().qmv_kernel == 0 && qmv_rows_few_preferred(p)) || (options().qmv_kernel == 3 && qmv_rows_few_takes(p)))) {
+        int rc = launch_qmv_rows_few(p, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
     if (qmv_few_routed_rows(p) && mode != 2) {
         int rc = launch_qmv_dot2(p, lc);
         if (rc != ERR_UNSUPPORTED) return rc;

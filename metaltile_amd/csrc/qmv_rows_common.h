@@ -1,0 +1,52 @@
+// Device helpers shared by the GEMV kernels that feed the 4x4x4 matrix instruction straight from registers:
+// lane 4 b + i of block b supplies row i of the first operand (four 16-bit values along the reduction), lane 4 b + j
+// column j of the second, and lane 4 b + j receives column j of the block's 4 x 4 result in four registers (register i =
+// row i).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "mtq_device.h"
+
+namespace mtq {
+
+typedef uint32_t rp_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned rp_u32x2 __attribute__((ext_vector_type(2)));
+typedef short rp_s16x4 __attribute__((ext_vector_type(4)));
+typedef float rp_f32x4 __attribute__((ext_vector_type(4)));
+
+#define RP_KEEP_ORDER() do { asm volatile("" ::: "memory"); __builtin_amdgcn_sched_barrier(0); } while (0)
+
+typedef _Float16 rp_f16x4 __attribute__((ext_vector_type(4)));
+template <int DT> __device__ __forceinline__ rp_f32x4 rp_mfma(rp_u32x2 a, rp_u32x2 b, rp_f32x4 c) {
+    if constexpr (DT == DT_BF16) return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(rp_s16x4, a), __builtin_bit_cast(rp_s16x4, b), c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(rp_f16x4, a), __builtin_bit_cast(rp_f16x4, b), c, 0, 0, 0);
+}
+// a 16-bit element (zero-extended) as f32
+template <int DT> __device__ __forceinline__ float rp_up(uint32_t h) {
+    if constexpr (DT == DT_BF16) return __uint_as_float(h << 16);
+    else return f16_bits_to_f32(h);
+}
+// register (lane % 4) of a block's result: the lane's own product
+__device__ __forceinline__ float rp_diag(rp_f32x4 v, bool b0, bool b1) {
+    const float lo = b0 ? v.y : v.x, hi = b0 ? v.w : v.z;
+    return b1 ? hi : lo;
+}
+__device__ __forceinline__ float rp_swap32_add(float a, float b) {
+    rp_u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r.x) + __uint_as_float(r.y);
+}
+__device__ __forceinline__ float rp_swap16_add(float a, float b) {
+    rp_u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r.x) + __uint_as_float(r.y);
+}
+// position class of pair i of a 2-bit weight dword and the shift that brings it there
+template <int DT> __host__ __device__ constexpr int rp_crumb_class(int i) { return DT == DT_F16 ? (i < 5 ? i : i - 5) : i % 3; }
+template <int DT> __host__ __device__ constexpr int rp_crumb_shift(int i) { return DT == DT_F16 ? (i < 5 ? 0 : 10) : 6 * (i / 3); }
+// the OR-constant of class p: 2^(MB - 2 p) in both halves (f16: exponent bias 15, 10 mantissa bits; bf16: 127, 7)
+template <int DT> __host__ __device__ constexpr uint32_t rp_crumb_kor(int p) {
+    const uint32_t h = DT == DT_F16 ? (uint32_t)(15 + 10 - 2 * p) << 10 : (uint32_t)(127 + 7 - 2 * p) << 7;
+    return h | (h << 16);
+}
+
+}  // namespace mtq

@@ -183,7 +183,7 @@ def test_dynamic_m_helpers_match_reference_values():
 
 def test_two_bit_operand_constants_are_exact():
     """The one-row-per-wave GEMV makes a pair of 2-bit codes an MFMA operand by masking it in place and OR-ing it into
-    the mantissa of a power of two chosen by its bit position (csrc/qmv_rows.hip: rp_crumb_class / _shift / _kor). The
+    the mantissa of a power of two chosen by its bit position (csrc/qmv_rows_common.h: rp_crumb_class / _shift / _kor). The
     same constants, restated here, must give exactly offset + code in both halves for every pair of every dword."""
     def cls(dt, i): return (i if i < 5 else i - 5) if dt == "f16" else i % 3
     def sh(dt, i): return (0 if i < 5 else 10) if dt == "f16" else 6 * (i // 3)
@@ -194,7 +194,7 @@ def test_two_bit_operand_constants_are_exact():
         if dt == "f16":
             return float(np.array([h], dtype=np.uint16).view(np.float16)[0])
         return float(np.array([h << 16], dtype=np.uint32).view(np.float32)[0])
-    src = open(os.path.join(ROOT, "metaltile_amd", "csrc", "qmv_rows.hip")).read()
+    src = open(os.path.join(ROOT, "metaltile_amd", "csrc", "qmv_rows_common.h")).read()
     assert "DT == DT_F16 ? (i < 5 ? i : i - 5) : i % 3" in src and "DT == DT_F16 ? (i < 5 ? 0 : 10) : 6 * (i / 3)" in src
     assert "(uint32_t)(15 + 10 - 2 * p) << 10 : (uint32_t)(127 + 7 - 2 * p) << 7" in src
     rng = np.random.default_rng(1)

@@ -132,6 +132,15 @@ def test_benchmark_configurations_are_routed_as_documented():
         assert "qmv_rows_long_kernel" + name in ks[0] and ls[0][1][0] == 512, ks
     ks, _ = kernels("qmv", DType.F16, 8, 64, 1, 8192, 8192)
     assert "qmv_rows" not in ks[0]
+    # the four-row cells of the sweep: one wave per four weight rows where that is ahead (2-bit codes, 4-bit in groups of 32,
+    # three or four rows of 4-bit codes); two rows of 4-bit g64 / g128, fewer weight rows and 8-bit codes stay on the matrix-core GEMV
+    for bits, G, M, name in ((2, 32, 4, "<1, 2, 8, 5, false>"), (2, 64, 2, "<1, 2, 8, 6, false>"), (4, 32, 2, "<1, 4, 16, 5, false>"), (4, 64, 4, "<1, 4, 16, 6, false>"),
+                             (4, 128, 3, "<1, 4, 16, 7, false>")):
+        ks, ls = kernels("qmv", DType.F16, bits, G, M, 8192, 8192)
+        assert "qmv_rows_few_kernel" + name in ks[0] and ls[0][1][0] == 256 and ls[0][2][0] == 1024, ks
+    for args in ((DType.F16, 4, 64, 2, 8192, 8192), (DType.F16, 4, 64, 4, 4096, 8192), (DType.F16, 8, 64, 4, 8192, 8192), (DType.BF16, 4, 64, 4, 14336, 4096),
+                 (DType.F16, 2, 64, 5, 8192, 8192)):
+        assert "qmv_mfma_kernel" in kernels("qmv", *args)[0][0]
     ks, _ = kernels("qmv", DType.F32, 4, 64, 1, 4096, 4096)
     assert "qmv_stream_kernel<0, 4" in ks[0] or "qmv_kernel<0, 4" in ks[0]
     for M, mb in ((512, 2), (1024, 4), (2048, 8)):     # 64-, 128-, 256-row load-to-LDS tiles
