@@ -263,6 +263,8 @@ def leg_qmv(a, runner, info):
     for bufs in keep:
         for b in bufs.values():
             b.free()
+    from metaltile_amd import ops
+    kernels = {f"{n}x{k}": ops.plan("qmv", dt, 4, 64, 1, n, k)[1][0][0].split("(")[0].replace("void ", "") for n, k in sorted(set(shapes))}
     return {
         "metric": "qmv GB/s & % HBM peak (4-bit g64, 4096x14336 bf16); qmm TFLOP/s M=512", "value": round(gbs, 1), "unit": "GB/s",
         "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
@@ -273,7 +275,7 @@ def leg_qmv(a, runner, info):
         "pct_hbm_peak_whole_job": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_from_profiles("qmv_bf16_b4_llama_mlp"),
-                     "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, 1 row>", "bytes_per_launch": launch_bytes,
+                     "kernel": "; ".join(f"{v} ({k})" for k, v in kernels.items()), "bytes_per_launch": launch_bytes,
                      "avg_launch_us_timed_region": round(kern_avg, 3), "clock": clock, "peak_basis": hbm_peak_basis(info),
                      "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "min_us": round(st.min_us, 3),
                                            "median_us": round(st.median_us, 3), "p95_us": round(st.p95_us, 3),

@@ -76,6 +76,8 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(QmvRowsArgs a) {
     RP_KEEP_ORDER();
     const rp_u32x4* wbase = a.w + (size_t)r0 * C + lane;
     rp_u32x4 wv[R][2];
+    // (Every load at once is the fastest form here: with the loads of only one, two or three rows ahead of the row
+    // being worked on, 14336 x 4096 bf16 takes 8.3, 8.5 and 9.1 us against 7.75 in the same run.)
 #pragma unroll
     for (int r = 0; r < R; r++) {
         wv[r][0] = __builtin_nontemporal_load(wbase + r * C);
@@ -179,14 +181,15 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(QmvRowsArgs a) {
 
 // ---- one wave per row, activations shared by the workgroup: other row lengths, group sizes and 2-bit codes -----------
 // The same ownership (lane l holds chunks l, 64 + l, ... of a row, the diagonal of the 4x4x4 blocks, scales loaded per
-// lane, one shot of loads), with what longer rows change. A lane's share of the activations grows with the row (112
-// registers for 14336 4-bit codes), so a wave owns one row and a workgroup of sixteen waves owns sixteen - one workgroup
-// per compute unit at 4096 rows, every load of the launch issued in its first microsecond. And the activations are put
-// into operand order once per workgroup, not once per wave: thread t prepares chunk t (its values and their sums) into
-// LDS while the weights are in flight, and after the one barrier of the kernel every lane takes its operands from there
-// (laid out by 16-byte quarter, so that consecutive lanes read consecutive 16 bytes). Measured in one run on
-// 4096 x 14336 bf16: streaming kernel 8.60 us, this with two rows per wave on eight waves 8.34, as here 8.11. (The same
-// sharing for rows of 4096 4-bit codes gains nothing over one preparation per wave: 8.00 against 7.95 us.)
+// lane), with what longer rows change. A lane's share of the activations grows with the row (112 registers for 14336
+// 4-bit codes), so a wave owns one row and a workgroup of sixteen waves owns sixteen - one workgroup per compute unit at
+// 4096 rows. And the activations are put into operand order once per workgroup, not once per wave: thread t prepares
+// chunk t (its values and their sums) into LDS while the first weights are in flight, and after the one barrier of the
+// kernel every lane takes its operands from there (laid out by 16-byte quarter, so that consecutive lanes read
+// consecutive 16 bytes). Measured in one run on 4096 x 14336 bf16: streaming kernel 8.60 us, this with two rows per wave
+// on eight waves 8.34, one row per wave and every load issued at the start 8.11, as here (loads four chunks ahead, see
+// below) 7.2. (The same sharing for rows of 4096 4-bit codes gains nothing over one preparation per wave: 8.00 against
+// 7.95 us.)
 //
 // A chunk is 16 bytes: CPC = 32 4-bit or 64 2-bit codes. Groups of 32, 64 or 128 codes: the two halves of a chunk are
 // accumulated apart and each takes the scale of its own group (the same one unless 2-bit codes come in groups of 32).
@@ -263,8 +266,15 @@ __global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) {
     RP_KEEP_ORDER();
     const rp_u32x4* wbase = a.w + (size_t)rr * C + lane;
     rp_u32x4 wv[CH];
+    // Rows of more than four chunks per lane: the loads run four chunks ahead of the chunk being worked on and only two
+    // are issued before the activations are prepared. A compute unit takes loads only as fast as earlier ones return, so
+    // with all seven issued here the slowest wave reaches the barrier below when most of the data has arrived, and all
+    // the arithmetic follows in one piece (4096 x 14336 bf16, same run: 8.40 us; two ahead of the barrier and four in
+    // flight 7.17; 1 / 4 7.21, 3 / 4 7.39, 2 / 3 7.3, 2 / 5 7.55). Rows of two or four chunks are faster with every load
+    // at once (8192 x 8192 4-bit: 7.82 us against 9.05 with one ahead of the barrier, 10.2 with two).
+    constexpr int W0 = CH > 4 ? 4 : CH, PRE = CH > 4 ? 2 : CH;
 #pragma unroll
-    for (int i = 0; i < CH; i++) wv[i] = __builtin_nontemporal_load(wbase + i * 64);
+    for (int i = 0; i < PRE; i++) wv[i] = __builtin_nontemporal_load(wbase + i * 64);
     RP_KEEP_ORDER();
     __builtin_amdgcn_s_setprio(0);
     const bool j0 = lane & 1u, j1 = lane & 2u;
@@ -332,6 +342,9 @@ __global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) {
     }
     __syncthreads();
     if (!live) return;
+#pragma unroll
+    for (int i = PRE; i < W0; i++) wv[i] = __builtin_nontemporal_load(wbase + i * 64);
+    RP_KEEP_ORDER();
     // bias term: over this lane's GPL groups, b X - s XM (4-bit codes: XM = MAGIC X). A group is SPG half chunks, so the
     // lane's groups are a run of GPL SPG consecutive half-chunk sums.
     float t = 0.f;
@@ -371,6 +384,8 @@ __global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) {
     }
 #pragma unroll
     for (int i = 0; i < CH; i++) {
+        if (i + W0 < CH) wv[i + W0] = __builtin_nontemporal_load(wbase + (i + W0) * 64);
+        RP_KEEP_ORDER();
         rp_f32x4 dh[NH];
 #pragma unroll
         for (int h = 0; h < NH; h++) dh[h] = rp_f32x4{0.f, 0.f, 0.f, 0.f};
