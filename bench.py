@@ -15,6 +15,15 @@ attaches an event pair to every launch for the per-kernel distribution. The CPU
 baseline is the oracle restatement of the reference's CPU path timed on the
 host cores on a bounded sample.
 
+Every timed leg starts from the same state, whatever `--warmup` says: the
+last-level cache is flushed, the card is kept busy for 40 ms, and untimed
+steps of the leg's own chain run until at least 30 ms of GPU time have passed
+(the card's clocks settle over the first ~20 ms of load; 5 warm-up steps are 1
+ms). The shader clock is sampled on the launch stream right before and after
+the timed region (a chain of dependent adds against the constant-rate counter)
+and reported in `roofline.clock`, with the peak the fraction is priced against
+in `roofline.peak_basis`.
+
 The default run then times, in the same process, the two other figures the
 headline metric and its configurations name and reports them under
 "secondary": qmm at M = 512 (4-bit g64 bf16, N = K = 4096; bound: bf16 MFMA)
@@ -26,7 +35,12 @@ sweep (f16, 8192 x 8192, batch 1 and 4); `--workload batch` a decode batch of
 `--rows` rows (default 16) against one large matrix (`--shape`, default the
 128256 x 4096 lm-head), by the exact-dequant kernel name mt_qmm; `--workload
 qkv` / `gated_norm` the fused one-launch decode pieces (Q + K + V projections;
-gated RMSNorm + out projection at the reference's bench shape).
+gated RMSNorm + out projection at the reference's bench shape); `--workload
+rows_probe` the headline gate / up launch taken apart (the shipped kernel, the
+streaming kernel it replaced, a launch that only reads the same bytes, and the
+shipped kernel without its arithmetic / with its weight loads only, plus its
+per-wave timeline), which is where the distance to the HBM peak is accounted
+for.
 
 Prints ONE JSON line on stdout.
 """
