@@ -119,7 +119,7 @@ def test_benchmark_configurations_are_routed_as_documented():
         return [l[0] for l in launches], launches
 
     ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 14336, 4096)
-    assert "qmv_rows_kernel<2, 0, false>" in ks[0] and ls[0][1][0] * 16 == 14336   # 4 waves x 4 rows per workgroup
+    assert "qmv_rows_kernel<2, 0, false>" in ks[0] and ls[0][1][0] == 256 and ls[0][2][0] == 14 * 64   # one workgroup of 14 waves x 4 rows per compute unit
     ks, _ = kernels("qmv", DType.F16, 4, 64, 1, 4100, 4096)
     assert "qmv_rows_kernel<1, 0, false>" in ks[0]
     for args in ((DType.BF16, 4, 64, 1, 4098, 4096), (DType.BF16, 4, 32, 1, 4096, 4096), (DType.BF16, 4, 64, 2, 4096, 4096),
