@@ -227,7 +227,7 @@ __global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) {
     __shared__ __align__(16) float xs_lds[2 * C];        // activation sum of each half chunk
     __shared__ __align__(16) float xm_lds[BITS == 2 ? 2 * C : 4];   // 2-bit codes: the sum weighted with the pairs' offsets
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t r0 = blockIdx.x * 16u + wave;
+    const uint32_t r0 = blockIdx.x * (blockDim.x >> 6) + wave;   // (a workgroup is 8 or 16 waves, at least C threads)
     const bool live = r0 < a.N;
     const uint32_t rr = live ? r0 : 0u;    // idle waves of the last workgroup still prepare their chunks
     __builtin_amdgcn_s_setprio(3);
@@ -505,7 +505,13 @@ int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
     void* args[] = {&a};
     const void* fn = p.dtype == DT_BF16 ? rows_long_fn<DT_BF16>(p.bits, ch, p.group_size) : rows_long_fn<DT_F16>(p.bits, ch, p.group_size);
     if (!fn) return fail(ERR_UNSUPPORTED, "qmv rows kernels: no instance for this row length and group size");
-    hipError_t e = launch_kernel(fn, dim3((p.N + 15) / 16), dim3(1024), args, 0, lc);
+    // Sixteen rows per workgroup, eight for the long rows. One workgroup of sixteen per compute unit (4096 x 14336: 256
+    // of them) is the fastest form on some machines of the pool and 9 % behind on others, where the same launch as 512
+    // workgroups of eight holds (same run, 1024 / 512 threads: 7.34 / 7.40 us on one machine, 8.19 / 7.48 and 8.60 /
+    // 7.70 on two others); shorter rows keep sixteen (8192 x 8192: 4-bit 8.00 / 7.97, 2-bit 6.27 / 6.95).
+    const uint32_t block = ch > 4 ? 512u : 1024u;
+    if (block < 64u * (uint32_t)ch) return fail(ERR_UNSUPPORTED, "qmv rows kernels: workgroup smaller than the row's chunks");   // (thread t prepares chunk t)
+    hipError_t e = launch_kernel(fn, dim3((p.N + block / 64u - 1u) / (block / 64u)), dim3(block), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "qmv long rows kernel launch");
     return ERR_OK;
 }

@@ -126,7 +126,7 @@ def test_benchmark_configurations_are_routed_as_documented():
                  (DType.BF16, 8, 64, 1, 4096, 4096), (DType.BF16, 4, 64, 1, 512, 4096)):
         assert "qmv_rows_kernel" not in kernels("qmv", *args)[0][0]          # what that kernel does not take
     ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 4096, 14336)
-    assert "qmv_rows_long_kernel<2, 4, 7, 6>" in ks[0] and ls[0][1][0] == 256 and ls[0][2][0] == 1024   # one workgroup of 16 rows per compute unit
+    assert "qmv_rows_long_kernel<2, 4, 7, 6>" in ks[0] and ls[0][1][0] == 512 and ls[0][2][0] == 512   # workgroups of eight rows
     for bits, G, name in ((2, 32, "<1, 2, 2, 5>"), (2, 128, "<1, 2, 2, 7>"), (4, 64, "<1, 4, 4, 6>")):   # the one-row cells of the width / group sweep
         ks, ls = kernels("qmv", DType.F16, bits, G, 1, 8192, 8192)
         assert "qmv_rows_long_kernel" + name in ks[0] and ls[0][1][0] == 512, ks
