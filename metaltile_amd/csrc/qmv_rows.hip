@@ -448,11 +448,13 @@ static int launch_rows(int dtype, const void* w, const void* s, const void* b, c
     QmvRowsArgs a{(const rp_u32x4*)w, (const uint16_t*)s, (const uint16_t*)b, (const uint16_t*)x, (uint16_t*)out, N, stamps};
     void* args[] = {&a};
     const void* fn = dtype == DT_BF16 ? qmv_rows_fn<DT_BF16>(mode, stamps != nullptr) : qmv_rows_fn<DT_F16>(mode, stamps != nullptr);
-    // A workgroup is only a container here (no LDS, no barrier). Up to 16384 rows it is sized so that the launch is one
-    // workgroup per compute unit (14336 rows: 256 workgroups of 14 waves, 7.88 us against 7.97 as 896 workgroups of 4;
-    // 1024 rows: 256 single waves, 3.15 against 3.60); beyond that, workgroups of 4 waves (28672 rows: 13.9 against 14.2).
+    // A workgroup is only a container here (no LDS, no barrier). It is sized so that the workgroups are a whole number
+    // per compute unit: one of up to 16 waves up to 16384 rows (14336 rows: 256 workgroups of 14 waves, 7.88 us against
+    // 7.97 as 896 workgroups of 4; 1024 rows: 256 single waves, 3.15 against 3.60), beyond that as few rounds of at most
+    // 8 waves as it takes (28672 rows: 1024 workgroups of 7 waves, 13.25 us against 14.1 as 1792 of 4).
     const uint32_t waves = (N + 3u) / 4u;
-    const uint32_t wpw = waves <= 256u * 16u ? (waves + 255u) / 256u : 4u;
+    const uint32_t rounds = waves <= 256u * 16u ? 1u : (waves + 256u * 8u - 1u) / (256u * 8u);
+    const uint32_t wpw = (waves + 256u * rounds - 1u) / (256u * rounds);
     hipError_t e = launch_kernel(fn, dim3((waves + wpw - 1u) / wpw), dim3(wpw * 64u), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "qmv rows kernel launch");
     return ERR_OK;
