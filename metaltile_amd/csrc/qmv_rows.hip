@@ -35,7 +35,42 @@ struct QmvRowsArgs {
     uint16_t* out;
     uint32_t N;
     uint64_t* stamps;   // [N / 4][MTQ_ROWS_PROBE_STAMPS] or null
+    const uint32_t* route;   // routed instances: expert_offsets[E + 1] or indices[T]; w / s / b then hold E matrices, x and out T rows
+    uint32_t E, T;
 };
+
+// Routed rows (GM = GATHER_CSR / GATHER_INDICES; a decode step of a few tokens through a mixture-of-experts layer, fewer
+// rows than experts): grid row blockIdx.y serves the blockIdx.y-th expert that has a row and runs the kernel's body once
+// per row of that expert -- one row each when a token's experts are distinct, as top-k routing makes them. The same
+// rules as the streaming kernel's routed form (at most 64 experts and 64 rows: the routing is read by one wave-wide load).
+struct RowsRoute {
+    uint32_t expert = 0, n_pass = 1, lo = 0, n1 = 1, lo2 = 0;
+    unsigned long long mask = 0;
+};
+template <int GM> __device__ __forceinline__ bool rows_route(const uint32_t* route, uint32_t E, uint32_t T, uint32_t lane, RowsRoute& r) {
+    if constexpr (GM == GATHER_CSR) {
+        r.n_pass = csr_route64(route, E, T, blockIdx.y, true, lane, r.expert, r.lo, r.n1, r.lo2);
+        if (r.n_pass == 0) return false;
+        r.expert = __builtin_amdgcn_readfirstlane(r.expert);
+    }
+    if constexpr (GM == GATHER_INDICES) {
+        r.expert = __builtin_amdgcn_readfirstlane(ids_slot_expert(route, E, T, blockIdx.y, lane));
+        if (r.expert == 0xFFFFFFFFu) return false;
+        r.mask = __ballot(lane < T && route[lane] == r.expert);
+        r.n_pass = (uint32_t)__popcll(r.mask);
+    }
+    return true;
+}
+// the activation (and output) row of a pass
+template <int GM> __device__ __forceinline__ uint32_t rows_route_row(const RowsRoute& r, uint32_t pass) {
+    if constexpr (GM == GATHER_CSR) return pass < r.n1 ? r.lo + pass : r.lo2 + (pass - r.n1);
+    if constexpr (GM == GATHER_INDICES) {
+        unsigned long long m = r.mask;
+        for (uint32_t i = 0; i < pass; i++) m &= m - 1ull;
+        return (uint32_t)__ffsll((long long)m) - 1u;
+    }
+    return 0u;
+}
 
 template <bool TL> __device__ __forceinline__ void rp_stamp(uint64_t (&st)[MTQ_ROWS_PROBE_STAMPS], int i) {
     if constexpr (TL) {
@@ -45,8 +80,9 @@ template <bool TL> __device__ __forceinline__ void rp_stamp(uint64_t (&st)[MTQ_R
     }
 }
 
-template <int DT, int MODE, bool TL>
-__global__ __launch_bounds__(1024) void qmv_rows_kernel(QmvRowsArgs a) {
+template <int DT, int MODE, bool TL, int GM>
+__device__ __forceinline__ void qmv_rows_body(const QmvRowsArgs& a) {
+    static_assert(GM == GATHER_NONE || (MODE == 0 && !TL), "routed instances are product instances");
     constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
     constexpr int GPR = 64, C = 128, R = 4;
     uint64_t st[MTQ_ROWS_PROBE_STAMPS];
@@ -55,12 +91,19 @@ __global__ __launch_bounds__(1024) void qmv_rows_kernel(QmvRowsArgs a) {
     const uint32_t gw = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const uint32_t r0 = gw * R;
     if (r0 >= a.N) return;
+    RowsRoute rt;
+    if (!rows_route<GM>(a.route, a.E, a.T, lane, rt)) return;
+    const size_t er0 = (size_t)rt.expert * a.N + r0;   // this wave's first row among the rows of all experts
+    for (uint32_t pass = 0; pass < rt.n_pass; pass++) {
+    const uint32_t trow = rows_route_row<GM>(rt, pass);
+    const uint16_t* const xrow = a.x + (size_t)trow * 4096u;
+    uint16_t* const orow = a.out + (size_t)trow * a.N;
     __builtin_amdgcn_s_setprio(3);
     uint4 xraw[2][4];
     if constexpr (MODE != 2) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            const uint4* xv = (const uint4*)(a.x + ((size_t)i * 64 + lane) * 32);
+            const uint4* xv = (const uint4*)(xrow + ((size_t)i * 64 + lane) * 32);
 #pragma unroll
             for (int v = 0; v < 4; v++) xraw[i][v] = xv[v];
         }
@@ -68,13 +111,13 @@ __global__ __launch_bounds__(1024) void qmv_rows_kernel(QmvRowsArgs a) {
     RP_KEEP_ORDER();
     uint32_t s0[R], s1[R], bb[R];
     if constexpr (MODE != 2) {
-        const uint16_t* sp = a.s + (size_t)r0 * GPR + (lane >> 1);
-        const uint16_t* bp = a.b + (size_t)r0 * GPR + lane;
+        const uint16_t* sp = a.s + er0 * GPR + (lane >> 1);
+        const uint16_t* bp = a.b + er0 * GPR + lane;
 #pragma unroll
         for (int r = 0; r < R; r++) { s0[r] = sp[r * GPR]; s1[r] = sp[r * GPR + 32]; bb[r] = bp[r * GPR]; }
     }
     RP_KEEP_ORDER();
-    const rp_u32x4* wbase = a.w + (size_t)r0 * C + lane;
+    const rp_u32x4* wbase = a.w + er0 * C + lane;
     rp_u32x4 wv[R][2];
     // (Every load at once is the fastest form here: with the loads of only one, two or three rows ahead of the row
     // being worked on, 14336 x 4096 bf16 takes 8.3, 8.5 and 9.1 us against 7.75 in the same run.)
@@ -171,13 +214,18 @@ __global__ __launch_bounds__(1024) void qmv_rows_kernel(QmvRowsArgs a) {
     tot += dpp_f32<0x140>(tot);
     // 16-lane row r of the wave now holds the total of row {0, 2, 1, 3}[r]
     const uint32_t slot = ((lane >> 4) & 1u) * 2u + (lane >> 5);
-    if ((lane & 15u) == 0) a.out[r0 + slot] = f32_to_elem_bits<DT>(tot);
+    if ((lane & 15u) == 0) orow[r0 + slot] = f32_to_elem_bits<DT>(tot);
     rp_stamp<TL>(st, 5);                                  // stored
     if constexpr (TL) {
         if (lane == 0)
             for (int i = 0; i < MTQ_ROWS_PROBE_STAMPS; i++) a.stamps[(size_t)gw * MTQ_ROWS_PROBE_STAMPS + i] = st[i];
     }
+    }   // pass
 }
+template <int DT, int MODE, bool TL>
+__global__ __launch_bounds__(1024) void qmv_rows_kernel(QmvRowsArgs a) { qmv_rows_body<DT, MODE, TL, GATHER_NONE>(a); }
+template <int DT, int GM>
+__global__ __launch_bounds__(1024) void qmv_rows_routed_kernel(QmvRowsArgs a) { qmv_rows_body<DT, 0, false, GM>(a); }
 
 // ---- one wave per row, activations shared by the workgroup: other row lengths, group sizes and 2-bit codes -----------
 // The same ownership (lane l holds chunks l, 64 + l, ... of a row, the diagonal of the 4x4x4 blocks, scales loaded per
@@ -207,10 +255,12 @@ struct QmvRowsLArgs {
     const uint16_t* x;
     uint16_t* out;
     uint32_t N;
+    const uint32_t* route;   // routed instances (see RowsRoute): expert_offsets[E + 1] or indices[T]
+    uint32_t E, T;
 };
 
-template <int DT, int BITS, int CH, int LOG2G>
-__global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) {
+template <int DT, int BITS, int CH, int LOG2G, int GM>
+__device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
     static_assert(BITS == 2 || BITS == 4, "2- or 4-bit codes");
     constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;   // 4-bit codes: one offset for every pair
     constexpr int CPC = 128 / BITS;        // codes per chunk
@@ -229,12 +279,18 @@ __global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) {
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t r0 = blockIdx.x * (blockDim.x >> 6) + wave;   // (a workgroup is 8 or 16 waves, at least C threads)
     const bool live = r0 < a.N;
-    const uint32_t rr = live ? r0 : 0u;    // idle waves of the last workgroup still prepare their chunks
+    RowsRoute rt;
+    if (!rows_route<GM>(a.route, a.E, a.T, lane, rt)) return;   // (the same for every wave of the workgroup: no barrier is left waiting)
+    const size_t rr = (size_t)rt.expert * a.N + (live ? r0 : 0u);   // idle waves of the last workgroup still prepare their chunks
+    for (uint32_t pass = 0; pass < rt.n_pass; pass++) {
+    const uint32_t trow = rows_route_row<GM>(rt, pass);
+    const uint16_t* const xrow = a.x + (size_t)trow * K;
+    uint16_t* const orow = a.out + (size_t)trow * a.N;
     __builtin_amdgcn_s_setprio(3);
     // this thread's chunk of the activations
     uint4 xraw[Q];
     if (tid < (uint32_t)C) {
-        const uint4* xv = (const uint4*)(a.x + (size_t)tid * CPC);
+        const uint4* xv = (const uint4*)(xrow + (size_t)tid * CPC);
 #pragma unroll
         for (int v = 0; v < Q; v++) xraw[v] = xv[v];
     }
@@ -244,8 +300,8 @@ __global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) {
     uint32_t sw[2] = {0u, 0u}, bw[2] = {0u, 0u};   // GPL elements each, two per dword
     const uint32_t gl = min(lane, (uint32_t)(GPR / GPL - 1));
     {
-        const uint16_t* sp = a.s + (size_t)rr * GPR;
-        const uint16_t* bp = a.b + (size_t)rr * GPR;
+        const uint16_t* sp = a.s + rr * GPR;
+        const uint16_t* bp = a.b + rr * GPR;
 #pragma unroll
         for (int i = 0; i < CH; i++) {
             const uint32_t k0 = (uint32_t)(i * 64 + (int)lane) * CPC;
@@ -264,7 +320,7 @@ __global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) {
         }
     }
     RP_KEEP_ORDER();
-    const rp_u32x4* wbase = a.w + (size_t)rr * C + lane;
+    const rp_u32x4* wbase = a.w + rr * C + lane;
     rp_u32x4 wv[CH];
     // Rows of more than four chunks per lane: the loads run four chunks ahead of the chunk being worked on and only two
     // are issued before the activations are prepared. A compute unit takes loads only as fast as earlier ones return, so
@@ -341,7 +397,10 @@ __global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) {
         }
     }
     __syncthreads();
-    if (!live) return;
+    if constexpr (GM == GATHER_NONE) {
+        if (!live) return;
+    }
+    if (GM == GATHER_NONE || live) {
 #pragma unroll
     for (int i = PRE; i < W0; i++) wv[i] = __builtin_nontemporal_load(wbase + i * 64);
     RP_KEEP_ORDER();
@@ -432,8 +491,17 @@ __global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) {
     t += dpp_f32<0x141>(t);
     t += dpp_f32<0x140>(t);
     t += __shfl_xor(t, 16, 64);
-    if (lane == 0) a.out[r0] = f32_to_elem_bits<DT>(t);
+    if (lane == 0) orow[r0] = f32_to_elem_bits<DT>(t);
+    }   // live
+    if constexpr (GM != GATHER_NONE) {
+        if (pass + 1 < rt.n_pass) __syncthreads();   // the next pass overwrites the activations in LDS
+    }
+    }   // pass
 }
+template <int DT, int BITS, int CH, int LOG2G>
+__global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) { qmv_rows_long_body<DT, BITS, CH, LOG2G, GATHER_NONE>(a); }
+template <int DT, int BITS, int CH, int LOG2G, int GM>
+__global__ __launch_bounds__(1024) void qmv_rows_long_routed_kernel(QmvRowsLArgs a) { qmv_rows_long_body<DT, BITS, CH, LOG2G, GM>(a); }
 
 template <int DT> static const void* qmv_rows_fn(int mode, bool tl) {
     switch (mode) {
@@ -443,11 +511,19 @@ template <int DT> static const void* qmv_rows_fn(int mode, bool tl) {
     }
 }
 
+template <int DT> static const void* qmv_rows_routed_fn(int gather) {
+    return gather == GATHER_CSR ? (const void*)qmv_rows_routed_kernel<DT, GATHER_CSR> : (const void*)qmv_rows_routed_kernel<DT, GATHER_INDICES>;
+}
+
+// slots: grid rows of a routed launch (the experts that can have a row), 1 for a plain one
 static int launch_rows(int dtype, const void* w, const void* s, const void* b, const void* x, void* out, uint32_t N, int mode,
-                       uint64_t* stamps, const LaunchCtx& lc) {
-    QmvRowsArgs a{(const rp_u32x4*)w, (const uint16_t*)s, (const uint16_t*)b, (const uint16_t*)x, (uint16_t*)out, N, stamps};
+                       uint64_t* stamps, const LaunchCtx& lc, int gather = GATHER_NONE, const uint32_t* route = nullptr, uint32_t E = 1,
+                       uint32_t T = 1, uint32_t slots = 1) {
+    QmvRowsArgs a{(const rp_u32x4*)w, (const uint16_t*)s, (const uint16_t*)b, (const uint16_t*)x, (uint16_t*)out, N, stamps, route, E, T};
     void* args[] = {&a};
-    const void* fn = dtype == DT_BF16 ? qmv_rows_fn<DT_BF16>(mode, stamps != nullptr) : qmv_rows_fn<DT_F16>(mode, stamps != nullptr);
+    const void* fn = gather != GATHER_NONE ? (dtype == DT_BF16 ? qmv_rows_routed_fn<DT_BF16>(gather) : qmv_rows_routed_fn<DT_F16>(gather))
+                     : dtype == DT_BF16    ? qmv_rows_fn<DT_BF16>(mode, stamps != nullptr)
+                                           : qmv_rows_fn<DT_F16>(mode, stamps != nullptr);
     // A workgroup is only a container here (no LDS, no barrier). It is sized so that the workgroups are a whole number
     // per compute unit: one of up to 16 waves up to 16384 rows (14336 rows: 256 workgroups of 14 waves, 7.88 us against
     // 7.97 as 896 workgroups of 4; 1024 rows: 256 single waves, 3.15 against 3.60), beyond that as few rounds of at most
@@ -455,7 +531,7 @@ static int launch_rows(int dtype, const void* w, const void* s, const void* b, c
     const uint32_t waves = (N + 3u) / 4u;
     const uint32_t rounds = waves <= 256u * 16u ? 1u : (waves + 256u * 8u - 1u) / (256u * 8u);
     const uint32_t wpw = (waves + 256u * rounds - 1u) / (256u * rounds);
-    hipError_t e = launch_kernel(fn, dim3((waves + wpw - 1u) / wpw), dim3(wpw * 64u), args, 0, lc);
+    hipError_t e = launch_kernel(fn, dim3((waves + wpw - 1u) / wpw, slots), dim3(wpw * 64u), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "qmv rows kernel launch");
     return ERR_OK;
 }
@@ -473,17 +549,35 @@ static int rows_long_ch(const QmvParams& p) {
 }
 
 bool qmv_rows_takes(const QmvParams& p) {
-    if (p.gather != GATHER_NONE || p.M != 1 || (p.dtype != DT_F16 && p.dtype != DT_BF16) || p.N == 0) return false;
+    if ((p.dtype != DT_F16 && p.dtype != DT_BF16) || p.N == 0) return false;
+    const bool routed = p.gather == GATHER_CSR || p.gather == GATHER_INDICES;
+    if (routed) {
+        // at most 64 experts and 64 rows (the routing is read by one wave-wide load); 4-bit codes in groups of 64 on rows
+        // of 4096, 8192 or 14336 codes (the instances that exist); every expert's block of scales as aligned as the first
+        if (!p.route || p.E == 0 || p.E > 64 || p.T == 0 || p.T > 64 || p.bits != 4 || p.group_size != 64) return false;
+        if (((size_t)p.N * (p.K / 64u) * 2u) % 8u) return false;
+    } else if (p.gather != GATHER_NONE || p.M != 1) {
+        return false;
+    }
     if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.scales % 8 || (uintptr_t)p.biases % 8 || (uintptr_t)p.out % 2) return false;
     if (p.bits == 4 && p.group_size == 64 && p.K == 4096) return p.N % 4 == 0;   // one wave per four rows
-    return rows_long_ch(p) != 0;
+    const int ch = rows_long_ch(p);
+    return routed ? ch == 4 || ch == 7 : ch != 0;
 }
 
 // Where these kernels are the fastest the library has (measured against the streaming kernel in one run, f16 / bf16, us):
 // 14336 x 4096 4-bit g64 8.11 -> 7.86; 4096 x 14336 8.60 -> 8.11 on one machine, 8.63 -> 8.73 on another; 8192 x 8192:
 // 2-bit g32 / g64 / g128 8.98 / 8.55 / 8.41 -> 6.65 / 6.16 / 6.03, 4-bit 9.63 / 9.47 / 9.27 -> 8.53 / 7.90 / 7.78.
 // Small matrices stay where they were (a workgroup here is sixteen rows: few rows leave compute units idle).
-bool qmv_rows_preferred(const QmvParams& p) { return qmv_rows_takes(p) && p.N >= 1024; }
+bool qmv_rows_preferred(const QmvParams& p) {
+    if (!qmv_rows_takes(p) || p.N < 1024) return false;
+    // Routed rows: fewer rows than experts, each streaming its expert's matrix on its own grid row. 8 experts, bf16, us,
+    // against the kernels that served these before (the one-row streaming kernel for one row, the matrix-core GEMV
+    // beyond): 14336 x 4096, 1 / 2 / 3 / 4 rows on distinct experts 10.8 -> 8.4, 17.6 -> 15.8, 22.4 -> 23.3, 28.0 -> 31.1,
+    // two rows on one expert 16.4 -> 14.0; 4096 x 14336: 9.0 -> 8.0, 16.6 -> 14.6, 41.8 -> 21.0, 34.8 -> 27.8, 15.8 -> 13.4.
+    if (p.gather != GATHER_NONE) return p.T < p.E && p.T <= (p.K == 4096 ? 2u : 4u);
+    return true;
+}
 
 template <int DT, int LOG2G> static const void* rows_long_fn_g(int bits, int ch) {
     if (bits == 4) {
@@ -498,14 +592,23 @@ template <int DT, int LOG2G> static const void* rows_long_fn_g(int bits, int ch)
 template <int DT> static const void* rows_long_fn(int bits, int ch, uint32_t G) {
     return G == 32 ? rows_long_fn_g<DT, 5>(bits, ch) : G == 64 ? rows_long_fn_g<DT, 6>(bits, ch) : rows_long_fn_g<DT, 7>(bits, ch);
 }
+template <int DT, int GM> static const void* rows_long_routed_fn(int ch) {   // 4-bit codes in groups of 64
+    return ch == 4 ? (const void*)qmv_rows_long_routed_kernel<DT, 4, 4, 6, GM> : ch == 7 ? (const void*)qmv_rows_long_routed_kernel<DT, 4, 7, 6, GM> : nullptr;
+}
 
 int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
     if (!qmv_rows_takes(p)) return fail(ERR_UNSUPPORTED, "qmv rows kernels: one activation row, 2- or 4-bit codes, f16 / bf16, rows of 4096, 8192, 14336 or 16384 codes");
-    if (p.bits == 4 && p.group_size == 64 && p.K == 4096) return launch_rows(p.dtype, p.w, p.scales, p.biases, p.x, p.out, p.N, 0, nullptr, lc);
+    const bool routed = p.gather != GATHER_NONE;
+    const uint32_t slots = routed ? (p.T < p.E ? p.T : p.E) : 1u;   // the experts that can have a row
+    if (p.bits == 4 && p.group_size == 64 && p.K == 4096)
+        return launch_rows(p.dtype, p.w, p.scales, p.biases, p.x, p.out, p.N, 0, nullptr, lc, p.gather, p.route, p.E, p.T, slots);
     const int ch = rows_long_ch(p);
-    QmvRowsLArgs a{(const rp_u32x4*)p.w, (const uint16_t*)p.scales, (const uint16_t*)p.biases, (const uint16_t*)p.x, (uint16_t*)p.out, p.N};
+    QmvRowsLArgs a{(const rp_u32x4*)p.w, (const uint16_t*)p.scales, (const uint16_t*)p.biases, (const uint16_t*)p.x, (uint16_t*)p.out, p.N, p.route, p.E, p.T};
     void* args[] = {&a};
-    const void* fn = p.dtype == DT_BF16 ? rows_long_fn<DT_BF16>(p.bits, ch, p.group_size) : rows_long_fn<DT_F16>(p.bits, ch, p.group_size);
+    const void* fn = p.gather == GATHER_CSR       ? (p.dtype == DT_BF16 ? rows_long_routed_fn<DT_BF16, GATHER_CSR>(ch) : rows_long_routed_fn<DT_F16, GATHER_CSR>(ch))
+                     : p.gather == GATHER_INDICES ? (p.dtype == DT_BF16 ? rows_long_routed_fn<DT_BF16, GATHER_INDICES>(ch) : rows_long_routed_fn<DT_F16, GATHER_INDICES>(ch))
+                     : p.dtype == DT_BF16         ? rows_long_fn<DT_BF16>(p.bits, ch, p.group_size)
+                                                  : rows_long_fn<DT_F16>(p.bits, ch, p.group_size);
     if (!fn) return fail(ERR_UNSUPPORTED, "qmv rows kernels: no instance for this row length and group size");
     // Sixteen rows per workgroup, eight for the long rows. One workgroup of sixteen per compute unit (4096 x 14336: 256
     // of them) is the fastest form on some machines of the pool and 9 % behind on others, where the same launch as 512
@@ -513,7 +616,7 @@ int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
     // 7.70 on two others); shorter rows keep sixteen (8192 x 8192: 4-bit 8.00 / 7.97, 2-bit 6.27 / 6.95).
     const uint32_t block = ch > 4 ? 512u : 1024u;
     if (block < 64u * (uint32_t)ch) return fail(ERR_UNSUPPORTED, "qmv rows kernels: workgroup smaller than the row's chunks");   // (thread t prepares chunk t)
-    hipError_t e = launch_kernel(fn, dim3((p.N + block / 64u - 1u) / (block / 64u)), dim3(block), args, 0, lc);
+    hipError_t e = launch_kernel(fn, dim3((p.N + block / 64u - 1u) / (block / 64u), slots), dim3(block), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "qmv long rows kernel launch");
     return ERR_OK;
 }

@@ -178,3 +178,72 @@ def test_one_routed_row_on_rows_the_streaming_kernel_cannot_tile(oracle, dt, K):
     assert rel_err(unpack_f32(out.read_bytes(), dt), exp) <= 1e-2
     for buf in (w, s, b, x, out, r, off):
         buf.free()
+
+
+@pytest.fixture
+def wave_per_row_kernels():
+    lib = _lib.load()
+    assert lib.mtq_set_option(b"qmv.kernel", 3) == 0
+    yield
+    lib.mtq_set_option(b"qmv.kernel", 0)
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("N,K,kernel", [(20, 4096, "qmv_rows_routed_kernel"), (1028, 4096, "qmv_rows_routed_kernel"), (19, 14336, "qmv_rows_long_routed_kernel"),
+                                        (1030, 8192, "qmv_rows_long_routed_kernel")])
+def test_routed_rows_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, wave_per_row_kernels):
+    """The wave-per-row GEMV kernels with a grid row per expert that has a row (their automatic range is up to four rows
+    on fewer rows than experts from 1024 weight rows; forced here below that too): one row, two experts, the same expert
+    twice (a second pass over its matrix), seven rows, both routing views, CSR offsets that end short or step back, ids
+    that name no expert (those output rows keep their bytes), ragged last workgroups, behind a cache flush."""
+    import metaltile_amd as m
+    bits, G, E = 4, 64, 8
+    rb = N * dt.size_bytes
+    for ids in ([3], [1, 6], [4, 4], [2, 2, 5], [0, 1, 2, 3, 4, 5, 7]):
+        T = len(ids)
+        idn = np.array(ids, dtype="<u4")
+        c = make_case(8700 + N + K + T, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
+        exp = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=idn, f64=True, threads=8)
+        exp = oracle.round_through(exp.astype(np.float32), ODT[dt]).reshape(T, N)
+        w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                      GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+        for view, route, fn in (("csr", _offsets(idn, E), ops.gather_qmv_csr), ("indices", idn, ops.gather_qmv_indices)):
+            print(f"[case] routed rows {view} {dt.name} N{N} K{K} ids={ids}", flush=True)
+            rc, launches, _, n = ops.plan("gather_" + view, dt, bits, G, 1, N, K, E, T)
+            assert rc == 0 and n == 1 and kernel in launches[0][0] and launches[0][1][1] == T, launches
+            out, r = GpuBuffer.from_bytes(b"\xab" * (T * rb + 64)), GpuBuffer.from_bytes(route.tobytes())
+            m.GpuRunner(0).flush_slc()
+            fn(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+            raw = out.read_bytes()
+            assert raw[T * rb:] == b"\xab" * 64
+            assert rel_err(unpack_f32(raw[:T * rb], dt), exp.reshape(-1)) <= 1e-2, view
+            out.free(); r.free()
+        if T == 3:
+            # the same rows under offsets that end short (the last row goes to expert 0) and offsets that step back
+            #                      e: 0  1  2  3  4  5  6  7
+            for off, ids_equiv, label in (([0, 0, 0, 2, 2, 2, 2, 2, 2], [2, 2, 0], "tail to expert 0"),
+                                          ([0, 1, 1, 3, 2, 2, 3, 3, 3], [0, 2, 2], "an offset that steps back")):
+                e2 = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=np.array(ids_equiv, dtype="<u4"),
+                                       f64=True, threads=8)
+                e2 = oracle.round_through(e2.astype(np.float32), ODT[dt])
+                via = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, expert_offsets=np.array(off, dtype="<u4"),
+                                        f64=True, threads=8)
+                assert np.array_equal(oracle.round_through(via.astype(np.float32), ODT[dt]), e2), label   # the rule, as the oracle reads it
+                print(f"[case] routed rows csr {dt.name} N{N} K{K} {label}", flush=True)
+                out, r = GpuBuffer(T * rb), GpuBuffer.from_bytes(np.array(off, dtype="<u4").tobytes())
+                ops.gather_qmv_csr(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+                assert rel_err(unpack_f32(out.read_bytes(), dt), e2) <= 1e-2, label
+                out.free(); r.free()
+            nameless = np.array([7, E + 1, 2], dtype="<u4")
+            e3 = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=np.array([7, 0, 2], dtype="<u4"), f64=True, threads=8)
+            e3 = oracle.round_through(e3.astype(np.float32), ODT[dt]).reshape(T, N)
+            print(f"[case] routed rows indices {dt.name} N{N} K{K} an id that names no expert", flush=True)
+            out, r = GpuBuffer.from_bytes(b"\xab" * (T * rb)), GpuBuffer.from_bytes(nameless.tobytes())
+            ops.gather_qmv_indices(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+            raw = out.read_bytes()
+            assert raw[rb:2 * rb] == b"\xab" * rb
+            got = unpack_f32(raw, dt).reshape(T, N)
+            assert rel_err(got[0], e3[0]) <= 1e-2 and rel_err(got[2], e3[2]) <= 1e-2
+            out.free(); r.free()
+        for buf in (w, s, b, x):
+            buf.free()

@@ -159,12 +159,20 @@ def test_benchmark_configurations_are_routed_as_documented():
     assert "qmm_direct_kernel<2, 6," in ks[0]          # other code widths stay on the register-staged tiles
     ks, ls = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 32)   # 4 rows per expert: the routed 16-row GEMV
     assert "qmv_wide_kernel<2, 64, 2, 2, 2>" in ks[0] and ls[0][1][:2] == (28, 8) and ls[0][2][0] == 1024
+    for T in (1, 2, 4):   # the down projection's experts: up to four rows on the routed one-row-per-wave kernel, eight-row workgroups
+        ks, ls = kernels("gather_csr", DType.BF16, 4, 64, 1, 4096, 14336, 8, T)
+        assert "qmv_rows_long_routed_kernel<2, 4, 7, 6, 1>" in ks[0] and ls[0][1][:2] == (512, T) and ls[0][2][0] == 512, ls
+    ks, _ = kernels("gather_csr", DType.BF16, 4, 64, 1, 4096, 14336, 8, 5)
+    assert "qmv_mfma_kernel<2, 4," in ks[0]
+    ks, ls = kernels("gather_indices", DType.BF16, 4, 64, 1, 2048, 2048, 8, 1)           # other row lengths: the one-row streaming kernel
+    assert "qmv_stream_kernel<2, 4, 1," in ks[0]
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 16)           # 2 rows per expert: 8-row passes
     assert "qmv_mfma_kernel<2, 4," in ks[0]
     for view in ("gather_csr", "gather_indices"):      # fewer rows than experts: a grid row per row, not per expert
         for T, E in ((1, 8), (2, 8), (7, 8), (8, 128), (32, 128)):
             ks, ls = kernels(view, DType.BF16, 4, 64, 1, 14336, 4096, E, T)
-            kernel = "qmv_stream_kernel<2, 4, 1," if T == 1 and E <= 64 else "qmv_mfma_kernel<2, 4,"   # one row: the one-row kernel
+            # one or two rows on at most 64 experts of 14336 x 4096: the routed wave-per-four-rows kernel
+            kernel = "qmv_rows_routed_kernel<2, " if T <= 2 and E <= 64 else "qmv_mfma_kernel<2, 4,"
             assert kernel in ks[0] and ls[0][1][1] == T, (view, T, E, ls)
         ks, ls = kernels(view, DType.BF16, 4, 64, 1, 2048, 768, 128, 33)   # (more than 32 rows: a grid row per expert)
         assert ls[0][1][1] == 128
