@@ -53,6 +53,7 @@ template <int GM> __device__ __forceinline__ bool rows_route(const uint32_t* rou
         if (r.n_pass == 0) return false;
         r.expert = __builtin_amdgcn_readfirstlane(r.expert);
     }
+    if constexpr (GM == GATHER_SINGLE) r.expert = min(route[0], E - 1u);   // one row on the expert named on the device; an id past the last expert names the last
     if constexpr (GM == GATHER_INDICES) {
         r.expert = __builtin_amdgcn_readfirstlane(ids_slot_expert(route, E, T, blockIdx.y, lane));
         if (r.expert == 0xFFFFFFFFu) return false;
@@ -512,7 +513,9 @@ template <int DT> static const void* qmv_rows_fn(int mode, bool tl) {
 }
 
 template <int DT> static const void* qmv_rows_routed_fn(int gather) {
-    return gather == GATHER_CSR ? (const void*)qmv_rows_routed_kernel<DT, GATHER_CSR> : (const void*)qmv_rows_routed_kernel<DT, GATHER_INDICES>;
+    return gather == GATHER_CSR       ? (const void*)qmv_rows_routed_kernel<DT, GATHER_CSR>
+           : gather == GATHER_INDICES ? (const void*)qmv_rows_routed_kernel<DT, GATHER_INDICES>
+                                      : (const void*)qmv_rows_routed_kernel<DT, GATHER_SINGLE>;
 }
 
 // slots: grid rows of a routed launch (the experts that can have a row), 1 for a plain one
@@ -550,11 +553,13 @@ static int rows_long_ch(const QmvParams& p) {
 
 bool qmv_rows_takes(const QmvParams& p) {
     if ((p.dtype != DT_F16 && p.dtype != DT_BF16) || p.N == 0) return false;
-    const bool routed = p.gather == GATHER_CSR || p.gather == GATHER_INDICES;
+    const bool routed = p.gather == GATHER_CSR || p.gather == GATHER_INDICES || p.gather == GATHER_SINGLE;
     if (routed) {
-        // at most 64 experts and 64 rows (the routing is read by one wave-wide load); 4-bit codes in groups of 64 on rows
-        // of 4096, 8192 or 14336 codes (the instances that exist); every expert's block of scales as aligned as the first
-        if (!p.route || p.E == 0 || p.E > 64 || p.T == 0 || p.T > 64 || p.bits != 4 || p.group_size != 64) return false;
+        // at most 64 experts and 64 rows (the routing is read by one wave-wide load; the single-index form reads one id
+        // and takes any number of experts); 4-bit codes in groups of 64 on rows of 4096, 8192 or 14336 codes (the
+        // instances that exist); every expert's block of scales as aligned as the first
+        if (!p.route || p.E == 0 || p.bits != 4 || p.group_size != 64) return false;
+        if (p.gather != GATHER_SINGLE && (p.E > 64 || p.T == 0 || p.T > 64)) return false;
         if (((size_t)p.N * (p.K / 64u) * 2u) % 8u) return false;
     } else if (p.gather != GATHER_NONE || p.M != 1) {
         return false;
@@ -575,6 +580,7 @@ bool qmv_rows_preferred(const QmvParams& p) {
     // against the kernels that served these before (the one-row streaming kernel for one row, the matrix-core GEMV
     // beyond): 14336 x 4096, 1 / 2 / 3 / 4 rows on distinct experts 10.8 -> 8.4, 17.6 -> 15.8, 22.4 -> 23.3, 28.0 -> 31.1,
     // two rows on one expert 16.4 -> 14.0; 4096 x 14336: 9.0 -> 8.0, 16.6 -> 14.6, 41.8 -> 21.0, 34.8 -> 27.8, 15.8 -> 13.4.
+    if (p.gather == GATHER_SINGLE) return true;   // (one row, as the plain launch)
     if (p.gather != GATHER_NONE) return p.T < p.E && p.T <= (p.K == 4096 ? 2u : 4u);
     return true;
 }
@@ -599,7 +605,7 @@ template <int DT, int GM> static const void* rows_long_routed_fn(int ch) {   // 
 int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
     if (!qmv_rows_takes(p)) return fail(ERR_UNSUPPORTED, "qmv rows kernels: one activation row, 2- or 4-bit codes, f16 / bf16, rows of 4096, 8192, 14336 or 16384 codes");
     const bool routed = p.gather != GATHER_NONE;
-    const uint32_t slots = routed ? (p.T < p.E ? p.T : p.E) : 1u;   // the experts that can have a row
+    const uint32_t slots = routed && p.gather != GATHER_SINGLE ? (p.T < p.E ? p.T : p.E) : 1u;   // the experts that can have a row
     if (p.bits == 4 && p.group_size == 64 && p.K == 4096)
         return launch_rows(p.dtype, p.w, p.scales, p.biases, p.x, p.out, p.N, 0, nullptr, lc, p.gather, p.route, p.E, p.T, slots);
     const int ch = rows_long_ch(p);
@@ -607,6 +613,7 @@ int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
     void* args[] = {&a};
     const void* fn = p.gather == GATHER_CSR       ? (p.dtype == DT_BF16 ? rows_long_routed_fn<DT_BF16, GATHER_CSR>(ch) : rows_long_routed_fn<DT_F16, GATHER_CSR>(ch))
                      : p.gather == GATHER_INDICES ? (p.dtype == DT_BF16 ? rows_long_routed_fn<DT_BF16, GATHER_INDICES>(ch) : rows_long_routed_fn<DT_F16, GATHER_INDICES>(ch))
+                     : p.gather == GATHER_SINGLE  ? (p.dtype == DT_BF16 ? rows_long_routed_fn<DT_BF16, GATHER_SINGLE>(ch) : rows_long_routed_fn<DT_F16, GATHER_SINGLE>(ch))
                      : p.dtype == DT_BF16         ? rows_long_fn<DT_BF16>(p.bits, ch, p.group_size)
                                                   : rows_long_fn<DT_F16>(p.bits, ch, p.group_size);
     if (!fn) return fail(ERR_UNSUPPORTED, "qmv rows kernels: no instance for this row length and group size");

@@ -247,3 +247,33 @@ def test_routed_rows_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, wave_
             out.free(); r.free()
         for buf in (w, s, b, x):
             buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("N,K,kernel", [(1028, 4096, "qmv_rows_routed_kernel"), (40, 14336, "qmv_rows_long_routed_kernel"), (1030, 8192, "qmv_rows_long_routed_kernel")])
+def test_single_index_expert_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, wave_per_row_kernels):
+    """One row against the expert whose index is read on the device (the reference's expert-indexed GEMV,
+    crates/metaltile-std/src/ffai/dequant_gemv_expert_indexed.rs): the first, a middle and the last expert, and an index
+    past the last expert, which names the last one as in the other kernels of this ABI."""
+    import metaltile_amd as m
+    bits, G, E = 4, 64, 6
+    c = make_case(8800 + N + K, dt, bits, G, 1, N, K, E=E, bias_rule="midpoint")
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    rb = N * dt.size_bytes
+    for idx in (0, 3, E - 1, E + 7):
+        e = min(idx, E - 1)
+        exp = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, 1, K, N, E, bits, G, indices=np.array([e], dtype="<u4"), f64=True, threads=8)
+        exp = oracle.round_through(exp.astype(np.float32), ODT[dt])
+        print(f"[case] single-index expert {dt.name} N{N} K{K} index {idx}", flush=True)
+        rc, launches, _, n = ops.plan("gather_single", dt, bits, G, 1, N, K, E, 1)
+        assert rc == 0 and n == 1 and kernel in launches[0][0] and launches[0][1][1] == 1, launches
+        out, ei = GpuBuffer.from_bytes(b"\xab" * (rb + 64)), GpuBuffer.from_bytes(np.array([idx], dtype="<u4").tobytes())
+        m.GpuRunner(0).flush_slc()
+        ops.gather_qmv_single(dt, bits, G, w, s, b, x, ei, out, N, K, E)
+        raw = out.read_bytes()
+        assert raw[rb:] == b"\xab" * 64
+        assert rel_err(unpack_f32(raw[:rb], dt), exp) <= 1e-2, idx
+        out.free(); ei.free()
+    for buf in (w, s, b, x):
+        buf.free()
