@@ -36,7 +36,8 @@ sweep (f16, 8192 x 8192, batch 1 and 4); `--workload batch` a decode batch of
 128256 x 4096 lm-head), by the exact-dequant kernel name mt_qmm; `--workload
 qkv` / `gated_norm` the fused one-launch decode pieces (Q + K + V projections;
 gated RMSNorm + out projection at the reference's bench shape); `--workload
-rows_probe` the headline gate / up launch taken apart (the shipped kernel, the
+gather_decode` one token's top-2 routed gate / up / down launches over 8
+experts (the routed wave-per-row kernels); `--workload rows_probe` the headline gate / up launch taken apart (the shipped kernel, the
 streaming kernel it replaced, a launch that only reads the same bytes, and the
 shipped kernel without its arithmetic / with its weight loads only, plus its
 per-wave timeline), which is where the distance to the HBM peak is accounted
@@ -67,7 +68,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--layers", type=int, default=8, help="distinct MLP weight sets streamed per step")
     ap.add_argument("--workload", default="qmv",
-                    choices=["qmv", "qkv", "gated_norm", "qmm", "batch", "gather", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep", "rows_probe"],
+                    choices=["qmv", "qkv", "gated_norm", "qmm", "batch", "gather", "gather_decode", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep", "rows_probe"],
                     help="qmv is the headline (its line also carries qmm M=512 and the gather as secondary legs); "
                          "qmm / gather report those configurations alone; sweep the bit-width / group-size cells; "
                          "copy runs only the known-size copy kernel (counter calibration); read times a kernel that only reads the "
@@ -420,6 +421,57 @@ def leg_gather(a, runner, info):
     }
 
 
+def leg_gather_decode(a, runner, info):
+    """One token through a Mixtral-style layer's experts (8 experts, top-2): three expert-routed launches per step --
+    gate and up (experts of 14336 x 4096) and down (experts of 4096 x 14336), two rows on two experts each -- under the
+    CSR name, over 3 rotating copies of the experts (cold). GB/s on the bytes of the two experts that are hit."""
+    import numpy as np
+    import metaltile_amd as m
+    from metaltile_amd import DType, GpuBuffer
+    from metaltile_amd.synth import make_case
+    dt = DType.BF16
+    E, G, T = 8, 64, 2
+    ids = np.array([2, 5], dtype=np.int64)
+    offsets = np.concatenate([[0], np.cumsum(np.bincount(ids, minlength=E))]).astype("<u4")
+    shapes = [(14336, 4096), (14336, 4096), (4096, 14336)]
+    specs, keep, step_bytes, by_shape_bytes = [], [], 0, []
+    cases = {nk: make_case(8100 + i, dt, 4, G, T, nk[0], nk[1], E=E) for i, nk in enumerate(sorted(set(shapes)))}
+    for copy in range(3):
+        for (n, k) in shapes:
+            c = cases[(n, k)]
+            bufs = {"x": GpuBuffer.from_bytes(c.x_bytes), "weight_packed": GpuBuffer.from_bytes(c.w.tobytes()),
+                    "scales": GpuBuffer.from_bytes(c.scales_bytes), "biases": GpuBuffer.from_bytes(c.biases_bytes),
+                    "expert_offsets": GpuBuffer.from_bytes(offsets.tobytes()), "out": GpuBuffer(T * n * 2)}
+            keep.append(bufs)
+            specs.append(("mt_moe_gather_qmm_int4", dt, bufs, {"k_in": k, "m_out": n, "n_experts": E, "group_size": G}))
+    launch_bytes = T * (14336 * 4096 // 2 + 2 * 14336 * (4096 // G) * 2) + T * 4096 * 2 + T * 14336 * 2 + 4 * (E + 1)   # gate / up; down differs by the row bytes only
+    wall_us, chain_us, clock = timed_chain(a, runner, specs)
+    kern_avg = chain_us / (a.steps * len(specs))
+    per, _, _ = runner.dispatch_chain(specs, repeat=min(a.steps, 20), per_kernel=True)
+    per = np.array(per).reshape(-1, len(specs))
+    by_shape = {"gate_up_8x14336x4096": round(float(per[:, [i for i in range(len(specs)) if i % 3 != 2]].mean()), 3),
+                "down_8x4096x14336": round(float(per[:, 2::3].mean()), 3)}
+    from metaltile_amd import ops
+    kernels = {f"{n}x{k}": ops.plan("gather_csr", dt, 4, G, 1, n, k, E, T)[1][0][0].split("(")[0].replace("void ", "") for n, k in sorted(set(shapes))}
+    for bufs in keep:
+        for b in bufs.values():
+            b.free()
+    return {
+        "metric": "gather_qmv GB/s on unique-expert bytes, one token top-2 of 8 experts (gate, up 14336x4096; down 4096x14336; 4-bit g64 bf16)",
+        "value": round(launch_bytes * len(specs) * a.steps / wall_us / 1e3, 1), "unit": "GB/s",
+        "ms_per_step": round(wall_us / a.steps / 1e3, 5), "dtype": "bf16",
+        "config": {"workload": "gather_qmv E=8, 2 (token,expert) rows on 2 experts, gate / up / down of one layer per 3 launches",
+                   "launches_per_step": len(specs), "bytes_per_launch": launch_bytes, "weights": "cold (3 rotating copies of the experts)",
+                   "device": info["name"] or info["arch"]},
+        "roofline": {"bound": "hbm", "achieved": round(launch_bytes / kern_avg / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(launch_bytes / kern_avg / 1e3 / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": launch_bytes,
+                     "kernel": "; ".join(f"{v} ({k})" for k, v in kernels.items()),
+                     "avg_launch_us_timed_region": round(kern_avg, 3), "clock": clock, "peak_basis": hbm_peak_basis(info),
+                     "per_kernel_events": {"avg_us": round(float(per.mean()), 3), "median_us": round(float(np.median(per)), 3),
+                                           "min_us": round(float(per.min()), 3), "avg_us_by_shape": by_shape}},
+    }
+
+
 def leg_sweep(a, runner, info):
     """Bit widths {2, 4, 8} x group sizes {32, 64, 128} x batch {1, 4}, W[8192, 8192], f16, through the typed
     entry point mtq_qmv: per cell the kernels' own durations (GPU timestamps attached to each launch) over
@@ -636,6 +688,11 @@ def main():
 
     if a.workload == "gather":
         out.update(leg_gather(a, runner, info))
+        print(json.dumps(out))
+        return
+
+    if a.workload == "gather_decode":
+        out.update(leg_gather_decode(a, runner, info))
         print(json.dumps(out))
         return
 
