@@ -269,11 +269,11 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
     constexpr int C = 64 * CH;             // chunks per row
     constexpr int K = C * CPC;
     constexpr int GPR = K >> LOG2G;        // groups per row
-    constexpr int GPL = GPR > 128 ? 4 : GPR > 64 ? 2 : 1;   // groups a lane owns in the bias term (lanes below GPR / GPL)
+    constexpr int GPL = GPR > 256 ? 8 : GPR > 128 ? 4 : GPR > 64 ? 2 : 1;   // groups a lane owns in the bias term (lanes below GPR / GPL)
     constexpr int SPG = (1 << LOG2G) / (CPC / 2);            // half chunks per group
     constexpr int NH = (1 << LOG2G) < CPC ? 2 : 1;           // groups a chunk spans: its halves are then accumulated and scaled apart
     static_assert(C <= 1024, "one thread per chunk");
-    static_assert(LOG2G >= 5 && LOG2G <= 7 && GPR % GPL == 0 && GPR / GPL <= 64 && SPG >= 1, "groups of 32, 64 or 128 codes, at most 256 per row");
+    static_assert(LOG2G >= 5 && LOG2G <= 7 && GPR % GPL == 0 && GPR / GPL <= 64 && SPG >= 1, "groups of 32, 64 or 128 codes, at most 512 per row");
     __shared__ __align__(16) uint32_t xp_lds[Q][C][4];   // [quarter][chunk][4 pair dwords]
     __shared__ __align__(16) float xs_lds[2 * C];        // activation sum of each half chunk
     __shared__ __align__(16) float xm_lds[BITS == 2 ? 2 * C : 4];   // 2-bit codes: the sum weighted with the pairs' offsets
@@ -298,7 +298,7 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
     RP_KEEP_ORDER();
     // scales of the two halves of this lane's CH chunks, and for the bias term scales and biases of groups GPL lane .. + GPL - 1
     uint32_t sc[CH][NH];
-    uint32_t sw[2] = {0u, 0u}, bw[2] = {0u, 0u};   // GPL elements each, two per dword
+    uint32_t sw[4] = {0u, 0u, 0u, 0u}, bw[4] = {0u, 0u, 0u, 0u};   // GPL elements each, two per dword
     const uint32_t gl = min(lane, (uint32_t)(GPR / GPL - 1));
     {
         const uint16_t* sp = a.s + rr * GPR;
@@ -309,7 +309,11 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
             sc[i][0] = sp[k0 >> LOG2G];
             if constexpr (NH == 2) sc[i][1] = sp[(k0 + CPC / 2) >> LOG2G];
         }
-        if constexpr (GPL == 4) {
+        if constexpr (GPL == 8) {   // (rows of 448 groups: 896 bytes, the operands 16-byte aligned)
+            const uint4 sv = ((const uint4*)sp)[gl], bv = ((const uint4*)bp)[gl];
+            sw[0] = sv.x; sw[1] = sv.y; sw[2] = sv.z; sw[3] = sv.w;
+            bw[0] = bv.x; bw[1] = bv.y; bw[2] = bv.z; bw[3] = bv.w;
+        } else if constexpr (GPL == 4) {
             const uint2 sv = ((const uint2*)sp)[gl], bv = ((const uint2*)bp)[gl];
             sw[0] = sv.x; sw[1] = sv.y; bw[0] = bv.x; bw[1] = bv.y;
         } else if constexpr (GPL == 2) {
@@ -548,10 +552,13 @@ static int rows_long_ch(const QmvParams& p) {
     if (p.bits != 2 && p.bits != 4) return 0;
     const uint32_t G = p.group_size, cpc = 128u / (uint32_t)p.bits;
     if (G != 32 && G != 64 && G != 128) return 0;
-    if (p.K % (64u * cpc) || p.K / G > 256u || (p.K / G) % 4u) return 0;
+    if (p.K % (64u * cpc) || p.K / G > 512u || (p.K / G) % 8u) return 0;
     const uint32_t ch = p.K / (64u * cpc);
-    if (p.bits == 4 && (ch == 4 || ch == 7)) return (int)ch;     // 8192, 14336 codes
-    if (p.bits == 2 && (ch == 2 || ch == 4)) return (int)ch;     // 8192, 16384 codes
+    if (p.K / G > 256u && ((uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)) return 0;   // (a lane's eight groups of the bias term: one 16-byte load)
+    // 8192, 14336, 28672 codes (16384, in workgroups of eight rows as for 14336, is behind the streaming kernel:
+    // 8192 x 16384 16.5 us against 14.8)
+    if (p.bits == 4 && (ch == 4 || ((ch == 7 || ch == 14) && G >= 64))) return (int)ch;
+    if (p.bits == 2 && (ch == 2 || ch == 4) && p.K / G <= 256u) return (int)ch;     // 8192, 16384 codes
     return 0;
 }
 
@@ -586,13 +593,24 @@ bool qmv_rows_preferred(const QmvParams& p) {
     // two rows on one expert 16.4 -> 14.0; 4096 x 14336: 9.0 -> 8.0, 16.6 -> 14.6, 41.8 -> 21.0, 34.8 -> 27.8, 15.8 -> 13.4.
     if (p.gather == GATHER_SINGLE) return true;   // (one row, as the plain launch)
     if (p.gather != GATHER_NONE) return p.T < p.E && p.T <= (p.K == 4096 ? 2u : 4u);
+    // Large launches have a steady state, and there the streaming kernel is ahead again (bf16, us, streaming / these):
+    // rows of 4096 codes, 28672 / 57344 / 128256 rows 13.1 / 13.5, 22.6 / 24.1, 47.6 / 50.4 (14336 rows: 8.1 / 7.85);
+    // rows of 8192, 16384 / 28672 rows 14.7 / 14.3, 22.5 / 23.0; rows of 14336, 8192 / 14336 rows 14.3 / 13.2, 21.7 / 21.3.
+    // Rows of 28672 codes stay here at every size (4096 / 8192 / 16384 rows 14.6 / 12.1, 24.5 / 22.3, 51.8 / 42.1), and so
+    // do 2-bit codes (28672 x 8192: 19.7 / 17.6).
+    if (p.bits == 4 && p.K == 4096) return p.N <= 16384;
+    if (p.bits == 4 && p.K == 8192) return p.N <= 20480;
+    if (p.bits == 4 && p.K == 14336) return p.N <= 16384;
     return true;
 }
 
 template <int DT, int LOG2G> static const void* rows_long_fn_g(int bits, int ch) {
     if (bits == 4) {
         if (ch == 4) return (const void*)qmv_rows_long_kernel<DT, 4, 4, LOG2G>;
-        if constexpr (LOG2G >= 6) return (const void*)qmv_rows_long_kernel<DT, 4, 7, LOG2G>;   // (14336 codes in groups of 32: 448 groups per row)
+        if constexpr (LOG2G >= 6) {   // (14336 / 28672 codes in groups of 32: 448 / 896 groups per row, 448 of which need 16-byte aligned scales)
+            if (ch == 7) return (const void*)qmv_rows_long_kernel<DT, 4, 7, LOG2G>;
+            if (ch == 14) return (const void*)qmv_rows_long_kernel<DT, 4, 14, LOG2G>;
+        }
         return nullptr;
     }
     if (ch == 2) return (const void*)qmv_rows_long_kernel<DT, 2, 2, LOG2G>;
@@ -625,7 +643,7 @@ int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
     // of them) is the fastest form on some machines of the pool and 9 % behind on others, where the same launch as 512
     // workgroups of eight holds (same run, 1024 / 512 threads: 7.34 / 7.40 us on one machine, 8.19 / 7.48 and 8.60 /
     // 7.70 on two others); shorter rows keep sixteen (8192 x 8192: 4-bit 8.00 / 7.97, 2-bit 6.27 / 6.95).
-    const uint32_t block = ch > 4 ? 512u : 1024u;
+    const uint32_t block = ch > 8 ? 1024u : ch > 4 ? 512u : 1024u;   // (28672 codes: 896 chunks to prepare)
     if (block < 64u * (uint32_t)ch) return fail(ERR_UNSUPPORTED, "qmv rows kernels: workgroup smaller than the row's chunks");   // (thread t prepares chunk t)
     hipError_t e = launch_kernel(fn, dim3((p.N + block / 64u - 1u) / (block / 64u), slots), dim3(block), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "qmv long rows kernel launch");

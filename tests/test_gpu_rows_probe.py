@@ -69,12 +69,13 @@ def test_rows_probe_matches_oracle(oracle, N):
 
 @pytest.mark.parametrize("dt_name", ["F16", "BF16"])
 @pytest.mark.parametrize("bits,G,N,K", [(2, 32, 50, 8192), (2, 64, 1, 8192), (2, 128, 8192, 8192), (2, 64, 33, 16384), (2, 32, 8192, 8192),
-                                        (4, 32, 50, 8192), (4, 64, 8192, 8192), (4, 128, 17, 8192), (4, 128, 40, 14336)])
+                                        (4, 32, 50, 8192), (4, 64, 8192, 8192), (4, 128, 17, 8192), (4, 128, 40, 14336),
+                                        (4, 64, 33, 28672), (4, 128, 1030, 28672)])
 def test_one_row_per_wave_kernel_other_widths_and_groups(oracle, dt_name, bits, G, N, K):
     """The one-row-per-wave kernel on the shapes it takes beyond the two of the headline: 2-bit codes (made operands in
     place, with an offset that depends on the crumb's position) and 4-bit codes in groups of 32 / 64 / 128 on rows of
-    8192, 14336 and 16384 codes, forced with qmv.kernel = 3, ragged last workgroups, behind a cache flush, against the
-    f64 oracle on full-range codes."""
+    8192, 14336, 16384 (2-bit) and 28672 codes (the last with eight groups of the bias term per lane), forced with
+    qmv.kernel = 3, ragged last workgroups, behind a cache flush, against the f64 oracle on full-range codes."""
     import metaltile_amd as m
     from metaltile_amd import DType, GpuBuffer, ops, _lib
     from metaltile_amd.synth import make_case
@@ -108,7 +109,8 @@ def test_shapes_the_one_row_per_wave_kernel_refuses():
     lib = _lib.load()
     assert lib.mtq_set_option(b"qmv.kernel", 3) == 0
     try:
-        for bits, G, K in ((4, 32, 14336), (8, 64, 8192), (4, 64, 11008), (2, 16, 8192), (4, 64, 2048), (3, 64, 8192)):
+        for bits, G, K in ((4, 32, 14336), (8, 64, 8192), (4, 64, 11008), (2, 16, 8192), (4, 64, 2048), (3, 64, 8192), (4, 32, 28672), (2, 32, 16384), (4, 64, 16384),
+                           (4, 64, 57344)):
             rc, launches, _, _ = ops.plan("qmv", DType.F16, bits, G, 1, 4096, K)
             assert rc == 0 and "qmv_rows" not in launches[0][0], (bits, G, K, launches[0][0])
     finally:
