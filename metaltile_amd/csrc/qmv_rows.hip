@@ -595,12 +595,11 @@ bool qmv_rows_preferred(const QmvParams& p) {
     if (p.gather != GATHER_NONE) return p.T < p.E && p.T <= (p.K == 4096 ? 2u : 4u);
     // Large launches have a steady state, and there the streaming kernel is ahead again (bf16, us, streaming / these):
     // rows of 4096 codes, 28672 / 57344 / 128256 rows 13.1 / 13.5, 22.6 / 24.1, 47.6 / 50.4 (14336 rows: 8.1 / 7.85);
-    // rows of 8192, 16384 / 28672 rows 14.7 / 14.3, 22.5 / 23.0; rows of 14336, 8192 / 14336 rows 14.3 / 13.2, 21.7 / 21.3.
-    // Rows of 28672 codes stay here at every size (4096 / 8192 / 16384 rows 14.6 / 12.1, 24.5 / 22.3, 51.8 / 42.1), and so
-    // do 2-bit codes (28672 x 8192: 19.7 / 17.6).
+    // rows of 8192, 16384 / 28672 rows 14.7 / 14.3, 22.5 / 23.0. Longer rows stay here at every size (14336 codes, 8192 /
+    // 14336 / 28672 rows 14.2 / 12.65, 21.5 / 20.35, 37.8 / 36.5; 28672 codes, 4096 / 8192 / 16384 rows 14.6 / 12.1, 24.5 /
+    // 22.3, 51.8 / 42.1), and so do 2-bit codes (28672 x 8192: 19.7 / 17.6).
     if (p.bits == 4 && p.K == 4096) return p.N <= 16384;
     if (p.bits == 4 && p.K == 8192) return p.N <= 20480;
-    if (p.bits == 4 && p.K == 14336) return p.N <= 16384;
     return true;
 }
 
@@ -643,7 +642,9 @@ int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
     // of them) is the fastest form on some machines of the pool and 9 % behind on others, where the same launch as 512
     // workgroups of eight holds (same run, 1024 / 512 threads: 7.34 / 7.40 us on one machine, 8.19 / 7.48 and 8.60 /
     // 7.70 on two others); shorter rows keep sixteen (8192 x 8192: 4-bit 8.00 / 7.97, 2-bit 6.27 / 6.95).
-    const uint32_t block = ch > 8 ? 1024u : ch > 4 ? 512u : 1024u;   // (28672 codes: 896 chunks to prepare)
+    // From 8192 rows on (two or more workgroups of sixteen per compute unit) sixteen are ahead again: 8192 x 14336 13.2 ->
+    // 12.65 us, 14336 x 14336 21.25 -> 20.35. (28672 codes: 896 chunks to prepare, always sixteen.)
+    const uint32_t block = ch > 8 || (ch == 7 && p.N >= 8192u) ? 1024u : ch > 4 ? 512u : 1024u;
     if (block < 64u * (uint32_t)ch) return fail(ERR_UNSUPPORTED, "qmv rows kernels: workgroup smaller than the row's chunks");   // (thread t prepares chunk t)
     hipError_t e = launch_kernel(fn, dim3((p.N + block / 64u - 1u) / (block / 64u), slots), dim3(block), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "qmv long rows kernel launch");
