@@ -445,6 +445,16 @@ static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const
     // 4-bit f16 / bf16: the norm applied as the matrix-core GEMV stages its row (two staged rows share one set of 4;
     // no per-workgroup renormalisation beyond the sum of squares). us, streaming kernel -> this: 14336 x 4096 12.6 ->
     // 10.6, 6144 x 4096 8.1 -> 7.3; it loses on short matrices and long rows (4096 x 4096 6.2 -> 6.4, 4096 x 14336 13.7 -> 14.1).
+    // Rows of 4096 / 8192 4-bit codes: the norm applied as the one-row-per-wave kernel puts the activations into LDS
+    // (qmv_rows_norm.hip). bf16, us, the forms below -> this: 4096 x 4096 6.8 -> 4.5, 6144 x 4096 7.3 -> 6.4, 14336 x 4096 10.7
+    // -> 10.0, 2048 x 8192 7.1 -> 4.7, 8192 x 8192 11.5 -> 11.5, 28672 x 8192 27.6 -> 25.9; behind on a few rows of 8192 codes
+    // and on the largest matrices (128256 x 4096: 50.2 -> 51.8). qmv.kernel = 2 keeps the older forms, = 3 takes this one
+    // wherever the shape allows.
+    const bool rows_norm = options().qmv_kernel == 3 || (options().qmv_kernel == 0 && N >= (K == 4096 ? 1024u : 2048u) && N <= 65536u);
+    if (options().qmv_norm_mfma != 2 && rows_norm && qmv_rows_norm_takes(p, norm_w)) {
+        rc = launch_qmv_rows_norm(p, norm_w, eps, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
     const bool norm_on_mfma = options().qmv_norm_mfma == 2 ||
                               (options().qmv_norm_mfma == 0 && K <= 8192 && (uint64_t)N * K >= 24000000ull);
     if (bits == 4 && dtype != DT_F32 && norm_on_mfma) {

@@ -86,6 +86,51 @@ template <int DT> struct RemSplit {
     }
 };
 
+// One 16-byte vector of activations (4 f32 or 8 16-bit elements): sum of squares, and
+// in-place (x * w) * inv rounded to the element type.
+template <int DT> __device__ __forceinline__ float raw_sumsq(uint4 v) {
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        if constexpr (DT == DT_F32) {
+            const float f = __uint_as_float(u[j]);
+            s += f * f;
+        } else {
+            const float lo = DT == DT_BF16 ? bf16_bits_to_f32(u[j] & 0xFFFFu) : f16_bits_to_f32(u[j] & 0xFFFFu);
+            const float hi = DT == DT_BF16 ? bf16_bits_to_f32(u[j] >> 16) : f16_bits_to_f32(u[j] >> 16);
+            s += lo * lo;
+            s += hi * hi;
+        }
+    }
+    return s;
+}
+// (x * w) * inv of one vector, as the element-type value `hi` nearest to it and (16-bit
+// types) the rounded, scaled remainder `lo` (RemSplit): hi + lo / kRemScale carries 16 significant bits of the f32 product.
+template <int DT> __device__ __forceinline__ void raw_normed(uint4 xv, uint4 wv, float inv, uint4& hi, uint4& lo) {
+    const uint32_t x[4] = {xv.x, xv.y, xv.z, xv.w};
+    const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        if constexpr (DT == DT_F32) {
+            h[j] = __float_as_uint(__uint_as_float(x[j]) * __uint_as_float(w[j]) * inv);
+            l[j] = 0;
+        } else {
+            auto up = [](uint32_t b) { return DT == DT_BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b); };
+            const float v0 = up(x[j] & 0xFFFFu) * up(w[j] & 0xFFFFu) * inv;
+            const float v1 = up(x[j] >> 16) * up(w[j] >> 16) * inv;
+            uint32_t h0, h1, l0, l1;
+            RemSplit<DT>::split(v0, h0, l0);
+            RemSplit<DT>::split(v1, h1, l1);
+            h[j] = h0 | (h1 << 16);
+            l[j] = l0 | (l1 << 16);
+        }
+    }
+    hi = make_uint4(h[0], h[1], h[2], h[3]);
+    lo = make_uint4(l[0], l[1], l[2], l[3]);
+}
+
 // ---- cross-lane sums -------------------------------------------------------
 
 template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {

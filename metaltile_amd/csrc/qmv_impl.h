@@ -378,51 +378,6 @@ __device__ __forceinline__ float wave_reduce4(float v0, float v1, float v2, floa
     return row16_allreduce(swap16_add(swap32_add(v0, v1), swap32_add(v2, v3)));
 }
 
-// One 16-byte vector of activations (4 f32 or 8 16-bit elements): sum of squares, and
-// in-place (x * w) * inv rounded to the element type.
-template <int DT> __device__ __forceinline__ float raw_sumsq(uint4 v) {
-    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
-    float s = 0.f;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        if constexpr (DT == DT_F32) {
-            const float f = __uint_as_float(u[j]);
-            s += f * f;
-        } else {
-            const float lo = DT == DT_BF16 ? bf16_bits_to_f32(u[j] & 0xFFFFu) : f16_bits_to_f32(u[j] & 0xFFFFu);
-            const float hi = DT == DT_BF16 ? bf16_bits_to_f32(u[j] >> 16) : f16_bits_to_f32(u[j] >> 16);
-            s += lo * lo;
-            s += hi * hi;
-        }
-    }
-    return s;
-}
-// (x * w) * inv of one vector, as the element-type value `hi` nearest to it and (16-bit
-// types) the rounded, scaled remainder `lo` (RemSplit): hi + lo / kRemScale carries 16 significant bits of the f32 product.
-template <int DT> __device__ __forceinline__ void raw_normed(uint4 xv, uint4 wv, float inv, uint4& hi, uint4& lo) {
-    const uint32_t x[4] = {xv.x, xv.y, xv.z, xv.w};
-    const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
-    uint32_t h[4], l[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        if constexpr (DT == DT_F32) {
-            h[j] = __float_as_uint(__uint_as_float(x[j]) * __uint_as_float(w[j]) * inv);
-            l[j] = 0;
-        } else {
-            auto up = [](uint32_t b) { return DT == DT_BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b); };
-            const float v0 = up(x[j] & 0xFFFFu) * up(w[j] & 0xFFFFu) * inv;
-            const float v1 = up(x[j] >> 16) * up(w[j] >> 16) * inv;
-            uint32_t h0, h1, l0, l1;
-            RemSplit<DT>::split(v0, h0, l0);
-            RemSplit<DT>::split(v1, h1, l1);
-            h[j] = h0 | (h1 << 16);
-            l[j] = l0 | (l1 << 16);
-        }
-    }
-    hi = make_uint4(h[0], h[1], h[2], h[3]);
-    lo = make_uint4(l[0], l[1], l[2], l[3]);
-}
-
 // One vector of the gated, normalised activation: element e = y[e] * inv * w[e] * silu(z[e]) in f32
 // (crates/metaltile-std/src/ffai/gated_rms_norm_qgemv.rs:138-149), y in f32 (two vectors of 4 for a 16-bit vector of
 // 8, one for an f32 vector of 4), z and w of the element type; split into `hi` and `lo` as in raw_normed.

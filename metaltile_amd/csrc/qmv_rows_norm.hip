@@ -1,0 +1,241 @@
+// RMS norm fused into a quantized GEMV: out[n] = sum_k (s q + b)[n, k] x'[k], x'[k] = x[k] norm_w[k] / sqrt(mean(x^2) + eps)
+// (ffai_rms_norm_qgemv / _fast, crates/metaltile-std/src/ffai/rms_norm_qgemv.rs:53-125, 128-456), 4-bit codes, f16 / bf16,
+// rows of 4096 or 8192 codes (the hidden sizes such a norm precedes), groups of 32 / 64 / 128.
+//
+// The make of the one-row-per-wave kernel (qmv_rows.hip): a wave owns a weight row, lane l its 16-byte chunks l, 64 + l, ...,
+// codes become operands of the 4x4x4 matrix instruction in place, the activations are put into operand order once per
+// workgroup in LDS. Two things differ. The activations are normalised on the way into LDS: every workgroup works out
+// the row's sum of squares itself (thread t from chunk t, one more barrier), and x', an f32 value in the reference, is
+// carried as the element-type value nearest to it and the rounded (f16: scaled) remainder -- two operand sets whose
+// products are added, 16 significant bits, as in the streaming kernel's fused form. And because that preparation is
+// no longer cheap, a workgroup does it once and then walks many rows: the launch is at most two workgroups of eight
+// waves per compute unit (one of sixteen up to 4096 rows), wave g of G takes rows g, g + G, g + 2 G, ..., each row's
+// loads issued while the row before it is worked on.
+#include <hip/hip_runtime.h>
+
+#include "../../include/mtq.h"
+#include "mtq_device.h"
+#include "mtq_internal.h"
+#include "qmv_rows_common.h"
+
+namespace mtq {
+
+struct QmvRowsNArgs {
+    const rp_u32x4* w;
+    const uint16_t* s;
+    const uint16_t* b;
+    const uint16_t* x;
+    uint16_t* out;
+    uint32_t N;
+    const uint16_t* norm_w;   // [K]
+    const float* norm_eps;    // one f32 on the device
+};
+
+template <int CH> struct RowsNormBuf {   // one row's loads of one lane
+    rp_u32x4 wv[CH];
+    uint32_t sc[CH];
+    uint32_t sw[2], bw[2];   // the lane's groups of the bias term, two 16-bit elements per dword
+};
+
+template <int DT, int CH, int LOG2G, int NWV>
+__global__ __launch_bounds__(64 * NWV) void qmv_rows_norm_kernel(QmvRowsNArgs a) {
+    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
+    constexpr float REM = 1.0f / RemSplit<DT>::kRemScale;
+    constexpr int CPC = 32, Q = 4;           // codes per 16-byte chunk; 16-byte quarters of a chunk's activations in operand order
+    constexpr int C = 64 * CH, K = C * CPC;
+    constexpr int GPR = K >> LOG2G;          // groups per row
+    constexpr int GPL = GPR > 128 ? 4 : GPR > 64 ? 2 : 1;   // groups a lane owns in the bias term (lanes below GPR / GPL)
+    constexpr int SPG = (1 << LOG2G) / (CPC / 2);            // half chunks per group
+    static_assert(C <= 64 * NWV && LOG2G >= 5 && LOG2G <= 7 && GPR % GPL == 0 && GPR / GPL <= 64, "one thread per chunk; groups of 32, 64 or 128 codes, at most 256 per row");
+    __shared__ __align__(16) uint32_t xp_lds[Q][C][4];   // [quarter][chunk][4 pair dwords]: the rounded values
+    __shared__ __align__(16) uint32_t xl_lds[Q][C][4];   // the remainders
+    __shared__ __align__(16) float xs_lds[2 * C];        // sum of x' over each half chunk
+    __shared__ float ssq_lds[NWV];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t gw = blockIdx.x * (uint32_t)NWV + wave, GW = gridDim.x * (uint32_t)NWV;
+    const uint32_t last = a.N - 1u;
+    const uint32_t gl = min(lane, (uint32_t)(GPR / GPL - 1));
+    auto load_row = [&](uint32_t row, RowsNormBuf<CH>& r) {   // row <= last
+        const uint16_t* sp = a.s + (size_t)row * GPR;
+        const uint16_t* bp = a.b + (size_t)row * GPR;
+#pragma unroll
+        for (int i = 0; i < CH; i++) r.sc[i] = sp[((uint32_t)(i * 64 + (int)lane) * CPC) >> LOG2G];
+        r.sw[0] = r.sw[1] = r.bw[0] = r.bw[1] = 0u;
+        if constexpr (GPL == 4) {
+            const uint2 sv = ((const uint2*)sp)[gl], bv = ((const uint2*)bp)[gl];
+            r.sw[0] = sv.x; r.sw[1] = sv.y; r.bw[0] = bv.x; r.bw[1] = bv.y;
+        } else if constexpr (GPL == 2) {
+            r.sw[0] = ((const uint32_t*)sp)[gl];
+            r.bw[0] = ((const uint32_t*)bp)[gl];
+        } else {
+            r.sw[0] = sp[gl];
+            r.bw[0] = bp[gl];
+        }
+        const rp_u32x4* wbase = a.w + (size_t)row * C + lane;
+#pragma unroll
+        for (int i = 0; i < CH; i++) r.wv[i] = __builtin_nontemporal_load(wbase + i * 64);
+    };
+    // ---- this thread's chunk of the activations and of the norm weights; the first row's loads ---------------------
+    uint4 xraw[Q], nraw[Q];
+    if (tid < (uint32_t)C) {
+        const uint4* xv = (const uint4*)(a.x + (size_t)tid * CPC);
+        const uint4* nv = (const uint4*)(a.norm_w + (size_t)tid * CPC);
+#pragma unroll
+        for (int v = 0; v < Q; v++) xraw[v] = xv[v];
+#pragma unroll
+        for (int v = 0; v < Q; v++) nraw[v] = nv[v];
+    }
+    const float eps = a.norm_eps[0];
+    RP_KEEP_ORDER();
+    RowsNormBuf<CH> bufA, bufB;
+    load_row(min(gw, last), bufA);   // (idle waves of a short launch load the last row and store nothing)
+    RP_KEEP_ORDER();
+    const bool j0 = lane & 1u, j1 = lane & 2u;
+    uint32_t kor = DT == DT_BF16 ? 0x43004300u : 0x64006400u;   // (2^7, 2^7) in bf16, (2^10, 2^10) in f16: a code OR-ed into the mantissa is MAGIC + q
+    asm volatile("" : "+v"(kor));
+    // ---- the row's sum of squares ------------------------------------------------------------------------------------
+    {
+        float ssq = 0.f;
+        if (tid < (uint32_t)C) {
+#pragma unroll
+            for (int v = 0; v < Q; v++) ssq += raw_sumsq<DT>(xraw[v]);
+        }
+        ssq = seg_allreduce(ssq, 64);
+        if (lane == 0) ssq_lds[wave] = ssq;
+    }
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int wv_ = 0; wv_ < NWV; wv_++) tot += ssq_lds[wv_];
+    const float inv = 1.0f / sqrtf(tot / (float)K + eps);
+    // ---- the normalised chunk into operand order, into LDS --------------------------------------------------------------
+    if (tid < (uint32_t)C) {
+        rp_u32x2 ones;
+        ones.x = ones.y = DT == DT_BF16 ? 0x3F803F80u : 0x3C003C00u;
+        rp_f32x4 sx[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, sl[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+        for (int d = 0; d < 4; d++) {       // weight dword d: activations 8 d .. 8 d + 7, pairs (j, j + 4)
+            uint4 v, rem;
+            raw_normed<DT>(xraw[d], nraw[d], inv, v, rem);
+            uint4 o, ol;
+            o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+            o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+            o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+            o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+            ol.x = __builtin_amdgcn_perm(rem.z, rem.x, 0x05040100u);
+            ol.y = __builtin_amdgcn_perm(rem.z, rem.x, 0x07060302u);
+            ol.z = __builtin_amdgcn_perm(rem.w, rem.y, 0x05040100u);
+            ol.w = __builtin_amdgcn_perm(rem.w, rem.y, 0x07060302u);
+            *(uint4*)xp_lds[d][tid] = o;
+            *(uint4*)xl_lds[d][tid] = ol;
+            rp_u32x2 a0, a1, l0, l1;
+            a0.x = o.x; a0.y = o.y; a1.x = o.z; a1.y = o.w;
+            l0.x = ol.x; l0.y = ol.y; l1.x = ol.z; l1.y = ol.w;
+            sx[d / 2] = rp_mfma<DT>(a0, ones, sx[d / 2]);
+            sx[d / 2] = rp_mfma<DT>(a1, ones, sx[d / 2]);
+            sl[d / 2] = rp_mfma<DT>(l0, ones, sl[d / 2]);
+            sl[d / 2] = rp_mfma<DT>(l1, ones, sl[d / 2]);
+        }
+        // (a lane's own sum is the diagonal entry of its block: its first operand against its own second operand)
+        xs_lds[2 * tid] = fmaf(rp_diag(sl[0], j0, j1), REM, rp_diag(sx[0], j0, j1));
+        xs_lds[2 * tid + 1] = fmaf(rp_diag(sl[1], j0, j1), REM, rp_diag(sx[1], j0, j1));
+    }
+    __syncthreads();
+    if (gw > last) return;
+    // the activation sums of this lane's GPL groups of the bias term (the same for every row)
+    float X[GPL];
+#pragma unroll
+    for (int v = 0; v < GPL; v++) {
+        X[v] = 0.f;
+#pragma unroll
+        for (int h = 0; h < SPG; h++) X[v] += xs_lds[(gl * GPL + (uint32_t)v) * SPG + (uint32_t)h];
+    }
+    auto work_row = [&](uint32_t row, const RowsNormBuf<CH>& r) {
+        float t = 0.f;
+        if (lane < (uint32_t)(GPR / GPL)) {
+#pragma unroll
+            for (int v = 0; v < GPL; v++) {
+                const float sf = rp_up<DT>((r.sw[v >> 1] >> (16 * (v & 1))) & 0xFFFFu), bf = rp_up<DT>((r.bw[v >> 1] >> (16 * (v & 1))) & 0xFFFFu);
+                t = fmaf(bf, X[v], t);
+                t = fmaf(0.f - sf, MAGIC * X[v], t);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            rp_f32x4 dh = {0.f, 0.f, 0.f, 0.f}, dl = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const uint32_t w = r.wv[i][d];
+                const uint4 xo = *(const uint4*)xp_lds[d][i * 64 + lane], xl = *(const uint4*)xl_lds[d][i * 64 + lane];
+                rp_u32x2 b0, b1, a0, a1, l0, l1;
+                b0.x = (w & 0x000F000Fu) | kor;
+                b0.y = ((w >> 4) & 0x000F000Fu) | kor;
+                b1.x = ((w >> 8) & 0x000F000Fu) | kor;
+                b1.y = ((w >> 12) & 0x000F000Fu) | kor;
+                a0.x = xo.x; a0.y = xo.y; a1.x = xo.z; a1.y = xo.w;
+                l0.x = xl.x; l0.y = xl.y; l1.x = xl.z; l1.y = xl.w;
+                dh = rp_mfma<DT>(a0, b0, dh);
+                dh = rp_mfma<DT>(a1, b1, dh);
+                dl = rp_mfma<DT>(l0, b0, dl);
+                dl = rp_mfma<DT>(l1, b1, dl);
+            }
+            t = fmaf(rp_up<DT>(r.sc[i]), fmaf(rp_diag(dl, j0, j1), REM, rp_diag(dh, j0, j1)), t);
+        }
+        t += __shfl_xor(t, 32, 64);
+        t += dpp_f32<0xB1>(t);
+        t += dpp_f32<0x4E>(t);
+        t += dpp_f32<0x141>(t);
+        t += dpp_f32<0x140>(t);
+        t += __shfl_xor(t, 16, 64);
+        if (lane == 0) a.out[row] = f32_to_elem_bits<DT>(t);
+    };
+    // ---- this wave's rows, each row's loads in flight while the row before it is worked on ------------------------------
+    uint32_t row = gw;
+    while (true) {
+        const uint32_t n1 = row + GW;
+        if (n1 <= last) load_row(n1, bufB);
+        RP_KEEP_ORDER();
+        work_row(row, bufA);
+        if (n1 > last) break;
+        const uint32_t n2 = n1 + GW;
+        if (n2 <= last) load_row(n2, bufA);
+        RP_KEEP_ORDER();
+        work_row(n1, bufB);
+        if (n2 > last) break;
+        row = n2;
+    }
+}
+
+// 4-bit codes, rows of 4096 or 8192 codes, groups of 32 / 64 / 128, f16 / bf16
+bool qmv_rows_norm_takes(const QmvParams& p, const void* norm_w) {
+    if ((p.dtype != DT_F16 && p.dtype != DT_BF16) || p.bits != 4 || p.N == 0 || (p.K != 4096 && p.K != 8192)) return false;
+    const uint32_t G = p.group_size;
+    if (G != 32 && G != 64 && G != 128) return false;
+    return !((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)norm_w % 16 || (uintptr_t)p.scales % 8 || (uintptr_t)p.biases % 8 || (uintptr_t)p.out % 2);
+}
+
+template <int DT, int LOG2G> static const void* rows_norm_fn(uint32_t K, bool sixteen) {
+    if (sixteen) return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 16>;
+    return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 8>;
+}
+
+int launch_qmv_rows_norm(const QmvParams& p, const void* norm_w, const float* eps, const LaunchCtx& lc) {
+    if (!qmv_rows_norm_takes(p, norm_w) || !eps) return fail(ERR_UNSUPPORTED, "norm + qmv rows kernel: 4-bit codes, rows of 4096 or 8192 codes, f16 / bf16");
+    QmvRowsNArgs a{(const rp_u32x4*)p.w, (const uint16_t*)p.scales, (const uint16_t*)p.biases, (const uint16_t*)p.x, (uint16_t*)p.out, p.N,
+                   (const uint16_t*)norm_w, eps};
+    void* args[] = {&a};
+    const uint32_t G = p.group_size;
+    // Up to 4096 rows one workgroup of sixteen waves per 16 rows (4096 x 4096 bf16: 4.5 us against 5.6 in workgroups of
+    // eight); beyond, two workgroups of eight waves per compute unit, which walk the rows (14336 x 4096: 10.0 either way;
+    // eight hold on the machines where a launch of exactly one large workgroup per compute unit falls behind).
+    const bool sixteen = p.N <= 4096;
+    const uint32_t nwv = sixteen ? 16u : 8u, cap = sixteen ? 256u : 512u;
+    const void* fn = p.dtype == DT_BF16 ? (G == 32 ? rows_norm_fn<DT_BF16, 5>(p.K, sixteen) : G == 64 ? rows_norm_fn<DT_BF16, 6>(p.K, sixteen) : rows_norm_fn<DT_BF16, 7>(p.K, sixteen))
+                                        : (G == 32 ? rows_norm_fn<DT_F16, 5>(p.K, sixteen) : G == 64 ? rows_norm_fn<DT_F16, 6>(p.K, sixteen) : rows_norm_fn<DT_F16, 7>(p.K, sixteen));
+    const uint32_t wgs = (p.N + nwv - 1u) / nwv;
+    hipError_t e = launch_kernel(fn, dim3(wgs < cap ? wgs : cap), dim3(64u * nwv), args, 0, lc);
+    if (e != hipSuccess) return hip_fail(e, "norm + qmv rows kernel launch");
+    return ERR_OK;
+}
+
+}  // namespace mtq

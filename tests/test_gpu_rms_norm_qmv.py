@@ -125,3 +125,43 @@ def test_norm_fused_into_the_matrix_core_gemv(oracle, dt, N, K, G):
     assert rel_err(got, exp) <= TOL[dt]
     for buf in (w, s, b, x, nwb, epsb, out):
         buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.F16, DType.BF16], ids=lambda d: d.name)
+@pytest.mark.parametrize("N,K,G", [(14336, 4096, 64), (1030, 4096, 32), (19, 4096, 128), (1, 4096, 64), (4096, 8192, 64), (33, 8192, 32), (1028, 8192, 128)])
+def test_norm_fused_into_the_one_row_per_wave_kernel(oracle, dt, N, K, G):
+    """The same operation with the norm applied as the one-row-per-wave GEMV puts the activation row into LDS (4-bit
+    codes, rows of 4096 / 8192 codes; automatic from 1024 weight rows, forced below that with qmv.kernel = 3): every
+    group size, ragged last workgroups, behind a cache flush, guard elements after the output, against the oracle at the
+    bound of the other fused kernels."""
+    import metaltile_amd as m
+    from metaltile_amd import _lib
+    lib = _lib.load()
+    bits = 4
+    print(f"[case] rms_norm_qmv on the one-row-per-wave GEMV {dt.name} g{G} N{N} K{K}", flush=True)
+    c = make_case(1500 + N + G, dt, bits, G, 1, N, K, bias_rule="midpoint")
+    rng = np.random.default_rng(N + K + G)
+    nw = oracle.round_through((1.0 + 0.2 * rng.standard_normal(K)).astype(np.float32), ODT[dt])
+    eps = np.float32(1e-5)
+    _, exp64, _ = oracle.rms_norm_qgemv(c.w, c.scales_f, c.biases_f, c.x_f, nw, K, G, N, bits, eps)
+    exp = oracle.round_through(exp64.astype(np.float32), ODT[dt])
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    nwb, epsb = GpuBuffer.from_bytes(pack_f32(nw, dt)), GpuBuffer.from_bytes(eps.tobytes())
+    rb = N * dt.size_bytes
+    out = GpuBuffer.from_bytes(b"\xab" * (rb + 64))
+    assert lib.mtq_set_option(b"qmv.kernel", 3) == 0
+    try:
+        rc, launches, _, n = ops.plan("rms_norm_qmv", dt, bits, G, 1, N, K)
+        assert rc == 0 and n == 1 and "qmv_rows_norm_kernel" in launches[0][0], launches
+        m.GpuRunner(0).flush_slc()
+        ops.rms_norm_qmv(dt, bits, G, x, nwb, w, s, b, out, epsb, N, K)
+    finally:
+        lib.mtq_set_option(b"qmv.kernel", 0)
+    raw = out.read_bytes()
+    assert raw[rb:] == b"\xab" * 64
+    got = unpack_f32(raw[:rb], dt)
+    assert np.isfinite(got).all()
+    assert rel_err(got, exp) <= TOL[dt]
+    for buf in (w, s, b, x, nwb, epsb, out):
+        buf.free()
