@@ -31,14 +31,17 @@ struct QmvRowsNArgs {
     const float* norm_eps;    // one f32 on the device
 };
 
-template <int CH> struct RowsNormBuf {   // one row's loads of one lane
+// One row's loads of one lane, as they come from memory: whatever has to be done to a loaded value (picking the 16-bit
+// half, widening) is done where the row is worked on. An operation on the value where it is loaded would be carried
+// round the row loop with it, and the wait for the load with that operation.
+template <int CH> struct RowsNormBuf {
     rp_u32x4 wv[CH];
-    uint32_t sc[CH];
-    uint32_t sw[2], bw[2];   // the lane's groups of the bias term, two 16-bit elements per dword
+    uint32_t sc[CH];         // the dword that holds the scale of chunk 64 i + lane
+    uint32_t sw[2], bw[2];   // the lane's groups of the bias term, two 16-bit elements per dword (one group per lane: the dword that holds it)
 };
 
-template <int DT, int CH, int LOG2G, int NWV>
-__global__ __launch_bounds__(64 * NWV) void qmv_rows_norm_kernel(QmvRowsNArgs a) {
+template <int DT, int CH, int LOG2G, int NWV, bool XREG = false>
+__global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs a) {
     constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
     constexpr float REM = 1.0f / RemSplit<DT>::kRemScale;
     constexpr int CPC = 32, Q = 4;           // codes per 16-byte chunk; 16-byte quarters of a chunk's activations in operand order
@@ -51,15 +54,16 @@ __global__ __launch_bounds__(64 * NWV) void qmv_rows_norm_kernel(QmvRowsNArgs a)
     __shared__ __align__(16) uint32_t xl_lds[Q][C][4];   // the remainders
     __shared__ __align__(16) float xs_lds[2 * C];        // sum of x' over each half chunk
     __shared__ float ssq_lds[NWV];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t gw = blockIdx.x * (uint32_t)NWV + wave, GW = gridDim.x * (uint32_t)NWV;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t gw = blockIdx.x * (uint32_t)NWV + wave, GW = gridDim.x * (uint32_t)NWV;   // (the same in every lane: row numbers stay in scalar registers)
     const uint32_t last = a.N - 1u;
     const uint32_t gl = min(lane, (uint32_t)(GPR / GPL - 1));
     auto load_row = [&](uint32_t row, RowsNormBuf<CH>& r) {   // row <= last
+        row = min(row, last);   // (it is; a scalar instruction keeps the loads inside the matrix whatever the caller does)
         const uint16_t* sp = a.s + (size_t)row * GPR;
         const uint16_t* bp = a.b + (size_t)row * GPR;
 #pragma unroll
-        for (int i = 0; i < CH; i++) r.sc[i] = sp[((uint32_t)(i * 64 + (int)lane) * CPC) >> LOG2G];
+        for (int i = 0; i < CH; i++) r.sc[i] = ((const uint32_t*)sp)[((uint32_t)(i * 64 + (int)lane) * CPC) >> (LOG2G + 1)];
         r.sw[0] = r.sw[1] = r.bw[0] = r.bw[1] = 0u;
         if constexpr (GPL == 4) {
             const uint2 sv = ((const uint2*)sp)[gl], bv = ((const uint2*)bp)[gl];
@@ -68,8 +72,8 @@ __global__ __launch_bounds__(64 * NWV) void qmv_rows_norm_kernel(QmvRowsNArgs a)
             r.sw[0] = ((const uint32_t*)sp)[gl];
             r.bw[0] = ((const uint32_t*)bp)[gl];
         } else {
-            r.sw[0] = sp[gl];
-            r.bw[0] = bp[gl];
+            r.sw[0] = ((const uint32_t*)sp)[gl >> 1];
+            r.bw[0] = ((const uint32_t*)bp)[gl >> 1];
         }
         const rp_u32x4* wbase = a.w + (size_t)row * C + lane;
 #pragma unroll
@@ -152,10 +156,15 @@ __global__ __launch_bounds__(64 * NWV) void qmv_rows_norm_kernel(QmvRowsNArgs a)
     }
     auto work_row = [&](uint32_t row, const RowsNormBuf<CH>& r) {
         float t = 0.f;
+        // (the lane number, made opaque once per row: the operand reads from LDS below are the same for every row, and
+        // lifted out of the row loop they would hold 32 registers per chunk)
+        uint32_t ln = lane;
+        if constexpr (!XREG) asm volatile("" : "+v"(ln));
         if (lane < (uint32_t)(GPR / GPL)) {
 #pragma unroll
             for (int v = 0; v < GPL; v++) {
-                const float sf = rp_up<DT>((r.sw[v >> 1] >> (16 * (v & 1))) & 0xFFFFu), bf = rp_up<DT>((r.bw[v >> 1] >> (16 * (v & 1))) & 0xFFFFu);
+                const uint32_t sh = GPL == 1 ? 16u * (gl & 1u) : 16u * (uint32_t)(v & 1);
+                const float sf = rp_up<DT>((r.sw[v >> 1] >> sh) & 0xFFFFu), bf = rp_up<DT>((r.bw[v >> 1] >> sh) & 0xFFFFu);
                 t = fmaf(bf, X[v], t);
                 t = fmaf(0.f - sf, MAGIC * X[v], t);
             }
@@ -166,7 +175,7 @@ __global__ __launch_bounds__(64 * NWV) void qmv_rows_norm_kernel(QmvRowsNArgs a)
 #pragma unroll
             for (int d = 0; d < 4; d++) {
                 const uint32_t w = r.wv[i][d];
-                const uint4 xo = *(const uint4*)xp_lds[d][i * 64 + lane], xl = *(const uint4*)xl_lds[d][i * 64 + lane];
+                const uint4 xo = *(const uint4*)xp_lds[d][i * 64 + ln], xl = *(const uint4*)xl_lds[d][i * 64 + ln];
                 rp_u32x2 b0, b1, a0, a1, l0, l1;
                 b0.x = (w & 0x000F000Fu) | kor;
                 b0.y = ((w >> 4) & 0x000F000Fu) | kor;
@@ -179,7 +188,8 @@ __global__ __launch_bounds__(64 * NWV) void qmv_rows_norm_kernel(QmvRowsNArgs a)
                 dl = rp_mfma<DT>(l0, b0, dl);
                 dl = rp_mfma<DT>(l1, b1, dl);
             }
-            t = fmaf(rp_up<DT>(r.sc[i]), fmaf(rp_diag(dl, j0, j1), REM, rp_diag(dh, j0, j1)), t);
+            const uint32_t sch = 16u * ((((uint32_t)(i * 64 + (int)lane) * CPC) >> LOG2G) & 1u);   // the half of the dword the chunk's group is in
+            t = fmaf(rp_up<DT>((r.sc[i] >> sch) & 0xFFFFu), fmaf(rp_diag(dl, j0, j1), REM, rp_diag(dh, j0, j1)), t);
         }
         t += __shfl_xor(t, 32, 64);
         t += dpp_f32<0xB1>(t);
@@ -187,28 +197,34 @@ __global__ __launch_bounds__(64 * NWV) void qmv_rows_norm_kernel(QmvRowsNArgs a)
         t += dpp_f32<0x141>(t);
         t += dpp_f32<0x140>(t);
         t += __shfl_xor(t, 16, 64);
-        if (lane == 0) a.out[row] = f32_to_elem_bits<DT>(t);
+        if (lane == 0 && row <= last) a.out[row] = f32_to_elem_bits<DT>(t);
     };
     // ---- this wave's rows, each row's loads in flight while the row before it is worked on ------------------------------
+    // A row's loads and the work on the row before it stand in one block of straight-line code, in a counted loop with
+    // no way out but its end: the wait that the compiler puts before the first use of a buffer then leaves the loads
+    // just issued in flight. (With the loads under a condition of their own, or with a way out of the loop between
+    // them, that wait has to hold for the path that issued nothing, and waits for them.)
+    const uint32_t cnt = (last - gw) / GW + 1u;   // rows of this wave: gw, gw + GW, ... (gw <= last here)
     uint32_t row = gw;
-    while (true) {
-        const uint32_t n1 = row + GW;
-        if (n1 <= last) load_row(n1, bufB);
+    if (cnt == 1u) {
+        work_row(row, bufA);
+        return;
+    }
+    for (uint32_t it = cnt >> 1; it != 0u; it--) {   // two rows a turn
+        load_row(row + GW, bufB);
         RP_KEEP_ORDER();
         work_row(row, bufA);
-        if (n1 > last) break;
-        const uint32_t n2 = n1 + GW;
-        if (n2 <= last) load_row(n2, bufA);
+        load_row(row + 2u * GW, bufA);   // (the last turn of an even number of rows loads the matrix's last row instead, and nobody reads it)
         RP_KEEP_ORDER();
-        work_row(n1, bufB);
-        if (n2 > last) break;
-        row = n2;
+        work_row(row + GW, bufB);
+        row += 2u * GW;
     }
+    if (cnt & 1u) work_row(row, bufA);
 }
 
 // 4-bit codes, rows of 4096 or 8192 codes, groups of 32 / 64 / 128, f16 / bf16
 bool qmv_rows_norm_takes(const QmvParams& p, const void* norm_w) {
-    if ((p.dtype != DT_F16 && p.dtype != DT_BF16) || p.bits != 4 || p.N == 0 || (p.K != 4096 && p.K != 8192)) return false;
+    if ((p.dtype != DT_F16 && p.dtype != DT_BF16) || p.bits != 4 || p.N == 0 || p.N > (1u << 24) || (p.K != 4096 && p.K != 8192)) return false;   // (row numbers plus the launch's waves stay below 2^32)
     const uint32_t G = p.group_size;
     if (G != 32 && G != 64 && G != 128) return false;
     return !((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)norm_w % 16 || (uintptr_t)p.scales % 8 || (uintptr_t)p.biases % 8 || (uintptr_t)p.out % 2);
