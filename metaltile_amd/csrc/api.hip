@@ -1741,7 +1741,7 @@ int mtq_set_option(const char* name, int value) {
         return MTQ_OK;
     }
     if (!strcmp(name, "qmv.kernel")) {
-        if (value < 0 || value > 3) return fail(ERR_BAD_ARG, "qmv.kernel must be 0 (auto), 1 (one-shot), 2 (streaming) or 3 (wave per four rows)");
+        if (value < 0 || value > 4) return fail(ERR_BAD_ARG, "qmv.kernel must be 0 (auto), 1 (one-shot), 2 (streaming), 3 (wave per four rows / per row) or 4 (waves walking the rows)");
         options().qmv_kernel = value;
         return MTQ_OK;
     }

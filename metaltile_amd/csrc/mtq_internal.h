@@ -218,6 +218,10 @@ int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc);
 // RMS norm fused into the one-row-per-wave kernel (4-bit codes, rows of 4096 or 8192 codes, f16 / bf16).
 bool qmv_rows_norm_takes(const QmvParams& p, const void* norm_w);
 int launch_qmv_rows_norm(const QmvParams& p, const void* norm_w, const float* eps, const LaunchCtx& lc);
+// The same walk without the norm (one activation row): qmv.kernel = 4 takes it wherever it applies.
+bool qmv_rows_walk_takes(const QmvParams& p);
+bool qmv_rows_walk_preferred(const QmvParams& p);
+int launch_qmv_rows_walk(const QmvParams& p, const LaunchCtx& lc);
 // Two to four activation rows (qmv_rows_few.hip): one wave per four weight rows; 4096 or 8192 4-bit codes or 8192 2-bit codes per
 // row, groups of 32 / 64 / 128, f16 / bf16.
 bool qmv_rows_few_takes(const QmvParams& p);

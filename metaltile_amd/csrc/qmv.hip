@@ -251,6 +251,10 @@ int launch_qmv_fast(const QmvParams& p, const LaunchCtx& lc) {
     // routing sits ahead of the first weight load); 2 rows on 2 experts 17.6 -> 18.1, so those stay where they were.
     // One row of 4096 4-bit codes (the gate / up shapes of the headline): the wave-per-four-rows kernel, 3 % ahead of the
     // streaming kernel in the same run (14336 x 4096 bf16: 7.86 against 8.11 us).
+    if (mode != 2 && ((options().qmv_kernel == 0 && qmv_rows_walk_preferred(p)) || (options().qmv_kernel == 4 && qmv_rows_walk_takes(p)))) {
+        int rc = launch_qmv_rows_walk(p, lc);
+        if (rc != ERR_UNSUPPORTED) return rc;
+    }
     if (mode != 2 && ((options().qmv_kernel == 0 && qmv_rows_preferred(p)) || (options().qmv_kernel == 3 && qmv_rows_takes(p)))) {
         int rc = launch_qmv_rows(p, lc);
         if (rc != ERR_UNSUPPORTED) return rc;

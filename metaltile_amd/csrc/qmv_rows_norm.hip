@@ -40,8 +40,8 @@ template <int CH> struct RowsNormBuf {
     uint32_t sw[2], bw[2];   // the lane's groups of the bias term, two 16-bit elements per dword (one group per lane: the dword that holds it)
 };
 
-template <int DT, int CH, int LOG2G, int NWV, bool XREG = false>
-__global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs a) {
+template <int DT, int CH, int LOG2G, int NWV, bool NORM>
+__device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
     constexpr float REM = 1.0f / RemSplit<DT>::kRemScale;
     constexpr int CPC = 32, Q = 4;           // codes per 16-byte chunk; 16-byte quarters of a chunk's activations in operand order
@@ -51,7 +51,7 @@ __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs
     constexpr int SPG = (1 << LOG2G) / (CPC / 2);            // half chunks per group
     static_assert(C <= 64 * NWV && LOG2G >= 5 && LOG2G <= 7 && GPR % GPL == 0 && GPR / GPL <= 64, "one thread per chunk; groups of 32, 64 or 128 codes, at most 256 per row");
     __shared__ __align__(16) uint32_t xp_lds[Q][C][4];   // [quarter][chunk][4 pair dwords]: the rounded values
-    __shared__ __align__(16) uint32_t xl_lds[Q][C][4];   // the remainders
+    __shared__ __align__(16) uint32_t xl_lds[NORM ? Q : 1][NORM ? C : 1][4];   // the remainders
     __shared__ __align__(16) float xs_lds[2 * C];        // sum of x' over each half chunk
     __shared__ float ssq_lds[NWV];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -86,10 +86,13 @@ __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs
         const uint4* nv = (const uint4*)(a.norm_w + (size_t)tid * CPC);
 #pragma unroll
         for (int v = 0; v < Q; v++) xraw[v] = xv[v];
+        if constexpr (NORM) {
 #pragma unroll
-        for (int v = 0; v < Q; v++) nraw[v] = nv[v];
+            for (int v = 0; v < Q; v++) nraw[v] = nv[v];
+        }
     }
-    const float eps = a.norm_eps[0];
+    float eps = 0.f;
+    if constexpr (NORM) eps = a.norm_eps[0];
     RP_KEEP_ORDER();
     RowsNormBuf<CH> bufA, bufB;
     load_row(min(gw, last), bufA);   // (idle waves of a short launch load the last row and store nothing)
@@ -98,7 +101,8 @@ __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs
     uint32_t kor = DT == DT_BF16 ? 0x43004300u : 0x64006400u;   // (2^7, 2^7) in bf16, (2^10, 2^10) in f16: a code OR-ed into the mantissa is MAGIC + q
     asm volatile("" : "+v"(kor));
     // ---- the row's sum of squares ------------------------------------------------------------------------------------
-    {
+    float inv = 1.0f;
+    if constexpr (NORM) {
         float ssq = 0.f;
         if (tid < (uint32_t)C) {
 #pragma unroll
@@ -106,12 +110,12 @@ __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs
         }
         ssq = seg_allreduce(ssq, 64);
         if (lane == 0) ssq_lds[wave] = ssq;
-    }
-    __syncthreads();
-    float tot = 0.f;
+        __syncthreads();
+        float tot = 0.f;
 #pragma unroll
-    for (int wv_ = 0; wv_ < NWV; wv_++) tot += ssq_lds[wv_];
-    const float inv = 1.0f / sqrtf(tot / (float)K + eps);
+        for (int wv_ = 0; wv_ < NWV; wv_++) tot += ssq_lds[wv_];
+        inv = 1.0f / sqrtf(tot / (float)K + eps);
+    }
     // ---- the normalised chunk into operand order, into LDS --------------------------------------------------------------
     if (tid < (uint32_t)C) {
         rp_u32x2 ones;
@@ -119,8 +123,8 @@ __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs
         rp_f32x4 sx[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, sl[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
         for (int d = 0; d < 4; d++) {       // weight dword d: activations 8 d .. 8 d + 7, pairs (j, j + 4)
-            uint4 v, rem;
-            raw_normed<DT>(xraw[d], nraw[d], inv, v, rem);
+            uint4 v = xraw[d], rem = make_uint4(0u, 0u, 0u, 0u);
+            if constexpr (NORM) raw_normed<DT>(xraw[d], nraw[d], inv, v, rem);
             uint4 o, ol;
             o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
             o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
@@ -131,14 +135,16 @@ __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs
             ol.z = __builtin_amdgcn_perm(rem.w, rem.y, 0x05040100u);
             ol.w = __builtin_amdgcn_perm(rem.w, rem.y, 0x07060302u);
             *(uint4*)xp_lds[d][tid] = o;
-            *(uint4*)xl_lds[d][tid] = ol;
+            if constexpr (NORM) *(uint4*)xl_lds[d][tid] = ol;
             rp_u32x2 a0, a1, l0, l1;
             a0.x = o.x; a0.y = o.y; a1.x = o.z; a1.y = o.w;
             l0.x = ol.x; l0.y = ol.y; l1.x = ol.z; l1.y = ol.w;
             sx[d / 2] = rp_mfma<DT>(a0, ones, sx[d / 2]);
             sx[d / 2] = rp_mfma<DT>(a1, ones, sx[d / 2]);
-            sl[d / 2] = rp_mfma<DT>(l0, ones, sl[d / 2]);
-            sl[d / 2] = rp_mfma<DT>(l1, ones, sl[d / 2]);
+            if constexpr (NORM) {
+                sl[d / 2] = rp_mfma<DT>(l0, ones, sl[d / 2]);
+                sl[d / 2] = rp_mfma<DT>(l1, ones, sl[d / 2]);
+            }
         }
         // (a lane's own sum is the diagonal entry of its block: its first operand against its own second operand)
         xs_lds[2 * tid] = fmaf(rp_diag(sl[0], j0, j1), REM, rp_diag(sx[0], j0, j1));
@@ -159,7 +165,7 @@ __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs
         // (the lane number, made opaque once per row: the operand reads from LDS below are the same for every row, and
         // lifted out of the row loop they would hold 32 registers per chunk)
         uint32_t ln = lane;
-        if constexpr (!XREG) asm volatile("" : "+v"(ln));
+        asm volatile("" : "+v"(ln));
         if (lane < (uint32_t)(GPR / GPL)) {
 #pragma unroll
             for (int v = 0; v < GPL; v++) {
@@ -175,7 +181,9 @@ __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs
 #pragma unroll
             for (int d = 0; d < 4; d++) {
                 const uint32_t w = r.wv[i][d];
-                const uint4 xo = *(const uint4*)xp_lds[d][i * 64 + ln], xl = *(const uint4*)xl_lds[d][i * 64 + ln];
+                const uint4 xo = *(const uint4*)xp_lds[d][i * 64 + ln];
+                uint4 xl = make_uint4(0u, 0u, 0u, 0u);
+                if constexpr (NORM) xl = *(const uint4*)xl_lds[d][i * 64 + ln];
                 rp_u32x2 b0, b1, a0, a1, l0, l1;
                 b0.x = (w & 0x000F000Fu) | kor;
                 b0.y = ((w >> 4) & 0x000F000Fu) | kor;
@@ -185,8 +193,10 @@ __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs
                 l0.x = xl.x; l0.y = xl.y; l1.x = xl.z; l1.y = xl.w;
                 dh = rp_mfma<DT>(a0, b0, dh);
                 dh = rp_mfma<DT>(a1, b1, dh);
-                dl = rp_mfma<DT>(l0, b0, dl);
-                dl = rp_mfma<DT>(l1, b1, dl);
+                if constexpr (NORM) {
+                    dl = rp_mfma<DT>(l0, b0, dl);
+                    dl = rp_mfma<DT>(l1, b1, dl);
+                }
             }
             const uint32_t sch = 16u * ((((uint32_t)(i * 64 + (int)lane) * CPC) >> LOG2G) & 1u);   // the half of the dword the chunk's group is in
             t = fmaf(rp_up<DT>((r.sc[i] >> sch) & 0xFFFFu), fmaf(rp_diag(dl, j0, j1), REM, rp_diag(dh, j0, j1)), t);
@@ -206,20 +216,45 @@ __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs
     // them, that wait has to hold for the path that issued nothing, and waits for them.)
     const uint32_t cnt = (last - gw) / GW + 1u;   // rows of this wave: gw, gw + GW, ... (gw <= last here)
     uint32_t row = gw;
-    if (cnt == 1u) {
-        work_row(row, bufA);
-        return;
+    // (The norm's instances for rows of 8192 codes have no register to spare for a second way of ending: they run
+    // whole turns, the last of which loads the matrix's last row once more for nobody, and end on the odd row.)
+    constexpr bool WHOLE_TURNS = NORM && CH == 4;
+    if constexpr (WHOLE_TURNS) {
+        if (cnt == 1u) {
+            work_row(row, bufA);
+            return;
+        }
     }
-    for (uint32_t it = cnt >> 1; it != 0u; it--) {   // two rows a turn
+    for (uint32_t it = WHOLE_TURNS ? cnt >> 1 : (cnt - 1u) >> 1; it != 0u; it--) {   // two rows a turn (while a third is there to be loaded)
         load_row(row + GW, bufB);
         RP_KEEP_ORDER();
         work_row(row, bufA);
-        load_row(row + 2u * GW, bufA);   // (the last turn of an even number of rows loads the matrix's last row instead, and nobody reads it)
+        load_row(row + 2u * GW, bufA);
         RP_KEEP_ORDER();
         work_row(row + GW, bufB);
         row += 2u * GW;
     }
-    if (cnt & 1u) work_row(row, bufA);
+    if constexpr (WHOLE_TURNS) {
+        if (cnt & 1u) work_row(row, bufA);
+    } else if (cnt & 1u) {   // one row is left, or two; the first of them is loaded
+        RP_KEEP_ORDER();     // (both ways start behind a fence of their own, so that the work on the first row is not lifted above the branch)
+        work_row(row, bufA);
+    } else {
+        load_row(row + GW, bufB);
+        RP_KEEP_ORDER();
+        work_row(row, bufA);
+        RP_KEEP_ORDER();
+        work_row(row + GW, bufB);
+    }
+}
+
+// (four waves per SIMD: two workgroups of eight waves, or one of sixteen, per compute unit)
+template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs a) {
+    qmv_rows_walk_body<DT, CH, LOG2G, NWV, true>(a);
+}
+// The same walk without the norm: out[n] = sum_k (s q + b)[n, k] x[k], the activations as they are (one operand set).
+template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_walk_kernel(QmvRowsNArgs a) {
+    qmv_rows_walk_body<DT, CH, LOG2G, NWV, false>(a);
 }
 
 // 4-bit codes, rows of 4096 or 8192 codes, groups of 32 / 64 / 128, f16 / bf16
@@ -230,28 +265,63 @@ bool qmv_rows_norm_takes(const QmvParams& p, const void* norm_w) {
     return !((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)norm_w % 16 || (uintptr_t)p.scales % 8 || (uintptr_t)p.biases % 8 || (uintptr_t)p.out % 2);
 }
 
-template <int DT, int LOG2G> static const void* rows_norm_fn(uint32_t K, bool sixteen) {
-    if (sixteen) return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 16>;
-    return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 8>;
+template <int DT, int LOG2G, bool NORM> static const void* rows_walk_fn(uint32_t K, bool sixteen) {
+    if constexpr (NORM) {
+        if (sixteen) return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 16>;
+        return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 8>;
+    } else {
+        if (sixteen) return K == 4096 ? (const void*)qmv_rows_walk_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_walk_kernel<DT, 4, LOG2G, 16>;
+        return K == 4096 ? (const void*)qmv_rows_walk_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_walk_kernel<DT, 4, LOG2G, 8>;
+    }
 }
 
-int launch_qmv_rows_norm(const QmvParams& p, const void* norm_w, const float* eps, const LaunchCtx& lc) {
-    if (!qmv_rows_norm_takes(p, norm_w) || !eps) return fail(ERR_UNSUPPORTED, "norm + qmv rows kernel: 4-bit codes, rows of 4096 or 8192 codes, f16 / bf16");
+template <bool NORM> static int launch_rows_walk(const QmvParams& p, const void* norm_w, const float* eps, const LaunchCtx& lc) {
     QmvRowsNArgs a{(const rp_u32x4*)p.w, (const uint16_t*)p.scales, (const uint16_t*)p.biases, (const uint16_t*)p.x, (uint16_t*)p.out, p.N,
                    (const uint16_t*)norm_w, eps};
     void* args[] = {&a};
     const uint32_t G = p.group_size;
-    // Up to 4096 rows one workgroup of sixteen waves per 16 rows (4096 x 4096 bf16: 4.5 us against 5.6 in workgroups of
-    // eight); beyond, two workgroups of eight waves per compute unit, which walk the rows (14336 x 4096: 10.0 either way;
-    // eight hold on the machines where a launch of exactly one large workgroup per compute unit falls behind).
+    // Up to 4096 rows one workgroup of sixteen waves per 16 rows (norm, 4096 x 4096 bf16: 4.5 us against 5.6 in workgroups of
+    // eight); beyond, two workgroups of eight waves per compute unit, which walk the rows (14336 x 4096: the same either
+    // way; eight hold on the machines where a launch of exactly one large workgroup per compute unit falls behind).
     const bool sixteen = p.N <= 4096;
     const uint32_t nwv = sixteen ? 16u : 8u, cap = sixteen ? 256u : 512u;
-    const void* fn = p.dtype == DT_BF16 ? (G == 32 ? rows_norm_fn<DT_BF16, 5>(p.K, sixteen) : G == 64 ? rows_norm_fn<DT_BF16, 6>(p.K, sixteen) : rows_norm_fn<DT_BF16, 7>(p.K, sixteen))
-                                        : (G == 32 ? rows_norm_fn<DT_F16, 5>(p.K, sixteen) : G == 64 ? rows_norm_fn<DT_F16, 6>(p.K, sixteen) : rows_norm_fn<DT_F16, 7>(p.K, sixteen));
+    const void* fn = p.dtype == DT_BF16 ? (G == 32 ? rows_walk_fn<DT_BF16, 5, NORM>(p.K, sixteen) : G == 64 ? rows_walk_fn<DT_BF16, 6, NORM>(p.K, sixteen) : rows_walk_fn<DT_BF16, 7, NORM>(p.K, sixteen))
+                                        : (G == 32 ? rows_walk_fn<DT_F16, 5, NORM>(p.K, sixteen) : G == 64 ? rows_walk_fn<DT_F16, 6, NORM>(p.K, sixteen) : rows_walk_fn<DT_F16, 7, NORM>(p.K, sixteen));
     const uint32_t wgs = (p.N + nwv - 1u) / nwv;
     hipError_t e = launch_kernel(fn, dim3(wgs < cap ? wgs : cap), dim3(64u * nwv), args, 0, lc);
-    if (e != hipSuccess) return hip_fail(e, "norm + qmv rows kernel launch");
+    if (e != hipSuccess) return hip_fail(e, NORM ? "norm + qmv rows kernel launch" : "qmv walking rows kernel launch");
     return ERR_OK;
+}
+
+int launch_qmv_rows_norm(const QmvParams& p, const void* norm_w, const float* eps, const LaunchCtx& lc) {
+    if (!qmv_rows_norm_takes(p, norm_w) || !eps) return fail(ERR_UNSUPPORTED, "norm + qmv rows kernel: 4-bit codes, rows of 4096 or 8192 codes, f16 / bf16");
+    return launch_rows_walk<true>(p, norm_w, eps, lc);
+}
+
+// The plain GEMV on the same walk: one activation row against one matrix.
+bool qmv_rows_walk_takes(const QmvParams& p) {
+    return p.gather == GATHER_NONE && p.M == 1 && qmv_rows_norm_takes(p, p.x);   // (the alignment of x stands in for that of the norm weights)
+}
+
+// Where it is ahead of the kernels that work a row block per wave and end (bf16 g64, us, those -> this, same run):
+// rows of 4096 codes, 1536 / 2048 / 4096 / 6144 / 8192 / 14336 / 16384 / 28672 / 32768 weight rows 3.35 -> 3.25, 3.46 -> 3.30,
+// 4.14 -> 3.82, 5.07 -> 4.38, 5.58 -> 5.02, 7.93 -> 7.45, 8.35 -> 8.27, 13.07 -> 12.72, 14.32 -> 14.0 (1024 rows: 3.15 -> 3.19), level
+// at 40960, behind between (49152 / 57344 / 65536 rows 19.98 -> 20.2, 22.57 -> 23.19, 25.3 -> 25.65: the streaming kernel's
+// sizes) and ahead again from 81920 (30.8 against 32.1; 98304 36.0 / 37.5; 128256 45.96 / 47.45); other group sizes alike
+// (14336 x 4096: f16 g32 8.71 -> 7.7, bf16 g128 8.05 -> 7.2 - 7.5). Rows of 8192 codes from 10240 weight rows (10240 /
+// 12288 / 14336 / 16384 / 20480 / 28672 / 40960 / 57344: 10.7 -> 9.65, 11.4 -> 10.8, 13.8 -> 12.6, 14.5 -> 14.15, 18.3 -> 16.4, 22.5 -> 21.8,
+// 32.1 -> 30.4, 41.9 -> 41.3; f16 g32 14336 / 28672 14.3 -> 13.6, 24.9 -> 23.5); below that the one-row-per-wave kernel
+// holds (8192 x 8192 f16 g32 / g64 / g128 8.70 / 8.84, 8.4 / 8.37, 7.68 / 8.12; 4096 x 8192 5.04 / 5.42), and so it does
+// in groups of 128 (14336 x 8192: 12.59 / 12.80).
+bool qmv_rows_walk_preferred(const QmvParams& p) {
+    if (!qmv_rows_walk_takes(p)) return false;
+    if (p.K == 4096) return p.N >= 1536 && (p.N <= 40960 || p.N >= 81920);
+    return p.N >= 10240 && p.group_size != 128;
+}
+
+int launch_qmv_rows_walk(const QmvParams& p, const LaunchCtx& lc) {
+    if (!qmv_rows_walk_takes(p)) return fail(ERR_UNSUPPORTED, "qmv walking rows kernel: one activation row, 4-bit codes, rows of 4096 or 8192 codes, f16 / bf16");
+    return launch_rows_walk<false>(p, nullptr, nullptr, lc);
 }
 
 }  // namespace mtq

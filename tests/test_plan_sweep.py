@@ -119,12 +119,23 @@ def test_benchmark_configurations_are_routed_as_documented():
         return [l[0] for l in launches], launches
 
     ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 14336, 4096)
-    assert "qmv_rows_kernel<2, 0, false>" in ks[0] and ls[0][1][0] == 256 and ls[0][2][0] == 14 * 64   # one workgroup of 14 waves x 4 rows per compute unit
-    ks, _ = kernels("qmv", DType.F16, 4, 64, 1, 4100, 4096)
+    assert "qmv_rows_walk_kernel<2, 2, 6, 8>" in ks[0] and ls[0][1][0] == 512 and ls[0][2][0] == 512   # two workgroups of eight waves per compute unit walk the rows
+    ks, ls = kernels("qmv", DType.F16, 4, 32, 1, 4096, 4096)
+    assert "qmv_rows_walk_kernel<1, 2, 5, 16>" in ks[0] and ls[0][1][0] == 256 and ls[0][2][0] == 1024   # up to 4096 rows: sixteen rows per workgroup
+    ks, _ = kernels("qmv", DType.BF16, 4, 64, 1, 128256, 4096)
+    assert "qmv_rows_walk_kernel<2, 2, 6, 8>" in ks[0]
+    ks, _ = kernels("qmv", DType.BF16, 4, 64, 1, 57344, 4096)      # the sizes between stay on the streaming kernel
+    assert "qmv_stream_kernel" in ks[0]
+    ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 28672, 8192)
+    assert "qmv_rows_walk_kernel<2, 4, 6, 8>" in ks[0] and ls[0][1][0] == 512
+    ks, _ = kernels("qmv", DType.F16, 4, 64, 1, 1100, 4096)        # below the walk's sizes: the wave-per-four-rows kernel
     assert "qmv_rows_kernel<1, 0, false>" in ks[0]
-    for args in ((DType.BF16, 4, 64, 1, 4098, 4096), (DType.BF16, 4, 32, 1, 4096, 4096), (DType.BF16, 4, 64, 2, 4096, 4096),
+    for args in ((DType.BF16, 4, 64, 1, 1026, 4096), (DType.BF16, 4, 32, 1, 1024, 4096), (DType.BF16, 4, 64, 2, 4096, 4096),
                  (DType.BF16, 8, 64, 1, 4096, 4096), (DType.BF16, 4, 64, 1, 512, 4096)):
         assert "qmv_rows_kernel" not in kernels("qmv", *args)[0][0]          # what that kernel does not take
+    for args in ((DType.BF16, 4, 64, 2, 14336, 4096), (DType.BF16, 8, 64, 1, 14336, 4096), (DType.BF16, 2, 64, 1, 14336, 8192),
+                 (DType.F32, 4, 64, 1, 14336, 4096), (DType.BF16, 4, 64, 1, 14336, 2048), (DType.BF16, 4, 16, 1, 14336, 4096)):
+        assert "qmv_rows_walk_kernel" not in kernels("qmv", *args)[0][0]     # nor the walk: one row, 4-bit, 4096 / 8192 codes, groups of 32 / 64 / 128
     ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 4096, 14336)
     assert "qmv_rows_long_kernel<2, 4, 7, 6>" in ks[0] and ls[0][1][0] == 512 and ls[0][2][0] == 512   # workgroups of eight rows
     for bits, G, name in ((2, 32, "<1, 2, 2, 5>"), (2, 128, "<1, 2, 2, 7>"), (4, 64, "<1, 4, 4, 6>")):   # the one-row cells of the width / group sweep
