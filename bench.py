@@ -38,8 +38,8 @@ qkv` / `gated_norm` the fused one-launch decode pieces (Q + K + V projections;
 gated RMSNorm + out projection at the reference's bench shape); `--workload
 gather_decode` one token's top-2 routed gate / up / down launches over 8
 experts (the routed wave-per-row kernels); `--workload rows_probe` the headline gate / up launch taken apart (the shipped kernel, the
-streaming kernel it replaced, a launch that only reads the same bytes, and the
-shipped kernel without its arithmetic / with its weight loads only, plus its
+streaming and wave-per-four-rows kernels it replaced, a launch that only reads the same bytes, and the
+wave-per-four-rows kernel without its arithmetic / with its weight loads only, plus its
 per-wave timeline), which is where the distance to the HBM peak is accounted
 for.
 
@@ -516,9 +516,10 @@ def leg_sweep(a, runner, info):
 
 def leg_rows_probe(a, runner, info):
     """The 14336 x 4096 launch of the headline on the same 24 cold operand sets, in one process: mt_qmv on the streaming
-    kernel (LDS-staged scales, dot2) and as shipped (the wave-per-four-rows kernel), a launch that only reads the same
-    weights, and the wave-per-four-rows kernel through its measurement entry point in full, without its arithmetic and
-    with its weight loads only; then that kernel's per-wave timeline (constant-rate counter, 10 ns)."""
+    kernel (LDS-staged scales, dot2), on the wave-per-four-rows kernel and as shipped (the kernel whose waves walk the
+    rows), a launch that only reads the same weights, and the wave-per-four-rows kernel through its measurement entry
+    point in full, without its arithmetic and with its weight loads only; then that kernel's per-wave timeline
+    (constant-rate counter, 10 ns)."""
     import numpy as np
     from metaltile_amd import DType, GpuBuffer
     from metaltile_amd.synth import make_case, qmv_bytes
@@ -544,10 +545,10 @@ def leg_rows_probe(a, runner, info):
     # rounds' averages is reported (each average is over reps x 24 back-to-back launches)
     from metaltile_amd import _lib
     lib = _lib.load()
-    rounds = {k: [] for k in ("mt_qmv_streaming_kernel", "mt_qmv_shipped", "read_only", "probe_full", "probe_no_arithmetic", "probe_weight_loads_only")}
+    rounds = {k: [] for k in ("mt_qmv_streaming_kernel", "mt_qmv_wave_per_four_rows", "mt_qmv_shipped", "read_only", "probe_full", "probe_no_arithmetic", "probe_weight_loads_only")}
     wbytes = N * K // 2 // 16 * 16
     for _ in range(3):
-        for key, opt in (("mt_qmv_streaming_kernel", 2), ("mt_qmv_shipped", 0)):   # (shipped: the wave-per-four-rows kernel at this shape)
+        for key, opt in (("mt_qmv_streaming_kernel", 2), ("mt_qmv_wave_per_four_rows", 3), ("mt_qmv_shipped", 0)):   # (shipped: waves walking the rows at this shape)
             _lib.check(lib.mtq_set_option(b"qmv.kernel", opt))
             try:
                 runner.dispatch_chain(specs, repeat=max(reps // 2, 40), per_kernel=False)
@@ -737,7 +738,7 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBS, 4),
                          "traffic": traffic_from_profiles("qkv_fused_bf16_b4_llama_attn"),
-                         "kernel": "mtq::qmv_stream_kernel<bf16, 4-bit, 1 row>, 3 matrices per launch",
+                         "kernel": "mtq::qmv_rows_walk_batched_kernel<2, 2, 6, 8> (bf16, rows of 4096 4-bit codes in groups of 64), 3 matrices per launch",
                          "avg_launch_us_timed_region": round(kern_avg, 3), "clock": clock},
         })
         print(json.dumps(out))

@@ -222,6 +222,9 @@ int launch_qmv_rows_norm(const QmvParams& p, const void* norm_w, const float* ep
 bool qmv_rows_walk_takes(const QmvParams& p);
 bool qmv_rows_walk_preferred(const QmvParams& p);
 int launch_qmv_rows_walk(const QmvParams& p, const LaunchCtx& lc);
+bool qmv_rows_walk_batched_takes(const QmvParams& p, const QmvBatch& b);       // (p: dtype, bits, group size, x, K)
+bool qmv_rows_walk_batched_preferred(const QmvParams& p, const QmvBatch& b);
+int launch_qmv_rows_walk_batched(const QmvParams& p, const QmvBatch& b, const LaunchCtx& lc);
 // Two to four activation rows (qmv_rows_few.hip): one wave per four weight rows; 4096 or 8192 4-bit codes or 8192 2-bit codes per
 // row, groups of 32 / 64 / 128, f16 / bf16.
 bool qmv_rows_few_takes(const QmvParams& p);

@@ -29,6 +29,13 @@ struct QmvRowsNArgs {
     uint32_t N;
     const uint16_t* norm_w;   // [K]
     const float* norm_eps;    // one f32 on the device
+    // Several matrices against the one activation row (the batched instances): the rows of matrix m are rows
+    // first[m] .. first[m + 1] - 1 of the launch, N is their total; unused slots hold the total.
+    const rp_u32x4* mw[4];
+    const uint16_t* ms[4];
+    const uint16_t* mb[4];
+    uint16_t* mo[4];
+    uint32_t first[5];
 };
 
 // One row's loads of one lane, as they come from memory: whatever has to be done to a loaded value (picking the 16-bit
@@ -40,7 +47,7 @@ template <int CH> struct RowsNormBuf {
     uint32_t sw[2], bw[2];   // the lane's groups of the bias term, two 16-bit elements per dword (one group per lane: the dword that holds it)
 };
 
-template <int DT, int CH, int LOG2G, int NWV, bool NORM>
+template <int DT, int CH, int LOG2G, int NWV, bool NORM, bool BATCH = false>
 __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
     constexpr float REM = 1.0f / RemSplit<DT>::kRemScale;
@@ -60,8 +67,19 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     const uint32_t gl = min(lane, (uint32_t)(GPR / GPL - 1));
     auto load_row = [&](uint32_t row, RowsNormBuf<CH>& r) {   // row <= last
         row = min(row, last);   // (it is; a scalar instruction keeps the loads inside the matrix whatever the caller does)
-        const uint16_t* sp = a.s + (size_t)row * GPR;
-        const uint16_t* bp = a.b + (size_t)row * GPR;
+        const uint16_t *sp, *bp;
+        const rp_u32x4* wrow;
+        if constexpr (BATCH) {   // (row numbers are the same in every lane: the matrix is picked by scalar code)
+            const uint32_t m = (uint32_t)(row >= a.first[1]) + (uint32_t)(row >= a.first[2]) + (uint32_t)(row >= a.first[3]);
+            const uint32_t local = row - a.first[m];   // < the rows of matrix m, as row < first[m + 1]
+            sp = a.ms[m] + (size_t)local * GPR;
+            bp = a.mb[m] + (size_t)local * GPR;
+            wrow = a.mw[m] + (size_t)local * C;
+        } else {
+            sp = a.s + (size_t)row * GPR;
+            bp = a.b + (size_t)row * GPR;
+            wrow = a.w + (size_t)row * C;
+        }
 #pragma unroll
         for (int i = 0; i < CH; i++) r.sc[i] = ((const uint32_t*)sp)[((uint32_t)(i * 64 + (int)lane) * CPC) >> (LOG2G + 1)];
         r.sw[0] = r.sw[1] = r.bw[0] = r.bw[1] = 0u;
@@ -75,7 +93,7 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
             r.sw[0] = ((const uint32_t*)sp)[gl >> 1];
             r.bw[0] = ((const uint32_t*)bp)[gl >> 1];
         }
-        const rp_u32x4* wbase = a.w + (size_t)row * C + lane;
+        const rp_u32x4* wbase = wrow + lane;
 #pragma unroll
         for (int i = 0; i < CH; i++) r.wv[i] = __builtin_nontemporal_load(wbase + i * 64);
     };
@@ -207,7 +225,14 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
         t += dpp_f32<0x141>(t);
         t += dpp_f32<0x140>(t);
         t += __shfl_xor(t, 16, 64);
-        if (lane == 0 && row <= last) a.out[row] = f32_to_elem_bits<DT>(t);
+        if (lane == 0 && row <= last) {
+            if constexpr (BATCH) {
+                const uint32_t m = (uint32_t)(row >= a.first[1]) + (uint32_t)(row >= a.first[2]) + (uint32_t)(row >= a.first[3]);
+                a.mo[m][row - a.first[m]] = f32_to_elem_bits<DT>(t);
+            } else {
+                a.out[row] = f32_to_elem_bits<DT>(t);
+            }
+        }
     };
     // ---- this wave's rows, each row's loads in flight while the row before it is worked on ------------------------------
     // A row's loads and the work on the row before it stand in one block of straight-line code, in a counted loop with
@@ -256,6 +281,12 @@ template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * 
 template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_walk_kernel(QmvRowsNArgs a) {
     qmv_rows_walk_body<DT, CH, LOG2G, NWV, false>(a);
 }
+// Two to four matrices against the one activation row in one launch (the fused projections of a decode step:
+// ffai_batched_qkv_qgemv_fast, crates/metaltile-std/src/ffai/batched_qkv_qgemv.rs:157; ffai_batched_4_qgemv_fast,
+// crates/metaltile-std/src/ffai/batched_4_qgemv.rs:60): the launch's rows are the matrices' rows one after the other.
+template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_walk_batched_kernel(QmvRowsNArgs a) {
+    qmv_rows_walk_body<DT, CH, LOG2G, NWV, false, true>(a);
+}
 
 // 4-bit codes, rows of 4096 or 8192 codes, groups of 32 / 64 / 128, f16 / bf16
 bool qmv_rows_norm_takes(const QmvParams& p, const void* norm_w) {
@@ -263,6 +294,11 @@ bool qmv_rows_norm_takes(const QmvParams& p, const void* norm_w) {
     const uint32_t G = p.group_size;
     if (G != 32 && G != 64 && G != 128) return false;
     return !((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)norm_w % 16 || (uintptr_t)p.scales % 8 || (uintptr_t)p.biases % 8 || (uintptr_t)p.out % 2);
+}
+
+template <int DT, int LOG2G> static const void* rows_walk_batched_fn(uint32_t K, bool sixteen) {
+    if (sixteen) return K == 4096 ? (const void*)qmv_rows_walk_batched_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_walk_batched_kernel<DT, 4, LOG2G, 16>;
+    return K == 4096 ? (const void*)qmv_rows_walk_batched_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_walk_batched_kernel<DT, 4, LOG2G, 8>;
 }
 
 template <int DT, int LOG2G, bool NORM> static const void* rows_walk_fn(uint32_t K, bool sixteen) {
@@ -275,9 +311,23 @@ template <int DT, int LOG2G, bool NORM> static const void* rows_walk_fn(uint32_t
     }
 }
 
-template <bool NORM> static int launch_rows_walk(const QmvParams& p, const void* norm_w, const float* eps, const LaunchCtx& lc) {
-    QmvRowsNArgs a{(const rp_u32x4*)p.w, (const uint16_t*)p.scales, (const uint16_t*)p.biases, (const uint16_t*)p.x, (uint16_t*)p.out, p.N,
-                   (const uint16_t*)norm_w, eps};
+// p.N is the launch's rows: the matrix's, or the total of the batch's matrices
+template <bool NORM> static int launch_rows_walk(const QmvParams& p, const void* norm_w, const float* eps, const LaunchCtx& lc, const QmvBatch* batch = nullptr) {
+    QmvRowsNArgs a{};
+    a.w = (const rp_u32x4*)p.w; a.s = (const uint16_t*)p.scales; a.b = (const uint16_t*)p.biases; a.x = (const uint16_t*)p.x; a.out = (uint16_t*)p.out;
+    a.N = p.N; a.norm_w = (const uint16_t*)norm_w; a.norm_eps = eps;
+    if (batch) {
+        uint32_t at = 0;
+        for (int j = 0; j < 4; j++) {
+            const int k = j < batch->n ? j : 0;   // (unused slots repeat matrix 0 and start at the total: no row reaches them)
+            a.mw[j] = (const rp_u32x4*)batch->w[k]; a.ms[j] = (const uint16_t*)batch->scales[k]; a.mb[j] = (const uint16_t*)batch->biases[k];
+            a.mo[j] = (uint16_t*)batch->out[k];
+            a.first[j] = at;
+            if (j < batch->n) at += batch->N[j];
+        }
+        a.first[4] = at;
+        if (at != p.N) return fail(ERR_BAD_ARG, "qmv walking rows kernel: the batch's rows do not add up");
+    }
     void* args[] = {&a};
     const uint32_t G = p.group_size;
     // Up to 4096 rows one workgroup of sixteen waves per 16 rows (norm, 4096 x 4096 bf16: 4.5 us against 5.6 in workgroups of
@@ -287,6 +337,11 @@ template <bool NORM> static int launch_rows_walk(const QmvParams& p, const void*
     const uint32_t nwv = sixteen ? 16u : 8u, cap = sixteen ? 256u : 512u;
     const void* fn = p.dtype == DT_BF16 ? (G == 32 ? rows_walk_fn<DT_BF16, 5, NORM>(p.K, sixteen) : G == 64 ? rows_walk_fn<DT_BF16, 6, NORM>(p.K, sixteen) : rows_walk_fn<DT_BF16, 7, NORM>(p.K, sixteen))
                                         : (G == 32 ? rows_walk_fn<DT_F16, 5, NORM>(p.K, sixteen) : G == 64 ? rows_walk_fn<DT_F16, 6, NORM>(p.K, sixteen) : rows_walk_fn<DT_F16, 7, NORM>(p.K, sixteen));
+    if (batch) {
+        if constexpr (NORM) return fail(ERR_UNSUPPORTED, "norm + qmv rows kernel: one matrix");
+        fn = p.dtype == DT_BF16 ? (G == 32 ? rows_walk_batched_fn<DT_BF16, 5>(p.K, sixteen) : G == 64 ? rows_walk_batched_fn<DT_BF16, 6>(p.K, sixteen) : rows_walk_batched_fn<DT_BF16, 7>(p.K, sixteen))
+                                : (G == 32 ? rows_walk_batched_fn<DT_F16, 5>(p.K, sixteen) : G == 64 ? rows_walk_batched_fn<DT_F16, 6>(p.K, sixteen) : rows_walk_batched_fn<DT_F16, 7>(p.K, sixteen));
+    }
     const uint32_t wgs = (p.N + nwv - 1u) / nwv;
     hipError_t e = launch_kernel(fn, dim3(wgs < cap ? wgs : cap), dim3(64u * nwv), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, NORM ? "norm + qmv rows kernel launch" : "qmv walking rows kernel launch");
@@ -317,6 +372,36 @@ bool qmv_rows_walk_preferred(const QmvParams& p) {
     if (!qmv_rows_walk_takes(p)) return false;
     if (p.K == 4096) return p.N >= 1536 && (p.N <= 40960 || p.N >= 81920);
     return p.N >= 10240 && p.group_size != 128;
+}
+
+// The batch on one walk: every matrix as the single one would have to be, the rows counted together.
+static bool rows_walk_batch_as_one(const QmvParams& p0, const QmvBatch& b, QmvParams& p) {
+    if (b.n < 2 || b.n > 4) return false;
+    p = p0;
+    p.gather = GATHER_NONE;
+    p.M = 1;
+    uint64_t total = 0;
+    for (int j = 0; j < b.n; j++) {
+        p.w = b.w[j]; p.scales = b.scales[j]; p.biases = b.biases[j]; p.out = b.out[j]; p.N = b.N[j];
+        if (!b.w[j] || !b.scales[j] || !b.biases[j] || !b.out[j] || !qmv_rows_walk_takes(p)) return false;
+        total += b.N[j];
+    }
+    if (total > (1u << 24)) return false;
+    p.N = (uint32_t)total;
+    return true;
+}
+bool qmv_rows_walk_batched_takes(const QmvParams& p0, const QmvBatch& b) {
+    QmvParams p;
+    return rows_walk_batch_as_one(p0, b, p);
+}
+bool qmv_rows_walk_batched_preferred(const QmvParams& p0, const QmvBatch& b) {
+    QmvParams p;
+    return rows_walk_batch_as_one(p0, b, p) && qmv_rows_walk_preferred(p);   // (sized as one matrix of all the rows)
+}
+int launch_qmv_rows_walk_batched(const QmvParams& p0, const QmvBatch& b, const LaunchCtx& lc) {
+    QmvParams p;
+    if (!rows_walk_batch_as_one(p0, b, p)) return fail(ERR_UNSUPPORTED, "qmv walking rows kernel: 2 to 4 matrices of 4-bit codes, rows of 4096 or 8192 codes, f16 / bf16");
+    return launch_rows_walk<false>(p, nullptr, nullptr, lc, &b);
 }
 
 int launch_qmv_rows_walk(const QmvParams& p, const LaunchCtx& lc) {

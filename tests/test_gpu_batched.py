@@ -49,31 +49,56 @@ def _expected(oracle, c, x_f, dt):
     return oracle.round_through(exp.astype(np.float32), ODT[dt])
 
 
+def _walks(dt, bits, G, K, Ns):
+    """What the kernel whose waves walk the rows takes of a batch: 2 to 4 matrices of 4-bit codes in rows of 4096 / 8192
+    codes, groups of 32 / 64 / 128, f16 / bf16."""
+    return bits == 4 and K in (4096, 8192) and G in (32, 64, 128) and dt != DType.F32 and 2 <= len(Ns) <= 4
+
+
+CASES += [
+    (DType.F16, 4, 32, 4096, (5, 1030, 77, 4100)),    # the walking kernel, ragged: four matrices, 5212 rows (two per wave and one)
+    (DType.BF16, 4, 128, 8192, (1024, 40)),           # rows of 8192 codes, one row per wave
+    (DType.BF16, 4, 64, 8192, (8192, 1024, 1027)),    # 10243 rows of 8192 codes: its automatic size
+    (DType.F16, 4, 64, 4096, (16, 16)),               # two waves' worth
+]
+
+
 @pytest.mark.parametrize("dt,bits,G,K,Ns", CASES, ids=lambda v: getattr(v, "name", str(v).replace(" ", "")))
 def test_batched_matches_single_and_oracle(oracle, dt, bits, G, K, Ns):
+    """As routed (qmv.kernel = 0), on the streaming kernel (2) and, where it applies, on the kernel whose waves walk the
+    rows (4): against the oracle every time, and bit for bit against the single-matrix launch on the same kernel."""
     print(f"[case] qmv_batched {dt.name} b{bits} g{G} K{K} N{Ns}", flush=True)
     cases, x, dev = _operands(900, dt, bits, G, K, Ns)
     esz = dt.size_bytes
-    outs = [GpuBuffer.from_bytes(b"\xff" * (N * esz)) for N in Ns]  # NaN fill: every element must be written
-    ops.qmv_batched(dt, bits, G, [d[0] for d in dev], [d[1] for d in dev], [d[2] for d in dev], x, outs, list(Ns), K)
-    for c, d, o, N in zip(cases, dev, outs, Ns):
-        raw = o.read_bytes(N * esz)
-        got = unpack_f32(raw, dt)
-        assert np.isfinite(got).all()
-        assert rel_err(got, _expected(oracle, c, cases[0].x_f, dt)) <= TOL[dt]
-        if bits in (2, 4, 8):
-            # the batched launch is the streaming kernel: the single launch on that kernel (a row of 4096 4-bit codes
-            # would otherwise take the wave-per-four-rows kernel, whose f32 sums meet in another order)
-            single = GpuBuffer(N * esz)
-            lib = _lib.load()
-            assert lib.mtq_set_option(b"qmv.kernel", 2) == 0
-            try:
-                ops.qmv(dt, bits, G, d[0], d[1], d[2], x, single, 1, N, K)
-            finally:
-                lib.mtq_set_option(b"qmv.kernel", 0)
-            assert single.read_bytes(N * esz) == raw, "batched launch must reproduce the single launch bit for bit"
-            single.free()
-    for b in [x] + outs + [t for d in dev for t in d]:
+    lib = _lib.load()
+    from metaltile_amd import GpuRunner
+    for opt in (0, 2, 4):
+        if opt == 4 and not _walks(dt, bits, G, K, Ns):
+            continue
+        outs = [GpuBuffer.from_bytes(b"\xff" * (N * esz + 16)) for N in Ns]  # NaN fill: every element must be written, none after the last
+        assert lib.mtq_set_option(b"qmv.kernel", opt) == 0
+        try:
+            GpuRunner(0).flush_slc()
+            ops.qmv_batched(dt, bits, G, [d[0] for d in dev], [d[1] for d in dev], [d[2] for d in dev], x, outs, list(Ns), K)
+            for c, d, o, N in zip(cases, dev, outs, Ns):
+                whole = o.read_bytes(N * esz + 16)
+                raw = whole[:N * esz]
+                assert whole[N * esz:] == b"\xff" * 16
+                got = unpack_f32(raw, dt)
+                assert np.isfinite(got).all()
+                assert rel_err(got, _expected(oracle, c, cases[0].x_f, dt)) <= TOL[dt]
+                if opt != 0 and bits in (2, 4, 8):
+                    # (as routed, a single row of 4096 4-bit codes may take another kernel than the batch, whose f32 sums
+                    # meet in another order; with the kernel named, batch and single launch are the same arithmetic)
+                    single = GpuBuffer(N * esz)
+                    ops.qmv(dt, bits, G, d[0], d[1], d[2], x, single, 1, N, K)
+                    assert single.read_bytes(N * esz) == raw, "batched launch must reproduce the single launch bit for bit"
+                    single.free()
+        finally:
+            lib.mtq_set_option(b"qmv.kernel", 0)
+        for o in outs:
+            o.free()
+    for b in [x] + [t for d in dev for t in d]:
         b.free()
 
 
