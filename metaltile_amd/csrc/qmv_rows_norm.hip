@@ -47,19 +47,22 @@ template <int CH> struct RowsNormBuf {
     uint32_t sw[2], bw[2];   // the lane's groups of the bias term, two 16-bit elements per dword (one group per lane: the dword that holds it)
 };
 
-template <int DT, int CH, int LOG2G, int NWV, bool NORM, bool BATCH = false>
+template <int DT, int CH, int LOG2G, int NWV, bool NORM, bool BATCH = false, int BITS = 4>
 __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
-    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
+    static_assert(BITS == 4 || (BITS == 2 && !NORM && !BATCH), "4-bit codes; 2-bit codes on the plain walk");
+    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;   // 4-bit codes: one offset for every pair
     constexpr float REM = 1.0f / RemSplit<DT>::kRemScale;
-    constexpr int CPC = 32, Q = 4;           // codes per 16-byte chunk; 16-byte quarters of a chunk's activations in operand order
+    constexpr int CPC = 128 / BITS, Q = CPC / 8;   // codes per 16-byte chunk; 16-byte quarters of a chunk's activations in operand order
     constexpr int C = 64 * CH, K = C * CPC;
     constexpr int GPR = K >> LOG2G;          // groups per row
     constexpr int GPL = GPR > 128 ? 4 : GPR > 64 ? 2 : 1;   // groups a lane owns in the bias term (lanes below GPR / GPL)
-    constexpr int SPG = (1 << LOG2G) / (CPC / 2);            // half chunks per group
+    constexpr int NH = (1 << LOG2G) < CPC ? 2 : 1;           // groups a chunk spans (2-bit codes in groups of 32: its halves are accumulated and scaled apart)
+    constexpr int SPG = NH == 2 ? 1 : (1 << LOG2G) / (CPC / 2);   // half chunks per group
     static_assert(C <= 64 * NWV && LOG2G >= 5 && LOG2G <= 7 && GPR % GPL == 0 && GPR / GPL <= 64, "one thread per chunk; groups of 32, 64 or 128 codes, at most 256 per row");
     __shared__ __align__(16) uint32_t xp_lds[Q][C][4];   // [quarter][chunk][4 pair dwords]: the rounded values
     __shared__ __align__(16) uint32_t xl_lds[NORM ? Q : 1][NORM ? C : 1][4];   // the remainders
     __shared__ __align__(16) float xs_lds[2 * C];        // sum of x' over each half chunk
+    __shared__ __align__(16) float xm_lds[BITS == 2 ? 2 * C : 4];   // 2-bit codes: that sum weighted with the pairs' offsets
     __shared__ float ssq_lds[NWV];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t gw = blockIdx.x * (uint32_t)NWV + wave, GW = gridDim.x * (uint32_t)NWV;   // (the same in every lane: row numbers stay in scalar registers)
@@ -81,7 +84,7 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
             wrow = a.w + (size_t)row * C;
         }
 #pragma unroll
-        for (int i = 0; i < CH; i++) r.sc[i] = ((const uint32_t*)sp)[((uint32_t)(i * 64 + (int)lane) * CPC) >> (LOG2G + 1)];
+        for (int i = 0; i < CH; i++) r.sc[i] = ((const uint32_t*)sp)[((uint32_t)(i * 64 + (int)lane) * CPC) >> (LOG2G + 1)];   // (a chunk that spans two groups: both of them)
         r.sw[0] = r.sw[1] = r.bw[0] = r.bw[1] = 0u;
         if constexpr (GPL == 4) {
             const uint2 sv = ((const uint2*)sp)[gl], bv = ((const uint2*)bp)[gl];
@@ -118,6 +121,16 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     const bool j0 = lane & 1u, j1 = lane & 2u;
     uint32_t kor = DT == DT_BF16 ? 0x43004300u : 0x64006400u;   // (2^7, 2^7) in bf16, (2^10, 2^10) in f16: a code OR-ed into the mantissa is MAGIC + q
     asm volatile("" : "+v"(kor));
+    // 2-bit codes: a pair of crumbs masked where it sits (bit 2 p) and OR-ed into 2^(MB - 2 p) is that power of two
+    // plus the code (qmv_rows_common.h); one constant per position class, kept opaque so that an and-or has one literal
+    uint32_t kor2[BITS == 2 ? (DT == DT_F16 ? 5 : 3) : 1] = {};
+    if constexpr (BITS == 2) {
+#pragma unroll
+        for (int p = 0; p < (DT == DT_F16 ? 5 : 3); p++) {
+            kor2[p] = rp_crumb_kor<DT>(p);
+            asm volatile("" : "+v"(kor2[p]));
+        }
+    }
     // ---- the row's sum of squares ------------------------------------------------------------------------------------
     float inv = 1.0f;
     if constexpr (NORM) {
@@ -139,6 +152,8 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
         rp_u32x2 ones;
         ones.x = ones.y = DT == DT_BF16 ? 0x3F803F80u : 0x3C003C00u;
         rp_f32x4 sx[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, sl[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        rp_f32x4 sm[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        if constexpr (BITS == 4) {
 #pragma unroll
         for (int d = 0; d < 4; d++) {       // weight dword d: activations 8 d .. 8 d + 7, pairs (j, j + 4)
             uint4 v = xraw[d], rem = make_uint4(0u, 0u, 0u, 0u);
@@ -164,19 +179,53 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
                 sl[d / 2] = rp_mfma<DT>(l1, ones, sl[d / 2]);
             }
         }
+        } else {
+#pragma unroll
+            for (int d = 0; d < 4; d++) {       // weight dword d: activations 16 d .. 16 d + 15, pairs (i, i + 8)
+                const uint4 lo = xraw[2 * d], hi = xraw[2 * d + 1];
+                uint4 o[2];
+                o[0].x = __builtin_amdgcn_perm(hi.x, lo.x, 0x05040100u);
+                o[0].y = __builtin_amdgcn_perm(hi.x, lo.x, 0x07060302u);
+                o[0].z = __builtin_amdgcn_perm(hi.y, lo.y, 0x05040100u);
+                o[0].w = __builtin_amdgcn_perm(hi.y, lo.y, 0x07060302u);
+                o[1].x = __builtin_amdgcn_perm(hi.z, lo.z, 0x05040100u);
+                o[1].y = __builtin_amdgcn_perm(hi.z, lo.z, 0x07060302u);
+                o[1].z = __builtin_amdgcn_perm(hi.w, lo.w, 0x05040100u);
+                o[1].w = __builtin_amdgcn_perm(hi.w, lo.w, 0x07060302u);
+                *(uint4*)xp_lds[2 * d][tid] = o[0];
+                *(uint4*)xp_lds[2 * d + 1][tid] = o[1];
+                const uint32_t pw[8] = {o[0].x, o[0].y, o[0].z, o[0].w, o[1].x, o[1].y, o[1].z, o[1].w};
+#pragma unroll
+                for (int m = 0; m < 4; m++) {   // pairs 2 m, 2 m + 1
+                    rp_u32x2 av, kv;
+                    av.x = pw[2 * m]; av.y = pw[2 * m + 1];
+                    kv.x = kor2[rp_crumb_class<DT>(2 * m)]; kv.y = kor2[rp_crumb_class<DT>(2 * m + 1)];
+                    sx[d / 2] = rp_mfma<DT>(av, ones, sx[d / 2]);
+                    sm[d / 2] = rp_mfma<DT>(av, kv, sm[d / 2]);
+                }
+            }
+        }
         // (a lane's own sum is the diagonal entry of its block: its first operand against its own second operand)
         xs_lds[2 * tid] = fmaf(rp_diag(sl[0], j0, j1), REM, rp_diag(sx[0], j0, j1));
         xs_lds[2 * tid + 1] = fmaf(rp_diag(sl[1], j0, j1), REM, rp_diag(sx[1], j0, j1));
+        if constexpr (BITS == 2) {
+            xm_lds[2 * tid] = rp_diag(sm[0], j0, j1);
+            xm_lds[2 * tid + 1] = rp_diag(sm[1], j0, j1);
+        }
     }
     __syncthreads();
     if (gw > last) return;
     // the activation sums of this lane's GPL groups of the bias term (the same for every row)
-    float X[GPL];
+    float X[GPL], XM[GPL];   // (XM: the sum weighted with the codes' offsets; 4-bit codes have the one offset)
 #pragma unroll
     for (int v = 0; v < GPL; v++) {
-        X[v] = 0.f;
+        X[v] = XM[v] = 0.f;
 #pragma unroll
-        for (int h = 0; h < SPG; h++) X[v] += xs_lds[(gl * GPL + (uint32_t)v) * SPG + (uint32_t)h];
+        for (int h = 0; h < SPG; h++) {
+            X[v] += xs_lds[(gl * GPL + (uint32_t)v) * SPG + (uint32_t)h];
+            if constexpr (BITS == 2) XM[v] += xm_lds[(gl * GPL + (uint32_t)v) * SPG + (uint32_t)h];
+        }
+        if constexpr (BITS == 4) XM[v] = MAGIC * X[v];
     }
     auto work_row = [&](uint32_t row, const RowsNormBuf<CH>& r) {
         float t = 0.f;
@@ -190,34 +239,68 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
                 const uint32_t sh = GPL == 1 ? 16u * (gl & 1u) : 16u * (uint32_t)(v & 1);
                 const float sf = rp_up<DT>((r.sw[v >> 1] >> sh) & 0xFFFFu), bf = rp_up<DT>((r.bw[v >> 1] >> sh) & 0xFFFFu);
                 t = fmaf(bf, X[v], t);
-                t = fmaf(0.f - sf, MAGIC * X[v], t);
+                t = fmaf(0.f - sf, XM[v], t);
             }
         }
 #pragma unroll
         for (int i = 0; i < CH; i++) {
-            rp_f32x4 dh = {0.f, 0.f, 0.f, 0.f}, dl = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (BITS == 4) {
+                rp_f32x4 dh = {0.f, 0.f, 0.f, 0.f}, dl = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int d = 0; d < 4; d++) {
-                const uint32_t w = r.wv[i][d];
-                const uint4 xo = *(const uint4*)xp_lds[d][i * 64 + ln];
-                uint4 xl = make_uint4(0u, 0u, 0u, 0u);
-                if constexpr (NORM) xl = *(const uint4*)xl_lds[d][i * 64 + ln];
-                rp_u32x2 b0, b1, a0, a1, l0, l1;
-                b0.x = (w & 0x000F000Fu) | kor;
-                b0.y = ((w >> 4) & 0x000F000Fu) | kor;
-                b1.x = ((w >> 8) & 0x000F000Fu) | kor;
-                b1.y = ((w >> 12) & 0x000F000Fu) | kor;
-                a0.x = xo.x; a0.y = xo.y; a1.x = xo.z; a1.y = xo.w;
-                l0.x = xl.x; l0.y = xl.y; l1.x = xl.z; l1.y = xl.w;
-                dh = rp_mfma<DT>(a0, b0, dh);
-                dh = rp_mfma<DT>(a1, b1, dh);
-                if constexpr (NORM) {
-                    dl = rp_mfma<DT>(l0, b0, dl);
-                    dl = rp_mfma<DT>(l1, b1, dl);
+                for (int d = 0; d < 4; d++) {
+                    const uint32_t w = r.wv[i][d];
+                    const uint4 xo = *(const uint4*)xp_lds[d][i * 64 + ln];
+                    uint4 xl = make_uint4(0u, 0u, 0u, 0u);
+                    if constexpr (NORM) xl = *(const uint4*)xl_lds[d][i * 64 + ln];
+                    rp_u32x2 b0, b1, a0, a1, l0, l1;
+                    b0.x = (w & 0x000F000Fu) | kor;
+                    b0.y = ((w >> 4) & 0x000F000Fu) | kor;
+                    b1.x = ((w >> 8) & 0x000F000Fu) | kor;
+                    b1.y = ((w >> 12) & 0x000F000Fu) | kor;
+                    a0.x = xo.x; a0.y = xo.y; a1.x = xo.z; a1.y = xo.w;
+                    l0.x = xl.x; l0.y = xl.y; l1.x = xl.z; l1.y = xl.w;
+                    dh = rp_mfma<DT>(a0, b0, dh);
+                    dh = rp_mfma<DT>(a1, b1, dh);
+                    if constexpr (NORM) {
+                        dl = rp_mfma<DT>(l0, b0, dl);
+                        dl = rp_mfma<DT>(l1, b1, dl);
+                    }
+                }
+                const uint32_t sch = 16u * ((((uint32_t)(i * 64 + (int)lane) * CPC) >> LOG2G) & 1u);   // the half of the dword the chunk's group is in
+                t = fmaf(rp_up<DT>((r.sc[i] >> sch) & 0xFFFFu), fmaf(rp_diag(dl, j0, j1), REM, rp_diag(dh, j0, j1)), t);
+            } else {
+                rp_f32x4 dq[NH];
+#pragma unroll
+                for (int h = 0; h < NH; h++) dq[h] = rp_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+                    const uint32_t w = r.wv[i][d];
+                    constexpr int HSH = NH == 2 ? 1 : 2;   // dword d adds to half d >> HSH
+                    const uint4 xo0 = *(const uint4*)xp_lds[2 * d][i * 64 + ln], xo1 = *(const uint4*)xp_lds[2 * d + 1][i * 64 + ln];
+                    const uint32_t xa[8] = {xo0.x, xo0.y, xo0.z, xo0.w, xo1.x, xo1.y, xo1.z, xo1.w};
+                    uint32_t pq[8];
+#pragma unroll
+                    for (int pi = 0; pi < 8; pi++) {
+                        constexpr uint32_t M2 = 0x00030003u;
+                        const int p = rp_crumb_class<DT>(pi), sh = rp_crumb_shift<DT>(pi);
+                        pq[pi] = ((w >> sh) & (M2 << (2 * p))) | kor2[p];
+                    }
+#pragma unroll
+                    for (int m = 0; m < 4; m++) {
+                        rp_u32x2 av, bvv;
+                        av.x = xa[2 * m]; av.y = xa[2 * m + 1];
+                        bvv.x = pq[2 * m]; bvv.y = pq[2 * m + 1];
+                        dq[d >> HSH] = rp_mfma<DT>(av, bvv, dq[d >> HSH]);
+                    }
+                }
+                if constexpr (NH == 2) {   // the dword holds the chunk's two groups: half h is group h
+                    t = fmaf(rp_up<DT>(r.sc[i] & 0xFFFFu), rp_diag(dq[0], j0, j1), t);
+                    t = fmaf(rp_up<DT>(r.sc[i] >> 16), rp_diag(dq[NH - 1], j0, j1), t);
+                } else {
+                    const uint32_t sch = 16u * ((((uint32_t)(i * 64 + (int)lane) * CPC) >> LOG2G) & 1u);
+                    t = fmaf(rp_up<DT>((r.sc[i] >> sch) & 0xFFFFu), rp_diag(dq[0], j0, j1), t);
                 }
             }
-            const uint32_t sch = 16u * ((((uint32_t)(i * 64 + (int)lane) * CPC) >> LOG2G) & 1u);   // the half of the dword the chunk's group is in
-            t = fmaf(rp_up<DT>((r.sc[i] >> sch) & 0xFFFFu), fmaf(rp_diag(dl, j0, j1), REM, rp_diag(dh, j0, j1)), t);
         }
         t += __shfl_xor(t, 32, 64);
         t += dpp_f32<0xB1>(t);
@@ -281,6 +364,10 @@ template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * 
 template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_walk_kernel(QmvRowsNArgs a) {
     qmv_rows_walk_body<DT, CH, LOG2G, NWV, false>(a);
 }
+// 2-bit codes (rows of 8192: 128 chunks of 64 codes), made operands in place as in the one-row-per-wave kernel.
+template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_walk2_kernel(QmvRowsNArgs a) {
+    qmv_rows_walk_body<DT, CH, LOG2G, NWV, false, false, 2>(a);
+}
 // Two to four matrices against the one activation row in one launch (the fused projections of a decode step:
 // ffai_batched_qkv_qgemv_fast, crates/metaltile-std/src/ffai/batched_qkv_qgemv.rs:157; ffai_batched_4_qgemv_fast,
 // crates/metaltile-std/src/ffai/batched_4_qgemv.rs:60): the launch's rows are the matrices' rows one after the other.
@@ -299,6 +386,10 @@ bool qmv_rows_norm_takes(const QmvParams& p, const void* norm_w) {
 template <int DT, int LOG2G> static const void* rows_walk_batched_fn(uint32_t K, bool sixteen) {
     if (sixteen) return K == 4096 ? (const void*)qmv_rows_walk_batched_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_walk_batched_kernel<DT, 4, LOG2G, 16>;
     return K == 4096 ? (const void*)qmv_rows_walk_batched_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_walk_batched_kernel<DT, 4, LOG2G, 8>;
+}
+
+template <int DT, int LOG2G> static const void* rows_walk2_fn(bool sixteen) {   // 2-bit codes, rows of 8192
+    return sixteen ? (const void*)qmv_rows_walk2_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_walk2_kernel<DT, 2, LOG2G, 8>;
 }
 
 template <int DT, int LOG2G, bool NORM> static const void* rows_walk_fn(uint32_t K, bool sixteen) {
@@ -337,6 +428,11 @@ template <bool NORM> static int launch_rows_walk(const QmvParams& p, const void*
     const uint32_t nwv = sixteen ? 16u : 8u, cap = sixteen ? 256u : 512u;
     const void* fn = p.dtype == DT_BF16 ? (G == 32 ? rows_walk_fn<DT_BF16, 5, NORM>(p.K, sixteen) : G == 64 ? rows_walk_fn<DT_BF16, 6, NORM>(p.K, sixteen) : rows_walk_fn<DT_BF16, 7, NORM>(p.K, sixteen))
                                         : (G == 32 ? rows_walk_fn<DT_F16, 5, NORM>(p.K, sixteen) : G == 64 ? rows_walk_fn<DT_F16, 6, NORM>(p.K, sixteen) : rows_walk_fn<DT_F16, 7, NORM>(p.K, sixteen));
+    if (p.bits == 2) {
+        if (NORM || batch || p.K != 8192) return fail(ERR_UNSUPPORTED, "qmv walking rows kernel: 2-bit codes on one matrix with rows of 8192 codes");
+        fn = p.dtype == DT_BF16 ? (G == 32 ? rows_walk2_fn<DT_BF16, 5>(sixteen) : G == 64 ? rows_walk2_fn<DT_BF16, 6>(sixteen) : rows_walk2_fn<DT_BF16, 7>(sixteen))
+                                : (G == 32 ? rows_walk2_fn<DT_F16, 5>(sixteen) : G == 64 ? rows_walk2_fn<DT_F16, 6>(sixteen) : rows_walk2_fn<DT_F16, 7>(sixteen));
+    }
     if (batch) {
         if constexpr (NORM) return fail(ERR_UNSUPPORTED, "norm + qmv rows kernel: one matrix");
         fn = p.dtype == DT_BF16 ? (G == 32 ? rows_walk_batched_fn<DT_BF16, 5>(p.K, sixteen) : G == 64 ? rows_walk_batched_fn<DT_BF16, 6>(p.K, sixteen) : rows_walk_batched_fn<DT_BF16, 7>(p.K, sixteen))
@@ -355,7 +451,13 @@ int launch_qmv_rows_norm(const QmvParams& p, const void* norm_w, const float* ep
 
 // The plain GEMV on the same walk: one activation row against one matrix.
 bool qmv_rows_walk_takes(const QmvParams& p) {
-    return p.gather == GATHER_NONE && p.M == 1 && qmv_rows_norm_takes(p, p.x);   // (the alignment of x stands in for that of the norm weights)
+    if (p.gather != GATHER_NONE || p.M != 1) return false;
+    if (p.bits == 2) {   // rows of 8192 2-bit codes: the 4-bit instance's conditions on a matrix of that width
+        QmvParams q = p;
+        q.bits = 4;
+        return p.K == 8192 && qmv_rows_norm_takes(q, p.x);
+    }
+    return qmv_rows_norm_takes(p, p.x);   // (the alignment of x stands in for that of the norm weights)
 }
 
 // Where it is ahead of the kernels that work a row block per wave and end (bf16 g64, us, those -> this, same run):
@@ -370,13 +472,16 @@ bool qmv_rows_walk_takes(const QmvParams& p) {
 // in groups of 128 (14336 x 8192: 12.59 / 12.80).
 bool qmv_rows_walk_preferred(const QmvParams& p) {
     if (!qmv_rows_walk_takes(p)) return false;
+    // 2-bit codes (rows of 8192), the one-row-per-wave kernel -> this: 8192 rows f16 g32 / g64 / g128 6.76 -> 6.30, 6.27 -> 5.91,
+    // 6.09 -> 5.61; bf16 g64 14336 / 28672 rows 9.51 -> 8.75, 16.2 -> 14.4; 2048 / 4096 rows 3.62 -> 3.84, 4.01 -> 4.30
+    if (p.bits == 2) return p.N >= 8192;
     if (p.K == 4096) return p.N >= 1536 && (p.N <= 40960 || p.N >= 81920);
     return p.N >= 10240 && p.group_size != 128;
 }
 
 // The batch on one walk: every matrix as the single one would have to be, the rows counted together.
 static bool rows_walk_batch_as_one(const QmvParams& p0, const QmvBatch& b, QmvParams& p) {
-    if (b.n < 2 || b.n > 4) return false;
+    if (b.n < 2 || b.n > 4 || p0.bits != 4) return false;
     p = p0;
     p.gather = GATHER_NONE;
     p.M = 1;

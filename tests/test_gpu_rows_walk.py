@@ -50,6 +50,41 @@ def test_rows_walk_kernel_against_the_oracle(oracle, dt_name, G, K, N):
         b.free()
 
 
+@pytest.mark.parametrize("dt_name", ["BF16", "F16"])
+@pytest.mark.parametrize("G", [32, 64, 128])
+@pytest.mark.parametrize("N", [1, 50, 4096, 8192, 12289])
+def test_rows_walk_kernel_two_bit_codes(oracle, dt_name, G, N):
+    """2-bit codes on rows of 8192 (made operands in place, with an offset that depends on the crumb's position; groups
+    of 32 span half a chunk, so a chunk's halves are scaled apart): forced with qmv.kernel = 4, full-range codes, behind
+    a cache flush, guard elements, against the f64 oracle."""
+    import metaltile_amd as m
+    from metaltile_amd import DType, GpuBuffer, ops, _lib
+    from metaltile_amd.synth import make_case
+    from tests.parity import rel_err
+    dt, K = getattr(DType, dt_name), 8192
+    print(f"[case] rows walk 2-bit {dt_name} g{G} N{N}", flush=True)
+    c = make_case(5300 + N + G, dt, 2, G, 1, N, K, bias_rule="midpoint")
+    bw, bs, bb, bx = (GpuBuffer.from_bytes(v) for v in (c.w.tobytes(), c.scales_bytes, c.biases_bytes, c.x_bytes))
+    out = GpuBuffer.from_bytes(np.full(N + 8, 0xABAB, np.uint16).tobytes())
+    lib = _lib.load()
+    assert lib.mtq_set_option(b"qmv.kernel", 4) == 0
+    try:
+        rc, launches, _, n = ops.plan("qmv", dt, 2, G, 1, N, K)
+        assert rc == 0 and n == 1 and "qmv_rows_walk2_kernel" in launches[0][0], launches
+        m.GpuRunner(0).flush_slc()
+        ops.qmv(dt, 2, G, bw, bs, bb, bx, out, 1, N, K)
+    finally:
+        lib.mtq_set_option(b"qmv.kernel", 0)
+    raw = out.read_array(np.uint16)
+    assert np.all(raw[N:] == 0xABAB)
+    got = m.unpack_f32(raw[:N].tobytes(), dt)
+    assert np.isfinite(got).all()
+    exp = oracle.qmm_f64(c.w, c.scales_f, c.biases_f, c.x_f, 1, N, K, 2, G)
+    assert rel_err(got, exp) <= 1e-2
+    for b in (bw, bs, bb, bx, out):
+        b.free()
+
+
 def test_rows_walk_kernel_is_the_automatic_route_of_the_headline_shapes(oracle):
     """With no option set, the gate / up shape of the headline and a vocabulary projection take this kernel, and the
     result equals the forced wave-per-four-rows kernel's to the rounding of the output type."""

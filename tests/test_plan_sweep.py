@@ -138,9 +138,11 @@ def test_benchmark_configurations_are_routed_as_documented():
         assert "qmv_rows_walk_kernel" not in kernels("qmv", *args)[0][0]     # nor the walk: one row, 4-bit, 4096 / 8192 codes, groups of 32 / 64 / 128
     ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 4096, 14336)
     assert "qmv_rows_long_kernel<2, 4, 7, 6>" in ks[0] and ls[0][1][0] == 512 and ls[0][2][0] == 512   # workgroups of eight rows
-    for bits, G, name in ((2, 32, "<1, 2, 2, 5>"), (2, 128, "<1, 2, 2, 7>"), (4, 64, "<1, 4, 4, 6>")):   # the one-row cells of the width / group sweep
+    for bits, G, name in ((2, 32, "qmv_rows_walk2_kernel<1, 2, 5, 8>"), (2, 128, "qmv_rows_walk2_kernel<1, 2, 7, 8>"), (4, 64, "qmv_rows_long_kernel<1, 4, 4, 6>")):   # the one-row cells of the width / group sweep
         ks, ls = kernels("qmv", DType.F16, bits, G, 1, 8192, 8192)
-        assert "qmv_rows_long_kernel" + name in ks[0] and ls[0][1][0] == 512, ks
+        assert name in ks[0] and ls[0][1][0] == 512, ks
+    ks, ls = kernels("qmv", DType.F16, 2, 64, 1, 4096, 8192)      # fewer rows of 2-bit codes: the one-row-per-wave kernel
+    assert "qmv_rows_long_kernel<1, 2, 2, 6>" in ks[0], ks
     ks, _ = kernels("qmv", DType.F16, 8, 64, 1, 8192, 8192)
     assert "qmv_rows" not in ks[0]
     # the four-row cells of the sweep: one wave per four weight rows where that is ahead (2-bit codes, 4-bit in groups of 32,
