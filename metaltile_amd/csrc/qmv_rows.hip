@@ -39,40 +39,6 @@ struct QmvRowsArgs {
     uint32_t E, T;
 };
 
-// Routed rows (GM = GATHER_CSR / GATHER_INDICES; a decode step of a few tokens through a mixture-of-experts layer, fewer
-// rows than experts): grid row blockIdx.y serves the blockIdx.y-th expert that has a row and runs the kernel's body once
-// per row of that expert -- one row each when a token's experts are distinct, as top-k routing makes them. The same
-// rules as the streaming kernel's routed form (at most 64 experts and 64 rows: the routing is read by one wave-wide load).
-struct RowsRoute {
-    uint32_t expert = 0, n_pass = 1, lo = 0, n1 = 1, lo2 = 0;
-    unsigned long long mask = 0;
-};
-template <int GM> __device__ __forceinline__ bool rows_route(const uint32_t* route, uint32_t E, uint32_t T, uint32_t lane, RowsRoute& r) {
-    if constexpr (GM == GATHER_CSR) {
-        r.n_pass = csr_route64(route, E, T, blockIdx.y, true, lane, r.expert, r.lo, r.n1, r.lo2);
-        if (r.n_pass == 0) return false;
-        r.expert = __builtin_amdgcn_readfirstlane(r.expert);
-    }
-    if constexpr (GM == GATHER_SINGLE) r.expert = min(route[0], E - 1u);   // one row on the expert named on the device; an id past the last expert names the last
-    if constexpr (GM == GATHER_INDICES) {
-        r.expert = __builtin_amdgcn_readfirstlane(ids_slot_expert(route, E, T, blockIdx.y, lane));
-        if (r.expert == 0xFFFFFFFFu) return false;
-        r.mask = __ballot(lane < T && route[lane] == r.expert);
-        r.n_pass = (uint32_t)__popcll(r.mask);
-    }
-    return true;
-}
-// the activation (and output) row of a pass
-template <int GM> __device__ __forceinline__ uint32_t rows_route_row(const RowsRoute& r, uint32_t pass) {
-    if constexpr (GM == GATHER_CSR) return pass < r.n1 ? r.lo + pass : r.lo2 + (pass - r.n1);
-    if constexpr (GM == GATHER_INDICES) {
-        unsigned long long m = r.mask;
-        for (uint32_t i = 0; i < pass; i++) m &= m - 1ull;
-        return (uint32_t)__ffsll((long long)m) - 1u;
-    }
-    return 0u;
-}
-
 template <bool TL> __device__ __forceinline__ void rp_stamp(uint64_t (&st)[MTQ_ROWS_PROBE_STAMPS], int i) {
     if constexpr (TL) {
         RP_KEEP_ORDER();

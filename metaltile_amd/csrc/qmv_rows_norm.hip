@@ -36,6 +36,10 @@ struct QmvRowsNArgs {
     const uint16_t* mb[4];
     uint16_t* mo[4];
     uint32_t first[5];
+    // Routed rows (the routed instances): expert_offsets[E + 1], indices[T] or the one expert id; w / s / b then hold E
+    // matrices of N rows, x and out T rows.
+    const uint32_t* route;
+    uint32_t E, T;
 };
 
 // One row's loads of one lane, as they come from memory: whatever has to be done to a loaded value (picking the 16-bit
@@ -47,9 +51,11 @@ template <int CH> struct RowsNormBuf {
     uint32_t sw[2], bw[2];   // the lane's groups of the bias term, two 16-bit elements per dword (one group per lane: the dword that holds it)
 };
 
-template <int DT, int CH, int LOG2G, int NWV, bool NORM, bool BATCH = false, int BITS = 4>
+template <int DT, int CH, int LOG2G, int NWV, bool NORM, bool BATCH = false, int BITS = 4, int GM = GATHER_NONE>
 __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     static_assert(BITS == 4 || (BITS == 2 && !NORM && !BATCH), "4-bit codes; 2-bit codes on the plain walk");
+    constexpr bool ROUTED = GM != GATHER_NONE;
+    static_assert(!ROUTED || (!NORM && !BATCH && BITS == 4), "routed rows: the plain walk on 4-bit codes");
     constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;   // 4-bit codes: one offset for every pair
     constexpr float REM = 1.0f / RemSplit<DT>::kRemScale;
     constexpr int CPC = 128 / BITS, Q = CPC / 8;   // codes per 16-byte chunk; 16-byte quarters of a chunk's activations in operand order
@@ -68,6 +74,13 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     const uint32_t gw = blockIdx.x * (uint32_t)NWV + wave, GW = gridDim.x * (uint32_t)NWV;   // (the same in every lane: row numbers stay in scalar registers)
     const uint32_t last = a.N - 1u;
     const uint32_t gl = min(lane, (uint32_t)(GPR / GPL - 1));
+    // Routed rows: grid row blockIdx.y serves the blockIdx.y-th expert that has a row, and the walk below runs once per
+    // row of that expert (a pass), on that expert's matrix.
+    RowsRoute rt;
+    if constexpr (ROUTED) {
+        if (!rows_route<GM>(a.route, a.E, a.T, lane, rt)) return;   // (the same for every wave of the workgroup: no barrier is left waiting)
+    }
+    const size_t eoff = ROUTED ? (size_t)rt.expert * a.N : (size_t)0;   // the expert's first row among the rows of all experts
     auto load_row = [&](uint32_t row, RowsNormBuf<CH>& r) {   // row <= last
         row = min(row, last);   // (it is; a scalar instruction keeps the loads inside the matrix whatever the caller does)
         const uint16_t *sp, *bp;
@@ -79,9 +92,9 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
             bp = a.mb[m] + (size_t)local * GPR;
             wrow = a.mw[m] + (size_t)local * C;
         } else {
-            sp = a.s + (size_t)row * GPR;
-            bp = a.b + (size_t)row * GPR;
-            wrow = a.w + (size_t)row * C;
+            sp = a.s + (eoff + row) * GPR;
+            bp = a.b + (eoff + row) * GPR;
+            wrow = a.w + (eoff + row) * C;
         }
 #pragma unroll
         for (int i = 0; i < CH; i++) r.sc[i] = ((const uint32_t*)sp)[((uint32_t)(i * 64 + (int)lane) * CPC) >> (LOG2G + 1)];   // (a chunk that spans two groups: both of them)
@@ -100,10 +113,14 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
 #pragma unroll
         for (int i = 0; i < CH; i++) r.wv[i] = __builtin_nontemporal_load(wbase + i * 64);
     };
+    for (uint32_t pass = 0; pass < rt.n_pass; pass++) {   // (one pass unless routed)
+    const uint32_t trow = rows_route_row<GM>(rt, pass);
+    const uint16_t* const xrow = a.x + (size_t)trow * K;
+    uint16_t* const orow = a.out + (size_t)trow * a.N;
     // ---- this thread's chunk of the activations and of the norm weights; the first row's loads ---------------------
     uint4 xraw[Q], nraw[Q];
     if (tid < (uint32_t)C) {
-        const uint4* xv = (const uint4*)(a.x + (size_t)tid * CPC);
+        const uint4* xv = (const uint4*)(xrow + (size_t)tid * CPC);
         const uint4* nv = (const uint4*)(a.norm_w + (size_t)tid * CPC);
 #pragma unroll
         for (int v = 0; v < Q; v++) xraw[v] = xv[v];
@@ -214,7 +231,7 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
         }
     }
     __syncthreads();
-    if (gw > last) return;
+    if (gw <= last) {
     // the activation sums of this lane's GPL groups of the bias term (the same for every row)
     float X[GPL], XM[GPL];   // (XM: the sum weighted with the codes' offsets; 4-bit codes have the one offset)
 #pragma unroll
@@ -313,7 +330,7 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
                 const uint32_t m = (uint32_t)(row >= a.first[1]) + (uint32_t)(row >= a.first[2]) + (uint32_t)(row >= a.first[3]);
                 a.mo[m][row - a.first[m]] = f32_to_elem_bits<DT>(t);
             } else {
-                a.out[row] = f32_to_elem_bits<DT>(t);
+                orow[row] = f32_to_elem_bits<DT>(t);
             }
         }
     };
@@ -327,33 +344,36 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     // (The norm's instances for rows of 8192 codes have no register to spare for a second way of ending: they run
     // whole turns, the last of which loads the matrix's last row once more for nobody, and end on the odd row.)
     constexpr bool WHOLE_TURNS = NORM && CH == 4;
-    if constexpr (WHOLE_TURNS) {
-        if (cnt == 1u) {
-            work_row(row, bufA);
-            return;
-        }
-    }
-    for (uint32_t it = WHOLE_TURNS ? cnt >> 1 : (cnt - 1u) >> 1; it != 0u; it--) {   // two rows a turn (while a third is there to be loaded)
-        load_row(row + GW, bufB);
-        RP_KEEP_ORDER();
-        work_row(row, bufA);
-        load_row(row + 2u * GW, bufA);
-        RP_KEEP_ORDER();
-        work_row(row + GW, bufB);
-        row += 2u * GW;
-    }
-    if constexpr (WHOLE_TURNS) {
-        if (cnt & 1u) work_row(row, bufA);
-    } else if (cnt & 1u) {   // one row is left, or two; the first of them is loaded
-        RP_KEEP_ORDER();     // (both ways start behind a fence of their own, so that the work on the first row is not lifted above the branch)
+    if (WHOLE_TURNS && cnt == 1u) {
         work_row(row, bufA);
     } else {
-        load_row(row + GW, bufB);
-        RP_KEEP_ORDER();
-        work_row(row, bufA);
-        RP_KEEP_ORDER();
-        work_row(row + GW, bufB);
+        for (uint32_t it = WHOLE_TURNS ? cnt >> 1 : (cnt - 1u) >> 1; it != 0u; it--) {   // two rows a turn (while a third is there to be loaded)
+            load_row(row + GW, bufB);
+            RP_KEEP_ORDER();
+            work_row(row, bufA);
+            load_row(row + 2u * GW, bufA);
+            RP_KEEP_ORDER();
+            work_row(row + GW, bufB);
+            row += 2u * GW;
+        }
+        if constexpr (WHOLE_TURNS) {
+            if (cnt & 1u) work_row(row, bufA);
+        } else if (cnt & 1u) {   // one row is left, or two; the first of them is loaded
+            RP_KEEP_ORDER();     // (both ways start behind a fence of their own, so that the work on the first row is not lifted above the branch)
+            work_row(row, bufA);
+        } else {
+            load_row(row + GW, bufB);
+            RP_KEEP_ORDER();
+            work_row(row, bufA);
+            RP_KEEP_ORDER();
+            work_row(row + GW, bufB);
+        }
     }
+    }   // this wave has rows
+    if constexpr (ROUTED) {
+        if (pass + 1u < rt.n_pass) __syncthreads();   // the next pass overwrites the activations in LDS
+    }
+    }   // pass
 }
 
 // (four waves per SIMD: two workgroups of eight waves, or one of sixteen, per compute unit)
@@ -367,6 +387,13 @@ template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * 
 // 2-bit codes (rows of 8192: 128 chunks of 64 codes), made operands in place as in the one-row-per-wave kernel.
 template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_walk2_kernel(QmvRowsNArgs a) {
     qmv_rows_walk_body<DT, CH, LOG2G, NWV, false, false, 2>(a);
+}
+// Routed rows (a decode step of a few tokens through a mixture-of-experts layer: fewer rows than experts, or the one
+// row of dequant_gemv_int4_expert_indexed, crates/metaltile-std/src/ffai/dequant_gemv_expert_indexed.rs:58-105; the
+// routing rules of mt_moe_gather_qmm_int4, crates/metaltile-std/src/ffai/moe.rs:376-385): grid row y walks the rows of the
+// y-th expert that has a row, once per row of x routed to it.
+template <int DT, int CH, int LOG2G, int GM> __global__ __launch_bounds__(512, 4) void qmv_rows_walk_routed_kernel(QmvRowsNArgs a) {
+    qmv_rows_walk_body<DT, CH, LOG2G, 8, false, false, 4, GM>(a);
 }
 // Two to four matrices against the one activation row in one launch (the fused projections of a decode step:
 // ffai_batched_qkv_qgemv_fast, crates/metaltile-std/src/ffai/batched_qkv_qgemv.rs:157; ffai_batched_4_qgemv_fast,
@@ -392,6 +419,10 @@ template <int DT, int LOG2G> static const void* rows_walk2_fn(bool sixteen) {   
     return sixteen ? (const void*)qmv_rows_walk2_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_walk2_kernel<DT, 2, LOG2G, 8>;
 }
 
+template <int DT, int GM> static const void* rows_walk_routed_fn(uint32_t K) {   // groups of 64
+    return K == 4096 ? (const void*)qmv_rows_walk_routed_kernel<DT, 2, 6, GM> : (const void*)qmv_rows_walk_routed_kernel<DT, 4, 6, GM>;
+}
+
 template <int DT, int LOG2G, bool NORM> static const void* rows_walk_fn(uint32_t K, bool sixteen) {
     if constexpr (NORM) {
         if (sixteen) return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 16>;
@@ -407,6 +438,7 @@ template <bool NORM> static int launch_rows_walk(const QmvParams& p, const void*
     QmvRowsNArgs a{};
     a.w = (const rp_u32x4*)p.w; a.s = (const uint16_t*)p.scales; a.b = (const uint16_t*)p.biases; a.x = (const uint16_t*)p.x; a.out = (uint16_t*)p.out;
     a.N = p.N; a.norm_w = (const uint16_t*)norm_w; a.norm_eps = eps;
+    a.route = p.route; a.E = p.E; a.T = p.T;
     if (batch) {
         uint32_t at = 0;
         for (int j = 0; j < 4; j++) {
@@ -438,6 +470,18 @@ template <bool NORM> static int launch_rows_walk(const QmvParams& p, const void*
         fn = p.dtype == DT_BF16 ? (G == 32 ? rows_walk_batched_fn<DT_BF16, 5>(p.K, sixteen) : G == 64 ? rows_walk_batched_fn<DT_BF16, 6>(p.K, sixteen) : rows_walk_batched_fn<DT_BF16, 7>(p.K, sixteen))
                                 : (G == 32 ? rows_walk_batched_fn<DT_F16, 5>(p.K, sixteen) : G == 64 ? rows_walk_batched_fn<DT_F16, 6>(p.K, sixteen) : rows_walk_batched_fn<DT_F16, 7>(p.K, sixteen));
     }
+    if (p.gather != GATHER_NONE) {
+        // a grid row per expert that can have a row, workgroups of eight waves, about two of them per compute unit over all grid rows
+        if (NORM || batch || p.bits != 4 || G != 64) return fail(ERR_UNSUPPORTED, "qmv walking rows kernel: routed rows on the plain 4-bit walk, groups of 64");
+        const uint32_t slots = p.gather == GATHER_SINGLE ? 1u : (p.T < p.E ? p.T : p.E);
+        fn = p.gather == GATHER_CSR       ? (p.dtype == DT_BF16 ? rows_walk_routed_fn<DT_BF16, GATHER_CSR>(p.K) : rows_walk_routed_fn<DT_F16, GATHER_CSR>(p.K))
+             : p.gather == GATHER_INDICES ? (p.dtype == DT_BF16 ? rows_walk_routed_fn<DT_BF16, GATHER_INDICES>(p.K) : rows_walk_routed_fn<DT_F16, GATHER_INDICES>(p.K))
+                                          : (p.dtype == DT_BF16 ? rows_walk_routed_fn<DT_BF16, GATHER_SINGLE>(p.K) : rows_walk_routed_fn<DT_F16, GATHER_SINGLE>(p.K));
+        const uint32_t per_slot = 512u / slots > 0u ? 512u / slots : 1u, all = (p.N + 7u) / 8u;
+        hipError_t e = launch_kernel(fn, dim3(all < per_slot ? all : per_slot, slots), dim3(512), args, 0, lc);
+        if (e != hipSuccess) return hip_fail(e, "qmv walking rows kernel launch (routed)");
+        return ERR_OK;
+    }
     const uint32_t wgs = (p.N + nwv - 1u) / nwv;
     hipError_t e = launch_kernel(fn, dim3(wgs < cap ? wgs : cap), dim3(64u * nwv), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, NORM ? "norm + qmv rows kernel launch" : "qmv walking rows kernel launch");
@@ -451,7 +495,17 @@ int launch_qmv_rows_norm(const QmvParams& p, const void* norm_w, const float* ep
 
 // The plain GEMV on the same walk: one activation row against one matrix.
 bool qmv_rows_walk_takes(const QmvParams& p) {
-    if (p.gather != GATHER_NONE || p.M != 1) return false;
+    if (p.gather != GATHER_NONE) {
+        // routed rows: at most 64 experts and 64 rows (the routing is read by one wave-wide load; the single-index form
+        // reads one id and takes any number of experts), 4-bit codes in groups of 64, every expert's block of scales as
+        // aligned as the first
+        if (p.gather != GATHER_CSR && p.gather != GATHER_INDICES && p.gather != GATHER_SINGLE) return false;
+        if (!p.route || p.E == 0 || p.bits != 4 || p.group_size != 64) return false;
+        if (p.gather != GATHER_SINGLE && (p.E > 64 || p.T == 0 || p.T > 64)) return false;
+        if (((size_t)p.N * (p.K / 64u) * 2u) % 8u) return false;
+        return qmv_rows_norm_takes(p, p.x);
+    }
+    if (p.M != 1) return false;
     if (p.bits == 2) {   // rows of 8192 2-bit codes: the 4-bit instance's conditions on a matrix of that width
         QmvParams q = p;
         q.bits = 4;
@@ -472,6 +526,13 @@ bool qmv_rows_walk_takes(const QmvParams& p) {
 // in groups of 128 (14336 x 8192: 12.59 / 12.80).
 bool qmv_rows_walk_preferred(const QmvParams& p) {
     if (!qmv_rows_walk_takes(p)) return false;
+    // Routed rows, fewer than the experts (8 experts, bf16, us, the routed wave-per-row kernels or, from three rows of 4096
+    // codes, the matrix-core GEMV -> this): experts of 14336 x 4096, 1 / 2 / 3 / 4 rows on distinct experts 8.6 -> 7.4, 15.3 ->
+    // 12.3, 22.1 -> 18.5, 27.9 -> 23.4; of 4096 x 8192 6.3 - 6.9 -> 5.9, 10.6 -> 8.2, 15.4 -> 10.9, 20.6 -> 13.4; of 14336 x 8192 18.0 ->
+    // 12.5, 31.5 -> 22.2, 48.0 -> 32.8, 63.4 -> 41.4. Two rows on one expert are two passes over its matrix: 13.4 -> 14.2 on
+    // 14336 x 4096 (the older kernel's second pass is shorter), 9.8 -> 8.6 and 29.9 -> 22.2 on the others.
+    if (p.gather == GATHER_SINGLE) return p.N >= 1536;
+    if (p.gather != GATHER_NONE) return p.N >= 1024 && p.T < p.E && p.T <= 4;
     // 2-bit codes (rows of 8192), the one-row-per-wave kernel -> this: 8192 rows f16 g32 / g64 / g128 6.76 -> 6.30, 6.27 -> 5.91,
     // 6.09 -> 5.61; bf16 g64 14336 / 28672 rows 9.51 -> 8.75, 16.2 -> 14.4; 2048 / 4096 rows 3.62 -> 3.84, 4.01 -> 4.30
     if (p.bits == 2) return p.N >= 8192;

@@ -188,10 +188,22 @@ def wave_per_row_kernels():
     lib.mtq_set_option(b"qmv.kernel", 0)
 
 
+@pytest.fixture
+def forced_qmv_kernel(request):
+    lib = _lib.load()
+    assert lib.mtq_set_option(b"qmv.kernel", request.param) == 0
+    yield
+    lib.mtq_set_option(b"qmv.kernel", 0)
+
+
 @pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
-@pytest.mark.parametrize("N,K,kernel", [(20, 4096, "qmv_rows_routed_kernel"), (1028, 4096, "qmv_rows_routed_kernel"), (19, 14336, "qmv_rows_long_routed_kernel"),
-                                        (1030, 8192, "qmv_rows_long_routed_kernel")])
-def test_routed_rows_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, wave_per_row_kernels):
+@pytest.mark.parametrize("N,K,kernel,forced_qmv_kernel",
+                         [(20, 4096, "qmv_rows_routed_kernel", 3), (1028, 4096, "qmv_rows_routed_kernel", 3), (19, 14336, "qmv_rows_long_routed_kernel", 3),
+                          (1030, 8192, "qmv_rows_long_routed_kernel", 3),
+                          # the kernel whose waves walk the rows (qmv.kernel = 4): one row per wave, and 5000 rows so that waves walk
+                          (20, 4096, "qmv_rows_walk_routed_kernel", 4), (5000, 4096, "qmv_rows_walk_routed_kernel", 4), (1030, 8192, "qmv_rows_walk_routed_kernel", 4)],
+                         indirect=["forced_qmv_kernel"])
+def test_routed_rows_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, forced_qmv_kernel):
     """The wave-per-row GEMV kernels with a grid row per expert that has a row (their automatic range is up to four rows
     on fewer rows than experts from 1024 weight rows; forced here below that too): one row, two experts, the same expert
     twice (a second pass over its matrix), seven rows, both routing views, CSR offsets that end short or step back, ids
@@ -250,8 +262,10 @@ def test_routed_rows_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, wave_
 
 
 @pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
-@pytest.mark.parametrize("N,K,kernel", [(1028, 4096, "qmv_rows_routed_kernel"), (40, 14336, "qmv_rows_long_routed_kernel"), (1030, 8192, "qmv_rows_long_routed_kernel")])
-def test_single_index_expert_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, wave_per_row_kernels):
+@pytest.mark.parametrize("N,K,kernel,forced_qmv_kernel",
+                         [(1028, 4096, "qmv_rows_routed_kernel", 3), (40, 14336, "qmv_rows_long_routed_kernel", 3), (1030, 8192, "qmv_rows_long_routed_kernel", 3),
+                          (9000, 4096, "qmv_rows_walk_routed_kernel", 4), (40, 8192, "qmv_rows_walk_routed_kernel", 4)], indirect=["forced_qmv_kernel"])
+def test_single_index_expert_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, forced_qmv_kernel):
     """One row against the expert whose index is read on the device (the reference's expert-indexed GEMV,
     crates/metaltile-std/src/ffai/dequant_gemv_expert_indexed.rs): the first, a middle and the last expert, and an index
     past the last expert, which names the last one as in the other kernels of this ABI."""

@@ -182,11 +182,17 @@ def test_benchmark_configurations_are_routed_as_documented():
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 16)           # 2 rows per expert: 8-row passes
     assert "qmv_mfma_kernel<2, 4," in ks[0]
     for view in ("gather_csr", "gather_indices"):      # fewer rows than experts: a grid row per row, not per expert
-        for T, E in ((1, 8), (2, 8), (7, 8), (8, 128), (32, 128)):
+        for T, E in ((1, 8), (2, 8), (4, 8), (7, 8), (8, 128), (32, 128)):
             ks, ls = kernels(view, DType.BF16, 4, 64, 1, 14336, 4096, E, T)
-            # one or two rows on at most 64 experts of 14336 x 4096: the routed wave-per-four-rows kernel
-            kernel = "qmv_rows_routed_kernel<2, " if T <= 2 and E <= 64 else "qmv_mfma_kernel<2, 4,"
+            # up to four rows on at most 64 experts of 14336 x 4096: the routed walk, about 512 workgroups over the grid rows
+            kernel = "qmv_rows_walk_routed_kernel<2, 2, 6, " if T <= 4 and E <= 64 else "qmv_mfma_kernel<2, 4,"
             assert kernel in ks[0] and ls[0][1][1] == T, (view, T, E, ls)
+            if T <= 4 and E <= 64:
+                assert ls[0][1][0] == 512 // T and ls[0][2][0] == 512, ls
+        ks, ls = kernels("gather_single", DType.BF16, 4, 64, 1, 14336, 4096, 8, 1)
+        assert "qmv_rows_walk_routed_kernel<2, 2, 6, 3>" in ks[0] and ls[0][1][:2] == (512, 1)
+        ks, ls = kernels(view, DType.BF16, 4, 64, 1, 4096, 14336, 8, 2)     # rows of 14336 codes: the routed one-row-per-wave kernel
+        assert "qmv_rows_long_routed_kernel<2, 4, 7, 6, " in ks[0] and ls[0][1][1] == 2, ls
         ks, ls = kernels(view, DType.BF16, 4, 64, 1, 2048, 768, 128, 33)   # (more than 32 rows: a grid row per expert)
         assert ls[0][1][1] == 128
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 4096, 4096, 8, 2048)
