@@ -55,14 +55,26 @@ template <int DT> __host__ __device__ constexpr uint32_t rp_crumb_kor(int p) {
 // per row of that expert -- one row each when a token's experts are distinct, as top-k routing makes them. The same
 // rules as the streaming kernel's routed form (at most 64 experts and 64 rows: the routing is read by one wave-wide load).
 struct RowsRoute {
-    uint32_t expert = 0, n_pass = 1, lo = 0, n1 = 1, lo2 = 0;
-    unsigned long long mask = 0;
+    uint32_t expert = 0, n_pass = 1;
+    unsigned long long mask = 1;   // the rows of x routed to the expert, one bit per row
 };
 template <int GM> __device__ __forceinline__ bool rows_route(const uint32_t* route, uint32_t E, uint32_t T, uint32_t lane, RowsRoute& r) {
     if constexpr (GM == GATHER_CSR) {
-        r.n_pass = csr_route64(route, E, T, blockIdx.y, true, lane, r.expert, r.lo, r.n1, r.lo2);
-        if (r.n_pass == 0) return false;
+        uint32_t lo, n1, lo2;
+        if (csr_route64(route, E, T, blockIdx.y, true, lane, r.expert, lo, n1, lo2) == 0) return false;
+        // (the same in every lane; said so, the pass loop and everything in it stay uniform control flow on scalar registers)
         r.expert = __builtin_amdgcn_readfirstlane(r.expert);
+        lo = __builtin_amdgcn_readfirstlane(lo);
+        n1 = __builtin_amdgcn_readfirstlane(n1);
+        lo2 = __builtin_amdgcn_readfirstlane(lo2);
+        // the expert's rows lo .. lo + n1 - 1 and, for expert 0, the rows past the last offset lo2 .. T - 1 (T <= 64), as a mask
+        // like the one the per-row ids give, so that both views share the code behind this point
+        const unsigned long long all = T >= 64u ? ~0ull : (1ull << T) - 1ull;
+        unsigned long long m = n1 ? ((n1 >= 64u ? ~0ull : (1ull << n1) - 1ull) << lo) : 0ull;
+        if (r.expert == 0u && lo2 < T) m |= (~0ull << lo2);
+        r.mask = m & all;
+        r.n_pass = (uint32_t)__popcll(r.mask);
+        if (r.n_pass == 0) return false;
     }
     if constexpr (GM == GATHER_SINGLE) r.expert = min(route[0], E - 1u);   // one row on the expert named on the device; an id past the last expert names the last
     if constexpr (GM == GATHER_INDICES) {
@@ -75,8 +87,7 @@ template <int GM> __device__ __forceinline__ bool rows_route(const uint32_t* rou
 }
 // the activation (and output) row of a pass
 template <int GM> __device__ __forceinline__ uint32_t rows_route_row(const RowsRoute& r, uint32_t pass) {
-    if constexpr (GM == GATHER_CSR) return pass < r.n1 ? r.lo + pass : r.lo2 + (pass - r.n1);
-    if constexpr (GM == GATHER_INDICES) {
+    if constexpr (GM == GATHER_CSR || GM == GATHER_INDICES) {
         unsigned long long m = r.mask;
         for (uint32_t i = 0; i < pass; i++) m &= m - 1ull;
         return (uint32_t)__ffsll((long long)m) - 1u;

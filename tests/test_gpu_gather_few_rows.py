@@ -181,14 +181,6 @@ def test_one_routed_row_on_rows_the_streaming_kernel_cannot_tile(oracle, dt, K):
 
 
 @pytest.fixture
-def wave_per_row_kernels():
-    lib = _lib.load()
-    assert lib.mtq_set_option(b"qmv.kernel", 3) == 0
-    yield
-    lib.mtq_set_option(b"qmv.kernel", 0)
-
-
-@pytest.fixture
 def forced_qmv_kernel(request):
     lib = _lib.load()
     assert lib.mtq_set_option(b"qmv.kernel", request.param) == 0
