@@ -445,14 +445,14 @@ static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const
     // 4-bit f16 / bf16: the norm applied as the matrix-core GEMV stages its row (two staged rows share one set of 4;
     // no per-workgroup renormalisation beyond the sum of squares). us, streaming kernel -> this: 14336 x 4096 12.6 ->
     // 10.6, 6144 x 4096 8.1 -> 7.3; it loses on short matrices and long rows (4096 x 4096 6.2 -> 6.4, 4096 x 14336 13.7 -> 14.1).
-    // Rows of 4096 / 8192 4-bit codes: the norm applied as the one-row-per-wave kernel puts the activations into LDS
-    // (qmv_rows_norm.hip). bf16, us, the forms below -> this: 4096 x 4096 6.8 -> 4.5, 6144 x 4096 7.3 -> 6.4, 14336 x 4096 10.7
-    // -> 10.0, 28672 x 4096 17.2 -> 16.6, 2048 x 8192 7.1 -> 4.7, 4096 x 8192 8.7 -> 7.2, 6144 x 8192 11.0 -> 10.4. From 8192 rows
-    // of 8192 codes on it is level with the matrix-core form or behind, depending on the machine (8192 x 8192 11.8 -> 12.4,
-    // 28672 x 8192 28.3 -> 28.3 - 29.2), and so it is on the largest matrices of 4096-code rows (65536 x 4096 30.5 -> 31.6,
-    // 128256 x 4096 50.2 -> 51.8). qmv.kernel = 2 keeps the older forms, = 3 takes this one wherever the shape allows.
+    // Rows of 4096 / 8192 4-bit codes: the norm applied as the kernel whose waves walk the rows puts the activations into
+    // LDS (qmv_rows_norm.hip). bf16, us, the better of the forms below -> this, same run: 1024 / 2048 / 4096 / 6144 / 8192 / 14336 /
+    // 28672 x 4096 4.65 -> 4.41, 4.75 -> 4.42, 6.52 -> 4.57, 7.37 -> 5.90, 7.57 -> 6.93, 10.61 -> 8.91, 16.76 -> 15.79; 2048 / 4096 /
+    // 6144 / 8192 / 14336 / 20480 / 28672 x 8192 6.81 -> 6.19, 8.73 -> 7.09, 11.01 -> 9.79, 11.73 -> 11.59, 17.17 -> 16.05, 22.28 -> 20.75,
+    // 27.51 -> 26.48. On the largest matrices the matrix-core form is level or ahead (65536 x 4096 29.0 / 29.4 - 32.2, 65536 x 8192
+    // 52.2 / 52.9 - 54.3). qmv.kernel = 2 keeps the older forms, = 3 takes this one wherever the shape allows.
     const bool rows_norm = options().qmv_kernel == 3 ||
-                           (options().qmv_kernel == 0 && (K == 4096 ? N >= 1024u && N <= 32768u : N >= 2048u && N < 8192u));
+                           (options().qmv_kernel == 0 && N >= (K == 4096 ? 1024u : 2048u) && N <= 32768u);
     if (options().qmv_norm_mfma != 2 && rows_norm && qmv_rows_norm_takes(p, norm_w)) {
         rc = launch_qmv_rows_norm(p, norm_w, eps, lc);
         if (rc != ERR_UNSUPPORTED) return rc;
