@@ -26,8 +26,8 @@ HIPFLAGS = [
     "-Wall", "-Wno-unused-function",
 ]
 # per-source additions: the wave-per-four-rows GEMV keeps its matrix-core results in ordinary vector registers (no accumulator-register copies)
-EXTRA_FLAGS = {"qmv_rows.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"], "qmv_rows_few.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"], "qmv_rows_norm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
-SOURCES = ["api.hip", "qmv.hip", "qmv_f32.hip", "qmv_f16.hip", "qmv_bf16.hip", "qmv_mfma.hip", "qmv_mfma_f16.hip", "qmv_mfma_bf16.hip", "qmv_mfma_f16_odd.hip", "qmv_mfma_bf16_odd.hip", "qmv_wide.hip", "qmv_wide_gather.hip", "generic.hip", "qmm.hip", "qmm_direct.hip", "qmm_direct_odd.hip", "qmm_dma.hip", "qmm_dma_b8.hip", "qmm_f32.hip", "affine.hip", "norm.hip", "moe.hip", "moe_down.hip", "qvm.hip", "qmv_rows.hip", "qmv_rows_few.hip", "qmv_rows_norm.hip"]
+EXTRA_FLAGS = {"qmv_rows.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"], "qmv_rows_few.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"], "qmv_rows_walk.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+SOURCES = ["api.hip", "qmv.hip", "qmv_f32.hip", "qmv_f16.hip", "qmv_bf16.hip", "qmv_mfma.hip", "qmv_mfma_f16.hip", "qmv_mfma_bf16.hip", "qmv_mfma_f16_odd.hip", "qmv_mfma_bf16_odd.hip", "qmv_wide.hip", "qmv_wide_gather.hip", "generic.hip", "qmm.hip", "qmm_direct.hip", "qmm_direct_odd.hip", "qmm_dma.hip", "qmm_dma_b8.hip", "qmm_f32.hip", "affine.hip", "norm.hip", "moe.hip", "moe_down.hip", "qvm.hip", "qmv_rows.hip", "qmv_rows_few.hip", "qmv_rows_walk.hip"]
 
 
 def _headers():

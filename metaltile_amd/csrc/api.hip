@@ -446,7 +446,7 @@ static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const
     // no per-workgroup renormalisation beyond the sum of squares). us, streaming kernel -> this: 14336 x 4096 12.6 ->
     // 10.6, 6144 x 4096 8.1 -> 7.3; it loses on short matrices and long rows (4096 x 4096 6.2 -> 6.4, 4096 x 14336 13.7 -> 14.1).
     // Rows of 4096 / 8192 4-bit codes: the norm applied as the kernel whose waves walk the rows puts the activations into
-    // LDS (qmv_rows_norm.hip). bf16, us, the better of the forms below -> this, same run: 1024 / 2048 / 4096 / 6144 / 8192 / 14336 /
+    // LDS (qmv_rows_walk.hip). bf16, us, the better of the forms below -> this, same run: 1024 / 2048 / 4096 / 6144 / 8192 / 14336 /
     // 28672 x 4096 4.65 -> 4.41, 4.75 -> 4.42, 6.52 -> 4.57, 7.37 -> 5.90, 7.57 -> 6.93, 10.61 -> 8.91, 16.76 -> 15.79; 2048 / 4096 /
     // 6144 / 8192 / 14336 / 20480 / 28672 x 8192 6.81 -> 6.19, 8.73 -> 7.09, 11.01 -> 9.79, 11.73 -> 11.59, 17.17 -> 16.05, 22.28 -> 20.75,
     // 27.51 -> 26.48. On the largest matrices the matrix-core form is level or ahead (65536 x 4096 29.0 / 29.4 - 32.2, 65536 x 8192

@@ -1,16 +1,21 @@
-// RMS norm fused into a quantized GEMV: out[n] = sum_k (s q + b)[n, k] x'[k], x'[k] = x[k] norm_w[k] / sqrt(mean(x^2) + eps)
-// (ffai_rms_norm_qgemv / _fast, crates/metaltile-std/src/ffai/rms_norm_qgemv.rs:53-125, 128-456), 4-bit codes, f16 / bf16,
-// rows of 4096 or 8192 codes (the hidden sizes such a norm precedes), groups of 32 / 64 / 128.
+// The GEMV whose waves walk the rows: out[n] = sum_k (s q + b)[n, k] x[k] for one row of x against rows of 4096 / 8192
+// codes (mt_qmv and the affine_qmv family, crates/metaltile-std/src/mlx/quantized.rs:8-308; dequant_gemv_int2 / int4,
+// crates/metaltile-std/src/ffai/dequant_gemv.rs:52-100), f16 / bf16, groups of 32 / 64 / 128, and on the same body
+//   - the RMS norm fused in front of it, x'[k] = x[k] norm_w[k] / sqrt(mean(x^2) + eps) (ffai_rms_norm_qgemv / _fast,
+//     crates/metaltile-std/src/ffai/rms_norm_qgemv.rs:53-125, 128-456),
+//   - two to four matrices against the one row in one launch (the fused projections of a decode step),
+//   - expert-routed rows, fewer than the experts, and the single-index expert GEMV,
+//   - 2-bit codes.
 //
 // The make of the one-row-per-wave kernel (qmv_rows.hip): a wave owns a weight row, lane l its 16-byte chunks l, 64 + l, ...,
 // codes become operands of the 4x4x4 matrix instruction in place, the activations are put into operand order once per
-// workgroup in LDS. Two things differ. The activations are normalised on the way into LDS: every workgroup works out
-// the row's sum of squares itself (thread t from chunk t, one more barrier), and x', an f32 value in the reference, is
-// carried as the element-type value nearest to it and the rounded (f16: scaled) remainder -- two operand sets whose
-// products are added, 16 significant bits, as in the streaming kernel's fused form. And because that preparation is
-// no longer cheap, a workgroup does it once and then walks many rows: the launch is at most two workgroups of eight
-// waves per compute unit (one of sixteen up to 4096 rows), wave g of G takes rows g, g + G, g + 2 G, ..., each row's
-// loads issued while the row before it is worked on.
+// workgroup in LDS. What differs is that a workgroup stays: the launch is at most two workgroups of eight waves per
+// compute unit (one of sixteen up to 4096 rows), wave g of G takes rows g, g + G, g + 2 G, ..., each row's loads issued
+// while the row before it is worked on, so the activations are read and prepared once per few dozen rows. With the norm,
+// the activations are normalised on the way into LDS: every workgroup works out the row's sum of squares itself
+// (thread t from chunk t, one more barrier), and x', an f32 value in the reference, is carried as the element-type value
+// nearest to it and the rounded (f16: scaled) remainder -- two operand sets whose products are added, 16 significant
+// bits, as in the streaming kernel's fused form.
 #include <hip/hip_runtime.h>
 
 #include "../../include/mtq.h"
