@@ -531,14 +531,14 @@ bool qmv_rows_walk_takes(const QmvParams& p) {
 // in groups of 128 (14336 x 8192: 12.59 / 12.80).
 bool qmv_rows_walk_preferred(const QmvParams& p) {
     if (!qmv_rows_walk_takes(p)) return false;
-    // Routed rows, fewer than the experts (8 experts, bf16, us, the routed wave-per-row kernels or, from three rows of 4096
-    // codes, the matrix-core GEMV -> this): experts of 14336 x 4096, 1 / 2 / 3 / 4 rows on distinct experts 8.6 -> 7.4, 15.3 ->
-    // 12.3, 22.1 -> 18.5, 27.9 -> 23.4; of 4096 x 8192 6.3 - 6.9 -> 5.9, 10.6 -> 8.2, 15.4 -> 10.9, 20.6 -> 13.4; of 14336 x 8192 18.0 ->
-    // 12.5, 31.5 -> 22.2, 48.0 -> 32.8, 63.4 -> 41.4. Two rows on one expert are two passes over its matrix: 13.4 -> 14.2 on
-    // 14336 x 4096 (the older kernel's second pass is shorter), 9.8 -> 8.6 and 29.9 -> 22.2 on the others.
-    // Five and seven rows on eight experts (the matrix-core GEMV -> this, in a chain): 14336 x 4096 41.2 -> 28.6, 51.2 -> 39.2;
-    // 4096 x 8192 25.2 -> 17.3, 31.3 -> 23.2. The single-index form as the plain launch of the same matrix (14336 x 4096 7.4 -> 6.7,
-    // 14336 x 8192 13.8 -> 12.8, 4096 x 8192 5.0 -> 5.4).
+    // Routed rows, fewer than the experts (8 experts, bf16, us per launch in a chain of launches, the routed wave-per-row
+    // kernels or, from three rows of 4096 codes, the matrix-core GEMV -> this): experts of 14336 x 4096, 1 / 2 / 3 / 4 / 5 / 7 rows
+    // on distinct experts 8.1 - 8.3 -> 7.9 - 8.2, 14.9 -> 12.8, 22.3 -> 18.7, 28.4 -> 24.1, 41.2 -> 28.6, 51.2 -> 39.2; of 4096 x 8192 5.9 -> 5.4,
+    // 10.3 -> 8.8, (5 / 7 rows) 25.2 -> 17.3, 31.3 -> 23.2. Launched alone, with a host wait behind each launch, the gains are
+    // larger (14336 x 4096 one row 8.6 -> 7.4; 14336 x 8192, 1 / 4 rows 18.0 -> 12.5, 63.4 -> 41.4). Two rows on one expert are two
+    // passes over its matrix: 13.4 -> 14.2 alone on 14336 x 4096 (the older kernel's second pass is shorter), 9.8 -> 8.6 and
+    // 29.9 -> 22.2 on the others. The single-index form is routed as the plain launch of the same matrix (in a chain:
+    // 14336 x 4096 7.4 -> 6.7, 14336 x 8192 13.8 -> 12.8, 4096 x 8192 5.0 -> 5.4).
     if (p.gather != GATHER_NONE && p.gather != GATHER_SINGLE) return p.N >= 1024 && p.T < p.E && p.T <= 8;
     // 2-bit codes (rows of 8192), the one-row-per-wave kernel -> this: 8192 rows f16 g32 / g64 / g128 6.76 -> 6.30, 6.27 -> 5.91,
     // 6.09 -> 5.61; bf16 g64 14336 / 28672 rows 9.51 -> 8.75, 16.2 -> 14.4; 2048 / 4096 rows 3.62 -> 3.84, 4.01 -> 4.30
