@@ -151,14 +151,30 @@ template <int DT, int BITS> __global__ __launch_bounds__(256) void qvm32_partial
             for (; d < ge; d += 64) {
                 uint32_t cw[4][BITS];
                 float xv[4];
+                // The four activations first, as loaded, then the rows' words, and only then the conversions: the order is
+                // pinned (left to itself the compiler converts each activation behind its load, a wait per row; loaded under
+                // a condition of its own it would sit in a branch). Rows past the group read row d again and count as zero.
+                uint32_t xbits[4];
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const uint32_t dr = d + 16 * r;
-                    const bool on = dr < ge;
-                    const uint32_t* row = a.w + (size_t)(on ? dr : d) * a.wpr + wi;
+                    const size_t xi = (size_t)m * a.K + (dr < ge ? dr : d);
+                    if constexpr (DT == DT_F32) xbits[r] = ((const uint32_t*)a.x)[xi];
+                    else xbits[r] = ((const uint16_t*)a.x)[xi];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const uint32_t dr = d + 16 * r;
+                    const uint32_t* row = a.w + (size_t)(dr < ge ? dr : d) * a.wpr + wi;
 #pragma unroll
                     for (int i = 0; i < BITS; i++) cw[r][i] = row[i];
-                    xv[r] = on ? load_elem<DT>(a.x, (size_t)m * a.K + dr) : 0.f;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float xr = DT == DT_F32 ? __uint_as_float(xbits[r]) : DT == DT_BF16 ? bf16_bits_to_f32(xbits[r]) : f16_bits_to_f32(xbits[r]);
+                    xv[r] = d + 16 * r < ge ? xr : 0.f;
                 }
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
