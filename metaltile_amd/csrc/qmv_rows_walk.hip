@@ -32,6 +32,7 @@ struct QmvRowsNArgs {
     const uint16_t* x;
     uint16_t* out;
     uint32_t N;
+    uint32_t slot_major;      // wave w of workgroup g starts at row w * gridDim.x + g instead of g * waves + w
     const uint16_t* norm_w;   // [K]
     const float* norm_eps;    // one f32 on the device
     // Several matrices against the one activation row (the batched instances): the rows of matrix m are rows
@@ -76,7 +77,11 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     __shared__ __align__(16) float xm_lds[BITS == 2 ? 2 * C : 4];   // 2-bit codes: that sum weighted with the pairs' offsets
     __shared__ float ssq_lds[NWV];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t gw = blockIdx.x * (uint32_t)NWV + wave, GW = gridDim.x * (uint32_t)NWV;   // (the same in every lane: row numbers stay in scalar registers)
+    // (the same in every lane: row numbers stay in scalar registers) A turn's rows go to the launch's waves workgroup by
+    // workgroup (a workgroup's waves on consecutive rows), or wave slot by wave slot (a workgroup's waves gridDim.x rows
+    // apart): which of the two the launch picks is a measured rule, stated where it is set.
+    const uint32_t GW = gridDim.x * (uint32_t)NWV;
+    const uint32_t gw = a.slot_major ? wave * gridDim.x + blockIdx.x : blockIdx.x * (uint32_t)NWV + wave;
     const uint32_t last = a.N - 1u;
     const uint32_t gl = min(lane, (uint32_t)(GPR / GPL - 1));
     // Routed rows: grid row blockIdx.y serves the blockIdx.y-th expert that has a row, and the walk below runs once per
@@ -444,6 +449,15 @@ template <bool NORM> static int launch_rows_walk(const QmvParams& p, const void*
     a.w = (const rp_u32x4*)p.w; a.s = (const uint16_t*)p.scales; a.b = (const uint16_t*)p.biases; a.x = (const uint16_t*)p.x; a.out = (uint16_t*)p.out;
     a.N = p.N; a.norm_w = (const uint16_t*)norm_w; a.norm_eps = eps;
     a.route = p.route; a.E = p.E; a.T = p.T;
+    // Rows of 4096 4-bit codes in groups of 64, from 16384 rows: slot by slot (bf16, us per launch in a chain, workgroup by
+    // workgroup -> slot by slot, two machines: 16384 rows 8.44 -> 8.05 and 8.28 -> 7.93, 28672 13.0 -> 12.4 and 12.7 -> 12.3, 40960
+    // 17.8 -> 16.7, 57344 23.5 -> 22.3 and 23.1 -> 22.2, 98304 37.2 -> 36.6; 14336 rows 7.47 -> 7.55 and 7.40 -> 7.43, 8192 rows the
+    // same). Other shapes stay workgroup by workgroup: groups of 32 / 128 on 28672 x 4096 13.2 -> 13.2, 12.2 -> 12.3 (11.8 -> 12.2
+    // on the other machine); rows of 8192 codes 14336 / 28672 / 57344 rows 12.9 -> 13.0, 22.1 -> 24.0, 42.3 -> 46.0.
+    // The norm's and the batched instances alike (norm 16384 / 28672 / 32768 rows 9.9 -> 9.8, 14.3 -> 14.2, 16.0 -> 15.8; two matrices
+    // of 14336 rows 13.0 -> 12.6, three of 8192 11.5 -> 11.2). The kernels that work one long row per wave and end lose by it
+    // (4096 x 14336 7.33 -> 7.42, 8192 x 8192 8.0 -> 8.2).
+    a.slot_major = p.bits == 4 && p.K == 4096 && p.group_size == 64 && p.N >= 16384 && p.gather == GATHER_NONE;
     if (batch) {
         uint32_t at = 0;
         for (int j = 0; j < 4; j++) {

@@ -128,7 +128,7 @@ def test_norm_fused_into_the_matrix_core_gemv(oracle, dt, N, K, G):
 
 
 @pytest.mark.parametrize("dt", [DType.F16, DType.BF16], ids=lambda d: d.name)
-@pytest.mark.parametrize("N,K,G", [(14336, 4096, 64), (1030, 4096, 32), (19, 4096, 128), (1, 4096, 64), (4096, 8192, 64), (33, 8192, 32), (1028, 8192, 128)])
+@pytest.mark.parametrize("N,K,G", [(14336, 4096, 64), (16390, 4096, 64), (1030, 4096, 32), (19, 4096, 128), (1, 4096, 64), (4096, 8192, 64), (33, 8192, 32), (1028, 8192, 128)])
 def test_norm_fused_into_the_one_row_per_wave_kernel(oracle, dt, N, K, G):
     """The same operation with the norm applied as the one-row-per-wave GEMV puts the activation row into LDS (4-bit
     codes, rows of 4096 / 8192 codes; automatic from 1024 weight rows, forced below that with qmv.kernel = 3): every

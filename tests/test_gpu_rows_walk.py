@@ -9,8 +9,9 @@ pytestmark = pytest.mark.gpu
 
 # Rows per launch chosen for the ways a wave's share can end: one workgroup of sixteen rows per 16 rows up to 4096 rows
 # (every wave one row or none), 4096 waves beyond (8192: two rows each; 12289: three, and one wave a fourth; 20481: five
-# or six), ragged last workgroups, a single row.
-ROWS = [1, 5, 16, 1030, 4096, 4100, 8192, 12289, 20481]
+# or six), ragged last workgroups, a single row. From 16384 rows of 4096 codes in groups of 64 a turn's rows are dealt to
+# the waves slot by slot instead of workgroup by workgroup (16384: the first such size, four rows each; 20481).
+ROWS = [1, 5, 16, 1030, 4096, 4100, 8192, 12289, 16384, 20481]
 
 
 @pytest.mark.parametrize("dt_name", ["BF16", "F16"])
