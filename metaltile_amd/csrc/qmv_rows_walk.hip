@@ -457,7 +457,10 @@ template <bool NORM> static int launch_rows_walk(const QmvParams& p, const void*
     // The norm's and the batched instances alike (norm 16384 / 28672 / 32768 rows 9.9 -> 9.8, 14.3 -> 14.2, 16.0 -> 15.8; two matrices
     // of 14336 rows 13.0 -> 12.6, three of 8192 11.5 -> 11.2). The kernels that work one long row per wave and end lose by it
     // (4096 x 14336 7.33 -> 7.42, 8192 x 8192 8.0 -> 8.2).
-    a.slot_major = p.bits == 4 && p.K == 4096 && p.group_size == 64 && p.N >= 16384 && p.gather == GATHER_NONE;
+    // 2-bit codes (rows of 8192, the same 2 KB): groups of 32 and 64 gain from 16384 rows (f16, 16384 / 28672 rows: g32 10.8 -> 10.6,
+    // 17.0 -> 16.4; g64 10.6 -> 10.1, 17.7 -> 17.1), groups of 128 do not (10.7 -> 10.7, 16.8 -> 16.9), 8192 rows are the same.
+    a.slot_major = p.gather == GATHER_NONE && p.N >= 16384 &&
+                   ((p.bits == 4 && p.K == 4096 && p.group_size == 64) || (p.bits == 2 && p.group_size <= 64));
     if (batch) {
         uint32_t at = 0;
         for (int j = 0; j < 4; j++) {

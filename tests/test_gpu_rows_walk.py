@@ -53,11 +53,11 @@ def test_rows_walk_kernel_against_the_oracle(oracle, dt_name, G, K, N):
 
 @pytest.mark.parametrize("dt_name", ["BF16", "F16"])
 @pytest.mark.parametrize("G", [32, 64, 128])
-@pytest.mark.parametrize("N", [1, 50, 4096, 8192, 12289])
+@pytest.mark.parametrize("N", [1, 50, 4096, 8192, 12289, 16390])
 def test_rows_walk_kernel_two_bit_codes(oracle, dt_name, G, N):
     """2-bit codes on rows of 8192 (made operands in place, with an offset that depends on the crumb's position; groups
     of 32 span half a chunk, so a chunk's halves are scaled apart): forced with qmv.kernel = 4, full-range codes, behind
-    a cache flush, guard elements, against the f64 oracle."""
+    a cache flush, guard elements, against the f64 oracle. (16390 rows: dealt to the waves slot by slot in groups of 32 / 64.)"""
     import metaltile_amd as m
     from metaltile_amd import DType, GpuBuffer, ops, _lib
     from metaltile_amd.synth import make_case
