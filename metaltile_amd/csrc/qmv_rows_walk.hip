@@ -1,5 +1,5 @@
 // The GEMV whose waves walk the rows: out[n] = sum_k (s q + b)[n, k] x[k] for one row of x against rows of 4096 / 8192
-// codes (mt_qmv and the affine_qmv family, crates/metaltile-std/src/mlx/quantized.rs:8-308; dequant_gemv_int2 / int4,
+// codes (the plain form also 2048 / 6144; mt_qmv and the affine_qmv family, crates/metaltile-std/src/mlx/quantized.rs:8-308; dequant_gemv_int2 / int4,
 // crates/metaltile-std/src/ffai/dequant_gemv.rs:52-100), f16 / bf16, groups of 32 / 64 / 128, and on the same body
 //   - the RMS norm fused in front of it, x'[k] = x[k] norm_w[k] / sqrt(mean(x^2) + eps) (ffai_rms_norm_qgemv / _fast,
 //     crates/metaltile-std/src/ffai/rms_norm_qgemv.rs:53-125, 128-456),
@@ -438,6 +438,8 @@ template <int DT, int LOG2G, bool NORM> static const void* rows_walk_fn(uint32_t
         if (sixteen) return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 16>;
         return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 8>;
     } else {
+        if (K == 2048) return sixteen ? (const void*)qmv_rows_walk_kernel<DT, 1, LOG2G, 16> : (const void*)qmv_rows_walk_kernel<DT, 1, LOG2G, 8>;
+        if (K == 6144) return sixteen ? (const void*)qmv_rows_walk_kernel<DT, 3, LOG2G, 16> : (const void*)qmv_rows_walk_kernel<DT, 3, LOG2G, 8>;
         if (sixteen) return K == 4096 ? (const void*)qmv_rows_walk_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_walk_kernel<DT, 4, LOG2G, 16>;
         return K == 4096 ? (const void*)qmv_rows_walk_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_walk_kernel<DT, 4, LOG2G, 8>;
     }
@@ -533,6 +535,11 @@ bool qmv_rows_walk_takes(const QmvParams& p) {
         q.bits = 4;
         return p.K == 8192 && qmv_rows_norm_takes(q, p.x);
     }
+    if (p.K == 2048 || p.K == 6144) {   // one matrix of 4-bit codes also in rows of 2048 and 6144 codes: everything else as for 4096
+        QmvParams q = p;
+        q.K = 4096;
+        return qmv_rows_norm_takes(q, p.x);
+    }
     return qmv_rows_norm_takes(p, p.x);   // (the alignment of x stands in for that of the norm weights)
 }
 
@@ -560,13 +567,21 @@ bool qmv_rows_walk_preferred(const QmvParams& p) {
     // 2-bit codes (rows of 8192), the one-row-per-wave kernel -> this: 8192 rows f16 g32 / g64 / g128 6.76 -> 6.30, 6.27 -> 5.91,
     // 6.09 -> 5.61; bf16 g64 14336 / 28672 rows 9.51 -> 8.75, 16.2 -> 14.4; 2048 / 4096 rows 3.62 -> 3.84, 4.01 -> 4.30
     if (p.bits == 2) return p.N >= 8192;
+    // Rows of 2048 / 6144 codes (bf16 g64, the kernels that end after a row block -> this): 2048 codes, 1024 / 2048 / 4096 / 8192 /
+    // 16384 / 20480 rows 3.4 - 3.7 -> 3.2, 3.4 - 3.6 -> 2.7 - 3.3, 3.5 -> 2.9 - 3.3, 4.56 -> 3.80, 5.87 -> 5.57, 6.66 -> 6.54, level at
+    // 24576 and behind beyond (128256 rows 24.8 -> 29.2: a wave's two rows in flight are 2 KB; four workgroups per compute unit
+    // bring that to 26.6 and cost the sizes below 16384 rows 5 %); 6144 codes, 1024 / 2048 / 4096 / 8192 / 16384 / 32768 / 102400 rows
+    // 4.22 -> 3.66, 4.59 -> 3.83, 5.66 -> 4.38, 7.68 -> 6.56, 12.0 -> 11.4, 20.3 -> 19.7, 60.5 -> 57.8; groups of 32 / 128 alike
+    // (8192 x 2048 f16 4.60 -> 3.89, 4.58 -> 3.81; 16384 x 6144 12.7 -> 11.8, 12.0 -> 11.3).
+    if (p.K == 2048) return p.N >= 1024 && p.N <= 20480;
+    if (p.K == 6144) return p.N >= 1024;
     if (p.K == 4096) return p.N >= 1536 && (p.N <= 40960 || p.N >= 81920);
     return p.N >= 10240 && p.group_size != 128;
 }
 
 // The batch on one walk: every matrix as the single one would have to be, the rows counted together.
 static bool rows_walk_batch_as_one(const QmvParams& p0, const QmvBatch& b, QmvParams& p) {
-    if (b.n < 2 || b.n > 4 || p0.bits != 4) return false;
+    if (b.n < 2 || b.n > 4 || p0.bits != 4 || (p0.K != 4096 && p0.K != 8192)) return false;
     p = p0;
     p.gather = GATHER_NONE;
     p.M = 1;
@@ -595,7 +610,7 @@ int launch_qmv_rows_walk_batched(const QmvParams& p0, const QmvBatch& b, const L
 }
 
 int launch_qmv_rows_walk(const QmvParams& p, const LaunchCtx& lc) {
-    if (!qmv_rows_walk_takes(p)) return fail(ERR_UNSUPPORTED, "qmv walking rows kernel: one activation row, 4-bit codes, rows of 4096 or 8192 codes, f16 / bf16");
+    if (!qmv_rows_walk_takes(p)) return fail(ERR_UNSUPPORTED, "qmv walking rows kernel: one activation row, 4-bit codes, rows of 2048, 4096, 6144 or 8192 codes, f16 / bf16");
     return launch_rows_walk<false>(p, nullptr, nullptr, lc);
 }
 
