@@ -1,5 +1,5 @@
 // The GEMV whose waves walk the rows: out[n] = sum_k (s q + b)[n, k] x[k] for one row of x against rows of 4096 / 8192
-// codes (the plain form also 2048 / 6144; mt_qmv and the affine_qmv family, crates/metaltile-std/src/mlx/quantized.rs:8-308; dequant_gemv_int2 / int4,
+// codes (the plain form also 2048 / 3072 / 3584 / 5120 / 6144 / 7168; mt_qmv and the affine_qmv family, crates/metaltile-std/src/mlx/quantized.rs:8-308; dequant_gemv_int2 / int4,
 // crates/metaltile-std/src/ffai/dequant_gemv.rs:52-100), f16 / bf16, groups of 32 / 64 / 128, and on the same body
 //   - the RMS norm fused in front of it, x'[k] = x[k] norm_w[k] / sqrt(mean(x^2) + eps) (ffai_rms_norm_qgemv / _fast,
 //     crates/metaltile-std/src/ffai/rms_norm_qgemv.rs:53-125, 128-456),
@@ -57,15 +57,18 @@ template <int CH> struct RowsNormBuf {
     uint32_t sw[2], bw[2];   // the lane's groups of the bias term, two 16-bit elements per dword (one group per lane: the dword that holds it)
 };
 
-template <int DT, int CH, int LOG2G, int NWV, bool NORM, bool BATCH = false, int BITS = 4, int GM = GATHER_NONE>
+// TAIL: the chunks of the last 64 a row has (0: all 64; a row of 3584 codes is 112 chunks, CH = 2 and TAIL = 48). The lanes
+// past them load the row's last chunk and add nothing.
+template <int DT, int CH, int LOG2G, int NWV, bool NORM, bool BATCH = false, int BITS = 4, int GM = GATHER_NONE, int TAIL = 0>
 __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     static_assert(BITS == 4 || (BITS == 2 && !NORM && !BATCH), "4-bit codes; 2-bit codes on the plain walk");
     constexpr bool ROUTED = GM != GATHER_NONE;
     static_assert(!ROUTED || (!NORM && !BATCH && BITS == 4), "routed rows: the plain walk on 4-bit codes");
+    static_assert(TAIL == 0 || (TAIL > 0 && TAIL < 64 && TAIL % 16 == 0 && BITS == 4 && !NORM && !BATCH && !ROUTED), "ragged rows: the plain walk on 4-bit codes, whole 4-lane blocks");
     constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;   // 4-bit codes: one offset for every pair
     constexpr float REM = 1.0f / RemSplit<DT>::kRemScale;
     constexpr int CPC = 128 / BITS, Q = CPC / 8;   // codes per 16-byte chunk; 16-byte quarters of a chunk's activations in operand order
-    constexpr int C = 64 * CH, K = C * CPC;
+    constexpr int C = TAIL ? 64 * (CH - 1) + TAIL : 64 * CH, K = C * CPC;   // chunks and codes per row
     constexpr int GPR = K >> LOG2G;          // groups per row
     constexpr int GPL = GPR > 128 ? 4 : GPR > 64 ? 2 : 1;   // groups a lane owns in the bias term (lanes below GPR / GPL)
     constexpr int NH = (1 << LOG2G) < CPC ? 2 : 1;           // groups a chunk spans (2-bit codes in groups of 32: its halves are accumulated and scaled apart)
@@ -106,8 +109,11 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
             bp = a.b + (eoff + row) * GPR;
             wrow = a.w + (eoff + row) * C;
         }
+        uint32_t ci[CH];   // this lane's chunks (past the row's end: its last chunk)
 #pragma unroll
-        for (int i = 0; i < CH; i++) r.sc[i] = ((const uint32_t*)sp)[((uint32_t)(i * 64 + (int)lane) * CPC) >> (LOG2G + 1)];   // (a chunk that spans two groups: both of them)
+        for (int i = 0; i < CH; i++) ci[i] = TAIL && i == CH - 1 ? min((uint32_t)(i * 64) + lane, (uint32_t)(C - 1)) : (uint32_t)(i * 64) + lane;
+#pragma unroll
+        for (int i = 0; i < CH; i++) r.sc[i] = ((const uint32_t*)sp)[(ci[i] * CPC) >> (LOG2G + 1)];   // (a chunk that spans two groups: both of them)
         r.sw[0] = r.sw[1] = r.bw[0] = r.bw[1] = 0u;
         if constexpr (GPL == 4) {
             const uint2 sv = ((const uint2*)sp)[gl], bv = ((const uint2*)bp)[gl];
@@ -121,7 +127,7 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
         }
         const rp_u32x4* wbase = wrow + lane;
 #pragma unroll
-        for (int i = 0; i < CH; i++) r.wv[i] = __builtin_nontemporal_load(wbase + i * 64);
+        for (int i = 0; i < CH; i++) r.wv[i] = TAIL && i == CH - 1 ? __builtin_nontemporal_load(wrow + ci[i]) : __builtin_nontemporal_load(wbase + i * 64);
     };
     for (uint32_t pass = 0; pass < rt.n_pass; pass++) {   // (one pass unless routed)
     const uint32_t trow = rows_route_row<GM>(rt, pass);
@@ -276,7 +282,7 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
 #pragma unroll
                 for (int d = 0; d < 4; d++) {
                     const uint32_t w = r.wv[i][d];
-                    const uint4 xo = *(const uint4*)xp_lds[d][i * 64 + ln];
+                    const uint4 xo = *(const uint4*)xp_lds[d][TAIL && i == CH - 1 ? min((uint32_t)(i * 64) + ln, (uint32_t)(C - 1)) : (uint32_t)(i * 64) + ln];
                     uint4 xl = make_uint4(0u, 0u, 0u, 0u);
                     if constexpr (NORM) xl = *(const uint4*)xl_lds[d][i * 64 + ln];
                     rp_u32x2 b0, b1, a0, a1, l0, l1;
@@ -293,8 +299,9 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
                         dl = rp_mfma<DT>(l1, b1, dl);
                     }
                 }
-                const uint32_t sch = 16u * ((((uint32_t)(i * 64 + (int)lane) * CPC) >> LOG2G) & 1u);   // the half of the dword the chunk's group is in
-                t = fmaf(rp_up<DT>((r.sc[i] >> sch) & 0xFFFFu), fmaf(rp_diag(dl, j0, j1), REM, rp_diag(dh, j0, j1)), t);
+                const uint32_t sch = 16u * ((((TAIL && i == CH - 1 ? min((uint32_t)(i * 64) + lane, (uint32_t)(C - 1)) : (uint32_t)(i * 64) + lane) * CPC) >> LOG2G) & 1u);   // the half of the dword the chunk's group is in
+                const float ti = fmaf(rp_up<DT>((r.sc[i] >> sch) & 0xFFFFu), fmaf(rp_diag(dl, j0, j1), REM, rp_diag(dh, j0, j1)), t);
+                t = TAIL && i == CH - 1 && lane >= (uint32_t)TAIL ? t : ti;   // (lanes past the row's end hold its last chunk again)
             } else {
                 rp_f32x4 dq[NH];
 #pragma unroll
@@ -394,6 +401,11 @@ template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * 
 template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_walk_kernel(QmvRowsNArgs a) {
     qmv_rows_walk_body<DT, CH, LOG2G, NWV, false>(a);
 }
+// Rows that do not fill whole groups of 64 chunks (3072 / 3584 / 5120 / 7168 codes: the hidden sizes of other models).
+template <int DT, int CH, int LOG2G, int NWV, int TAIL> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_walk_ragged_kernel(QmvRowsNArgs a) {
+    qmv_rows_walk_body<DT, CH, LOG2G, NWV, false, false, 4, GATHER_NONE, TAIL>(a);
+}
+
 // 2-bit codes (rows of 8192: 128 chunks of 64 codes), made operands in place as in the one-row-per-wave kernel.
 template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_walk2_kernel(QmvRowsNArgs a) {
     qmv_rows_walk_body<DT, CH, LOG2G, NWV, false, false, 2>(a);
@@ -439,6 +451,10 @@ template <int DT, int LOG2G, bool NORM> static const void* rows_walk_fn(uint32_t
         return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 8>;
     } else {
         if (K == 2048) return sixteen ? (const void*)qmv_rows_walk_kernel<DT, 1, LOG2G, 16> : (const void*)qmv_rows_walk_kernel<DT, 1, LOG2G, 8>;
+        if (K == 3072) return sixteen ? (const void*)qmv_rows_walk_ragged_kernel<DT, 2, LOG2G, 16, 32> : (const void*)qmv_rows_walk_ragged_kernel<DT, 2, LOG2G, 8, 32>;
+        if (K == 3584) return sixteen ? (const void*)qmv_rows_walk_ragged_kernel<DT, 2, LOG2G, 16, 48> : (const void*)qmv_rows_walk_ragged_kernel<DT, 2, LOG2G, 8, 48>;
+        if (K == 5120) return sixteen ? (const void*)qmv_rows_walk_ragged_kernel<DT, 3, LOG2G, 16, 32> : (const void*)qmv_rows_walk_ragged_kernel<DT, 3, LOG2G, 8, 32>;
+        if (K == 7168) return sixteen ? (const void*)qmv_rows_walk_ragged_kernel<DT, 4, LOG2G, 16, 32> : (const void*)qmv_rows_walk_ragged_kernel<DT, 4, LOG2G, 8, 32>;
         if (K == 6144) return sixteen ? (const void*)qmv_rows_walk_kernel<DT, 3, LOG2G, 16> : (const void*)qmv_rows_walk_kernel<DT, 3, LOG2G, 8>;
         if (sixteen) return K == 4096 ? (const void*)qmv_rows_walk_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_walk_kernel<DT, 4, LOG2G, 16>;
         return K == 4096 ? (const void*)qmv_rows_walk_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_walk_kernel<DT, 4, LOG2G, 8>;
@@ -535,7 +551,7 @@ bool qmv_rows_walk_takes(const QmvParams& p) {
         q.bits = 4;
         return p.K == 8192 && qmv_rows_norm_takes(q, p.x);
     }
-    if (p.K == 2048 || p.K == 6144) {   // one matrix of 4-bit codes also in rows of 2048 and 6144 codes: everything else as for 4096
+    if (p.K == 2048 || p.K == 6144 || p.K == 3072 || p.K == 3584 || p.K == 5120 || p.K == 7168) {   // one matrix of 4-bit codes also in these row lengths: everything else as for 4096
         QmvParams q = p;
         q.K = 4096;
         return qmv_rows_norm_takes(q, p.x);
@@ -573,6 +589,12 @@ bool qmv_rows_walk_preferred(const QmvParams& p) {
     // bring that to 26.6 and cost the sizes below 16384 rows 5 %); 6144 codes, 1024 / 2048 / 4096 / 8192 / 16384 / 32768 / 102400 rows
     // 4.22 -> 3.66, 4.59 -> 3.83, 5.66 -> 4.38, 7.68 -> 6.56, 12.0 -> 11.4, 20.3 -> 19.7, 60.5 -> 57.8; groups of 32 / 128 alike
     // (8192 x 2048 f16 4.60 -> 3.89, 4.58 -> 3.81; 16384 x 6144 12.7 -> 11.8, 12.0 -> 11.3).
+    // Rows that end inside a group of 64 chunks (bf16 g64, the streaming kernel -> this): 3072 codes, 1024 / 4096 / 8192 / 18944 /
+    // 57344 rows 5.01 -> 3.30, 4.57 -> 3.38, 6.00 -> 4.56, 12.8 -> 8.45, 23.1 -> 19.9; 3584 codes 4.93 -> 3.3, 4.64 -> 3.46, 6.19 -> 4.83,
+    // 12.9 -> 8.85, 23.5 -> 21.0 (151936 rows 55.6 -> 51.1); 5120 codes 3.86 -> 3.62, 5.91 -> 4.15, 8.27 -> 6.21, 13.8 -> 12.4, 32.2 -> 28.3
+    // (13824 rows f16 g32 / g128 12.2 -> 9.85, 11.0 -> 10.5); 7168 codes 5.31 -> 4.15, 6.22 -> 4.94, 9.56 -> 7.65, 17.9 -> 15.4, 41.5 -> 39.2
+    // (129280 rows 91.9 -> 86.4).
+    if (p.K == 3072 || p.K == 3584 || p.K == 5120 || p.K == 7168) return p.N >= 1024;
     if (p.K == 2048) return p.N >= 1024 && p.N <= 20480;
     if (p.K == 6144) return p.N >= 1024;
     if (p.K == 4096) return p.N >= 1536 && (p.N <= 40960 || p.N >= 81920);
@@ -610,7 +632,7 @@ int launch_qmv_rows_walk_batched(const QmvParams& p0, const QmvBatch& b, const L
 }
 
 int launch_qmv_rows_walk(const QmvParams& p, const LaunchCtx& lc) {
-    if (!qmv_rows_walk_takes(p)) return fail(ERR_UNSUPPORTED, "qmv walking rows kernel: one activation row, 4-bit codes, rows of 2048, 4096, 6144 or 8192 codes, f16 / bf16");
+    if (!qmv_rows_walk_takes(p)) return fail(ERR_UNSUPPORTED, "qmv walking rows kernel: one activation row, 4-bit codes, rows of 2048 to 8192 codes in steps of 1024 (and 3584), f16 / bf16");
     return launch_rows_walk<false>(p, nullptr, nullptr, lc);
 }
 

@@ -134,10 +134,12 @@ def test_benchmark_configurations_are_routed_as_documented():
                  (DType.BF16, 8, 64, 1, 4096, 4096), (DType.BF16, 4, 64, 1, 512, 4096)):
         assert "qmv_rows_kernel" not in kernels("qmv", *args)[0][0]          # what that kernel does not take
     for args in ((DType.BF16, 4, 64, 2, 14336, 4096), (DType.BF16, 8, 64, 1, 14336, 4096), (DType.BF16, 2, 64, 1, 14336, 8192),
-                 (DType.F32, 4, 64, 1, 14336, 4096), (DType.BF16, 4, 64, 1, 14336, 3072), (DType.BF16, 4, 16, 1, 14336, 4096), (DType.BF16, 4, 64, 1, 24576, 2048)):
-        assert "qmv_rows_walk_kernel" not in kernels("qmv", *args)[0][0]     # nor the walk: one row, 4-bit, 2048 / 4096 / 6144 / 8192 codes (2048: up to 20480 rows), groups of 32 / 64 / 128
+                 (DType.F32, 4, 64, 1, 14336, 4096), (DType.BF16, 4, 64, 1, 14336, 2560), (DType.BF16, 4, 16, 1, 14336, 4096), (DType.BF16, 4, 64, 1, 24576, 2048)):
+        assert "qmv_rows_walk_kernel" not in kernels("qmv", *args)[0][0]     # nor the walk: one row, 4-bit, 2048 ... 8192 codes in steps of 1024 or 3584 (2048: up to 20480 rows), groups of 32 / 64 / 128
     ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 8192, 2048)
     assert "qmv_rows_walk_kernel<2, 1, 6, 8>" in ks[0] and ls[0][1][0] == 512 and ls[0][2][0] == 512
+    ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 18944, 3584)      # rows that end inside a group of 64 chunks
+    assert "qmv_rows_walk_ragged_kernel<2, 2, 6, 8, 48>" in ks[0] and ls[0][1][0] == 512 and ls[0][2][0] == 512
     ks, ls = kernels("qmv", DType.F16, 4, 128, 1, 4096, 6144)
     assert "qmv_rows_walk_kernel<1, 3, 7, 16>" in ks[0] and ls[0][1][0] == 256 and ls[0][2][0] == 1024
     ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 4096, 14336)
