@@ -226,13 +226,16 @@ struct QmvRowsLArgs {
     uint32_t E, T;
 };
 
-template <int DT, int BITS, int CH, int LOG2G, int GM>
+// TAIL: the chunks of the last 64 a row has (0: all 64; a row of 11008 codes is 344 chunks, CH = 6 and TAIL = 24). The lanes
+// past them load the row's last chunk and add nothing.
+template <int DT, int BITS, int CH, int LOG2G, int GM, int TAIL = 0>
 __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
     static_assert(BITS == 2 || BITS == 4, "2- or 4-bit codes");
+    static_assert(TAIL == 0 || (TAIL > 0 && TAIL < 64 && TAIL % 4 == 0 && BITS == 4 && GM == GATHER_NONE), "ragged rows: 4-bit codes, unrouted, whole 4-lane blocks");
     constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;   // 4-bit codes: one offset for every pair
     constexpr int CPC = 128 / BITS;        // codes per chunk
     constexpr int Q = CPC / 8;             // 16-byte quarters of a chunk's activations in operand order (4 pair dwords each)
-    constexpr int C = 64 * CH;             // chunks per row
+    constexpr int C = TAIL ? 64 * (CH - 1) + TAIL : 64 * CH;   // chunks per row
     constexpr int K = C * CPC;
     constexpr int GPR = K >> LOG2G;        // groups per row
     constexpr int GPL = GPR > 256 ? 8 : GPR > 128 ? 4 : GPR > 64 ? 2 : 1;   // groups a lane owns in the bias term (lanes below GPR / GPL)
@@ -271,7 +274,7 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
         const uint16_t* bp = a.b + rr * GPR;
 #pragma unroll
         for (int i = 0; i < CH; i++) {
-            const uint32_t k0 = (uint32_t)(i * 64 + (int)lane) * CPC;
+            const uint32_t k0 = (TAIL && i == CH - 1 ? min((uint32_t)(i * 64) + lane, (uint32_t)(C - 1)) : (uint32_t)(i * 64) + lane) * CPC;   // (past the row's end: its last chunk)
             sc[i][0] = sp[k0 >> LOG2G];
             if constexpr (NH == 2) sc[i][1] = sp[(k0 + CPC / 2) >> LOG2G];
         }
@@ -292,6 +295,7 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
     }
     RP_KEEP_ORDER();
     const rp_u32x4* wbase = a.w + rr * C + lane;
+    const rp_u32x4* wlast = a.w + rr * C + min((uint32_t)((CH - 1) * 64) + lane, (uint32_t)(C - 1));   // the lane's chunk of the last group, inside the row
     rp_u32x4 wv[CH];
     // Rows of more than four chunks per lane: the loads run four chunks ahead of the chunk being worked on and only two
     // are issued before the activations are prepared. A compute unit takes loads only as fast as earlier ones return, so
@@ -301,7 +305,7 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
     // at once (8192 x 8192 4-bit: 7.82 us against 9.05 with one ahead of the barrier, 10.2 with two).
     constexpr int W0 = CH > 4 ? 4 : CH, PRE = CH > 4 ? 2 : CH;
 #pragma unroll
-    for (int i = 0; i < PRE; i++) wv[i] = __builtin_nontemporal_load(wbase + i * 64);
+    for (int i = 0; i < PRE; i++) wv[i] = TAIL && i == CH - 1 ? __builtin_nontemporal_load(wlast) : __builtin_nontemporal_load(wbase + i * 64);
     RP_KEEP_ORDER();
     __builtin_amdgcn_s_setprio(0);
     const bool j0 = lane & 1u, j1 = lane & 2u;
@@ -373,7 +377,7 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
     }
     if (GM == GATHER_NONE || live) {
 #pragma unroll
-    for (int i = PRE; i < W0; i++) wv[i] = __builtin_nontemporal_load(wbase + i * 64);
+    for (int i = PRE; i < W0; i++) wv[i] = TAIL && i == CH - 1 ? __builtin_nontemporal_load(wlast) : __builtin_nontemporal_load(wbase + i * 64);
     RP_KEEP_ORDER();
     // bias term: over this lane's GPL groups, b X - s XM (4-bit codes: XM = MAGIC X). A group is SPG half chunks, so the
     // lane's groups are a run of GPL SPG consecutive half-chunk sums.
@@ -414,7 +418,7 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
     }
 #pragma unroll
     for (int i = 0; i < CH; i++) {
-        if (i + W0 < CH) wv[i + W0] = __builtin_nontemporal_load(wbase + (i + W0) * 64);
+        if (i + W0 < CH) wv[i + W0] = TAIL && i + W0 == CH - 1 ? __builtin_nontemporal_load(wlast) : __builtin_nontemporal_load(wbase + (i + W0) * 64);
         RP_KEEP_ORDER();
         rp_f32x4 dh[NH];
 #pragma unroll
@@ -424,7 +428,7 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
             const uint32_t w = wv[i][d];
             constexpr int HSH = NH == 2 ? 1 : 2;   // dword d adds to half d >> HSH
             if constexpr (BITS == 4) {
-                const uint4 xo = *(const uint4*)xp_lds[d][i * 64 + lane];
+                const uint4 xo = *(const uint4*)xp_lds[d][TAIL && i == CH - 1 ? min((uint32_t)(i * 64) + lane, (uint32_t)(C - 1)) : (uint32_t)(i * 64) + lane];
                 rp_u32x2 b0, b1, a0, a1;
                 b0.x = (w & 0x000F000Fu) | kor[0];
                 b0.y = ((w >> 4) & 0x000F000Fu) | kor[0];
@@ -454,7 +458,10 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
             }
         }
 #pragma unroll
-        for (int h = 0; h < NH; h++) t = fmaf(rp_up<DT>(sc[i][h]), rp_diag(dh[h], j0, j1), t);
+        for (int h = 0; h < NH; h++) {
+            const float ti = fmaf(rp_up<DT>(sc[i][h]), rp_diag(dh[h], j0, j1), t);
+            t = TAIL && i == CH - 1 && lane >= (uint32_t)TAIL ? t : ti;   // (lanes past the row's end hold its last chunk again)
+        }
     }
     t += __shfl_xor(t, 32, 64);
     t += dpp_f32<0xB1>(t);
@@ -471,6 +478,9 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
 }
 template <int DT, int BITS, int CH, int LOG2G>
 __global__ __launch_bounds__(1024) void qmv_rows_long_kernel(QmvRowsLArgs a) { qmv_rows_long_body<DT, BITS, CH, LOG2G, GATHER_NONE>(a); }
+// 4-bit codes on rows that end inside a group of 64 chunks (11008 / 13824 / 18944 / 27648 codes: the widths of other models).
+template <int DT, int CH, int LOG2G, int TAIL>
+__global__ __launch_bounds__(1024) void qmv_rows_long_ragged_kernel(QmvRowsLArgs a) { qmv_rows_long_body<DT, 4, CH, LOG2G, GATHER_NONE, TAIL>(a); }
 template <int DT, int BITS, int CH, int LOG2G, int GM>
 __global__ __launch_bounds__(1024) void qmv_rows_long_routed_kernel(QmvRowsLArgs a) { qmv_rows_long_body<DT, BITS, CH, LOG2G, GM>(a); }
 
@@ -514,10 +524,24 @@ static int launch_rows(int dtype, const void* w, const void* s, const void* b, c
 }
 
 // chunks of 16 bytes per lane and row for the one-row-per-wave kernel, or 0 if it has no instance for the shape
-static int rows_long_ch(const QmvParams& p) {
+// (*tail: the chunks of the row's last group of 64 where that group is not full, else 0)
+static int rows_long_ch(const QmvParams& p, int* tail = nullptr) {
+    if (tail) *tail = 0;
     if (p.bits != 2 && p.bits != 4) return 0;
     const uint32_t G = p.group_size, cpc = 128u / (uint32_t)p.bits;
     if (G != 32 && G != 64 && G != 128) return 0;
+    // 4-bit codes in groups of 64 / 128 on the row lengths of other models: 10240, 12288, 18432 codes (whole groups of 64
+    // chunks) and 11008, 13824, 18944, 27648 (the last group partly filled). Every lane's groups of the bias term are one
+    // aligned load: up to 256 groups per row the rows' scales are 8-byte multiples, beyond that 16-byte multiples.
+    if (p.bits == 4 && G >= 64 && p.gather == GATHER_NONE) {
+        static const struct { uint32_t K; int ch, tail; } kMore[] = {{10240, 5, 0}, {12288, 6, 0}, {18432, 9, 0}, {11008, 6, 24}, {13824, 7, 48}, {18944, 10, 16}, {27648, 14, 32}};
+        for (const auto& m : kMore) {
+            if (p.K != m.K) continue;
+            if (p.K / G > 256u && ((uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)) return 0;
+            if (tail) *tail = m.tail;
+            return m.ch;
+        }
+    }
     if (p.K % (64u * cpc) || p.K / G > 512u || (p.K / G) % 8u) return 0;
     const uint32_t ch = p.K / (64u * cpc);
     if (p.K / G > 256u && ((uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)) return 0;   // (a lane's eight groups of the bias term: one 16-byte load)
@@ -544,7 +568,7 @@ bool qmv_rows_takes(const QmvParams& p) {
     if ((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)p.scales % 8 || (uintptr_t)p.biases % 8 || (uintptr_t)p.out % 2) return false;
     if (p.bits == 4 && p.group_size == 64 && p.K == 4096) return p.N % 4 == 0;   // one wave per four rows
     const int ch = rows_long_ch(p);
-    return routed ? ch == 4 || ch == 7 : ch != 0;
+    return routed ? (p.K == 8192 || p.K == 14336) && (ch == 4 || ch == 7) : ch != 0;
 }
 
 // Where these kernels are the fastest the library has (measured against the streaming kernel in one run, f16 / bf16, us):
@@ -564,6 +588,11 @@ bool qmv_rows_preferred(const QmvParams& p) {
     // rows of 8192, 16384 / 28672 rows 14.7 / 14.3, 22.5 / 23.0. Longer rows stay here at every size (14336 codes, 8192 /
     // 14336 / 28672 rows 14.2 / 12.65, 21.5 / 20.35, 37.8 / 36.5; 28672 codes, 4096 / 8192 / 16384 rows 14.6 / 12.1, 24.5 /
     // 22.3, 51.8 / 42.1), and so do 2-bit codes (28672 x 8192: 19.7 / 17.6).
+    // The row lengths of other models (bf16 g64, us in a chain, the streaming kernel or the matrix-core GEMV -> these): 4096 x 10240 7.20 -> 5.83, 1024 /
+    // 4096 / 8192 x 11008 5.53 -> 3.65, 7.91 -> 6.35, 12.0 -> 11.9 (g128 7.92 -> 6.22), 4096 x 12288 7.98 -> 6.45, 2048 / 5120 / 16384 x
+    // 13824 6.98 -> 4.69, 11.67 -> 9.36, 24.8 -> 22.3, 7168 x 18432 15.6 -> 14.3, 3584 x 18944 10.97 -> 8.44 (g128 10.7 -> 8.43);
+    // 5120 x 27648 is level (18.6 / 18.8) and stays.
+    if (p.bits == 4 && p.K != 4096 && p.K != 8192 && p.K != 14336 && p.K != 28672) return p.K != 27648;
     if (p.bits == 4 && p.K == 4096) return p.N <= 16384;
     if (p.bits == 4 && p.K == 8192) return p.N <= 20480;
     return true;
@@ -582,6 +611,18 @@ template <int DT, int LOG2G> static const void* rows_long_fn_g(int bits, int ch)
     if constexpr (LOG2G >= 6) return (const void*)qmv_rows_long_kernel<DT, 2, 4, LOG2G>;       // (16384 codes in groups of 32: 512)
     return nullptr;
 }
+template <int DT, int LOG2G> static const void* rows_long_more_fn(uint32_t K) {   // groups of 64 / 128
+    switch (K) {
+        case 10240: return (const void*)qmv_rows_long_kernel<DT, 4, 5, LOG2G>;
+        case 12288: return (const void*)qmv_rows_long_kernel<DT, 4, 6, LOG2G>;
+        case 18432: return (const void*)qmv_rows_long_kernel<DT, 4, 9, LOG2G>;
+        case 11008: return (const void*)qmv_rows_long_ragged_kernel<DT, 6, LOG2G, 24>;
+        case 13824: return (const void*)qmv_rows_long_ragged_kernel<DT, 7, LOG2G, 48>;
+        case 18944: return (const void*)qmv_rows_long_ragged_kernel<DT, 10, LOG2G, 16>;
+        case 27648: return (const void*)qmv_rows_long_ragged_kernel<DT, 14, LOG2G, 32>;
+        default: return nullptr;
+    }
+}
 template <int DT> static const void* rows_long_fn(int bits, int ch, uint32_t G) {
     return G == 32 ? rows_long_fn_g<DT, 5>(bits, ch) : G == 64 ? rows_long_fn_g<DT, 6>(bits, ch) : rows_long_fn_g<DT, 7>(bits, ch);
 }
@@ -590,12 +631,13 @@ template <int DT, int GM> static const void* rows_long_routed_fn(int ch) {   // 
 }
 
 int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
-    if (!qmv_rows_takes(p)) return fail(ERR_UNSUPPORTED, "qmv rows kernels: one activation row, 2- or 4-bit codes, f16 / bf16, rows of 4096, 8192, 14336 or 16384 codes");
+    if (!qmv_rows_takes(p)) return fail(ERR_UNSUPPORTED, "qmv rows kernels: one activation row, 2- or 4-bit codes, f16 / bf16, rows of 4096, 8192, 14336, 16384 or 28672 codes or one of the other lengths it is built for");
     const bool routed = p.gather != GATHER_NONE;
     const uint32_t slots = routed && p.gather != GATHER_SINGLE ? (p.T < p.E ? p.T : p.E) : 1u;   // the experts that can have a row
     if (p.bits == 4 && p.group_size == 64 && p.K == 4096)
         return launch_rows(p.dtype, p.w, p.scales, p.biases, p.x, p.out, p.N, 0, nullptr, lc, p.gather, p.route, p.E, p.T, slots);
-    const int ch = rows_long_ch(p);
+    int tail = 0;
+    const int ch = rows_long_ch(p, &tail);
     QmvRowsLArgs a{(const rp_u32x4*)p.w, (const uint16_t*)p.scales, (const uint16_t*)p.biases, (const uint16_t*)p.x, (uint16_t*)p.out, p.N, p.route, p.E, p.T};
     void* args[] = {&a};
     const void* fn = p.gather == GATHER_CSR       ? (p.dtype == DT_BF16 ? rows_long_routed_fn<DT_BF16, GATHER_CSR>(ch) : rows_long_routed_fn<DT_F16, GATHER_CSR>(ch))
@@ -603,6 +645,9 @@ int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
                      : p.gather == GATHER_SINGLE  ? (p.dtype == DT_BF16 ? rows_long_routed_fn<DT_BF16, GATHER_SINGLE>(ch) : rows_long_routed_fn<DT_F16, GATHER_SINGLE>(ch))
                      : p.dtype == DT_BF16         ? rows_long_fn<DT_BF16>(p.bits, ch, p.group_size)
                                                   : rows_long_fn<DT_F16>(p.bits, ch, p.group_size);
+    if (p.gather == GATHER_NONE && p.bits == 4 && p.K != 8192 && p.K != 14336 && p.K != 28672)   // the other models' row lengths
+        fn = p.dtype == DT_BF16 ? (p.group_size == 64 ? rows_long_more_fn<DT_BF16, 6>(p.K) : p.group_size == 128 ? rows_long_more_fn<DT_BF16, 7>(p.K) : nullptr)
+                                : (p.group_size == 64 ? rows_long_more_fn<DT_F16, 6>(p.K) : p.group_size == 128 ? rows_long_more_fn<DT_F16, 7>(p.K) : nullptr);
     if (!fn) return fail(ERR_UNSUPPORTED, "qmv rows kernels: no instance for this row length and group size");
     // Sixteen rows per workgroup, eight for the long rows. One workgroup of sixteen per compute unit (4096 x 14336: 256
     // of them) is the fastest form on some machines of the pool and 9 % behind on others, where the same launch as 512
@@ -611,6 +656,7 @@ int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
     // From 8192 rows on (two or more workgroups of sixteen per compute unit) sixteen are ahead again: 8192 x 14336 13.2 ->
     // 12.65 us, 14336 x 14336 21.25 -> 20.35. (28672 codes: 896 chunks to prepare, always sixteen.)
     const uint32_t block = ch > 8 || (ch == 7 && p.N >= 8192u) ? 1024u : ch > 4 ? 512u : 1024u;
+    (void)tail;
     if (block < 64u * (uint32_t)ch) return fail(ERR_UNSUPPORTED, "qmv rows kernels: workgroup smaller than the row's chunks");   // (thread t prepares chunk t)
     hipError_t e = launch_kernel(fn, dim3((p.N + block / 64u - 1u) / (block / 64u), slots), dim3(block), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "qmv long rows kernel launch");

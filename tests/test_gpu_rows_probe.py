@@ -70,12 +70,18 @@ def test_rows_probe_matches_oracle(oracle, N):
 @pytest.mark.parametrize("dt_name", ["F16", "BF16"])
 @pytest.mark.parametrize("bits,G,N,K", [(2, 32, 50, 8192), (2, 64, 1, 8192), (2, 128, 8192, 8192), (2, 64, 33, 16384), (2, 32, 8192, 8192),
                                         (4, 32, 50, 8192), (4, 64, 8192, 8192), (4, 128, 17, 8192), (4, 128, 40, 14336),
-                                        (4, 64, 33, 28672), (4, 128, 1030, 28672)])
+                                        (4, 64, 33, 28672), (4, 128, 1030, 28672),
+                                        # the row lengths of other models: whole groups of 64 chunks (10240, 12288, 18432 codes)
+                                        # and the last group partly filled (11008: 24 of 64, 13824: 48, 18944: 16, 27648: 32)
+                                        (4, 64, 1030, 10240), (4, 128, 33, 12288), (4, 64, 515, 18432), (4, 64, 4100, 11008), (4, 128, 19, 11008),
+                                        (4, 64, 5120, 13824), (4, 128, 1, 13824), (4, 64, 3584, 18944), (4, 128, 50, 18944), (4, 64, 1027, 27648),
+                                        (4, 128, 16, 27648)])
 def test_one_row_per_wave_kernel_other_widths_and_groups(oracle, dt_name, bits, G, N, K):
     """The one-row-per-wave kernel on the shapes it takes beyond the two of the headline: 2-bit codes (made operands in
     place, with an offset that depends on the crumb's position) and 4-bit codes in groups of 32 / 64 / 128 on rows of
-    8192, 14336, 16384 (2-bit) and 28672 codes (the last with eight groups of the bias term per lane), forced with
-    qmv.kernel = 3, ragged last workgroups, behind a cache flush, against the f64 oracle on full-range codes."""
+    8192, 14336, 16384 (2-bit) and 28672 codes (the last with eight groups of the bias term per lane), and 4-bit codes in
+    groups of 64 / 128 on the row lengths of other models, forced with qmv.kernel = 3, ragged last workgroups, behind a
+    cache flush, against the f64 oracle on full-range codes."""
     import metaltile_amd as m
     from metaltile_amd import DType, GpuBuffer, ops, _lib
     from metaltile_amd.synth import make_case
@@ -88,7 +94,7 @@ def test_one_row_per_wave_kernel_other_widths_and_groups(oracle, dt_name, bits, 
     assert lib.mtq_set_option(b"qmv.kernel", 3) == 0
     try:
         name = ops.plan("qmv", dt, bits, G, 1, N, K)[1][0][0]
-        assert "qmv_rows_long_kernel" in name, name
+        assert "qmv_rows_long_kernel" in name or "qmv_rows_long_ragged_kernel" in name, name
         m.GpuRunner(0).flush_slc()
         ops.qmv(dt, bits, G, bw, bs, bb, bx, out, 1, N, K)
     finally:
@@ -109,7 +115,7 @@ def test_shapes_the_one_row_per_wave_kernel_refuses():
     lib = _lib.load()
     assert lib.mtq_set_option(b"qmv.kernel", 3) == 0
     try:
-        for bits, G, K in ((4, 32, 14336), (8, 64, 8192), (4, 64, 11008), (2, 16, 8192), (4, 64, 2048), (3, 64, 8192), (4, 32, 28672), (2, 32, 16384), (4, 64, 16384),
+        for bits, G, K in ((4, 32, 14336), (8, 64, 8192), (4, 32, 11008), (4, 64, 9216), (2, 16, 8192), (4, 64, 2048), (3, 64, 8192), (4, 32, 28672), (2, 32, 16384), (4, 64, 16384),
                            (4, 64, 57344)):
             rc, launches, _, _ = ops.plan("qmv", DType.F16, bits, G, 1, 4096, K)
             assert rc == 0 and "qmv_rows" not in launches[0][0], (bits, G, K, launches[0][0])

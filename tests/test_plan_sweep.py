@@ -144,6 +144,12 @@ def test_benchmark_configurations_are_routed_as_documented():
     assert "qmv_rows_walk_kernel<1, 3, 7, 16>" in ks[0] and ls[0][1][0] == 256 and ls[0][2][0] == 1024
     ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 4096, 14336)
     assert "qmv_rows_long_kernel<2, 4, 7, 6>" in ks[0] and ls[0][1][0] == 512 and ls[0][2][0] == 512   # workgroups of eight rows
+    ks, ls = kernels("qmv", DType.BF16, 4, 64, 1, 4096, 11008)      # a long row that ends inside a group of 64 chunks
+    assert "qmv_rows_long_ragged_kernel<2, 6, 6, 24>" in ks[0] and ls[0][1][0] == 512 and ls[0][2][0] == 512
+    ks, ls = kernels("qmv", DType.F16, 4, 128, 1, 3584, 18944)
+    assert "qmv_rows_long_ragged_kernel<1, 10, 7, 16>" in ks[0] and ls[0][1][0] == 224 and ls[0][2][0] == 1024
+    ks, _ = kernels("qmv", DType.BF16, 4, 64, 1, 5120, 27648)       # built, level with the kernel that serves it, not routed
+    assert "qmv_rows" not in ks[0]
     for bits, G, name in ((2, 32, "qmv_rows_walk2_kernel<1, 2, 5, 8>"), (2, 128, "qmv_rows_walk2_kernel<1, 2, 7, 8>"), (4, 64, "qmv_rows_long_kernel<1, 4, 4, 6>")):   # the one-row cells of the width / group sweep
         ks, ls = kernels("qmv", DType.F16, bits, G, 1, 8192, 8192)
         assert name in ks[0] and ls[0][1][0] == 512, ks
