@@ -419,7 +419,7 @@ MTQ_API int mtq_flush_cache(void);
  *   "qmv.kernel"           0 = choose per shape (default), 1 = one-shot kernel, 2 = streaming kernel, 3 = the wave-per-four-rows /
  *                          wave-per-row kernels wherever they apply (2- and 4-bit codes, f16 / bf16), 4 = the kernel whose
  *                          waves walk the rows wherever it applies (one row of x, rows of 2048 to 8192 4-bit codes in steps of 1024, or 3584, in
- *                          groups of 32 / 64 / 128, f16 / bf16; also the batched form of mtq_qmv_batched, rows of 4096 / 8192)
+ *                          groups of 32 / 64 / 128, f16 / bf16; also the batched form of mtq_qmv_batched)
  *   "qmv.rows_per_thread"  one-shot kernel: 0 = choose per shape, or 4 / 7 / 8
  *   "qmv.stream_depth"     streaming kernel: 0 = choose per shape, or 4 / 8 loads in flight per thread
  *   "qmv.stream_batches"   streaming kernel: 0 = choose per shape, or 1..16 batches per thread

@@ -445,14 +445,22 @@ static int op_rms_norm_qmv(int dtype, int bits, uint32_t G, const void* x, const
     // 4-bit f16 / bf16: the norm applied as the matrix-core GEMV stages its row (two staged rows share one set of 4;
     // no per-workgroup renormalisation beyond the sum of squares). us, streaming kernel -> this: 14336 x 4096 12.6 ->
     // 10.6, 6144 x 4096 8.1 -> 7.3; it loses on short matrices and long rows (4096 x 4096 6.2 -> 6.4, 4096 x 14336 13.7 -> 14.1).
-    // Rows of 4096 / 8192 4-bit codes: the norm applied as the kernel whose waves walk the rows puts the activations into
+    // Rows of 2048 ... 8192 4-bit codes: the norm applied as the kernel whose waves walk the rows puts the activations into
     // LDS (qmv_rows_walk.hip). bf16, us, the better of the forms below -> this, same run: 1024 / 2048 / 4096 / 6144 / 8192 / 14336 /
     // 28672 x 4096 4.65 -> 4.41, 4.75 -> 4.42, 6.52 -> 4.57, 7.37 -> 5.90, 7.57 -> 6.93, 10.61 -> 8.91, 16.76 -> 15.79; 2048 / 4096 /
     // 6144 / 8192 / 14336 / 20480 / 28672 x 8192 6.81 -> 6.19, 8.73 -> 7.09, 11.01 -> 9.79, 11.73 -> 11.59, 17.17 -> 16.05, 22.28 -> 20.75,
     // 27.51 -> 26.48. On the largest matrices the matrix-core form is level or ahead (65536 x 4096 29.0 / 29.4 - 32.2, 65536 x 8192
     // 52.2 / 52.9 - 54.3). qmv.kernel = 2 keeps the older forms, = 3 takes this one wherever the shape allows.
+    // The other row lengths it is built for (2048 / 3072 / 3584 / 5120 / 6144 / 7168 codes; bf16 g64, us, the forms below -> this):
+    // 2048 codes, 2048 / 8192 / 16384 / 32768 rows 4.96 -> 4.51, 6.59 -> 5.04, 8.49 -> 6.78, 11.7 -> 10.7; 3072 codes, 512 / 3072 / 8192 /
+    // 28672 rows 12.8 -> 4.15, 13.0 -> 4.61, 7.25 -> 6.88, 15.5 -> 13.8; 3584 codes, 1024 / 3584 / 18944 / 37888 rows 14.3 -> 4.26, 13.6 -> 4.73,
+    // 14.7 -> 10.9, 20.1 -> 17.5; 5120 codes, 1024 / 5120 / 13824 / 27648 rows 12.4 -> 5.09, 9.56 -> 7.14, 13.9 -> 11.0, 19.6 -> 18.2; 6144
+    // codes, 1024 / 6144 / 16384 rows 6.46 -> 5.22, 10.1 -> 7.74, 14.7 -> 14.1; 7168 codes, 2048 / 7168 / 18432 rows 14.2 -> 6.18, 11.0 -> 10.4,
+    // 20.5 -> 18.3 (rows that the streaming kernel does not take whole were a norm launch and a GEMV). From 65536 rows the
+    // forms below are ahead (65536 x 3584 26.1 / 27.5, 65536 x 7168 47.9 / 56.3, 151936 x 2048 32.6 / 38.9).
     const bool rows_norm = options().qmv_kernel == 3 ||
-                           (options().qmv_kernel == 0 && N >= (K == 4096 ? 1024u : 2048u) && N <= 32768u);
+                           (options().qmv_kernel == 0 && ((K == 4096 || K == 8192) ? N >= (K == 4096 ? 1024u : 2048u) && N <= 32768u
+                                                                                     : N >= 512u && N <= 40960u));
     if (options().qmv_norm_mfma != 2 && rows_norm && qmv_rows_norm_takes(p, norm_w)) {
         rc = launch_qmv_rows_norm(p, norm_w, eps, lc);
         if (rc != ERR_UNSUPPORTED) return rc;

@@ -157,7 +157,7 @@ static int launch_qmv_stream(const QmvParams& p, uint32_t C, uint32_t rps, uint3
 
 int launch_qmv_batched(const QmvParams& p0, const QmvBatch& b, const LaunchCtx& lc) {
     if (b.n < 2 || b.n > 4) return fail(ERR_BAD_ARG, "batched qmv takes 2 to 4 matrices");
-    // Rows of 4096 / 8192 4-bit codes: the matrices' rows one after the other on the kernel whose waves walk the rows,
+    // Rows of 2048 ... 8192 4-bit codes: the matrices' rows one after the other on the kernel whose waves walk the rows,
     // sized as the one matrix of all of them would be.
     if ((options().qmv_kernel == 0 && qmv_rows_walk_batched_preferred(p0, b)) || (options().qmv_kernel == 4 && qmv_rows_walk_batched_takes(p0, b))) {
         int rc = launch_qmv_rows_walk_batched(p0, b, lc);

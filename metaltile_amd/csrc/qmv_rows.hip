@@ -50,7 +50,7 @@ template <bool TL> __device__ __forceinline__ void rp_stamp(uint64_t (&st)[MTQ_R
 template <int DT, int MODE, bool TL, int GM>
 __device__ __forceinline__ void qmv_rows_body(const QmvRowsArgs& a) {
     static_assert(GM == GATHER_NONE || (MODE == 0 && !TL), "routed instances are product instances");
-    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;
+    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 64.0f;
     constexpr int GPR = 64, C = 128, R = 4;
     uint64_t st[MTQ_ROWS_PROBE_STAMPS];
     rp_stamp<TL>(st, 0);                                  // wave started
@@ -99,7 +99,7 @@ __device__ __forceinline__ void qmv_rows_body(const QmvRowsArgs& a) {
     const bool j0 = lane & 1u, j1 = lane & 2u;
     uint32_t xp[2][16];
     float gsum = 0.f;
-    uint32_t kor = DT == DT_BF16 ? 0x43004300u : 0x64006400u;   // (2^7, 2^7) in bf16, (2^10, 2^10) in f16: a code OR-ed into the mantissa is MAGIC + q
+    uint32_t kor = DT == DT_BF16 ? 0x43004300u : 0x54005400u;   // (2^7, 2^7) in bf16, a code OR-ed into mantissa bits 0-3; (2^6, 2^6) in f16, a code in mantissa bits 4-7: MAGIC + q
     asm volatile("" : "+v"(kor));
     if constexpr (MODE == 0) {
         rp_u32x2 ones;
@@ -143,10 +143,17 @@ __device__ __forceinline__ void qmv_rows_body(const QmvRowsArgs& a) {
                 for (int i = 0; i < 2; i++) {
                     const uint32_t w = wv[r][i][q];
                     rp_u32x2 b0, b1, a0, a1;
-                    b0.x = (w & 0x000F000Fu) | kor;
-                    b0.y = ((w >> 4) & 0x000F000Fu) | kor;
-                    b1.x = ((w >> 8) & 0x000F000Fu) | kor;
-                    b1.y = ((w >> 12) & 0x000F000Fu) | kor;
+                    if constexpr (DT == DT_BF16) {
+                        b0.x = (w & 0x000F000Fu) | kor;
+                        b0.y = ((w >> 4) & 0x000F000Fu) | kor;
+                        b1.x = ((w >> 8) & 0x000F000Fu) | kor;
+                        b1.y = ((w >> 12) & 0x000F000Fu) | kor;
+                    } else {   // (f16: the codes into mantissa bits 4-7, where the second nibble already is)
+                        b0.x = ((w << 4) & 0x00F000F0u) | kor;
+                        b0.y = (w & 0x00F000F0u) | kor;
+                        b1.x = ((w >> 4) & 0x00F000F0u) | kor;
+                        b1.y = ((w >> 8) & 0x00F000F0u) | kor;
+                    }
                     a0.x = xp[i][4 * q + 0]; a0.y = xp[i][4 * q + 1];
                     a1.x = xp[i][4 * q + 2]; a1.y = xp[i][4 * q + 3];
                     if (i == 0) { d0 = rp_mfma<DT>(a0, b0, d0); d0 = rp_mfma<DT>(a1, b1, d0); }
@@ -232,7 +239,7 @@ template <int DT, int BITS, int CH, int LOG2G, int GM, int TAIL = 0>
 __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
     static_assert(BITS == 2 || BITS == 4, "2- or 4-bit codes");
     static_assert(TAIL == 0 || (TAIL > 0 && TAIL < 64 && TAIL % 4 == 0 && BITS == 4 && GM == GATHER_NONE), "ragged rows: 4-bit codes, unrouted, whole 4-lane blocks");
-    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;   // 4-bit codes: one offset for every pair
+    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 64.0f;   // 4-bit codes: one offset for every pair
     constexpr int CPC = 128 / BITS;        // codes per chunk
     constexpr int Q = CPC / 8;             // 16-byte quarters of a chunk's activations in operand order (4 pair dwords each)
     constexpr int C = TAIL ? 64 * (CH - 1) + TAIL : 64 * CH;   // chunks per row
@@ -311,7 +318,7 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
     const bool j0 = lane & 1u, j1 = lane & 2u;
     // OR-constants in registers the optimiser cannot see through (an and-or then has one literal operand, its mask)
     uint32_t kor[BITS == 2 ? (DT == DT_F16 ? 5 : 3) : 1];
-    if constexpr (BITS == 4) kor[0] = DT == DT_BF16 ? 0x43004300u : 0x64006400u;
+    if constexpr (BITS == 4) kor[0] = DT == DT_BF16 ? 0x43004300u : 0x54005400u;
     else {
 #pragma unroll
         for (int p = 0; p < (DT == DT_F16 ? 5 : 3); p++) kor[p] = rp_crumb_kor<DT>(p);
@@ -430,10 +437,17 @@ __device__ __forceinline__ void qmv_rows_long_body(const QmvRowsLArgs& a) {
             if constexpr (BITS == 4) {
                 const uint4 xo = *(const uint4*)xp_lds[d][TAIL && i == CH - 1 ? min((uint32_t)(i * 64) + lane, (uint32_t)(C - 1)) : (uint32_t)(i * 64) + lane];
                 rp_u32x2 b0, b1, a0, a1;
-                b0.x = (w & 0x000F000Fu) | kor[0];
-                b0.y = ((w >> 4) & 0x000F000Fu) | kor[0];
-                b1.x = ((w >> 8) & 0x000F000Fu) | kor[0];
-                b1.y = ((w >> 12) & 0x000F000Fu) | kor[0];
+                if constexpr (DT == DT_BF16) {
+                    b0.x = (w & 0x000F000Fu) | kor[0];
+                    b0.y = ((w >> 4) & 0x000F000Fu) | kor[0];
+                    b1.x = ((w >> 8) & 0x000F000Fu) | kor[0];
+                    b1.y = ((w >> 12) & 0x000F000Fu) | kor[0];
+                } else {   // (f16: the codes into mantissa bits 4-7, where the second nibble already is)
+                    b0.x = ((w << 4) & 0x00F000F0u) | kor[0];
+                    b0.y = (w & 0x00F000F0u) | kor[0];
+                    b1.x = ((w >> 4) & 0x00F000F0u) | kor[0];
+                    b1.y = ((w >> 8) & 0x00F000F0u) | kor[0];
+                }
                 a0.x = xo.x; a0.y = xo.y;
                 a1.x = xo.z; a1.y = xo.w;
                 dh[d >> HSH] = rp_mfma<DT>(a0, b0, dh[d >> HSH]);

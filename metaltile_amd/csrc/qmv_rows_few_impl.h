@@ -72,7 +72,7 @@ template <int DT, int BITS, int T, int LOG2G, bool TL = false>
 __global__ __launch_bounds__(1024) void qmv_rows_few_kernel(QmvRowsFArgs a) {
     static_assert(BITS == 2 || BITS == 4, "2- or 4-bit codes");
     using Geo = RowsFewGeom<BITS, T, LOG2G>;
-    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;   // 4-bit codes: one offset for every pair
+    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 64.0f;   // 4-bit codes: one offset for every pair
     constexpr int CPC = Geo::CPC, Q = Geo::Q, C = Geo::C, K = Geo::K, GPR = Geo::GPR, SPG = Geo::SPG, NH = Geo::NH, SP = Geo::SP;
     uint64_t st[ROWS_FEW_STAMPS];
     auto stamp = [&](int i) {
@@ -150,7 +150,7 @@ __global__ __launch_bounds__(1024) void qmv_rows_few_kernel(QmvRowsFArgs a) {
     const bool j0 = lane & 1u, j1 = lane & 2u;
     // OR-constants in registers the optimiser cannot see through (an and-or then has one literal operand, its mask)
     uint32_t kor[BITS == 2 ? (DT == DT_F16 ? 5 : 3) : 1];
-    if constexpr (BITS == 4) kor[0] = DT == DT_BF16 ? 0x43004300u : 0x64006400u;
+    if constexpr (BITS == 4) kor[0] = DT == DT_BF16 ? 0x43004300u : 0x54005400u;
     else {
 #pragma unroll
         for (int p = 0; p < (DT == DT_F16 ? 5 : 3); p++) kor[p] = rp_crumb_kor<DT>(p);
@@ -281,10 +281,17 @@ __global__ __launch_bounds__(1024) void qmv_rows_few_kernel(QmvRowsFArgs a) {
             if constexpr (BITS == 4) {
                 const uint4 xo = xp[((uint32_t)(d * C) + c) * 4u + j];
                 rp_u32x2 b0, b1, a0, a1;
-                b0.x = (w & 0x000F000Fu) | kor[0];
-                b0.y = ((w >> 4) & 0x000F000Fu) | kor[0];
-                b1.x = ((w >> 8) & 0x000F000Fu) | kor[0];
-                b1.y = ((w >> 12) & 0x000F000Fu) | kor[0];
+                if constexpr (DT == DT_BF16) {
+                    b0.x = (w & 0x000F000Fu) | kor[0];
+                    b0.y = ((w >> 4) & 0x000F000Fu) | kor[0];
+                    b1.x = ((w >> 8) & 0x000F000Fu) | kor[0];
+                    b1.y = ((w >> 12) & 0x000F000Fu) | kor[0];
+                } else {   // (f16: the codes into mantissa bits 4-7, where the second nibble already is)
+                    b0.x = ((w << 4) & 0x00F000F0u) | kor[0];
+                    b0.y = (w & 0x00F000F0u) | kor[0];
+                    b1.x = ((w >> 4) & 0x00F000F0u) | kor[0];
+                    b1.y = ((w >> 8) & 0x00F000F0u) | kor[0];
+                }
                 a0.x = xo.x; a0.y = xo.y;
                 a1.x = xo.z; a1.y = xo.w;
                 dh[d >> HSH] = rp_mfma<DT>(a0, b0, dh[d >> HSH]);

@@ -64,8 +64,8 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     static_assert(BITS == 4 || (BITS == 2 && !NORM && !BATCH), "4-bit codes; 2-bit codes on the plain walk");
     constexpr bool ROUTED = GM != GATHER_NONE;
     static_assert(!ROUTED || (!NORM && !BATCH && BITS == 4), "routed rows: the plain walk on 4-bit codes");
-    static_assert(TAIL == 0 || (TAIL > 0 && TAIL < 64 && TAIL % 16 == 0 && BITS == 4 && !NORM && !BATCH && !ROUTED), "ragged rows: the plain walk on 4-bit codes, whole 4-lane blocks");
-    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 1024.0f;   // 4-bit codes: one offset for every pair
+    static_assert(TAIL == 0 || (TAIL > 0 && TAIL < 64 && TAIL % 16 == 0 && BITS == 4 && !ROUTED), "ragged rows: 4-bit codes, unrouted, whole 4-lane blocks");
+    constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 64.0f;   // 4-bit codes: one offset for every pair
     constexpr float REM = 1.0f / RemSplit<DT>::kRemScale;
     constexpr int CPC = 128 / BITS, Q = CPC / 8;   // codes per 16-byte chunk; 16-byte quarters of a chunk's activations in operand order
     constexpr int C = TAIL ? 64 * (CH - 1) + TAIL : 64 * CH, K = C * CPC;   // chunks and codes per row
@@ -152,7 +152,9 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     load_row(min(gw, last), bufA);   // (idle waves of a short launch load the last row and store nothing)
     RP_KEEP_ORDER();
     const bool j0 = lane & 1u, j1 = lane & 2u;
-    uint32_t kor = DT == DT_BF16 ? 0x43004300u : 0x64006400u;   // (2^7, 2^7) in bf16, (2^10, 2^10) in f16: a code OR-ed into the mantissa is MAGIC + q
+    // (2^7, 2^7) in bf16, a code OR-ed into mantissa bits 0-3; (2^6, 2^6) in f16, a code in mantissa bits 4-7 (where the second nibble
+    // already is: the same three shifts per dword as for bits 0-3, and a sixteenth of the offset that the f32 sums carry): MAGIC + q
+    uint32_t kor = DT == DT_BF16 ? 0x43004300u : 0x54005400u;
     asm volatile("" : "+v"(kor));
     // 2-bit codes: a pair of crumbs masked where it sits (bit 2 p) and OR-ed into 2^(MB - 2 p) is that power of two
     // plus the code (qmv_rows_common.h); one constant per position class, kept opaque so that an and-or has one literal
@@ -284,12 +286,19 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
                     const uint32_t w = r.wv[i][d];
                     const uint4 xo = *(const uint4*)xp_lds[d][TAIL && i == CH - 1 ? min((uint32_t)(i * 64) + ln, (uint32_t)(C - 1)) : (uint32_t)(i * 64) + ln];
                     uint4 xl = make_uint4(0u, 0u, 0u, 0u);
-                    if constexpr (NORM) xl = *(const uint4*)xl_lds[d][i * 64 + ln];
+                    if constexpr (NORM) xl = *(const uint4*)xl_lds[d][TAIL && i == CH - 1 ? min((uint32_t)(i * 64) + ln, (uint32_t)(C - 1)) : (uint32_t)(i * 64) + ln];
                     rp_u32x2 b0, b1, a0, a1, l0, l1;
-                    b0.x = (w & 0x000F000Fu) | kor;
-                    b0.y = ((w >> 4) & 0x000F000Fu) | kor;
-                    b1.x = ((w >> 8) & 0x000F000Fu) | kor;
-                    b1.y = ((w >> 12) & 0x000F000Fu) | kor;
+                    if constexpr (DT == DT_BF16) {
+                        b0.x = (w & 0x000F000Fu) | kor;
+                        b0.y = ((w >> 4) & 0x000F000Fu) | kor;
+                        b1.x = ((w >> 8) & 0x000F000Fu) | kor;
+                        b1.y = ((w >> 12) & 0x000F000Fu) | kor;
+                    } else {   // (the second nibble is where it has to be)
+                        b0.x = ((w << 4) & 0x00F000F0u) | kor;
+                        b0.y = (w & 0x00F000F0u) | kor;
+                        b1.x = ((w >> 4) & 0x00F000F0u) | kor;
+                        b1.y = ((w >> 8) & 0x00F000F0u) | kor;
+                    }
                     a0.x = xo.x; a0.y = xo.y; a1.x = xo.z; a1.y = xo.w;
                     l0.x = xl.x; l0.y = xl.y; l1.x = xl.z; l1.y = xl.w;
                     dh = rp_mfma<DT>(a0, b0, dh);
@@ -397,6 +406,9 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
 template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_kernel(QmvRowsNArgs a) {
     qmv_rows_walk_body<DT, CH, LOG2G, NWV, true>(a);
 }
+template <int DT, int CH, int LOG2G, int NWV, int TAIL> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_norm_ragged_kernel(QmvRowsNArgs a) {
+    qmv_rows_walk_body<DT, CH, LOG2G, NWV, true, false, 4, GATHER_NONE, TAIL>(a);   // (rows that end inside a group of 64 chunks)
+}
 // The same walk without the norm: out[n] = sum_k (s q + b)[n, k] x[k], the activations as they are (one operand set).
 template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_walk_kernel(QmvRowsNArgs a) {
     qmv_rows_walk_body<DT, CH, LOG2G, NWV, false>(a);
@@ -424,15 +436,25 @@ template <int DT, int CH, int LOG2G, int NWV> __global__ __launch_bounds__(64 * 
     qmv_rows_walk_body<DT, CH, LOG2G, NWV, false, true>(a);
 }
 
-// 4-bit codes, rows of 4096 or 8192 codes, groups of 32 / 64 / 128, f16 / bf16
+// 4-bit codes, rows of 2048 ... 8192 codes in steps of 1024 or 3584, groups of 32 / 64 / 128, f16 / bf16
 bool qmv_rows_norm_takes(const QmvParams& p, const void* norm_w) {
-    if ((p.dtype != DT_F16 && p.dtype != DT_BF16) || p.bits != 4 || p.N == 0 || p.N > (1u << 24) || (p.K != 4096 && p.K != 8192)) return false;   // (row numbers plus the launch's waves stay below 2^32)
+    if ((p.dtype != DT_F16 && p.dtype != DT_BF16) || p.bits != 4 || p.N == 0 || p.N > (1u << 24)) return false;   // (row numbers plus the launch's waves stay below 2^32)
+    if (p.K != 3584 && (p.K < 2048 || p.K > 8192 || p.K % 1024)) return false;
     const uint32_t G = p.group_size;
     if (G != 32 && G != 64 && G != 128) return false;
     return !((uintptr_t)p.w % 16 || (uintptr_t)p.x % 16 || (uintptr_t)norm_w % 16 || (uintptr_t)p.scales % 8 || (uintptr_t)p.biases % 8 || (uintptr_t)p.out % 2);
 }
 
+template <int DT, int CH, int LOG2G, int NWV, int TAIL> __global__ __launch_bounds__(64 * NWV, 4) void qmv_rows_walk_batched_ragged_kernel(QmvRowsNArgs a) {
+    qmv_rows_walk_body<DT, CH, LOG2G, NWV, false, true, 4, GATHER_NONE, TAIL>(a);   // (rows that end inside a group of 64 chunks)
+}
 template <int DT, int LOG2G> static const void* rows_walk_batched_fn(uint32_t K, bool sixteen) {
+    if (K == 2048) return sixteen ? (const void*)qmv_rows_walk_batched_kernel<DT, 1, LOG2G, 16> : (const void*)qmv_rows_walk_batched_kernel<DT, 1, LOG2G, 8>;
+    if (K == 6144) return sixteen ? (const void*)qmv_rows_walk_batched_kernel<DT, 3, LOG2G, 16> : (const void*)qmv_rows_walk_batched_kernel<DT, 3, LOG2G, 8>;
+    if (K == 3072) return sixteen ? (const void*)qmv_rows_walk_batched_ragged_kernel<DT, 2, LOG2G, 16, 32> : (const void*)qmv_rows_walk_batched_ragged_kernel<DT, 2, LOG2G, 8, 32>;
+    if (K == 3584) return sixteen ? (const void*)qmv_rows_walk_batched_ragged_kernel<DT, 2, LOG2G, 16, 48> : (const void*)qmv_rows_walk_batched_ragged_kernel<DT, 2, LOG2G, 8, 48>;
+    if (K == 5120) return sixteen ? (const void*)qmv_rows_walk_batched_ragged_kernel<DT, 3, LOG2G, 16, 32> : (const void*)qmv_rows_walk_batched_ragged_kernel<DT, 3, LOG2G, 8, 32>;
+    if (K == 7168) return sixteen ? (const void*)qmv_rows_walk_batched_ragged_kernel<DT, 4, LOG2G, 16, 32> : (const void*)qmv_rows_walk_batched_ragged_kernel<DT, 4, LOG2G, 8, 32>;
     if (sixteen) return K == 4096 ? (const void*)qmv_rows_walk_batched_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_walk_batched_kernel<DT, 4, LOG2G, 16>;
     return K == 4096 ? (const void*)qmv_rows_walk_batched_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_walk_batched_kernel<DT, 4, LOG2G, 8>;
 }
@@ -447,6 +469,12 @@ template <int DT, int GM> static const void* rows_walk_routed_fn(uint32_t K) {  
 
 template <int DT, int LOG2G, bool NORM> static const void* rows_walk_fn(uint32_t K, bool sixteen) {
     if constexpr (NORM) {
+        if (K == 2048) return sixteen ? (const void*)qmv_rows_norm_kernel<DT, 1, LOG2G, 16> : (const void*)qmv_rows_norm_kernel<DT, 1, LOG2G, 8>;
+        if (K == 6144) return sixteen ? (const void*)qmv_rows_norm_kernel<DT, 3, LOG2G, 16> : (const void*)qmv_rows_norm_kernel<DT, 3, LOG2G, 8>;
+        if (K == 3072) return sixteen ? (const void*)qmv_rows_norm_ragged_kernel<DT, 2, LOG2G, 16, 32> : (const void*)qmv_rows_norm_ragged_kernel<DT, 2, LOG2G, 8, 32>;
+        if (K == 3584) return sixteen ? (const void*)qmv_rows_norm_ragged_kernel<DT, 2, LOG2G, 16, 48> : (const void*)qmv_rows_norm_ragged_kernel<DT, 2, LOG2G, 8, 48>;
+        if (K == 5120) return sixteen ? (const void*)qmv_rows_norm_ragged_kernel<DT, 3, LOG2G, 16, 32> : (const void*)qmv_rows_norm_ragged_kernel<DT, 3, LOG2G, 8, 32>;
+        if (K == 7168) return sixteen ? (const void*)qmv_rows_norm_ragged_kernel<DT, 4, LOG2G, 16, 32> : (const void*)qmv_rows_norm_ragged_kernel<DT, 4, LOG2G, 8, 32>;
         if (sixteen) return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 16>;
         return K == 4096 ? (const void*)qmv_rows_norm_kernel<DT, 2, LOG2G, 8> : (const void*)qmv_rows_norm_kernel<DT, 4, LOG2G, 8>;
     } else {
@@ -529,7 +557,7 @@ template <bool NORM> static int launch_rows_walk(const QmvParams& p, const void*
 }
 
 int launch_qmv_rows_norm(const QmvParams& p, const void* norm_w, const float* eps, const LaunchCtx& lc) {
-    if (!qmv_rows_norm_takes(p, norm_w) || !eps) return fail(ERR_UNSUPPORTED, "norm + qmv rows kernel: 4-bit codes, rows of 4096 or 8192 codes, f16 / bf16");
+    if (!qmv_rows_norm_takes(p, norm_w) || !eps) return fail(ERR_UNSUPPORTED, "norm + qmv rows kernel: 4-bit codes, rows of 2048 to 8192 codes in steps of 1024 (and 3584), f16 / bf16");
     return launch_rows_walk<true>(p, norm_w, eps, lc);
 }
 
@@ -543,18 +571,13 @@ bool qmv_rows_walk_takes(const QmvParams& p) {
         if (!p.route || p.E == 0 || p.bits != 4 || p.group_size != 64) return false;
         if (p.gather != GATHER_SINGLE && (p.E > 64 || p.T == 0 || p.T > 64)) return false;
         if (((size_t)p.N * (p.K / 64u) * 2u) % 8u) return false;
-        return qmv_rows_norm_takes(p, p.x);
+        return (p.K == 4096 || p.K == 8192) && qmv_rows_norm_takes(p, p.x);
     }
     if (p.M != 1) return false;
     if (p.bits == 2) {   // rows of 8192 2-bit codes: the 4-bit instance's conditions on a matrix of that width
         QmvParams q = p;
         q.bits = 4;
         return p.K == 8192 && qmv_rows_norm_takes(q, p.x);
-    }
-    if (p.K == 2048 || p.K == 6144 || p.K == 3072 || p.K == 3584 || p.K == 5120 || p.K == 7168) {   // one matrix of 4-bit codes also in these row lengths: everything else as for 4096
-        QmvParams q = p;
-        q.K = 4096;
-        return qmv_rows_norm_takes(q, p.x);
     }
     return qmv_rows_norm_takes(p, p.x);   // (the alignment of x stands in for that of the norm weights)
 }
@@ -603,7 +626,7 @@ bool qmv_rows_walk_preferred(const QmvParams& p) {
 
 // The batch on one walk: every matrix as the single one would have to be, the rows counted together.
 static bool rows_walk_batch_as_one(const QmvParams& p0, const QmvBatch& b, QmvParams& p) {
-    if (b.n < 2 || b.n > 4 || p0.bits != 4 || (p0.K != 4096 && p0.K != 8192)) return false;
+    if (b.n < 2 || b.n > 4 || p0.bits != 4) return false;
     p = p0;
     p.gather = GATHER_NONE;
     p.M = 1;
@@ -627,7 +650,7 @@ bool qmv_rows_walk_batched_preferred(const QmvParams& p0, const QmvBatch& b) {
 }
 int launch_qmv_rows_walk_batched(const QmvParams& p0, const QmvBatch& b, const LaunchCtx& lc) {
     QmvParams p;
-    if (!rows_walk_batch_as_one(p0, b, p)) return fail(ERR_UNSUPPORTED, "qmv walking rows kernel: 2 to 4 matrices of 4-bit codes, rows of 4096 or 8192 codes, f16 / bf16");
+    if (!rows_walk_batch_as_one(p0, b, p)) return fail(ERR_UNSUPPORTED, "qmv walking rows kernel: 2 to 4 matrices of 4-bit codes, rows of 2048 to 8192 codes in steps of 1024 (and 3584), f16 / bf16");
     return launch_rows_walk<false>(p, nullptr, nullptr, lc, &b);
 }
 

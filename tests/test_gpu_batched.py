@@ -50,9 +50,9 @@ def _expected(oracle, c, x_f, dt):
 
 
 def _walks(dt, bits, G, K, Ns):
-    """What the kernel whose waves walk the rows takes of a batch: 2 to 4 matrices of 4-bit codes in rows of 4096 / 8192
-    codes, groups of 32 / 64 / 128, f16 / bf16."""
-    return bits == 4 and K in (4096, 8192) and G in (32, 64, 128) and dt != DType.F32 and 2 <= len(Ns) <= 4
+    """What the kernel whose waves walk the rows takes of a batch: 2 to 4 matrices of 4-bit codes in rows of 2048 ... 8192
+    codes in steps of 1024, or 3584, groups of 32 / 64 / 128, f16 / bf16."""
+    return bits == 4 and (K == 3584 or (2048 <= K <= 8192 and K % 1024 == 0)) and G in (32, 64, 128) and dt != DType.F32 and 2 <= len(Ns) <= 4
 
 
 CASES += [
@@ -60,6 +60,11 @@ CASES += [
     (DType.BF16, 4, 128, 8192, (1024, 40)),           # rows of 8192 codes, one row per wave
     (DType.BF16, 4, 64, 8192, (8192, 1024, 1027)),    # 10243 rows of 8192 codes: its automatic size
     (DType.F16, 4, 64, 4096, (16, 16)),               # two waves' worth
+    (DType.BF16, 4, 64, 3072, (3072, 1024, 1030)),    # rows that end inside a group of 64 chunks: Q, K, V of a 3072-wide model
+    (DType.F16, 4, 128, 3584, (3584, 512, 512)),
+    (DType.BF16, 4, 32, 5120, (5120, 1024, 1024, 7)),
+    (DType.BF16, 4, 64, 7168, (1536, 2050)),
+    (DType.F16, 4, 64, 6144, (6144, 1024)),
 ]
 
 
