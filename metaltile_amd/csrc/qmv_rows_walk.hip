@@ -64,7 +64,7 @@ __device__ __forceinline__ void qmv_rows_walk_body(const QmvRowsNArgs& a) {
     static_assert(BITS == 4 || (BITS == 2 && !NORM && !BATCH), "4-bit codes; 2-bit codes on the plain walk");
     constexpr bool ROUTED = GM != GATHER_NONE;
     static_assert(!ROUTED || (!NORM && !BATCH && BITS == 4), "routed rows: the plain walk on 4-bit codes");
-    static_assert(TAIL == 0 || (TAIL > 0 && TAIL < 64 && TAIL % 16 == 0 && BITS == 4 && !ROUTED), "ragged rows: 4-bit codes, unrouted, whole 4-lane blocks");
+    static_assert(TAIL == 0 || (TAIL > 0 && TAIL < 64 && TAIL % 16 == 0 && BITS == 4), "ragged rows: 4-bit codes, whole 4-lane blocks");
     constexpr float MAGIC = DT == DT_BF16 ? 128.0f : 64.0f;   // 4-bit codes: one offset for every pair
     constexpr float REM = 1.0f / RemSplit<DT>::kRemScale;
     constexpr int CPC = 128 / BITS, Q = CPC / 8;   // codes per 16-byte chunk; 16-byte quarters of a chunk's activations in operand order
@@ -463,7 +463,13 @@ template <int DT, int LOG2G> static const void* rows_walk2_fn(bool sixteen) {   
     return sixteen ? (const void*)qmv_rows_walk2_kernel<DT, 2, LOG2G, 16> : (const void*)qmv_rows_walk2_kernel<DT, 2, LOG2G, 8>;
 }
 
+template <int DT, int CH, int LOG2G, int GM, int TAIL> __global__ __launch_bounds__(512, 4) void qmv_rows_walk_routed_ragged_kernel(QmvRowsNArgs a) {
+    qmv_rows_walk_body<DT, CH, LOG2G, 8, false, false, 4, GM, TAIL>(a);   // (rows that end inside a group of 64 chunks)
+}
 template <int DT, int GM> static const void* rows_walk_routed_fn(uint32_t K) {   // groups of 64
+    if (K == 2048) return (const void*)qmv_rows_walk_routed_kernel<DT, 1, 6, GM>;
+    if (K == 5120) return (const void*)qmv_rows_walk_routed_ragged_kernel<DT, 3, 6, GM, 32>;
+    if (K == 7168) return (const void*)qmv_rows_walk_routed_ragged_kernel<DT, 4, 6, GM, 32>;
     return K == 4096 ? (const void*)qmv_rows_walk_routed_kernel<DT, 2, 6, GM> : (const void*)qmv_rows_walk_routed_kernel<DT, 4, 6, GM>;
 }
 
@@ -571,7 +577,7 @@ bool qmv_rows_walk_takes(const QmvParams& p) {
         if (!p.route || p.E == 0 || p.bits != 4 || p.group_size != 64) return false;
         if (p.gather != GATHER_SINGLE && (p.E > 64 || p.T == 0 || p.T > 64)) return false;
         if (((size_t)p.N * (p.K / 64u) * 2u) % 8u) return false;
-        return (p.K == 4096 || p.K == 8192) && qmv_rows_norm_takes(p, p.x);
+        return (p.K == 4096 || p.K == 8192 || p.K == 2048 || p.K == 5120 || p.K == 7168) && qmv_rows_norm_takes(p, p.x);   // (the widths of expert layers it is built for)
     }
     if (p.M != 1) return false;
     if (p.bits == 2) {   // rows of 8192 2-bit codes: the 4-bit instance's conditions on a matrix of that width

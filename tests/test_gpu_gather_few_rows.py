@@ -193,7 +193,9 @@ def forced_qmv_kernel(request):
                          [(20, 4096, "qmv_rows_routed_kernel", 3), (1028, 4096, "qmv_rows_routed_kernel", 3), (19, 14336, "qmv_rows_long_routed_kernel", 3),
                           (1030, 8192, "qmv_rows_long_routed_kernel", 3),
                           # the kernel whose waves walk the rows (qmv.kernel = 4): one row per wave, and 5000 rows so that waves walk
-                          (20, 4096, "qmv_rows_walk_routed_kernel", 4), (5000, 4096, "qmv_rows_walk_routed_kernel", 4), (1030, 8192, "qmv_rows_walk_routed_kernel", 4)],
+                          (20, 4096, "qmv_rows_walk_routed_kernel", 4), (5000, 4096, "qmv_rows_walk_routed_kernel", 4), (1030, 8192, "qmv_rows_walk_routed_kernel", 4),
+                          # the expert widths of other models: 2048 codes, and rows that end inside a group of 64 chunks
+                          (1030, 2048, "qmv_rows_walk_routed_kernel", 4), (40, 7168, "qmv_rows_walk_routed_ragged_kernel", 4), (2050, 5120, "qmv_rows_walk_routed_ragged_kernel", 4)],
                          indirect=["forced_qmv_kernel"])
 def test_routed_rows_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, forced_qmv_kernel):
     """The wave-per-row GEMV kernels with a grid row per expert that has a row (their automatic range is up to four rows
@@ -256,7 +258,8 @@ def test_routed_rows_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, force
 @pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
 @pytest.mark.parametrize("N,K,kernel,forced_qmv_kernel",
                          [(1028, 4096, "qmv_rows_routed_kernel", 3), (40, 14336, "qmv_rows_long_routed_kernel", 3), (1030, 8192, "qmv_rows_long_routed_kernel", 3),
-                          (9000, 4096, "qmv_rows_walk_routed_kernel", 4), (40, 8192, "qmv_rows_walk_routed_kernel", 4)], indirect=["forced_qmv_kernel"])
+                          (9000, 4096, "qmv_rows_walk_routed_kernel", 4), (40, 8192, "qmv_rows_walk_routed_kernel", 4),
+                          (1030, 7168, "qmv_rows_walk_routed_ragged_kernel", 4), (768, 2048, "qmv_rows_walk_routed_kernel", 4)], indirect=["forced_qmv_kernel"])
 def test_single_index_expert_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, forced_qmv_kernel):
     """One row against the expert whose index is read on the device (the reference's expert-indexed GEMV,
     crates/metaltile-std/src/ffai/dequant_gemv_expert_indexed.rs): the first, a middle and the last expert, and an index

@@ -189,8 +189,12 @@ def test_benchmark_configurations_are_routed_as_documented():
         assert "qmv_rows_long_routed_kernel<2, 4, 7, 6, 1>" in ks[0] and ls[0][1][:2] == (512, T) and ls[0][2][0] == 512, ls
     ks, _ = kernels("gather_csr", DType.BF16, 4, 64, 1, 4096, 14336, 8, 5)
     assert "qmv_mfma_kernel<2, 4," in ks[0]
-    ks, ls = kernels("gather_indices", DType.BF16, 4, 64, 1, 2048, 2048, 8, 1)           # other row lengths: the one-row streaming kernel
-    assert "qmv_stream_kernel<2, 4, 1," in ks[0]
+    ks, ls = kernels("gather_indices", DType.BF16, 4, 64, 1, 2048, 2048, 8, 1)           # the expert widths of other models walk too
+    assert "qmv_rows_walk_routed_kernel<2, 1, 6, 2>" in ks[0]
+    ks, ls = kernels("gather_csr", DType.BF16, 4, 64, 1, 2048, 7168, 8, 4)
+    assert "qmv_rows_walk_routed_ragged_kernel<2, 4, 6, 1, 32>" in ks[0] and ls[0][1][:2] == (128, 4), ls
+    ks, ls = kernels("gather_indices", DType.BF16, 4, 64, 1, 2048, 3072, 8, 1)           # other row lengths: the kernels that served them before
+    assert "qmv_rows" not in ks[0]
     ks, _ = kernels("gather_indices", DType.BF16, 4, 64, 1, 14336, 4096, 8, 16)           # 2 rows per expert: 8-row passes
     assert "qmv_mfma_kernel<2, 4," in ks[0]
     for view in ("gather_csr", "gather_indices"):      # fewer rows than experts: a grid row per row, not per expert
