@@ -158,7 +158,9 @@ __device__ __forceinline__ float seg_allreduce(float v, int seg) {
 //
 // Two arithmetic paths:
 //  * dot2 path (f16/bf16 activations, 2- and 4-bit codes): a masked pair of
-//    codes OR-ed into the mantissa of 2^7 (bf16) or 2^10 (f16) is the pair
+//    codes OR-ed into the mantissa of 2^7 (bf16) or 2^10 (f16; 4-bit codes: into
+//    mantissa bits 4-7 of 2^6, where the dword's second nibble already is, so the
+//    f32 sums carry a sixteenth of the offset for the same instructions) is the pair
 //    (MAGIC+q_a, MAGIC+q_b) in element format; v_dot2_f32_{bf16,f16} multiplies
 //    it with the matching activation pair and accumulates in f32. The MAGIC
 //    offset is folded into the bias: s*(dot - MAGIC*sum_x) + b*sum_x =
@@ -168,7 +170,7 @@ __device__ __forceinline__ float seg_allreduce(float v, int seg) {
 
 template <int DT, int BITS> struct PathSel {
     static constexpr bool kDot2 = (DT != DT_F32) && (BITS == 2 || BITS == 4);
-    static constexpr float kMagic = kDot2 ? (DT == DT_BF16 ? 128.0f : 1024.0f) : 0.0f;
+    static constexpr float kMagic = kDot2 ? (DT == DT_BF16 ? 128.0f : BITS == 4 ? 64.0f : 1024.0f) : 0.0f;
 };
 
 template <int DT> __device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float acc) {
@@ -185,9 +187,10 @@ template <int DT> __device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t
     }
 }
 
-// MAGIC pair (2^7 twice in bf16, 2^10 twice in f16) as an opaque VGPR value.
-template <int DT> __device__ __forceinline__ uint32_t magic_or_vgpr() {
-    uint32_t k = DT == DT_BF16 ? 0x43004300u : 0x64006400u;
+// MAGIC pair (2^7 twice in bf16, 2^10 twice in f16; SIXTY_FOUR: 2^6 twice in f16, for codes in mantissa bits 4-7) as an
+// opaque VGPR value.
+template <int DT, bool SIXTY_FOUR = false> __device__ __forceinline__ uint32_t magic_or_vgpr() {
+    uint32_t k = DT == DT_BF16 ? 0x43004300u : SIXTY_FOUR ? 0x54005400u : 0x64006400u;
     asm volatile("" : "+v"(k));
     return k;
 }
@@ -213,7 +216,7 @@ template <int DT, int BITS> struct XSlice<DT, BITS, true> {
         for (int i = 0; i < NRAW; i++) raw[i] = xv[i];
     }
     __device__ __forceinline__ void prepare(const uint4 (&raw)[NRAW]) {
-        kor = magic_or_vgpr<DT>();
+        kor = magic_or_vgpr<DT, BITS == 4>();
         float s01 = 0.f, s23 = 0.f;
         if constexpr (BITS == 4) {
 #pragma unroll
@@ -251,7 +254,7 @@ template <int DT, int BITS> struct XSlice<DT, BITS, true> {
         prepare(raw);
     }
     __device__ __forceinline__ void zero() {
-        kor = magic_or_vgpr<DT>();
+        kor = magic_or_vgpr<DT, BITS == 4>();
 #pragma unroll
         for (int i = 0; i < CPC / 2; i++) xp[i] = 0;
         xsum[0] = xsum[1] = 0.f;
@@ -272,11 +275,16 @@ template <int DT, int BITS> struct XSlice<DT, BITS, true> {
         // the mask as the one scalar/literal operand, (w & mask) | k then fits a
         // single v_and_or_b32 (two literal constants would not).
         const uint32_t kOr = kor;
-        if constexpr (BITS == 4) {
+        if constexpr (BITS == 4 && DT == DT_BF16) {
             acc = dot2_acc<DT>((w & 0x000F000Fu) | kOr, xp[4 * d + 0], acc);
             acc = dot2_acc<DT>(((w >> 4) & 0x000F000Fu) | kOr, xp[4 * d + 1], acc);
             acc = dot2_acc<DT>(((w >> 8) & 0x000F000Fu) | kOr, xp[4 * d + 2], acc);
             acc = dot2_acc<DT>(((w >> 12) & 0x000F000Fu) | kOr, xp[4 * d + 3], acc);
+        } else if constexpr (BITS == 4) {   // f16: the codes into mantissa bits 4-7
+            acc = dot2_acc<DT>(((w << 4) & 0x00F000F0u) | kOr, xp[4 * d + 0], acc);
+            acc = dot2_acc<DT>((w & 0x00F000F0u) | kOr, xp[4 * d + 1], acc);
+            acc = dot2_acc<DT>(((w >> 4) & 0x00F000F0u) | kOr, xp[4 * d + 2], acc);
+            acc = dot2_acc<DT>(((w >> 8) & 0x00F000F0u) | kOr, xp[4 * d + 3], acc);
         } else {
 #pragma unroll
             for (int i = 0; i < 8; i++)
