@@ -37,7 +37,8 @@ sweep (f16, 8192 x 8192, batch 1 and 4); `--workload batch` a decode batch of
 qkv` / `gated_norm` the fused one-launch decode pieces (Q + K + V projections;
 gated RMSNorm + out projection at the reference's bench shape); `--workload
 gather_decode` one token's top-2 routed gate / up / down launches over 8
-experts (the routed wave-per-row kernels); `--workload rows_probe` the headline gate / up launch taken apart (the shipped kernel, the
+experts (the routed wave-per-row kernels); `--workload widths` one row of x on the matrix shapes of other model families, as routed and with the rows
+kernels switched off; `--workload rows_probe` the headline gate / up launch taken apart (the shipped kernel, the
 streaming and wave-per-four-rows kernels it replaced, a launch that only reads the same bytes, and the
 wave-per-four-rows kernel without its arithmetic / with its weight loads only, plus its
 per-wave timeline), which is where the distance to the HBM peak is accounted
@@ -68,7 +69,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--layers", type=int, default=8, help="distinct MLP weight sets streamed per step")
     ap.add_argument("--workload", default="qmv",
-                    choices=["qmv", "qkv", "gated_norm", "qmm", "batch", "gather", "gather_decode", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep", "rows_probe"],
+                    choices=["qmv", "qkv", "gated_norm", "qmm", "batch", "gather", "gather_decode", "gather_prefill", "quantize", "dequantize", "copy", "read", "sweep", "rows_probe", "widths"],
                     help="qmv is the headline (its line also carries qmm M=512 and the gather as secondary legs); "
                          "qmm / gather report those configurations alone; sweep the bit-width / group-size cells; "
                          "copy runs only the known-size copy kernel (counter calibration); read times a kernel that only reads the "
@@ -603,6 +604,56 @@ def leg_rows_probe(a, runner, info):
             "probe_vs_streaming_kernel_max_rel_dev": dev, "timeline_us": timeline}
 
 
+def leg_widths(a, runner, info):
+    """One row of x on 4-bit g64 bf16 matrices of the shapes other model families bring (hidden sizes 2048 ... 7168 and their
+    MLP widths): every launch in a chain over cold rotating operand sets, as routed (qmv.kernel = 0) and with the rows
+    kernels switched off (qmv.kernel = 2: the streaming kernel or the matrix-core GEMV, which served these shapes
+    before), the kernel that the route names, and the fraction of the HBM peak on the algorithmic bytes."""
+    from metaltile_amd import DType, GpuBuffer, _lib, ops
+    from metaltile_amd.synth import make_case, qmv_bytes
+    lib = _lib.load()
+    dt = DType.BF16
+    shapes = [(8192, 2048), (2048, 8192), (8192, 3072), (3072, 8192), (18944, 3584), (3584, 18944), (13824, 5120), (5120, 13824),
+              (11008, 4096), (4096, 11008), (16384, 6144), (18432, 7168), (7168, 18432), (151936, 3584)]
+    cells = {}
+    for N, K in shapes:
+        nb = qmv_bytes(N, K, 4, 64, 1, 2)
+        nset = max(8, -(-(640 << 20) // nb))
+        c = make_case(9000 + N % 977 + K, dt, 4, 64, 1, N, K, bias_rule="midpoint")
+        specs = []
+        for _ in range(nset):
+            bufs = {"w": GpuBuffer.from_bytes(c.w.tobytes()), "scales": GpuBuffer.from_bytes(c.scales_bytes), "biases": GpuBuffer.from_bytes(c.biases_bytes),
+                    "x": GpuBuffer.from_bytes(c.x_bytes), "out": GpuBuffer(N * 2)}
+            specs.append(("mt_qmv", dt, bufs, {"k": K, "gs_per_row": K // 64}))
+        cell = {"bytes": nb, "kernel": ops.plan("qmv", dt, 4, 64, 1, N, K)[1][0][0].split("(")[0].replace("void mtq::", "")}
+        reps = max(1, 3000 // nset)
+        for key, opt in (("routed_us", 0), ("rows_kernels_off_us", 2)):
+            _lib.check(lib.mtq_set_option(b"qmv.kernel", opt))
+            try:
+                runner.wake_clocks(WAKE_MS)
+                best = None
+                for _ in range(3):
+                    runner.dispatch_chain(specs, repeat=max(1, reps // 2), per_kernel=False)
+                    _, _, us = runner.dispatch_chain(specs, repeat=reps, per_kernel=False, stream_events=True)
+                    us /= reps * nset
+                    best = us if best is None or us < best else best
+            finally:
+                lib.mtq_set_option(b"qmv.kernel", 0)
+            cell[key] = round(best, 2)
+        cell["frac"] = round(nb / cell["routed_us"] / 1e3 / HBM_PEAK_GBS, 4)
+        cells[f"{N}x{K}"] = cell
+        for sp in specs:
+            for buf in sp[2].values():
+                buf.free()
+    head = cells["18944x3584"]
+    return {"metric": "qmv GB/s on the row lengths of other model families (4-bit g64 bf16, batch 1); value = 18944x3584",
+            "value": round(head["bytes"] / head["routed_us"] / 1e3, 1), "unit": "GB/s", "ms_per_step": head["routed_us"] / 1e3, "dtype": "bf16",
+            "config": {"workload": "one launch per step in a chain over cold rotating operand sets; cells = min over 3 rounds of the average launch duration",
+                       "device": info["name"] or info["arch"]},
+            "roofline": {"bound": "hbm", "achieved": round(head["bytes"] / head["routed_us"] / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head["frac"], "traffic": None},
+            "cells": cells}
+
+
 def m_unpack(b):
     import metaltile_amd as m
     from metaltile_amd import DType
@@ -674,6 +725,11 @@ def main():
 
     if a.workload == "rows_probe":
         out.update(leg_rows_probe(a, runner, info))
+        print(json.dumps(out))
+        return
+
+    if a.workload == "widths":
+        out.update(leg_widths(a, runner, info))
         print(json.dumps(out))
         return
 
