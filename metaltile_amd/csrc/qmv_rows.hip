@@ -538,9 +538,8 @@ static int launch_rows(int dtype, const void* w, const void* s, const void* b, c
 }
 
 // chunks of 16 bytes per lane and row for the one-row-per-wave kernel, or 0 if it has no instance for the shape
-// (*tail: the chunks of the row's last group of 64 where that group is not full, else 0)
-static int rows_long_ch(const QmvParams& p, int* tail = nullptr) {
-    if (tail) *tail = 0;
+// (rows whose last group of 64 chunks is not full count that group)
+static int rows_long_ch(const QmvParams& p) {
     if (p.bits != 2 && p.bits != 4) return 0;
     const uint32_t G = p.group_size, cpc = 128u / (uint32_t)p.bits;
     if (G != 32 && G != 64 && G != 128) return 0;
@@ -548,11 +547,10 @@ static int rows_long_ch(const QmvParams& p, int* tail = nullptr) {
     // chunks) and 11008, 13824, 18944, 27648 (the last group partly filled). Every lane's groups of the bias term are one
     // aligned load: up to 256 groups per row the rows' scales are 8-byte multiples, beyond that 16-byte multiples.
     if (p.bits == 4 && G >= 64 && p.gather == GATHER_NONE) {
-        static const struct { uint32_t K; int ch, tail; } kMore[] = {{10240, 5, 0}, {12288, 6, 0}, {18432, 9, 0}, {11008, 6, 24}, {13824, 7, 48}, {18944, 10, 16}, {27648, 14, 32}};
+        static const struct { uint32_t K; int ch; } kMore[] = {{10240, 5}, {12288, 6}, {18432, 9}, {11008, 6}, {13824, 7}, {18944, 10}, {27648, 14}};
         for (const auto& m : kMore) {
             if (p.K != m.K) continue;
             if (p.K / G > 256u && ((uintptr_t)p.scales % 16 || (uintptr_t)p.biases % 16)) return 0;
-            if (tail) *tail = m.tail;
             return m.ch;
         }
     }
@@ -650,8 +648,7 @@ int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
     const uint32_t slots = routed && p.gather != GATHER_SINGLE ? (p.T < p.E ? p.T : p.E) : 1u;   // the experts that can have a row
     if (p.bits == 4 && p.group_size == 64 && p.K == 4096)
         return launch_rows(p.dtype, p.w, p.scales, p.biases, p.x, p.out, p.N, 0, nullptr, lc, p.gather, p.route, p.E, p.T, slots);
-    int tail = 0;
-    const int ch = rows_long_ch(p, &tail);
+    const int ch = rows_long_ch(p);
     QmvRowsLArgs a{(const rp_u32x4*)p.w, (const uint16_t*)p.scales, (const uint16_t*)p.biases, (const uint16_t*)p.x, (uint16_t*)p.out, p.N, p.route, p.E, p.T};
     void* args[] = {&a};
     const void* fn = p.gather == GATHER_CSR       ? (p.dtype == DT_BF16 ? rows_long_routed_fn<DT_BF16, GATHER_CSR>(ch) : rows_long_routed_fn<DT_F16, GATHER_CSR>(ch))
@@ -670,7 +667,6 @@ int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
     // From 8192 rows on (two or more workgroups of sixteen per compute unit) sixteen are ahead again: 8192 x 14336 13.2 ->
     // 12.65 us, 14336 x 14336 21.25 -> 20.35. (28672 codes: 896 chunks to prepare, always sixteen.)
     const uint32_t block = ch > 8 || (ch == 7 && p.N >= 8192u) ? 1024u : ch > 4 ? 512u : 1024u;
-    (void)tail;
     if (block < 64u * (uint32_t)ch) return fail(ERR_UNSUPPORTED, "qmv rows kernels: workgroup smaller than the row's chunks");   // (thread t prepares chunk t)
     hipError_t e = launch_kernel(fn, dim3((p.N + block / 64u - 1u) / (block / 64u), slots), dim3(block), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "qmv long rows kernel launch");
