@@ -527,10 +527,13 @@ template <bool NORM> static int launch_rows_walk(const QmvParams& p, const void*
     }
     void* args[] = {&a};
     const uint32_t G = p.group_size;
-    // Up to 4096 rows one workgroup of sixteen waves per 16 rows (norm, 4096 x 4096 bf16: 4.5 us against 5.6 in workgroups of
-    // eight); beyond, two workgroups of eight waves per compute unit, which walk the rows (14336 x 4096: the same either
-    // way; eight hold on the machines where a launch of exactly one large workgroup per compute unit falls behind).
-    const bool sixteen = p.N <= 4096;
+    // From 2049 to 4096 rows one workgroup of sixteen waves per 16 rows (norm, 4096 x 4096 bf16: 4.5 us against 5.6 in
+    // workgroups of eight); beyond, two workgroups of eight waves per compute unit, which walk the rows (14336 x 4096: the
+    // same either way; eight hold on the machines where a launch of exactly one large workgroup per compute unit falls
+    // behind). Up to 2048 rows workgroups of eight again: sixteen rows per workgroup would leave compute units without one
+    // (bf16 g64, sixteen -> eight: 2048 x 7168 4.32 -> 3.66, 1024 x 7168 4.15 -> 3.26, 2048 x 5120 3.79 -> 3.29, 2048 x 4096
+    // 3.2 - 3.4 -> 3.0, 1024 x 3072 3.05 - 3.35 -> 2.76).
+    const bool sixteen = p.N > 2048 && p.N <= 4096;
     const uint32_t nwv = sixteen ? 16u : 8u, cap = sixteen ? 256u : 512u;
     const void* fn = p.dtype == DT_BF16 ? (G == 32 ? rows_walk_fn<DT_BF16, 5, NORM>(p.K, sixteen) : G == 64 ? rows_walk_fn<DT_BF16, 6, NORM>(p.K, sixteen) : rows_walk_fn<DT_BF16, 7, NORM>(p.K, sixteen))
                                         : (G == 32 ? rows_walk_fn<DT_F16, 5, NORM>(p.K, sixteen) : G == 64 ? rows_walk_fn<DT_F16, 6, NORM>(p.K, sixteen) : rows_walk_fn<DT_F16, 7, NORM>(p.K, sixteen));
