@@ -286,3 +286,45 @@ def test_single_index_expert_on_the_wave_per_row_kernels(oracle, dt, N, K, kerne
         out.free(); ei.free()
     for buf in (w, s, b, x):
         buf.free()
+
+
+@pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
+@pytest.mark.parametrize("N,K,kernel", [(1030, 2048, "qmv_rows_walk_routed_kernel"), (520, 7168, "qmv_rows_walk_routed_ragged_kernel")])
+def test_routed_walk_with_more_than_64_experts_under_per_row_ids(oracle, dt, N, K, kernel):
+    """Per-row ids name any number of experts (only the offsets view is read by one wave-wide load and stops at 64): 130
+    experts, rows on experts beyond the 64th, one expert named twice, an id that names no expert (its output row keeps its
+    bytes); the same routing under the offsets view falls to the kernels that take it. Forced with qmv.kernel = 4, behind
+    a cache flush, against the f64 oracle."""
+    import metaltile_amd as m
+    bits, G, E = 4, 64, 130
+    ids = [129, 3, 64, 129, 131]
+    T = len(ids)
+    idn = np.array(ids, dtype="<u4")
+    valid = np.array([129, 3, 64, 129, 0], dtype="<u4")
+    rb = N * dt.size_bytes
+    print(f"[case] routed walk, 130 experts, ids {dt.name} N{N} K{K}", flush=True)
+    c = make_case(8800 + N + K, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
+    exp = oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=valid, f64=True, threads=8)
+    exp = oracle.round_through(exp.astype(np.float32), ODT[dt]).reshape(T, N)
+    w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
+                  GpuBuffer.from_bytes(c.biases_bytes), GpuBuffer.from_bytes(c.x_bytes))
+    lib = _lib.load()
+    assert lib.mtq_set_option(b"qmv.kernel", 4) == 0
+    try:
+        rc, launches, _, n = ops.plan("gather_indices", dt, bits, G, 1, N, K, E, T)
+        assert rc == 0 and n == 1 and kernel in launches[0][0] and launches[0][1][1] == T, launches
+        rc, launches, _, n = ops.plan("gather_csr", dt, bits, G, 1, N, K, E, T)
+        assert rc == 0 and "qmv_rows_walk" not in launches[0][0], launches
+        out, r = GpuBuffer.from_bytes(b"\xab" * (T * rb + 64)), GpuBuffer.from_bytes(idn.tobytes())
+        m.GpuRunner(0).flush_slc()
+        ops.gather_qmv_indices(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+    finally:
+        lib.mtq_set_option(b"qmv.kernel", 0)
+    raw = out.read_bytes()
+    assert raw[T * rb:] == b"\xab" * 64
+    assert raw[4 * rb:5 * rb] == b"\xab" * rb          # the row whose id names no expert
+    got = unpack_f32(raw[:4 * rb], dt).reshape(4, N)
+    for t in range(4):
+        assert rel_err(got[t], exp[t]) <= 1e-2, t
+    for buf in (w, s, b, x, out, r):
+        buf.free()
