@@ -61,7 +61,13 @@ struct RowsRoute {
 template <int GM> __device__ __forceinline__ bool rows_route(const uint32_t* route, uint32_t E, uint32_t T, uint32_t lane, RowsRoute& r) {
     if constexpr (GM == GATHER_CSR) {
         uint32_t lo, n1, lo2;
-        if (csr_route64(route, E, T, blockIdx.y, true, lane, r.expert, lo, n1, lo2) == 0) return false;
+        if (E <= 64u) {   // (one read of the offsets)
+            if (csr_route64(route, E, T, blockIdx.y, true, lane, r.expert, lo, n1, lo2) == 0) return false;
+        } else {          // (more experts than lanes: the offsets scanned 64 at a time, once for the slot's expert and once for its rows)
+            r.expert = csr_slot_expert(route, E, T, blockIdx.y, lane);
+            if (r.expert == 0xFFFFFFFFu) return false;
+            if (csr_expert_rows(route, E, T, r.expert, lane, lo, n1, lo2) == 0) return false;
+        }
         // (the same in every lane; said so, the pass loop and everything in it stay uniform control flow on scalar registers)
         r.expert = __builtin_amdgcn_readfirstlane(r.expert);
         lo = __builtin_amdgcn_readfirstlane(lo);

@@ -573,13 +573,11 @@ int launch_qmv_rows_norm(const QmvParams& p, const void* norm_w, const float* ep
 // The plain GEMV on the same walk: one activation row against one matrix.
 bool qmv_rows_walk_takes(const QmvParams& p) {
     if (p.gather != GATHER_NONE) {
-        // routed rows: at most 64 rows, and at most 64 experts under the offsets view (the routing is read by one wave-wide
-        // load; per-row ids and the single-index form name any number of experts), 4-bit codes in groups of 64, every
-        // expert's block of scales as aligned as the first
+        // routed rows: at most 64 rows (a wave-wide mask of an expert's rows) on any number of experts, 4-bit codes in groups
+        // of 64, every expert's block of scales as aligned as the first
         if (p.gather != GATHER_CSR && p.gather != GATHER_INDICES && p.gather != GATHER_SINGLE) return false;
         if (!p.route || p.E == 0 || p.bits != 4 || p.group_size != 64) return false;
         if (p.gather != GATHER_SINGLE && (p.T == 0 || p.T > 64)) return false;
-        if (p.gather == GATHER_CSR && p.E > 64) return false;   // (the offsets are read by one wave-wide load; per-row ids name any number of experts)
         if (((size_t)p.N * (p.K / 64u) * 2u) % 8u) return false;
         return (p.K == 4096 || p.K == 8192 || p.K == 2048 || p.K == 5120 || p.K == 7168) && qmv_rows_norm_takes(p, p.x);   // (the widths of expert layers it is built for)
     }

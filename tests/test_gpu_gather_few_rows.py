@@ -290,11 +290,10 @@ def test_single_index_expert_on_the_wave_per_row_kernels(oracle, dt, N, K, kerne
 
 @pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
 @pytest.mark.parametrize("N,K,kernel", [(1030, 2048, "qmv_rows_walk_routed_kernel"), (520, 7168, "qmv_rows_walk_routed_ragged_kernel")])
-def test_routed_walk_with_more_than_64_experts_under_per_row_ids(oracle, dt, N, K, kernel):
-    """Per-row ids name any number of experts (only the offsets view is read by one wave-wide load and stops at 64): 130
-    experts, rows on experts beyond the 64th, one expert named twice, an id that names no expert (its output row keeps its
-    bytes); the same routing under the offsets view falls to the kernels that take it. Forced with qmv.kernel = 4, behind
-    a cache flush, against the f64 oracle."""
+def test_routed_walk_with_more_than_64_experts(oracle, dt, N, K, kernel):
+    """Any number of experts under both routing views (up to 64 the offsets are read by one wave-wide load, beyond that
+    scanned 64 at a time): 130 experts, rows on experts beyond the 64th, one expert named twice, an id that names no
+    expert (its output row keeps its bytes). Forced with qmv.kernel = 4, behind a cache flush, against the f64 oracle."""
     import metaltile_amd as m
     bits, G, E = 4, 64, 130
     ids = [129, 3, 64, 129, 131]
@@ -313,11 +312,21 @@ def test_routed_walk_with_more_than_64_experts_under_per_row_ids(oracle, dt, N, 
     try:
         rc, launches, _, n = ops.plan("gather_indices", dt, bits, G, 1, N, K, E, T)
         assert rc == 0 and n == 1 and kernel in launches[0][0] and launches[0][1][1] == T, launches
-        rc, launches, _, n = ops.plan("gather_csr", dt, bits, G, 1, N, K, E, T)
-        assert rc == 0 and "qmv_rows_walk" not in launches[0][0], launches
         out, r = GpuBuffer.from_bytes(b"\xab" * (T * rb + 64)), GpuBuffer.from_bytes(idn.tobytes())
         m.GpuRunner(0).flush_slc()
         ops.gather_qmv_indices(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
+        # the offsets view of four sorted rows on the same experts (its offsets are scanned 64 at a time beyond 64 experts)
+        srt = np.array([3, 64, 129, 129], dtype="<u4")
+        rc, launches, _, n = ops.plan("gather_csr", dt, bits, G, 1, N, K, E, 4)
+        assert rc == 0 and n == 1 and kernel in launches[0][0] and launches[0][1][1] == 4, launches
+        e4 = oracle.gather_qmm(c.x_f[:4 * K], c.w, c.scales_f, c.biases_f, 4, K, N, E, bits, G, indices=srt, f64=True, threads=8)
+        e4 = oracle.round_through(e4.astype(np.float32), ODT[dt])
+        out4, r4 = GpuBuffer.from_bytes(b"\xab" * (4 * rb + 64)), GpuBuffer.from_bytes(_offsets(srt, E).tobytes())
+        ops.gather_qmv_csr(dt, bits, G, x, w, s, b, r4, out4, 4, N, K, E)
+        raw4 = out4.read_bytes()
+        assert raw4[4 * rb:] == b"\xab" * 64
+        assert rel_err(unpack_f32(raw4[:4 * rb], dt), e4.reshape(-1)) <= 1e-2
+        out4.free(); r4.free()
     finally:
         lib.mtq_set_option(b"qmv.kernel", 0)
     raw = out.read_bytes()

@@ -200,9 +200,8 @@ def test_benchmark_configurations_are_routed_as_documented():
     for view in ("gather_csr", "gather_indices"):      # fewer rows than experts: a grid row per row, not per expert
         for T, E in ((1, 8), (2, 8), (4, 8), (7, 8), (8, 128), (32, 128)):
             ks, ls = kernels(view, DType.BF16, 4, 64, 1, 14336, 4096, E, T)
-            # up to eight rows on experts of 14336 x 4096 (under the offsets view at most 64 experts): the routed walk, about
-            # 512 workgroups over the grid rows
-            kernel = "qmv_rows_walk_routed_kernel<2, 2, 6, " if T <= 8 and (E <= 64 or view == "gather_indices") else "qmv_mfma_kernel<2, 4,"
+            # up to eight rows on experts of 14336 x 4096: the routed walk, about 512 workgroups over the grid rows
+            kernel = "qmv_rows_walk_routed_kernel<2, 2, 6, " if T <= 8 else "qmv_mfma_kernel<2, 4,"
             assert kernel in ks[0] and ls[0][1][1] == T, (view, T, E, ls)
             if T <= 8 and E <= 64:
                 assert ls[0][1][0] == 512 // T and ls[0][2][0] == 512, ls
