@@ -610,7 +610,9 @@ bool qmv_rows_walk_preferred(const QmvParams& p) {
     // passes over its matrix: 13.4 -> 14.2 alone on 14336 x 4096 (the older kernel's second pass is shorter), 9.8 -> 8.6 and
     // 29.9 -> 22.2 on the others. The single-index form is routed as the plain launch of the same matrix (in a chain:
     // 14336 x 4096 7.4 -> 6.7, 14336 x 8192 13.8 -> 12.8, 4096 x 8192 5.0 -> 5.4).
-    if (p.gather != GATHER_NONE && p.gather != GATHER_SINGLE) return p.N >= 1024 && p.T < p.E && p.T <= 8;
+    // Small experts too (8 experts, 1 / 2 / 4 / 7 rows: 768 x 2048 4.13 -> 4.16, 4.47 -> 4.05, 6.14 -> 3.97, 7.46 -> 4.30; 768 x 8192 4.09 -> 4.00,
+    // 7.49 -> 4.03, 10.7 -> 5.27, 13.1 -> 6.69; 96 experts of 768 x 2048 5.37 -> 4.19, 5.82 -> 4.71, 7.17 -> 5.71, 8.55 -> 6.67 at 1 / 2 / 4 / 8 rows).
+    if (p.gather != GATHER_NONE && p.gather != GATHER_SINGLE) return p.N >= 256 && p.T < p.E && p.T <= 8;
     // 2-bit codes (rows of 8192), the one-row-per-wave kernel -> this: 8192 rows f16 g32 / g64 / g128 6.76 -> 6.30, 6.27 -> 5.91,
     // 6.09 -> 5.61; bf16 g64 14336 / 28672 rows 9.51 -> 8.75, 16.2 -> 14.4; 2048 / 4096 rows 3.62 -> 3.84, 4.01 -> 4.30
     if (p.bits == 2) return p.N >= 8192;

@@ -37,8 +37,9 @@ def test_fewer_rows_than_experts(oracle, dt, E, ids, K):
     for view, route, fn in (("csr", _offsets(idn, E), ops.gather_qmv_csr), ("indices", idn, ops.gather_qmv_indices)):
         print(f"[case] few-row gather {view} {dt.name} E{E} ids={ids}", flush=True)
         rc, launches, _, n = ops.plan("gather_" + view, dt, bits, G, 1, N, K, E, T)
-        # one row on at most 64 experts: the one-row streaming kernel (rows of whole waves of 16-byte chunks)
-        kernel = "qmv_stream_kernel" if T == 1 and E <= 64 and K >= 2048 else "qmv_mfma_kernel"
+        # up to eight rows on rows of 2048 codes: the kernel whose waves walk the rows, a grid row per expert that has a row;
+        # otherwise the matrix-core GEMV
+        kernel = "qmv_rows_walk_routed_kernel" if T <= 8 and K == 2048 else "qmv_mfma_kernel"
         assert rc == 0 and n == 1 and kernel in launches[0][0] and launches[0][1][1] == T, launches
         out, r = GpuBuffer.from_bytes(b"\xff" * (T * N * dt.size_bytes)), GpuBuffer.from_bytes(route.tobytes())
         fn(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
@@ -153,9 +154,9 @@ def test_two_rows_on_the_one_row_kernel(oracle, dt, prefer_streaming):
 @pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
 @pytest.mark.parametrize("K", [1024, 1536, 2048])
 def test_one_routed_row_on_rows_the_streaming_kernel_cannot_tile(oracle, dt, K):
-    """One routed row: rows of whole waves of 16-byte chunks (K = 2048) take the one-row streaming kernel; shorter or
-    ragged rows (K = 1024, 1536) must land on a gather instance of the tiled kernels, not on the one-wave-per-output
-    fallback, and give the same answer either way."""
+    """One routed row: rows of 2048 codes take the routed kernel whose waves walk the rows; shorter or ragged rows
+    (K = 1024, 1536) must land on a gather instance of the tiled kernels, not on the one-wave-per-output fallback, and
+    give the same answer either way."""
     bits, G, N, E, T = 4, 64, 264, 8, 1
     c = make_case(8700 + K, dt, bits, G, T, N, K, E=E, bias_rule="midpoint")
     w, s, b, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes),
@@ -165,7 +166,7 @@ def test_one_routed_row_on_rows_the_streaming_kernel_cannot_tile(oracle, dt, K):
         assert rc == 0
         name = launches[0][0]
         assert "generic" not in name, name
-        assert ("qmv_stream_kernel" in name) == (K == 2048), name
+        assert ("qmv_rows_walk_routed_kernel" in name) == (K == 2048), name
     ids = np.array([5], dtype="<u4")
     exp = oracle.round_through(oracle.gather_qmm(c.x_f, c.w, c.scales_f, c.biases_f, T, K, N, E, bits, G, indices=ids, f64=True, threads=8)
                                .astype(np.float32), ODT[dt])
