@@ -612,7 +612,12 @@ bool qmv_rows_walk_preferred(const QmvParams& p) {
     // 14336 x 4096 7.4 -> 6.7, 14336 x 8192 13.8 -> 12.8, 4096 x 8192 5.0 -> 5.4).
     // Small experts too (8 experts, 1 / 2 / 4 / 7 rows: 768 x 2048 4.13 -> 4.16, 4.47 -> 4.05, 6.14 -> 3.97, 7.46 -> 4.30; 768 x 8192 4.09 -> 4.00,
     // 7.49 -> 4.03, 10.7 -> 5.27, 13.1 -> 6.69; 96 experts of 768 x 2048 5.37 -> 4.19, 5.82 -> 4.71, 7.17 -> 5.71, 8.55 -> 6.67 at 1 / 2 / 4 / 8 rows).
-    if (p.gather != GATHER_NONE && p.gather != GATHER_SINGLE) return p.N >= 256 && p.T < p.E && p.T <= 8;
+    // More rows than eight, on many small experts (96 experts, rows on distinct ones, 12 / 16 / 32 / 64 rows: experts of 2048 x 7168
+    // 31.1 -> 19.1, 27.1 -> 22.8, 52.9 -> 43.8, 90.2 -> 84.1; of 768 x 2048 11.3 -> 7.58, 12.8 -> 7.94, 15.0 -> 10.7, 15.8 -> 16.8; of 7168 x 2048
+    // 23.4 -> 24.0, 26.8 -> 29.5, 55.1 -> 56.5, 90.5 -> 110): up to 32 rows where an expert has at most 2048 rows and the experts are
+    // at least twice the rows.
+    if (p.gather != GATHER_NONE && p.gather != GATHER_SINGLE)
+        return p.N >= 256 && p.T < p.E && (p.T <= 8 || (p.T <= 32 && p.N <= 2048 && p.E >= 2u * p.T));
     // 2-bit codes (rows of 8192), the one-row-per-wave kernel -> this: 8192 rows f16 g32 / g64 / g128 6.76 -> 6.30, 6.27 -> 5.91,
     // 6.09 -> 5.61; bf16 g64 14336 / 28672 rows 9.51 -> 8.75, 16.2 -> 14.4; 2048 / 4096 rows 3.62 -> 3.84, 4.01 -> 4.30
     if (p.bits == 2) return p.N >= 8192;

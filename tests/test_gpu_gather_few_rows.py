@@ -22,7 +22,7 @@ def _offsets(ids, E):
 @pytest.mark.parametrize("dt", [DType.BF16, DType.F16], ids=lambda d: d.name)
 @pytest.mark.parametrize("E,ids", [(8, [3]), (8, [1, 6]), (8, [0, 7]), (8, [4, 4]), (64, [0, 63]), (8, [2, 2, 5]), (8, [0, 1, 2, 3, 4, 5, 6]),
                                    (130, [0, 63, 64, 65, 128, 129]), (130, [129]), (70, [64, 64, 64, 69]),
-                                   (40, list(range(4, 36)))],
+                                   (40, list(range(4, 36))), (130, list(range(0, 130, 5)))],
                          ids=lambda v: str(v) if isinstance(v, int) else "-".join(map(str, v[:6])))
 @pytest.mark.parametrize("K", [1024, 2048])
 def test_fewer_rows_than_experts(oracle, dt, E, ids, K):
@@ -39,7 +39,8 @@ def test_fewer_rows_than_experts(oracle, dt, E, ids, K):
         rc, launches, _, n = ops.plan("gather_" + view, dt, bits, G, 1, N, K, E, T)
         # up to eight rows on rows of 2048 codes: the kernel whose waves walk the rows, a grid row per expert that has a row;
         # otherwise the matrix-core GEMV
-        kernel = "qmv_rows_walk_routed_kernel" if T <= 8 and K == 2048 else "qmv_mfma_kernel"
+        # (and up to 32 rows on at least twice as many small experts)
+        kernel = "qmv_rows_walk_routed_kernel" if (T <= 8 or (T <= 32 and E >= 2 * T)) and K == 2048 else "qmv_mfma_kernel"
         assert rc == 0 and n == 1 and kernel in launches[0][0] and launches[0][1][1] == T, launches
         out, r = GpuBuffer.from_bytes(b"\xff" * (T * N * dt.size_bytes)), GpuBuffer.from_bytes(route.tobytes())
         fn(dt, bits, G, x, w, s, b, r, out, T, N, K, E)
