@@ -468,6 +468,7 @@ template <int DT, int CH, int LOG2G, int GM, int TAIL> __global__ __launch_bound
 }
 template <int DT, int GM> static const void* rows_walk_routed_fn(uint32_t K) {   // groups of 64
     if (K == 2048) return (const void*)qmv_rows_walk_routed_kernel<DT, 1, 6, GM>;
+    if (K == 6144) return (const void*)qmv_rows_walk_routed_kernel<DT, 3, 6, GM>;
     if (K == 5120) return (const void*)qmv_rows_walk_routed_ragged_kernel<DT, 3, 6, GM, 32>;
     if (K == 7168) return (const void*)qmv_rows_walk_routed_ragged_kernel<DT, 4, 6, GM, 32>;
     return K == 4096 ? (const void*)qmv_rows_walk_routed_kernel<DT, 2, 6, GM> : (const void*)qmv_rows_walk_routed_kernel<DT, 4, 6, GM>;
@@ -579,7 +580,7 @@ bool qmv_rows_walk_takes(const QmvParams& p) {
         if (!p.route || p.E == 0 || p.bits != 4 || p.group_size != 64) return false;
         if (p.gather != GATHER_SINGLE && (p.T == 0 || p.T > 64)) return false;
         if (((size_t)p.N * (p.K / 64u) * 2u) % 8u) return false;
-        return (p.K == 4096 || p.K == 8192 || p.K == 2048 || p.K == 5120 || p.K == 7168) && qmv_rows_norm_takes(p, p.x);   // (the widths of expert layers it is built for)
+        return (p.K == 4096 || p.K == 8192 || p.K == 2048 || p.K == 5120 || p.K == 6144 || p.K == 7168) && qmv_rows_norm_takes(p, p.x);   // (the widths of expert layers it is built for)
     }
     if (p.M != 1) return false;
     if (p.bits == 2) {   // rows of 8192 2-bit codes: the 4-bit instance's conditions on a matrix of that width

@@ -197,7 +197,8 @@ def forced_qmv_kernel(request):
                           # the kernel whose waves walk the rows (qmv.kernel = 4): one row per wave, and 5000 rows so that waves walk
                           (20, 4096, "qmv_rows_walk_routed_kernel", 4), (5000, 4096, "qmv_rows_walk_routed_kernel", 4), (1030, 8192, "qmv_rows_walk_routed_kernel", 4),
                           # the expert widths of other models: 2048 codes, and rows that end inside a group of 64 chunks
-                          (1030, 2048, "qmv_rows_walk_routed_kernel", 4), (40, 7168, "qmv_rows_walk_routed_ragged_kernel", 4), (2050, 5120, "qmv_rows_walk_routed_ragged_kernel", 4)],
+                          (1030, 2048, "qmv_rows_walk_routed_kernel", 4), (40, 7168, "qmv_rows_walk_routed_ragged_kernel", 4), (2050, 5120, "qmv_rows_walk_routed_ragged_kernel", 4),
+                          (1027, 6144, "qmv_rows_walk_routed_kernel", 4)],
                          indirect=["forced_qmv_kernel"])
 def test_routed_rows_on_the_wave_per_row_kernels(oracle, dt, N, K, kernel, forced_qmv_kernel):
     """The wave-per-row GEMV kernels with a grid row per expert that has a row (their automatic range is up to four rows
