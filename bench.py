@@ -608,7 +608,9 @@ def leg_widths(a, runner, info):
     """One row of x on 4-bit g64 bf16 matrices of the shapes other model families bring (hidden sizes 2048 ... 7168 and their
     MLP widths): every launch in a chain over cold rotating operand sets, as routed (qmv.kernel = 0) and with the rows
     kernels switched off (qmv.kernel = 2: the streaming kernel or the matrix-core GEMV, which served these shapes
-    before), the kernel that the route names, and the fraction of the HBM peak on the algorithmic bytes."""
+    before), the kernel that the route names, and the fraction of the HBM peak on the algorithmic bytes; then a few routed
+    rows on the expert shapes of those families, the same two ways."""
+    import numpy as np
     from metaltile_amd import DType, GpuBuffer, _lib, ops
     from metaltile_amd.synth import make_case, qmv_bytes
     lib = _lib.load()
@@ -645,13 +647,42 @@ def leg_widths(a, runner, info):
         for sp in specs:
             for buf in sp[2].values():
                 buf.free()
+    # routed rows (per-row ids) on the expert shapes of other families: each launch timed on its own, operands of the
+    # experts that are hit warm in the last-level cache (the same for both routes)
+    routed = {}
+    for E, N, K in ((96, 2048, 7168), (96, 7168, 2048), (96, 768, 2048), (8, 16384, 6144)):
+        c = make_case(9100 + N % 977 + K, dt, 4, 64, 8, N, K, E=E)
+        w, sc, bi, x = (GpuBuffer.from_bytes(c.w.tobytes()), GpuBuffer.from_bytes(c.scales_bytes), GpuBuffer.from_bytes(c.biases_bytes),
+                        GpuBuffer.from_bytes(c.x_bytes))
+        for T in (1, 4, 8) if E > 8 else (1, 2, 4):
+            ids = (np.arange(T, dtype="<u4") * (E // T) + 1) % E
+            route, outb = GpuBuffer.from_bytes(ids.tobytes()), GpuBuffer(T * N * 2)
+            cell = {"bytes": T * qmv_bytes(N, K, 4, 64, 1, 2)}
+            for key, opt in (("routed_us", 0), ("rows_kernels_off_us", 2)):
+                _lib.check(lib.mtq_set_option(b"qmv.kernel", opt))
+                try:
+                    runner.wake_clocks(WAKE_MS)
+                    best = None
+                    for _ in range(2):
+                        us = [ops.timed(ops.gather_qmv_indices, dt, 4, 64, x, w, sc, bi, route, outb, T, N, K, E) for _ in range(44)][4:]
+                        avg = float(np.mean(us))
+                        best = avg if best is None or avg < best else best
+                finally:
+                    lib.mtq_set_option(b"qmv.kernel", 0)
+                cell[key] = round(best, 2)
+            cell["kernel"] = ops.plan("gather_indices", dt, 4, 64, 1, N, K, E, T)[1][0][0].split("(")[0].replace("void mtq::", "")
+            routed[f"E{E} {N}x{K} T{T}"] = cell
+            route.free()
+            outb.free()
+        for buf in (w, sc, bi, x):
+            buf.free()
     head = cells["18944x3584"]
     return {"metric": "qmv GB/s on the row lengths of other model families (4-bit g64 bf16, batch 1); value = 18944x3584",
             "value": round(head["bytes"] / head["routed_us"] / 1e3, 1), "unit": "GB/s", "ms_per_step": head["routed_us"] / 1e3, "dtype": "bf16",
             "config": {"workload": "one launch per step in a chain over cold rotating operand sets; cells = min over 3 rounds of the average launch duration",
                        "device": info["name"] or info["arch"]},
             "roofline": {"bound": "hbm", "achieved": round(head["bytes"] / head["routed_us"] / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head["frac"], "traffic": None},
-            "cells": cells}
+            "cells": cells, "routed_cells": routed}
 
 
 def m_unpack(b):
