@@ -666,9 +666,10 @@ int launch_qmv_rows(const QmvParams& p, const LaunchCtx& lc) {
     // 7.70 on two others); shorter rows keep sixteen (8192 x 8192: 4-bit 8.00 / 7.97, 2-bit 6.27 / 6.95).
     // From 8192 rows on (two or more workgroups of sixteen per compute unit) sixteen are ahead again: 8192 x 14336 13.2 ->
     // 12.65 us, 14336 x 14336 21.25 -> 20.35. (28672 codes: 896 chunks to prepare, always sixteen.)
-    // Few rows of 8192 4-bit codes: workgroups of eight rows up to 2048 rows, so that every compute unit has one (1024 / 2048
-    // rows 3.98 -> 3.27, 4.16 -> 3.78 us; 3072 / 4096 rows 4.55 -> 4.87, 5.02 -> 5.22: sixteen again).
-    const uint32_t block = ch > 8 || (ch == 7 && p.N >= 8192u) ? 1024u : ch > 4 ? 512u : (ch == 4 && p.bits == 4 && p.N <= 2048u ? 512u : 1024u);
+    // Few rows of up to four chunks per lane: workgroups of eight rows up to 2048 rows, so that every compute unit has one
+    // (8192 4-bit codes, 1024 / 2048 rows 3.98 -> 3.27, 4.16 -> 3.78 us; 3072 / 4096 rows 4.55 -> 4.87, 5.02 -> 5.22: sixteen again;
+    // 2-bit codes, 1024 / 2048 rows of 8192 3.52 -> 3.25, 3.57 -> 3.23, of 16384 5.56 -> 4.27, 5.70 -> 4.62).
+    const uint32_t block = ch > 8 || (ch == 7 && p.N >= 8192u) ? 1024u : ch > 4 ? 512u : (p.N <= 2048u ? 512u : 1024u);
     if (block < 64u * (uint32_t)ch) return fail(ERR_UNSUPPORTED, "qmv rows kernels: workgroup smaller than the row's chunks");   // (thread t prepares chunk t)
     hipError_t e = launch_kernel(fn, dim3((p.N + block / 64u - 1u) / (block / 64u), slots), dim3(block), args, 0, lc);
     if (e != hipSuccess) return hip_fail(e, "qmv long rows kernel launch");
