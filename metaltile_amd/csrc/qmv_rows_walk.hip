@@ -633,7 +633,8 @@ bool qmv_rows_walk_preferred(const QmvParams& p) {
     // 12.9 -> 8.85, 23.5 -> 21.0 (151936 rows 55.6 -> 51.1); 5120 codes 3.86 -> 3.62, 5.91 -> 4.15, 8.27 -> 6.21, 13.8 -> 12.4, 32.2 -> 28.3
     // (13824 rows f16 g32 / g128 12.2 -> 9.85, 11.0 -> 10.5); 7168 codes 5.31 -> 4.15, 6.22 -> 4.94, 9.56 -> 7.65, 17.9 -> 15.4, 41.5 -> 39.2
     // (129280 rows 91.9 -> 86.4).
-    if (p.K == 3072 || p.K == 3584 || p.K == 5120 || p.K == 7168) return p.N >= 1024;
+    // (fewer rows too: 256 / 512 x 7168 5.24 -> 3.2, 256 / 768 x 3072 4.84 -> 2.7 - 3.2, 4.87 -> 2.7 - 3.4, 512 x 3584 4.97 -> 2.7 - 3.3, 512 x 5120 3.85 -> 3.0 - 3.3)
+    if (p.K == 3072 || p.K == 3584 || p.K == 5120 || p.K == 7168) return p.N >= 256;
     if (p.K == 2048) return p.N >= 1024 && p.N <= 20480;
     if (p.K == 6144) return p.N >= 1024;
     if (p.K == 4096) return p.N >= 1536 && (p.N <= 40960 || p.N >= 81920);
