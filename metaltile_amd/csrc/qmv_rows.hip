@@ -588,7 +588,8 @@ bool qmv_rows_takes(const QmvParams& p) {
 // 2-bit g32 / g64 / g128 8.98 / 8.55 / 8.41 -> 6.65 / 6.16 / 6.03, 4-bit 9.63 / 9.47 / 9.27 -> 8.53 / 7.90 / 7.78.
 // Small matrices stay where they were (a workgroup here is sixteen rows: few rows leave compute units idle).
 bool qmv_rows_preferred(const QmvParams& p) {
-    if (!qmv_rows_takes(p) || p.N < 1024) return false;
+    // (rows of 8192 4-bit codes from 256 weight rows: 256 / 512 / 768 rows 3.51 -> 3.15, 3.56 -> 3.17, 3.61 -> 3.22)
+    if (!qmv_rows_takes(p) || p.N < (p.bits == 4 && p.K == 8192 && p.gather == GATHER_NONE ? 256u : 1024u)) return false;
     // Routed rows: fewer rows than experts, each streaming its expert's matrix on its own grid row. 8 experts, bf16, us,
     // against the kernels that served these before (the one-row streaming kernel for one row, the matrix-core GEMV
     // beyond): 14336 x 4096, 1 / 2 / 3 / 4 rows on distinct experts 10.8 -> 8.4, 17.6 -> 15.8, 22.4 -> 23.3, 28.0 -> 31.1,

@@ -636,7 +636,7 @@ bool qmv_rows_walk_preferred(const QmvParams& p) {
     // (fewer rows too: 256 / 512 x 7168 5.24 -> 3.2, 256 / 768 x 3072 4.84 -> 2.7 - 3.2, 4.87 -> 2.7 - 3.4, 512 x 3584 4.97 -> 2.7 - 3.3, 512 x 5120 3.85 -> 3.0 - 3.3)
     if (p.K == 3072 || p.K == 3584 || p.K == 5120 || p.K == 7168) return p.N >= 256;
     if (p.K == 2048) return p.N >= 1024 && p.N <= 20480;
-    if (p.K == 6144) return p.N >= 1024;
+    if (p.K == 6144) return p.N >= 256;   // (256 / 512 / 768 rows 5.31 -> 2.93, 4.19 -> 2.94, 4.18 -> 2.96)
     if (p.K == 4096) return p.N >= 1536 && (p.N <= 40960 || p.N >= 81920);
     return p.N >= 10240 && p.group_size != 128;
 }
