@@ -1,16 +1,18 @@
-// The GEMV whose waves walk the rows: out[n] = sum_k (s q + b)[n, k] x[k] for one row of x against rows of 4096 / 8192
-// codes (the plain form also 2048 / 3072 / 3584 / 5120 / 6144 / 7168; mt_qmv and the affine_qmv family, crates/metaltile-std/src/mlx/quantized.rs:8-308; dequant_gemv_int2 / int4,
-// crates/metaltile-std/src/ffai/dequant_gemv.rs:52-100), f16 / bf16, groups of 32 / 64 / 128, and on the same body
+// The GEMV whose waves walk the rows: out[n] = sum_k (s q + b)[n, k] x[k] for one row of x against rows of 2048 ... 8192
+// 4-bit codes in steps of 1024, or 3584 (mt_qmv and the affine_qmv family, crates/metaltile-std/src/mlx/quantized.rs:8-308;
+// dequant_gemv_int2 / int4, crates/metaltile-std/src/ffai/dequant_gemv.rs:52-100), f16 / bf16, groups of 32 / 64 / 128; a row
+// that ends inside a group of 64 chunks is the *_ragged_kernel instances' (TAIL). On the same body
 //   - the RMS norm fused in front of it, x'[k] = x[k] norm_w[k] / sqrt(mean(x^2) + eps) (ffai_rms_norm_qgemv / _fast,
 //     crates/metaltile-std/src/ffai/rms_norm_qgemv.rs:53-125, 128-456),
 //   - two to four matrices against the one row in one launch (the fused projections of a decode step),
-//   - expert-routed rows, fewer than the experts, and the single-index expert GEMV,
-//   - 2-bit codes.
+//   - expert-routed rows, fewer than the experts, and the single-index expert GEMV (rows of 2048 / 4096 / 5120 / 6144 / 7168 /
+//     8192 codes in groups of 64),
+//   - 2-bit codes (rows of 8192).
 //
 // The make of the one-row-per-wave kernel (qmv_rows.hip): a wave owns a weight row, lane l its 16-byte chunks l, 64 + l, ...,
 // codes become operands of the 4x4x4 matrix instruction in place, the activations are put into operand order once per
 // workgroup in LDS. What differs is that a workgroup stays: the launch is at most two workgroups of eight waves per
-// compute unit (one of sixteen up to 4096 rows), wave g of G takes rows g, g + G, g + 2 G, ..., each row's loads issued
+// compute unit (one of sixteen from 2049 to 4096 rows), wave g of G takes rows g, g + G, g + 2 G, ..., each row's loads issued
 // while the row before it is worked on, so the activations are read and prepared once per few dozen rows. With the norm,
 // the activations are normalised on the way into LDS: every workgroup works out the row's sum of squares itself
 // (thread t from chunk t, one more barrier), and x', an f32 value in the reference, is carried as the element-type value
